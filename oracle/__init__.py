@@ -1,0 +1,237 @@
+"""CPU oracle bindings -- TEST INFRASTRUCTURE ONLY.
+
+ctypes/numpy front end of ``oracle/liboracle.so`` (the C restatement of the
+dlprimitives CPU operators in ``dlp_oracle.c``) and, when it has been built, of
+``oracle/_ref/libdlprim_ref.so`` (the reference's own internal BLAS and
+activation helpers compiled from the reference sources).
+
+Only tests, the smoke check and the CPU-baseline leg of the benchmark may import
+this package, and only as the checker.  The shipped library never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libdlprim_ref.so")
+
+ACTIVATIONS = {"identity": 0, "relu": 1, "tanh": 2, "sigmoid": 3, "relu6": 4}
+
+
+def build(force=False):
+    """Compile the oracle (and oracle/_ref when the reference tree is present)."""
+    args = ["make", "-C", _HERE]
+    if force:
+        args.insert(1, "-B")
+    subprocess.run(args, check=True, stdout=subprocess.DEVNULL)
+
+
+class _Cfg(ctypes.Structure):
+    _fields_ = [
+        ("channels_in", ctypes.c_int),
+        ("channels_out", ctypes.c_int),
+        ("kernel", ctypes.c_int * 2),
+        ("stride", ctypes.c_int * 2),
+        ("dilate", ctypes.c_int * 2),
+        ("pad", ctypes.c_int * 2),
+        ("groups", ctypes.c_int),
+    ]
+
+
+_lib = None
+_ref = None
+_fp = ctypes.POINTER(ctypes.c_float)
+_dp = ctypes.POINTER(ctypes.c_double)
+_ip = ctypes.POINTER(ctypes.c_int)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.orc_conv2d_output_shape.restype = ctypes.c_int
+        L.orc_conv2d_workspace.restype = ctypes.c_size_t
+        L.orc_conv2d_forward.restype = ctypes.c_int
+        L.orc_conv2d_forward_mt.restype = ctypes.c_int
+        L.orc_conv2d_direct_f64.restype = ctypes.c_int
+        L.orc_winograd_forward.restype = ctypes.c_int
+        L.orc_depthwise_forward.restype = ctypes.c_int
+        L.orc_bf16_round.restype = ctypes.c_float
+        L.orc_bf16_round.argtypes = [ctypes.c_float]
+        _lib = L
+    return _lib
+
+
+def ref():
+    """The compiled reference pieces, or None when oracle/_ref was not built."""
+    global _ref
+    if _ref is None and os.path.exists(_REF_PATH):
+        _ref = ctypes.CDLL(_REF_PATH)
+    return _ref
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_fp) if a is not None else None
+
+
+def _pair(v):
+    if isinstance(v, (tuple, list)):
+        return int(v[0]), int(v[1])
+    return int(v), int(v)
+
+
+def make_cfg(cin, cout, kernel, stride=1, dilate=1, pad=0, groups=1):
+    c = _Cfg()
+    c.channels_in, c.channels_out, c.groups = int(cin), int(cout), int(groups)
+    c.kernel[:] = _pair(kernel)
+    c.stride[:] = _pair(stride)
+    c.dilate[:] = _pair(dilate)
+    c.pad[:] = _pair(pad)
+    return c
+
+
+def _act(a):
+    return ACTIVATIONS[a] if isinstance(a, str) else int(a)
+
+
+def conv2d_output_shape(cfg, in_shape):
+    ish = (ctypes.c_int * 4)(*[int(v) for v in in_shape])
+    osh = (ctypes.c_int * 4)()
+    if lib().orc_conv2d_output_shape(ctypes.byref(cfg), ish, osh) != 0:
+        raise ValueError("invalid convolution configuration")
+    return tuple(osh)
+
+
+def conv2d_forward(x, w, bias, cfg, activation="identity", threads=1):
+    """Convolution2D::forward_cpu restated; ``threads`` != 1 distributes images over OpenMP."""
+    x, w = _f32(x), _f32(w)
+    bias = _f32(bias) if bias is not None else None
+    ish = (ctypes.c_int * 4)(*x.shape)
+    y = np.empty(conv2d_output_shape(cfg, x.shape), dtype=np.float32)
+    if threads == 1:
+        ws = np.empty(max(1, lib().orc_conv2d_workspace(ctypes.byref(cfg), ish) // 4), dtype=np.float32)
+        r = lib().orc_conv2d_forward(ctypes.byref(cfg), ish, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), _act(activation))
+    else:
+        r = lib().orc_conv2d_forward_mt(ctypes.byref(cfg), ish, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _act(activation), int(threads))
+    if r < 0:
+        raise ValueError("invalid convolution configuration")
+    return y
+
+
+def conv2d_direct_f64(x, w, bias, cfg, activation="identity"):
+    x, w = _f32(x), _f32(w)
+    bias = _f32(bias) if bias is not None else None
+    ish = (ctypes.c_int * 4)(*x.shape)
+    y = np.empty(conv2d_output_shape(cfg, x.shape), dtype=np.float64)
+    r = lib().orc_conv2d_direct_f64(ctypes.byref(cfg), ish, _ptr(x), _ptr(w), _ptr(bias), y.ctypes.data_as(_dp), _act(activation))
+    if r != 0:
+        raise ValueError("invalid convolution configuration")
+    return y
+
+
+def apply_factor(y_new, y_old, factor):
+    y = _f32(y_new).copy()
+    yo = _f32(y_old)
+    lib().orc_apply_factor(_ptr(y), _ptr(yo), ctypes.c_size_t(y.size), ctypes.c_float(factor))
+    return y
+
+
+def apply_activation(a, activation):
+    a = _f32(a).copy()
+    lib().orc_apply_activation(_ptr(a), ctypes.c_size_t(a.size), _act(activation))
+    return a
+
+
+def sgemm_nt(A, B, C=None, alpha=1.0, beta=0.0):
+    A, B = _f32(A), _f32(B)
+    M, K = A.shape
+    N = B.shape[0]
+    C = np.zeros((M, N), dtype=np.float32) if C is None else _f32(C).copy()
+    lib().orc_sgemm_nt(M, N, K, ctypes.c_float(alpha), _ptr(A), K, _ptr(B), K, ctypes.c_float(beta), _ptr(C), N)
+    return C
+
+
+def im2col(img, cfg, out_hw):
+    img = _f32(img)
+    cin_g, H, W = img.shape
+    OH, OW = out_hw
+    mat = np.empty((OH * OW, cin_g * cfg.kernel[0] * cfg.kernel[1]), dtype=np.float32)
+    lib().orc_im2col(ctypes.byref(cfg), cin_g, H, W, OH, OW, _ptr(img), _ptr(mat))
+    return mat
+
+
+def ip_forward(x, w, bias, activation="identity"):
+    x, w = _f32(x), _f32(w)
+    batch = x.shape[0]
+    x2 = x.reshape(batch, -1)
+    bias = _f32(bias) if bias is not None else None
+    y = np.empty((batch, w.shape[0]), dtype=np.float32)
+    lib().orc_ip_forward(batch, x2.shape[1], w.shape[0], _ptr(x2), _ptr(w), _ptr(bias), _ptr(y), _act(activation))
+    return y
+
+
+def winograd_filter_transform(w):
+    w = _f32(w)
+    cout, cin = w.shape[:2]
+    u = np.empty((cout, cin, 16), dtype=np.float32)
+    lib().orc_winograd_filter_transform(cout, cin, _ptr(w), _ptr(u))
+    return u
+
+
+def winograd_forward(x, w, bias, activation="identity", factor=0.0, y_old=None):
+    x, w = _f32(x), _f32(w)
+    bias = _f32(bias) if bias is not None else None
+    B, C, H, W = x.shape
+    N = w.shape[0]
+    y = np.zeros((B, N, H, W), dtype=np.float32) if y_old is None else _f32(y_old).copy()
+    u = np.empty(16 * C * N, dtype=np.float32)
+    r = lib().orc_winograd_forward(B, C, N, H, W, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(u), _act(activation), ctypes.c_float(factor))
+    if r != 0:
+        raise ValueError("invalid winograd configuration")
+    return y
+
+
+def depthwise_forward(x, w, bias, activation="identity", factor=0.0, y_old=None):
+    x, w = _f32(x), _f32(w)
+    bias = _f32(bias) if bias is not None else None
+    B, C, H, W = x.shape
+    kern = w.shape[-1]
+    y = np.zeros((B, C, H, W), dtype=np.float32) if y_old is None else _f32(y_old).copy()
+    r = lib().orc_depthwise_forward(B, C, H, W, kern, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _act(activation), ctypes.c_float(factor))
+    if r != 0:
+        raise ValueError("invalid depthwise configuration")
+    return y
+
+
+def bf16_round(a):
+    a = _f32(a).copy()
+    lib().orc_bf16_round_array(_ptr(a), ctypes.c_size_t(a.size))
+    return a
+
+
+# --- the compiled reference pieces (oracle/_ref) ---------------------------------
+
+def ref_sgemm(A, B, trans_a=False, trans_b=False, C=None, alpha=1.0, beta=0.0):
+    R = ref()
+    A, B = _f32(A), _f32(B)
+    M = A.shape[1] if trans_a else A.shape[0]
+    K = A.shape[0] if trans_a else A.shape[1]
+    N = B.shape[0] if trans_b else B.shape[1]
+    C = np.zeros((M, N), dtype=np.float32) if C is None else _f32(C).copy()
+    R.ref_cblas_sgemm(int(trans_a), int(trans_b), M, N, K, ctypes.c_float(alpha), _ptr(A), A.shape[1], _ptr(B), B.shape[1], ctypes.c_float(beta), _ptr(C), N)
+    return C
+
+
+def ref_apply_activation(a, activation):
+    a = _f32(a).copy()
+    ref().ref_apply_activation(_ptr(a), ctypes.c_size_t(a.size), _act(activation))
+    return a
