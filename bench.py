@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the convolution forward hot path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): the 20 convolutions
+of the ResNet-18 conv stack, forward, fp32 NCHW, batch 64, BN folded into
+weights + bias, fused ReLU, algorithm "gemm" (implicit GEMM on fp32 MFMA).
+A step = one pass over all 20 layers, launched back to back on one stream, with
+every tensor already resident in HBM.  Synthetic data: inputs uniform[-1,1],
+weights Kaiming-normal, bias uniform[-0.1,0.1], fixed seed.
+
+Prints ONE JSON line.  `value` = images/s of the whole stack; `gflops_per_s` is the
+same run expressed with the reference's flop accounting (tools/flops.cpp:660).
+`roofline` describes the kernel instantiation that takes the largest share of a
+step; per-launch durations are measured with HIP events on the launch stream in a
+second pass with one event pair per launch.  `cpu_baseline` is the CPU oracle
+(a restatement of the reference's single-threaded im2col + sgemm CPU path) timed
+on this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 images/sec"
+
+
+def build_layers(batch, seed, algo, activation_all_relu=True):
+    import numpy as np
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.workloads import RESNET18_CONVS, conv_bytes, conv_flops
+
+    rng = np.random.default_rng(seed)
+    out = []
+    for L in RESNET18_CONVS:
+        cin_g = L["cin"] // L["groups"]
+        x = torch.from_numpy(rng.uniform(-1, 1, (batch, L["cin"], L["hw"], L["hw"])).astype(np.float32)).cuda()
+        w = torch.from_numpy((rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) *
+                              np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)).cuda()
+        b = torch.from_numpy(rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)).cuda()
+        y = torch.empty((batch, L["cout"], L["ohw"], L["ohw"]), dtype=torch.float32, device="cuda")
+        st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], tuple(x.shape))
+        op = dlp.Conv2DForward.create(st, True, "relu", algo)
+        ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
+        out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch)))
+    return out
+
+
+def kernel_class(L):
+    """Which kernel instantiation serves a layer (tile selection is by Cout per group)."""
+    m = L["cout"] // L["groups"]
+    return "conv_gemm_f32<128x128>" if m > 64 else ("conv_gemm_f32<64x256>" if m > 32 else "conv_gemm_f32<32x256>")
+
+
+def cpu_baseline(images, seed):
+    """Oracle (port of the reference CPU path), 1 thread, `images` images through all 20 layers."""
+    import numpy as np
+
+    import oracle
+    from dlprimitives_amd.workloads import RESNET18_CONVS, conv_flops
+
+    rng = np.random.default_rng(seed)
+    total = 0.0
+    flops = 0.0
+    for L in RESNET18_CONVS:
+        cin_g = L["cin"] // L["groups"]
+        x = rng.uniform(-1, 1, (images, L["cin"], L["hw"], L["hw"])).astype(np.float32)
+        w = (rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) * np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)
+        b = rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)
+        cfg = oracle.make_cfg(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"])
+        t0 = time.perf_counter()
+        oracle.conv2d_forward(x, w, b, cfg, "relu", threads=1)
+        total += time.perf_counter() - t0
+        flops += conv_flops(L, images)
+    return dict(value=images / total, unit="images/s", cores=1, kind="port",
+                sample="%d of 64 images through all 20 ResNet-18 conv layers, single thread, %.1f s" % (images, total),
+                gflops_per_s=flops / total / 1e9)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--algo", default="gemm")
+    ap.add_argument("--cpu-images", type=int, default=4, help="images of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over batch with no exchange)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    dlp.lib()  # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    layers = build_layers(args.batch, 2024, args.algo)
+    stream = torch.cuda.current_stream()
+
+    def step():
+        for e in layers:
+            e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    total_flops = sum(e["flops"] for e in layers)
+
+    # second pass: one HIP event pair per launch, on the launch stream
+    nl = len(layers)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(nl + 1)] for _ in range(args.steps)]
+    for s in range(args.steps):
+        ev[s][0].record(stream)
+        for i, e in enumerate(layers):
+            e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+            ev[s][i + 1].record(stream)
+    torch.cuda.synchronize()
+    layer_ms = [sum(ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(args.steps)) / args.steps for i in range(nl)]
+
+    table = []
+    classes = {}
+    for e, ms in zip(layers, layer_ms):
+        L = e["layer"]
+        ai = e["flops"] / e["bytes"]
+        roof = min(FP32_MATRIX_PEAK_TFLOPS * 1e12, ai * HBM_PEAK_GBS * 1e9)
+        ach = e["flops"] / (ms * 1e-3)
+        table.append(dict(name=L["name"], ms=round(ms, 4), tflops=round(ach / 1e12, 2), gbs=round(e["bytes"] / (ms * 1e-3) / 1e9, 1),
+                          bound="mfma" if ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12 else "hbm",
+                          frac_of_roofline=round(ach / roof, 4), kernel=kernel_class(L)))
+        c = classes.setdefault(kernel_class(L), dict(ms=0.0, flops=0.0, launches=0))
+        c["ms"] += ms
+        c["flops"] += e["flops"]
+        c["launches"] += 1
+    dom_name, dom = max(classes.items(), key=lambda kv: kv[1]["ms"])
+    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel=dom_name, launches_per_step=dom["launches"],
+                    avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
+                    flops_per_launch=dom["flops"] / dom["launches"],
+                    achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / FP32_MATRIX_PEAK_TFLOPS, 4), traffic=None)
+    if args.layers:
+        for r in table:
+            print(json.dumps(r), file=sys.stderr)
+
+    cpu = cpu_baseline(args.cpu_images, 2024) if args.cpu_images > 0 else None
+
+    out = {
+        "metric": BASELINE_METRIC,
+        "value": round(args.batch / (ms_per_step * 1e-3), 1),
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "ResNet-18 conv stack forward: 20 convs, fp32 NCHW, batch %d, BN folded, fused ReLU, algo %s" % (args.batch, args.algo),
+                   "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1)},
+        "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac_of_fp32_matrix_peak": round(total_flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
+        "event_ms_per_step": round(sum(layer_ms), 4),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "layers": table,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,22 @@
+"""MI355X (gfx950) implementation of dlprimitives' convolution forward hot path.
+
+The product is the C-ABI library ``libdlprim_hip.so`` (declared in
+``include/dlprim_hip.h``, built from ``dlprimitives_amd/csrc``) and the C++
+header layer in ``include/dlprim/`` that keeps the ``dlprim::core`` names.
+This package is the Python binding used by the tests and the benchmark: a
+ctypes front end of the same C ABI, operating on torch device tensors.
+"""
+from .capi import (  # noqa: F401
+    ACTIVATIONS,
+    Conv2DForward,
+    Conv2DSettings,
+    DlprimError,
+    IPForward,
+    IPSettings,
+    NotImplementedErrorDlprim,
+    ValidationError,
+    build_library,
+    conv2d_output_shape,
+    lib,
+    library_path,
+)

@@ -1,0 +1,224 @@
+"""ctypes binding of include/dlprim_hip.h, mirroring dlprim::core's operator API.
+
+Names follow the reference (include/dlprim/core/conv.hpp:17-58,
+include/dlprim/core/ip.hpp:19-45): ``Conv2DSettings``, ``Conv2DForward.create``
+/ ``enqueue`` / ``algo`` / ``workspace`` / ``get_output_shape``, ``IPSettings``,
+``IPForward.create`` / ``enqueue``.  Errors come back as the reference's
+exception kinds (ValidationError, NotImplementedError).
+
+There is no fallback of any kind: if the HIP library is missing, loading fails.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libdlprim_hip.so")
+
+ACTIVATIONS = {"identity": 0, "relu": 1, "tanh": 2, "sigmoid": 3, "relu6": 4}
+FLOAT_DATA, HALF_DATA, BFLOAT16_DATA = 3, 2, 10
+
+
+class DlprimError(RuntimeError):
+    pass
+
+
+class ValidationError(DlprimError):
+    """dlprim::ValidationError"""
+
+
+class NotImplementedErrorDlprim(DlprimError):
+    """dlprim::NotImplementedError"""
+
+
+class _Settings(ctypes.Structure):
+    _fields_ = [
+        ("channels_in", ctypes.c_int),
+        ("channels_out", ctypes.c_int),
+        ("kernel", ctypes.c_int * 2),
+        ("stride", ctypes.c_int * 2),
+        ("dilate", ctypes.c_int * 2),
+        ("pad", ctypes.c_int * 2),
+        ("groups", ctypes.c_int),
+        ("shape", ctypes.c_int * 4),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+class _IPSettings(ctypes.Structure):
+    _fields_ = [
+        ("inputs", ctypes.c_int),
+        ("outputs", ctypes.c_int),
+        ("optimal_batch_size", ctypes.c_int),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+def library_path():
+    return _LIB
+
+
+def build_library():
+    """Compile libdlprim_hip.so for gfx950 (hipcc cross-compiles without a GPU)."""
+    subprocess.run(["make", "-C", os.path.join(_HERE, "csrc"), "-j8"], check=True, stdout=subprocess.DEVNULL)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise DlprimError(
+                "libdlprim_hip.so is not built (%s); run `make -C dlprimitives_amd/csrc` -- there is no CPU fallback" % _LIB)
+        L = ctypes.CDLL(_LIB)
+        L.dlp_last_error.restype = ctypes.c_char_p
+        L.dlp_conv2d_fwd_algo.restype = ctypes.c_char_p
+        L.dlp_conv2d_fwd_algo.argtypes = [ctypes.c_void_p]
+        L.dlp_conv2d_fwd_workspace.restype = ctypes.c_size_t
+        L.dlp_conv2d_fwd_workspace.argtypes = [ctypes.c_void_p]
+        L.dlp_conv2d_fwd_create.argtypes = [ctypes.POINTER(_Settings), ctypes.c_int, ctypes.c_int, ctypes.c_char_p,
+                                            ctypes.POINTER(ctypes.c_void_p)]
+        L.dlp_conv2d_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float,
+                                             ctypes.c_void_p]
+        L.dlp_conv2d_fwd_destroy.argtypes = [ctypes.c_void_p]
+        L.dlp_conv2d_fwd_destroy.restype = None
+        L.dlp_conv2d_output_shape.argtypes = [ctypes.POINTER(_Settings), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+        L.dlp_ip_fwd_create.argtypes = [ctypes.POINTER(_IPSettings), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+        L.dlp_ip_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_void_p, ctypes.c_void_p]
+        L.dlp_ip_fwd_destroy.argtypes = [ctypes.c_void_p]
+        L.dlp_ip_fwd_destroy.restype = None
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc == 0:
+        return
+    msg = lib().dlp_last_error().decode()
+    if rc == 1:
+        raise ValidationError(msg)
+    if rc == 2:
+        raise NotImplementedErrorDlprim(msg)
+    raise DlprimError(msg)
+
+
+def _pair(v):
+    if isinstance(v, (tuple, list)):
+        return int(v[0]), int(v[1])
+    return int(v), int(v)
+
+
+def _act(a):
+    return ACTIVATIONS[a] if isinstance(a, str) else int(a)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(int(stream))
+
+
+class Conv2DSettings:
+    """core::Conv2DSettings: Convolution2DConfigBase + input shape (batch is a hint) + dtype."""
+
+    def __init__(self, channels_in, channels_out, kernel, stride=1, dilate=1, pad=0, groups=1, shape=None, dtype=FLOAT_DATA):
+        self.channels_in, self.channels_out, self.groups = int(channels_in), int(channels_out), int(groups)
+        self.kernel, self.stride, self.dilate, self.pad = _pair(kernel), _pair(stride), _pair(dilate), _pair(pad)
+        self.shape = tuple(int(v) for v in shape)
+        self.dtype = dtype
+
+    def _c(self):
+        s = _Settings()
+        s.channels_in, s.channels_out, s.groups, s.dtype = self.channels_in, self.channels_out, self.groups, self.dtype
+        s.kernel[:], s.stride[:], s.dilate[:], s.pad[:] = self.kernel, self.stride, self.dilate, self.pad
+        s.shape[:] = self.shape
+        return s
+
+
+def conv2d_output_shape(settings, in_shape):
+    """Conv2DBase::get_output_shape"""
+    ish = (ctypes.c_int * 4)(*[int(v) for v in in_shape])
+    osh = (ctypes.c_int * 4)()
+    c = settings._c()
+    _check(lib().dlp_conv2d_output_shape(ctypes.byref(c), ish, osh))
+    return tuple(osh)
+
+
+class Conv2DForward:
+    """core::Conv2DForward"""
+
+    def __init__(self, handle, settings):
+        self._h = handle
+        self.settings = settings
+
+    @staticmethod
+    def create(settings, bias, activation="identity", algo=""):
+        h = ctypes.c_void_p()
+        c = settings._c()
+        _check(lib().dlp_conv2d_fwd_create(ctypes.byref(c), int(bool(bias)), _act(activation), (algo or "").encode(), ctypes.byref(h)))
+        return Conv2DForward(h, settings)
+
+    get_output_shape = staticmethod(conv2d_output_shape)
+
+    def algo(self):
+        return lib().dlp_conv2d_fwd_algo(self._h).decode()
+
+    def workspace(self):
+        return int(lib().dlp_conv2d_fwd_workspace(self._h))
+
+    def enqueue(self, x, w, bias, y, ws=None, factor=0.0, stream=None):
+        """x, w, bias, y, ws: torch device tensors (ws: uint8 of >= workspace() bytes)."""
+        xs = (ctypes.c_int * 4)(*x.shape)
+        ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
+        _check(lib().dlp_conv2d_fwd_enqueue(self._h, xs, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
+                                            float(factor), _stream(stream)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().dlp_conv2d_fwd_destroy(self._h)
+            self._h = None
+
+
+class IPSettings:
+    """core::IPSettings"""
+
+    def __init__(self, inputs, outputs, optimal_batch_size=-1, dtype=FLOAT_DATA):
+        self.inputs, self.outputs, self.optimal_batch_size, self.dtype = int(inputs), int(outputs), int(optimal_batch_size), dtype
+
+    def _c(self):
+        s = _IPSettings()
+        s.inputs, s.outputs, s.optimal_batch_size, s.dtype = self.inputs, self.outputs, self.optimal_batch_size, self.dtype
+        return s
+
+
+class IPForward:
+    """core::IPForward"""
+
+    def __init__(self, handle, settings):
+        self._h = handle
+        self.settings = settings
+
+    @staticmethod
+    def create(settings, bias, activation="identity"):
+        h = ctypes.c_void_p()
+        c = settings._c()
+        _check(lib().dlp_ip_fwd_create(ctypes.byref(c), int(bool(bias)), _act(activation), ctypes.byref(h)))
+        return IPForward(h, settings)
+
+    def enqueue(self, x, w, bias, y, stream=None):
+        _check(lib().dlp_ip_fwd_enqueue(self._h, int(x.shape[0]), _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _stream(stream)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().dlp_ip_fwd_destroy(self._h)
+            self._h = None

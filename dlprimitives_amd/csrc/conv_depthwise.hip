@@ -1,0 +1,209 @@
+// Depthwise (groups == channels) convolution forward for gfx950.
+//
+// Replaces the reference's Conv2DForwardDepthwiseSeparable / `conv` kernel
+// (src/core/conv.cpp:436-510, src/kernels/depthwise_separable_conv.cl:20-105),
+// which covers stride 1 only, and adds stride 2 (the reference falls back to a
+// grouped GEMM with M = 1 there, src/core/conv.cpp:725-727).
+//
+// The op is HBM-bound (about 2 flop per byte), so no matrix cores: the kernel is
+// organised around reading every input element exactly once and writing every
+// output exactly once, in wide contiguous runs.
+//
+// 3x3 kernel, lanes own output columns.  The (plane, column) pairs of the whole
+// tensor are laid on one flat axis; a wavefront covers 64 consecutive pairs and
+// walks down the rows keeping a three-row register window.  Each lane loads only
+// the input columns it owns; the columns to its left/right come from the
+// neighbouring lanes through wavefront shuffles.  Lanes at the edge of the
+// wavefront are halo lanes: they load and feed their neighbours but store
+// nothing, and adjacent wavefronts overlap by the halo, so there is no
+// divergent patch-up load.  Accumulation order is the reference's:
+// sum = bias; sum = fma(k[dr][dc], x, sum) for dr, dc ascending.
+//
+// Other odd kernel sizes (stride 1) use a plain direct kernel.
+#include "dlp_internal.hpp"
+
+namespace dlp {
+namespace {
+
+struct DwArgs {
+    const float *x;
+    const float *w;
+    const float *bias;
+    float *y;
+    int planes; // B*C
+    int C, H, W, OH, OW;
+    long long total_cols; // planes * OW
+    float factor;
+    int act;
+};
+
+// STRIDE 1: halo lanes 0 and 63 (62 outputs per wavefront)
+// STRIDE 2: halo lane 0 only (63 outputs per wavefront)
+template <int STRIDE>
+__global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
+{
+    constexpr int OUT_PER_WAVE = (STRIDE == 1) ? 62 : 63;
+    const int lane = threadIdx.x & 63;
+    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long f = wave * OUT_PER_WAVE + lane - 1; // flat (plane, ox) index
+    const bool in_range = f >= 0 && f < a.total_cols;
+    const int plane = in_range ? (int)(f / a.OW) : 0;
+    const int ox = in_range ? (int)(f - (long long)plane * a.OW) : 0;
+    const bool is_out = in_range && lane >= 1 && (STRIDE == 2 || lane <= 62);
+    const int c = plane % a.C;
+
+    float k[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++)
+        k[i] = a.w[c * 9 + i];
+    const float bias = a.bias ? a.bias[c] : 0.0f;
+
+    const float *xp = a.x + (size_t)plane * a.H * a.W;
+    float *yp = a.y + (size_t)plane * a.OH * a.OW + ox;
+
+    // columns owned by this lane
+    const int x0 = ox * STRIDE;
+    const bool v0 = in_range; // x0 < W always holds
+    const bool v1 = in_range && (STRIDE == 2) && (x0 + 1 < a.W);
+    const bool has_left = ox > 0;                        // column x0-1 exists in this plane
+    const bool has_right = (STRIDE == 1) && (ox + 1 < a.W); // column x0+1 (stride 1 only)
+
+    // window rows: r[dr][dc] for input columns (x0-1, x0, x0+1)
+    float r0[3], r1[3], r2[3];
+    auto load_row = [&](int yy, float (&row)[3]) {
+        const bool vy = yy >= 0 && yy < a.H;
+        const float *p = xp + (size_t)(vy ? yy : 0) * a.W + x0;
+        float c0 = (vy && v0) ? p[0] : 0.0f;
+        float c1 = 0.0f;
+        if (STRIDE == 2)
+            c1 = (vy && v1) ? p[1] : 0.0f;
+        if (STRIDE == 1) {
+            float left = __shfl_up(c0, 1);
+            float right = __shfl_down(c0, 1);
+            row[0] = has_left ? left : 0.0f;
+            row[1] = c0;
+            row[2] = has_right ? right : 0.0f;
+        } else {
+            float left = __shfl_up(c1, 1); // previous lane's odd column = 2*ox - 1
+            row[0] = has_left ? left : 0.0f;
+            row[1] = c0;
+            row[2] = c1;
+        }
+    };
+
+    // output row oy uses input rows oy*STRIDE - 1 + {0,1,2}
+    if (STRIDE == 1) {
+        load_row(-1, r0);
+        load_row(0, r1);
+    } else {
+        load_row(-1, r0);
+    }
+    for (int oy = 0; oy < a.OH; oy++) {
+        if (STRIDE == 1) {
+            load_row(oy + 1, r2);
+        } else {
+            load_row(2 * oy, r1);
+            load_row(2 * oy + 1, r2);
+        }
+        float sum = bias;
+#pragma unroll
+        for (int dc = 0; dc < 3; dc++)
+            sum = fmaf(k[dc], r0[dc], sum);
+#pragma unroll
+        for (int dc = 0; dc < 3; dc++)
+            sum = fmaf(k[3 + dc], r1[dc], sum);
+#pragma unroll
+        for (int dc = 0; dc < 3; dc++)
+            sum = fmaf(k[6 + dc], r2[dc], sum);
+        if (is_out)
+            store_out(yp + (size_t)oy * a.OW, apply_act(sum, a.act), a.factor);
+        if (STRIDE == 1) {
+#pragma unroll
+            for (int dc = 0; dc < 3; dc++) {
+                r0[dc] = r1[dc];
+                r1[dc] = r2[dc];
+            }
+        } else {
+#pragma unroll
+            for (int dc = 0; dc < 3; dc++)
+                r0[dc] = r2[dc];
+        }
+    }
+}
+
+// Any odd kernel size, stride 1 or 2, pad = K/2: one output per thread.
+__global__ __launch_bounds__(256) void depthwise_direct_kernel(DwArgs a, int K, int stride)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long total = (long long)a.planes * a.OH * a.OW;
+    if (idx >= total)
+        return;
+    const int ox = (int)(idx % a.OW);
+    const long long t = idx / a.OW;
+    const int oy = (int)(t % a.OH);
+    const int plane = (int)(t / a.OH);
+    const int c = plane % a.C;
+    const int pad = K / 2;
+    const float *xp = a.x + (size_t)plane * a.H * a.W;
+    const float *kp = a.w + (size_t)c * K * K;
+    float sum = a.bias ? a.bias[c] : 0.0f;
+    for (int dr = 0; dr < K; dr++) {
+        const int yy = oy * stride - pad + dr;
+        for (int dc = 0; dc < K; dc++) {
+            const int xx = ox * stride - pad + dc;
+            const float v = (yy >= 0 && yy < a.H && xx >= 0 && xx < a.W) ? xp[(size_t)yy * a.W + xx] : 0.0f;
+            sum = fmaf(kp[dr * K + dc], v, sum);
+        }
+    }
+    store_out(a.y + idx, apply_act(sum, a.act), a.factor);
+}
+
+} // namespace
+
+bool depthwise_supported(const ConvGeom &g)
+{
+    return g.dtype == DLP_FLOAT && g.groups == g.Cin && g.Cout == g.Cin && g.Cin > 1 && g.KH == g.KW && g.KH % 2 == 1 &&
+           g.ph == g.KH / 2 && g.pw == g.KW / 2 && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2);
+}
+
+int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream)
+{
+    DLP_REQUIRE(depthwise_supported(g), "geometry is not depthwise separable");
+    if (g.B == 0)
+        return DLP_OK;
+    DwArgs a;
+    a.x = (const float *)x;
+    a.w = (const float *)w;
+    a.bias = ep.bias;
+    a.y = (float *)y;
+    a.planes = g.B * g.Cin;
+    a.C = g.Cin;
+    a.H = g.H;
+    a.W = g.W;
+    a.OH = g.OH;
+    a.OW = g.OW;
+    a.total_cols = (long long)a.planes * g.OW;
+    a.factor = ep.factor;
+    a.act = ep.activation;
+    if (g.KH == 3) {
+        const int per_wave = g.sh == 1 ? 62 : 63;
+        const long long waves = (a.total_cols + per_wave - 1) / per_wave;
+        const long long blocks = (waves + 3) / 4;
+        if (blocks > 0x7fffffffLL)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
+        if (g.sh == 1)
+            hipLaunchKernelGGL(depthwise3x3_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(depthwise3x3_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    } else {
+        const long long total = (long long)a.planes * g.OH * g.OW;
+        const long long blocks = (total + 255) / 256;
+        if (blocks > 0x7fffffffLL)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
+        hipLaunchKernelGGL(depthwise_direct_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+} // namespace dlp

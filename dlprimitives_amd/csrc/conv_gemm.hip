@@ -1,0 +1,312 @@
+// Implicit-GEMM convolution forward for gfx950 (fp32 MFMA).
+//
+// Replaces the reference's ConvSGEMM / sgemm.cl CONVGEMM=1 path
+// (src/core/conv.cpp:45-111, src/gemm.cpp:429-565, src/kernels/sgemm.cl:75-133,296-715):
+//   C[M x N] = W[M x K] * im2col(X)[K x N],  M = Cout/groups, N = B*OH*OW, K = Cin/groups*KH*KW
+// with the im2col gather fused into the B-tile load, and bias + activation +
+// factor applied in registers before the NCHW store.
+//
+// Mapping to the hardware:
+//  * one workgroup = 4 wavefronts of 64 lanes; each wavefront owns a register
+//    tile made of 32x32 v_mfma_f32_32x32x2_f32 blocks.  The pixel dimension N is
+//    put on the MFMA column axis, so that the 32 lanes of a half-wave hold 32
+//    consecutive output pixels and every store is a 128-byte run in NCHW.
+//  * A (weights) and B (gathered input) tiles are staged through LDS in [k][m]
+//    and [k][n] order: an MFMA operand fetch is one conflict-free ds_read_b32.
+//  * all addressing of the gather is hoisted: per pixel a base offset and two
+//    bit masks (valid rows / valid columns of the window), per k a table entry
+//    (offset, tap) read through the scalar unit.  Out-of-window taps and tile
+//    tails are redirected to an out-of-range buffer offset, which the buffer
+//    load returns as 0.0 -- no divergent control flow in the main loop.
+//  * global loads of tile kt+1 are issued before the MFMAs of tile kt
+//    (register-staged double buffering, one barrier per K step).
+#include "dlp_internal.hpp"
+
+#include <vector>
+
+namespace dlp {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int BK = 16;
+constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
+
+struct GemmArgs {
+    const float *x;
+    const float *w;
+    const float *bias;
+    float *y;
+    const KTabEntry *ktab;
+    int M, N, K, nkt;
+    int mtiles, ntiles;
+    int Cin, Cin_g, H, W, Cout, OW, OHW;
+    int sh, sw, ph, pw, dh, dw, KH, KW;
+    uint32_t x_bytes, w_bytes;
+    float factor;
+    int act;
+};
+
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
+{
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
+    constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA blocks per wavefront
+    static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "tile shape");
+    constexpr int LDA = BM + 2; // stride = 2 (mod 32): transposed A stores hit 32 distinct banks
+    constexpr int LDB = BN;
+    constexpr int KSPLIT = kThreads / BN;   // k slices among the B loader threads
+    static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK % KSPLIT == 0, "B loader shape");
+    constexpr int B_LD = BK / KSPLIT;       // gathered elements per thread per K step
+    constexpr int A_LD = BM * BK / kThreads; // weight elements per thread per K step
+
+    __shared__ float As[2][BK][LDA];
+    __shared__ float Bs[2][BK][LDB];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // tile decode: m tile fastest, then n tile, then group
+    int t = blockIdx.x;
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    const int g = t / a.ntiles;
+    const int m0 = mt * BM, n0 = nt * BN;
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+    // ---- per-thread gather state (one output pixel per thread) ----
+    const int p = tid % BN;
+    const int ks = __builtin_amdgcn_readfirstlane(tid / BN);
+    int base;
+    uint32_t my = 0, mx = 0;
+    {
+        const int n = n0 + p;
+        const bool vn = n < a.N;
+        const int b = n / a.OHW;
+        const int pix = n - b * a.OHW;
+        const int oy = pix / a.OW;
+        const int ox = pix - oy * a.OW;
+        const int iy0 = oy * a.sh - a.ph;
+        const int ix0 = ox * a.sw - a.pw;
+        base = ((b * a.Cin + g * a.Cin_g) * a.H + iy0) * a.W + ix0;
+        if (vn) {
+            for (int ky = 0; ky < a.KH; ky++) {
+                int yy = iy0 + ky * a.dh;
+                if (yy >= 0 && yy < a.H)
+                    my |= 1u << ky;
+            }
+            for (int kx = 0; kx < a.KW; kx++) {
+                int xx = ix0 + kx * a.dw;
+                if (xx >= 0 && xx < a.W)
+                    mx |= 1u << kx;
+            }
+        }
+    }
+
+    // ---- per-thread weight loader state ----
+    const int ak = tid & 15;
+    const int am = tid >> 4;
+    uint32_t a_off[A_LD];
+#pragma unroll
+    for (int j = 0; j < A_LD; j++) {
+        int m = m0 + am + 16 * j;
+        a_off[j] = (m < a.M) ? (uint32_t)(((g * a.M + m) * a.K + ak) * 4) : kOutOfRange;
+    }
+
+    float ra[A_LD], rb[B_LD];
+
+    auto load_tiles = [&](int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int j = 0; j < A_LD; j++) {
+            uint32_t off = (k0 + ak < a.K) ? a_off[j] + (uint32_t)(k0 * 4) : kOutOfRange;
+            ra[j] = buf_load(wr, off);
+        }
+#pragma unroll
+        for (int i = 0; i < B_LD; i++) {
+            const KTabEntry e = a.ktab[k0 + ks + i * KSPLIT];
+            const int ky = e.tap & 0xff, kx = e.tap >> 8;
+            const bool ok = ((my >> ky) & (mx >> kx) & 1u) != 0;
+            uint32_t off = ok ? (uint32_t)((base + e.offset) * 4) : kOutOfRange;
+            rb[i] = buf_load(xr, off);
+        }
+    };
+    auto store_tiles = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < A_LD; j++)
+            As[buf][ak][am + 16 * j] = ra[j];
+#pragma unroll
+        for (int i = 0; i < B_LD; i++)
+            Bs[buf][ks + i * KSPLIT][p] = rb[i];
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    load_tiles(0);
+    store_tiles(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < a.nkt; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < a.nkt)
+            load_tiles(kt + 1);
+#pragma unroll
+        for (int kk = 0; kk < BK / 2; kk++) {
+            const int k = 2 * kk + h;
+            float fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                fa[i] = As[buf][k][wm * WTM + i * 32 + l32];
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                fb[j] = Bs[buf][k][wn * WTN + j * 32 + l32];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < a.nkt)
+            store_tiles(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: bias, activation, factor, NCHW store ----
+    // accumulator register r of a 32x32 block holds row 8*(r/4) + 4*h + r%4, column l32
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + l32;
+        if (n >= a.N)
+            continue;
+        const int b = n / a.OHW;
+        const int pix = n - b * a.OHW;
+        float *yb = a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < a.M) {
+                    float v = acc[i][j][r];
+                    if (a.bias)
+                        v += a.bias[g * a.M + m];
+                    v = apply_act(v, a.act);
+                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_cfg(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+{
+    a.mtiles = (a.M + BM - 1) / BM;
+    a.ntiles = (a.N + BN - 1) / BN;
+    long long blocks = (long long)a.mtiles * a.ntiles * g.groups;
+    if (blocks > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+} // namespace
+
+size_t conv_gemm_ktab_entries(const ConvGeom &g)
+{
+    size_t K = (size_t)(g.Cin / g.groups) * g.KH * g.KW;
+    return (K + BK - 1) / BK * BK;
+}
+
+void conv_gemm_fill_ktab(const ConvGeom &g, KTabEntry *tab)
+{
+    const int cin_g = g.Cin / g.groups;
+    const size_t K = (size_t)cin_g * g.KH * g.KW;
+    const size_t Kp = conv_gemm_ktab_entries(g);
+    size_t k = 0;
+    for (int c = 0; c < cin_g; c++)
+        for (int ky = 0; ky < g.KH; ky++)
+            for (int kx = 0; kx < g.KW; kx++, k++) {
+                tab[k].offset = (c * g.H + ky * g.dh) * g.W + kx * g.dw;
+                tab[k].tap = ky | (kx << 8);
+            }
+    for (; k < Kp; k++) {
+        tab[k].offset = 0;
+        tab[k].tap = 31 | (31 << 8); // bit 31 of the masks is never set
+    }
+    (void)K;
+}
+
+int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid)
+{
+    if (g.dtype != DLP_FLOAT)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: only float_data is implemented");
+    DLP_REQUIRE(g.KH <= 31 && g.KW <= 31, "kernel extent above 31 is not supported by the gather masks");
+    const size_t x_elems = (size_t)g.B * g.Cin * g.H * g.W;
+    const size_t w_elems = (size_t)g.Cout * (g.Cin / g.groups) * g.KH * g.KW;
+    const size_t y_elems = (size_t)g.B * g.Cout * g.OH * g.OW;
+    if (x_elems * 4 >= kOutOfRange || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
+    if (g.B == 0)
+        return DLP_OK;
+
+    GemmArgs a;
+    a.x = (const float *)x;
+    a.w = (const float *)w;
+    a.bias = ep.bias;
+    a.y = (float *)y;
+    a.ktab = dev_ktab;
+    a.M = g.Cout / g.groups;
+    a.N = g.B * g.OH * g.OW;
+    if (n_valid >= 0 && n_valid < a.N)
+        a.N = n_valid;
+    if (a.N == 0)
+        return DLP_OK;
+    a.K = (g.Cin / g.groups) * g.KH * g.KW;
+    a.nkt = (a.K + BK - 1) / BK;
+    a.Cin = g.Cin;
+    a.Cin_g = g.Cin / g.groups;
+    a.H = g.H;
+    a.W = g.W;
+    a.Cout = g.Cout;
+    a.OW = g.OW;
+    a.OHW = g.OH * g.OW;
+    a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw; a.dh = g.dh; a.dw = g.dw;
+    a.KH = g.KH; a.KW = g.KW;
+    a.x_bytes = (uint32_t)(x_elems * 4);
+    a.w_bytes = (uint32_t)(w_elems * 4);
+    a.factor = ep.factor;
+    a.act = ep.activation;
+
+    if (a.M > 64)
+        return launch_cfg<128, 128, 2, 2>(g, a, stream);
+    if (a.M > 32)
+        return launch_cfg<64, 256, 1, 4>(g, a, stream);
+    return launch_cfg<32, 256, 1, 4>(g, a, stream);
+}
+
+} // namespace dlp

@@ -1,0 +1,366 @@
+// C ABI of the gfx950 convolution forward path (see include/dlprim_hip.h).
+//
+// Host-side logic only: argument validation with the reference's rules,
+// algorithm selection (src/core/conv.cpp:672-729 in the reference), ownership of
+// the per-op gather tables, and dispatch to the HIP kernels.  There is no CPU
+// fallback: every compute entry launches a device kernel or fails.
+#include "dlp_internal.hpp"
+
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace dlp {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+
+int fail(int code, const std::string &msg)
+{
+    g_last_error = msg;
+    return code;
+}
+
+} // namespace dlp
+
+using namespace dlp;
+
+enum ConvAlgo { ALGO_GEMM = 0, ALGO_WINOGRAD = 1, ALGO_DEPTHWISE = 2 };
+
+struct dlp_conv2d_fwd {
+    dlp_conv2d_settings cfg;
+    bool bias;
+    int activation;
+    ConvAlgo algo;
+    int device;
+    KTabEntry *ktab; // device gather table of the GEMM stage
+    WinoPlan wino;
+    size_t workspace;
+};
+
+struct dlp_ip_fwd {
+    dlp_ip_settings cfg;
+    bool bias;
+    int activation;
+    int device;
+    KTabEntry *ktab;
+};
+
+static int upload_ktab(const ConvGeom &g, KTabEntry **out)
+{
+    const size_t n = conv_gemm_ktab_entries(g);
+    std::vector<KTabEntry> host(n ? n : 1);
+    conv_gemm_fill_ktab(g, host.data());
+    KTabEntry *dev = nullptr;
+    DLP_HIP_TRY(hipMalloc((void **)&dev, host.size() * sizeof(KTabEntry)));
+    hipError_t e = hipMemcpy(dev, host.data(), host.size() * sizeof(KTabEntry), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail(DLP_ERR_RUNTIME, std::string("hipMemcpy(gather table): ") + hipGetErrorString(e));
+    }
+    *out = dev;
+    return DLP_OK;
+}
+
+static bool valid_activation(int a) { return a >= DLP_ACT_IDENTITY && a <= DLP_ACT_RELU6; }
+
+// Conv2DBase::get_output_shape, src/core/conv.cpp:17-29
+static int output_shape(const dlp_conv2d_settings *cfg, const int in[4], int out[4])
+{
+    DLP_REQUIRE(cfg != nullptr && in != nullptr && out != nullptr, "null argument");
+    DLP_REQUIRE(in[1] == cfg->channels_in, "input channels differ from channels_in");
+    for (int i = 0; i < 2; i++) {
+        DLP_REQUIRE(cfg->kernel[i] > 0 && cfg->stride[i] > 0 && cfg->dilate[i] > 0 && cfg->pad[i] >= 0, "kernel/stride/dilate/pad");
+        int o = (in[2 + i] + 2 * cfg->pad[i] - cfg->dilate[i] * (cfg->kernel[i] - 1) - 1) / cfg->stride[i] + 1;
+        DLP_REQUIRE(o > 0, "empty output");
+        out[2 + i] = o;
+    }
+    out[0] = in[0];
+    out[1] = cfg->channels_out;
+    return DLP_OK;
+}
+
+static int make_geom(const dlp_conv2d_settings &c, const int x_shape[4], ConvGeom &g)
+{
+    int out[4];
+    int rc = output_shape(&c, x_shape, out);
+    if (rc != DLP_OK)
+        return rc;
+    g.B = x_shape[0];
+    g.Cin = c.channels_in;
+    g.H = x_shape[2];
+    g.W = x_shape[3];
+    g.Cout = c.channels_out;
+    g.OH = out[2];
+    g.OW = out[3];
+    g.KH = c.kernel[0];
+    g.KW = c.kernel[1];
+    g.sh = c.stride[0];
+    g.sw = c.stride[1];
+    g.ph = c.pad[0];
+    g.pw = c.pad[1];
+    g.dh = c.dilate[0];
+    g.dw = c.dilate[1];
+    g.groups = c.groups;
+    g.dtype = c.dtype;
+    return DLP_OK;
+}
+
+extern "C" {
+
+const char *dlp_last_error(void) { return g_last_error.c_str(); }
+
+int dlp_version(void) { return 100; }
+
+int dlp_device_count(int *count)
+{
+    DLP_REQUIRE(count != nullptr, "null argument");
+    DLP_HIP_TRY(hipGetDeviceCount(count));
+    return DLP_OK;
+}
+
+int dlp_set_device(int device)
+{
+    DLP_HIP_TRY(hipSetDevice(device));
+    return DLP_OK;
+}
+
+int dlp_device_name(int device, char *buf, size_t buf_len)
+{
+    DLP_REQUIRE(buf != nullptr && buf_len > 0, "null argument");
+    hipDeviceProp_t prop;
+    DLP_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    std::string s = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+    std::strncpy(buf, s.c_str(), buf_len - 1);
+    buf[buf_len - 1] = 0;
+    return DLP_OK;
+}
+
+int dlp_malloc(void **dev_ptr, size_t bytes)
+{
+    DLP_REQUIRE(dev_ptr != nullptr, "null argument");
+    *dev_ptr = nullptr;
+    if (bytes == 0)
+        return DLP_OK;
+    DLP_HIP_TRY(hipMalloc(dev_ptr, bytes));
+    return DLP_OK;
+}
+
+int dlp_free(void *dev_ptr)
+{
+    if (dev_ptr)
+        DLP_HIP_TRY(hipFree(dev_ptr));
+    return DLP_OK;
+}
+
+int dlp_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, void *stream)
+{
+    if (bytes == 0)
+        return DLP_OK;
+    DLP_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    DLP_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return DLP_OK;
+}
+
+int dlp_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, void *stream)
+{
+    if (bytes == 0)
+        return DLP_OK;
+    DLP_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    DLP_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return DLP_OK;
+}
+
+int dlp_stream_create(void **stream)
+{
+    DLP_REQUIRE(stream != nullptr, "null argument");
+    hipStream_t s;
+    DLP_HIP_TRY(hipStreamCreate(&s)); // default priority
+    *stream = (void *)s;
+    return DLP_OK;
+}
+
+int dlp_stream_sync(void *stream)
+{
+    DLP_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return DLP_OK;
+}
+
+int dlp_stream_destroy(void *stream)
+{
+    if (stream)
+        DLP_HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+    return DLP_OK;
+}
+
+int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], int out_shape[4])
+{
+    return output_shape(cfg, in_shape, out_shape);
+}
+
+int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activation, const char *algo, dlp_conv2d_fwd **out)
+{
+    DLP_REQUIRE(cfg != nullptr && out != nullptr, "null argument");
+    *out = nullptr;
+    DLP_REQUIRE(cfg->channels_in > 0 && cfg->channels_out > 0 && cfg->groups > 0, "channels/groups must be positive");
+    // src/ops/conv2d.cpp:105-106
+    DLP_REQUIRE(cfg->channels_in % cfg->groups == 0 && cfg->channels_out % cfg->groups == 0, "channels not divisible by groups");
+    DLP_REQUIRE(valid_activation(activation), "unknown activation");
+    if (cfg->dtype != DLP_FLOAT) // the reference: DLPRIM_CHECK(dtype == float_data), src/gemm.cpp:593
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "only float_data is implemented for Conv2DForward");
+    std::string al = algo ? algo : "";
+    DLP_REQUIRE(al == "" || al == "auto" || al == "gemm" || al == "winograd" || al == "depthwise_separable", "unknown algorithm name");
+
+    ConvGeom g;
+    int rc = make_geom(*cfg, cfg->shape, g);
+    if (rc != DLP_OK)
+        return rc;
+
+    // src/core/conv.cpp:704-729: requested-but-incompatible silently becomes gemm.
+    // The depthwise kernel here also covers stride 2, which the reference's does not.
+    const bool win = winograd_supported(g);
+    const bool dsc = depthwise_supported(g);
+    const bool auto_algo = al == "" || al == "auto";
+    ConvAlgo chosen = ALGO_GEMM;
+    if ((al == "winograd" && win) || (auto_algo && win && cfg->channels_in >= 8 && cfg->channels_out >= 8))
+        chosen = ALGO_WINOGRAD;
+    else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))
+        chosen = ALGO_DEPTHWISE;
+
+    dlp_conv2d_fwd *op = new (std::nothrow) dlp_conv2d_fwd();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *cfg;
+    op->bias = bias != 0;
+    op->activation = activation;
+    op->algo = chosen;
+    op->ktab = nullptr;
+    op->workspace = 0;
+    if (hipGetDevice(&op->device) != hipSuccess)
+        op->device = 0;
+    if (chosen == ALGO_GEMM) {
+        rc = upload_ktab(g, &op->ktab);
+    } else if (chosen == ALGO_WINOGRAD) {
+        op->wino = winograd_plan(g);
+        op->workspace = op->wino.ws_bytes;
+        rc = upload_ktab(op->wino.gemm, &op->ktab);
+    }
+    if (rc != DLP_OK) {
+        delete op;
+        return rc;
+    }
+    *out = op;
+    return DLP_OK;
+}
+
+const char *dlp_conv2d_fwd_algo(const dlp_conv2d_fwd *op)
+{
+    if (!op)
+        return "";
+    switch (op->algo) {
+    case ALGO_WINOGRAD:
+        return "winograd";
+    case ALGO_DEPTHWISE:
+        return "depthwise_separable";
+    default:
+        return "gemm";
+    }
+}
+
+size_t dlp_conv2d_fwd_workspace(const dlp_conv2d_fwd *op) { return op ? op->workspace : 0; }
+
+int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void *x, const void *w, const void *bias, void *y,
+                           void *ws, size_t ws_bytes, float factor, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[0] >= 0, "negative batch");
+    // the op is specialised for the H x W it was created with (the reference
+    // re-runs setup_algo when they change, src/ops/conv2d.cpp:200-209)
+    DLP_REQUIRE(x_shape[1] == op->cfg.channels_in && x_shape[2] == op->cfg.shape[2] && x_shape[3] == op->cfg.shape[3],
+                "input shape differs from the shape given at create (only the batch may change)");
+    // bias pointer present iff created with bias (src/gemm.cpp:526-533)
+    DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
+    ConvGeom g;
+    int rc = make_geom(op->cfg, x_shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    if (g.B == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && w != nullptr && y != nullptr, "null tensor pointer");
+    Epilogue ep;
+    ep.bias = (const float *)bias;
+    ep.factor = factor;
+    ep.activation = op->activation;
+    hipStream_t s = (hipStream_t)stream;
+    switch (op->algo) {
+    case ALGO_WINOGRAD:
+        return winograd_launch(g, op->wino, op->ktab, x, w, y, ws, ws_bytes, ep, s);
+    case ALGO_DEPTHWISE:
+        return depthwise_launch(g, x, w, y, ep, s);
+    default:
+        return conv_gemm_launch(g, op->ktab, x, w, y, ep, s);
+    }
+}
+
+void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op)
+{
+    if (!op)
+        return;
+    if (op->ktab)
+        (void)hipFree(op->ktab);
+    delete op;
+}
+
+int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_ip_fwd **out)
+{
+    DLP_REQUIRE(cfg != nullptr && out != nullptr, "null argument");
+    *out = nullptr;
+    DLP_REQUIRE(cfg->inputs > 0 && cfg->outputs > 0, "inputs/outputs must be positive");
+    DLP_REQUIRE(valid_activation(activation), "unknown activation");
+    if (cfg->dtype != DLP_FLOAT) // src/gemm.cpp:577
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "only float_data is implemented for IPForward");
+    dlp_ip_fwd *op = new (std::nothrow) dlp_ip_fwd();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *cfg;
+    op->bias = bias != 0;
+    op->activation = activation;
+    op->ktab = nullptr;
+    if (hipGetDevice(&op->device) != hipSuccess)
+        op->device = 0;
+    int rc = upload_ktab(ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype), &op->ktab);
+    if (rc != DLP_OK) {
+        delete op;
+        return rc;
+    }
+    *out = op;
+    return DLP_OK;
+}
+
+int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, const void *bias, void *y, void *stream)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    DLP_REQUIRE(batch >= 0, "negative batch");
+    DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
+    if (batch == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && w != nullptr && y != nullptr, "null tensor pointer");
+    Epilogue ep;
+    ep.bias = (const float *)bias;
+    ep.factor = 0.0f; // src/core/ip.cpp:38
+    ep.activation = op->activation;
+    return conv_gemm_launch(ip_gemm_geom(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype), op->ktab, x, w, y, ep,
+                            (hipStream_t)stream);
+}
+
+void dlp_ip_fwd_destroy(dlp_ip_fwd *op)
+{
+    if (!op)
+        return;
+    if (op->ktab)
+        (void)hipFree(op->ktab);
+    delete op;
+}
+
+} // extern "C"

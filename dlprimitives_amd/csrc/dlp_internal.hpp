@@ -1,0 +1,103 @@
+// Shared declarations of the gfx950 convolution forward path (host + device).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "../../include/dlprim_hip.h"
+
+namespace dlp {
+
+// Thread-local error message behind dlp_last_error().
+void set_error(const std::string &msg);
+int fail(int code, const std::string &msg);
+
+#define DLP_HIP_TRY(expr)                                                                      \
+    do {                                                                                       \
+        hipError_t e__ = (expr);                                                               \
+        if (e__ != hipSuccess)                                                                 \
+            return ::dlp::fail(DLP_ERR_RUNTIME, std::string(#expr) + ": " + hipGetErrorString(e__)); \
+    } while (0)
+
+#define DLP_REQUIRE(cond, msg)                                    \
+    do {                                                          \
+        if (!(cond))                                              \
+            return ::dlp::fail(DLP_ERR_VALIDATION, std::string("check failed: ") + #cond + " -- " + (msg)); \
+    } while (0)
+
+// Geometry of one forward convolution call (whole tensor, all groups).
+struct ConvGeom {
+    int B, Cin, H, W;
+    int Cout, OH, OW;
+    int KH, KW;
+    int sh, sw, ph, pw, dh, dw;
+    int groups;
+    int dtype; // DLP_FLOAT / DLP_BFLOAT16 / DLP_HALF
+};
+
+// Fused epilogue: v = act(acc + bias[c]); y = factor != 0 ? factor*y + v : v
+// (src/kernels/sgemm.cl:658-672,707-710 in the reference).
+struct Epilogue {
+    const float *bias; // nullptr when the op was created without bias
+    float factor;
+    int activation;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act)
+{
+    switch (act) {
+    case DLP_ACT_RELU:
+        return fmaxf(v, 0.0f);
+    case DLP_ACT_TANH:
+        return tanhf(v);
+    case DLP_ACT_SIGMOID:
+        return 1.0f / (1.0f + expf(-v));
+    case DLP_ACT_RELU6:
+        return fminf(fmaxf(v, 0.0f), 6.0f);
+    default:
+        return v;
+    }
+}
+
+__device__ __forceinline__ void store_out(float *p, float v, float factor)
+{
+    if (factor != 0.0f)
+        *p = fmaf(*p, factor, v);
+    else
+        *p = v;
+}
+
+// ---- implicit-GEMM convolution (conv_gemm.hip) ------------------------------
+// Per-k gather table entry: element offset of tap (c,ky,kx) inside one image's
+// group slice, and the tap coordinates for the padding mask.
+struct KTabEntry {
+    int32_t offset;
+    int32_t tap; // ky | (kx << 8); 31|31<<8 marks a padding entry (k >= K)
+};
+size_t conv_gemm_ktab_entries(const ConvGeom &g);
+void conv_gemm_fill_ktab(const ConvGeom &g, KTabEntry *host_tab);
+// n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
+int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1);
+
+// ---- depthwise (conv_depthwise.hip) ------------------------------------------
+bool depthwise_supported(const ConvGeom &g);
+int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
+
+// ---- Winograd F(2x2,3x3) (conv_winograd.hip) ---------------------------------
+struct WinoPlan {
+    int chunk_imgs;  // images transformed and multiplied per pass
+    int tcap;        // tiles per pass = row stride of the V and M workspace matrices
+    size_t ws_bytes; // workspace() of the op
+    ConvGeom gemm;   // grouped 1x1 geometry that runs the 16 GEMMs of a pass
+};
+bool winograd_supported(const ConvGeom &g);
+WinoPlan winograd_plan(const ConvGeom &g); // g.B = batch hint
+int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *gemm_ktab, const void *x, const void *w, void *y,
+                    void *ws, size_t ws_bytes, const Epilogue &ep, hipStream_t stream);
+
+// ---- InnerProduct GEMM (ip_gemm.hip) ------------------------------------------
+ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype);
+
+} // namespace dlp

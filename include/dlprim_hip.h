@@ -1,0 +1,124 @@
+/*
+ * dlprim_hip.h -- C ABI of the MI355X (gfx950) convolution forward path.
+ *
+ * This is the boundary a dlprimitives build binds in place of its OpenCL
+ * context / program-cache / kernel plumbing for Conv2DForward and IPForward.
+ * Plain C: pointers, sizes and ints only.  Device pointers are ordinary HIP
+ * device addresses, already advanced by the tensor's element offset.
+ *
+ * Every call returns DLP_OK or an error code; dlp_last_error() gives the
+ * thread-local message (the C++ header layer in include/dlprim/ turns codes
+ * back into dlprim::ValidationError / NotImplementedError exceptions).
+ *
+ * Citations (file:line) name the dlprimitives interface each entry replaces.
+ */
+#ifndef DLPRIM_HIP_H
+#define DLPRIM_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLP_OK 0
+#define DLP_ERR_VALIDATION 1      /* dlprim::ValidationError, include/dlprim/definitions.hpp:54-60 */
+#define DLP_ERR_NOT_IMPLEMENTED 2 /* dlprim::NotImplementedError, include/dlprim/definitions.hpp:46-52 */
+#define DLP_ERR_RUNTIME 3         /* HIP runtime failure (the reference raises cl::Error) */
+
+/* dlprim::DataType, include/dlprim/definitions.hpp:78-94 (same numeric values) */
+#define DLP_FLOAT 3
+#define DLP_HALF 2
+#define DLP_BFLOAT16 10
+
+/* dlprim::StandardActivations, include/dlprim/definitions.hpp:278-284 */
+#define DLP_ACT_IDENTITY 0
+#define DLP_ACT_RELU 1
+#define DLP_ACT_TANH 2
+#define DLP_ACT_SIGMOID 3
+#define DLP_ACT_RELU6 4
+
+/* core::Conv2DSettings = Convolution2DConfigBase + input shape + dtype,
+ * include/dlprim/definitions.hpp:313-321, include/dlprim/core/conv.hpp:17-28.
+ * shape[0] (batch) is a hint used for kernel selection, not a requirement. */
+typedef struct dlp_conv2d_settings {
+    int channels_in;
+    int channels_out;
+    int kernel[2];
+    int stride[2];
+    int dilate[2];
+    int pad[2];
+    int groups;
+    int shape[4];
+    int dtype;
+} dlp_conv2d_settings;
+
+/* core::IPSettings, include/dlprim/core/ip.hpp:19-24 */
+typedef struct dlp_ip_settings {
+    int inputs;
+    int outputs;
+    int optimal_batch_size;
+    int dtype;
+} dlp_ip_settings;
+
+typedef struct dlp_conv2d_fwd dlp_conv2d_fwd; /* core::Conv2DForward object */
+typedef struct dlp_ip_fwd dlp_ip_fwd;         /* core::IPForward object */
+
+/* Thread-local message of the last failing call on this thread. */
+const char *dlp_last_error(void);
+
+/* ABI version of this library (major*100 + minor). */
+int dlp_version(void);
+
+/* ---- device plumbing: replaces dlprim::Context / ExecutionContext / cl::Buffer
+ *      for this path (include/dlprim/context.hpp:128-299,309-431,
+ *      include/dlprim/tensor.hpp:106-294) ------------------------------------ */
+int dlp_device_count(int *count);
+int dlp_set_device(int device);
+int dlp_device_name(int device, char *buf, size_t buf_len);
+int dlp_malloc(void **dev_ptr, size_t bytes);
+int dlp_free(void *dev_ptr);
+int dlp_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, void *stream); /* Tensor::to_device */
+int dlp_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, void *stream); /* Tensor::to_host */
+int dlp_stream_create(void **stream);   /* ExecutionContext's in-order queue */
+int dlp_stream_sync(void *stream);      /* ExecutionContext::finish, context.hpp:216-220 */
+int dlp_stream_destroy(void *stream);
+
+/* ---- Conv2DBase::get_output_shape, src/core/conv.cpp:17-29 ------------------ */
+int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], int out_shape[4]);
+
+/* ---- core::Conv2DForward::create, include/dlprim/core/conv.hpp:49-53,
+ *      src/core/conv.cpp:704-729.  algo: NULL, "", "auto", "gemm", "winograd",
+ *      "depthwise_separable"; a requested but incompatible algorithm falls back
+ *      to "gemm" exactly as the reference does (:725-727). -------------------- */
+int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activation,
+                          const char *algo, dlp_conv2d_fwd **out);
+
+/* Conv2DBase::algo(), include/dlprim/core/conv.hpp:33 */
+const char *dlp_conv2d_fwd_algo(const dlp_conv2d_fwd *op);
+
+/* Conv2DBase::workspace() in bytes, include/dlprim/core/conv.hpp:34 */
+size_t dlp_conv2d_fwd_workspace(const dlp_conv2d_fwd *op);
+
+/* core::Conv2DForward::enqueue, include/dlprim/core/conv.hpp:48.
+ * x [B,Cin,H,W], w [Cout,Cin/groups,KH,KW], bias [Cout] or NULL (must match the
+ * `bias` flag given at create), y [B,Cout,OH,OW]; ws >= workspace() bytes;
+ * y = factor != 0 ? factor*y + act(conv+bias) : act(conv+bias).
+ * Asynchronous on `stream` (a hipStream_t, NULL = default stream). */
+int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4],
+                           const void *x, const void *w, const void *bias, void *y,
+                           void *ws, size_t ws_bytes, float factor, void *stream);
+
+void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
+
+/* ---- core::IPForward::create / enqueue, include/dlprim/core/ip.hpp:30-45,
+ *      src/core/ip.cpp:15-50: y[B,Out] = act(x[B,In] * w[Out,In]^T + bias[Out]) */
+int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_ip_fwd **out);
+int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w,
+                       const void *bias, void *y, void *stream);
+void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,255 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same
+seeded inputs.  fp32 bar: max-abs/rel 1e-4 (written as rtol=atol=1e-4 below);
+integer-valued inputs must match exactly."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conv_cases import REFERENCE_MATRIX, case, case_id, make_tensors, small_cases
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(rtol=1e-4, atol=1e-4)
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def cfg_of(orc, c):
+    return orc.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+
+
+def oracle_conv(orc, c, x, w, bias, threads=8):
+    return orc.conv2d_forward(x, w, bias, cfg_of(orc, c), c["activation"], threads=threads)
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import gpu_util
+
+    return gpu_util
+
+
+# ------------------------------------------------------------ implicit GEMM
+@pytest.mark.parametrize("c,bhw", small_cases(), ids=case_id)
+def test_gemm_reference_matrix(gpu, oracle_mod, c, bhw):
+    x, w, bias = make_tensors(c, bhw, seed=99)
+    print("case", case_id(c), bhw, flush=True)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+
+
+def test_config1_single_layer(gpu, oracle_mod):
+    # [16,64,56,56] * [64,64,3,3], s1 p1, bias, fused ReLU
+    c = case(3, 1, 1, 1, 64, 64, True, 1, True)
+    x, w, bias = make_tensors(c, (16, 56, 56), seed=1)
+    got, algo = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+    assert (got == 0).any() and (got > 0).any()  # the ReLU really cut something
+
+
+RESNET18_LAYERS = [  # (kernel, pad, stride, cin, cout, HW) -- the conv shapes of the ResNet-18 stack
+    (7, 3, 2, 3, 64, 224), (3, 1, 1, 64, 64, 56), (3, 1, 2, 64, 128, 56), (1, 0, 2, 64, 128, 56), (3, 1, 1, 128, 128, 28),
+    (3, 1, 2, 128, 256, 28), (1, 0, 2, 128, 256, 28), (3, 1, 1, 256, 256, 14), (3, 1, 2, 256, 512, 14),
+    (1, 0, 2, 256, 512, 14), (3, 1, 1, 512, 512, 7),
+]
+
+
+@pytest.mark.parametrize("layer", RESNET18_LAYERS, ids=lambda l: "k%d_s%d_%dto%d_at%d" % (l[0], l[2], l[3], l[4], l[5]))
+def test_resnet18_layer_shapes(gpu, oracle_mod, layer):
+    k, p, s, cin, cout, hw = layer
+    c = case(k, p, s, 1, cin, cout, True, 1, True)
+    batch = 2 if hw > 56 else 3
+    x, w, bias = make_tensors(c, (batch, hw, hw), seed=hw + cin)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm", batch_hint=64)
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+
+
+def test_gemm_integer_exact(gpu):
+    # integer-valued inputs: fp32 sums are exact in any order, so the MFMA result must
+    # EQUAL the integer result -- catches any indexing/layout slip that a tolerance could hide
+    rng = np.random.default_rng(7)
+    c = case(3, 1, 2, 1, 20, 70, True, 1, False)
+    x = np.round(rng.standard_normal((3, 20, 13, 17)) * 3).astype(np.float32)
+    w = np.round(rng.standard_normal((70, 20, 3, 3)) * 3).astype(np.float32)
+    bias = np.round(rng.standard_normal(70) * 3).astype(np.float32)
+    import torch
+
+    want = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(bias).double(),
+                                      stride=2, padding=1).numpy()
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm")
+    assert np.array_equal(got.astype(np.float64), want)
+
+
+@pytest.mark.parametrize("algo,c,bhw", [
+    ("gemm", case(3, 1, 1, 1, 16, 24, True, 1, True), (2, 11, 9)),
+    ("winograd", case(3, 1, 1, 1, 16, 24, True, 1, True), (2, 11, 9)),
+    ("depthwise_separable", case(3, 1, 1, 1, 24, 24, True, 24, True), (2, 11, 9)),
+    ("depthwise_separable", case(3, 1, 2, 1, 24, 24, True, 24, True), (2, 11, 9)),
+], ids=lambda v: v if isinstance(v, str) else None)
+def test_factor_contract(gpu, oracle_mod, algo, c, bhw):
+    # y = factor*y_old + act(conv + bias); activation applies to the new term only
+    x, w, bias = make_tensors(c, bhw, seed=5)
+    base, used = gpu.run_conv(c, x, w, bias, algo=algo, expect_algo=algo)
+    old = np.random.default_rng(1).standard_normal(base.shape).astype(np.float32)
+    got, _ = gpu.run_conv(c, x, w, bias, algo=algo, factor=0.5, y_init=old)
+    want = oracle_mod.apply_factor(oracle_conv(oracle_mod, c, x, w, bias), old, 0.5)
+    np.testing.assert_allclose(got, want, **TOL)
+
+
+@pytest.mark.parametrize("act", ["identity", "relu", "tanh", "sigmoid", "relu6"])
+def test_activations(gpu, oracle_mod, act):
+    c = case(3, 1, 1, 1, 8, 12, True, 1, False)
+    c["activation"] = act
+    x, w, bias = make_tensors(c, (2, 9, 9), seed=3)
+    w *= 6  # push values beyond the relu6 knee
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm")
+    np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
+
+
+def test_empty_batch_and_shape_errors(gpu):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    st = dlp.Conv2DSettings(4, 8, 3, 1, 1, 1, 1, (2, 4, 8, 8))
+    op = dlp.Conv2DForward.create(st, True, "relu", "gemm")
+    x = torch.zeros((0, 4, 8, 8), device="cuda:0")
+    w = torch.zeros((8, 4, 3, 3), device="cuda:0")
+    b = torch.zeros(8, device="cuda:0")
+    y = torch.zeros((0, 8, 8, 8), device="cuda:0")
+    op.enqueue(x, w, b, y)  # empty batch is a no-op
+    with pytest.raises(dlp.ValidationError):  # bias flag mismatch (src/gemm.cpp:526-533)
+        op.enqueue(torch.zeros((1, 4, 8, 8), device="cuda:0"), w, None, torch.zeros((1, 8, 8, 8), device="cuda:0"))
+    with pytest.raises(dlp.ValidationError):  # H/W changed without re-create
+        op.enqueue(torch.zeros((1, 4, 9, 8), device="cuda:0"), w, b, torch.zeros((1, 8, 9, 8), device="cuda:0"))
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------ algorithm choice
+def test_algorithm_selection_rules(gpu):
+    import dlprimitives_amd as dlp
+
+    def algo(c, hw, name):
+        st = gpu.settings_of(c, (2, c["cin"], hw, hw))
+        return dlp.Conv2DForward.create(st, False, "identity", name).algo()
+
+    c33 = case(3, 1, 1, 1, 16, 16, False, 1, False)
+    assert algo(c33, 8, "") == "winograd" and algo(c33, 8, "auto") == "winograd" and algo(c33, 8, "gemm") == "gemm"
+    assert algo(case(3, 1, 1, 1, 4, 16, False, 1, False), 8, "") == "gemm"  # < 8 channels: not recommended
+    assert algo(case(3, 1, 1, 1, 4, 16, False, 1, False), 8, "winograd") == "winograd"
+    assert algo(case(3, 1, 2, 1, 16, 16, False, 1, False), 8, "winograd") == "gemm"  # incompatible -> silent gemm
+    dw = case(3, 1, 1, 1, 16, 16, False, 16, False)
+    assert algo(dw, 8, "") == "depthwise_separable" and algo(dw, 8, "gemm") == "gemm"
+    assert algo(case(5, 2, 1, 1, 16, 16, False, 16, False), 8, "depthwise_separable") == "depthwise_separable"
+    assert algo(case(3, 0, 1, 1, 16, 16, False, 16, False), 8, "depthwise_separable") == "gemm"  # pad != k/2
+
+
+# ------------------------------------------------------------ Winograd
+@pytest.mark.parametrize("shape", [(2, 128, 128, 28, 28), (2, 256, 256, 14, 14), (3, 8, 16, 7, 9), (1, 16, 8, 1, 1), (2, 24, 40, 5, 6),
+                                   (5, 16, 16, 13, 13)],
+                         ids=lambda s: "b%d_c%d_n%d_%dx%d" % s)
+def test_winograd_three_way(gpu, oracle_mod, shape):
+    B, C, N, H, W = shape
+    c = case(3, 1, 1, 1, C, N, True, 1, True)
+    x, w, bias = make_tensors(c, (B, H, W), seed=C + H)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="winograd", expect_algo="winograd")
+    gemm, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    wino_cpu = oracle_mod.winograd_forward(x, w, bias, "relu")
+    direct = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, wino_cpu, **TOL)
+    np.testing.assert_allclose(got, direct, **TOL)
+    np.testing.assert_allclose(got, gemm, **TOL)
+
+
+def test_winograd_batch_larger_than_hint_is_chunked(gpu, oracle_mod):
+    c = case(3, 1, 1, 1, 16, 16, True, 1, False)
+    x, w, bias = make_tensors(c, (7, 10, 10), seed=2)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="winograd", expect_algo="winograd", batch_hint=2)
+    np.testing.assert_allclose(got, oracle_mod.winograd_forward(x, w, bias, "identity"), **TOL)
+
+
+# ------------------------------------------------------------ depthwise
+DW_SHAPES = [(144, 56), (192, 28), (384, 14), (960, 7)]
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("ch,hw", DW_SHAPES)
+def test_depthwise_mobilenet_shapes(gpu, oracle_mod, ch, hw, stride):
+    c = case(3, 1, stride, 1, ch, ch, True, ch, False)
+    c["activation"] = "relu6"
+    x, w, bias = make_tensors(c, (2, hw, hw), seed=ch)
+    w *= 4
+    got, _ = gpu.run_conv(c, x, w, bias, algo="depthwise_separable", expect_algo="depthwise_separable", batch_hint=64)
+    want = oracle_conv(oracle_mod, c, x, w, bias)  # reference semantics for stride 2: grouped GEMM conv
+    np.testing.assert_allclose(got, want, **TOL)
+    if stride == 1:
+        np.testing.assert_allclose(got, oracle_mod.depthwise_forward(x, w, bias, "relu6"), **TOL)
+    as_gemm, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    np.testing.assert_allclose(got, as_gemm, **TOL)
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 5, 9, 31), (3, 2, 5, 9, 31), (3, 1, 3, 1, 1), (3, 2, 6, 2, 3), (5, 1, 7, 12, 10), (7, 1, 4, 9, 9), (3, 1, 2, 70, 3),
+                                  (3, 2, 2, 3, 70)], ids=lambda g: "k%d_s%d_c%d_%dx%d" % g)
+def test_depthwise_odd_shapes(gpu, oracle_mod, geom):
+    k, s, ch, h, w_ = geom
+    c = case(k, k // 2, s, 1, ch, ch, True, ch, True)
+    x, w, bias = make_tensors(c, (3, h, w_), seed=h * w_)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="depthwise_separable", expect_algo="depthwise_separable")
+    np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
+
+
+# ------------------------------------------------------------ pointwise followers of the depthwise blocks
+@pytest.mark.parametrize("pw", [(144, 24, 56), (192, 64, 14), (960, 320, 7)], ids=lambda p: "%dto%d_at%d" % p)
+def test_pointwise_1x1(gpu, oracle_mod, pw):
+    cin, cout, hw = pw
+    c = case(1, 0, 1, 1, cin, cout, True, 1, False)
+    c["activation"] = "relu6"
+    x, w, bias = make_tensors(c, (2, hw, hw), seed=cin)
+    got, _ = gpu.run_conv(c, x, w, bias, expect_algo="gemm")
+    np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
+
+
+# ------------------------------------------------------------ InnerProduct
+def test_inner_product_reference_goldens(gpu):
+    doc = json.load(open(os.path.join(GOLDEN, "inner_product_fwd.json")))
+    n = 0
+    for t in doc["tests"]:
+        o = t["options"]
+        if not t["params"]:
+            continue
+        w = np.array(t["params"][0], dtype=np.float32).reshape(o["outputs"], o["inputs"])
+        bias = np.array(t["params"][1], dtype=np.float32) if o["bias"] else None
+        for cs in t["cases"]:
+            if "in" not in cs:
+                continue
+            x = np.array(cs["in"][0], dtype=np.float32).reshape(cs["in_shapes"][0])
+            want = np.array(cs["out"][0], dtype=np.float32).reshape(cs["out_shapes"][0])
+            np.testing.assert_allclose(gpu.run_ip(x, w, bias, o["activation"]), want, **TOL)
+            n += 1
+    assert n == 28
+
+
+@pytest.mark.parametrize("bio", [(128, 2048, 1000), (1, 512, 1000), (8, 1024, 1024), (50, 333, 77), (2, 1, 1)], ids=lambda v: "b%d_%dto%d" % v)
+@pytest.mark.parametrize("bias", [True, False])
+def test_inner_product_vs_oracle(gpu, oracle_mod, bio, bias):
+    B, I, O = bio
+    rng = np.random.default_rng(B + I)
+    x = rng.uniform(-1, 1, (B, I)).astype(np.float32)
+    w = (rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, O).astype(np.float32) if bias else None
+    np.testing.assert_allclose(gpu.run_ip(x, w, b, "relu"), oracle_mod.ip_forward(x, w, b, "relu"), **TOL)
+
+
+def test_inner_product_flattens_trailing_dims(gpu, oracle_mod):
+    # x may be rank > 2: inputs = size_no_batch (src/core/ip.cpp:30)
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, (4, 8, 3, 3)).astype(np.float32)
+    w = rng.standard_normal((10, 72)).astype(np.float32)
+    np.testing.assert_allclose(gpu.run_ip(x, w, None), oracle_mod.ip_forward(x, w, None), **TOL)
