@@ -12,17 +12,15 @@
 //    put on the MFMA column axis, so that the 32 lanes of a half-wave hold 32
 //    consecutive output pixels and every store is a 128-byte run in NCHW.
 //  * A (weights) and B (gathered input) tiles are staged through LDS in [k][m]
-//    and [k][n] order: an MFMA operand fetch is one conflict-free ds_read_b32.
-//  * all addressing of the gather is hoisted: per pixel a base offset and two
-//    bit masks (valid rows / valid columns of the window), per k a table entry
-//    (offset, tap) read through the scalar unit.  Out-of-window taps and tile
+//    and [k][n] order: an MFMA operand fetch is a conflict-free ds_read.
+//  * all addressing of the gather is hoisted: per pixel a base offset and a bit
+//    mask of the window taps that fall inside the image, per k a table entry
+//    (offset, tap bit) read through the scalar unit.  Out-of-window taps and tile
 //    tails are redirected to an out-of-range buffer offset, which the buffer
-//    load returns as 0.0 -- no divergent control flow in the main loop.
+//    load returns as 0.0 -- the main loop has no divergent control flow.
 //  * global loads of tile kt+1 are issued before the MFMAs of tile kt
 //    (register-staged double buffering, one barrier per K step).
 #include "dlp_internal.hpp"
-
-#include <vector>
 
 namespace dlp {
 
@@ -33,6 +31,14 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int BK = 16;
 constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
+
+// How the validity of a gathered tap is decided:
+//  MASK_NONE : every tap of every pixel is inside the image (pad 0 fits) -- only tile tails are masked
+//  MASK_TAPS : KH*KW <= 32, one bit per tap in a single per-pixel word
+//  MASK_ROWCOL: any kernel up to 31x31, separate row and column masks
+enum { MASK_NONE = 0, MASK_TAPS = 1, MASK_ROWCOL = 2 };
+// Epilogue flavour: clamp covers identity / relu / relu6 with two constants, no branches
+enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
 struct GemmArgs {
     const float *x;
@@ -47,14 +53,20 @@ struct GemmArgs {
     uint32_t x_bytes, w_bytes;
     float factor;
     int act;
+    float clamp_lo, clamp_hi;
 };
+
+typedef __attribute__((address_space(4))) KTabEntry KTabConst;
 
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
 {
+    // keep the offset a single opaque value: the select that produced it must stay a
+    // v_cndmask, not become two loads under divergent branches
+    asm volatile("" : "+v"(byte_off));
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -63,9 +75,9 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "tile shape");
     constexpr int LDA = BM + 2; // stride = 2 (mod 32): transposed A stores hit 32 distinct banks
     constexpr int LDB = BN;
-    constexpr int KSPLIT = kThreads / BN;   // k slices among the B loader threads
+    constexpr int KSPLIT = kThreads / BN;    // k slices among the B loader threads
     static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK % KSPLIT == 0, "B loader shape");
-    constexpr int B_LD = BK / KSPLIT;       // gathered elements per thread per K step
+    constexpr int B_LD = BK / KSPLIT;        // gathered elements per thread per K step (contiguous k)
     constexpr int A_LD = BM * BK / kThreads; // weight elements per thread per K step
 
     __shared__ float As[2][BK][LDA];
@@ -91,9 +103,9 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 
     // ---- per-thread gather state (one output pixel per thread) ----
     const int p = tid % BN;
-    const int ks = __builtin_amdgcn_readfirstlane(tid / BN);
+    const int ks = (KSPLIT == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid / BN);
     int base;
-    uint32_t my = 0, mx = 0;
+    uint32_t my = 0, mx = 0; // MASK_TAPS: my = tap mask; MASK_ROWCOL: row / column masks
     {
         const int n = n0 + p;
         const bool vn = n < a.N;
@@ -104,16 +116,29 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         const int iy0 = oy * a.sh - a.ph;
         const int ix0 = ox * a.sw - a.pw;
         base = ((b * a.Cin + g * a.Cin_g) * a.H + iy0) * a.W + ix0;
-        if (vn) {
+        if (MASK == MASK_NONE) {
+            // (base + offset)*4 lands in [2^31, 2^32) for every table offset: out of range
+            if (!vn)
+                base = 0x20000000;
+        } else if (vn) {
+            uint32_t ry = 0, rx = 0;
             for (int ky = 0; ky < a.KH; ky++) {
                 int yy = iy0 + ky * a.dh;
                 if (yy >= 0 && yy < a.H)
-                    my |= 1u << ky;
+                    ry |= 1u << ky;
             }
             for (int kx = 0; kx < a.KW; kx++) {
                 int xx = ix0 + kx * a.dw;
                 if (xx >= 0 && xx < a.W)
-                    mx |= 1u << kx;
+                    rx |= 1u << kx;
+            }
+            if (MASK == MASK_TAPS) {
+                for (int ky = 0; ky < a.KH; ky++)
+                    if ((ry >> ky) & 1u)
+                        my |= rx << (ky * a.KW);
+            } else {
+                my = ry;
+                mx = rx;
             }
         }
     }
@@ -132,17 +157,23 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 
     auto load_tiles = [&](int kt) {
         const int k0 = kt * BK;
+        const uint32_t kmask = (k0 + ak < a.K) ? 0u : kOutOfRange;
 #pragma unroll
-        for (int j = 0; j < A_LD; j++) {
-            uint32_t off = (k0 + ak < a.K) ? a_off[j] + (uint32_t)(k0 * 4) : kOutOfRange;
-            ra[j] = buf_load(wr, off);
-        }
+        for (int j = 0; j < A_LD; j++)
+            ra[j] = buf_load(wr, (a_off[j] + (uint32_t)(k0 * 4)) | kmask);
+        // the table is read-only for the whole launch and the index is wavefront-uniform:
+        // constant address space makes these scalar loads (s_load), off the vector path
+        const KTabConst *tab = (const KTabConst *)(a.ktab) + k0 + ks * B_LD;
 #pragma unroll
         for (int i = 0; i < B_LD; i++) {
-            const KTabEntry e = a.ktab[k0 + ks + i * KSPLIT];
-            const int ky = e.tap & 0xff, kx = e.tap >> 8;
-            const bool ok = ((my >> ky) & (mx >> kx) & 1u) != 0;
-            uint32_t off = ok ? (uint32_t)((base + e.offset) * 4) : kOutOfRange;
+            const KTabEntry e = {tab[i].offset, tab[i].tap};
+            uint32_t off = (uint32_t)((base + e.offset) * 4);
+            if (MASK == MASK_TAPS) {
+                off = (my & (uint32_t)e.tap) ? off : kOutOfRange;
+            } else if (MASK == MASK_ROWCOL) {
+                const int ky = e.tap & 0xff, kx = e.tap >> 8;
+                off = ((my >> ky) & (mx >> kx) & 1u) ? off : kOutOfRange;
+            }
             rb[i] = buf_load(xr, off);
         }
     };
@@ -152,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             As[buf][ak][am + 16 * j] = ra[j];
 #pragma unroll
         for (int i = 0; i < B_LD; i++)
-            Bs[buf][ks + i * KSPLIT][p] = rb[i];
+            Bs[buf][ks * B_LD + i][p] = rb[i];
     };
 
     f32x16 acc[TM][TN];
@@ -164,14 +195,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
 
-    load_tiles(0);
-    store_tiles(0);
-    __syncthreads();
-
-    for (int kt = 0; kt < a.nkt; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < a.nkt)
-            load_tiles(kt + 1);
+    auto compute = [&](int buf) {
 #pragma unroll
         for (int kk = 0; kk < BK / 2; kk++) {
             const int k = 2 * kk + h;
@@ -188,10 +212,19 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < a.nkt)
-            store_tiles(buf ^ 1);
+    };
+
+    load_tiles(0);
+    store_tiles(0);
+    __syncthreads();
+    for (int kt = 0; kt < a.nkt - 1; kt++) {
+        const int buf = kt & 1;
+        load_tiles(kt + 1);
+        compute(buf);
+        store_tiles(buf ^ 1);
         __syncthreads();
     }
+    compute((a.nkt - 1) & 1);
 
     // ---- epilogue: bias, activation, factor, NCHW store ----
     // accumulator register r of a 32x32 block holds row 8*(r/4) + 4*h + r%4, column l32
@@ -212,7 +245,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                     float v = acc[i][j][r];
                     if (a.bias)
                         v += a.bias[g * a.M + m];
-                    v = apply_act(v, a.act);
+                    if (ACT == ACT_CLAMP) {
+                        if (a.act != DLP_ACT_IDENTITY) // identity must keep NaNs: no min/max
+                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                    } else
+                        v = apply_act(v, a.act);
                     store_out(yb + (size_t)m * a.OHW, v, a.factor);
                 }
             }
@@ -220,17 +257,48 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     }
 }
 
-template <int BM, int BN, int WM, int WN>
-int launch_cfg(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+template <int BM, int BN, int WM, int WN, int MASK, int ACT>
+int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 {
     a.mtiles = (a.M + BM - 1) / BM;
     a.ntiles = (a.N + BN - 1) / BN;
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
-    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_tile(const ConvGeom &g, GemmArgs &a, int mask, int act, hipStream_t stream)
+{
+    if (act == ACT_CLAMP) {
+        if (mask == MASK_NONE)
+            return launch_inst<BM, BN, WM, WN, MASK_NONE, ACT_CLAMP>(g, a, stream);
+        if (mask == MASK_TAPS)
+            return launch_inst<BM, BN, WM, WN, MASK_TAPS, ACT_CLAMP>(g, a, stream);
+        return launch_inst<BM, BN, WM, WN, MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
+    }
+    // tanh / sigmoid: rare, one generic instantiation per tile
+    return launch_inst<BM, BN, WM, WN, MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
+}
+
+bool generic_act(int activation) { return activation == DLP_ACT_TANH || activation == DLP_ACT_SIGMOID; }
+
+int mask_mode(const ConvGeom &g, int activation)
+{
+    if (generic_act(activation))
+        return MASK_ROWCOL; // the rare activations share one instantiation per tile
+    // no tap can fall outside the image (no padding, last window fits) and no K tail
+    const bool fits_h = g.ph == 0 && (g.OH - 1) * g.sh + (g.KH - 1) * g.dh < g.H;
+    const bool fits_w = g.pw == 0 && (g.OW - 1) * g.sw + (g.KW - 1) * g.dw < g.W;
+    const int K = (g.Cin / g.groups) * g.KH * g.KW;
+    if (fits_h && fits_w && K % BK == 0)
+        return MASK_NONE;
+    if (g.KH * g.KW <= 32)
+        return MASK_TAPS;
+    return MASK_ROWCOL;
 }
 
 } // namespace
@@ -241,23 +309,23 @@ size_t conv_gemm_ktab_entries(const ConvGeom &g)
     return (K + BK - 1) / BK * BK;
 }
 
-void conv_gemm_fill_ktab(const ConvGeom &g, KTabEntry *tab)
+void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab)
 {
     const int cin_g = g.Cin / g.groups;
-    const size_t K = (size_t)cin_g * g.KH * g.KW;
     const size_t Kp = conv_gemm_ktab_entries(g);
+    const int mode = mask_mode(g, activation);
     size_t k = 0;
     for (int c = 0; c < cin_g; c++)
         for (int ky = 0; ky < g.KH; ky++)
             for (int kx = 0; kx < g.KW; kx++, k++) {
                 tab[k].offset = (c * g.H + ky * g.dh) * g.W + kx * g.dw;
-                tab[k].tap = ky | (kx << 8);
+                tab[k].tap = (mode == MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << ((ky * g.KW + kx) & 31));
             }
     for (; k < Kp; k++) {
+        // padding rows of the last K tile: never valid (MASK_NONE has no K tail)
         tab[k].offset = 0;
-        tab[k].tap = 31 | (31 << 8); // bit 31 of the masks is never set
+        tab[k].tap = (mode == MASK_ROWCOL) ? (31 | (31 << 8)) : 0;
     }
-    (void)K;
 }
 
 int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
@@ -269,7 +337,7 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     const size_t x_elems = (size_t)g.B * g.Cin * g.H * g.W;
     const size_t w_elems = (size_t)g.Cout * (g.Cin / g.groups) * g.KH * g.KW;
     const size_t y_elems = (size_t)g.B * g.Cout * g.OH * g.OW;
-    if (x_elems * 4 >= kOutOfRange || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
+    if (x_elems * 4 >= 0x20000000ULL * 4 || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
@@ -301,12 +369,20 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     a.w_bytes = (uint32_t)(w_elems * 4);
     a.factor = ep.factor;
     a.act = ep.activation;
+    a.clamp_lo = -__builtin_huge_valf();
+    a.clamp_hi = __builtin_huge_valf();
+    if (ep.activation == DLP_ACT_RELU || ep.activation == DLP_ACT_RELU6)
+        a.clamp_lo = 0.0f;
+    if (ep.activation == DLP_ACT_RELU6)
+        a.clamp_hi = 6.0f;
+    const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
+    const int mask = mask_mode(g, ep.activation); // same rule the gather table was built with
 
     if (a.M > 64)
-        return launch_cfg<128, 128, 2, 2>(g, a, stream);
+        return launch_tile<128, 128, 2, 2>(g, a, mask, act, stream);
     if (a.M > 32)
-        return launch_cfg<64, 256, 1, 4>(g, a, stream);
-    return launch_cfg<32, 256, 1, 4>(g, a, stream);
+        return launch_tile<64, 256, 1, 4>(g, a, mask, act, stream);
+    return launch_tile<32, 256, 1, 4>(g, a, mask, act, stream);
 }
 
 } // namespace dlp

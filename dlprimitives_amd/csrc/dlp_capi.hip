@@ -47,11 +47,11 @@ struct dlp_ip_fwd {
     KTabEntry *ktab;
 };
 
-static int upload_ktab(const ConvGeom &g, KTabEntry **out)
+static int upload_ktab(const ConvGeom &g, int activation, KTabEntry **out)
 {
     const size_t n = conv_gemm_ktab_entries(g);
     std::vector<KTabEntry> host(n ? n : 1);
-    conv_gemm_fill_ktab(g, host.data());
+    conv_gemm_fill_ktab(g, activation, host.data());
     KTabEntry *dev = nullptr;
     DLP_HIP_TRY(hipMalloc((void **)&dev, host.size() * sizeof(KTabEntry)));
     hipError_t e = hipMemcpy(dev, host.data(), host.size() * sizeof(KTabEntry), hipMemcpyHostToDevice);
@@ -240,11 +240,11 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
-        rc = upload_ktab(g, &op->ktab);
+        rc = upload_ktab(g, activation, &op->ktab);
     } else if (chosen == ALGO_WINOGRAD) {
         op->wino = winograd_plan(g);
         op->workspace = op->wino.ws_bytes;
-        rc = upload_ktab(op->wino.gemm, &op->ktab);
+        rc = upload_ktab(op->wino.gemm, DLP_ACT_IDENTITY, &op->ktab);
     }
     if (rc != DLP_OK) {
         delete op;
@@ -329,7 +329,7 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
     op->ktab = nullptr;
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
-    int rc = upload_ktab(ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype), &op->ktab);
+    int rc = upload_ktab(ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype), activation, &op->ktab);
     if (rc != DLP_OK) {
         delete op;
         return rc;

@@ -73,10 +73,11 @@ __device__ __forceinline__ void store_out(float *p, float v, float factor)
 // group slice, and the tap coordinates for the padding mask.
 struct KTabEntry {
     int32_t offset;
-    int32_t tap; // ky | (kx << 8); 31|31<<8 marks a padding entry (k >= K)
+    int32_t tap; // tap bit (1 << (ky*KW+kx)), or ky | (kx << 8) for large kernels; padding entries never match
 };
 size_t conv_gemm_ktab_entries(const ConvGeom &g);
-void conv_gemm_fill_ktab(const ConvGeom &g, KTabEntry *host_tab);
+// The table layout depends on the geometry AND on the activation the op was created with.
+void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *host_tab);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
                      void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1);
