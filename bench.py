@@ -93,6 +93,7 @@ def main():
     ap.add_argument("--algo", default="gemm")
     ap.add_argument("--cpu-images", type=int, default=4, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
+    ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over batch with no exchange)" % args.gpus,
@@ -109,6 +110,11 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     layers = build_layers(args.batch, 2024, args.algo)
+    if args.only:
+        layers = [e for e in layers if args.only in e["layer"]["name"]]
+        if not layers:
+            print("bench.py: --only matches no layer", file=sys.stderr)
+            sys.exit(2)
     stream = torch.cuda.current_stream()
 
     def step():
@@ -177,7 +183,8 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "ResNet-18 conv stack forward: 20 convs, fp32 NCHW, batch %d, BN folded, fused ReLU, algo %s" % (args.batch, args.algo),
+        "config": {"workload": "ResNet-18 conv stack forward: %d convs%s, fp32 NCHW, batch %d, BN folded, fused ReLU, algo %s" %
+                   (nl, " (subset --only %s)" % args.only if args.only else "", args.batch, args.algo),
                    "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1)},
         "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_fp32_matrix_peak": round(total_flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),

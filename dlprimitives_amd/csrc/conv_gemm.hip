@@ -22,6 +22,8 @@
 //    (register-staged double buffering, one barrier per K step).
 #include "dlp_internal.hpp"
 
+#include <type_traits>
+
 namespace dlp {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -62,13 +64,42 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byt
 {
     // keep the offset a single opaque value: the select that produced it must stay a
     // v_cndmask, not become two loads under divergent branches
-    asm volatile("" : "+v"(byte_off));
+    asm("" : "+v"(byte_off));
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+
+// call f(integral_constant<int, kk>) for the compile-time value matching the runtime-unrolled kk
+template <class F>
+__device__ __forceinline__ void static_for_slice(int kk, F &&f)
+{
+    switch (kk) {
+    case 0: f(std::integral_constant<int, 0>{}); break;
+    case 1: f(std::integral_constant<int, 1>{}); break;
+    case 2: f(std::integral_constant<int, 2>{}); break;
+    case 3: f(std::integral_constant<int, 3>{}); break;
+    case 4: f(std::integral_constant<int, 4>{}); break;
+    case 5: f(std::integral_constant<int, 5>{}); break;
+    case 6: f(std::integral_constant<int, 6>{}); break;
+    default: f(std::integral_constant<int, 7>{}); break;
+    }
+}
+template <class F>
+__device__ __forceinline__ void static_for_all(F &&f)
+{
+    f(std::integral_constant<int, 0>{});
+    f(std::integral_constant<int, 1>{});
+    f(std::integral_constant<int, 2>{});
+    f(std::integral_constant<int, 3>{});
+    f(std::integral_constant<int, 4>{});
+    f(std::integral_constant<int, 5>{});
+    f(std::integral_constant<int, 6>{});
+    f(std::integral_constant<int, 7>{});
 }
 
 template <int BM, int BN, int WM, int WN, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 {
+    static_assert(BK == 16, "the slice helpers assume 8 MFMA steps per K tile");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
     constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA blocks per wavefront
@@ -153,19 +184,30 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         a_off[j] = (m < a.M) ? (uint32_t)(((g * a.M + m) * a.K + ak) * 4) : kOutOfRange;
     }
 
-    float ra[A_LD], rb[B_LD];
+    // Two register sets for staged tiles: tile kt+2 is being fetched from memory
+    // into one set while tile kt+1 moves from the other set into LDS and tile kt
+    // (already in LDS) feeds the matrix cores.  A global load therefore has a whole
+    // K step to land before anything waits on it.
+    float ra[2][A_LD], rb[2][B_LD];
 
-    auto load_tiles = [&](int kt) {
+    // one slice of the loads of tile kt into register set S: called once per MFMA
+    // group so that address arithmetic and vector-memory issue hide under MFMAs
+    auto load_slice = [&](auto set, int kt, auto slice) {
+        constexpr int S = decltype(set)::value;
+        constexpr int Q = decltype(slice)::value;
         const int k0 = kt * BK;
         const uint32_t kmask = (k0 + ak < a.K) ? 0u : kOutOfRange;
 #pragma unroll
         for (int j = 0; j < A_LD; j++)
-            ra[j] = buf_load(wr, (a_off[j] + (uint32_t)(k0 * 4)) | kmask);
+            if (j % (BK / 2) == Q)
+                ra[S][j] = buf_load(wr, (a_off[j] + (uint32_t)(k0 * 4)) | kmask);
         // the table is read-only for the whole launch and the index is wavefront-uniform:
         // constant address space makes these scalar loads (s_load), off the vector path
         const KTabConst *tab = (const KTabConst *)(a.ktab) + k0 + ks * B_LD;
 #pragma unroll
         for (int i = 0; i < B_LD; i++) {
+            if (i % (BK / 2) != Q)
+                continue;
             const KTabEntry e = {tab[i].offset, tab[i].tap};
             uint32_t off = (uint32_t)((base + e.offset) * 4);
             if (MASK == MASK_TAPS) {
@@ -174,16 +216,20 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 const int ky = e.tap & 0xff, kx = e.tap >> 8;
                 off = ((my >> ky) & (mx >> kx) & 1u) ? off : kOutOfRange;
             }
-            rb[i] = buf_load(xr, off);
+            rb[S][i] = buf_load(xr, off);
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_slice = [&](auto set, int buf, auto slice) {
+        constexpr int S = decltype(set)::value;
+        constexpr int Q = decltype(slice)::value;
 #pragma unroll
         for (int j = 0; j < A_LD; j++)
-            As[buf][ak][am + 16 * j] = ra[j];
+            if (j % (BK / 2) == Q)
+                As[buf][ak][am + 16 * j] = ra[S][j];
 #pragma unroll
         for (int i = 0; i < B_LD; i++)
-            Bs[buf][ks * B_LD + i][p] = rb[i];
+            if (i % (BK / 2) == Q)
+                Bs[buf][ks * B_LD + i][p] = rb[S][i];
     };
 
     f32x16 acc[TM][TN];
@@ -195,36 +241,53 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
 
-    auto compute = [&](int buf) {
+    float fa[2][TM], fb[2][TN]; // MFMA operands, double buffered across the kk steps
+    auto read_operands = [&](int buf, int kk, int slot) {
+        const int k = 2 * kk + h;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            fa[slot][i] = As[buf][k][wm * WTM + i * 32 + l32];
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+            fb[slot][j] = Bs[buf][k][wn * WTN + j * 32 + l32];
+    };
+
+    // One K step: MFMAs of tile kt (in LDS[buf]); register set SN (tile kt+1) goes to
+    // LDS[buf^1]; tile kt+2 is fetched into register set SL.  Operands of step kk+1
+    // are read from LDS before the MFMAs of step kk are issued.
+    auto k_step = [&](auto set_next, auto set_load, int kt) {
+        const int buf = kt & 1;
+        read_operands(buf, 0, 0);
 #pragma unroll
         for (int kk = 0; kk < BK / 2; kk++) {
-            const int k = 2 * kk + h;
-            float fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                fa[i] = As[buf][k][wm * WTM + i * 32 + l32];
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                fb[j] = Bs[buf][k][wn * WTN + j * 32 + l32];
+            const int cur = kk & 1;
+            if (kk + 1 < BK / 2)
+                read_operands(buf, kk + 1, cur ^ 1);
+            static_for_slice(kk, [&](auto q) {
+                store_slice(set_next, buf ^ 1, q);
+                load_slice(set_load, kt + 2, q);
+            });
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
         }
+        __syncthreads();
     };
 
-    load_tiles(0);
-    store_tiles(0);
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    // prologue: tile 0 -> set 0 -> LDS[0]; tile 1 -> set 1
+    static_for_all([&](auto q) { load_slice(I0{}, 0, q); });
+    static_for_all([&](auto q) { load_slice(I1{}, 1, q); });
+    static_for_all([&](auto q) { store_slice(I0{}, 0, q); });
     __syncthreads();
-    for (int kt = 0; kt < a.nkt - 1; kt++) {
-        const int buf = kt & 1;
-        load_tiles(kt + 1);
-        compute(buf);
-        store_tiles(buf ^ 1);
-        __syncthreads();
+    // nkt is even (the host rounds it up; tiles past K load zeros through the masks)
+    for (int kt = 0; kt < a.nkt; kt += 2) {
+        k_step(I1{}, I0{}, kt);
+        k_step(I0{}, I1{}, kt + 1);
     }
-    compute((a.nkt - 1) & 1);
 
     // ---- epilogue: bias, activation, factor, NCHW store ----
     // accumulator register r of a 32x32 block holds row 8*(r/4) + 4*h + r%4, column l32
@@ -305,8 +368,12 @@ int mask_mode(const ConvGeom &g, int activation)
 
 size_t conv_gemm_ktab_entries(const ConvGeom &g)
 {
+    // K tiles rounded up to an even count, plus two tiles of never-valid entries that
+    // the software pipeline prefetches past the end
     size_t K = (size_t)(g.Cin / g.groups) * g.KH * g.KW;
-    return (K + BK - 1) / BK * BK;
+    size_t tiles = (K + BK - 1) / BK;
+    tiles = (tiles + 1) / 2 * 2 + 2;
+    return tiles * BK;
 }
 
 void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab)
@@ -355,7 +422,7 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     if (a.N == 0)
         return DLP_OK;
     a.K = (g.Cin / g.groups) * g.KH * g.KW;
-    a.nkt = (a.K + BK - 1) / BK;
+    a.nkt = ((a.K + BK - 1) / BK + 1) / 2 * 2;
     a.Cin = g.Cin;
     a.Cin_g = g.Cin / g.groups;
     a.H = g.H;
