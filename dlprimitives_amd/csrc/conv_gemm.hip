@@ -50,7 +50,9 @@ struct GemmArgs {
     const KTabEntry *ktab;
     int M, N, K, nkt;
     int mtiles, ntiles;
-    int Cin, Cin_g, H, W, Cout, OW, OHW;
+    int splitk, kt_per_slice; // K tiles are dealt to `splitk` slices of kt_per_slice (even) tiles
+    float *part;              // split-K partial sums [slice][Cout][N]
+    int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, w_bytes;
     float factor;
@@ -126,8 +128,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     const int mt = t % a.mtiles;
     t /= a.mtiles;
     const int nt = t % a.ntiles;
-    const int g = t / a.ntiles;
+    t /= a.ntiles;
+    const int g = t % a.groups;
+    const int slice = t / a.groups;
     const int m0 = mt * BM, n0 = nt * BN;
+    const int kt_begin = slice * a.kt_per_slice;
+    const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
@@ -278,15 +284,36 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
-    // prologue: tile 0 -> set 0 -> LDS[0]; tile 1 -> set 1
-    static_for_all([&](auto q) { load_slice(I0{}, 0, q); });
-    static_for_all([&](auto q) { load_slice(I1{}, 1, q); });
+    // prologue: first tile -> set 0 -> LDS[0]; second tile -> set 1
+    static_for_all([&](auto q) { load_slice(I0{}, kt_begin, q); });
+    static_for_all([&](auto q) { load_slice(I1{}, kt_begin + 1, q); });
     static_for_all([&](auto q) { store_slice(I0{}, 0, q); });
     __syncthreads();
-    // nkt is even (the host rounds it up; tiles past K load zeros through the masks)
-    for (int kt = 0; kt < a.nkt; kt += 2) {
+    // tile counts are even (the host rounds up; tiles past K load zeros through the masks)
+    for (int kt = kt_begin; kt < kt_end; kt += 2) {
         k_step(I1{}, I0{}, kt);
         k_step(I0{}, I1{}, kt + 1);
+    }
+
+    // ---- split-K: raw partial sums to the workspace, reduced by a second kernel ----
+    if (a.splitk > 1) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            if (n >= a.N)
+                continue;
+            float *pb = a.part + ((size_t)slice * a.Cout + (size_t)g * a.M) * a.N + n;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < a.M)
+                        pb[(size_t)m * a.N] = acc[i][j][r];
+                }
+            }
+        }
+        return;
     }
 
     // ---- epilogue: bias, activation, factor, NCHW store ----
@@ -320,22 +347,86 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     }
 }
 
-template <int BM, int BN, int WM, int WN, int MASK, int ACT>
-int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+// Sums the split-K slices in slice order (deterministic) and applies the epilogue.
+template <int ACT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; // row * N + n
+    const long long total = (long long)a.Cout * a.N;
+    if (idx >= total)
+        return;
+    const int row = (int)(idx / a.N);
+    const int n = (int)(idx - (long long)row * a.N);
+    float v = 0.0f;
+    for (int s = 0; s < a.splitk; s++)
+        v += a.part[(size_t)s * total + idx];
+    if (a.bias)
+        v += a.bias[row];
+    if (ACT == ACT_CLAMP) {
+        if (a.act != DLP_ACT_IDENTITY)
+            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+    } else
+        v = apply_act(v, a.act);
+    const int b = n / a.OHW;
+    const int pix = n - b * a.OHW;
+    store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, v, a.factor);
+}
+
+// Split-K factor for a launch of `tiles` output tiles over `nkt` (even) K tiles.
+// Workgroups of one launch are co-resident, so the time is set by the busiest CU:
+// pick the factor that fills whole rounds of the 256 CUs best, keeping at least
+// 8 K tiles per slice; 1 = no split.
+int choose_splitk(long long tiles, int nkt)
+{
+    const int kCUs = 256;
+    if (tiles >= 2 * kCUs || nkt < 16)
+        return 1;
+    int best = 1;
+    double best_eff = (double)tiles / (double)(((tiles + kCUs - 1) / kCUs) * kCUs);
+    for (int s = 2; s <= 8; s++) {
+        if (nkt / s < 8)
+            break;
+        const long long blocks = tiles * s;
+        const double eff = (double)blocks / (double)(((blocks + kCUs - 1) / kCUs) * kCUs);
+        if (eff > best_eff + 0.05) {
+            best_eff = eff;
+            best = s;
+        }
+    }
+    return best;
+}
+
+template <int BM, int BN>
+void plan_split(GemmArgs &a, int groups, size_t ws_bytes)
 {
     a.mtiles = (a.M + BM - 1) / BM;
     a.ntiles = (a.N + BN - 1) / BN;
-    long long blocks = (long long)a.mtiles * a.ntiles * g.groups;
+    int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt);
+    if (s > 1 && (a.part == nullptr || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
+        s = 1; // no (or too small a) workspace: run unsplit
+    a.splitk = s;
+    a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;
+}
+
+template <int BM, int BN, int WM, int WN, int MASK, int ACT>
+int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+{
+    long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    if (a.splitk > 1) {
+        const long long total = (long long)a.Cout * a.N;
+        hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
 
 template <int BM, int BN, int WM, int WN>
-int launch_tile(const ConvGeom &g, GemmArgs &a, int mask, int act, hipStream_t stream)
+int launch_tile(const ConvGeom &g, GemmArgs &a, int mask, int act, size_t ws_bytes, hipStream_t stream)
 {
+    plan_split<BM, BN>(a, g.groups, ws_bytes);
     if (act == ACT_CLAMP) {
         if (mask == MASK_NONE)
             return launch_inst<BM, BN, WM, WN, MASK_NONE, ACT_CLAMP>(g, a, stream);
@@ -395,8 +486,28 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab)
     }
 }
 
+// Workspace the split-K path wants for this geometry (0 when it would not split).
+size_t conv_gemm_workspace_bytes(const ConvGeom &g)
+{
+    if (g.B <= 0)
+        return 0;
+    GemmArgs a;
+    a.M = g.Cout / g.groups;
+    a.N = g.B * g.OH * g.OW;
+    a.Cout = g.Cout;
+    a.nkt = (((g.Cin / g.groups) * g.KH * g.KW + BK - 1) / BK + 1) / 2 * 2;
+    a.part = (float *)16; // any non-null value: ask for the unconstrained plan
+    if (a.M > 64)
+        plan_split<128, 128>(a, g.groups, (size_t)-1);
+    else if (a.M > 32)
+        plan_split<64, 256>(a, g.groups, (size_t)-1);
+    else
+        plan_split<32, 256>(a, g.groups, (size_t)-1);
+    return a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0;
+}
+
 int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid)
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *ws, size_t ws_bytes)
 {
     if (g.dtype != DLP_FLOAT)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: only float_data is implemented");
@@ -428,6 +539,8 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     a.H = g.H;
     a.W = g.W;
     a.Cout = g.Cout;
+    a.groups = g.groups;
+    a.part = (float *)ws;
     a.OW = g.OW;
     a.OHW = g.OH * g.OW;
     a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw; a.dh = g.dh; a.dw = g.dw;
@@ -446,10 +559,10 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     const int mask = mask_mode(g, ep.activation); // same rule the gather table was built with
 
     if (a.M > 64)
-        return launch_tile<128, 128, 2, 2>(g, a, mask, act, stream);
+        return launch_tile<128, 128, 2, 2>(g, a, mask, act, ws_bytes, stream);
     if (a.M > 32)
-        return launch_tile<64, 256, 1, 4>(g, a, mask, act, stream);
-    return launch_tile<32, 256, 1, 4>(g, a, mask, act, stream);
+        return launch_tile<64, 256, 1, 4>(g, a, mask, act, ws_bytes, stream);
+    return launch_tile<32, 256, 1, 4>(g, a, mask, act, ws_bytes, stream);
 }
 
 } // namespace dlp

@@ -240,6 +240,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
+        op->workspace = conv_gemm_workspace_bytes(g);
         rc = upload_ktab(g, activation, &op->ktab);
     } else if (chosen == ALGO_WINOGRAD) {
         op->wino = winograd_plan(g);
@@ -299,7 +300,7 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
     case ALGO_DEPTHWISE:
         return depthwise_launch(g, x, w, y, ep, s);
     default:
-        return conv_gemm_launch(g, op->ktab, x, w, y, ep, s);
+        return conv_gemm_launch(g, op->ktab, x, w, y, ep, s, -1, ws, ws_bytes);
     }
 }
 

@@ -78,9 +78,14 @@ struct KTabEntry {
 size_t conv_gemm_ktab_entries(const ConvGeom &g);
 // The table layout depends on the geometry AND on the activation the op was created with.
 void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *host_tab);
+// Workspace (bytes) with which the launch may split the K dimension over several
+// workgroups when there are too few output tiles to fill the chip; 0 = never splits.
+size_t conv_gemm_workspace_bytes(const ConvGeom &g);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
+// ws/ws_bytes: optional split-K workspace; without it the launch runs unsplit.
 int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1);
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *ws = nullptr,
+                     size_t ws_bytes = 0);
 
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);

@@ -1,0 +1,99 @@
+// Device peak probes used only to put the roofline numbers in context:
+// an MFMA-only loop (no memory traffic) and a streaming copy.  Not part of the
+// operator ABI; built as a separate library, libdlp_microbench.so.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma_f32_loop(float *out, int iters, float a0, float b0)
+{
+    f32x16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    float a = a0 + threadIdx.x, b = b0;
+    for (int i = 0; i < iters; i++) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c3, 0, 0, 0);
+    }
+    float s = 0;
+    for (int r = 0; r < 16; r++)
+        s += c0[r] + c1[r] + c2[r] + c3[r];
+    if (s == 12345.678f) // never true: keeps the result alive without a store per thread
+        out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride)
+        dst[i] = src[i];
+}
+
+static float time_ms(hipStream_t s, hipEvent_t e0, hipEvent_t e1)
+{
+    float ms = 0;
+    hipEventSynchronize(e1);
+    hipEventElapsedTime(&ms, e0, e1);
+    (void)s;
+    return ms;
+}
+
+extern "C" {
+
+// fp32 MFMA throughput in TFLOP/s with `waves_per_simd` wavefronts resident per SIMD.
+int dlp_probe_mfma_f32(int waves_per_simd, double *tflops)
+{
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess)
+        return 1;
+    const int cus = prop.multiProcessorCount;
+    const int blocks = cus * waves_per_simd; // 256 threads = 4 waves = one per SIMD
+    const int iters = 20000;
+    float *out = nullptr;
+    if (hipMalloc(&out, (size_t)blocks * 256 * 4) != hipSuccess)
+        return 1;
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    mfma_f32_loop<<<blocks, 256>>>(out, 1000, 1.0f, 2.0f);
+    hipEventRecord(e0, 0);
+    mfma_f32_loop<<<blocks, 256>>>(out, iters, 1.0f, 2.0f);
+    hipEventRecord(e1, 0);
+    float ms = time_ms(0, e0, e1);
+    double flops = (double)blocks * 4 /*waves*/ * iters * 4 /*mfma*/ * 4096.0;
+    *tflops = flops / (ms * 1e-3) / 1e12;
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    hipFree(out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// streaming copy bandwidth in GB/s (read + write bytes) over `mbytes` MiB per direction.
+int dlp_probe_copy(int mbytes, double *gbs)
+{
+    size_t bytes = (size_t)mbytes << 20;
+    float4 *a = nullptr, *b = nullptr;
+    if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess)
+        return 1;
+    hipMemset(a, 1, bytes);
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    size_t n = bytes / 16;
+    copy_f4<<<256 * 16, 256>>>(a, b, n);
+    hipEventRecord(e0, 0);
+    const int reps = 10;
+    for (int r = 0; r < reps; r++)
+        copy_f4<<<256 * 16, 256>>>(a, b, n);
+    hipEventRecord(e1, 0);
+    float ms = time_ms(0, e0, e1);
+    *gbs = 2.0 * bytes * reps / (ms * 1e-3) / 1e9;
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    hipFree(a);
+    hipFree(b);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+}

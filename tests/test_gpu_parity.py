@@ -71,6 +71,32 @@ def test_resnet18_layer_shapes(gpu, oracle_mod, layer):
     np.testing.assert_allclose(got, want, **TOL)
 
 
+def test_split_k_with_and_without_workspace(gpu, oracle_mod):
+    # few output tiles, long K: the launch splits K over several workgroups when it is
+    # given workspace() bytes, and must give the same answer unsplit when it is not
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    c = case(3, 1, 1, 1, 256, 512, True, 1, True)
+    x, w, bias = make_tensors(c, (2, 7, 7), seed=4)
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    st = gpu.settings_of(c, x.shape)
+    op = dlp.Conv2DForward.create(st, True, "relu", "gemm")
+    assert op.workspace() > 0
+    xd, wd, bd = gpu.dev(x), gpu.dev(w), gpu.dev(bias)
+    for ws in (torch.empty(op.workspace(), dtype=torch.uint8, device="cuda:0"), None):
+        y = torch.full(want.shape, float("nan"), device="cuda:0")
+        op.enqueue(xd, wd, bd, y, ws, 0.0)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+    old = np.random.default_rng(0).standard_normal(want.shape).astype(np.float32)
+    y = gpu.dev(old)
+    op.enqueue(xd, wd, bd, y, torch.empty(op.workspace(), dtype=torch.uint8, device="cuda:0"), 0.25)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(y.cpu().numpy(), oracle_mod.apply_factor(want, old, 0.25), **TOL)
+
+
 def test_gemm_integer_exact(gpu):
     # integer-valued inputs: fp32 sums are exact in any order, so the MFMA result must
     # EQUAL the integer result -- catches any indexing/layout slip that a tolerance could hide
