@@ -13,16 +13,29 @@
 //    consecutive output pixels and every store is a 128-byte run in NCHW.
 //  * A (weights) and B (gathered input) tiles are staged through LDS in [k][m]
 //    and [k][n] order: an MFMA operand fetch is a conflict-free ds_read.
-//  * all addressing of the gather is hoisted: per pixel a base offset and a bit
-//    mask of the window taps that fall inside the image, per k a table entry
-//    (offset, tap bit) read through the scalar unit.  Out-of-window taps and tile
-//    tails are redirected to an out-of-range buffer offset, which the buffer
-//    load returns as 0.0 -- the main loop has no divergent control flow.
-//  * global loads of tile kt+1 are issued before the MFMAs of tile kt
-//    (register-staged double buffering, one barrier per K step).
+//  * on this chip a vector-ALU instruction takes issue cycles away from the matrix
+//    pipe of its SIMD (measured: MFMA time and VALU time add up), so the gather is
+//    built to need almost no VALU work in the main loop:
+//      - every global load is a buffer load whose address is
+//        resource base + per-thread VGPR offset (loop invariant) + SGPR offset (per k),
+//        the SGPR part coming from a small table read through the scalar unit;
+//      - padding and tile tails are handled by swapping the VGPR offset for an
+//        out-of-range one, which the buffer load returns as 0.0 (no branches);
+//      - K is walked tap-major whenever Cin/groups is a multiple of 16: one K tile =
+//        one filter tap x 16 input channels, so the in-image test is one bit test
+//        per K tile instead of one per element.  The sum over K is order-free, the
+//        weights are fetched in the matching order (stride KH*KW, L2 resident).
+//        Other shapes (e.g. the 3-channel stem) use a per-element table.
+//  * software pipeline of distance two: tile kt+2 is in flight from memory to
+//    registers while tile kt+1 moves registers -> LDS and tile kt feeds the MFMAs.
+//  * layers with too few output tiles for 256 CUs split K over several
+//    workgroups; partial sums go through the workspace and are reduced in a
+//    fixed order by a second kernel (deterministic).
 #include "dlp_internal.hpp"
 
+#include <cstdlib>
 #include <type_traits>
+#include <vector>
 
 namespace dlp {
 
@@ -34,12 +47,11 @@ constexpr int kThreads = 256;
 constexpr int BK = 16;
 constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
 
-// How the validity of a gathered tap is decided:
-//  MASK_NONE : every tap of every pixel is inside the image (pad 0 fits) -- only tile tails are masked
-//  MASK_TAPS : KH*KW <= 32, one bit per tap in a single per-pixel word
-//  MASK_ROWCOL: any kernel up to 31x31, separate row and column masks
-enum { MASK_NONE = 0, MASK_TAPS = 1, MASK_ROWCOL = 2 };
-// Epilogue flavour: clamp covers identity / relu / relu6 with two constants, no branches
+// K ordering / gather table flavour
+enum { ORDER_CHANNEL = 0, ORDER_TAP = 1 };
+// In-image test: one bit per tap (KH*KW <= 32) or separate row / column masks
+enum { MASK_TAPS = 1, MASK_ROWCOL = 2 };
+// Epilogue flavour: clamp covers identity / relu / relu6 with two constants
 enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
 struct GemmArgs {
@@ -47,7 +59,7 @@ struct GemmArgs {
     const float *w;
     const float *bias;
     float *y;
-    const KTabEntry *ktab;
+    const int32_t *ktab;
     int M, N, K, nkt;
     int mtiles, ntiles;
     int splitk, kt_per_slice; // K tiles are dealt to `splitk` slices of kt_per_slice (even) tiles
@@ -55,22 +67,36 @@ struct GemmArgs {
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, w_bytes;
+    uint32_t x_shift; // bytes by which the X resource base is moved back (padding offset)
+    uint32_t hw4;     // H*W*4: byte stride between input channels
+    uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
     float factor;
     int act;
     float clamp_lo, clamp_hi;
 };
 
-typedef __attribute__((address_space(4))) KTabEntry KTabConst;
+typedef __attribute__((address_space(4))) const int32_t ConstInt;
 
-__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
+// q = n / d for 0 <= n < 2^31 with host-made (magic, shift)
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shift)
 {
-    // keep the offset a single opaque value: the select that produced it must stay a
-    // v_cndmask, not become two loads under divergent branches
-    asm("" : "+v"(byte_off));
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+    return (__umulhi(n, magic) + n) >> shift;
 }
 
-// call f(integral_constant<int, kk>) for the compile-time value matching the runtime-unrolled kk
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+
+// keep a selected offset one opaque value, so that the select stays a v_cndmask
+// instead of being turned into two loads under divergent branches
+__device__ __forceinline__ uint32_t opaque(uint32_t v)
+{
+    asm("" : "+v"(v));
+    return v;
+}
+
+// call f(integral_constant<int, kk>) for the compile-time value matching the unrolled kk
 template <class F>
 __device__ __forceinline__ void static_for_slice(int kk, F &&f)
 {
@@ -98,7 +124,7 @@ __device__ __forceinline__ void static_for_all(F &&f)
     f(std::integral_constant<int, 7>{});
 }
 
-template <int BM, int BN, int WM, int WN, int MASK, int ACT>
+template <int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 {
     static_assert(BK == 16, "the slice helpers assume 8 MFMA steps per K tile");
@@ -112,6 +138,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK % KSPLIT == 0, "B loader shape");
     constexpr int B_LD = BK / KSPLIT;        // gathered elements per thread per K step (contiguous k)
     constexpr int A_LD = BM * BK / kThreads; // weight elements per thread per K step
+    static_assert(A_LD >= 1, "weight loader shape");
 
     __shared__ float As[2][BK][LDA];
     __shared__ float Bs[2][BK][LDB];
@@ -123,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     const int h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
 
-    // tile decode: m tile fastest, then n tile, then group
+    // tile decode: m tile fastest, then n tile, then group, then K slice
     int t = blockIdx.x;
     const int mt = t % a.mtiles;
     t /= a.mtiles;
@@ -135,29 +162,30 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     const int kt_begin = slice * a.kt_per_slice;
     const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
 
-    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    // The X resource starts one padding offset before the tensor, so that the
+    // per-pixel window origin is a non-negative offset; taps that the masks let
+    // through never address below the tensor.
+    const __amdgpu_buffer_rsrc_t xr =
+        __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.x - a.x_shift), 0, a.x_bytes + a.x_shift, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+    ConstInt *ktab = (ConstInt *)a.ktab; // read-only, wavefront-uniform index: scalar loads
 
     // ---- per-thread gather state (one output pixel per thread) ----
     const int p = tid % BN;
     const int ks = (KSPLIT == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid / BN);
-    int base;
+    uint32_t vbase;          // byte offset of the window origin from the shifted base
     uint32_t my = 0, mx = 0; // MASK_TAPS: my = tap mask; MASK_ROWCOL: row / column masks
     {
         const int n = n0 + p;
         const bool vn = n < a.N;
-        const int b = n / a.OHW;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
         const int pix = n - b * a.OHW;
-        const int oy = pix / a.OW;
+        const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
         const int ox = pix - oy * a.OW;
         const int iy0 = oy * a.sh - a.ph;
         const int ix0 = ox * a.sw - a.pw;
-        base = ((b * a.Cin + g * a.Cin_g) * a.H + iy0) * a.W + ix0;
-        if (MASK == MASK_NONE) {
-            // (base + offset)*4 lands in [2^31, 2^32) for every table offset: out of range
-            if (!vn)
-                base = 0x20000000;
-        } else if (vn) {
+        vbase = (uint32_t)((((b * a.Cin + g * a.Cin_g) * a.H + oy * a.sh) * a.W + ox * a.sw) * 4);
+        if (vn) {
             uint32_t ry = 0, rx = 0;
             for (int ky = 0; ky < a.KH; ky++) {
                 int yy = iy0 + ky * a.dh;
@@ -180,14 +208,19 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         }
     }
 
-    // ---- per-thread weight loader state ----
+    // ---- per-thread weight loader state: row (m) part of the address ----
     const int ak = tid & 15;
     const int am = tid >> 4;
-    uint32_t a_off[A_LD];
+    uint32_t a_voff[A_LD];
 #pragma unroll
     for (int j = 0; j < A_LD; j++) {
-        int m = m0 + am + 16 * j;
-        a_off[j] = (m < a.M) ? (uint32_t)(((g * a.M + m) * a.K + ak) * 4) : kOutOfRange;
+        const int m = m0 + am + 16 * j;
+        uint32_t off;
+        if (ORDER == ORDER_TAP)
+            off = (uint32_t)((((g * a.M + m) * a.Cin_g + ak) * (a.KH * a.KW)) * 4);
+        else
+            off = (uint32_t)(((g * a.M + m) * a.K + ak) * 4);
+        a_voff[j] = (m < a.M) ? off : kOutOfRange;
     }
 
     // Two register sets for staged tiles: tile kt+2 is being fetched from memory
@@ -195,47 +228,65 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // (already in LDS) feeds the matrix cores.  A global load therefore has a whole
     // K step to land before anything waits on it.
     float ra[2][A_LD], rb[2][B_LD];
+    uint32_t vsel[2] = {kOutOfRange, kOutOfRange}; // ORDER_TAP: this tile's (masked) pixel offset
+    uint32_t akm[2] = {0, 0};                      // ORDER_CHANNEL: K-tail mask of the weight loads
 
     // one slice of the loads of tile kt into register set S: called once per MFMA
-    // group so that address arithmetic and vector-memory issue hide under MFMAs
-    auto load_slice = [&](auto set, int kt, auto slice) {
+    // group so that vector-memory issue is spread under the MFMAs
+    auto load_slice = [&](auto set, int kt, auto slice_q) {
         constexpr int S = decltype(set)::value;
-        constexpr int Q = decltype(slice)::value;
-        const int k0 = kt * BK;
-        const uint32_t kmask = (k0 + ak < a.K) ? 0u : kOutOfRange;
+        constexpr int Q = decltype(slice_q)::value;
+        if (ORDER == ORDER_TAP) {
+            // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, weight byte offset, -}
+            ConstInt *e = ktab + kt * 4;
+            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1], woff = (uint32_t)e[2];
+            if (Q == 0)
+                vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
 #pragma unroll
-        for (int j = 0; j < A_LD; j++)
-            if (j % (BK / 2) == Q)
-                ra[S][j] = buf_load(wr, (a_off[j] + (uint32_t)(k0 * 4)) | kmask);
-        // the table is read-only for the whole launch and the index is wavefront-uniform:
-        // constant address space makes these scalar loads (s_load), off the vector path
-        const KTabConst *tab = (const KTabConst *)(a.ktab) + k0 + ks * B_LD;
+            for (int j = 0; j < A_LD; j++)
+                if (j % (BK / 2) == Q)
+                    ra[S][j] = buf_load(wr, a_voff[j], woff);
 #pragma unroll
-        for (int i = 0; i < B_LD; i++) {
-            if (i % (BK / 2) != Q)
-                continue;
-            const KTabEntry e = {tab[i].offset, tab[i].tap};
-            uint32_t off = (uint32_t)((base + e.offset) * 4);
-            if (MASK == MASK_TAPS) {
-                off = (my & (uint32_t)e.tap) ? off : kOutOfRange;
-            } else if (MASK == MASK_ROWCOL) {
-                const int ky = e.tap & 0xff, kx = e.tap >> 8;
-                off = ((my >> ky) & (mx >> kx) & 1u) ? off : kOutOfRange;
+            for (int i = 0; i < B_LD; i++)
+                if (i % (BK / 2) == Q)
+                    rb[S][i] = buf_load(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4);
+        } else {
+            const int k0 = kt * BK;
+            if (Q == 0) // rows past K (tail of the last tile, tiles fetched past the end) read nothing
+                akm[S] = (k0 + ak < a.K) ? 0u : kOutOfRange;
+            const uint32_t k0c = (uint32_t)min(k0, (a.nkt - 1) * BK) * 4u; // SGPR part stays inside the tensor
+#pragma unroll
+            for (int j = 0; j < A_LD; j++)
+                if (j % (BK / 2) == Q)
+                    ra[S][j] = buf_load(wr, opaque(a_voff[j] | akm[S]), k0c);
+            // table entry of a k: {x byte offset of (c,ky,kx), tap bit or ky|kx<<8}
+            ConstInt *e = ktab + (k0 + ks * B_LD) * 2;
+#pragma unroll
+            for (int i = 0; i < B_LD; i++) {
+                if (i % (BK / 2) != Q)
+                    continue;
+                const uint32_t xoff = (uint32_t)e[2 * i], tap = (uint32_t)e[2 * i + 1];
+                bool ok;
+                if (MASK == MASK_TAPS)
+                    ok = (my & tap) != 0;
+                else
+                    ok = ((my >> (tap & 0xff)) & (mx >> (tap >> 8)) & 1u) != 0;
+                rb[S][i] = buf_load(xr, opaque(ok ? vbase : kOutOfRange), xoff);
             }
-            rb[S][i] = buf_load(xr, off);
         }
     };
-    auto store_slice = [&](auto set, int buf, auto slice) {
+    auto store_slice = [&](auto set, auto buf_c, auto slice_q) {
         constexpr int S = decltype(set)::value;
-        constexpr int Q = decltype(slice)::value;
+        constexpr int BUF = decltype(buf_c)::value;
+        constexpr int Q = decltype(slice_q)::value;
 #pragma unroll
         for (int j = 0; j < A_LD; j++)
             if (j % (BK / 2) == Q)
-                As[buf][ak][am + 16 * j] = ra[S][j];
+                As[BUF][ak][am + 16 * j] = ra[S][j];
 #pragma unroll
         for (int i = 0; i < B_LD; i++)
             if (i % (BK / 2) == Q)
-                Bs[buf][ks * B_LD + i][p] = rb[S][i];
+                Bs[BUF][ks * B_LD + i][p] = rb[S][i];
     };
 
     f32x16 acc[TM][TN];
@@ -248,29 +299,31 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 acc[i][j][r] = 0.0f;
 
     float fa[2][TM], fb[2][TN]; // MFMA operands, double buffered across the kk steps
-    auto read_operands = [&](int buf, int kk, int slot) {
+    auto read_operands = [&](auto buf_c, int kk, int slot) {
+        constexpr int BUF = decltype(buf_c)::value;
         const int k = 2 * kk + h;
 #pragma unroll
         for (int i = 0; i < TM; i++)
-            fa[slot][i] = As[buf][k][wm * WTM + i * 32 + l32];
+            fa[slot][i] = As[BUF][k][wm * WTM + i * 32 + l32];
 #pragma unroll
         for (int j = 0; j < TN; j++)
-            fb[slot][j] = Bs[buf][k][wn * WTN + j * 32 + l32];
+            fb[slot][j] = Bs[BUF][k][wn * WTN + j * 32 + l32];
     };
 
-    // One K step: MFMAs of tile kt (in LDS[buf]); register set SN (tile kt+1) goes to
-    // LDS[buf^1]; tile kt+2 is fetched into register set SL.  Operands of step kk+1
+    // One K step on tile kt, resident in LDS[BUF]: register set SN (tile kt+1) goes to
+    // LDS[BUF^1]; tile kt+2 is fetched into register set SL.  Operands of step kk+1
     // are read from LDS before the MFMAs of step kk are issued.
-    auto k_step = [&](auto set_next, auto set_load, int kt) {
-        const int buf = kt & 1;
-        read_operands(buf, 0, 0);
+    auto k_step = [&](auto buf_c, auto set_next, auto set_load, int kt) {
+        constexpr int BUF = decltype(buf_c)::value;
+        using NextBuf = std::integral_constant<int, BUF ^ 1>;
+        read_operands(buf_c, 0, 0);
 #pragma unroll
         for (int kk = 0; kk < BK / 2; kk++) {
             const int cur = kk & 1;
             if (kk + 1 < BK / 2)
-                read_operands(buf, kk + 1, cur ^ 1);
+                read_operands(buf_c, kk + 1, cur ^ 1);
             static_for_slice(kk, [&](auto q) {
-                store_slice(set_next, buf ^ 1, q);
+                store_slice(set_next, NextBuf{}, q);
                 load_slice(set_load, kt + 2, q);
             });
 #pragma unroll
@@ -287,13 +340,16 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // prologue: first tile -> set 0 -> LDS[0]; second tile -> set 1
     static_for_all([&](auto q) { load_slice(I0{}, kt_begin, q); });
     static_for_all([&](auto q) { load_slice(I1{}, kt_begin + 1, q); });
-    static_for_all([&](auto q) { store_slice(I0{}, 0, q); });
+    static_for_all([&](auto q) { store_slice(I0{}, I0{}, q); });
     __syncthreads();
-    // tile counts are even (the host rounds up; tiles past K load zeros through the masks)
-    for (int kt = kt_begin; kt < kt_end; kt += 2) {
-        k_step(I1{}, I0{}, kt);
-        k_step(I0{}, I1{}, kt + 1);
+    // tiles fetched past kt_end are never multiplied: the table has two spare entries
+    int kt = kt_begin;
+    for (; kt + 1 < kt_end; kt += 2) {
+        k_step(I0{}, I1{}, I0{}, kt);
+        k_step(I1{}, I0{}, I1{}, kt + 1);
     }
+    if (kt < kt_end)
+        k_step(I0{}, I1{}, I0{}, kt);
 
     // ---- split-K: raw partial sums to the workspace, reduced by a second kernel ----
     if (a.splitk > 1) {
@@ -323,7 +379,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         const int n = n0 + wn * WTN + j * 32 + l32;
         if (n >= a.N)
             continue;
-        const int b = n / a.OHW;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
         const int pix = n - b * a.OHW;
         float *yb = a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
 #pragma unroll
@@ -372,7 +428,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
     store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, v, a.factor);
 }
 
-// Split-K factor for a launch of `tiles` output tiles over `nkt` (even) K tiles.
+// Split-K factor for a launch of `tiles` output tiles over `nkt` K tiles.
 // Workgroups of one launch are co-resident, so the time is set by the busiest CU:
 // pick the factor that fills whole rounds of the 256 CUs best, keeping at least
 // 8 K tiles per slice; 1 = no split.
@@ -396,6 +452,28 @@ int choose_splitk(long long tiles, int nkt)
     return best;
 }
 
+bool generic_act(int activation) { return activation == DLP_ACT_TANH || activation == DLP_ACT_SIGMOID; }
+
+// K ordering and mask flavour of a geometry (the gather table is built to match).
+void gather_mode(const ConvGeom &g, int activation, int &order, int &mask)
+{
+    const int cin_g = g.Cin / g.groups;
+    if (generic_act(activation)) { // the rare activations share one instantiation per tile
+        order = ORDER_CHANNEL;
+        mask = MASK_ROWCOL;
+        return;
+    }
+    const bool small_kernel = g.KH * g.KW <= 32;
+    order = (small_kernel && cin_g % BK == 0) ? ORDER_TAP : ORDER_CHANNEL;
+    mask = small_kernel ? MASK_TAPS : MASK_ROWCOL;
+}
+
+int k_tiles(const ConvGeom &g)
+{
+    const int K = (g.Cin / g.groups) * g.KH * g.KW; // tap-major order has the same count: K is a multiple of 16 there
+    return (K + BK - 1) / BK;
+}
+
 template <int BM, int BN>
 void plan_split(GemmArgs &a, int groups, size_t ws_bytes)
 {
@@ -404,17 +482,17 @@ void plan_split(GemmArgs &a, int groups, size_t ws_bytes)
     int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt);
     if (s > 1 && (a.part == nullptr || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
         s = 1; // no (or too small a) workspace: run unsplit
-    a.splitk = s;
-    a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;
+    a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
+    a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
 }
 
-template <int BM, int BN, int WM, int WN, int MASK, int ACT>
+template <int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
-    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     if (a.splitk > 1) {
         const long long total = (long long)a.Cout * a.N;
         hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
@@ -424,65 +502,108 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 }
 
 template <int BM, int BN, int WM, int WN>
-int launch_tile(const ConvGeom &g, GemmArgs &a, int mask, int act, size_t ws_bytes, hipStream_t stream)
+int launch_tile(const ConvGeom &g, GemmArgs &a, int order, int mask, int act, size_t ws_bytes, hipStream_t stream)
 {
     plan_split<BM, BN>(a, g.groups, ws_bytes);
-    if (act == ACT_CLAMP) {
-        if (mask == MASK_NONE)
-            return launch_inst<BM, BN, WM, WN, MASK_NONE, ACT_CLAMP>(g, a, stream);
-        if (mask == MASK_TAPS)
-            return launch_inst<BM, BN, WM, WN, MASK_TAPS, ACT_CLAMP>(g, a, stream);
-        return launch_inst<BM, BN, WM, WN, MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
-    }
-    // tanh / sigmoid: rare, one generic instantiation per tile
-    return launch_inst<BM, BN, WM, WN, MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
+    if (act == ACT_GENERIC)
+        return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
+    if (order == ORDER_TAP)
+        return launch_inst<BM, BN, WM, WN, ORDER_TAP, MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    if (mask == MASK_TAPS)
+        return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
 }
 
-bool generic_act(int activation) { return activation == DLP_ACT_TANH || activation == DLP_ACT_SIGMOID; }
-
-int mask_mode(const ConvGeom &g, int activation)
+void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
 {
-    if (generic_act(activation))
-        return MASK_ROWCOL; // the rare activations share one instantiation per tile
-    // no tap can fall outside the image (no padding, last window fits) and no K tail
-    const bool fits_h = g.ph == 0 && (g.OH - 1) * g.sh + (g.KH - 1) * g.dh < g.H;
-    const bool fits_w = g.pw == 0 && (g.OW - 1) * g.sw + (g.KW - 1) * g.dw < g.W;
-    const int K = (g.Cin / g.groups) * g.KH * g.KW;
-    if (fits_h && fits_w && K % BK == 0)
-        return MASK_NONE;
-    if (g.KH * g.KW <= 32)
-        return MASK_TAPS;
-    return MASK_ROWCOL;
+    // q = (umulhi(n, magic) + n) >> shift  ==  n / d   for 0 <= n < 2^31
+    shift = 0;
+    while ((1ull << shift) < d)
+        shift++;
+    magic = (uint32_t)(((1ull << 32) * ((1ull << shift) - d)) / d + 1);
+}
+
+// tile shape by rows per group; the experiment knob is for tuning runs only
+int tile_choice(int M)
+{
+    if (const char *e = getenv("DLP_TILE_EXPERIMENT")) {
+        int v = atoi(e);
+        if (v > 0)
+            return v;
+    }
+    if (M > 64)
+        return 6;
+    if (M > 32)
+        return 5;
+    return 8;
 }
 
 } // namespace
 
 size_t conv_gemm_ktab_entries(const ConvGeom &g)
 {
-    // K tiles rounded up to an even count, plus two tiles of never-valid entries that
-    // the software pipeline prefetches past the end
-    size_t K = (size_t)(g.Cin / g.groups) * g.KH * g.KW;
-    size_t tiles = (K + BK - 1) / BK;
-    tiles = (tiles + 1) / 2 * 2 + 2;
-    return tiles * BK;
+    // one 8-byte entry per k (ORDER_TAP uses two entries per K tile); two spare tiles of
+    // never-valid entries are what the software pipeline fetches past the end
+    return (size_t)(k_tiles(g) + 2) * BK;
 }
 
-void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab)
+void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entries)
 {
+    int32_t *tab = (int32_t *)tab_entries;
+    const size_t words = conv_gemm_ktab_entries(g) * 2;
+    for (size_t i = 0; i < words; i++)
+        tab[i] = 0; // spare entries: no tap bit (row/col code 31 below), offsets 0
+    int order, mask;
+    gather_mode(g, activation, order, mask);
     const int cin_g = g.Cin / g.groups;
-    const size_t Kp = conv_gemm_ktab_entries(g);
-    const int mode = mask_mode(g, activation);
+    const int khw = g.KH * g.KW;
+    if (order == ORDER_TAP) {
+        int t = 0;
+        for (int cb = 0; cb < cin_g / BK; cb++)
+            for (int ky = 0; ky < g.KH; ky++)
+                for (int kx = 0; kx < g.KW; kx++, t++) {
+                    tab[4 * t + 0] = ((cb * BK * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
+                    tab[4 * t + 1] = (int32_t)(1u << (ky * g.KW + kx));
+                    tab[4 * t + 2] = (cb * BK * khw + ky * g.KW + kx) * 4;
+                }
+        return;
+    }
     size_t k = 0;
     for (int c = 0; c < cin_g; c++)
         for (int ky = 0; ky < g.KH; ky++)
             for (int kx = 0; kx < g.KW; kx++, k++) {
-                tab[k].offset = (c * g.H + ky * g.dh) * g.W + kx * g.dw;
-                tab[k].tap = (mode == MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << ((ky * g.KW + kx) & 31));
+                tab[2 * k + 0] = ((c * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
+                tab[2 * k + 1] = (mask == MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << (ky * g.KW + kx));
             }
-    for (; k < Kp; k++) {
-        // padding rows of the last K tile: never valid (MASK_NONE has no K tail)
-        tab[k].offset = 0;
-        tab[k].tap = (mode == MASK_ROWCOL) ? (31 | (31 << 8)) : 0;
+    if (mask == MASK_ROWCOL)
+        for (; 2 * k + 1 < words; k++)
+            tab[2 * k + 1] = 31 | (31 << 8); // bit 31 of the row / column masks is never set
+}
+
+static void fill_dims(const ConvGeom &g, GemmArgs &a, int n_valid)
+{
+    a.M = g.Cout / g.groups;
+    a.N = g.B * g.OH * g.OW;
+    if (n_valid >= 0 && n_valid < a.N)
+        a.N = n_valid;
+    a.K = (g.Cin / g.groups) * g.KH * g.KW;
+    a.nkt = k_tiles(g);
+    a.Cout = g.Cout;
+    a.groups = g.groups;
+}
+
+template <class F>
+static auto with_tile(int choice, F &&f)
+{
+    switch (choice) {
+    case 1: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+    case 2: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    case 3: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    case 5: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 256>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+    case 7: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    case 8: return f(std::integral_constant<int, 32>{}, std::integral_constant<int, 256>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+    case 9: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
+    default: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
     }
 }
 
@@ -492,17 +613,12 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g)
     if (g.B <= 0)
         return 0;
     GemmArgs a;
-    a.M = g.Cout / g.groups;
-    a.N = g.B * g.OH * g.OW;
-    a.Cout = g.Cout;
-    a.nkt = (((g.Cin / g.groups) * g.KH * g.KW + BK - 1) / BK + 1) / 2 * 2;
+    fill_dims(g, a, -1);
     a.part = (float *)16; // any non-null value: ask for the unconstrained plan
-    if (a.M > 64)
-        plan_split<128, 128>(a, g.groups, (size_t)-1);
-    else if (a.M > 32)
-        plan_split<64, 256>(a, g.groups, (size_t)-1);
-    else
-        plan_split<32, 256>(a, g.groups, (size_t)-1);
+    with_tile(tile_choice(a.M), [&](auto bm, auto bn, auto, auto) {
+        plan_split<decltype(bm)::value, decltype(bn)::value>(a, g.groups, (size_t)-1);
+        return 0;
+    });
     return a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0;
 }
 
@@ -515,7 +631,8 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     const size_t x_elems = (size_t)g.B * g.Cin * g.H * g.W;
     const size_t w_elems = (size_t)g.Cout * (g.Cin / g.groups) * g.KH * g.KW;
     const size_t y_elems = (size_t)g.B * g.Cout * g.OH * g.OW;
-    if (x_elems * 4 >= 0x20000000ULL * 4 || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
+    const size_t x_shift = ((size_t)g.ph * g.W + g.pw) * 4;
+    if (x_elems * 4 + x_shift >= kOutOfRange || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
@@ -525,28 +642,25 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     a.w = (const float *)w;
     a.bias = ep.bias;
     a.y = (float *)y;
-    a.ktab = dev_ktab;
-    a.M = g.Cout / g.groups;
-    a.N = g.B * g.OH * g.OW;
-    if (n_valid >= 0 && n_valid < a.N)
-        a.N = n_valid;
+    a.ktab = (const int32_t *)dev_ktab;
+    fill_dims(g, a, n_valid);
     if (a.N == 0)
         return DLP_OK;
-    a.K = (g.Cin / g.groups) * g.KH * g.KW;
-    a.nkt = ((a.K + BK - 1) / BK + 1) / 2 * 2;
+    a.part = (float *)ws;
     a.Cin = g.Cin;
     a.Cin_g = g.Cin / g.groups;
     a.H = g.H;
     a.W = g.W;
-    a.Cout = g.Cout;
-    a.groups = g.groups;
-    a.part = (float *)ws;
     a.OW = g.OW;
     a.OHW = g.OH * g.OW;
     a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw; a.dh = g.dh; a.dw = g.dw;
     a.KH = g.KH; a.KW = g.KW;
     a.x_bytes = (uint32_t)(x_elems * 4);
     a.w_bytes = (uint32_t)(w_elems * 4);
+    a.x_shift = (uint32_t)x_shift;
+    a.hw4 = (uint32_t)(g.H * g.W * 4);
+    make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
+    make_magic((uint32_t)a.OW, a.ow_magic, a.ow_shift);
     a.factor = ep.factor;
     a.act = ep.activation;
     a.clamp_lo = -__builtin_huge_valf();
@@ -556,13 +670,13 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     if (ep.activation == DLP_ACT_RELU6)
         a.clamp_hi = 6.0f;
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
-    const int mask = mask_mode(g, ep.activation); // same rule the gather table was built with
+    int order, mask;
+    gather_mode(g, ep.activation, order, mask); // same rule the gather table was built with
 
-    if (a.M > 64)
-        return launch_tile<128, 128, 2, 2>(g, a, mask, act, ws_bytes, stream);
-    if (a.M > 32)
-        return launch_tile<64, 256, 1, 4>(g, a, mask, act, ws_bytes, stream);
-    return launch_tile<32, 256, 1, 4>(g, a, mask, act, ws_bytes, stream);
+    return with_tile(tile_choice(a.M), [&](auto bm, auto bn, auto wm, auto wn) {
+        return launch_tile<decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, a, order, mask, act,
+                                                                                                                    ws_bytes, stream);
+    });
 }
 
 } // namespace dlp
