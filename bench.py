@@ -56,7 +56,7 @@ def build_layers(batch, seed, algo, activation_all_relu=True):
 def kernel_class(L):
     """Which kernel instantiation serves a layer (tile selection is by Cout per group)."""
     m = L["cout"] // L["groups"]
-    return "conv_gemm_f32<128x128>" if m > 64 else ("conv_gemm_f32<64x256>" if m > 32 else "conv_gemm_f32<32x256>")
+    return "conv_gemm_f32<64x64>" if m > 32 else "conv_gemm_f32<32x128>"
 
 
 def cpu_baseline(images, seed):

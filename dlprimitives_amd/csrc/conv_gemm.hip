@@ -14,8 +14,8 @@
 //  * A (weights) and B (gathered input) tiles are staged through LDS in [k][m]
 //    and [k][n] order: an MFMA operand fetch is a conflict-free ds_read.
 //  * on this chip a vector-ALU instruction takes issue cycles away from the matrix
-//    pipe of its SIMD (measured: MFMA time and VALU time add up), so the gather is
-//    built to need almost no VALU work in the main loop:
+//    pipe of its SIMD (measured: MFMA time and VALU time add up), so the main loop
+//    is built to need almost no VALU work:
 //      - every global load is a buffer load whose address is
 //        resource base + per-thread VGPR offset (loop invariant) + SGPR offset (per k),
 //        the SGPR part coming from a small table read through the scalar unit;
@@ -23,9 +23,12 @@
 //        out-of-range one, which the buffer load returns as 0.0 (no branches);
 //      - K is walked tap-major whenever Cin/groups is a multiple of 16: one K tile =
 //        one filter tap x 16 input channels, so the in-image test is one bit test
-//        per K tile instead of one per element.  The sum over K is order-free, the
-//        weights are fetched in the matching order (stride KH*KW, L2 resident).
-//        Other shapes (e.g. the 3-channel stem) use a per-element table.
+//        per K tile instead of one per element (the sum over K is order-free).
+//        Other shapes (e.g. the 3-channel stem) use a per-element table;
+//      - the weights are repacked once per call (a small kernel, like the reference's
+//        Winograd filter transform) into the exact [m tile][K tile][k][m] image of the
+//        LDS A tile, zero padded: the A load is one coalesced 16-byte load per thread
+//        with no masks, whatever the K order.
 //  * software pipeline of distance two: tile kt+2 is in flight from memory to
 //    registers while tile kt+1 moves registers -> LDS and tile kt feeds the MFMAs.
 //  * layers with too few output tiles for 256 CUs split K over several
@@ -33,13 +36,13 @@
 //    fixed order by a second kernel (deterministic).
 #include "dlp_internal.hpp"
 
-#include <cstdlib>
 #include <type_traits>
-#include <vector>
 
 namespace dlp {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -47,16 +50,11 @@ constexpr int kThreads = 256;
 constexpr int BK = 16;
 constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
 
-// K ordering / gather table flavour
-enum { ORDER_CHANNEL = 0, ORDER_TAP = 1 };
-// In-image test: one bit per tap (KH*KW <= 32) or separate row / column masks
-enum { MASK_TAPS = 1, MASK_ROWCOL = 2 };
-// Epilogue flavour: clamp covers identity / relu / relu6 with two constants
 enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
 struct GemmArgs {
     const float *x;
-    const float *w;
+    const float *wp; // packed weights
     const float *bias;
     float *y;
     const int32_t *ktab;
@@ -66,7 +64,7 @@ struct GemmArgs {
     float *part;              // split-K partial sums [slice][Cout][N]
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
-    uint32_t x_bytes, w_bytes;
+    uint32_t x_bytes, wp_bytes;
     uint32_t x_shift; // bytes by which the X resource base is moved back (padding offset)
     uint32_t hw4;     // H*W*4: byte stride between input channels
     uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
@@ -86,6 +84,11 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
 {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+
+__device__ __forceinline__ f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
 
 // keep a selected offset one opaque value, so that the select stays a v_cndmask
@@ -132,15 +135,16 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
     constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA blocks per wavefront
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "tile shape");
-    constexpr int LDA = BM + 2; // stride = 2 (mod 32): transposed A stores hit 32 distinct banks
+    constexpr int LDA = BM + 4; // rows stay 16-byte aligned for the b128 stores
     constexpr int LDB = BN;
     constexpr int KSPLIT = kThreads / BN;    // k slices among the B loader threads
     static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK % KSPLIT == 0, "B loader shape");
     constexpr int B_LD = BK / KSPLIT;        // gathered elements per thread per K step (contiguous k)
-    constexpr int A_LD = BM * BK / kThreads; // weight elements per thread per K step
-    static_assert(A_LD >= 1, "weight loader shape");
+    constexpr int A_V4 = BM * BK / 4;        // 16-byte pieces of a packed A tile
+    constexpr int A_LD = (A_V4 + kThreads - 1) / kThreads; // ... per thread
+    static_assert(BM % 4 == 0, "packed A rows are read in 16-byte pieces");
 
-    __shared__ float As[2][BK][LDA];
+    __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
     __shared__ float Bs[2][BK][LDB];
 
     const int tid = threadIdx.x;
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // through never address below the tensor.
     const __amdgpu_buffer_rsrc_t xr =
         __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.x - a.x_shift), 0, a.x_bytes + a.x_shift, 0x00020000);
-    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
     ConstInt *ktab = (ConstInt *)a.ktab; // read-only, wavefront-uniform index: scalar loads
 
     // ---- per-thread gather state (one output pixel per thread) ----
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 if (xx >= 0 && xx < a.W)
                     rx |= 1u << kx;
             }
-            if (MASK == MASK_TAPS) {
+            if (MASK == GEMM_MASK_TAPS) {
                 for (int ky = 0; ky < a.KH; ky++)
                     if ((ry >> ky) & 1u)
                         my |= rx << (ky * a.KW);
@@ -208,66 +212,50 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         }
     }
 
-    // ---- per-thread weight loader state: row (m) part of the address ----
-    const int ak = tid & 15;
-    const int am = tid >> 4;
-    uint32_t a_voff[A_LD];
-#pragma unroll
-    for (int j = 0; j < A_LD; j++) {
-        const int m = m0 + am + 16 * j;
-        uint32_t off;
-        if (ORDER == ORDER_TAP)
-            off = (uint32_t)((((g * a.M + m) * a.Cin_g + ak) * (a.KH * a.KW)) * 4);
-        else
-            off = (uint32_t)(((g * a.M + m) * a.K + ak) * 4);
-        a_voff[j] = (m < a.M) ? off : kOutOfRange;
-    }
+    // ---- weight loader: 16-byte pieces of the packed tile, in tile order ----
+    const uint32_t a_tile_bytes = BK * BM * 4;
+    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes; // SGPR
+    const bool a_active = (A_V4 >= kThreads) || (tid < A_V4);
 
     // Two register sets for staged tiles: tile kt+2 is being fetched from memory
     // into one set while tile kt+1 moves from the other set into LDS and tile kt
     // (already in LDS) feeds the matrix cores.  A global load therefore has a whole
     // K step to land before anything waits on it.
-    float ra[2][A_LD], rb[2][B_LD];
-    uint32_t vsel[2] = {kOutOfRange, kOutOfRange}; // ORDER_TAP: this tile's (masked) pixel offset
-    uint32_t akm[2] = {0, 0};                      // ORDER_CHANNEL: K-tail mask of the weight loads
+    f32x4 ra[2][A_LD];
+    float rb[2][B_LD];
+    uint32_t vsel[2] = {kOutOfRange, kOutOfRange}; // GEMM_ORDER_TAP: this tile's (masked) pixel offset
 
     // one slice of the loads of tile kt into register set S: called once per MFMA
     // group so that vector-memory issue is spread under the MFMAs
     auto load_slice = [&](auto set, int kt, auto slice_q) {
         constexpr int S = decltype(set)::value;
         constexpr int Q = decltype(slice_q)::value;
-        if (ORDER == ORDER_TAP) {
-            // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, weight byte offset, -}
+        // tiles fetched past the end of K are never multiplied: re-read the last tile
+        const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
+#pragma unroll
+        for (int j = 0; j < A_LD; j++)
+            if (j % (BK / 2) == Q)
+                ra[S][j] = buf_load4(wr, a_active ? (uint32_t)(tid * 16 + j * kThreads * 16) : kOutOfRange, a_soff);
+        if (ORDER == GEMM_ORDER_TAP) {
+            // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
-            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1], woff = (uint32_t)e[2];
+            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
             if (Q == 0)
                 vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
-#pragma unroll
-            for (int j = 0; j < A_LD; j++)
-                if (j % (BK / 2) == Q)
-                    ra[S][j] = buf_load(wr, a_voff[j], woff);
 #pragma unroll
             for (int i = 0; i < B_LD; i++)
                 if (i % (BK / 2) == Q)
                     rb[S][i] = buf_load(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4);
         } else {
-            const int k0 = kt * BK;
-            if (Q == 0) // rows past K (tail of the last tile, tiles fetched past the end) read nothing
-                akm[S] = (k0 + ak < a.K) ? 0u : kOutOfRange;
-            const uint32_t k0c = (uint32_t)min(k0, (a.nkt - 1) * BK) * 4u; // SGPR part stays inside the tensor
-#pragma unroll
-            for (int j = 0; j < A_LD; j++)
-                if (j % (BK / 2) == Q)
-                    ra[S][j] = buf_load(wr, opaque(a_voff[j] | akm[S]), k0c);
             // table entry of a k: {x byte offset of (c,ky,kx), tap bit or ky|kx<<8}
-            ConstInt *e = ktab + (k0 + ks * B_LD) * 2;
+            ConstInt *e = ktab + (kt * BK + ks * B_LD) * 2;
 #pragma unroll
             for (int i = 0; i < B_LD; i++) {
                 if (i % (BK / 2) != Q)
                     continue;
                 const uint32_t xoff = (uint32_t)e[2 * i], tap = (uint32_t)e[2 * i + 1];
                 bool ok;
-                if (MASK == MASK_TAPS)
+                if (MASK == GEMM_MASK_TAPS)
                     ok = (my & tap) != 0;
                 else
                     ok = ((my >> (tap & 0xff)) & (mx >> (tap >> 8)) & 1u) != 0;
@@ -281,8 +269,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         constexpr int Q = decltype(slice_q)::value;
 #pragma unroll
         for (int j = 0; j < A_LD; j++)
-            if (j % (BK / 2) == Q)
-                As[BUF][ak][am + 16 * j] = ra[S][j];
+            if (j % (BK / 2) == Q) {
+                const int idx = (tid + j * kThreads) * 4; // float index inside the [BK][BM] tile
+                if (a_active)
+                    *(f32x4 *)&As[BUF][idx / BM][idx % BM] = ra[S][j];
+            }
 #pragma unroll
         for (int i = 0; i < B_LD; i++)
             if (i % (BK / 2) == Q)
@@ -428,59 +419,62 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
     store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, v, a.factor);
 }
 
+// Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
+__global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int groups, int cin_g, int khw, const float *__restrict__ w,
+                                                           float *__restrict__ out)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long total = (long long)groups * p.mtiles * p.nkt * BK * p.BM;
+    if (idx >= total)
+        return;
+    const int mi = (int)(idx % p.BM);
+    long long r = idx / p.BM;
+    const int k = (int)(r % BK);
+    r /= BK;
+    const int kt = (int)(r % p.nkt);
+    r /= p.nkt;
+    const int mt = (int)(r % p.mtiles);
+    const int g = (int)(r / p.mtiles);
+    const int m = mt * p.BM + mi;
+    int col; // column of the [M][K] weight matrix of this group
+    if (p.order == GEMM_ORDER_TAP) {
+        const int cb = kt / khw, tap = kt - cb * khw;
+        col = (cb * BK + k) * khw + tap;
+    } else {
+        col = kt * BK + k;
+    }
+    float v = 0.0f;
+    if (m < p.M && col < p.K)
+        v = w[((size_t)g * p.M + m) * p.K + col];
+    out[idx] = v;
+}
+
 // Split-K factor for a launch of `tiles` output tiles over `nkt` K tiles.
-// Workgroups of one launch are co-resident, so the time is set by the busiest CU:
-// pick the factor that fills whole rounds of the 256 CUs best, keeping at least
-// 8 K tiles per slice; 1 = no split.
+// The 64x64 tile runs up to 8 workgroups per CU; measured on the ResNet shapes the
+// kernel needs on the order of 1200 workgroups in flight to keep the matrix pipes of
+// 256 CUs busy, and a split only pays when every slice still has a long K loop
+// (the partial sums cost one extra pass over the output per slice).
 int choose_splitk(long long tiles, int nkt)
 {
-    const int kCUs = 256;
-    if (tiles >= 2 * kCUs || nkt < 16)
+    if (tiles >= 1000)
         return 1;
-    int best = 1;
-    double best_eff = (double)tiles / (double)(((tiles + kCUs - 1) / kCUs) * kCUs);
-    for (int s = 2; s <= 8; s++) {
-        if (nkt / s < 8)
-            break;
-        const long long blocks = tiles * s;
-        const double eff = (double)blocks / (double)(((blocks + kCUs - 1) / kCUs) * kCUs);
-        if (eff > best_eff + 0.05) {
-            best_eff = eff;
-            best = s;
-        }
-    }
-    return best;
+    long long s = (1200 + tiles / 2) / tiles; // round(1200 / tiles)
+    const long long max_by_k = nkt / 24;
+    if (s > max_by_k)
+        s = max_by_k;
+    if (s > 16)
+        s = 16;
+    return s < 1 ? 1 : (int)s;
 }
 
 bool generic_act(int activation) { return activation == DLP_ACT_TANH || activation == DLP_ACT_SIGMOID; }
 
-// K ordering and mask flavour of a geometry (the gather table is built to match).
-void gather_mode(const ConvGeom &g, int activation, int &order, int &mask)
+void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t ws_bytes)
 {
-    const int cin_g = g.Cin / g.groups;
-    if (generic_act(activation)) { // the rare activations share one instantiation per tile
-        order = ORDER_CHANNEL;
-        mask = MASK_ROWCOL;
-        return;
-    }
-    const bool small_kernel = g.KH * g.KW <= 32;
-    order = (small_kernel && cin_g % BK == 0) ? ORDER_TAP : ORDER_CHANNEL;
-    mask = small_kernel ? MASK_TAPS : MASK_ROWCOL;
-}
-
-int k_tiles(const ConvGeom &g)
-{
-    const int K = (g.Cin / g.groups) * g.KH * g.KW; // tap-major order has the same count: K is a multiple of 16 there
-    return (K + BK - 1) / BK;
-}
-
-template <int BM, int BN>
-void plan_split(GemmArgs &a, int groups, size_t ws_bytes)
-{
-    a.mtiles = (a.M + BM - 1) / BM;
-    a.ntiles = (a.N + BN - 1) / BN;
+    a.mtiles = p.mtiles;
+    a.ntiles = (a.N + p.BN - 1) / p.BN;
     int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt);
-    if (s > 1 && (a.part == nullptr || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
+    if (s > 1 && (!have_ws || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
@@ -502,16 +496,15 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 }
 
 template <int BM, int BN, int WM, int WN>
-int launch_tile(const ConvGeom &g, GemmArgs &a, int order, int mask, int act, size_t ws_bytes, hipStream_t stream)
+int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipStream_t stream)
 {
-    plan_split<BM, BN>(a, g.groups, ws_bytes);
     if (act == ACT_GENERIC)
-        return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
-    if (order == ORDER_TAP)
-        return launch_inst<BM, BN, WM, WN, ORDER_TAP, MASK_TAPS, ACT_CLAMP>(g, a, stream);
-    if (mask == MASK_TAPS)
-        return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_TAPS, ACT_CLAMP>(g, a, stream);
-    return launch_inst<BM, BN, WM, WN, ORDER_CHANNEL, MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
+        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
+    if (p.order == GEMM_ORDER_TAP)
+        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_TAP, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    if (p.mask == GEMM_MASK_TAPS)
+        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
 }
 
 void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
@@ -523,28 +516,62 @@ void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
     magic = (uint32_t)(((1ull << 32) * ((1ull << shift) - d)) / d + 1);
 }
 
-// tile shape by rows per group; the experiment knob is for tuning runs only
-int tile_choice(int M)
+// Workgroup tiles.  Small tiles win on this chip: fp32 MFMA is slow enough (64 cycles
+// per 32x32x2 block) that one 32x32 block per wavefront already hides the LDS traffic,
+// and 8 resident workgroups per CU hide everything else.
+struct TileShape {
+    int id, BM, BN;
+};
+constexpr TileShape kTiles[] = {{0, 64, 64}, {1, 32, 128}};
+
+int tile_choice(int M) { return M > 32 ? 0 : 1; }
+
+template <class F>
+int with_tile(int choice, F &&f)
 {
-    if (const char *e = getenv("DLP_TILE_EXPERIMENT")) {
-        int v = atoi(e);
-        if (v > 0)
-            return v;
-    }
-    if (M > 64)
-        return 6;
-    if (M > 32)
-        return 5;
-    return 8;
+    using std::integral_constant;
+    if (choice == 1)
+        return f(integral_constant<int, 32>{}, integral_constant<int, 128>{}, integral_constant<int, 1>{}, integral_constant<int, 4>{});
+    return f(integral_constant<int, 64>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}, integral_constant<int, 2>{});
 }
 
 } // namespace
 
+GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
+{
+    GemmPlan p;
+    const int cin_g = g.Cin / g.groups;
+    p.M = g.Cout / g.groups;
+    p.K = cin_g * g.KH * g.KW;
+    p.nkt = (p.K + BK - 1) / BK; // the tap-major order has the same count: K is a multiple of 16 there
+    const bool small_kernel = g.KH * g.KW <= 32;
+    if (generic_act(activation)) { // the rare activations share one instantiation per tile
+        p.order = GEMM_ORDER_CHANNEL;
+        p.mask = GEMM_MASK_ROWCOL;
+    } else {
+        p.order = (small_kernel && cin_g % BK == 0) ? GEMM_ORDER_TAP : GEMM_ORDER_CHANNEL;
+        p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
+    }
+    p.tile = tile_choice(p.M);
+    p.BM = 64;
+    p.BN = 64;
+    for (const TileShape &ts : kTiles)
+        if (ts.id == p.tile) {
+            p.BM = ts.BM;
+            p.BN = ts.BN;
+        }
+    p.mtiles = (p.M + p.BM - 1) / p.BM;
+    p.wpack_bytes = (size_t)g.groups * p.mtiles * p.nkt * BK * p.BM * sizeof(float);
+    p.wpack_bytes = (p.wpack_bytes + 255) / 256 * 256;
+    return p;
+}
+
 size_t conv_gemm_ktab_entries(const ConvGeom &g)
 {
-    // one 8-byte entry per k (ORDER_TAP uses two entries per K tile); two spare tiles of
-    // never-valid entries are what the software pipeline fetches past the end
-    return (size_t)(k_tiles(g) + 2) * BK;
+    // one 8-byte entry per k (the tap-major order uses two entries per K tile); two spare
+    // tiles of never-valid entries are what the software pipeline fetches past the end
+    const int K = (g.Cin / g.groups) * g.KH * g.KW;
+    return (size_t)((K + BK - 1) / BK + 2) * BK;
 }
 
 void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entries)
@@ -553,18 +580,15 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
     const size_t words = conv_gemm_ktab_entries(g) * 2;
     for (size_t i = 0; i < words; i++)
         tab[i] = 0; // spare entries: no tap bit (row/col code 31 below), offsets 0
-    int order, mask;
-    gather_mode(g, activation, order, mask);
+    const GemmPlan p = conv_gemm_plan(g, activation);
     const int cin_g = g.Cin / g.groups;
-    const int khw = g.KH * g.KW;
-    if (order == ORDER_TAP) {
+    if (p.order == GEMM_ORDER_TAP) {
         int t = 0;
         for (int cb = 0; cb < cin_g / BK; cb++)
             for (int ky = 0; ky < g.KH; ky++)
                 for (int kx = 0; kx < g.KW; kx++, t++) {
                     tab[4 * t + 0] = ((cb * BK * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
                     tab[4 * t + 1] = (int32_t)(1u << (ky * g.KW + kx));
-                    tab[4 * t + 2] = (cb * BK * khw + ky * g.KW + kx) * 4;
                 }
         return;
     }
@@ -573,80 +597,68 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
         for (int ky = 0; ky < g.KH; ky++)
             for (int kx = 0; kx < g.KW; kx++, k++) {
                 tab[2 * k + 0] = ((c * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
-                tab[2 * k + 1] = (mask == MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << (ky * g.KW + kx));
+                tab[2 * k + 1] = (p.mask == GEMM_MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << (ky * g.KW + kx));
             }
-    if (mask == MASK_ROWCOL)
+    if (p.mask == GEMM_MASK_ROWCOL)
         for (; 2 * k + 1 < words; k++)
             tab[2 * k + 1] = 31 | (31 << 8); // bit 31 of the row / column masks is never set
 }
 
-static void fill_dims(const ConvGeom &g, GemmArgs &a, int n_valid)
-{
-    a.M = g.Cout / g.groups;
-    a.N = g.B * g.OH * g.OW;
-    if (n_valid >= 0 && n_valid < a.N)
-        a.N = n_valid;
-    a.K = (g.Cin / g.groups) * g.KH * g.KW;
-    a.nkt = k_tiles(g);
-    a.Cout = g.Cout;
-    a.groups = g.groups;
-}
-
-template <class F>
-static auto with_tile(int choice, F &&f)
-{
-    switch (choice) {
-    case 1: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
-    case 2: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
-    case 3: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
-    case 5: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 256>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
-    case 7: return f(std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
-    case 8: return f(std::integral_constant<int, 32>{}, std::integral_constant<int, 256>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
-    case 9: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
-    default: return f(std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
-    }
-}
-
-// Workspace the split-K path wants for this geometry (0 when it would not split).
-size_t conv_gemm_workspace_bytes(const ConvGeom &g)
+size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
 {
     if (g.B <= 0)
         return 0;
+    const GemmPlan p = conv_gemm_plan(g, activation);
     GemmArgs a;
-    fill_dims(g, a, -1);
-    a.part = (float *)16; // any non-null value: ask for the unconstrained plan
-    with_tile(tile_choice(a.M), [&](auto bm, auto bn, auto, auto) {
-        plan_split<decltype(bm)::value, decltype(bn)::value>(a, g.groups, (size_t)-1);
-        return 0;
-    });
-    return a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0;
+    a.N = g.B * g.OH * g.OW;
+    a.Cout = g.Cout;
+    a.nkt = p.nkt;
+    plan_split(p, a, g.groups, true, (size_t)-1);
+    return p.wpack_bytes + (a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0);
 }
 
-int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *ws, size_t ws_bytes)
+int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream)
+{
+    const long long total = (long long)g.groups * p.mtiles * p.nkt * BK * p.BM;
+    if (total >= 0x7fffffffLL * 256)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
+    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups, g.Cin / g.groups,
+                       g.KH * g.KW, (const float *)w, (float *)wpacked);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes)
 {
     if (g.dtype != DLP_FLOAT)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: only float_data is implemented");
     DLP_REQUIRE(g.KH <= 31 && g.KW <= 31, "kernel extent above 31 is not supported by the gather masks");
     const size_t x_elems = (size_t)g.B * g.Cin * g.H * g.W;
-    const size_t w_elems = (size_t)g.Cout * (g.Cin / g.groups) * g.KH * g.KW;
     const size_t y_elems = (size_t)g.B * g.Cout * g.OH * g.OW;
     const size_t x_shift = ((size_t)g.ph * g.W + g.pw) * 4;
-    if (x_elems * 4 + x_shift >= kOutOfRange || w_elems * 4 >= kOutOfRange || y_elems >= 0x7fffffffULL)
+    if (x_elems * 4 + x_shift >= kOutOfRange || p.wpack_bytes >= kOutOfRange || y_elems >= 0x7fffffffULL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
 
     GemmArgs a;
     a.x = (const float *)x;
-    a.w = (const float *)w;
+    a.wp = (const float *)wpacked;
     a.bias = ep.bias;
     a.y = (float *)y;
     a.ktab = (const int32_t *)dev_ktab;
-    fill_dims(g, a, n_valid);
+    a.M = p.M;
+    a.K = p.K;
+    a.nkt = p.nkt;
+    a.N = g.B * g.OH * g.OW;
+    if (n_valid >= 0 && n_valid < a.N)
+        a.N = n_valid;
     if (a.N == 0)
         return DLP_OK;
-    a.part = (float *)ws;
+    a.Cout = g.Cout;
+    a.groups = g.groups;
+    a.part = (float *)part_ws;
     a.Cin = g.Cin;
     a.Cin_g = g.Cin / g.groups;
     a.H = g.H;
@@ -656,7 +668,7 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw; a.dh = g.dh; a.dw = g.dw;
     a.KH = g.KH; a.KW = g.KW;
     a.x_bytes = (uint32_t)(x_elems * 4);
-    a.w_bytes = (uint32_t)(w_elems * 4);
+    a.wp_bytes = (uint32_t)p.wpack_bytes;
     a.x_shift = (uint32_t)x_shift;
     a.hw4 = (uint32_t)(g.H * g.W * 4);
     make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
@@ -670,12 +682,10 @@ int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x
     if (ep.activation == DLP_ACT_RELU6)
         a.clamp_hi = 6.0f;
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
-    int order, mask;
-    gather_mode(g, ep.activation, order, mask); // same rule the gather table was built with
+    plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
 
-    return with_tile(tile_choice(a.M), [&](auto bm, auto bn, auto wm, auto wn) {
-        return launch_tile<decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, a, order, mask, act,
-                                                                                                                    ws_bytes, stream);
+    return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
+        return launch_tile<decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);
     });
 }
 

@@ -15,7 +15,7 @@
 // launch (16 groups of a 1x1 "convolution" over a T x 1 image).  U, V and M live
 // in the workspace; the batch is processed in chunks sized so that V and M of a
 // chunk stay resident in the on-package caches between the three stages.
-//   workspace = U[16][Cout][Cin] | V[16][Cin][Tcap] | M[16][Cout][Tcap]   (floats)
+//   workspace = U (packed GEMM tile order) | V[16][Cin][Tcap] | M[16][Cout][Tcap]   (floats)
 // All loads and stores of the transform kernels have consecutive lanes on
 // consecutive tiles / channels, so HBM and workspace traffic is coalesced.
 #include "dlp_internal.hpp"
@@ -49,33 +49,47 @@ WinoShape wino_shape(const ConvGeom &g, const WinoPlan &plan, int batch)
     return s;
 }
 
-// U[e][n][c] = (G k G^T)[e], src/kernels/winograd_fwd.cl:103-135
-__global__ __launch_bounds__(256) void wino_filter_kernel(int N, int C, const float *__restrict__ w, float *__restrict__ U)
+// U_e[n][c] = (G k G^T)[e], src/kernels/winograd_fwd.cl:103-135, written straight into
+// the packed A layout of the GEMM stage: [e][m tile][K tile][k][m in tile], zero padded.
+__global__ __launch_bounds__(256) void wino_filter_kernel(int N, int C, GemmPlan p, const float *__restrict__ w, float *__restrict__ U)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x; // n*C + c
-    if (idx >= N * C)
+    const int npad = p.mtiles * p.BM, cpad = p.nkt * 16;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x; // n * cpad + c over the padded domain
+    if (idx >= npad * cpad)
         return;
-    const float *kp = w + (size_t)idx * 9;
-    float k[9];
+    const int n = idx / cpad, c = idx - n * cpad;
+    float u[16];
 #pragma unroll
-    for (int i = 0; i < 9; i++)
-        k[i] = kp[i];
-    float gk[3][4];
+    for (int e = 0; e < 16; e++)
+        u[e] = 0.0f;
+    if (n < N && c < C) {
+        const float *kp = w + ((size_t)n * C + c) * 9;
+        float k[9];
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
-        gk[j][0] = k[j];
-        gk[j][1] = 0.5f * (k[j] + k[3 + j] + k[6 + j]);
-        gk[j][2] = 0.5f * (k[j] - k[3 + j] + k[6 + j]);
-        gk[j][3] = k[6 + j];
+        for (int i = 0; i < 9; i++)
+            k[i] = kp[i];
+        float gk[3][4];
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            gk[j][0] = k[j];
+            gk[j][1] = 0.5f * (k[j] + k[3 + j] + k[6 + j]);
+            gk[j][2] = 0.5f * (k[j] - k[3 + j] + k[6 + j]);
+            gk[j][3] = k[6 + j];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            u[4 * i + 0] = gk[0][i];
+            u[4 * i + 1] = 0.5f * (gk[0][i] + gk[1][i] + gk[2][i]);
+            u[4 * i + 2] = 0.5f * (gk[0][i] - gk[1][i] + gk[2][i]);
+            u[4 * i + 3] = gk[2][i];
+        }
     }
-    const size_t estride = (size_t)N * C;
+    // group e, m tile n / BM, K tile c / 16 (1x1 "kernel": both K orders coincide)
+    const size_t in_group = ((size_t)(n / p.BM) * p.nkt + c / 16) * (16 * p.BM) + (size_t)(c % 16) * p.BM + n % p.BM;
+    const size_t estride = (size_t)p.mtiles * p.nkt * 16 * p.BM;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        U[(size_t)(4 * i + 0) * estride + idx] = gk[0][i];
-        U[(size_t)(4 * i + 1) * estride + idx] = 0.5f * (gk[0][i] + gk[1][i] + gk[2][i]);
-        U[(size_t)(4 * i + 2) * estride + idx] = 0.5f * (gk[0][i] - gk[1][i] + gk[2][i]);
-        U[(size_t)(4 * i + 3) * estride + idx] = gk[2][i];
-    }
+    for (int e = 0; e < 16; e++)
+        U[(size_t)e * estride + in_group] = u[e];
 }
 
 // V[e][c][t] = (B^T d B)[e] for tile t of channel c, src/kernels/winograd_fwd.cl:35-69
@@ -186,7 +200,6 @@ WinoPlan winograd_plan(const ConvGeom &g)
         imgs = hint;
     p.chunk_imgs = (int)imgs;
     p.tcap = p.chunk_imgs * tiles_per_img;
-    p.ws_bytes = sizeof(float) * 16 * ((size_t)g.Cin * g.Cout + (size_t)p.tcap * ((size_t)g.Cin + g.Cout));
     ConvGeom &q = p.gemm;
     q.B = 1;
     q.Cin = 16 * g.Cin;
@@ -201,6 +214,8 @@ WinoPlan winograd_plan(const ConvGeom &g)
     q.dh = q.dw = 1;
     q.groups = 16;
     q.dtype = DLP_FLOAT;
+    p.gplan = conv_gemm_plan(q, DLP_ACT_IDENTITY);
+    p.ws_bytes = p.gplan.wpack_bytes + sizeof(float) * 16 * (size_t)p.tcap * ((size_t)g.Cin + g.Cout);
     return p;
 }
 
@@ -214,12 +229,12 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *ge
     const WinoShape s = wino_shape(g, plan, g.B);
 
     float *U = (float *)ws;
-    float *V = U + (size_t)16 * g.Cin * g.Cout;
+    float *V = (float *)((char *)ws + plan.gplan.wpack_bytes);
     float *Mw = V + (size_t)16 * g.Cin * s.tcap;
 
     {
-        const int total = g.Cout * g.Cin;
-        hipLaunchKernelGGL(wino_filter_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, g.Cout, g.Cin, (const float *)w, U);
+        const int total = plan.gplan.mtiles * plan.gplan.BM * plan.gplan.nkt * 16;
+        hipLaunchKernelGGL(wino_filter_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, g.Cout, g.Cin, plan.gplan, (const float *)w, U);
     }
     Epilogue none;
     none.bias = nullptr;
@@ -232,7 +247,7 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *ge
             const long long total = (long long)g.Cin * T;
             hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, s, b0, nb, (const float *)x, V);
         }
-        int rc = conv_gemm_launch(plan.gemm, gemm_ktab, V, U, Mw, none, stream, T);
+        int rc = conv_gemm_launch(plan.gemm, plan.gplan, gemm_ktab, V, U, Mw, none, stream, T);
         if (rc != DLP_OK)
             return rc;
         {

@@ -39,12 +39,16 @@ struct dlp_conv2d_fwd {
     size_t workspace;
 };
 
+static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
 struct dlp_ip_fwd {
     dlp_ip_settings cfg;
     bool bias;
     int activation;
     int device;
     KTabEntry *ktab;
+    GemmPlan plan;
+    void *wpacked; // op-owned: IPForward::enqueue has no workspace argument
 };
 
 static int upload_ktab(const ConvGeom &g, int activation, KTabEntry **out)
@@ -240,7 +244,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
-        op->workspace = conv_gemm_workspace_bytes(g);
+        op->workspace = conv_gemm_workspace_bytes(g, activation);
         rc = upload_ktab(g, activation, &op->ktab);
     } else if (chosen == ALGO_WINOGRAD) {
         op->wino = winograd_plan(g);
@@ -299,8 +303,17 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
         return winograd_launch(g, op->wino, op->ktab, x, w, y, ws, ws_bytes, ep, s);
     case ALGO_DEPTHWISE:
         return depthwise_launch(g, x, w, y, ep, s);
-    default:
-        return conv_gemm_launch(g, op->ktab, x, w, y, ep, s, -1, ws, ws_bytes);
+    default: {
+        // workspace = packed weights | split-K partial sums
+        const GemmPlan plan = conv_gemm_plan(g, op->activation);
+        DLP_REQUIRE(ws != nullptr && ws_bytes >= plan.wpack_bytes, "workspace smaller than workspace()");
+        rc = conv_gemm_pack_weights(g, plan, w, ws, s);
+        if (rc != DLP_OK)
+            return rc;
+        const size_t used = round256(plan.wpack_bytes);
+        void *part = ws_bytes > used ? (char *)ws + used : nullptr;
+        return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0);
+    }
     }
 }
 
@@ -330,8 +343,15 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
     op->ktab = nullptr;
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
-    int rc = upload_ktab(ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype), activation, &op->ktab);
+    const ConvGeom g1 = ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype);
+    op->plan = conv_gemm_plan(g1, activation);
+    op->wpacked = nullptr;
+    int rc = upload_ktab(g1, activation, &op->ktab);
+    if (rc == DLP_OK && hipMalloc(&op->wpacked, op->plan.wpack_bytes) != hipSuccess)
+        rc = fail(DLP_ERR_RUNTIME, "hipMalloc(packed weights) failed");
     if (rc != DLP_OK) {
+        if (op->ktab)
+            (void)hipFree(op->ktab);
         delete op;
         return rc;
     }
@@ -351,8 +371,11 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
     ep.bias = (const float *)bias;
     ep.factor = 0.0f; // src/core/ip.cpp:38
     ep.activation = op->activation;
-    return conv_gemm_launch(ip_gemm_geom(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype), op->ktab, x, w, y, ep,
-                            (hipStream_t)stream);
+    const ConvGeom g = ip_gemm_geom(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype);
+    int rc = conv_gemm_pack_weights(g, op->plan, w, op->wpacked, (hipStream_t)stream);
+    if (rc != DLP_OK)
+        return rc;
+    return conv_gemm_launch(g, op->plan, op->ktab, x, op->wpacked, y, ep, (hipStream_t)stream);
 }
 
 void dlp_ip_fwd_destroy(dlp_ip_fwd *op)
@@ -361,6 +384,8 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op)
         return;
     if (op->ktab)
         (void)hipFree(op->ktab);
+    if (op->wpacked)
+        (void)hipFree(op->wpacked);
     delete op;
 }
 

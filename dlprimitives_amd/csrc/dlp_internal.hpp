@@ -69,23 +69,42 @@ __device__ __forceinline__ void store_out(float *p, float v, float factor)
 }
 
 // ---- implicit-GEMM convolution (conv_gemm.hip) ------------------------------
-// Per-k gather table entry: element offset of tap (c,ky,kx) inside one image's
-// group slice, and the tap coordinates for the padding mask.
+// Gather table entry (8 bytes).  Channel-major K order: one entry per k = {byte offset
+// of tap (c,ky,kx) inside one image's group slice, tap bit or ky|kx<<8}.  Tap-major K
+// order: two entries per K tile = {byte offset of (channel block, tap), tap bit, -, -}.
 struct KTabEntry {
     int32_t offset;
-    int32_t tap; // tap bit (1 << (ky*KW+kx)), or ky | (kx << 8) for large kernels; padding entries never match
+    int32_t tap;
 };
+
+// K ordering: k = (c,ky,kx) with a per-element table, or one tap x 16 channels per K tile
+enum { GEMM_ORDER_CHANNEL = 0, GEMM_ORDER_TAP = 1 };
+// In-image test: one bit per tap (KH*KW <= 32) or separate row / column masks
+enum { GEMM_MASK_TAPS = 1, GEMM_MASK_ROWCOL = 2 };
+
+// Everything about a GEMM launch that is fixed by geometry + activation
+// (the batch only changes the number of N tiles and the split-K factor).
+struct GemmPlan {
+    int order, mask;
+    int tile, BM, BN;   // workgroup tile
+    int M, K, nkt;      // per group: rows, reduction length, K tiles of 16
+    int mtiles;         // ceil(M / BM)
+    size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded
+};
+GemmPlan conv_gemm_plan(const ConvGeom &g, int activation);
 size_t conv_gemm_ktab_entries(const ConvGeom &g);
 // The table layout depends on the geometry AND on the activation the op was created with.
 void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *host_tab);
-// Workspace (bytes) with which the launch may split the K dimension over several
-// workgroups when there are too few output tiles to fill the chip; 0 = never splits.
-size_t conv_gemm_workspace_bytes(const ConvGeom &g);
+// Workspace (bytes) of a convolution run through this path: packed weights, plus the
+// split-K partial sums when there are too few output tiles to fill the chip.
+size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation);
+// Repack [Cout][Cin/groups][KH][KW] weights into the tile order the kernel loads.
+int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
-// ws/ws_bytes: optional split-K workspace; without it the launch runs unsplit.
-int conv_gemm_launch(const ConvGeom &g, const KTabEntry *dev_ktab, const void *x, const void *w,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *ws = nullptr,
-                     size_t ws_bytes = 0);
+// part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.
+int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *part_ws = nullptr,
+                     size_t part_bytes = 0);
 
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);
@@ -97,6 +116,7 @@ struct WinoPlan {
     int tcap;        // tiles per pass = row stride of the V and M workspace matrices
     size_t ws_bytes; // workspace() of the op
     ConvGeom gemm;   // grouped 1x1 geometry that runs the 16 GEMMs of a pass
+    GemmPlan gplan;  // its launch plan (the filter transform writes the packed layout directly)
 };
 bool winograd_supported(const ConvGeom &g);
 WinoPlan winograd_plan(const ConvGeom &g); // g.B = batch hint

@@ -71,9 +71,9 @@ def test_resnet18_layer_shapes(gpu, oracle_mod, layer):
     np.testing.assert_allclose(got, want, **TOL)
 
 
-def test_split_k_with_and_without_workspace(gpu, oracle_mod):
-    # few output tiles, long K: the launch splits K over several workgroups when it is
-    # given workspace() bytes, and must give the same answer unsplit when it is not
+def test_split_k_through_workspace(gpu, oracle_mod):
+    # few output tiles, long K: the launch splits K over several workgroups and reduces the
+    # partial sums from the workspace; a missing workspace is a validation error
     import torch
 
     import dlprimitives_amd as dlp
@@ -85,11 +85,12 @@ def test_split_k_with_and_without_workspace(gpu, oracle_mod):
     op = dlp.Conv2DForward.create(st, True, "relu", "gemm")
     assert op.workspace() > 0
     xd, wd, bd = gpu.dev(x), gpu.dev(w), gpu.dev(bias)
-    for ws in (torch.empty(op.workspace(), dtype=torch.uint8, device="cuda:0"), None):
-        y = torch.full(want.shape, float("nan"), device="cuda:0")
-        op.enqueue(xd, wd, bd, y, ws, 0.0)
-        torch.cuda.synchronize()
-        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+    y = torch.full(want.shape, float("nan"), device="cuda:0")
+    op.enqueue(xd, wd, bd, y, torch.empty(op.workspace(), dtype=torch.uint8, device="cuda:0"), 0.0)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+    with pytest.raises(dlp.ValidationError):
+        op.enqueue(xd, wd, bd, y, None, 0.0)
     old = np.random.default_rng(0).standard_normal(want.shape).astype(np.float32)
     y = gpu.dev(old)
     op.enqueue(xd, wd, bd, y, torch.empty(op.workspace(), dtype=torch.uint8, device="cuda:0"), 0.25)
