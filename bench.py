@@ -1,20 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the convolution forward hot path on one MI355X.
 
-Workload (the configuration the headline metric is quoted on): the 20 convolutions
-of the ResNet-18 conv stack, forward, fp32 NCHW, batch 64, BN folded into
-weights + bias, fused ReLU, algorithm "gemm" (implicit GEMM on fp32 MFMA).
-A step = one pass over all 20 layers, launched back to back on one stream, with
-every tensor already resident in HBM.  Synthetic data: inputs uniform[-1,1],
-weights Kaiming-normal, bias uniform[-0.1,0.1], fixed seed.
+Default workload (the configuration the headline metric is quoted on): the 20
+convolutions of the ResNet-18 conv stack, forward, fp32 NCHW, batch 64, BN folded
+into weights + bias, fused ReLU, algorithm "gemm" (implicit GEMM on fp32 MFMA).
+A step = one pass over all layers of the workload, launched back to back on one
+stream, with every tensor already resident in HBM.  Synthetic data: inputs
+uniform[-1,1], weights Kaiming-normal, bias uniform[-0.1,0.1], fixed seed.
 
-Prints ONE JSON line.  `value` = images/s of the whole stack; `gflops_per_s` is the
-same run expressed with the reference's flop accounting (tools/flops.cpp:660).
-`roofline` describes the kernel instantiation that takes the largest share of a
-step; per-launch durations are measured with HIP events on the launch stream in a
-second pass with one event pair per launch.  `cpu_baseline` is the CPU oracle
-(a restatement of the reference's single-threaded im2col + sgemm CPU path) timed
-on this host on a bounded sample of the same workload.
+Other workloads (same JSON contract, for the remaining configurations):
+  --workload mobilenet      depthwise 3x3 stride 1/2 (HBM bound) + 1x1 pointwise, ReLU6
+  --workload winograd       the two Winograd shapes, algo winograd
+  --workload winograd-gemm  the same two shapes through the implicit GEMM
+
+Prints ONE JSON line.  `value` = images/s of the whole workload; `gflops_per_s` is
+the same run expressed with the reference's flop accounting (tools/flops.cpp:660).
+`roofline` describes the kernel class that takes the largest share of a step;
+per-launch durations are measured with HIP events on the launch stream in a
+second pass with one event pair per layer.  `cpu_baseline` is the CPU oracle (a
+restatement of the reference's single-threaded im2col + sgemm CPU path) timed on
+this host on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -30,16 +35,37 @@ HBM_PEAK_GBS = 8000.0
 BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 images/sec"
 
 
-def build_layers(batch, seed, algo, activation_all_relu=True):
+def workload_layers(name):
+    from dlprimitives_amd.workloads import MOBILENET_DEPTHWISE, MOBILENET_POINTWISE, RESNET18_CONVS, WINOGRAD_SHAPES, conv
+
+    if name == "resnet18":
+        return [dict(L, algo="gemm") for L in RESNET18_CONVS], "ResNet-18 conv stack forward: 20 convs, BN folded, fused ReLU, algo gemm"
+    if name == "mobilenet":
+        layers = []
+        for (c, hw) in MOBILENET_DEPTHWISE:
+            for s in (1, 2):
+                layers.append(dict(conv("dw3x3s%d_c%d_at%d" % (s, c, hw), 3, s, 1, c, c, hw, groups=c, activation="relu6"),
+                                   algo="depthwise_separable"))
+        for (ci, co, hw) in MOBILENET_POINTWISE:
+            layers.append(dict(conv("pw1x1_%dto%d_at%d" % (ci, co, hw), 1, 1, 0, ci, co, hw, activation="relu6"), algo="gemm"))
+        return layers, "MobileNet-v2 style blocks: depthwise 3x3 stride 1 and 2 + 1x1 pointwise, ReLU6"
+    if name in ("winograd", "winograd-gemm"):
+        algo = "winograd" if name == "winograd" else "gemm"
+        layers = [dict(conv("3x3_%dto%d_at%d" % (ci, co, hw), 3, 1, 1, ci, co, hw), algo=algo) for (_, ci, co, hw) in WINOGRAD_SHAPES]
+        return layers, "Winograd configuration shapes (3x3 s1 p1), algo %s" % algo
+    raise SystemExit("unknown workload " + name)
+
+
+def build_layers(layer_list, batch, seed):
     import numpy as np
     import torch
 
     import dlprimitives_amd as dlp
-    from dlprimitives_amd.workloads import RESNET18_CONVS, conv_bytes, conv_flops
+    from dlprimitives_amd.workloads import conv_bytes, conv_flops
 
     rng = np.random.default_rng(seed)
     out = []
-    for L in RESNET18_CONVS:
+    for L in layer_list:
         cin_g = L["cin"] // L["groups"]
         x = torch.from_numpy(rng.uniform(-1, 1, (batch, L["cin"], L["hw"], L["hw"])).astype(np.float32)).cuda()
         w = torch.from_numpy((rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) *
@@ -47,41 +73,46 @@ def build_layers(batch, seed, algo, activation_all_relu=True):
         b = torch.from_numpy(rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)).cuda()
         y = torch.empty((batch, L["cout"], L["ohw"], L["ohw"]), dtype=torch.float32, device="cuda")
         st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], tuple(x.shape))
-        op = dlp.Conv2DForward.create(st, True, "relu", algo)
+        op = dlp.Conv2DForward.create(st, True, L["activation"], L["algo"])
+        assert op.algo() == L["algo"], (op.algo(), L["algo"])
         ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
         out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch)))
     return out
 
 
 def kernel_class(L):
-    """Which kernel instantiation serves a layer (tile selection is by Cout per group)."""
+    """Which kernel serves a layer."""
+    if L["algo"] == "depthwise_separable":
+        return "depthwise3x3<stride %d>" % L["stride"]
+    if L["algo"] == "winograd":
+        return "winograd(filter+input+gemm+output)"
     m = L["cout"] // L["groups"]
     return "conv_gemm_f32<64x64>" if m > 32 else "conv_gemm_f32<32x128>"
 
 
-def cpu_baseline(images, seed):
-    """Oracle (port of the reference CPU path), 1 thread, `images` images through all 20 layers."""
+def cpu_baseline(layer_list, images, seed):
+    """Oracle (port of the reference CPU path), 1 thread, `images` images through all layers."""
     import numpy as np
 
     import oracle
-    from dlprimitives_amd.workloads import RESNET18_CONVS, conv_flops
+    from dlprimitives_amd.workloads import conv_flops
 
     rng = np.random.default_rng(seed)
     total = 0.0
     flops = 0.0
-    for L in RESNET18_CONVS:
+    for L in layer_list:
         cin_g = L["cin"] // L["groups"]
         x = rng.uniform(-1, 1, (images, L["cin"], L["hw"], L["hw"])).astype(np.float32)
         w = (rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) * np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)
         b = rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)
         cfg = oracle.make_cfg(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"])
         t0 = time.perf_counter()
-        oracle.conv2d_forward(x, w, b, cfg, "relu", threads=1)
+        oracle.conv2d_forward(x, w, b, cfg, L["activation"], threads=1)
         total += time.perf_counter() - t0
         flops += conv_flops(L, images)
-    return dict(value=images / total, unit="images/s", cores=1, kind="port",
-                sample="%d of 64 images through all 20 ResNet-18 conv layers, single thread, %.1f s" % (images, total),
-                gflops_per_s=flops / total / 1e9)
+    return dict(value=round(images / total, 3), unit="images/s", cores=1, kind="port",
+                sample="%d images through all %d layers of the workload, single thread, %.1f s" % (images, len(layer_list), total),
+                gflops_per_s=round(flops / total / 1e9, 2))
 
 
 def main():
@@ -90,8 +121,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--algo", default="gemm")
-    ap.add_argument("--cpu-images", type=int, default=4, help="images of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenet", "winograd", "winograd-gemm"])
+    ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
     args = ap.parse_args()
@@ -109,12 +140,13 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
-    layers = build_layers(args.batch, 2024, args.algo)
+    layer_list, description = workload_layers(args.workload)
     if args.only:
-        layers = [e for e in layers if args.only in e["layer"]["name"]]
-        if not layers:
+        layer_list = [L for L in layer_list if args.only in L["name"]]
+        if not layer_list:
             print("bench.py: --only matches no layer", file=sys.stderr)
             sys.exit(2)
+    layers = build_layers(layer_list, args.batch, 2024)
     stream = torch.cuda.current_stream()
 
     def step():
@@ -131,8 +163,9 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     total_flops = sum(e["flops"] for e in layers)
+    total_bytes = sum(e["bytes"] for e in layers)
 
-    # second pass: one HIP event pair per launch, on the launch stream
+    # second pass: one HIP event pair per layer, on the launch stream
     nl = len(layers)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(nl + 1)] for _ in range(args.steps)]
     for s in range(args.steps):
@@ -148,27 +181,33 @@ def main():
     for e, ms in zip(layers, layer_ms):
         L = e["layer"]
         ai = e["flops"] / e["bytes"]
+        mfma_bound = ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12
         roof = min(FP32_MATRIX_PEAK_TFLOPS * 1e12, ai * HBM_PEAK_GBS * 1e9)
         ach = e["flops"] / (ms * 1e-3)
         table.append(dict(name=L["name"], ms=round(ms, 4), tflops=round(ach / 1e12, 2), gbs=round(e["bytes"] / (ms * 1e-3) / 1e9, 1),
-                          bound="mfma" if ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12 else "hbm",
-                          frac_of_roofline=round(ach / roof, 4), kernel=kernel_class(L)))
-        c = classes.setdefault(kernel_class(L), dict(ms=0.0, flops=0.0, launches=0))
+                          bound="mfma" if mfma_bound else "hbm", frac_of_roofline=round(ach / roof, 4), kernel=kernel_class(L)))
+        c = classes.setdefault(kernel_class(L), dict(ms=0.0, flops=0.0, bytes=0.0, launches=0, hbm=0))
         c["ms"] += ms
         c["flops"] += e["flops"]
+        c["bytes"] += e["bytes"]
         c["launches"] += 1
+        c["hbm"] += 0 if mfma_bound else 1
     dom_name, dom = max(classes.items(), key=lambda kv: kv[1]["ms"])
-    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel=dom_name, launches_per_step=dom["launches"],
-                    avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
-                    flops_per_launch=dom["flops"] / dom["launches"],
-                    achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS, unit="TFLOP/s",
-                    frac=round(achieved / FP32_MATRIX_PEAK_TFLOPS, 4), traffic=None)
+    if dom["hbm"] * 2 > dom["launches"]:  # a bandwidth-bound kernel class: score achieved bytes/s
+        achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
+        roofline = dict(bound="hbm", kernel=dom_name, launches_per_step=dom["launches"], avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
+                        bytes_per_launch=dom["bytes"] / dom["launches"], achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                        frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
+    else:
+        achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+        roofline = dict(bound="mfma", kernel=dom_name, launches_per_step=dom["launches"], avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
+                        flops_per_launch=dom["flops"] / dom["launches"], achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS,
+                        unit="TFLOP/s", frac=round(achieved / FP32_MATRIX_PEAK_TFLOPS, 4), traffic=None)
     if args.layers:
         for r in table:
             print(json.dumps(r), file=sys.stderr)
 
-    cpu = cpu_baseline(args.cpu_images, 2024) if args.cpu_images > 0 else None
+    cpu = cpu_baseline(layer_list, args.cpu_images, 2024) if args.cpu_images > 0 else None
 
     out = {
         "metric": BASELINE_METRIC,
@@ -183,9 +222,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "ResNet-18 conv stack forward: %d convs%s, fp32 NCHW, batch %d, BN folded, fused ReLU, algo %s" %
-                   (nl, " (subset --only %s)" % args.only if args.only else "", args.batch, args.algo),
-                   "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1)},
+        "config": {"workload": "%s%s, fp32 NCHW, batch %d" % (description, " (subset --only %s)" % args.only if args.only else "", args.batch),
+                   "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1),
+                   "mbytes_per_step": round(total_bytes / 1e6, 1)},
         "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_fp32_matrix_peak": round(total_flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
         "event_ms_per_step": round(sum(layer_ms), 4),

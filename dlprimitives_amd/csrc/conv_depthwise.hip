@@ -6,24 +6,29 @@
 // grouped GEMM with M = 1 there, src/core/conv.cpp:725-727).
 //
 // The op is HBM-bound (about 2 flop per byte), so no matrix cores: the kernel is
-// organised around reading every input element exactly once and writing every
-// output exactly once, in wide contiguous runs.
+// organised around reading every input element once (plus a two-row halo per strip)
+// and writing every output exactly once, in wide contiguous runs, with enough
+// loads in flight per CU to cover the HBM latency.
 //
-// 3x3 kernel, lanes own output columns.  The (plane, column) pairs of the whole
-// tensor are laid on one flat axis; a wavefront covers 64 consecutive pairs and
-// walks down the rows keeping a three-row register window.  Each lane loads only
-// the input columns it owns; the columns to its left/right come from the
+// 3x3 kernel, lanes own output columns.  The (plane, row strip, column) triples of
+// the whole tensor are laid on one flat axis; a wavefront covers 64 consecutive
+// ones.  A lane produces a strip of 7 output rows of its column: it first issues
+// the loads of ALL input rows the strip needs (9 at stride 1, 15 at stride 2), so a
+// wavefront has 9-30 independent loads in flight, then computes.  Each lane loads
+// only the input columns it owns; the columns to its left/right come from the
 // neighbouring lanes through wavefront shuffles.  Lanes at the edge of the
 // wavefront are halo lanes: they load and feed their neighbours but store
 // nothing, and adjacent wavefronts overlap by the halo, so there is no
 // divergent patch-up load.  Accumulation order is the reference's:
 // sum = bias; sum = fma(k[dr][dc], x, sum) for dr, dc ascending.
 //
-// Other odd kernel sizes (stride 1) use a plain direct kernel.
+// Other odd kernel sizes use a plain direct kernel.
 #include "dlp_internal.hpp"
 
 namespace dlp {
 namespace {
+
+constexpr int kStripRows = 7; // divides the usual 56/28/14/7 feature maps
 
 struct DwArgs {
     const float *x;
@@ -32,7 +37,8 @@ struct DwArgs {
     float *y;
     int planes; // B*C
     int C, H, W, OH, OW;
-    long long total_cols; // planes * OW
+    int nstrips;          // ceil(OH / kStripRows)
+    long long total_cols; // planes * nstrips * OW
     float factor;
     int act;
 };
@@ -43,14 +49,18 @@ template <int STRIDE>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
 {
     constexpr int OUT_PER_WAVE = (STRIDE == 1) ? 62 : 63;
+    constexpr int NIN = (kStripRows - 1) * STRIDE + 3; // input rows of a strip
     const int lane = threadIdx.x & 63;
     const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const long long f = wave * OUT_PER_WAVE + lane - 1; // flat (plane, ox) index
+    const long long f = wave * OUT_PER_WAVE + lane - 1; // flat (plane, strip, ox) index
     const bool in_range = f >= 0 && f < a.total_cols;
-    const int plane = in_range ? (int)(f / a.OW) : 0;
-    const int ox = in_range ? (int)(f - (long long)plane * a.OW) : 0;
+    const long long ps = in_range ? f / a.OW : 0;
+    const int ox = in_range ? (int)(f - ps * a.OW) : 0;
+    const int plane = (int)(ps / a.nstrips);
+    const int strip = (int)(ps - (long long)plane * a.nstrips);
     const bool is_out = in_range && lane >= 1 && (STRIDE == 2 || lane <= 62);
     const int c = plane % a.C;
+    const int oy0 = strip * kStripRows;
 
     float k[9];
 #pragma unroll
@@ -63,71 +73,51 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
 
     // columns owned by this lane
     const int x0 = ox * STRIDE;
-    const bool v0 = in_range; // x0 < W always holds
     const bool v1 = in_range && (STRIDE == 2) && (x0 + 1 < a.W);
-    const bool has_left = ox > 0;                        // column x0-1 exists in this plane
+    const bool has_left = ox > 0;                           // column x0-1 exists in this plane
     const bool has_right = (STRIDE == 1) && (ox + 1 < a.W); // column x0+1 (stride 1 only)
 
-    // window rows: r[dr][dc] for input columns (x0-1, x0, x0+1)
-    float r0[3], r1[3], r2[3];
-    auto load_row = [&](int yy, float (&row)[3]) {
-        const bool vy = yy >= 0 && yy < a.H;
+    // issue every load of the strip before anything consumes one
+    float c0[NIN], c1[NIN];
+    const int iy0 = oy0 * STRIDE - 1;
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+        const int yy = iy0 + r;
+        const bool vy = in_range && yy >= 0 && yy < a.H;
         const float *p = xp + (size_t)(vy ? yy : 0) * a.W + x0;
-        float c0 = (vy && v0) ? p[0] : 0.0f;
-        float c1 = 0.0f;
+        c0[r] = vy ? p[0] : 0.0f;
+        c1[r] = 0.0f;
         if (STRIDE == 2)
-            c1 = (vy && v1) ? p[1] : 0.0f;
-        if (STRIDE == 1) {
-            float left = __shfl_up(c0, 1);
-            float right = __shfl_down(c0, 1);
-            row[0] = has_left ? left : 0.0f;
-            row[1] = c0;
-            row[2] = has_right ? right : 0.0f;
-        } else {
-            float left = __shfl_up(c1, 1); // previous lane's odd column = 2*ox - 1
-            row[0] = has_left ? left : 0.0f;
-            row[1] = c0;
-            row[2] = c1;
-        }
-    };
-
-    // output row oy uses input rows oy*STRIDE - 1 + {0,1,2}
-    if (STRIDE == 1) {
-        load_row(-1, r0);
-        load_row(0, r1);
-    } else {
-        load_row(-1, r0);
+            c1[r] = (vy && v1) ? p[1] : 0.0f;
     }
-    for (int oy = 0; oy < a.OH; oy++) {
+    // window columns (x0-1, x0, x0+1) of every row
+    float left[NIN], right[NIN];
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
         if (STRIDE == 1) {
-            load_row(oy + 1, r2);
+            const float l = __shfl_up(c0[r], 1);
+            const float rr = __shfl_down(c0[r], 1);
+            left[r] = has_left ? l : 0.0f;
+            right[r] = has_right ? rr : 0.0f;
         } else {
-            load_row(2 * oy, r1);
-            load_row(2 * oy + 1, r2);
+            const float l = __shfl_up(c1[r], 1); // previous lane's odd column = 2*ox - 1
+            left[r] = has_left ? l : 0.0f;
+            right[r] = c1[r];
         }
+    }
+#pragma unroll
+    for (int j = 0; j < kStripRows; j++) {
+        const int oy = oy0 + j;
         float sum = bias;
 #pragma unroll
-        for (int dc = 0; dc < 3; dc++)
-            sum = fmaf(k[dc], r0[dc], sum);
-#pragma unroll
-        for (int dc = 0; dc < 3; dc++)
-            sum = fmaf(k[3 + dc], r1[dc], sum);
-#pragma unroll
-        for (int dc = 0; dc < 3; dc++)
-            sum = fmaf(k[6 + dc], r2[dc], sum);
-        if (is_out)
-            store_out(yp + (size_t)oy * a.OW, apply_act(sum, a.act), a.factor);
-        if (STRIDE == 1) {
-#pragma unroll
-            for (int dc = 0; dc < 3; dc++) {
-                r0[dc] = r1[dc];
-                r1[dc] = r2[dc];
-            }
-        } else {
-#pragma unroll
-            for (int dc = 0; dc < 3; dc++)
-                r0[dc] = r2[dc];
+        for (int dr = 0; dr < 3; dr++) {
+            const int r = j * STRIDE + dr;
+            sum = fmaf(k[3 * dr + 0], left[r], sum);
+            sum = fmaf(k[3 * dr + 1], c0[r], sum);
+            sum = fmaf(k[3 * dr + 2], right[r], sum);
         }
+        if (is_out && oy < a.OH)
+            store_out(yp + (size_t)oy * a.OW, apply_act(sum, a.act), a.factor);
     }
 }
 
@@ -182,7 +172,8 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.W = g.W;
     a.OH = g.OH;
     a.OW = g.OW;
-    a.total_cols = (long long)a.planes * g.OW;
+    a.nstrips = (g.OH + kStripRows - 1) / kStripRows;
+    a.total_cols = (long long)a.planes * a.nstrips * g.OW;
     a.factor = ep.factor;
     a.act = ep.activation;
     if (g.KH == 3) {

@@ -1,0 +1,108 @@
+// dlprim::core::Conv2DForward on the MI355X: same interface as dlprimitives'
+// include/dlprim/core/conv.hpp:17-58, implemented over the C ABI in dlprim_hip.h.
+#pragma once
+#include <memory>
+#include <string>
+
+#include "../context.hpp"
+#include "../tensor.hpp"
+
+namespace dlprim {
+namespace core {
+
+struct Conv2DSettings : public Convolution2DConfigBase {
+    Conv2DSettings(Conv2DSettings const &) = default;
+    Conv2DSettings(Convolution2DConfigBase const &v, Shape s, DataType dt) : Convolution2DConfigBase(v), shape(s), dtype(dt) {}
+
+    Shape shape; // input shape; the batch is a hint rather than a requirement
+    DataType dtype = float_data;
+};
+
+namespace details {
+inline dlp_conv2d_settings to_c(Convolution2DConfigBase const &c, Shape const &in, DataType dt)
+{
+    DLPRIM_CHECK(in.size() == 4);
+    dlp_conv2d_settings s;
+    s.channels_in = c.channels_in;
+    s.channels_out = c.channels_out;
+    for (int i = 0; i < 2; i++) {
+        s.kernel[i] = c.kernel[i];
+        s.stride[i] = c.stride[i];
+        s.dilate[i] = c.dilate[i];
+        s.pad[i] = c.pad[i];
+    }
+    s.groups = c.groups;
+    for (int i = 0; i < 4; i++)
+        s.shape[i] = int(in[i]);
+    s.dtype = int(dt);
+    return s;
+}
+} // namespace details
+
+class Conv2DBase {
+public:
+    virtual ~Conv2DBase() {}
+    virtual char const *algo() const = 0;
+    virtual size_t workspace() { return 0; }
+    static Shape get_output_shape(Convolution2DConfigBase const &config, Shape const &in)
+    {
+        dlp_conv2d_settings s = details::to_c(config, in, float_data);
+        int out[4];
+        dlprim::details::check_status(dlp_conv2d_output_shape(&s, s.shape, out));
+        return Shape(size_t(out[0]), out[1], out[2], out[3]);
+    }
+};
+
+class Conv2DForward : public Conv2DBase {
+public:
+    virtual ~Conv2DForward() {}
+    // y = factor != 0 ? factor * y + act(conv(x, w) + bias) : act(conv(x, w) + bias)
+    // ws: uint8 tensor of at least workspace() bytes; asynchronous on e
+    virtual void enqueue(Tensor &x, Tensor &w, Tensor *bias, Tensor &y, Tensor &ws, float factor, ExecutionContext const &e) = 0;
+    static std::unique_ptr<Conv2DForward> create(Context &ctx, Conv2DSettings const &config, bool bias,
+                                                 StandardActivations activation = StandardActivations::identity,
+                                                 std::string const &algo = std::string());
+};
+
+namespace details {
+class Conv2DForwardHip : public Conv2DForward {
+public:
+    Conv2DForwardHip(Context &ctx, Conv2DSettings const &config, bool bias, StandardActivations activation, std::string const &algo)
+    {
+        if (ctx.is_cpu_context())
+            throw NotImplementedError("core::Conv2DForward needs a device context");
+        ctx.select();
+        dlp_conv2d_settings s = to_c(config, config.shape, config.dtype);
+        dlprim::details::check_status(dlp_conv2d_fwd_create(&s, bias ? 1 : 0, int(activation), algo.c_str(), &op_));
+    }
+    ~Conv2DForwardHip() { dlp_conv2d_fwd_destroy(op_); }
+    Conv2DForwardHip(Conv2DForwardHip const &) = delete;
+    void operator=(Conv2DForwardHip const &) = delete;
+
+    char const *algo() const override { return dlp_conv2d_fwd_algo(op_); }
+    size_t workspace() override { return dlp_conv2d_fwd_workspace(op_); }
+    void enqueue(Tensor &x, Tensor &w, Tensor *bias, Tensor &y, Tensor &ws, float factor, ExecutionContext const &e) override
+    {
+        DLPRIM_CHECK(x.shape().size() == 4);
+        int xs[4];
+        for (int i = 0; i < 4; i++)
+            xs[i] = int(x.shape()[i]);
+        const size_t ws_bytes = workspace() ? ws.memory_size() : 0;
+        dlprim::details::check_status(dlp_conv2d_fwd_enqueue(op_, xs, x.device_ptr(), w.device_ptr(), bias ? bias->device_ptr() : nullptr,
+                                                             y.device_ptr(), ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, factor,
+                                                             e.stream()));
+    }
+
+private:
+    dlp_conv2d_fwd *op_ = nullptr;
+};
+} // namespace details
+
+inline std::unique_ptr<Conv2DForward> Conv2DForward::create(Context &ctx, Conv2DSettings const &config, bool bias,
+                                                            StandardActivations activation, std::string const &algo)
+{
+    return std::unique_ptr<Conv2DForward>(new details::Conv2DForwardHip(ctx, config, bias, activation, algo));
+}
+
+} // namespace core
+} // namespace dlprim

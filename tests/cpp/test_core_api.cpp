@@ -1,0 +1,201 @@
+// Exercises the C++ header layer the way dlprimitives' own callers use dlprim::core
+// (tools/flops.cpp:594-671, src/ops/conv2d.cpp:160-183,235, src/ops/inner_product.cpp:98-104,158):
+// Context -> Tensor -> Conv2DForward::create -> enqueue -> ExecutionContext::finish.
+// Results are compared with a plain direct convolution computed here in double.
+//
+//   test_core_api host   : everything that needs no GPU (shapes, exceptions)
+//   test_core_api <dev>  : the device checks on HIP device <dev> (default 0)
+#include <dlprim/core/conv.hpp>
+#include <dlprim/core/ip.hpp>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+namespace dp = dlprim;
+
+static int failures = 0;
+#define EXPECT(cond)                                                      \
+    do {                                                                  \
+        if (!(cond)) {                                                    \
+            std::printf("FAIL %s:%d %s\n", __FILE__, __LINE__, #cond);    \
+            failures++;                                                   \
+        }                                                                 \
+    } while (0)
+
+static double act(double v, dp::StandardActivations a)
+{
+    switch (a) {
+    case dp::StandardActivations::relu: return v < 0 ? 0 : v;
+    case dp::StandardActivations::relu6: return v < 0 ? 0 : (v > 6 ? 6 : v);
+    case dp::StandardActivations::tanh: return std::tanh(v);
+    case dp::StandardActivations::sigmoid: return 1 / (1 + std::exp(-v));
+    default: return v;
+    }
+}
+
+static void fill(dp::Tensor &t, std::mt19937 &rng, float lo, float hi)
+{
+    std::uniform_real_distribution<float> d(lo, hi);
+    float *p = t.data<float>();
+    for (size_t i = 0; i < t.shape().total_size(); i++)
+        p[i] = d(rng);
+}
+
+static void host_checks()
+{
+    dp::Convolution2DConfigBase c;
+    c.channels_in = 3;
+    c.channels_out = 64;
+    c.kernel[0] = c.kernel[1] = 7;
+    c.stride[0] = c.stride[1] = 2;
+    c.pad[0] = c.pad[1] = 3;
+    dp::Shape out = dp::core::Conv2DBase::get_output_shape(c, dp::Shape(64, 3, 224, 224));
+    EXPECT(out == dp::Shape(64, 64, 112, 112));
+    bool thrown = false;
+    try {
+        dp::core::Conv2DBase::get_output_shape(c, dp::Shape(64, 4, 224, 224));
+    } catch (dp::ValidationError const &) {
+        thrown = true;
+    }
+    EXPECT(thrown);
+    thrown = false;
+    try {
+        dp::Context cpu("cpu");
+        dp::core::Conv2DSettings s(c, dp::Shape(1, 3, 8, 8), dp::float_data);
+        dp::core::Conv2DForward::create(cpu, s, false);
+    } catch (dp::NotImplementedError const &) {
+        thrown = true;
+    }
+    EXPECT(thrown);
+    dp::Shape s(2, 3, 4);
+    EXPECT(s.size() == 3 && s.total_size() == 24 && s.size_no_batch() == 12 && s[-1] == 4);
+    EXPECT(dp::size_of_data_type(dp::float_data) == 4 && dp::size_of_data_type(dp::bfloat16_data) == 2);
+}
+
+static void conv_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int cin, int cout, int hw, int k, int stride, int pad, int groups,
+                      bool bias, dp::StandardActivations a, char const *algo, char const *expect_algo, float factor)
+{
+    dp::Convolution2DConfigBase c;
+    c.channels_in = cin;
+    c.channels_out = cout;
+    c.kernel[0] = c.kernel[1] = k;
+    c.stride[0] = c.stride[1] = stride;
+    c.pad[0] = c.pad[1] = pad;
+    c.groups = groups;
+    dp::Shape in(B, cin, hw, hw);
+    dp::core::Conv2DSettings cfg(c, in, dp::float_data);
+    std::unique_ptr<dp::core::Conv2DForward> conv = dp::core::Conv2DForward::create(ctx, cfg, bias, a, algo);
+    EXPECT(std::strcmp(conv->algo(), expect_algo) == 0);
+    dp::Shape os = dp::core::Conv2DBase::get_output_shape(c, in);
+    dp::Tensor X(ctx, in), W(ctx, dp::Shape(cout, cin / groups, k, k)), Bv(ctx, dp::Shape(cout)), Y(ctx, os);
+    size_t ws_size = conv->workspace();
+    dp::Tensor ws(ctx, dp::Shape(ws_size ? ws_size : 1), dp::uint8_data);
+    std::mt19937 rng(cin * 1000 + cout + hw);
+    fill(X, rng, -1, 1);
+    fill(W, rng, -0.3f, 0.3f);
+    fill(Bv, rng, -0.1f, 0.1f);
+    fill(Y, rng, -1, 1);
+    std::vector<float> y_old(Y.data<float>(), Y.data<float>() + os.total_size());
+    X.to_device(q);
+    W.to_device(q);
+    Bv.to_device(q);
+    Y.to_device(q);
+    conv->enqueue(X, W, bias ? &Bv : nullptr, Y, ws, factor, q);
+    Y.to_host(q);
+    q.finish();
+    const int OH = int(os[2]), OW = int(os[3]), cg = cin / groups, og = cout / groups;
+    const float *x = X.data<float>(), *w = W.data<float>(), *bv = Bv.data<float>(), *y = Y.data<float>();
+    double worst = 0;
+    for (int b = 0; b < B; b++)
+        for (int o = 0; o < cout; o++)
+            for (int oy = 0; oy < OH; oy++)
+                for (int ox = 0; ox < OW; ox++) {
+                    double acc = bias ? bv[o] : 0.0;
+                    const int g = o / og;
+                    for (int ci = 0; ci < cg; ci++)
+                        for (int ky = 0; ky < k; ky++)
+                            for (int kx = 0; kx < k; kx++) {
+                                int iy = oy * stride - pad + ky, ix = ox * stride - pad + kx;
+                                if (iy < 0 || iy >= hw || ix < 0 || ix >= hw)
+                                    continue;
+                                acc += double(x[((size_t(b) * cin + g * cg + ci) * hw + iy) * hw + ix]) * w[((size_t(o) * cg + ci) * k + ky) * k + kx];
+                            }
+                    size_t idx = ((size_t(b) * cout + o) * OH + oy) * OW + ox;
+                    double want = act(acc, a) + double(factor) * y_old[idx];
+                    double err = std::fabs(want - y[idx]) / (1.0 + std::fabs(want));
+                    if (err > worst)
+                        worst = err;
+                }
+    std::printf("conv %-20s b%d %d->%d @%d k%d s%d g%d factor %.2f : max err %.2e\n", expect_algo, B, cin, cout, hw, k, stride, groups, factor,
+                worst);
+    EXPECT(worst < 1e-4);
+}
+
+static void ip_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int in, int out)
+{
+    dp::core::IPSettings cfg;
+    cfg.inputs = in;
+    cfg.outputs = out;
+    cfg.optimal_batch_size = B;
+    std::unique_ptr<dp::core::IPForward> ip = dp::core::IPForward::create(ctx, cfg, true, dp::StandardActivations::relu);
+    dp::Tensor X(ctx, dp::Shape(B, in)), W(ctx, dp::Shape(out, in)), Bv(ctx, dp::Shape(out)), Y(ctx, dp::Shape(B, out));
+    std::mt19937 rng(in + out);
+    fill(X, rng, -1, 1);
+    fill(W, rng, -0.1f, 0.1f);
+    fill(Bv, rng, -0.1f, 0.1f);
+    X.to_device(q);
+    W.to_device(q);
+    Bv.to_device(q);
+    ip->enqueue(X, W, &Bv, Y, q);
+    Y.to_host(q);
+    q.finish();
+    double worst = 0;
+    for (int b = 0; b < B; b++)
+        for (int o = 0; o < out; o++) {
+            double acc = Bv.data<float>()[o];
+            for (int i = 0; i < in; i++)
+                acc += double(X.data<float>()[size_t(b) * in + i]) * W.data<float>()[size_t(o) * in + i];
+            double want = acc < 0 ? 0 : acc;
+            double err = std::fabs(want - Y.data<float>()[size_t(b) * out + o]) / (1.0 + std::fabs(want));
+            if (err > worst)
+                worst = err;
+        }
+    std::printf("ip b%d %d->%d : max err %.2e\n", B, in, out, worst);
+    EXPECT(worst < 1e-4);
+}
+
+int main(int argc, char **argv)
+{
+    std::string dev = argc > 1 ? argv[1] : "0";
+    try {
+        host_checks();
+        if (dev != "host") {
+            dp::Context ctx(dev);
+            std::printf("device: %s\n", ctx.name().c_str());
+            dp::ExecutionContext q = ctx.make_execution_context();
+            using A = dp::StandardActivations;
+            conv_case(ctx, q, 2, 16, 32, 14, 3, 1, 1, 1, true, A::relu, "gemm", "gemm", 0.0f);
+            conv_case(ctx, q, 2, 16, 32, 14, 3, 1, 1, 1, true, A::relu, "", "winograd", 0.0f);
+            conv_case(ctx, q, 2, 3, 8, 20, 7, 2, 3, 1, false, A::identity, "", "gemm", 0.5f);
+            conv_case(ctx, q, 3, 24, 24, 9, 3, 2, 1, 24, true, A::relu6, "", "depthwise_separable", 0.0f);
+            conv_case(ctx, q, 1, 8, 6, 5, 1, 1, 0, 2, true, A::sigmoid, "winograd", "gemm", 0.0f); // incompatible request -> gemm
+            ip_case(ctx, q, 5, 64, 10);
+            // sub-tensor views share memory: run on the second image of a batch-2 tensor
+            dp::Tensor big(ctx, dp::Shape(2, 4, 6, 6));
+            dp::Tensor second = big.sub_tensor(4 * 6 * 6, dp::Shape(1, 4, 6, 6));
+            EXPECT(second.device_offset() == 144 && static_cast<char *>(second.device_ptr()) == static_cast<char *>(big.device_ptr()) + 576);
+        }
+    } catch (std::exception const &e) {
+        std::printf("FAIL exception: %s\n", e.what());
+        return 1;
+    }
+    if (failures) {
+        std::printf("%d failure(s)\n", failures);
+        return 1;
+    }
+    std::printf("ok\n");
+    return 0;
+}
