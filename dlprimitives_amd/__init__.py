@@ -19,4 +19,8 @@ from .capi import (  # noqa: F401
     conv2d_output_shape,
     lib,
     library_path,
+    timing_count,
+    timing_enable,
+    timing_records,
+    timing_reset,
 )

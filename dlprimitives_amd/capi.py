@@ -95,6 +95,33 @@ def lib():
     return _lib
 
 
+def timing_enable(on=True):
+    """ExecutionContext::enable_timing analogue: bracket every kernel launch with HIP events."""
+    _check(lib().dlp_timing_enable(1 if on else 0))
+
+
+def timing_reset():
+    _check(lib().dlp_timing_reset())
+
+
+def timing_count():
+    n = ctypes.c_int()
+    _check(lib().dlp_timing_count(ctypes.byref(n)))
+    return n.value
+
+
+def timing_records(first=0, last=None):
+    """[(section, milliseconds)] of the kernels launched since the last reset (waits for them)."""
+    last = timing_count() if last is None else last
+    out = []
+    name = ctypes.create_string_buffer(64)
+    ms = ctypes.c_float()
+    for i in range(first, last):
+        _check(lib().dlp_timing_get(i, name, 64, ctypes.byref(ms)))
+        out.append((name.value.decode(), ms.value))
+    return out
+
+
 def _check(rc):
     if rc == 0:
         return

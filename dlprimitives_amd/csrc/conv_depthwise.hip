@@ -176,6 +176,7 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.total_cols = (long long)a.planes * a.nstrips * g.OW;
     a.factor = ep.factor;
     a.act = ep.activation;
+    TimingScope ts("sep_conv", stream);
     if (g.KH == 3) {
         const int per_wave = g.sh == 1 ? 62 : 63;
         const long long waves = (a.total_cols + per_wave - 1) / per_wave;

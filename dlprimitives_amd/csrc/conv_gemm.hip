@@ -154,8 +154,17 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     const int h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
 
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumber
+    // them so that every XCD walks one contiguous range of tiles: the m tiles of one pixel
+    // tile, and neighbouring pixel tiles (which share input rows), then hit the same L2.
+    int t;
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, r = nb & 7;
+        const int xcd = bid & 7, slot = bid >> 3;
+        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    }
     // tile decode: m tile fastest, then n tile, then group, then K slice
-    int t = blockIdx.x;
     const int mt = t % a.mtiles;
     t /= a.mtiles;
     const int nt = t % a.ntiles;
@@ -486,8 +495,12 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
-    hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    {
+        TimingScope ts("conv_gemm", stream);
+        hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    }
     if (a.splitk > 1) {
+        TimingScope ts("splitk_reduce", stream);
         const long long total = (long long)a.Cout * a.N;
         hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
     }
@@ -622,6 +635,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
     const long long total = (long long)g.groups * p.mtiles * p.nkt * BK * p.BM;
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
+    TimingScope ts("pack_weights", stream);
     hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups, g.Cin / g.groups,
                        g.KH * g.KW, (const float *)w, (float *)wpacked);
     DLP_HIP_TRY(hipGetLastError());

@@ -233,6 +233,7 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *ge
     float *Mw = V + (size_t)16 * g.Cin * s.tcap;
 
     {
+        TimingScope ts("winograd_filter", stream);
         const int total = plan.gplan.mtiles * plan.gplan.BM * plan.gplan.nkt * 16;
         hipLaunchKernelGGL(wino_filter_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, g.Cout, g.Cin, plan.gplan, (const float *)w, U);
     }
@@ -244,6 +245,7 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *ge
         const int nb = (g.B - b0 < s.chunk_imgs) ? g.B - b0 : s.chunk_imgs;
         const int T = nb * s.tiles_per_img;
         {
+            TimingScope ts("winograd_input", stream);
             const long long total = (long long)g.Cin * T;
             hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, s, b0, nb, (const float *)x, V);
         }
@@ -251,6 +253,7 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *ge
         if (rc != DLP_OK)
             return rc;
         {
+            TimingScope ts("winograd_output", stream);
             const long long total = (long long)g.Cout * T;
             hipLaunchKernelGGL(wino_output_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, s, b0, nb, Mw, ep.bias,
                                (float *)y, ep.factor, ep.activation);

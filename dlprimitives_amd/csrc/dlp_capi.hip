@@ -7,6 +7,7 @@
 #include "dlp_internal.hpp"
 
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -20,6 +21,43 @@ int fail(int code, const std::string &msg)
 {
     g_last_error = msg;
     return code;
+}
+
+namespace {
+struct TimingRecord {
+    const char *section;
+    hipEvent_t start, stop;
+};
+std::mutex g_timing_mutex;
+bool g_timing_enabled = false;
+std::vector<TimingRecord> g_timing_records;
+} // namespace
+
+TimingScope::TimingScope(const char *section, hipStream_t stream) : stream_(stream), index_(-1)
+{
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    if (!g_timing_enabled)
+        return;
+    TimingRecord r;
+    r.section = section;
+    if (hipEventCreate(&r.start) != hipSuccess)
+        return;
+    if (hipEventCreate(&r.stop) != hipSuccess) {
+        (void)hipEventDestroy(r.start);
+        return;
+    }
+    (void)hipEventRecord(r.start, stream);
+    index_ = (int)g_timing_records.size();
+    g_timing_records.push_back(r);
+}
+
+TimingScope::~TimingScope()
+{
+    if (index_ < 0)
+        return;
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    if (index_ < (int)g_timing_records.size())
+        (void)hipEventRecord(g_timing_records[index_].stop, stream_);
 }
 
 } // namespace dlp
@@ -116,6 +154,45 @@ extern "C" {
 const char *dlp_last_error(void) { return g_last_error.c_str(); }
 
 int dlp_version(void) { return 100; }
+
+int dlp_timing_enable(int on)
+{
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    g_timing_enabled = on != 0;
+    return DLP_OK;
+}
+
+int dlp_timing_reset(void)
+{
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    for (TimingRecord &r : g_timing_records) {
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    g_timing_records.clear();
+    return DLP_OK;
+}
+
+int dlp_timing_count(int *count)
+{
+    DLP_REQUIRE(count != nullptr, "null argument");
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    *count = (int)g_timing_records.size();
+    return DLP_OK;
+}
+
+int dlp_timing_get(int index, char *section, size_t section_len, float *milliseconds)
+{
+    DLP_REQUIRE(section != nullptr && section_len > 0 && milliseconds != nullptr, "null argument");
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    DLP_REQUIRE(index >= 0 && index < (int)g_timing_records.size(), "timing record index out of range");
+    const TimingRecord &r = g_timing_records[index];
+    DLP_HIP_TRY(hipEventSynchronize(r.stop));
+    DLP_HIP_TRY(hipEventElapsedTime(milliseconds, r.start, r.stop));
+    std::strncpy(section, r.section, section_len - 1);
+    section[section_len - 1] = 0;
+    return DLP_OK;
+}
 
 int dlp_device_count(int *count)
 {

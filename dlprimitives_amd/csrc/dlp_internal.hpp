@@ -26,6 +26,16 @@ int fail(int code, const std::string &msg);
             return ::dlp::fail(DLP_ERR_VALIDATION, std::string("check failed: ") + #cond + " -- " + (msg)); \
     } while (0)
 
+// Optional per-kernel timing (the analogue of dlprimitives' ExecutionContext::enable_timing,
+// include/dlprim/context.hpp:23-94,180,237-243): when enabled, every kernel launch of the
+// path is bracketed by a HIP event pair on its stream and recorded under a section name.
+struct TimingScope {
+    TimingScope(const char *section, hipStream_t stream);
+    ~TimingScope();
+    hipStream_t stream_;
+    int index_;
+};
+
 // Geometry of one forward convolution call (whole tensor, all groups).
 struct ConvGeom {
     int B, Cin, H, W;

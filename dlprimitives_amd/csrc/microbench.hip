@@ -34,8 +34,8 @@ __global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, f
 static float time_ms(hipStream_t s, hipEvent_t e0, hipEvent_t e1)
 {
     float ms = 0;
-    hipEventSynchronize(e1);
-    hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventSynchronize(e1);
+    (void)hipEventElapsedTime(&ms, e0, e1);
     (void)s;
     return ms;
 }
@@ -55,18 +55,18 @@ int dlp_probe_mfma_f32(int waves_per_simd, double *tflops)
     if (hipMalloc(&out, (size_t)blocks * 256 * 4) != hipSuccess)
         return 1;
     hipEvent_t e0, e1;
-    hipEventCreate(&e0);
-    hipEventCreate(&e1);
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
     mfma_f32_loop<<<blocks, 256>>>(out, 1000, 1.0f, 2.0f);
-    hipEventRecord(e0, 0);
+    (void)hipEventRecord(e0, 0);
     mfma_f32_loop<<<blocks, 256>>>(out, iters, 1.0f, 2.0f);
-    hipEventRecord(e1, 0);
+    (void)hipEventRecord(e1, 0);
     float ms = time_ms(0, e0, e1);
     double flops = (double)blocks * 4 /*waves*/ * iters * 4 /*mfma*/ * 4096.0;
     *tflops = flops / (ms * 1e-3) / 1e12;
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
-    hipFree(out);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(out);
     return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -77,23 +77,23 @@ int dlp_probe_copy(int mbytes, double *gbs)
     float4 *a = nullptr, *b = nullptr;
     if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess)
         return 1;
-    hipMemset(a, 1, bytes);
+    (void)hipMemset(a, 1, bytes);
     hipEvent_t e0, e1;
-    hipEventCreate(&e0);
-    hipEventCreate(&e1);
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
     size_t n = bytes / 16;
     copy_f4<<<256 * 16, 256>>>(a, b, n);
-    hipEventRecord(e0, 0);
+    (void)hipEventRecord(e0, 0);
     const int reps = 10;
     for (int r = 0; r < reps; r++)
         copy_f4<<<256 * 16, 256>>>(a, b, n);
-    hipEventRecord(e1, 0);
+    (void)hipEventRecord(e1, 0);
     float ms = time_ms(0, e0, e1);
     *gbs = 2.0 * bytes * reps / (ms * 1e-3) / 1e9;
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
-    hipFree(a);
-    hipFree(b);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(a);
+    (void)hipFree(b);
     return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 }

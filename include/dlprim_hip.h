@@ -84,6 +84,17 @@ int dlp_stream_create(void **stream);   /* ExecutionContext's in-order queue */
 int dlp_stream_sync(void *stream);      /* ExecutionContext::finish, context.hpp:216-220 */
 int dlp_stream_destroy(void *stream);
 
+/* ---- per-kernel timing: replaces ExecutionContext::enable_timing / TimingData
+ *      (include/dlprim/context.hpp:23-94,180,237-243).  While enabled, every kernel
+ *      launched by the calls below is bracketed by a HIP event pair on its stream and
+ *      recorded under a section name ("conv_gemm", "pack_weights", "splitk_reduce",
+ *      "sep_conv", "winograd_filter", "winograd_input", "winograd_output").
+ *      dlp_timing_get waits for the record's kernel to finish. -------------------- */
+int dlp_timing_enable(int on);
+int dlp_timing_reset(void);
+int dlp_timing_count(int *count);
+int dlp_timing_get(int index, char *section, size_t section_len, float *milliseconds);
+
 /* ---- Conv2DBase::get_output_shape, src/core/conv.cpp:17-29 ------------------ */
 int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], int out_shape[4]);
 
