@@ -14,11 +14,14 @@ from .capi import (  # noqa: F401
     IPForward,
     IPSettings,
     NotImplementedErrorDlprim,
+    Pooling2DForward,
     ValidationError,
     build_library,
     conv2d_output_shape,
+    eltwise_forward,
     lib,
     library_path,
+    pool2d_output_size,
     timing_count,
     timing_enable,
     timing_records,

@@ -249,3 +249,72 @@ class IPForward:
         if getattr(self, "_h", None):
             lib().dlp_ip_fwd_destroy(self._h)
             self._h = None
+
+
+# ---- glue operators (pooling, global pooling, elementwise) ---------------------------
+
+def pool2d_output_size(in_size, kernel, pad, stride, ceil_mode=False):
+    """core::calc_pooling_output_size"""
+    out = ctypes.c_int()
+    _check(lib().dlp_pool2d_output_size(int(in_size), int(kernel), int(pad), int(stride), int(bool(ceil_mode)), ctypes.byref(out)))
+    return out.value
+
+
+class Pooling2DForward:
+    """core::Pooling2DForward"""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    @staticmethod
+    def _create(fn, *args):
+        h = ctypes.c_void_p()
+        _check(fn(*args, ctypes.byref(h)))
+        return Pooling2DForward(h)
+
+    @staticmethod
+    def create_max_pooling(kernel, pad, stride, dtype=FLOAT_DATA):
+        i2 = ctypes.c_int * 2
+        return Pooling2DForward._create(lib().dlp_pool2d_fwd_create_max, i2(*_pair(kernel)), i2(*_pair(pad)), i2(*_pair(stride)), dtype)
+
+    @staticmethod
+    def create_avg_pooling(kernel, pad, stride, count_include_pad=False, dtype=FLOAT_DATA):
+        i2 = ctypes.c_int * 2
+        return Pooling2DForward._create(lib().dlp_pool2d_fwd_create_avg, i2(*_pair(kernel)), i2(*_pair(pad)), i2(*_pair(stride)),
+                                        int(bool(count_include_pad)), dtype)
+
+    @staticmethod
+    def create_global_max_pooling(dtype=FLOAT_DATA):
+        return Pooling2DForward._create(lib().dlp_pool2d_fwd_create_global_max, dtype)
+
+    @staticmethod
+    def create_global_avg_pooling(dtype=FLOAT_DATA):
+        return Pooling2DForward._create(lib().dlp_pool2d_fwd_create_global_avg, dtype)
+
+    def workspace(self):
+        return 0
+
+    def enqueue(self, x, y, stream=None):
+        xs = (ctypes.c_int * 4)(*x.shape)
+        ys = (ctypes.c_int * 4)(*y.shape)
+        lib().dlp_pool2d_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.c_void_p,
+                                                 ctypes.c_void_p, ctypes.c_void_p]
+        _check(lib().dlp_pool2d_fwd_enqueue(self._h, xs, ys, _ptr(x), _ptr(y), _stream(stream)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().dlp_pool2d_fwd_destroy.argtypes = [ctypes.c_void_p]
+            lib().dlp_pool2d_fwd_destroy.restype = None
+            lib().dlp_pool2d_fwd_destroy(self._h)
+            self._h = None
+
+
+ELTWISE_OPS = {"sum": 0, "prod": 1, "max": 2}
+
+
+def eltwise_forward(a, b, c, operation="sum", coef1=1.0, coef2=1.0, activation="identity", stream=None):
+    """Elementwise::forward for equal shapes: c = act(op(coef1*a, coef2*b))"""
+    lib().dlp_eltwise_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p,
+                                              ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    _check(lib().dlp_eltwise_fwd_enqueue(ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation), a.numel(), _ptr(a), _ptr(b),
+                                         _ptr(c), _stream(stream)))

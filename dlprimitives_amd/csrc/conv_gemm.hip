@@ -404,28 +404,49 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 }
 
 // Sums the split-K slices in slice order (deterministic) and applies the epilogue.
+// One grid row (blockIdx.y) per output channel, four consecutive pixels per thread:
+// 16-byte loads of the partial sums, no 64-bit index arithmetic.
 template <int ACT>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
 {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; // row * N + n
-    const long long total = (long long)a.Cout * a.N;
-    if (idx >= total)
+    const int row = blockIdx.y;
+    const int n4 = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (n4 >= a.N)
         return;
-    const int row = (int)(idx / a.N);
-    const int n = (int)(idx - (long long)row * a.N);
-    float v = 0.0f;
-    for (int s = 0; s < a.splitk; s++)
-        v += a.part[(size_t)s * total + idx];
-    if (a.bias)
-        v += a.bias[row];
-    if (ACT == ACT_CLAMP) {
-        if (a.act != DLP_ACT_IDENTITY)
-            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
-    } else
-        v = apply_act(v, a.act);
-    const int b = n / a.OHW;
-    const int pix = n - b * a.OHW;
-    store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, v, a.factor);
+    const size_t total = (size_t)a.Cout * a.N;
+    const float *pp = a.part + (size_t)row * a.N + n4;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool vec = ((a.N & 3) == 0); // then n4 + 3 < N and every slice row is 16-byte aligned
+    for (int s = 0; s < a.splitk; s++) {
+        if (vec) {
+            const f32x4 t = *(const f32x4 *)(pp + (size_t)s * total);
+            v[0] += t[0];
+            v[1] += t[1];
+            v[2] += t[2];
+            v[3] += t[3];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (n4 + i < a.N)
+                    v[i] += pp[(size_t)s * total + i];
+        }
+    }
+    const float bv = a.bias ? a.bias[row] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int n = n4 + i;
+        if (n >= a.N)
+            break;
+        float r = v[i] + bv;
+        if (ACT == ACT_CLAMP) {
+            if (a.act != DLP_ACT_IDENTITY)
+                r = fminf(fmaxf(r, a.clamp_lo), a.clamp_hi);
+        } else
+            r = apply_act(r, a.act);
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * a.OHW;
+        store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, r, a.factor);
+    }
 }
 
 // Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
@@ -501,8 +522,9 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
-        const long long total = (long long)a.Cout * a.N;
-        hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+        if (a.Cout > 65535)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
+        hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;

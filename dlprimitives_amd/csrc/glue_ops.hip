@@ -1,0 +1,246 @@
+// Glue operators of the ResNet / MobileNet graphs around the convolution path:
+// 2-D pooling, global pooling and element-wise combination of two tensors.
+// All three are HBM-bound streaming kernels (no LDS tiling, no matrix cores).
+//
+// They replace, for forward inference only:
+//   core::Pooling2DForward (include/dlprim/core/pool.hpp:29-70, src/core/pool.cpp) with the
+//     arithmetic of Pooling2D::forward_cpu (src/ops/pooling.cpp:281-328, functors :116-145),
+//   the global pooling variants (GlobalPooling::forward_cpu, src/ops/pooling.cpp:427-452),
+//   Elementwise::forward for equal shapes (src/ops/elementwise.cpp:517-559).
+#include "dlp_internal.hpp"
+
+#include <new>
+
+namespace dlp {
+namespace {
+
+struct PoolArgs {
+    const float *x;
+    float *y;
+    int planes, H, W, OH, OW;
+    int kh, kw, ph, pw, sh, sw;
+    int mode; // 0 max, 1 avg
+    int count_include_pad;
+};
+
+// one output element per thread; consecutive threads on consecutive output columns
+__global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long total = (long long)a.planes * a.OH * a.OW;
+    if (idx >= total)
+        return;
+    const int oc = (int)(idx % a.OW);
+    const long long t = idx / a.OW;
+    const int orow = (int)(t % a.OH);
+    const long long plane = t / a.OH;
+    const float *src = a.x + plane * a.H * a.W;
+    int row0 = orow * a.sh - a.ph, col0 = oc * a.sw - a.pw;
+    int row1 = row0 + a.kh, col1 = col0 + a.kw;
+    const int dr_pad = min(row1, a.H + a.ph) - max(-a.ph, row0);
+    const int dc_pad = min(col1, a.W + a.pw) - max(-a.pw, col0);
+    row0 = max(row0, 0);
+    col0 = max(col0, 0);
+    row1 = min(row1, a.H);
+    col1 = min(col1, a.W);
+    float val = a.mode == 0 ? -3.402823466e+38f : 0.0f;
+    for (int r = row0; r < row1; r++)
+        for (int c = col0; c < col1; c++) {
+            const float v = src[(size_t)r * a.W + c];
+            val = a.mode == 0 ? fmaxf(val, v) : val + v;
+        }
+    if (a.mode != 0) {
+        const int dr = row1 - row0, dc = col1 - col0;
+        if (dr == a.kh && dc == a.kw)
+            val = val * (1.0f / (a.kh * a.kw));
+        else if (a.count_include_pad)
+            val = val / (float)(dr_pad * dc_pad);
+        else
+            val = val * (1.0f / (dr * dc));
+    }
+    a.y[idx] = val;
+}
+
+// one wavefront per plane: lanes stride over the plane, then a shuffle reduction.
+// The average is accumulated per lane in ascending index order and combined pairwise,
+// so it differs from the reference's single running sum only by fp32 rounding.
+__global__ __launch_bounds__(256) void global_pool_kernel(const float *__restrict__ x, float *__restrict__ y, long long planes, int plane_size,
+                                                          int mode)
+{
+    const int lane = threadIdx.x & 63;
+    const long long plane = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (plane >= planes)
+        return;
+    const float *src = x + plane * plane_size;
+    float v = mode == 0 ? -3.402823466e+38f : 0.0f;
+    for (int i = lane; i < plane_size; i += 64) {
+        const float t = src[i];
+        v = mode == 0 ? fmaxf(v, t) : v + t;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float o = __shfl_down(v, off);
+        v = mode == 0 ? fmaxf(v, o) : v + o;
+    }
+    if (lane == 0)
+        y[plane] = mode == 0 ? v : v * (1.0f / plane_size);
+}
+
+__global__ __launch_bounds__(256) void eltwise_kernel(size_t n, int op, float c1, float c2, int act, const float *__restrict__ a,
+                                                      const float *__restrict__ b, float *__restrict__ c)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        const float x0 = a[i], x1 = b[i];
+        float r;
+        if (op == 0)
+            r = x0 * c1 + x1 * c2;
+        else if (op == 1)
+            r = x0 * x1 * (c1 * c2);
+        else
+            r = fmaxf(x0 * c1, x1 * c2);
+        c[i] = apply_act(r, act);
+    }
+}
+
+} // namespace
+} // namespace dlp
+
+using namespace dlp;
+
+struct dlp_pool2d_fwd {
+    int kernel[2], pad[2], stride[2];
+    int mode; // 0 max, 1 avg
+    int count_include_pad;
+    int global;
+};
+
+static int pool_create(const int kernel[2], const int pad[2], const int stride[2], int mode, int cip, int global, int dtype,
+                       dlp_pool2d_fwd **out)
+{
+    DLP_REQUIRE(out != nullptr, "null argument");
+    *out = nullptr;
+    if (dtype != DLP_FLOAT)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "pooling: only float_data is implemented");
+    dlp_pool2d_fwd *op = new (std::nothrow) dlp_pool2d_fwd();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    for (int i = 0; i < 2; i++) {
+        op->kernel[i] = kernel ? kernel[i] : 0;
+        op->pad[i] = pad ? pad[i] : 0;
+        op->stride[i] = stride ? stride[i] : 1;
+    }
+    op->mode = mode;
+    op->count_include_pad = cip;
+    op->global = global;
+    if (!global) {
+        for (int i = 0; i < 2; i++)
+            if (op->kernel[i] <= 0 || op->stride[i] <= 0 || op->pad[i] < 0) {
+                delete op;
+                return fail(DLP_ERR_VALIDATION, "check failed: kernel > 0 && stride > 0 && pad >= 0");
+            }
+    }
+    *out = op;
+    return DLP_OK;
+}
+
+extern "C" {
+
+int dlp_pool2d_output_size(int in_size, int kernel, int pad, int stride, int ceil_mode, int *out_size)
+{
+    DLP_REQUIRE(out_size != nullptr, "null argument");
+    DLP_REQUIRE(kernel > 0 && stride > 0 && pad >= 0, "kernel/stride/pad");
+    const int padded = in_size + pad * 2;
+    DLP_REQUIRE(padded >= kernel, "padded input smaller than the pooling window"); // pool.hpp:20
+    const int offset = ceil_mode ? (stride - 1) : 0;
+    int size = (padded - kernel + offset) / stride + 1;
+    if ((size - 1) * stride >= in_size + pad)
+        size--;
+    *out_size = size;
+    return DLP_OK;
+}
+
+int dlp_pool2d_fwd_create_max(const int kernel[2], const int pad[2], const int stride[2], int dtype, dlp_pool2d_fwd **out)
+{
+    return pool_create(kernel, pad, stride, 0, 0, 0, dtype, out);
+}
+
+int dlp_pool2d_fwd_create_avg(const int kernel[2], const int pad[2], const int stride[2], int count_include_pad, int dtype,
+                              dlp_pool2d_fwd **out)
+{
+    return pool_create(kernel, pad, stride, 1, count_include_pad != 0, 0, dtype, out);
+}
+
+int dlp_pool2d_fwd_create_global_max(int dtype, dlp_pool2d_fwd **out) { return pool_create(nullptr, nullptr, nullptr, 0, 0, 1, dtype, out); }
+
+int dlp_pool2d_fwd_create_global_avg(int dtype, dlp_pool2d_fwd **out) { return pool_create(nullptr, nullptr, nullptr, 1, 0, 1, dtype, out); }
+
+int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y_shape[4], const void *x, void *y, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr && y_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[0] == y_shape[0] && x_shape[1] == y_shape[1], "batch / channels of input and output differ");
+    const long long planes = (long long)x_shape[0] * x_shape[1];
+    if (planes == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && y != nullptr, "null tensor pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (op->global) {
+        DLP_REQUIRE(y_shape[2] == 1 && y_shape[3] == 1, "global pooling output must be [B,C,1,1]");
+        const long long plane_size = (long long)x_shape[2] * x_shape[3];
+        DLP_REQUIRE(plane_size > 0 && plane_size < 0x7fffffffLL, "plane size");
+        TimingScope ts("global_pooling", s);
+        hipLaunchKernelGGL(global_pool_kernel, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const float *)x, (float *)y, planes,
+                           (int)plane_size, op->mode);
+    } else {
+        // the output shape fixes ceil_mode; every window must start inside the padded input (pool.hpp:17-27)
+        for (int i = 0; i < 2; i++) {
+            DLP_REQUIRE(y_shape[2 + i] > 0, "empty pooling output");
+            DLP_REQUIRE((y_shape[2 + i] - 1) * op->stride[i] < x_shape[2 + i] + op->pad[i], "output larger than the pooling geometry allows");
+        }
+        PoolArgs a;
+        a.x = (const float *)x;
+        a.y = (float *)y;
+        a.planes = (int)planes;
+        a.H = x_shape[2];
+        a.W = x_shape[3];
+        a.OH = y_shape[2];
+        a.OW = y_shape[3];
+        a.kh = op->kernel[0];
+        a.kw = op->kernel[1];
+        a.ph = op->pad[0];
+        a.pw = op->pad[1];
+        a.sh = op->stride[0];
+        a.sw = op->stride[1];
+        a.mode = op->mode;
+        a.count_include_pad = op->count_include_pad;
+        const long long total = planes * a.OH * a.OW;
+        DLP_REQUIRE(planes < 0x7fffffffLL && total < 0x7fffffffLL * 256, "tensor too large");
+        TimingScope ts("pooling", s);
+        hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op) { delete op; }
+
+int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b, void *c,
+                            void *stream)
+{
+    DLP_REQUIRE(operation >= 0 && operation <= 2, "unknown elementwise operation");
+    DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
+    if (n == 0)
+        return DLP_OK;
+    DLP_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "null tensor pointer");
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 32)
+        blocks = 256 * 32;
+    TimingScope ts("eltwise", (hipStream_t)stream);
+    hipLaunchKernelGGL(eltwise_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n, operation, coef1, coef2, activation,
+                       (const float *)a, (const float *)b, (float *)c);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+} // extern "C"

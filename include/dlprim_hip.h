@@ -129,6 +129,35 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w,
                        const void *bias, void *y, void *stream);
 void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
 
+/* ===== glue operators around the convolution path (forward only) ================= */
+
+typedef struct dlp_pool2d_fwd dlp_pool2d_fwd; /* core::Pooling2DForward object */
+
+/* core::calc_pooling_output_size, include/dlprim/core/pool.hpp:17-27 */
+int dlp_pool2d_output_size(int in_size, int kernel, int pad, int stride, int ceil_mode, int *out_size);
+
+/* core::Pooling2DForward::create_max_pooling / create_avg_pooling /
+ * create_global_max_pooling / create_global_avg_pooling, include/dlprim/core/pool.hpp:38-69 */
+int dlp_pool2d_fwd_create_max(const int kernel[2], const int pad[2], const int stride[2], int dtype, dlp_pool2d_fwd **out);
+int dlp_pool2d_fwd_create_avg(const int kernel[2], const int pad[2], const int stride[2], int count_include_pad, int dtype,
+                              dlp_pool2d_fwd **out);
+int dlp_pool2d_fwd_create_global_max(int dtype, dlp_pool2d_fwd **out);
+int dlp_pool2d_fwd_create_global_avg(int dtype, dlp_pool2d_fwd **out);
+
+/* core::Pooling2DForward::enqueue(X, Y, e), include/dlprim/core/pool.hpp:36.
+ * x [B,C,H,W] -> y [B,C,OH,OW]; the output shape (from dlp_pool2d_output_size, with or
+ * without ceil_mode) is the caller's, as in the reference; global variants need [B,C,1,1]. */
+int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y_shape[4], const void *x, void *y, void *stream);
+void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op);
+
+/* Elementwise::forward for two tensors of equal shape, src/ops/elementwise.cpp:517-559:
+ * operation 0 sum: c = act(coef1*a + coef2*b); 1 prod: act(a*b*coef1*coef2); 2 max: act(max(coef1*a, coef2*b)) */
+#define DLP_ELTWISE_SUM 0
+#define DLP_ELTWISE_PROD 1
+#define DLP_ELTWISE_MAX 2
+int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b, void *c,
+                            void *stream);
+
 #ifdef __cplusplus
 }
 #endif

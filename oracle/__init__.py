@@ -61,6 +61,7 @@ def lib():
         L.orc_conv2d_direct_f64.restype = ctypes.c_int
         L.orc_winograd_forward.restype = ctypes.c_int
         L.orc_depthwise_forward.restype = ctypes.c_int
+        L.orc_pool_output_size.restype = ctypes.c_int
         L.orc_bf16_round.restype = ctypes.c_float
         L.orc_bf16_round.argtypes = [ctypes.c_float]
         _lib = L
@@ -210,6 +211,46 @@ def depthwise_forward(x, w, bias, activation="identity", factor=0.0, y_old=None)
     if r != 0:
         raise ValueError("invalid depthwise configuration")
     return y
+
+
+def pool_output_size(in_size, kernel, pad, stride, ceil_mode):
+    r = lib().orc_pool_output_size(int(in_size), int(kernel), int(pad), int(stride), int(bool(ceil_mode)))
+    if r < 0:
+        raise ValueError("invalid pooling configuration")
+    return r
+
+
+def pool2d_forward(x, kernel, pad, stride, mode, count_include_pad=False, ceil_mode=False):
+    """Pooling2D::forward_cpu restated; mode 'max' or 'avg'."""
+    x = _f32(x)
+    B, C, H, W = x.shape
+    k, p, s = _pair(kernel), _pair(pad), _pair(stride)
+    OH = pool_output_size(H, k[0], p[0], s[0], ceil_mode)
+    OW = pool_output_size(W, k[1], p[1], s[1], ceil_mode)
+    y = np.empty((B, C, OH, OW), dtype=np.float32)
+    i2 = ctypes.c_int * 2
+    lib().orc_pool2d_forward(B * C, H, W, OH, OW, i2(*k), i2(*p), i2(*s), 0 if mode == "max" else 1, int(bool(count_include_pad)),
+                             _ptr(x), _ptr(y))
+    return y
+
+
+def global_pool_forward(x, mode):
+    x = _f32(x)
+    B, C = x.shape[:2]
+    y = np.empty((B, C, 1, 1), dtype=np.float32)
+    lib().orc_global_pool_forward(ctypes.c_size_t(B * C), ctypes.c_size_t(x[0, 0].size), 0 if mode == "max" else 1, _ptr(x), _ptr(y))
+    return y
+
+
+ELTWISE_OPS = {"sum": 0, "prod": 1, "max": 2}
+
+
+def eltwise_forward(a, b, op="sum", coef1=1.0, coef2=1.0, activation="identity"):
+    a, b = _f32(a), _f32(b)
+    c = np.empty_like(a)
+    lib().orc_eltwise_forward(ctypes.c_size_t(a.size), ELTWISE_OPS[op], ctypes.c_float(coef1), ctypes.c_float(coef2), _act(activation),
+                              _ptr(a), _ptr(b), _ptr(c))
+    return c
 
 
 def bf16_round(a):

@@ -469,6 +469,96 @@ int orc_depthwise_forward(int B, int C, int H, int W, int kern,
     return 0;
 }
 
+/* include/dlprim/core/pool.hpp:17-27 */
+int orc_pool_output_size(int in_size, int kernel, int pad, int stride, int ceil_mode)
+{
+    int padded = in_size + pad * 2;
+    if (padded < kernel || stride <= 0)
+        return -1;
+    int offset = ceil_mode ? (stride - 1) : 0;
+    int size = (padded - kernel + offset) / stride + 1;
+    if ((size - 1) * stride >= in_size + pad)
+        size--;
+    return size;
+}
+
+/* src/ops/pooling.cpp:281-328; functors :116-145 (max: init -FLT_MAX; avg: sum then
+ * * (1/(kh*kw)) on full windows, * (1/(dr*dc)) or / (dr_pad*dc_pad) on clipped ones) */
+void orc_pool2d_forward(int planes, int H, int W, int OH, int OW, const int kernel[2], const int pad[2],
+                        const int stride[2], int mode, int count_include_pad, const float *x, float *y)
+{
+    const float full_factor = 1.0f / (kernel[0] * kernel[1]);
+    for (int p = 0; p < planes; p++, x += (size_t)H * W, y += (size_t)OH * OW)
+        for (int orow = 0; orow < OH; orow++)
+            for (int ocol = 0; ocol < OW; ocol++) {
+                int row0 = orow * stride[0] - pad[0], col0 = ocol * stride[1] - pad[1];
+                int row1 = row0 + kernel[0], col1 = col0 + kernel[1];
+                int top = -pad[0] > row0 ? -pad[0] : row0, left = -pad[1] > col0 ? -pad[1] : col0;
+                int dr_pad = (row1 < H + pad[0] ? row1 : H + pad[0]) - top;
+                int dc_pad = (col1 < W + pad[1] ? col1 : W + pad[1]) - left;
+                if (row0 < 0) row0 = 0;
+                if (col0 < 0) col0 = 0;
+                if (row1 > H) row1 = H;
+                if (col1 > W) col1 = W;
+                float val = mode == 0 ? -3.402823466e+38f : 0.0f;
+                for (int r = row0; r < row1; r++)
+                    for (int c = col0; c < col1; c++) {
+                        float v = x[(size_t)r * W + c];
+                        if (mode == 0)
+                            val = val < v ? v : val;
+                        else
+                            val = val + v;
+                    }
+                if (mode != 0) {
+                    int dr = row1 - row0, dc = col1 - col0;
+                    if (dr == kernel[0] && dc == kernel[1])
+                        val = val * full_factor;
+                    else if (count_include_pad)
+                        val = val / (dr_pad * dc_pad);
+                    else
+                        val = val * (1.0f / (dr * dc));
+                }
+                y[(size_t)orow * OW + ocol] = val;
+            }
+}
+
+/* src/ops/pooling.cpp:427-452 */
+void orc_global_pool_forward(size_t planes, size_t plane_size, int mode, const float *x, float *y)
+{
+    const float factor = 1.0f / plane_size;
+    for (size_t i = 0; i < planes; i++, x += plane_size) {
+        if (mode == 0) {
+            float m = x[0];
+            for (size_t j = 1; j < plane_size; j++)
+                m = m < x[j] ? x[j] : m;
+            y[i] = m;
+        } else {
+            float sum = 0;
+            for (size_t j = 0; j < plane_size; j++)
+                sum += x[j];
+            y[i] = sum * factor;
+        }
+    }
+}
+
+/* src/ops/elementwise.cpp:517-559 (equal shapes: no broadcasting) */
+void orc_eltwise_forward(size_t n, int op, float c1, float c2, int activation, const float *a, const float *b, float *c)
+{
+    const float w = c1 * c2;
+    for (size_t i = 0; i < n; i++) {
+        float x0 = a[i], x1 = b[i];
+        if (op == 0)
+            c[i] = x0 * c1 + x1 * c2;
+        else if (op == 1)
+            c[i] = x0 * x1 * w;
+        else {
+            float u = x0 * c1, v = x1 * c2;
+            c[i] = u < v ? v : u;
+        }
+    }
+    orc_apply_activation(c, n, activation);
+}
+
 float orc_bf16_round(float v)
 {
     uint32_t bits;

@@ -106,6 +106,23 @@ int orc_depthwise_forward(int B, int C, int H, int W, int kern,
                           const float *x, const float *w, const float *bias,
                           float *y, int activation, float factor);
 
+/* ---- glue operators of the ResNet graphs (next rows after the convolution path) ---- */
+
+/* core::calc_pooling_output_size, include/dlprim/core/pool.hpp:17-27; -1 on invalid */
+int orc_pool_output_size(int in_size, int kernel, int pad, int stride, int ceil_mode);
+
+/* Pooling2D::forward_cpu, src/ops/pooling.cpp:281-328 with the reduce functors :116-145.
+ * mode 0 = max, 1 = avg; x [planes][H][W] -> y [planes][OH][OW] */
+void orc_pool2d_forward(int planes, int H, int W, int OH, int OW, const int kernel[2], const int pad[2],
+                        const int stride[2], int mode, int count_include_pad, const float *x, float *y);
+
+/* GlobalPooling::forward_cpu, src/ops/pooling.cpp:427-452; mode 0 = max, 1 = avg */
+void orc_global_pool_forward(size_t planes, size_t plane_size, int mode, const float *x, float *y);
+
+/* Elementwise::forward_cpu for equal shapes, src/ops/elementwise.cpp:517-559:
+ * op 0: a*c1 + b*c2; op 1: a*b*(c1*c2); op 2: max(a*c1, b*c2); then activation */
+void orc_eltwise_forward(size_t n, int op, float c1, float c2, int activation, const float *a, const float *b, float *c);
+
 /* bf16 helpers for the reduced-precision configuration: round-to-nearest-even
  * float -> bfloat16 -> float (the reference has no bf16 path; this defines the
  * storage rounding the HIP kernels use so tests can build matching inputs). */

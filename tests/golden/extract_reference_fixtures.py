@@ -3,6 +3,8 @@
 Reads DATA files only (JSON written by the reference's PyTorch fixture generator):
   tests/test_case_inner_product.json  -> inner_product_fwd.json
   tests/test_case_activation.json     -> activation_fwd.json
+  tests/test_case_pooling2d.json      -> pooling2d_fwd.json
+  tests/test_case_global_pooling.json -> global_pooling_fwd.json
 keeping options, parameters, inputs and expected forward outputs (gradients are
 dropped: the path is forward only).  Run in the build container, where the
 reference tree is mounted:  python tests/golden/extract_reference_fixtures.py
@@ -46,3 +48,5 @@ def extract(src, dst):
 if __name__ == "__main__":
     extract("test_case_inner_product.json", "inner_product_fwd.json")
     extract("test_case_activation.json", "activation_fwd.json")
+    extract("test_case_pooling2d.json", "pooling2d_fwd.json")
+    extract("test_case_global_pooling.json", "global_pooling_fwd.json")

@@ -1,0 +1,172 @@
+"""Glue operators (pooling, global pooling, elementwise): oracle pinned by the reference's
+golden vectors on the CPU; HIP kernels against those goldens and the oracle on the GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOL = dict(rtol=1e-5, atol=1e-5)
+
+
+def golden_cases(name):
+    doc = json.load(open(os.path.join(GOLDEN, name)))
+    for t in doc["tests"]:
+        for cs in t["cases"]:
+            if "in" in cs:
+                x = np.array(cs["in"][0], dtype=np.float32).reshape(cs["in_shapes"][0])
+                y = np.array(cs["out"][0], dtype=np.float32).reshape(cs["out_shapes"][0])
+                yield t["options"], x, y
+
+
+def shape_cases(name):
+    doc = json.load(open(os.path.join(GOLDEN, name)))
+    for t in doc["tests"]:
+        for cs in t["cases"]:
+            yield t["options"], cs["in_shapes"][0], cs["out_shapes"][0]
+
+
+# ------------------------------------------------------------------ CPU: pin the oracle
+def test_oracle_pooling_reference_goldens(oracle_mod):
+    n = 0
+    for o, x, want in golden_cases("pooling2d_fwd.json"):
+        got = oracle_mod.pool2d_forward(x, o["kernel"], o["pad"], o["stride"], o["mode"], o["count_include_pad"], o["ceil_mode"])
+        assert got.shape == want.shape, (o, x.shape)
+        np.testing.assert_allclose(got, want, **TOL)
+        n += 1
+    assert n == 96
+
+
+def test_oracle_pool_output_size_matches_every_reference_shape(oracle_mod):
+    n = 0
+    for o, ish, osh in shape_cases("pooling2d_fwd.json"):
+        k, p, s = [v if isinstance(v, list) else [v, v] for v in (o["kernel"], o["pad"], o["stride"])]
+        for d in range(2):
+            assert oracle_mod.pool_output_size(ish[2 + d], k[d], p[d], s[d], o["ceil_mode"]) == osh[2 + d]
+        n += 1
+    assert n == 144
+
+
+def test_oracle_global_pooling_reference_goldens(oracle_mod):
+    n = 0
+    for o, x, want in golden_cases("global_pooling_fwd.json"):
+        np.testing.assert_allclose(oracle_mod.global_pool_forward(x, o["mode"]), want, **TOL)
+        n += 1
+    assert n == 8
+
+
+def test_oracle_eltwise_closed_forms(oracle_mod):
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal(1000).astype(np.float32)
+    b = rng.standard_normal(1000).astype(np.float32)
+    np.testing.assert_allclose(oracle_mod.eltwise_forward(a, b, "sum", 1.0, 1.0, "relu"), np.maximum(a + b, 0), rtol=1e-6)
+    np.testing.assert_allclose(oracle_mod.eltwise_forward(a, b, "sum", 2.0, -0.5), 2 * a - 0.5 * b, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(oracle_mod.eltwise_forward(a, b, "prod", 2.0, 3.0), a * b * 6, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(oracle_mod.eltwise_forward(a, b, "max", 1.0, 2.0), np.maximum(a, 2 * b), rtol=1e-6)
+
+
+def test_pool_output_size_host_side(oracle_mod):
+    import dlprimitives_amd as dlp
+
+    for (n, k, p, s, c) in [(224, 3, 1, 2, False), (112, 3, 1, 2, False), (5, 2, 0, 2, True), (7, 3, 1, 3, True), (65, 5, 2, 4, True)]:
+        assert dlp.pool2d_output_size(n, k, p, s, c) == oracle_mod.pool_output_size(n, k, p, s, c)
+    assert dlp.pool2d_output_size(112, 3, 1, 2) == 56  # the ResNet stem pooling
+    with pytest.raises(dlp.ValidationError):
+        dlp.pool2d_output_size(2, 5, 1, 1)
+
+
+# ------------------------------------------------------------------ GPU
+def _dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+
+
+def _make_pool(dlp, o):
+    if o["mode"] == "max":
+        return dlp.Pooling2DForward.create_max_pooling(o["kernel"], o["pad"], o["stride"])
+    return dlp.Pooling2DForward.create_avg_pooling(o["kernel"], o["pad"], o["stride"], o["count_include_pad"])
+
+
+@pytest.mark.gpu
+def test_gpu_pooling_reference_goldens():
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    n = 0
+    for o, x, want in golden_cases("pooling2d_fwd.json"):
+        y = torch.full(want.shape, float("nan"), device="cuda:0")
+        _make_pool(dlp, o).enqueue(_dev(x), y)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+        n += 1
+    assert n == 96
+
+
+@pytest.mark.gpu
+def test_gpu_pooling_large_shapes_vs_oracle(oracle_mod):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(1)
+    seen = 0
+    for o, ish, osh in shape_cases("pooling2d_fwd.json"):
+        if np.prod(ish) < 5000 or np.prod(ish) > 3e6:
+            continue
+        x = rng.standard_normal(ish).astype(np.float32)
+        y = torch.full(tuple(osh), float("nan"), device="cuda:0")
+        _make_pool(dlp, o).enqueue(_dev(x), y)
+        torch.cuda.synchronize()
+        want = oracle_mod.pool2d_forward(x, o["kernel"], o["pad"], o["stride"], o["mode"], o["count_include_pad"], o["ceil_mode"])
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+        seen += 1
+    assert seen >= 20
+    # the ResNet stem max pool 3x3/2 pad 1 at its real plane size
+    x = rng.standard_normal((2, 64, 112, 112)).astype(np.float32)
+    y = torch.empty((2, 64, 56, 56), device="cuda:0")
+    dlp.Pooling2DForward.create_max_pooling(3, 1, 2).enqueue(_dev(x), y)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), oracle_mod.pool2d_forward(x, 3, 1, 2, "max"))
+
+
+@pytest.mark.gpu
+def test_gpu_global_pooling(oracle_mod):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    for o, x, want in golden_cases("global_pooling_fwd.json"):
+        op = dlp.Pooling2DForward.create_global_max_pooling() if o["mode"] == "max" else dlp.Pooling2DForward.create_global_avg_pooling()
+        y = torch.full(want.shape, float("nan"), device="cuda:0")
+        op.enqueue(_dev(x), y)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+    rng = np.random.default_rng(2)
+    for shape in [(4, 2048, 7, 7), (3, 512, 7, 7), (2, 5, 33, 17), (1, 1, 1, 1)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        for mode in ("max", "avg"):
+            op = dlp.Pooling2DForward.create_global_max_pooling() if mode == "max" else dlp.Pooling2DForward.create_global_avg_pooling()
+            y = torch.full(shape[:2] + (1, 1), float("nan"), device="cuda:0")
+            op.enqueue(_dev(x), y)
+            torch.cuda.synchronize()
+            np.testing.assert_allclose(y.cpu().numpy(), oracle_mod.global_pool_forward(x, mode), **TOL)
+
+
+@pytest.mark.gpu
+def test_gpu_eltwise(oracle_mod):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(3)
+    for n in (1, 1000, 64 * 256 * 56 * 56 // 16 + 3):
+        a = rng.standard_normal(n).astype(np.float32)
+        b = rng.standard_normal(n).astype(np.float32)
+        for (op, c1, c2, act) in [("sum", 1.0, 1.0, "relu"), ("sum", 0.5, -2.0, "identity"), ("prod", 2.0, 3.0, "tanh"), ("max", 1.0, 2.0, "relu6")]:
+            c = torch.full((n,), float("nan"), device="cuda:0")
+            dlp.eltwise_forward(_dev(a), _dev(b), c, op, c1, c2, act)
+            torch.cuda.synchronize()
+            np.testing.assert_allclose(c.cpu().numpy(), oracle_mod.eltwise_forward(a, b, op, c1, c2, act), rtol=1e-6, atol=1e-6)
