@@ -12,6 +12,7 @@ Other workloads (same JSON contract, for the remaining configurations):
   --workload mobilenet      depthwise 3x3 stride 1/2 (HBM bound) + 1x1 pointwise, ReLU6
   --workload winograd       the two Winograd shapes, algo winograd
   --workload winograd-gemm  the same two shapes through the implicit GEMM
+  --workload resnet18-full / resnet50-full   whole network forward incl. pooling, adds, GAP, IP
 
 Prints ONE JSON line.  `value` = images/s of the whole workload; `gflops_per_s` is
 the same run expressed with the reference's flop accounting (tools/flops.cpp:660).
@@ -124,13 +125,66 @@ def cpu_baseline(layer_list, images, seed):
                 gflops_per_s=round(flops / total / 1e9, 2))
 
 
+def run_graph_workload(args):
+    """Whole-network forward (convolutions + pooling + residual adds + global pooling + inner
+    product) through the C-ABI operators; same JSON contract, no per-kernel roofline split."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd import graphs
+
+    net = args.workload[:-len("-full")]
+    ops = getattr(graphs, net)()
+    params = graphs.random_parameters(ops, 2024)
+    shape = (args.batch, 3, 224, 224)
+    runner = graphs.GraphRunner(ops, params, shape, algo=args.algo)
+    x = torch.rand(shape, device="cuda:0") * 2 - 1
+    runner.t["data"].copy_(x)
+    for _ in range(args.warmup):
+        runner.forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        runner.forward()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    dlp.timing_reset()
+    dlp.timing_enable(True)
+    runner.forward()
+    torch.cuda.synchronize()
+    dlp.timing_enable(False)
+    sections = {}
+    for (section, ms) in dlp.timing_records():
+        sections[section] = round(sections.get(section, 0.0) + ms, 4)
+    dlp.timing_reset()
+    flops = runner.flops()
+    conv_ms = sections.get("conv_gemm", 0.0)
+    out = {
+        "metric": BASELINE_METRIC, "value": round(args.batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds, global avg pool, inner product), "
+                               "fp32 NCHW, batch %d, 224x224, conv algo '%s'" % (net, args.batch, args.algo or "auto"),
+                   "batch": args.batch, "gflop_per_step": round(flops / 1e9, 1)},
+        "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac_of_fp32_matrix_peak": round(flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
+        "kernel_ms_by_section": sections,
+        "roofline": {"bound": "mfma", "kernel": "conv_gemm (all instantiations of one forward)", "achieved": round(flops / (conv_ms * 1e-3) / 1e12, 2) if conv_ms else None,
+                     "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (conv_ms * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4) if conv_ms else None,
+                     "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenet", "winograd", "winograd-gemm"])
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full"])
+    ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
@@ -149,6 +203,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.workload.endswith("-full"):
+        run_graph_workload(args)
+        return
     layer_list, description = workload_layers(args.workload)
     if args.only:
         layer_list = [L for L in layer_list if args.only in L["name"]]

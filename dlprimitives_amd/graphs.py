@@ -1,0 +1,171 @@
+"""ResNet-18 / ResNet-50 forward graphs (shapes of the reference's
+docs/nets_for_benchmark/resnet18-b16.js and resnet50-b16.js, torchvision v1.5: stride on
+the 3x3) with batch norm folded into the preceding convolution, and a small executor that
+runs them on the GPU through the C ABI: convolution, pooling, elementwise, global pooling
+and inner product are the library's operators; this module only wires tensors.
+
+An op is a dict: conv {cin,cout,k,s,p,act}, maxpool {k,s,p}, add {act}, gap, ip {inputs,outputs};
+`src` names its input tensor(s), `dst` its output.
+"""
+import numpy as np
+
+
+def _conv(ops, src, dst, cin, cout, k, s, p, act):
+    ops.append(dict(op="conv", src=src, dst=dst, cin=cin, cout=cout, k=k, s=s, p=p, act=act))
+    return dst
+
+
+def resnet18():
+    ops = []
+    t = _conv(ops, "data", "stem", 3, 64, 7, 2, 3, "relu")
+    ops.append(dict(op="maxpool", src=t, dst="pool", k=3, s=2, p=1))
+    t, cin = "pool", 64
+    for stage, cout in enumerate((64, 128, 256, 512), 1):
+        for block in range(2):
+            s = 2 if (stage > 1 and block == 0) else 1
+            name = "l%d_%d" % (stage, block)
+            a = _conv(ops, t, name + "_a", cin, cout, 3, s, 1, "relu")
+            b = _conv(ops, a, name + "_b", cout, cout, 3, 1, 1, "identity")
+            skip = t
+            if s != 1 or cin != cout:
+                skip = _conv(ops, t, name + "_ds", cin, cout, 1, s, 0, "identity")
+            ops.append(dict(op="add", src=[b, skip], dst=name, act="relu"))
+            t, cin = name, cout
+    ops.append(dict(op="gap", src=t, dst="gap"))
+    ops.append(dict(op="ip", src="gap", dst="logits", inputs=512, outputs=1000))
+    return ops
+
+
+def resnet50():
+    ops = []
+    t = _conv(ops, "data", "stem", 3, 64, 7, 2, 3, "relu")
+    ops.append(dict(op="maxpool", src=t, dst="pool", k=3, s=2, p=1))
+    t, cin = "pool", 64
+    for stage, (mid, blocks) in enumerate(((64, 3), (128, 4), (256, 6), (512, 3)), 1):
+        cout = mid * 4
+        for block in range(blocks):
+            s = 2 if (stage > 1 and block == 0) else 1
+            name = "l%d_%d" % (stage, block)
+            a = _conv(ops, t, name + "_a", cin, mid, 1, 1, 0, "relu")
+            b = _conv(ops, a, name + "_b", mid, mid, 3, s, 1, "relu")
+            c = _conv(ops, b, name + "_c", mid, cout, 1, 1, 0, "identity")
+            skip = t
+            if s != 1 or cin != cout:
+                skip = _conv(ops, t, name + "_ds", cin, cout, 1, s, 0, "identity")
+            ops.append(dict(op="add", src=[c, skip], dst=name, act="relu"))
+            t, cin = name, cout
+    ops.append(dict(op="gap", src=t, dst="gap"))
+    ops.append(dict(op="ip", src="gap", dst="logits", inputs=2048, outputs=1000))
+    return ops
+
+
+def fold_batchnorm(w, gamma, beta, mean, var, eps=1e-5):
+    """W' = W * gamma/sqrt(var+eps) per output channel, b' = beta - mean*gamma/sqrt(var+eps)
+    (closed form of the reference's BatchNorm inference, src/ops/batch_normalization.cpp:210-232)."""
+    scale = (gamma / np.sqrt(var + eps)).astype(np.float32)
+    return (w * scale[:, None, None, None]).astype(np.float32), (beta - mean * scale).astype(np.float32)
+
+
+def random_parameters(ops, seed):
+    """Kaiming-normal conv weights with random BN statistics folded in; inner product weights."""
+    rng = np.random.default_rng(seed)
+    params = {}
+    for o in ops:
+        if o["op"] == "conv":
+            fan_in = o["cin"] * o["k"] * o["k"]
+            w = (rng.standard_normal((o["cout"], o["cin"], o["k"], o["k"])) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+            gamma = rng.uniform(0.5, 1.0, o["cout"]).astype(np.float32)
+            beta = rng.uniform(-0.1, 0.1, o["cout"]).astype(np.float32)
+            mean = (rng.standard_normal(o["cout"]) * 0.1).astype(np.float32)
+            var = rng.uniform(0.5, 1.5, o["cout"]).astype(np.float32)
+            params[o["dst"]] = fold_batchnorm(w, gamma, beta, mean, var)
+        elif o["op"] == "ip":
+            w = (rng.standard_normal((o["outputs"], o["inputs"])) / np.sqrt(o["inputs"])).astype(np.float32)
+            params[o["dst"]] = (w, rng.uniform(-0.1, 0.1, o["outputs"]).astype(np.float32))
+    return params
+
+
+def conv_out(n, k, s, p):
+    return (n + 2 * p - (k - 1) - 1) // s + 1
+
+
+def infer_shapes(ops, in_shape):
+    """tensor name -> shape"""
+    import dlprimitives_amd as dlp
+
+    shapes = {"data": tuple(in_shape)}
+    for o in ops:
+        if o["op"] == "conv":
+            b, _, h, w = shapes[o["src"]]
+            shapes[o["dst"]] = (b, o["cout"], conv_out(h, o["k"], o["s"], o["p"]), conv_out(w, o["k"], o["s"], o["p"]))
+        elif o["op"] == "maxpool":
+            b, c, h, w = shapes[o["src"]]
+            shapes[o["dst"]] = (b, c, dlp.pool2d_output_size(h, o["k"], o["p"], o["s"]), dlp.pool2d_output_size(w, o["k"], o["p"], o["s"]))
+        elif o["op"] == "add":
+            shapes[o["dst"]] = shapes[o["src"][0]]
+        elif o["op"] == "gap":
+            b, c = shapes[o["src"]][:2]
+            shapes[o["dst"]] = (b, c, 1, 1)
+        elif o["op"] == "ip":
+            shapes[o["dst"]] = (shapes[o["src"]][0], o["outputs"])
+    return shapes
+
+
+class GraphRunner:
+    """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
+
+    def __init__(self, ops, params, in_shape, algo=""):
+        import torch
+
+        import dlprimitives_amd as dlp
+
+        self.ops = ops
+        self.shapes = infer_shapes(ops, in_shape)
+        self.t = {n: torch.empty(s, dtype=torch.float32, device="cuda:0") for n, s in self.shapes.items()}
+        self.p = {n: (torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()) for n, (w, b) in params.items()}
+        self.k = []
+        ws_bytes = 1
+        for o in ops:
+            if o["op"] == "conv":
+                st = dlp.Conv2DSettings(o["cin"], o["cout"], o["k"], o["s"], 1, o["p"], 1, self.shapes[o["src"]])
+                op = dlp.Conv2DForward.create(st, True, o["act"], algo)
+                ws_bytes = max(ws_bytes, op.workspace())
+            elif o["op"] == "maxpool":
+                op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"])
+            elif o["op"] == "gap":
+                op = dlp.Pooling2DForward.create_global_avg_pooling()
+            elif o["op"] == "ip":
+                op = dlp.IPForward.create(dlp.IPSettings(o["inputs"], o["outputs"], in_shape[0]), True, "identity")
+            else:
+                op = None
+            self.k.append(op)
+        # one workspace shared by all operators, as the reference's Net does
+        self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda:0")
+
+    def forward(self, x=None):
+        import dlprimitives_amd as dlp
+
+        if x is not None:
+            self.t["data"].copy_(x)
+        for o, op in zip(self.ops, self.k):
+            if o["op"] == "conv":
+                w, b = self.p[o["dst"]]
+                op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]], self.ws, 0.0)
+            elif o["op"] in ("maxpool", "gap"):
+                op.enqueue(self.t[o["src"]], self.t[o["dst"]])
+            elif o["op"] == "add":
+                dlp.eltwise_forward(self.t[o["src"][0]], self.t[o["src"][1]], self.t[o["dst"]], "sum", 1.0, 1.0, o["act"])
+            elif o["op"] == "ip":
+                w, b = self.p[o["dst"]]
+                op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]])
+        return self.t[self.ops[-1]["dst"]]
+
+    def flops(self):
+        total = 0.0
+        for o in self.ops:
+            if o["op"] == "conv":
+                b, c, h, w = self.shapes[o["dst"]]
+                total += 2.0 * b * c * h * w * o["cin"] * o["k"] * o["k"]
+            elif o["op"] == "ip":
+                total += 2.0 * self.shapes[o["dst"]][0] * o["inputs"] * o["outputs"]
+        return total
