@@ -94,7 +94,7 @@ def kernel_class(L):
     small = L["kernel"] ** 2 <= 32 or L["algo"] == "winograd"
     order = 1 if (small and cin_g % 16 == 0) else 0
     mask = 1 if small else 2
-    return "conv_gemm_f32_kernel<%s, %d, %d, 0>" % (tile, order, mask)
+    return "conv_gemm_f32_kernel<float, %s, %d, %d, 0>" % (tile, order, mask)
 
 
 MAIN_SECTION = {"gemm": "conv_gemm", "winograd": "conv_gemm", "depthwise_separable": "sep_conv"}
@@ -137,9 +137,10 @@ def run_graph_workload(args):
     ops = getattr(graphs, net)()
     params = graphs.random_parameters(ops, 2024)
     shape = (args.batch, 3, 224, 224)
-    runner = graphs.GraphRunner(ops, params, shape, algo=args.algo)
+    bf16 = args.dtype == "bf16"
+    runner = graphs.GraphRunner(ops, params, shape, algo="gemm" if bf16 else args.algo, dtype="bfloat16" if bf16 else "float32")
     x = torch.rand(shape, device="cuda:0") * 2 - 1
-    runner.t["data"].copy_(x)
+    runner.t["data"].copy_(x)  # converts to the storage type
     for _ in range(args.warmup):
         runner.forward()
     torch.cuda.synchronize()
@@ -162,9 +163,10 @@ def run_graph_workload(args):
     out = {
         "metric": BASELINE_METRIC, "value": round(args.batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32 arithmetic on bf16-stored tensors" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds, global avg pool, inner product), "
-                               "fp32 NCHW, batch %d, 224x224, conv algo '%s'" % (net, args.batch, args.algo or "auto"),
+                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, "bf16 storage" if bf16 else "fp32", args.batch,
+                                                                                 "gemm" if bf16 else (args.algo or "auto")),
                    "batch": args.batch, "gflop_per_step": round(flops / 1e9, 1)},
         "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_fp32_matrix_peak": round(flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
@@ -185,6 +187,7 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full"])
     ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the -full workloads (arithmetic is fp32 either way)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")

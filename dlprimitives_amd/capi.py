@@ -312,9 +312,20 @@ class Pooling2DForward:
 ELTWISE_OPS = {"sum": 0, "prod": 1, "max": 2}
 
 
+def torch_dtype_code(t):
+    """dlprim DataType of a torch tensor (float32 -> float_data, bfloat16 -> bfloat16_data)."""
+    import torch
+
+    if t.dtype == torch.float32:
+        return FLOAT_DATA
+    if t.dtype == torch.bfloat16:
+        return BFLOAT16_DATA
+    raise ValidationError("unsupported tensor dtype %s" % t.dtype)
+
+
 def eltwise_forward(a, b, c, operation="sum", coef1=1.0, coef2=1.0, activation="identity", stream=None):
     """Elementwise::forward for equal shapes: c = act(op(coef1*a, coef2*b))"""
-    lib().dlp_eltwise_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p,
-                                              ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
-    _check(lib().dlp_eltwise_fwd_enqueue(ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation), a.numel(), _ptr(a), _ptr(b),
-                                         _ptr(c), _stream(stream)))
+    lib().dlp_eltwise_fwd_enqueue_dtype.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_size_t,
+                                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    _check(lib().dlp_eltwise_fwd_enqueue_dtype(torch_dtype_code(a), ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation),
+                                               a.numel(), _ptr(a), _ptr(b), _ptr(c), _stream(stream)))

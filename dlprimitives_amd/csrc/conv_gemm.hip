@@ -53,10 +53,10 @@ constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer 
 enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
 struct GemmArgs {
-    const float *x;
-    const float *wp; // packed weights
+    const void *x;   // storage type T (float or bf16_t)
+    const float *wp; // packed weights, always fp32
     const float *bias;
-    float *y;
+    void *y;         // storage type T
     const int32_t *ktab;
     int M, N, K, nkt;
     int mtiles, ntiles;
@@ -66,7 +66,7 @@ struct GemmArgs {
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
     uint32_t x_shift; // bytes by which the X resource base is moved back (padding offset)
-    uint32_t hw4;     // H*W*4: byte stride between input channels
+    uint32_t hw4;     // H*W*sizeof(T): byte stride between input channels
     uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
     float factor;
     int act;
@@ -81,9 +81,18 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_
     return (__umulhi(n, magic) + n) >> shift;
 }
 
-__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+// one storage element, widened to fp32 (bf16 -> fp32 is a 16-bit shift)
+template <class T>
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff);
+template <>
+__device__ __forceinline__ float buf_load<float>(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
 {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+template <>
+__device__ __forceinline__ float buf_load<bf16_t>(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0) << 16);
 }
 
 __device__ __forceinline__ f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
@@ -127,7 +136,7 @@ __device__ __forceinline__ void static_for_all(F &&f)
     f(std::integral_constant<int, 7>{});
 }
 
-template <int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
+template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 {
     static_assert(BK == 16, "the slice helpers assume 8 MFMA steps per K tile");
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         const int ox = pix - oy * a.OW;
         const int iy0 = oy * a.sh - a.ph;
         const int ix0 = ox * a.sw - a.pw;
-        vbase = (uint32_t)((((b * a.Cin + g * a.Cin_g) * a.H + oy * a.sh) * a.W + ox * a.sw) * 4);
+        vbase = (uint32_t)((((b * a.Cin + g * a.Cin_g) * a.H + oy * a.sh) * a.W + ox * a.sw) * (int)sizeof(T));
         if (vn) {
             uint32_t ry = 0, rx = 0;
             for (int ky = 0; ky < a.KH; ky++) {
@@ -254,7 +263,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 #pragma unroll
             for (int i = 0; i < B_LD; i++)
                 if (i % (BK / 2) == Q)
-                    rb[S][i] = buf_load(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4);
+                    rb[S][i] = buf_load<T>(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4);
         } else {
             // table entry of a k: {x byte offset of (c,ky,kx), tap bit or ky|kx<<8}
             ConstInt *e = ktab + (kt * BK + ks * B_LD) * 2;
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                     ok = (my & tap) != 0;
                 else
                     ok = ((my >> (tap & 0xff)) & (mx >> (tap >> 8)) & 1u) != 0;
-                rb[S][i] = buf_load(xr, opaque(ok ? vbase : kOutOfRange), xoff);
+                rb[S][i] = buf_load<T>(xr, opaque(ok ? vbase : kOutOfRange), xoff);
             }
         }
     };
@@ -381,7 +390,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             continue;
         const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
         const int pix = n - b * a.OHW;
-        float *yb = a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
+        T *yb = (T *)a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -406,7 +415,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 // Sums the split-K slices in slice order (deterministic) and applies the epilogue.
 // One grid row (blockIdx.y) per output channel, four consecutive pixels per thread:
 // 16-byte loads of the partial sums, no 64-bit index arithmetic.
-template <int ACT>
+template <class T, int ACT>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
 {
     const int row = blockIdx.y;
@@ -445,12 +454,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
             r = apply_act(r, a.act);
         const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
         const int pix = n - b * a.OHW;
-        store_out(a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, r, a.factor);
+        store_out((T *)a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, r, a.factor);
     }
 }
 
 // Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
-__global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int groups, int cin_g, int khw, const float *__restrict__ w,
+template <class T>
+__global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int groups, int cin_g, int khw, const T *__restrict__ w,
                                                            float *__restrict__ out)
 {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -475,7 +485,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int group
     }
     float v = 0.0f;
     if (m < p.M && col < p.K)
-        v = w[((size_t)g * p.M + m) * p.K + col];
+        v = to_float(w[((size_t)g * p.M + m) * p.K + col]);
     out[idx] = v;
 }
 
@@ -510,7 +520,7 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
 }
 
-template <int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
+template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
@@ -518,28 +528,28 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     {
         TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL((conv_gemm_f32_kernel<BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
-        hipLaunchKernelGGL((splitk_reduce_kernel<ACT>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, ACT>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <class T, int BM, int BN, int WM, int WN>
 int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipStream_t stream)
 {
     if (act == ACT_GENERIC)
-        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
+        return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
     if (p.order == GEMM_ORDER_TAP)
-        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_TAP, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
+        return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_TAP, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
     if (p.mask == GEMM_MASK_TAPS)
-        return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
-    return launch_inst<BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
+        return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
 }
 
 void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
@@ -617,12 +627,13 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
         tab[i] = 0; // spare entries: no tap bit (row/col code 31 below), offsets 0
     const GemmPlan p = conv_gemm_plan(g, activation);
     const int cin_g = g.Cin / g.groups;
+    const int esize = (int)dtype_size(g.dtype); // gather offsets are bytes of the storage type
     if (p.order == GEMM_ORDER_TAP) {
         int t = 0;
         for (int cb = 0; cb < cin_g / BK; cb++)
             for (int ky = 0; ky < g.KH; ky++)
                 for (int kx = 0; kx < g.KW; kx++, t++) {
-                    tab[4 * t + 0] = ((cb * BK * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
+                    tab[4 * t + 0] = ((cb * BK * g.H + ky * g.dh) * g.W + kx * g.dw) * esize;
                     tab[4 * t + 1] = (int32_t)(1u << (ky * g.KW + kx));
                 }
         return;
@@ -631,7 +642,7 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
     for (int c = 0; c < cin_g; c++)
         for (int ky = 0; ky < g.KH; ky++)
             for (int kx = 0; kx < g.KW; kx++, k++) {
-                tab[2 * k + 0] = ((c * g.H + ky * g.dh) * g.W + kx * g.dw) * 4;
+                tab[2 * k + 0] = ((c * g.H + ky * g.dh) * g.W + kx * g.dw) * esize;
                 tab[2 * k + 1] = (p.mask == GEMM_MASK_ROWCOL) ? (ky | (kx << 8)) : (int32_t)(1u << (ky * g.KW + kx));
             }
     if (p.mask == GEMM_MASK_ROWCOL)
@@ -658,8 +669,12 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
     TimingScope ts("pack_weights", stream);
-    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups, g.Cin / g.groups,
-                       g.KH * g.KW, (const float *)w, (float *)wpacked);
+    if (g.dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(pack_weights_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
+                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked);
+    else
+        hipLaunchKernelGGL(pack_weights_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
+                           g.Cin / g.groups, g.KH * g.KW, (const float *)w, (float *)wpacked);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -667,22 +682,23 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
                      void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes)
 {
-    if (g.dtype != DLP_FLOAT)
-        return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: only float_data is implemented");
+    if (g.dtype != DLP_FLOAT && g.dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: float_data and bfloat16_data are implemented");
+    const size_t esize = dtype_size(g.dtype);
     DLP_REQUIRE(g.KH <= 31 && g.KW <= 31, "kernel extent above 31 is not supported by the gather masks");
     const size_t x_elems = (size_t)g.B * g.Cin * g.H * g.W;
     const size_t y_elems = (size_t)g.B * g.Cout * g.OH * g.OW;
-    const size_t x_shift = ((size_t)g.ph * g.W + g.pw) * 4;
-    if (x_elems * 4 + x_shift >= kOutOfRange || p.wpack_bytes >= kOutOfRange || y_elems >= 0x7fffffffULL)
+    const size_t x_shift = ((size_t)g.ph * g.W + g.pw) * esize;
+    if (x_elems * esize + x_shift >= kOutOfRange || p.wpack_bytes >= kOutOfRange || y_elems >= 0x7fffffffULL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
 
     GemmArgs a;
-    a.x = (const float *)x;
+    a.x = x;
     a.wp = (const float *)wpacked;
     a.bias = ep.bias;
-    a.y = (float *)y;
+    a.y = y;
     a.ktab = (const int32_t *)dev_ktab;
     a.M = p.M;
     a.K = p.K;
@@ -703,10 +719,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     a.OHW = g.OH * g.OW;
     a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw; a.dh = g.dh; a.dw = g.dw;
     a.KH = g.KH; a.KW = g.KW;
-    a.x_bytes = (uint32_t)(x_elems * 4);
+    a.x_bytes = (uint32_t)(x_elems * esize);
     a.wp_bytes = (uint32_t)p.wpack_bytes;
     a.x_shift = (uint32_t)x_shift;
-    a.hw4 = (uint32_t)(g.H * g.W * 4);
+    a.hw4 = (uint32_t)(g.H * g.W * esize);
     make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
     make_magic((uint32_t)a.OW, a.ow_magic, a.ow_shift);
     a.factor = ep.factor;
@@ -721,7 +737,9 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
 
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
-        return launch_tile<decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);
+        if (g.dtype == DLP_BFLOAT16)
+            return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);
+        return launch_tile<float, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);
     });
 }
 

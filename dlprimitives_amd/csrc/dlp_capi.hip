@@ -288,8 +288,11 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     // src/ops/conv2d.cpp:105-106
     DLP_REQUIRE(cfg->channels_in % cfg->groups == 0 && cfg->channels_out % cfg->groups == 0, "channels not divisible by groups");
     DLP_REQUIRE(valid_activation(activation), "unknown activation");
-    if (cfg->dtype != DLP_FLOAT) // the reference: DLPRIM_CHECK(dtype == float_data), src/gemm.cpp:593
-        return fail(DLP_ERR_NOT_IMPLEMENTED, "only float_data is implemented for Conv2DForward");
+    // The reference checks dtype == float_data (src/gemm.cpp:593).  Here bfloat16_data is
+    // also accepted: x, w, y are stored as bf16, bias stays fp32, all arithmetic is fp32
+    // (the implicit-GEMM algorithm serves it; Winograd / depthwise requests fall back to it).
+    if (cfg->dtype != DLP_FLOAT && cfg->dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "Conv2DForward: float_data and bfloat16_data are implemented");
     std::string al = algo ? algo : "";
     DLP_REQUIRE(al == "" || al == "auto" || al == "gemm" || al == "winograd" || al == "depthwise_separable", "unknown algorithm name");
 
@@ -409,8 +412,9 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
     *out = nullptr;
     DLP_REQUIRE(cfg->inputs > 0 && cfg->outputs > 0, "inputs/outputs must be positive");
     DLP_REQUIRE(valid_activation(activation), "unknown activation");
-    if (cfg->dtype != DLP_FLOAT) // src/gemm.cpp:577
-        return fail(DLP_ERR_NOT_IMPLEMENTED, "only float_data is implemented for IPForward");
+    // float_data as in the reference (src/gemm.cpp:577), plus bfloat16_data storage (fp32 bias and arithmetic)
+    if (cfg->dtype != DLP_FLOAT && cfg->dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "IPForward: float_data and bfloat16_data are implemented");
     dlp_ip_fwd *op = new (std::nothrow) dlp_ip_fwd();
     if (!op)
         return fail(DLP_ERR_RUNTIME, "out of host memory");

@@ -78,6 +78,50 @@ __device__ __forceinline__ void store_out(float *p, float v, float factor)
         *p = v;
 }
 
+// bfloat16 storage element (bfloat16_data): the upper 16 bits of an IEEE float.
+// Arithmetic is always done in fp32; conversion back rounds to nearest even.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __builtin_bit_cast(float, (uint32_t)v.bits << 16); }
+
+__device__ __forceinline__ bf16_t to_bf16(float f)
+{
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) { // NaN stays NaN
+        r.bits = (uint16_t)((u >> 16) | 0x40u);
+        return r;
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+    return r;
+}
+
+__device__ __forceinline__ void store_out(bf16_t *p, float v, float factor)
+{
+    if (factor != 0.0f)
+        v = fmaf(to_float(*p), factor, v);
+    *p = to_bf16(v);
+}
+
+template <class T>
+__device__ __forceinline__ void store_plain(T *p, float v);
+template <>
+__device__ __forceinline__ void store_plain<float>(float *p, float v)
+{
+    *p = v;
+}
+template <>
+__device__ __forceinline__ void store_plain<bf16_t>(bf16_t *p, float v)
+{
+    *p = to_bf16(v);
+}
+
+inline size_t dtype_size(int dtype) { return dtype == DLP_FLOAT ? 4 : 2; }
+
 // ---- implicit-GEMM convolution (conv_gemm.hip) ------------------------------
 // Gather table entry (8 bytes).  Channel-major K order: one entry per k = {byte offset
 // of tap (c,ky,kx) inside one image's group slice, tap bit or ky|kx<<8}.  Tap-major K

@@ -15,8 +15,8 @@ namespace dlp {
 namespace {
 
 struct PoolArgs {
-    const float *x;
-    float *y;
+    const void *x; // storage type T
+    void *y;
     int planes, H, W, OH, OW;
     int kh, kw, ph, pw, sh, sw;
     int mode; // 0 max, 1 avg
@@ -24,6 +24,7 @@ struct PoolArgs {
 };
 
 // one output element per thread; consecutive threads on consecutive output columns
+template <class T>
 __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
 {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
     const long long t = idx / a.OW;
     const int orow = (int)(t % a.OH);
     const long long plane = t / a.OH;
-    const float *src = a.x + plane * a.H * a.W;
+    const T *src = (const T *)a.x + plane * a.H * a.W;
     int row0 = orow * a.sh - a.ph, col0 = oc * a.sw - a.pw;
     int row1 = row0 + a.kh, col1 = col0 + a.kw;
     const int dr_pad = min(row1, a.H + a.ph) - max(-a.ph, row0);
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
     float val = a.mode == 0 ? -3.402823466e+38f : 0.0f;
     for (int r = row0; r < row1; r++)
         for (int c = col0; c < col1; c++) {
-            const float v = src[(size_t)r * a.W + c];
+            const float v = to_float(src[(size_t)r * a.W + c]);
             val = a.mode == 0 ? fmaxf(val, v) : val + v;
         }
     if (a.mode != 0) {
@@ -58,23 +59,24 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
         else
             val = val * (1.0f / (dr * dc));
     }
-    a.y[idx] = val;
+    store_plain((T *)a.y + idx, val);
 }
 
 // one wavefront per plane: lanes stride over the plane, then a shuffle reduction.
 // The average is accumulated per lane in ascending index order and combined pairwise,
 // so it differs from the reference's single running sum only by fp32 rounding.
-__global__ __launch_bounds__(256) void global_pool_kernel(const float *__restrict__ x, float *__restrict__ y, long long planes, int plane_size,
+template <class T>
+__global__ __launch_bounds__(256) void global_pool_kernel(const T *__restrict__ x, T *__restrict__ y, long long planes, int plane_size,
                                                           int mode)
 {
     const int lane = threadIdx.x & 63;
     const long long plane = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (plane >= planes)
         return;
-    const float *src = x + plane * plane_size;
+    const T *src = x + plane * plane_size;
     float v = mode == 0 ? -3.402823466e+38f : 0.0f;
     for (int i = lane; i < plane_size; i += 64) {
-        const float t = src[i];
+        const float t = to_float(src[i]);
         v = mode == 0 ? fmaxf(v, t) : v + t;
     }
 #pragma unroll
@@ -83,16 +85,17 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const float *__restric
         v = mode == 0 ? fmaxf(v, o) : v + o;
     }
     if (lane == 0)
-        y[plane] = mode == 0 ? v : v * (1.0f / plane_size);
+        store_plain(y + plane, mode == 0 ? v : v * (1.0f / plane_size));
 }
 
-__global__ __launch_bounds__(256) void eltwise_kernel(size_t n, int op, float c1, float c2, int act, const float *__restrict__ a,
-                                                      const float *__restrict__ b, float *__restrict__ c)
+template <class T>
+__global__ __launch_bounds__(256) void eltwise_kernel(size_t n, int op, float c1, float c2, int act, const T *__restrict__ a,
+                                                      const T *__restrict__ b, T *__restrict__ c)
 {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
-        const float x0 = a[i], x1 = b[i];
+        const float x0 = to_float(a[i]), x1 = to_float(b[i]);
         float r;
         if (op == 0)
             r = x0 * c1 + x1 * c2;
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(size_t n, int op, float c1
             r = x0 * x1 * (c1 * c2);
         else
             r = fmaxf(x0 * c1, x1 * c2);
-        c[i] = apply_act(r, act);
+        store_plain(c + i, apply_act(r, act));
     }
 }
 
@@ -114,6 +117,7 @@ struct dlp_pool2d_fwd {
     int mode; // 0 max, 1 avg
     int count_include_pad;
     int global;
+    int dtype;
 };
 
 static int pool_create(const int kernel[2], const int pad[2], const int stride[2], int mode, int cip, int global, int dtype,
@@ -121,8 +125,8 @@ static int pool_create(const int kernel[2], const int pad[2], const int stride[2
 {
     DLP_REQUIRE(out != nullptr, "null argument");
     *out = nullptr;
-    if (dtype != DLP_FLOAT)
-        return fail(DLP_ERR_NOT_IMPLEMENTED, "pooling: only float_data is implemented");
+    if (dtype != DLP_FLOAT && dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "pooling: float_data and bfloat16_data are implemented");
     dlp_pool2d_fwd *op = new (std::nothrow) dlp_pool2d_fwd();
     if (!op)
         return fail(DLP_ERR_RUNTIME, "out of host memory");
@@ -134,6 +138,7 @@ static int pool_create(const int kernel[2], const int pad[2], const int stride[2
     op->mode = mode;
     op->count_include_pad = cip;
     op->global = global;
+    op->dtype = dtype;
     if (!global) {
         for (int i = 0; i < 2; i++)
             if (op->kernel[i] <= 0 || op->stride[i] <= 0 || op->pad[i] < 0) {
@@ -190,8 +195,12 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         const long long plane_size = (long long)x_shape[2] * x_shape[3];
         DLP_REQUIRE(plane_size > 0 && plane_size < 0x7fffffffLL, "plane size");
         TimingScope ts("global_pooling", s);
-        hipLaunchKernelGGL(global_pool_kernel, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const float *)x, (float *)y, planes,
-                           (int)plane_size, op->mode);
+        if (op->dtype == DLP_BFLOAT16)
+            hipLaunchKernelGGL(global_pool_kernel<bf16_t>, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const bf16_t *)x, (bf16_t *)y,
+                               planes, (int)plane_size, op->mode);
+        else
+            hipLaunchKernelGGL(global_pool_kernel<float>, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const float *)x, (float *)y,
+                               planes, (int)plane_size, op->mode);
     } else {
         // the output shape fixes ceil_mode; every window must start inside the padded input (pool.hpp:17-27)
         for (int i = 0; i < 2; i++) {
@@ -199,8 +208,8 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
             DLP_REQUIRE((y_shape[2 + i] - 1) * op->stride[i] < x_shape[2 + i] + op->pad[i], "output larger than the pooling geometry allows");
         }
         PoolArgs a;
-        a.x = (const float *)x;
-        a.y = (float *)y;
+        a.x = x;
+        a.y = y;
         a.planes = (int)planes;
         a.H = x_shape[2];
         a.W = x_shape[3];
@@ -217,7 +226,10 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         const long long total = planes * a.OH * a.OW;
         DLP_REQUIRE(planes < 0x7fffffffLL && total < 0x7fffffffLL * 256, "tensor too large");
         TimingScope ts("pooling", s);
-        hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+        if (op->dtype == DLP_BFLOAT16)
+            hipLaunchKernelGGL(pool2d_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+        else
+            hipLaunchKernelGGL(pool2d_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
@@ -225,9 +237,28 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
 
 void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op) { delete op; }
 
+static int eltwise_launch(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b,
+                          void *c, void *stream);
+
 int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b, void *c,
                             void *stream)
 {
+    return eltwise_launch(DLP_FLOAT, operation, coef1, coef2, activation, n, a, b, c, stream);
+}
+
+int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a,
+                                  const void *b, void *c, void *stream)
+{
+    return eltwise_launch(dtype, operation, coef1, coef2, activation, n, a, b, c, stream);
+}
+
+} // extern "C"
+
+static int eltwise_launch(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b,
+                          void *c, void *stream)
+{
+    if (dtype != DLP_FLOAT && dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "elementwise: float_data and bfloat16_data are implemented");
     DLP_REQUIRE(operation >= 0 && operation <= 2, "unknown elementwise operation");
     DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
     if (n == 0)
@@ -237,10 +268,12 @@ int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activat
     if (blocks > 256 * 32)
         blocks = 256 * 32;
     TimingScope ts("eltwise", (hipStream_t)stream);
-    hipLaunchKernelGGL(eltwise_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n, operation, coef1, coef2, activation,
-                       (const float *)a, (const float *)b, (float *)c);
+    if (dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(eltwise_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n, operation, coef1, coef2,
+                           activation, (const bf16_t *)a, (const bf16_t *)b, (bf16_t *)c);
+    else
+        hipLaunchKernelGGL(eltwise_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n, operation, coef1, coef2,
+                           activation, (const float *)a, (const float *)b, (float *)c);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
-
-} // extern "C"

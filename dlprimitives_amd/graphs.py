@@ -114,28 +114,32 @@ def infer_shapes(ops, in_shape):
 class GraphRunner:
     """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
 
-    def __init__(self, ops, params, in_shape, algo=""):
+    def __init__(self, ops, params, in_shape, algo="", dtype="float32"):
+        """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32)."""
         import torch
 
         import dlprimitives_amd as dlp
+        from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA
 
         self.ops = ops
         self.shapes = infer_shapes(ops, in_shape)
-        self.t = {n: torch.empty(s, dtype=torch.float32, device="cuda:0") for n, s in self.shapes.items()}
-        self.p = {n: (torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()) for n, (w, b) in params.items()}
+        tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+        code = BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA
+        self.t = {n: torch.empty(s, dtype=tdt, device="cuda:0") for n, s in self.shapes.items()}
+        self.p = {n: (torch.from_numpy(w).cuda().to(tdt), torch.from_numpy(b).cuda()) for n, (w, b) in params.items()}
         self.k = []
         ws_bytes = 1
         for o in ops:
             if o["op"] == "conv":
-                st = dlp.Conv2DSettings(o["cin"], o["cout"], o["k"], o["s"], 1, o["p"], 1, self.shapes[o["src"]])
+                st = dlp.Conv2DSettings(o["cin"], o["cout"], o["k"], o["s"], 1, o["p"], 1, self.shapes[o["src"]], dtype=code)
                 op = dlp.Conv2DForward.create(st, True, o["act"], algo)
                 ws_bytes = max(ws_bytes, op.workspace())
             elif o["op"] == "maxpool":
-                op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"])
+                op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"], dtype=code)
             elif o["op"] == "gap":
-                op = dlp.Pooling2DForward.create_global_avg_pooling()
+                op = dlp.Pooling2DForward.create_global_avg_pooling(dtype=code)
             elif o["op"] == "ip":
-                op = dlp.IPForward.create(dlp.IPSettings(o["inputs"], o["outputs"], in_shape[0]), True, "identity")
+                op = dlp.IPForward.create(dlp.IPSettings(o["inputs"], o["outputs"], in_shape[0], dtype=code), True, "identity")
             else:
                 op = None
             self.k.append(op)

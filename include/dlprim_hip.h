@@ -157,6 +157,17 @@ void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op);
 #define DLP_ELTWISE_MAX 2
 int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b, void *c,
                             void *stream);
+/* same for tensors stored as `dtype` (DLP_FLOAT or DLP_BFLOAT16; arithmetic in fp32) */
+int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a,
+                                  const void *b, void *c, void *stream);
+
+/* ===== data types ==================================================================
+ * DLP_FLOAT: everything fp32, as in the reference (its conv/GEMM reject other types,
+ * src/gemm.cpp:577,593).  DLP_BFLOAT16 (an extension): x, w, y of Conv2DForward and
+ * IPForward and the tensors of the glue operators are stored as bfloat16; bias stays
+ * fp32; products are accumulated in fp32 on the matrix cores and the epilogue runs in
+ * fp32 before one round-to-nearest-even conversion of the result.  The "winograd" and
+ * "depthwise_separable" algorithms serve DLP_FLOAT only; other requests run as "gemm". */
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,119 @@
+"""bfloat16 storage (x, w, y as bf16; bias, accumulation and epilogue in fp32): the reference has
+no reduced-precision path, so the bar is 1e-2 relative to the fp32 reference (the oracle)."""
+import numpy as np
+import pytest
+
+from conv_cases import case, case_id, make_tensors
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0").to(torch.bfloat16)
+
+
+def run_conv_bf16(c, x, w, bias, algo="", factor=0.0, y_init=None):
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
+    op = dlp.Conv2DForward.create(st, bias is not None, c["activation"], algo)
+    assert op.algo() == "gemm"
+    y = _bf(y_init) if y_init is not None else torch.full(dlp.conv2d_output_shape(st, x.shape), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    bd = torch.from_numpy(bias).cuda() if bias is not None else None
+    op.enqueue(_bf(x), _bf(w), bd, y, ws, factor)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+CASES = [
+    (case(3, 1, 1, 1, 64, 64, True, 1, True), (2, 56, 56)),
+    (case(1, 0, 1, 1, 256, 64, True, 1, True), (2, 56, 56)),
+    (case(1, 0, 2, 1, 256, 512, True, 1, False), (2, 56, 56)),
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (2, 224, 224)),
+    (case(3, 1, 2, 1, 128, 128, True, 1, True), (2, 56, 56)),
+    (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),      # split-K path
+    (case((3, 5), (1, 2), (2, 3), (3, 2), 3, 8, False, 1, False), (2, 19, 19)),
+    (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise request falls back to gemm
+]
+
+
+@pytest.mark.parametrize("c,bhw", CASES, ids=case_id)
+def test_bf16_conv_vs_fp32_reference(oracle_mod, c, bhw):
+    x, w, bias = make_tensors(c, bhw, seed=21)
+    got = run_conv_bf16(c, x, w, bias)
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    # the fp32 reference on the fp32 tensors: bf16 storage may cost up to 1e-2 relative
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-2 * scale
+    # and against the oracle fed the same bf16-rounded operands only the output rounding (2^-9) remains
+    want_r = oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, c["activation"], threads=8)
+    np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=1e-4 * scale)
+
+
+def test_bf16_factor_contract(oracle_mod):
+    c = case(3, 1, 1, 1, 16, 24, True, 1, True)
+    x, w, bias = make_tensors(c, (2, 11, 9), seed=5)
+    cfg = oracle_mod.make_cfg(16, 24, 3, 1, 1, 1, 1)
+    old = np.random.default_rng(1).standard_normal((2, 24, 11, 9)).astype(np.float32)
+    got = run_conv_bf16(c, x, w, bias, factor=0.5, y_init=old)
+    want = oracle_mod.apply_factor(oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, "relu"),
+                                   oracle_mod.bf16_round(old), 0.5)
+    np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-3)
+
+
+def test_bf16_glue_and_inner_product(oracle_mod):
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    rng = np.random.default_rng(4)
+    x = oracle_mod.bf16_round(rng.standard_normal((2, 16, 14, 14)).astype(np.float32))
+    y = torch.empty((2, 16, 7, 7), dtype=torch.bfloat16, device="cuda:0")
+    dlp.Pooling2DForward.create_max_pooling(3, 1, 2, dtype=BFLOAT16_DATA).enqueue(_bf(x), y)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.float().cpu().numpy(), oracle_mod.pool2d_forward(x, 3, 1, 2, "max"))  # max of bf16 values is exact
+    g = torch.empty((2, 16, 1, 1), dtype=torch.bfloat16, device="cuda:0")
+    dlp.Pooling2DForward.create_global_avg_pooling(dtype=BFLOAT16_DATA).enqueue(_bf(x), g)
+    b2 = oracle_mod.bf16_round(rng.standard_normal(x.shape).astype(np.float32))
+    s = torch.empty(x.shape, dtype=torch.bfloat16, device="cuda:0")
+    dlp.eltwise_forward(_bf(x), _bf(b2), s, "sum", 1.0, 1.0, "relu")
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(g.float().cpu().numpy(), oracle_mod.global_pool_forward(x, "avg"), rtol=2 ** -8, atol=1e-3)
+    np.testing.assert_allclose(s.float().cpu().numpy(), oracle_mod.eltwise_forward(x, b2, "sum", 1.0, 1.0, "relu"), rtol=2 ** -8, atol=1e-3)
+    xi = rng.uniform(-1, 1, (128, 2048)).astype(np.float32)
+    wi = (rng.standard_normal((1000, 2048)) / np.sqrt(2048)).astype(np.float32)
+    bi = rng.uniform(-0.1, 0.1, 1000).astype(np.float32)
+    ip = dlp.IPForward.create(dlp.IPSettings(2048, 1000, 128, dtype=BFLOAT16_DATA), True, "identity")
+    yi = torch.empty((128, 1000), dtype=torch.bfloat16, device="cuda:0")
+    ip.enqueue(_bf(xi), _bf(wi), torch.from_numpy(bi).cuda(), yi)
+    torch.cuda.synchronize()
+    want = oracle_mod.ip_forward(xi, wi, bi)
+    assert np.abs(yi.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
+
+
+def test_resnet50_bf16_logits_vs_fp32_reference(oracle_mod):
+    """Configuration 5 at a batch the CPU oracle finishes in seconds: ResNet-50 forward with bf16
+    storage against the fp32 reference path on the same fp32 weights and inputs, 1e-2 relative."""
+    import torch
+
+    from dlprimitives_amd import graphs
+    from graph_oracle import run_graph_on_oracle
+
+    ops = graphs.resnet50()
+    params = graphs.random_parameters(ops, seed=11)
+    x = np.random.default_rng(3).standard_normal((4, 3, 224, 224)).astype(np.float32)
+    runner = graphs.GraphRunner(ops, params, x.shape, algo="", dtype="bfloat16")
+    got = runner.forward(torch.from_numpy(x).cuda().to(torch.bfloat16)).float().cpu().numpy()
+    want = run_graph_on_oracle(oracle_mod, ops, params, x)
+    rel = np.abs(got - want).max() / np.abs(want).max()
+    print("resnet50 bf16 vs fp32 reference: max relative error of the logits %.4f" % rel)
+    assert rel <= 1e-2
+    assert (got.argmax(1) == want.argmax(1)).all()
