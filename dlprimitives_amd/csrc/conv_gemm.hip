@@ -75,12 +75,6 @@ struct GemmArgs {
 
 typedef __attribute__((address_space(4))) const int32_t ConstInt;
 
-// q = n / d for 0 <= n < 2^31 with host-made (magic, shift)
-__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shift)
-{
-    return (__umulhi(n, magic) + n) >> shift;
-}
-
 // one storage element, widened to fp32 (bf16 -> fp32 is a 16-bit shift)
 template <class T>
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff);
@@ -550,15 +544,6 @@ int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipS
     if (p.mask == GEMM_MASK_TAPS)
         return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
     return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
-}
-
-void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
-{
-    // q = (umulhi(n, magic) + n) >> shift  ==  n / d   for 0 <= n < 2^31
-    shift = 0;
-    while ((1ull << shift) < d)
-        shift++;
-    magic = (uint32_t)(((1ull << 32) * ((1ull << shift) - d)) / d + 1);
 }
 
 // Workgroup tiles.  Small tiles win on this chip: fp32 MFMA is slow enough (64 cycles

@@ -290,7 +290,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     DLP_REQUIRE(valid_activation(activation), "unknown activation");
     // The reference checks dtype == float_data (src/gemm.cpp:593).  Here bfloat16_data is
     // also accepted: x, w, y are stored as bf16, bias stays fp32, all arithmetic is fp32
-    // (the implicit-GEMM algorithm serves it; Winograd / depthwise requests fall back to it).
+    // (the implicit-GEMM and Winograd algorithms serve it; depthwise requests fall back to gemm).
     if (cfg->dtype != DLP_FLOAT && cfg->dtype != DLP_BFLOAT16)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "Conv2DForward: float_data and bfloat16_data are implemented");
     std::string al = algo ? algo : "";
@@ -329,7 +329,6 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     } else if (chosen == ALGO_WINOGRAD) {
         op->wino = winograd_plan(g);
         op->workspace = op->wino.ws_bytes;
-        rc = upload_ktab(op->wino.gemm, DLP_ACT_IDENTITY, &op->ktab);
     }
     if (rc != DLP_OK) {
         delete op;
@@ -380,7 +379,7 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
     hipStream_t s = (hipStream_t)stream;
     switch (op->algo) {
     case ALGO_WINOGRAD:
-        return winograd_launch(g, op->wino, op->ktab, x, w, y, ws, ws_bytes, ep, s);
+        return winograd_launch(g, op->wino, x, w, y, ws, ws_bytes, ep, s);
     case ALGO_DEPTHWISE:
         return depthwise_launch(g, x, w, y, ep, s);
     default: {

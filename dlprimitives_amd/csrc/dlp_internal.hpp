@@ -122,6 +122,19 @@ __device__ __forceinline__ void store_plain<bf16_t>(bf16_t *p, float v)
 
 inline size_t dtype_size(int dtype) { return dtype == DLP_FLOAT ? 4 : 2; }
 
+// Division by a launch-time constant: q = (umulhi(n, magic) + n) >> shift == n / d for 0 <= n < 2^31.
+inline void make_magic(uint32_t d, uint32_t &magic, uint32_t &shift)
+{
+    shift = 0;
+    while ((1ull << shift) < d)
+        shift++;
+    magic = (uint32_t)(((1ull << 32) * ((1ull << shift) - d)) / d + 1);
+}
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shift)
+{
+    return (__umulhi(n, magic) + n) >> shift;
+}
+
 // ---- implicit-GEMM convolution (conv_gemm.hip) ------------------------------
 // Gather table entry (8 bytes).  Channel-major K order: one entry per k = {byte offset
 // of tap (c,ky,kx) inside one image's group slice, tap bit or ky|kx<<8}.  Tap-major K
@@ -166,16 +179,16 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
 
 // ---- Winograd F(2x2,3x3) (conv_winograd.hip) ---------------------------------
 struct WinoPlan {
-    int chunk_imgs;  // images transformed and multiplied per pass
-    int tcap;        // tiles per pass = row stride of the V and M workspace matrices
-    size_t ws_bytes; // workspace() of the op
-    ConvGeom gemm;   // grouped 1x1 geometry that runs the 16 GEMMs of a pass
-    GemmPlan gplan;  // its launch plan (the filter transform writes the packed layout directly)
+    int Cpad, Npad;  // input / output channels rounded up to the kernel's K chunk / channel tile
+    int chunk_imgs;  // images per launch (keeps 32-bit byte offsets in range)
+    int stage_stride; // floats per channel of the LDS row staging buffer; 0 = patches gathered from global memory
+    int stage_loads;  // staged variant: elements copied per thread and K chunk (8 or 16)
+    size_t ws_bytes; // workspace() of the op: the transformed filter U[16][Cpad][Npad], fp32
 };
 bool winograd_supported(const ConvGeom &g);
-WinoPlan winograd_plan(const ConvGeom &g); // g.B = batch hint
-int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const KTabEntry *gemm_ktab, const void *x, const void *w, void *y,
-                    void *ws, size_t ws_bytes, const Epilogue &ep, hipStream_t stream);
+WinoPlan winograd_plan(const ConvGeom &g);
+int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, size_t ws_bytes,
+                    const Epilogue &ep, hipStream_t stream);
 
 // ---- InnerProduct GEMM (ip_gemm.hip) ------------------------------------------
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype);

@@ -88,7 +88,7 @@ int dlp_stream_destroy(void *stream);
  *      (include/dlprim/context.hpp:23-94,180,237-243).  While enabled, every kernel
  *      launched by the calls below is bracketed by a HIP event pair on its stream and
  *      recorded under a section name ("conv_gemm", "pack_weights", "splitk_reduce",
- *      "sep_conv", "winograd_filter", "winograd_input", "winograd_output").
+ *      "sep_conv", "winograd_filter", "winograd_fused", "pooling", "global_pooling", "eltwise").
  *      dlp_timing_get waits for the record's kernel to finish. -------------------- */
 int dlp_timing_enable(int on);
 int dlp_timing_reset(void);
@@ -166,8 +166,9 @@ int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float c
  * src/gemm.cpp:577,593).  DLP_BFLOAT16 (an extension): x, w, y of Conv2DForward and
  * IPForward and the tensors of the glue operators are stored as bfloat16; bias stays
  * fp32; products are accumulated in fp32 on the matrix cores and the epilogue runs in
- * fp32 before one round-to-nearest-even conversion of the result.  The "winograd" and
- * "depthwise_separable" algorithms serve DLP_FLOAT only; other requests run as "gemm". */
+ * fp32 before one round-to-nearest-even conversion of the result ("gemm" and "winograd";
+ * the Winograd transforms also run in fp32).  The "depthwise_separable" algorithm serves
+ * DLP_FLOAT only; a DLP_BFLOAT16 request for it runs as "gemm". */
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@ def run_conv_bf16(c, x, w, bias, algo="", factor=0.0, y_init=None):
 
     st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
     op = dlp.Conv2DForward.create(st, bias is not None, c["activation"], algo)
-    assert op.algo() == "gemm"
+    assert op.algo() == (algo if algo in ("gemm", "winograd") else "gemm")
     y = _bf(y_init) if y_init is not None else torch.full(dlp.conv2d_output_shape(st, x.shape), float("nan"), dtype=torch.bfloat16, device="cuda:0")
     ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
     bd = torch.from_numpy(bias).cuda() if bias is not None else None
@@ -39,14 +39,14 @@ CASES = [
     (case(3, 1, 2, 1, 128, 128, True, 1, True), (2, 56, 56)),
     (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),      # split-K path
     (case((3, 5), (1, 2), (2, 3), (3, 2), 3, 8, False, 1, False), (2, 19, 19)),
-    (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise request falls back to gemm
+    (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise geometry, served by gemm
 ]
 
 
 @pytest.mark.parametrize("c,bhw", CASES, ids=case_id)
 def test_bf16_conv_vs_fp32_reference(oracle_mod, c, bhw):
     x, w, bias = make_tensors(c, bhw, seed=21)
-    got = run_conv_bf16(c, x, w, bias)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm")
     cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
     # the fp32 reference on the fp32 tensors: bf16 storage may cost up to 1e-2 relative
     want = oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8)
@@ -57,12 +57,25 @@ def test_bf16_conv_vs_fp32_reference(oracle_mod, c, bhw):
     np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=1e-4 * scale)
 
 
+@pytest.mark.parametrize("cin,cout,bhw", [(64, 64, (2, 56, 56)), (24, 40, (3, 13, 9)), (128, 128, (4, 28, 28)), (512, 512, (3, 7, 7))])
+def test_bf16_winograd_vs_fp32_reference(oracle_mod, cin, cout, bhw):
+    c = case(3, 1, 1, 1, cin, cout, True, 1, True)
+    x, w, bias = make_tensors(c, bhw, seed=22)
+    got = run_conv_bf16(c, x, w, bias, algo="winograd")
+    cfg = oracle_mod.make_cfg(cin, cout, 3, 1, 1, 1, 1)
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, "relu", threads=8)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-2 * scale
+    want_r = oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, "relu", threads=8)
+    np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=2e-4 * scale)
+
+
 def test_bf16_factor_contract(oracle_mod):
     c = case(3, 1, 1, 1, 16, 24, True, 1, True)
     x, w, bias = make_tensors(c, (2, 11, 9), seed=5)
     cfg = oracle_mod.make_cfg(16, 24, 3, 1, 1, 1, 1)
     old = np.random.default_rng(1).standard_normal((2, 24, 11, 9)).astype(np.float32)
-    got = run_conv_bf16(c, x, w, bias, factor=0.5, y_init=old)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
     want = oracle_mod.apply_factor(oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, "relu"),
                                    oracle_mod.bf16_round(old), 0.5)
     np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-3)
