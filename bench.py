@@ -36,6 +36,15 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
 BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 images/sec"
 
+# HBM bytes per launch of the dominant kernel of each workload at batch 64, from hardware
+# counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, one counter per run, KiB per dispatch,
+# scaled by what the same counter reads for a plain copy of known size: x2.0 / x1.0).
+# Measured offline (a benchmark run cannot collect counters on itself); keyed by (workload, kernel).
+MEASURED_TRAFFIC_BYTES = {
+    ("resnet18", "conv_gemm_f32_kernel<float, 64, 64, 2, 2, 1, 1, 0>"): (17849.2 * 2.0 + 27428.2) * 1024,
+    ("winograd", "wino_fused_kernel<float, ...>"): ((16818.7 + 40712.3) / 2 * 2.0 + (25373.0 + 12838.7) / 2) * 1024,
+}
+
 
 def workload_layers(name):
     from dlprimitives_amd.workloads import MOBILENET_DEPTHWISE, MOBILENET_POINTWISE, RESNET18_CONVS, WINOGRAD_SHAPES, conv
@@ -89,7 +98,7 @@ def kernel_class(L):
     cin_g = L["cin"] // L["groups"]
     m = L["cout"] // L["groups"]
     if L["algo"] == "winograd":
-        return "wino_fused_kernel<float>"
+        return "wino_fused_kernel<float, ...>"
     tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     small = L["kernel"] ** 2 <= 32
     order = 1 if (small and cin_g % 16 == 0) else 0
@@ -285,8 +294,11 @@ def main():
     else:
         achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
         roofline = dict(bound="mfma", kernel=dom_name, launches_per_step=dom["launches"], avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
-                        flops_per_launch=dom["flops"] / dom["launches"], achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS,
+                        flops_per_launch=dom["flops"] / dom["launches"], bytes_per_launch=dom["bytes"] / dom["launches"],
+                        achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS,
                         unit="TFLOP/s", frac=round(achieved / FP32_MATRIX_PEAK_TFLOPS, 4), traffic=None)
+    if args.batch == 64 and not args.only:
+        roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dom_name))
     if args.layers:
         for r in table:
             print(json.dumps(r), file=sys.stderr)

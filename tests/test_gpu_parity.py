@@ -180,7 +180,13 @@ def test_algorithm_selection_rules(gpu):
 
 # ------------------------------------------------------------ Winograd
 @pytest.mark.parametrize("shape", [(2, 128, 128, 28, 28), (2, 256, 256, 14, 14), (3, 8, 16, 7, 9), (1, 16, 8, 1, 1), (2, 24, 40, 5, 6),
-                                   (5, 16, 16, 13, 13)],
+                                   (5, 16, 16, 13, 13),
+                                   (2, 12, 20, 9, 10),    # Cin not a multiple of the K chunk (masked channel tail), rows staged in LDS
+                                   (3, 3, 8, 8, 8),       # fewer channels than one K chunk
+                                   (1, 16, 32, 56, 56),   # rows of 32 tiles do not fit the staging buffer: patches gathered from global memory
+                                   (1, 11, 8, 10, 120),   # the same with a masked channel tail and a wide image
+                                   (40, 8, 8, 3, 3),      # more than four images per workgroup
+                                   (9, 16, 16, 7, 7)],    # a workgroup's tiles span three images
                          ids=lambda s: "b%d_c%d_n%d_%dx%d" % s)
 def test_winograd_three_way(gpu, oracle_mod, shape):
     B, C, N, H, W = shape
