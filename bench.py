@@ -33,6 +33,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3
+BF16_MATRIX_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 images/sec"
 
@@ -51,6 +52,9 @@ def workload_layers(name):
 
     if name == "resnet18":
         return [dict(L, algo="gemm") for L in RESNET18_CONVS], "ResNet-18 conv stack forward: 20 convs, BN folded, fused ReLU, algo gemm"
+    if name == "resnet50":
+        from dlprimitives_amd.workloads import RESNET50_CONVS
+        return [dict(L, algo="gemm") for L in RESNET50_CONVS], "ResNet-50 conv stack forward: 53 convs, BN folded, algo gemm"
     if name == "mobilenet":
         layers = []
         for (c, hw) in MOBILENET_DEPTHWISE:
@@ -67,43 +71,52 @@ def workload_layers(name):
     raise SystemExit("unknown workload " + name)
 
 
-def build_layers(layer_list, batch, seed):
+def build_layers(layer_list, batch, seed, bf16=False):
     import numpy as np
     import torch
 
     import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA
     from dlprimitives_amd.workloads import conv_bytes, conv_flops
 
     rng = np.random.default_rng(seed)
+    tdt = torch.bfloat16 if bf16 else torch.float32
     out = []
     for L in layer_list:
         cin_g = L["cin"] // L["groups"]
-        x = torch.from_numpy(rng.uniform(-1, 1, (batch, L["cin"], L["hw"], L["hw"])).astype(np.float32)).cuda()
+        x = torch.from_numpy(rng.uniform(-1, 1, (batch, L["cin"], L["hw"], L["hw"])).astype(np.float32)).cuda().to(tdt)
         w = torch.from_numpy((rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) *
-                              np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)).cuda()
+                              np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)).cuda().to(tdt)
         b = torch.from_numpy(rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)).cuda()
-        y = torch.empty((batch, L["cout"], L["ohw"], L["ohw"]), dtype=torch.float32, device="cuda")
-        st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], tuple(x.shape))
+        y = torch.empty((batch, L["cout"], L["ohw"], L["ohw"]), dtype=tdt, device="cuda")
+        st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], tuple(x.shape),
+                                dtype=BFLOAT16_DATA if bf16 else FLOAT_DATA)
         op = dlp.Conv2DForward.create(st, True, L["activation"], L["algo"])
         assert op.algo() == L["algo"], (op.algo(), L["algo"])
         ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
-        out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch)))
+        out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch, 2 if bf16 else 4)))
     return out
 
 
-def kernel_class(L):
+def kernel_class(L, bf16=False):
     """Name of the kernel that does the layer's arithmetic, as a profiler lists it."""
     if L["algo"] == "depthwise_separable":
         return "depthwise3x3_kernel<%d>" % L["stride"]
     cin_g = L["cin"] // L["groups"]
     m = L["cout"] // L["groups"]
     if L["algo"] == "winograd":
-        return "wino_fused_kernel<float, ...>"
-    tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
+        return "wino_fused_kernel<%s, ...>" % ("bf16_t" if bf16 else "float")
     small = L["kernel"] ** 2 <= 32
+    if bf16 and small and cin_g % 32 == 0 and L["activation"] not in ("tanh", "sigmoid"):
+        return "conv_gemm_bf16_kernel<%s, 0>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4")
+    tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     order = 1 if (small and cin_g % 16 == 0) else 0
     mask = 1 if small else 2
-    return "conv_gemm_f32_kernel<float, %s, %d, %d, 0>" % (tile, order, mask)
+    return "conv_gemm_f32_kernel<%s, %s, %d, %d, 0>" % ("bf16_t" if bf16 else "float", tile, order, mask)
+
+
+def matrix_peak_tflops(kernel_name):
+    return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith("conv_gemm_bf16_kernel") else FP32_MATRIX_PEAK_TFLOPS
 
 
 MAIN_SECTION = {"gemm": "conv_gemm", "winograd": "winograd_fused", "depthwise_separable": "sep_conv"}
@@ -194,9 +207,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full"])
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full"])
     ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the -full workloads (arithmetic is fp32 either way)")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
@@ -224,7 +237,8 @@ def main():
         if not layer_list:
             print("bench.py: --only matches no layer", file=sys.stderr)
             sys.exit(2)
-    layers = build_layers(layer_list, args.batch, 2024)
+    bf16 = args.dtype == "bf16"
+    layers = build_layers(layer_list, args.batch, 2024, bf16)
     stream = torch.cuda.current_stream()
 
     def step():
@@ -271,13 +285,15 @@ def main():
     classes = {}
     for e, ms, kms in zip(layers, layer_ms, kernel_ms):
         L = e["layer"]
+        kname = kernel_class(L, bf16)
+        peak = matrix_peak_tflops(kname) * 1e12
         ai = e["flops"] / e["bytes"]
-        mfma_bound = ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12
-        roof = min(FP32_MATRIX_PEAK_TFLOPS * 1e12, ai * HBM_PEAK_GBS * 1e9)
+        mfma_bound = ai * HBM_PEAK_GBS * 1e9 >= peak
+        roof = min(peak, ai * HBM_PEAK_GBS * 1e9)
         ach = e["flops"] / (ms * 1e-3)
         table.append(dict(name=L["name"], ms=round(ms, 4), main_kernel_ms=round(kms, 4), tflops=round(ach / 1e12, 2), gbs=round(e["bytes"] / (ms * 1e-3) / 1e9, 1),
-                          bound="mfma" if mfma_bound else "hbm", frac_of_roofline=round(ach / roof, 4), kernel=kernel_class(L)))
-        c = classes.setdefault(kernel_class(L), dict(ms=0.0, flops=0.0, bytes=0.0, launches=0, hbm=0))
+                          bound="mfma" if mfma_bound else "hbm", frac_of_roofline=round(ach / roof, 4), kernel=kname))
+        c = classes.setdefault(kname, dict(ms=0.0, flops=0.0, bytes=0.0, launches=0, hbm=0))
         c["ms"] += kms
         # Winograd F(2x2,3x3) multiplies 16 values per 2x2 outputs instead of 36: the matrix-core
         # fraction is scored on the flops actually issued (direct / 2.25), so it cannot pass 100 %
@@ -293,17 +309,18 @@ def main():
                         frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
     else:
         achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+        peak_tf = matrix_peak_tflops(dom_name)
         roofline = dict(bound="mfma", kernel=dom_name, launches_per_step=dom["launches"], avg_launch_ms=round(dom["ms"] / dom["launches"], 4),
                         flops_per_launch=dom["flops"] / dom["launches"], bytes_per_launch=dom["bytes"] / dom["launches"],
-                        achieved=round(achieved, 2), peak=FP32_MATRIX_PEAK_TFLOPS,
-                        unit="TFLOP/s", frac=round(achieved / FP32_MATRIX_PEAK_TFLOPS, 4), traffic=None)
+                        achieved=round(achieved, 2), peak=peak_tf,
+                        unit="TFLOP/s", frac=round(achieved / peak_tf, 4), traffic=None)
     if args.batch == 64 and not args.only:
         roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dom_name))
     if args.layers:
         for r in table:
             print(json.dumps(r), file=sys.stderr)
 
-    cpu = cpu_baseline(layer_list, args.cpu_images, 2024) if args.cpu_images > 0 else None
+    cpu = cpu_baseline(layer_list, args.cpu_images, 2024) if args.cpu_images > 0 else None  # the fp32 reference path
 
     out = {
         "metric": BASELINE_METRIC,
@@ -316,9 +333,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32",
         "data": "synthetic",
-        "config": {"workload": "%s%s, fp32 NCHW, batch %d" % (description, " (subset --only %s)" % args.only if args.only else "", args.batch),
+        "config": {"workload": "%s%s, %s NCHW, batch %d" % (description, " (subset --only %s)" % args.only if args.only else "",
+                                                            "bf16" if bf16 else "fp32", args.batch),
                    "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1),
                    "mbytes_per_step": round(total_bytes / 1e6, 1)},
         "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),

@@ -406,6 +406,256 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     }
 }
 
+// ---- bfloat16 storage on the bf16 matrix instruction ------------------------------------
+// Same implicit GEMM for tensors stored as bf16 whose Cin/groups is a multiple of 32:
+// v_mfma_f32_32x32x16_bf16 (fp32 accumulate) is 16 times faster per flop than the fp32
+// instruction, so everything is sized for operand delivery instead:
+//  * K tile = one filter tap x 32 channels (two MFMA k steps);
+//  * an MFMA operand is 8 consecutive k of one row per lane, so LDS holds A as [m][k] and B
+//    as [pixel][k] with rows of 32 + 8 bf16 (80 bytes: the 16-byte accesses of 16 consecutive
+//    rows fall on distinct banks) and every operand fetch is one ds_read_b128;
+//  * the gathered input arrives pixel-per-lane (NCHW keeps pixels contiguous), one 16-bit
+//    element per load; a thread owns one pixel and 16 or 32 channels, packs pairs with one
+//    VALU op each and stores 16-byte pieces of its pixel's row;
+//  * weights are pre-packed as bf16 in [m tile][K tile][m][32] order (16-byte pieces per thread);
+//  * 128x128 tiles (wavefront 64x64), or 64x256 when M <= 64.
+// The sum over k is accumulated in fp32 exactly as in the fp32 kernel (products of bf16 values
+// are exact in fp32), only in a different order.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int BK2 = 32;
+constexpr int LDK = BK2 + 8;
+
+template <int BM, int BN, int WM, int WN, int ACT>
+__global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
+{
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "tile shape");
+    constexpr int KSPLIT = kThreads / BN;   // channel groups among the B loader threads
+    static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK2 % KSPLIT == 0, "B loader shape");
+    constexpr int B_LD = BK2 / KSPLIT;      // channels per thread per K tile
+    static_assert(B_LD % 8 == 0, "a thread stores whole 16-byte pieces");
+    constexpr int A_V4 = BM * BK2 * 2 / 16; // 16-byte pieces of a packed A tile
+    static_assert(A_V4 % kThreads == 0, "A loader shape");
+    constexpr int A_LD = A_V4 / kThreads;
+
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM][LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN][LDK];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+
+    int t; // XCD-aware renumbering, as in the fp32 kernel
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, r = nb & 7;
+        const int xcd = bid & 7, slot = bid >> 3;
+        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    }
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    t /= a.ntiles;
+    const int g = t % a.groups;
+    const int slice = t / a.groups;
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int kt_begin = slice * a.kt_per_slice;
+    const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
+
+    const __amdgpu_buffer_rsrc_t xr =
+        __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.x - a.x_shift), 0, a.x_bytes + a.x_shift, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
+    ConstInt *ktab = (ConstInt *)a.ktab;
+
+    // ---- per-thread gather state: one output pixel, B_LD channels of every K tile ----
+    const int p = tid % BN;
+    const int ks = (KSPLIT == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid / BN);
+    uint32_t vbase;
+    uint32_t my = 0;
+    {
+        const int n = n0 + p;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * a.OHW;
+        const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+        const int ox = pix - oy * a.OW;
+        const int iy0 = oy * a.sh - a.ph;
+        const int ix0 = ox * a.sw - a.pw;
+        vbase = (uint32_t)((((b * a.Cin + g * a.Cin_g) * a.H + oy * a.sh) * a.W + ox * a.sw) * 2);
+        if (n < a.N) {
+            uint32_t ry = 0, rx = 0;
+            for (int ky = 0; ky < a.KH; ky++) {
+                int yy = iy0 + ky * a.dh;
+                if (yy >= 0 && yy < a.H)
+                    ry |= 1u << ky;
+            }
+            for (int kx = 0; kx < a.KW; kx++) {
+                int xx = ix0 + kx * a.dw;
+                if (xx >= 0 && xx < a.W)
+                    rx |= 1u << kx;
+            }
+            for (int ky = 0; ky < a.KH; ky++)
+                if ((ry >> ky) & 1u)
+                    my |= rx << (ky * a.KW);
+        }
+    }
+
+    const uint32_t a_tile_bytes = BM * BK2 * 2;
+    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
+
+    u32x4 ra[2][A_LD];
+    uint32_t rb[2][B_LD]; // one bf16 each, zero extended
+    uint32_t vsel[2] = {kOutOfRange, kOutOfRange};
+
+    auto load_half = [&](auto set, int kt, auto half_c) {
+        constexpr int S = decltype(set)::value;
+        constexpr int Q = decltype(half_c)::value;
+        if (Q == 0) {
+            const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
+#pragma unroll
+            for (int j = 0; j < A_LD; j++)
+                ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
+        }
+        ConstInt *e = ktab + kt * 4;
+        const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
+        if (Q == 0)
+            vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
+#pragma unroll
+        for (int i = Q * (B_LD / 2); i < (Q + 1) * (B_LD / 2); i++)
+            rb[S][i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4, 0);
+    };
+    auto store_half = [&](auto set, auto buf_c, auto half_c) {
+        constexpr int S = decltype(set)::value;
+        constexpr int BUF = decltype(buf_c)::value;
+        constexpr int Q = decltype(half_c)::value;
+        if (Q == 0) {
+#pragma unroll
+            for (int j = 0; j < A_LD; j++) {
+                const int idx = tid + j * kThreads; // 16-byte piece of the [BM][32] tile: row idx/4, piece idx%4
+                *(u32x4 *)&As[BUF][idx >> 2][(idx & 3) * 8] = ra[S][j];
+            }
+        }
+#pragma unroll
+        for (int q = Q * (B_LD / 16); q < (Q + 1) * (B_LD / 16); q++) {
+            u32x4 v;
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                v[d] = rb[S][8 * q + 2 * d] | (rb[S][8 * q + 2 * d + 1] << 16);
+            *(u32x4 *)&Bs[BUF][p][ks * B_LD + 8 * q] = v;
+        }
+    };
+    static_assert(B_LD % 16 == 0, "each half of a K step stores whole pieces");
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    // K step on tile kt in LDS[BUF]: set_next (tile kt+1) -> LDS[BUF^1], tile kt+2 -> set_load
+    auto k_step = [&](auto buf_c, auto set_next, auto set_load, int kt) {
+        constexpr int BUF = decltype(buf_c)::value;
+        using NextBuf = std::integral_constant<int, BUF ^ 1>;
+        bf16x8 fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                fa[s][i] = *(const bf16x8 *)&As[BUF][wm * WTM + i * 32 + l32][s * 16 + h * 8];
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                fb[s][j] = *(const bf16x8 *)&Bs[BUF][wn * WTN + j * 32 + l32][s * 16 + h * 8];
+        }
+        store_half(set_next, NextBuf{}, std::integral_constant<int, 0>{});
+        load_half(set_load, kt + 2, std::integral_constant<int, 0>{});
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+        store_half(set_next, NextBuf{}, std::integral_constant<int, 1>{});
+        load_half(set_load, kt + 2, std::integral_constant<int, 1>{});
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+        __syncthreads();
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    load_half(I0{}, kt_begin, I0{});
+    load_half(I0{}, kt_begin, I1{});
+    load_half(I1{}, kt_begin + 1, I0{});
+    load_half(I1{}, kt_begin + 1, I1{});
+    store_half(I0{}, I0{}, I0{});
+    store_half(I0{}, I0{}, I1{});
+    __syncthreads();
+    int kt = kt_begin;
+    for (; kt + 1 < kt_end; kt += 2) {
+        k_step(I0{}, I1{}, I0{}, kt);
+        k_step(I1{}, I0{}, I1{}, kt + 1);
+    }
+    if (kt < kt_end)
+        k_step(I0{}, I1{}, I0{}, kt);
+
+    if (a.splitk > 1) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            if (n >= a.N)
+                continue;
+            float *pb = a.part + ((size_t)slice * a.Cout + (size_t)g * a.M) * a.N + n;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < a.M)
+                        pb[(size_t)m * a.N] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
+
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + l32;
+        if (n >= a.N)
+            continue;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * a.OHW;
+        bf16_t *yb = (bf16_t *)a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < a.M) {
+                    float v = acc[i][j][r];
+                    if (a.bias)
+                        v += a.bias[g * a.M + m];
+                    if (ACT == ACT_CLAMP) {
+                        if (a.act != DLP_ACT_IDENTITY)
+                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                    } else
+                        v = apply_act(v, a.act);
+                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
+                }
+            }
+        }
+    }
+}
+
 // Sums the split-K slices in slice order (deterministic) and applies the epilogue.
 // One grid row (blockIdx.y) per output channel, four consecutive pixels per thread:
 // 16-byte loads of the partial sums, no 64-bit index arithmetic.
@@ -483,13 +733,51 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int group
     out[idx] = v;
 }
 
+// bf16 matrix-instruction path: packed[group][m tile][K tile][m in tile][32 channels of one tap], bf16
+__global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int groups, int cin_g, int khw, const bf16_t *__restrict__ w,
+                                                                bf16_t *__restrict__ out)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long total = (long long)groups * p.mtiles * p.nkt * p.BM * BK2;
+    if (idx >= total)
+        return;
+    const int k = (int)(idx % BK2);
+    long long r = idx / BK2;
+    const int mi = (int)(r % p.BM);
+    r /= p.BM;
+    const int kt = (int)(r % p.nkt);
+    r /= p.nkt;
+    const int mt = (int)(r % p.mtiles);
+    const int g = (int)(r / p.mtiles);
+    const int m = mt * p.BM + mi;
+    const int cb = kt / khw, tap = kt - cb * khw;
+    const int col = (cb * BK2 + k) * khw + tap;
+    bf16_t v;
+    v.bits = 0;
+    if (m < p.M)
+        v = w[((size_t)g * p.M + m) * p.K + col];
+    out[idx] = v;
+}
+
 // Split-K factor for a launch of `tiles` output tiles over `nkt` K tiles.
 // The 64x64 tile runs up to 8 workgroups per CU; measured on the ResNet shapes the
 // kernel needs on the order of 1200 workgroups in flight to keep the matrix pipes of
 // 256 CUs busy, and a split only pays when every slice still has a long K loop
 // (the partial sums cost one extra pass over the output per slice).
-int choose_splitk(long long tiles, int nkt)
+int choose_splitk(long long tiles, int nkt, int order)
 {
+    if (order == GEMM_ORDER_TAP_BF16) {
+        // large tiles, two workgroups per CU: about 512 fill the chip; K tiles are 32 deep
+        if (tiles >= 400)
+            return 1;
+        long long s = (512 + tiles / 2) / tiles;
+        const long long max_by_k = nkt / 8;
+        if (s > max_by_k)
+            s = max_by_k;
+        if (s > 16)
+            s = 16;
+        return s < 1 ? 1 : (int)s;
+    }
     if (tiles >= 1000)
         return 1;
     long long s = (1200 + tiles / 2) / tiles; // round(1200 / tiles)
@@ -507,7 +795,7 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
 {
     a.mtiles = p.mtiles;
     a.ntiles = (a.N + p.BN - 1) / p.BN;
-    int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt);
+    int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt, p.order);
     if (s > 1 && (!have_ws || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
@@ -534,6 +822,26 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     return DLP_OK;
 }
 
+template <int BM, int BN, int WM, int WN>
+int launch_bf16_mfma(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+{
+    long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
+    if (blocks > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    {
+        TimingScope ts("conv_gemm", stream);
+        hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    }
+    if (a.splitk > 1) {
+        TimingScope ts("splitk_reduce", stream);
+        if (a.Cout > 65535)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
+        hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
 template <class T, int BM, int BN, int WM, int WN>
 int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipStream_t stream)
 {
@@ -552,7 +860,7 @@ int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipS
 struct TileShape {
     int id, BM, BN;
 };
-constexpr TileShape kTiles[] = {{0, 64, 64}, {1, 32, 128}};
+constexpr TileShape kTiles[] = {{0, 64, 64}, {1, 32, 128}, {2, 128, 128}, {3, 64, 256}}; // 2, 3: bf16 matrix-instruction path
 
 int tile_choice(int M) { return M > 32 ? 0 : 1; }
 
@@ -583,6 +891,12 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
     }
     p.tile = tile_choice(p.M);
+    if (g.dtype == DLP_BFLOAT16 && !generic_act(activation) && small_kernel && cin_g % BK2 == 0) {
+        p.order = GEMM_ORDER_TAP_BF16;
+        p.mask = GEMM_MASK_TAPS;
+        p.nkt = p.K / BK2;
+        p.tile = p.M > 64 ? 2 : 3;
+    }
     p.BM = 64;
     p.BN = 64;
     for (const TileShape &ts : kTiles)
@@ -592,6 +906,8 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         }
     p.mtiles = (p.M + p.BM - 1) / p.BM;
     p.wpack_bytes = (size_t)g.groups * p.mtiles * p.nkt * BK * p.BM * sizeof(float);
+    if (p.order == GEMM_ORDER_TAP_BF16)
+        p.wpack_bytes = (size_t)g.groups * p.mtiles * p.nkt * BK2 * p.BM * sizeof(bf16_t);
     p.wpack_bytes = (p.wpack_bytes + 255) / 256 * 256;
     return p;
 }
@@ -613,12 +929,13 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
     const GemmPlan p = conv_gemm_plan(g, activation);
     const int cin_g = g.Cin / g.groups;
     const int esize = (int)dtype_size(g.dtype); // gather offsets are bytes of the storage type
-    if (p.order == GEMM_ORDER_TAP) {
+    if (p.order == GEMM_ORDER_TAP || p.order == GEMM_ORDER_TAP_BF16) {
+        const int cblock = p.order == GEMM_ORDER_TAP ? BK : BK2; // channels per K tile
         int t = 0;
-        for (int cb = 0; cb < cin_g / BK; cb++)
+        for (int cb = 0; cb < cin_g / cblock; cb++)
             for (int ky = 0; ky < g.KH; ky++)
                 for (int kx = 0; kx < g.KW; kx++, t++) {
-                    tab[4 * t + 0] = ((cb * BK * g.H + ky * g.dh) * g.W + kx * g.dw) * esize;
+                    tab[4 * t + 0] = ((cb * cblock * g.H + ky * g.dh) * g.W + kx * g.dw) * esize;
                     tab[4 * t + 1] = (int32_t)(1u << (ky * g.KW + kx));
                 }
         return;
@@ -650,11 +967,14 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
 
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream)
 {
-    const long long total = (long long)g.groups * p.mtiles * p.nkt * BK * p.BM;
+    const long long total = (long long)g.groups * p.mtiles * p.nkt * (p.order == GEMM_ORDER_TAP_BF16 ? BK2 : BK) * p.BM;
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
     TimingScope ts("pack_weights", stream);
-    if (g.dtype == DLP_BFLOAT16)
+    if (p.order == GEMM_ORDER_TAP_BF16)
+        hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
+                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked);
+    else if (g.dtype == DLP_BFLOAT16)
         hipLaunchKernelGGL(pack_weights_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
                            g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked);
     else
@@ -721,6 +1041,8 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
 
+    if (p.order == GEMM_ORDER_TAP_BF16)
+        return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, a, stream);
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)
             return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);

@@ -307,7 +307,10 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     const bool dsc = depthwise_supported(g);
     const bool auto_algo = al == "" || al == "auto";
     ConvAlgo chosen = ALGO_GEMM;
-    if ((al == "winograd" && win) || (auto_algo && win && cfg->channels_in >= 8 && cfg->channels_out >= 8))
+    // bf16 tensors whose GEMM runs on the bf16 matrix instruction are faster there than through
+    // Winograd (whose transforms force fp32 matrix instructions): automatic choice keeps gemm
+    const bool bf16_mfma = conv_gemm_plan(g, activation).order == GEMM_ORDER_TAP_BF16;
+    if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && cfg->channels_in >= 8 && cfg->channels_out >= 8))
         chosen = ALGO_WINOGRAD;
     else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))
         chosen = ALGO_DEPTHWISE;

@@ -23,6 +23,29 @@ __global__ __launch_bounds__(256) void mfma_f32_loop(float *out, int iters, floa
         out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(256) void mfma_bf16_loop(float *out, int iters, float a0, float b0)
+{
+    f32x16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    bf16x8 a, b;
+    for (int i = 0; i < 8; i++) {
+        a[i] = (__bf16)(a0 + threadIdx.x + i);
+        b[i] = (__bf16)(b0 + i);
+    }
+    for (int i = 0; i < iters; i++) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+    }
+    float s = 0;
+    for (int r = 0; r < 16; r++)
+        s += c0[r] + c1[r] + c2[r] + c3[r];
+    if (s == 12345.678f)
+        out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 __global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n)
 {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -63,6 +86,33 @@ int dlp_probe_mfma_f32(int waves_per_simd, double *tflops)
     (void)hipEventRecord(e1, 0);
     float ms = time_ms(0, e0, e1);
     double flops = (double)blocks * 4 /*waves*/ * iters * 4 /*mfma*/ * 4096.0;
+    *tflops = flops / (ms * 1e-3) / 1e12;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// bf16 MFMA (32x32x16, fp32 accumulate) throughput in TFLOP/s.
+int dlp_probe_mfma_bf16(int waves_per_simd, double *tflops)
+{
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess)
+        return 1;
+    const int blocks = prop.multiProcessorCount * waves_per_simd;
+    const int iters = 40000;
+    float *out = nullptr;
+    if (hipMalloc(&out, (size_t)blocks * 256 * 4) != hipSuccess)
+        return 1;
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    mfma_bf16_loop<<<blocks, 256>>>(out, 1000, 1.0f, 2.0f);
+    (void)hipEventRecord(e0, 0);
+    mfma_bf16_loop<<<blocks, 256>>>(out, iters, 1.0f, 2.0f);
+    (void)hipEventRecord(e1, 0);
+    float ms = time_ms(0, e0, e1);
+    double flops = (double)blocks * 4 * iters * 4 * (2.0 * 32 * 32 * 16);
     *tflops = flops / (ms * 1e-3) / 1e12;
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);

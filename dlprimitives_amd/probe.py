@@ -24,6 +24,10 @@ def main():
             if lib.dlp_probe_mfma_f32(waves, ctypes.byref(v)) != 0:
                 raise SystemExit("MFMA probe failed")
             out["mfma_f32_tflops_%dwave_per_simd" % waves] = round(v.value, 1)
+        for waves in (1, 2):
+            if lib.dlp_probe_mfma_bf16(waves, ctypes.byref(v)) != 0:
+                raise SystemExit("bf16 MFMA probe failed")
+            out["mfma_bf16_tflops_%dwave_per_simd" % waves] = round(v.value, 1)
     if lib.dlp_probe_copy(args.copy_mb, ctypes.byref(v)) != 0:
         raise SystemExit("copy probe failed")
     out["copy_gbs_read_plus_write"] = round(v.value, 1)

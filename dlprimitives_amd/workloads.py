@@ -30,6 +30,28 @@ def _resnet18():
 
 RESNET18_CONVS = _resnet18()
 
+
+
+def _resnet50():
+    """The 53 convolutions of ResNet-50 (torchvision v1.5 layout: stride on the 3x3), in graph order."""
+    layers = [conv("conv1_7x7s2_3to64_at224", 7, 2, 3, 3, 64, 224)]
+    cin, hw = 64, 56
+    for stage, (mid, blocks) in enumerate(((64, 3), (128, 4), (256, 6), (512, 3)), start=1):
+        for b in range(blocks):
+            s = 2 if (b == 0 and stage > 1) else 1
+            pre = "l%d_%d" % (stage, b)
+            layers.append(conv("%s_1x1_%dto%d_at%d" % (pre, cin, mid, hw), 1, 1, 0, cin, mid, hw))
+            layers.append(conv("%s_3x3%s_%dto%d_at%d" % (pre, "s2" if s == 2 else "", mid, mid, hw), 3, s, 1, mid, mid, hw))
+            layers.append(conv("%s_1x1_%dto%d_at%d" % (pre, mid, 4 * mid, hw // s), 1, 1, 0, mid, 4 * mid, hw // s, activation="identity"))
+            if b == 0:
+                layers.append(conv("%s_ds_1x1%s_%dto%d_at%d" % (pre, "s2" if s == 2 else "", cin, 4 * mid, hw), 1, s, 0, cin, 4 * mid, hw,
+                                   activation="identity"))
+            cin, hw = 4 * mid, hw // s
+    return layers
+
+
+RESNET50_CONVS = _resnet50()
+
 # MobileNet-v2 style depthwise 3x3 shapes (C, HW), each at stride 1 and 2, and 1x1 followers
 MOBILENET_DEPTHWISE = [(144, 56), (192, 28), (384, 14), (960, 7)]
 MOBILENET_POINTWISE = [(144, 24, 56), (144, 32, 28), (192, 32, 28), (192, 64, 14), (384, 64, 14), (384, 96, 14), (960, 160, 7),

@@ -40,6 +40,16 @@ CASES = [
     (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),      # split-K path
     (case((3, 5), (1, 2), (2, 3), (3, 2), 3, 8, False, 1, False), (2, 19, 19)),
     (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise geometry, served by gemm
+    # bf16 matrix instruction, pixel-pair loader ("same" stride-1 convolutions with Cin/groups % 32 == 0)
+    (case(1, 0, 1, 1, 64, 256, True, 1, True), (5, 7, 7)),       # odd pixel count per image: padded column numbering
+    (case(1, 0, 1, 1, 2048, 512, True, 1, True), (3, 7, 7)),     # long K, split over workgroups
+    (case(3, 2, 1, 2, 64, 64, True, 1, True), (2, 13, 13)),      # dilated, odd width
+    (case(3, 1, 1, 1, 64, 96, False, 2, True), (3, 9, 12)),      # two groups, Cout off the tile sizes
+    (case(5, 2, 1, 1, 32, 48, True, 1, False), (2, 9, 9)),       # 25 taps
+    (case((3, 1), (1, 0), 1, 1, 32, 32, True, 1, False), (1, 1, 1)),  # a single pixel: both ends of the tensor in one pair
+    # per-pixel loader (strided or size-changing)
+    (case(3, 0, 1, 1, 32, 64, True, 1, True), (2, 12, 12)),
+    (case(3, 1, 2, 1, 256, 256, True, 1, True), (2, 28, 28)),
 ]
 
 
