@@ -65,6 +65,8 @@ struct GemmArgs {
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
+    uint32_t y_bytes; // size of y when it is below 2 GiB (buffer stores), else 0
+    uint32_t part_bytes; // likewise for the split-K partial sums
     uint32_t x_shift; // bytes by which the X resource base is moved back (padding offset)
     uint32_t hw4;     // H*W*sizeof(T): byte stride between input channels
     uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
@@ -356,6 +358,25 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 
     // ---- split-K: raw partial sums to the workspace, reduced by a second kernel ----
     if (a.splitk > 1) {
+        if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
+            const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + wn * WTN + j * 32 + l32;
+                const uint32_t voff =
+                    n < a.N ? (uint32_t)((slice * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.N + n) * 4u : kOutOfRange;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int mrow = i * 32 + 8 * (r >> 2) + (r & 3);
+                        const float v = acc[i][j][r]; // a copy: bit_cast of a vector element reads element 0
+                        if (m0 + wm * WTM + mrow < a.M)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, voff, (uint32_t)(mrow * a.N) * 4u, 0);
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int n = n0 + wn * WTN + j * 32 + l32;
@@ -376,6 +397,50 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     }
 
     // ---- epilogue: bias, activation, factor, NCHW store ----
+    // Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the tile's rows goes
+    // through LDS (free after the last barrier) and the stores are buffer stores whose row offset
+    // is scalar, instead of a bias load and 64-bit address arithmetic per value.
+    if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
+        float *bias_s = &As[0][0][0];
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+            const int pix = n - b * a.OHW;
+            const uint32_t voff =
+                n < a.N ? (uint32_t)(((b * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.OHW + pix) * (int)sizeof(T)) : kOutOfRange;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int mrow = wm * WTM + i * 32 + 8 * rq; // + 4*h + (r & 3); this part is uniform
+                    if (m0 + mrow >= a.M)
+                        continue;
+                    const f32x4 bv = *(const f32x4 *)&bias_s[mrow + 4 * h];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp) // identity must keep NaNs: no min/max
+                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                        } else
+                            v = apply_act(v, a.act);
+                        const uint32_t soff = (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * (int)sizeof(T));
+                        if (sizeof(T) == 4)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
+                        else
+                            __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, soff, 0);
+                    }
+                }
+            }
+        }
+        return;
+    }
     // accumulator register r of a 32x32 block holds row 8*(r/4) + 4*h + r%4, column l32
 #pragma unroll
     for (int j = 0; j < TN; j++) {
@@ -608,6 +673,25 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         k_step(I0{}, I1{}, I0{}, kt);
 
     if (a.splitk > 1) {
+        if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
+            const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + wn * WTN + j * 32 + l32;
+                const uint32_t voff =
+                    n < a.N ? (uint32_t)((slice * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.N + n) * 4u : kOutOfRange;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int mrow = i * 32 + 8 * (r >> 2) + (r & 3);
+                        const float v = acc[i][j][r]; // a copy: bit_cast of a vector element reads element 0
+                        if (m0 + wm * WTM + mrow < a.M)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, voff, (uint32_t)(mrow * a.N) * 4u, 0);
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int n = n0 + wn * WTN + j * 32 + l32;
@@ -627,6 +711,46 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         return;
     }
 
+    // ---- epilogue.  Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the
+    // tile's rows goes through LDS (free after the last barrier), the result is rounded by the
+    // hardware conversion and stored with buffer stores whose row offset is scalar: a handful of
+    // VALU operations per value instead of 64-bit address arithmetic and a bias load each. ----
+    if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
+        float *bias_s = (float *)&As[0][0][0];
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+            const int pix = n - b * a.OHW;
+            const uint32_t voff = n < a.N ? (uint32_t)(((b * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.OHW + pix) * 2) : kOutOfRange;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int mrow = wm * WTM + i * 32 + 8 * rq; // + 4*h + (r & 3); uniform part
+                    if (m0 + mrow >= a.M)
+                        continue;
+                    const f32x4 bv = *(const f32x4 *)&bias_s[mrow + 4 * h];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp)
+                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                        } else
+                            v = apply_act(v, a.act);
+                        __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * 2), 0);
+                    }
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int n = n0 + wn * WTN + j * 32 + l32;
@@ -1026,6 +1150,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     a.KH = g.KH; a.KW = g.KW;
     a.x_bytes = (uint32_t)(x_elems * esize);
     a.wp_bytes = (uint32_t)p.wpack_bytes;
+    a.y_bytes = y_elems * esize < kOutOfRange ? (uint32_t)(y_elems * esize) : 0;
     a.x_shift = (uint32_t)x_shift;
     a.hw4 = (uint32_t)(g.H * g.W * esize);
     make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
@@ -1040,6 +1165,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         a.clamp_hi = 6.0f;
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
+    {
+        const size_t used = (size_t)a.splitk * a.Cout * a.N * sizeof(float);
+        a.part_bytes = (a.splitk > 1 && used < kOutOfRange) ? (uint32_t)used : 0;
+    }
 
     if (p.order == GEMM_ORDER_TAP_BF16)
         return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, a, stream);

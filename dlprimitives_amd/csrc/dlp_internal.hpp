@@ -89,14 +89,9 @@ __device__ __forceinline__ float to_float(bf16_t v) { return __builtin_bit_cast(
 
 __device__ __forceinline__ bf16_t to_bf16(float f)
 {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    // one v_cvt_pk_bf16_f32 on gfx950: round to nearest even, NaN stays NaN
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { // NaN stays NaN
-        r.bits = (uint16_t)((u >> 16) | 0x40u);
-        return r;
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (uint16_t)(u >> 16);
+    r.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
     return r;
 }
 
