@@ -490,7 +490,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int BK2 = 32;
 constexpr int LDK = BK2 + 8;
 
-template <int BM, int BN, int WM, int WN, int ACT>
+template <int BM, int BN, int WM, int WN, int ORDER, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -541,7 +541,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     const int p = tid % BN;
     const int ks = (KSPLIT == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid / BN);
     uint32_t vbase;
-    uint32_t my = 0;
+    uint32_t my = 0, mx = 0; // tap-major: my = tap mask; channel-major: row / column masks
     {
         const int n = n0 + p;
         const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
@@ -563,9 +563,14 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
                 if (xx >= 0 && xx < a.W)
                     rx |= 1u << kx;
             }
-            for (int ky = 0; ky < a.KH; ky++)
-                if ((ry >> ky) & 1u)
-                    my |= rx << (ky * a.KW);
+            if (ORDER == GEMM_ORDER_TAP_BF16) {
+                for (int ky = 0; ky < a.KH; ky++)
+                    if ((ry >> ky) & 1u)
+                        my |= rx << (ky * a.KW);
+            } else {
+                my = ry;
+                mx = rx;
+            }
         }
     }
 
@@ -585,13 +590,26 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             for (int j = 0; j < A_LD; j++)
                 ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
         }
-        ConstInt *e = ktab + kt * 4;
-        const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
-        if (Q == 0)
-            vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
+        if (ORDER == GEMM_ORDER_TAP_BF16) {
+            // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
+            ConstInt *e = ktab + kt * 4;
+            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
+            if (Q == 0)
+                vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
 #pragma unroll
-        for (int i = Q * (B_LD / 2); i < (Q + 1) * (B_LD / 2); i++)
-            rb[S][i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4, 0);
+            for (int i = Q * (B_LD / 2); i < (Q + 1) * (B_LD / 2); i++)
+                rb[S][i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4, 0);
+        } else {
+            // channel-major (Cin/groups not a multiple of 32, e.g. the 3-channel stem): one table
+            // entry per k = {x byte offset of (c, ky, kx), ky | kx << 8}
+            ConstInt *e = ktab + (kt * BK2 + ks * B_LD) * 2;
+#pragma unroll
+            for (int i = Q * (B_LD / 2); i < (Q + 1) * (B_LD / 2); i++) {
+                const uint32_t xoff = (uint32_t)e[2 * i], tap = (uint32_t)e[2 * i + 1];
+                const bool ok = ((my >> (tap & 0xff)) & (mx >> (tap >> 8)) & 1u) != 0;
+                rb[S][i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(xr, opaque(ok ? vbase : kOutOfRange), xoff, 0);
+            }
+        }
     };
     auto store_half = [&](auto set, auto buf_c, auto half_c) {
         constexpr int S = decltype(set)::value;
@@ -874,14 +892,21 @@ __global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int 
     const int mt = (int)(r % p.mtiles);
     const int g = (int)(r / p.mtiles);
     const int m = mt * p.BM + mi;
-    const int cb = kt / khw, tap = kt - cb * khw;
-    const int col = (cb * BK2 + k) * khw + tap;
+    int col;
+    if (p.order == GEMM_ORDER_TAP_BF16) {
+        const int cb = kt / khw, tap = kt - cb * khw;
+        col = (cb * BK2 + k) * khw + tap;
+    } else {
+        col = kt * BK2 + k;
+    }
     bf16_t v;
     v.bits = 0;
-    if (m < p.M)
+    if (m < p.M && col < p.K)
         v = w[((size_t)g * p.M + m) * p.K + col];
     out[idx] = v;
 }
+
+bool bf16_mfma_order(int order) { return order == GEMM_ORDER_TAP_BF16 || order == GEMM_ORDER_CHANNEL_BF16; }
 
 // Split-K factor for a launch of `tiles` output tiles over `nkt` K tiles.
 // The 64x64 tile runs up to 8 workgroups per CU; measured on the ResNet shapes the
@@ -890,7 +915,7 @@ __global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int 
 // (the partial sums cost one extra pass over the output per slice).
 int choose_splitk(long long tiles, int nkt, int order)
 {
-    if (order == GEMM_ORDER_TAP_BF16) {
+    if (bf16_mfma_order(order)) {
         // large tiles, two workgroups per CU: about 512 fill the chip; K tiles are 32 deep
         if (tiles >= 400)
             return 1;
@@ -947,14 +972,19 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 }
 
 template <int BM, int BN, int WM, int WN>
-int launch_bf16_mfma(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+int launch_bf16_mfma(const ConvGeom &g, int order, GemmArgs &a, hipStream_t stream)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     {
         TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        if (order == GEMM_ORDER_TAP_BF16)
+            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                               stream, a);
+        else
+            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP>), dim3((unsigned)blocks),
+                               dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
@@ -1015,10 +1045,11 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
     }
     p.tile = tile_choice(p.M);
-    if (g.dtype == DLP_BFLOAT16 && !generic_act(activation) && small_kernel && cin_g % BK2 == 0) {
-        p.order = GEMM_ORDER_TAP_BF16;
-        p.mask = GEMM_MASK_TAPS;
-        p.nkt = p.K / BK2;
+    if (g.dtype == DLP_BFLOAT16 && !generic_act(activation)) { // bf16 matrix instruction
+        const bool tap_major = small_kernel && cin_g % BK2 == 0;
+        p.order = tap_major ? GEMM_ORDER_TAP_BF16 : GEMM_ORDER_CHANNEL_BF16;
+        p.mask = tap_major ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
+        p.nkt = (p.K + BK2 - 1) / BK2;
         p.tile = p.M > 64 ? 2 : 3;
     }
     p.BM = 64;
@@ -1030,7 +1061,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         }
     p.mtiles = (p.M + p.BM - 1) / p.BM;
     p.wpack_bytes = (size_t)g.groups * p.mtiles * p.nkt * BK * p.BM * sizeof(float);
-    if (p.order == GEMM_ORDER_TAP_BF16)
+    if (bf16_mfma_order(p.order))
         p.wpack_bytes = (size_t)g.groups * p.mtiles * p.nkt * BK2 * p.BM * sizeof(bf16_t);
     p.wpack_bytes = (p.wpack_bytes + 255) / 256 * 256;
     return p;
@@ -1041,7 +1072,7 @@ size_t conv_gemm_ktab_entries(const ConvGeom &g)
     // one 8-byte entry per k (the tap-major order uses two entries per K tile); two spare
     // tiles of never-valid entries are what the software pipeline fetches past the end
     const int K = (g.Cin / g.groups) * g.KH * g.KW;
-    return (size_t)((K + BK - 1) / BK + 2) * BK;
+    return (size_t)((K + BK2 - 1) / BK2 + 2) * BK2; // whole K tiles of the widest kernel (32)
 }
 
 void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entries)
@@ -1091,11 +1122,11 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
 
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream)
 {
-    const long long total = (long long)g.groups * p.mtiles * p.nkt * (p.order == GEMM_ORDER_TAP_BF16 ? BK2 : BK) * p.BM;
+    const long long total = (long long)g.groups * p.mtiles * p.nkt * (bf16_mfma_order(p.order) ? BK2 : BK) * p.BM;
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
     TimingScope ts("pack_weights", stream);
-    if (p.order == GEMM_ORDER_TAP_BF16)
+    if (bf16_mfma_order(p.order))
         hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
                            g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked);
     else if (g.dtype == DLP_BFLOAT16)
@@ -1170,8 +1201,8 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         a.part_bytes = (a.splitk > 1 && used < kOutOfRange) ? (uint32_t)used : 0;
     }
 
-    if (p.order == GEMM_ORDER_TAP_BF16)
-        return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, a, stream);
+    if (bf16_mfma_order(p.order))
+        return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, p.order, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, p.order, a, stream);
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)
             return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);

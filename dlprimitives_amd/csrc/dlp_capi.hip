@@ -309,7 +309,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     ConvAlgo chosen = ALGO_GEMM;
     // bf16 tensors whose GEMM runs on the bf16 matrix instruction are faster there than through
     // Winograd (whose transforms force fp32 matrix instructions): automatic choice keeps gemm
-    const bool bf16_mfma = conv_gemm_plan(g, activation).order == GEMM_ORDER_TAP_BF16;
+    const bool bf16_mfma = conv_gemm_plan(g, activation).order >= GEMM_ORDER_TAP_BF16;
     if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && cfg->channels_in >= 8 && cfg->channels_out >= 8))
         chosen = ALGO_WINOGRAD;
     else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))

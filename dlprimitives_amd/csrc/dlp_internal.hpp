@@ -140,8 +140,9 @@ struct KTabEntry {
 };
 
 // K ordering: k = (c,ky,kx) with a per-element table, or one tap x 16 channels per K tile
-// (GEMM_ORDER_TAP_BF16: one tap x 32 channels per K tile, bf16 operands on the bf16 matrix instruction)
-enum { GEMM_ORDER_CHANNEL = 0, GEMM_ORDER_TAP = 1, GEMM_ORDER_TAP_BF16 = 2 };
+// (the _BF16 orders feed bf16 operands to the bf16 matrix instruction, K tiles of 32: one tap x 32
+// channels, or 32 consecutive k = (c,ky,kx) with the per-element table)
+enum { GEMM_ORDER_CHANNEL = 0, GEMM_ORDER_TAP = 1, GEMM_ORDER_TAP_BF16 = 2, GEMM_ORDER_CHANNEL_BF16 = 3 };
 // In-image test: one bit per tap (KH*KW <= 32) or separate row / column masks
 enum { GEMM_MASK_TAPS = 1, GEMM_MASK_ROWCOL = 2 };
 

@@ -170,3 +170,24 @@ def test_gpu_eltwise(oracle_mod):
             dlp.eltwise_forward(_dev(a), _dev(b), c, op, c1, c2, act)
             torch.cuda.synchronize()
             np.testing.assert_allclose(c.cpu().numpy(), oracle_mod.eltwise_forward(a, b, op, c1, c2, act), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_eltwise_alignments_and_tails(oracle_mod, dtype):
+    """The 16-byte vector body, its scalar tail, and operands that are not 16-byte aligned."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(5)
+    for n, off in [(4099, 0), (4099, 1), (37, 3), (8 * 1024, 0), (5, 0)]:
+        a = oracle_mod.bf16_round(rng.standard_normal(n + off).astype(np.float32))
+        b = oracle_mod.bf16_round(rng.standard_normal(n + off).astype(np.float32))
+        ta, tb = _dev(a).to(tdt)[off:], _dev(b).to(tdt)[off:]
+        c = torch.full((n + off,), float("nan"), device="cuda:0", dtype=tdt)[off:]
+        dlp.eltwise_forward(ta, tb, c, "sum", 1.0, 1.0, "relu")
+        torch.cuda.synchronize()
+        want = oracle_mod.eltwise_forward(a[off:], b[off:], "sum", 1.0, 1.0, "relu")
+        np.testing.assert_allclose(c.float().cpu().numpy(), want, rtol=2 ** -8 if dtype == "bfloat16" else 1e-6, atol=1e-6)
