@@ -106,7 +106,7 @@ def kernel_class(L, bf16=False):
     m = L["cout"] // L["groups"]
     if L["algo"] == "winograd":
         return "wino_fused_kernel<%s, ...>" % ("bf16_t" if bf16 else "float")
-    small = L["kernel"] ** 2 <= 32
+    small = L["kernel"] ** 2 <= 31
     if bf16 and L["activation"] not in ("tanh", "sigmoid"):
         order = 2 if (small and cin_g % 32 == 0) else 3  # one tap x 32 channels per K tile, or the per-element table
         return "conv_gemm_bf16_kernel<%s, %d, 0>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4", order)

@@ -140,7 +140,10 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
     constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA blocks per wavefront
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "tile shape");
-    constexpr int LDA = BM + 4; // rows stay 16-byte aligned for the b128 stores
+    // Unpadded rows: two k steps are then a multiple of 256 bytes apart, so every operand fetch is a
+    // ds_read2st64 with immediate offsets (a padded row cost one VALU address add per pair of
+    // fetches; the two half-waves of a fetch read different rows in different cycles: no conflicts)
+    constexpr int LDA = BM;
     constexpr int LDB = BN;
     constexpr int KSPLIT = kThreads / BN;    // k slices among the B loader threads
     static_assert(KSPLIT >= 1 && BN % 64 == 0 && BK % KSPLIT == 0, "B loader shape");
@@ -253,9 +256,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         if (ORDER == GEMM_ORDER_TAP) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
-            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
-            if (Q == 0)
-                vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
+            const uint32_t xoff = (uint32_t)e[0], tap = (uint32_t)e[1];
+            if (Q == 0) {
+                // bit `tap` of the pixel's tap mask, spread over a word, picks the offset (two VALU operations)
+                const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)my, tap, 1u);
+                vsel[S] = opaque((vbase & m) | (kOutOfRange & ~m));
+            }
 #pragma unroll
             for (int i = 0; i < B_LD; i++)
                 if (i % (BK / 2) == Q)
@@ -593,9 +599,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         if (ORDER == GEMM_ORDER_TAP_BF16) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
-            const uint32_t xoff = (uint32_t)e[0], tapbit = (uint32_t)e[1];
-            if (Q == 0)
-                vsel[S] = opaque((my & tapbit) ? vbase : kOutOfRange);
+            const uint32_t xoff = (uint32_t)e[0], tap = (uint32_t)e[1];
+            if (Q == 0) {
+                // bit `tap` of the pixel's tap mask, spread over a word, picks the offset (two VALU operations)
+                const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)my, tap, 1u);
+                vsel[S] = opaque((vbase & m) | (kOutOfRange & ~m));
+            }
 #pragma unroll
             for (int i = Q * (B_LD / 2); i < (Q + 1) * (B_LD / 2); i++)
                 rb[S][i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4, 0);
@@ -1036,7 +1045,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
     p.M = g.Cout / g.groups;
     p.K = cin_g * g.KH * g.KW;
     p.nkt = (p.K + BK - 1) / BK; // the tap-major order has the same count: K is a multiple of 16 there
-    const bool small_kernel = g.KH * g.KW <= 32;
+    const bool small_kernel = g.KH * g.KW <= 31; // one mask bit per tap, bit 31 kept free for the never-valid spare tiles
     if (generic_act(activation)) { // the rare activations share one instantiation per tile
         p.order = GEMM_ORDER_CHANNEL;
         p.mask = GEMM_MASK_ROWCOL;
@@ -1080,7 +1089,7 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
     int32_t *tab = (int32_t *)tab_entries;
     const size_t words = conv_gemm_ktab_entries(g) * 2;
     for (size_t i = 0; i < words; i++)
-        tab[i] = 0; // spare entries: no tap bit (row/col code 31 below), offsets 0
+        tab[i] = 0; // spare entries: offsets 0, never-valid tap (tap 31 / row-col code 31 below)
     const GemmPlan p = conv_gemm_plan(g, activation);
     const int cin_g = g.Cin / g.groups;
     const int esize = (int)dtype_size(g.dtype); // gather offsets are bytes of the storage type
@@ -1091,8 +1100,10 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
             for (int ky = 0; ky < g.KH; ky++)
                 for (int kx = 0; kx < g.KW; kx++, t++) {
                     tab[4 * t + 0] = ((cb * cblock * g.H + ky * g.dh) * g.W + kx * g.dw) * esize;
-                    tab[4 * t + 1] = (int32_t)(1u << (ky * g.KW + kx));
+                    tab[4 * t + 1] = ky * g.KW + kx; // tap number = its bit in the per-pixel tap mask
                 }
+        for (; (size_t)(4 * t + 1) < words; t++)
+            tab[4 * t + 1] = 31; // bit 31 of a tap mask is never set (at most 31 taps use this order)
         return;
     }
     size_t k = 0;
