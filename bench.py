@@ -101,7 +101,7 @@ def build_layers(layer_list, batch, seed, bf16=False):
 def kernel_class(L, bf16=False):
     """Name of the kernel that does the layer's arithmetic, as a profiler lists it."""
     if L["algo"] == "depthwise_separable":
-        return "depthwise3x3_kernel<%d>" % L["stride"]
+        return "depthwise3x3_kernel<%s, %d>" % ("bf16_t" if bf16 else "float", L["stride"])
     cin_g = L["cin"] // L["groups"]
     m = L["cout"] // L["groups"]
     if L["algo"] == "winograd":

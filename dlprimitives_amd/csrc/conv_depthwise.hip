@@ -31,10 +31,10 @@ namespace {
 constexpr int kStripRows = 7; // divides the usual 56/28/14/7 feature maps
 
 struct DwArgs {
-    const float *x;
-    const float *w;
+    const void *x; // storage type T (float or bf16_t); arithmetic is fp32
+    const void *w;
     const float *bias;
-    float *y;
+    void *y;
     int planes; // B*C
     int C, H, W, OH, OW;
     int nstrips;          // ceil(OH / kStripRows)
@@ -45,7 +45,7 @@ struct DwArgs {
 
 // STRIDE 1: halo lanes 0 and 63 (62 outputs per wavefront)
 // STRIDE 2: halo lane 0 only (63 outputs per wavefront)
-template <int STRIDE>
+template <class T, int STRIDE>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
 {
     constexpr int OUT_PER_WAVE = (STRIDE == 1) ? 62 : 63;
@@ -65,11 +65,11 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
     float k[9];
 #pragma unroll
     for (int i = 0; i < 9; i++)
-        k[i] = a.w[c * 9 + i];
+        k[i] = to_float(((const T *)a.w)[c * 9 + i]);
     const float bias = a.bias ? a.bias[c] : 0.0f;
 
-    const float *xp = a.x + (size_t)plane * a.H * a.W;
-    float *yp = a.y + (size_t)plane * a.OH * a.OW + ox;
+    const T *xp = (const T *)a.x + (size_t)plane * a.H * a.W;
+    T *yp = (T *)a.y + (size_t)plane * a.OH * a.OW + ox;
 
     // columns owned by this lane
     const int x0 = ox * STRIDE;
@@ -84,11 +84,11 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
     for (int r = 0; r < NIN; r++) {
         const int yy = iy0 + r;
         const bool vy = in_range && yy >= 0 && yy < a.H;
-        const float *p = xp + (size_t)(vy ? yy : 0) * a.W + x0;
-        c0[r] = vy ? p[0] : 0.0f;
+        const T *p = xp + (size_t)(vy ? yy : 0) * a.W + x0;
+        c0[r] = vy ? to_float(p[0]) : 0.0f;
         c1[r] = 0.0f;
         if (STRIDE == 2)
-            c1[r] = (vy && v1) ? p[1] : 0.0f;
+            c1[r] = (vy && v1) ? to_float(p[1]) : 0.0f;
     }
     // window columns (x0-1, x0, x0+1) of every row
     float left[NIN], right[NIN];
@@ -122,6 +122,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
 }
 
 // Any odd kernel size, stride 1 or 2, pad = K/2: one output per thread.
+template <class T>
 __global__ __launch_bounds__(256) void depthwise_direct_kernel(DwArgs a, int K, int stride)
 {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -134,25 +135,25 @@ __global__ __launch_bounds__(256) void depthwise_direct_kernel(DwArgs a, int K, 
     const int plane = (int)(t / a.OH);
     const int c = plane % a.C;
     const int pad = K / 2;
-    const float *xp = a.x + (size_t)plane * a.H * a.W;
-    const float *kp = a.w + (size_t)c * K * K;
+    const T *xp = (const T *)a.x + (size_t)plane * a.H * a.W;
+    const T *kp = (const T *)a.w + (size_t)c * K * K;
     float sum = a.bias ? a.bias[c] : 0.0f;
     for (int dr = 0; dr < K; dr++) {
         const int yy = oy * stride - pad + dr;
         for (int dc = 0; dc < K; dc++) {
             const int xx = ox * stride - pad + dc;
-            const float v = (yy >= 0 && yy < a.H && xx >= 0 && xx < a.W) ? xp[(size_t)yy * a.W + xx] : 0.0f;
-            sum = fmaf(kp[dr * K + dc], v, sum);
+            const float v = (yy >= 0 && yy < a.H && xx >= 0 && xx < a.W) ? to_float(xp[(size_t)yy * a.W + xx]) : 0.0f;
+            sum = fmaf(to_float(kp[dr * K + dc]), v, sum);
         }
     }
-    store_out(a.y + idx, apply_act(sum, a.act), a.factor);
+    store_out((T *)a.y + idx, apply_act(sum, a.act), a.factor);
 }
 
 } // namespace
 
 bool depthwise_supported(const ConvGeom &g)
 {
-    return g.dtype == DLP_FLOAT && g.groups == g.Cin && g.Cout == g.Cin && g.Cin > 1 && g.KH == g.KW && g.KH % 2 == 1 &&
+    return (g.dtype == DLP_FLOAT || g.dtype == DLP_BFLOAT16) && g.groups == g.Cin && g.Cout == g.Cin && g.Cin > 1 && g.KH == g.KW && g.KH % 2 == 1 &&
            g.ph == g.KH / 2 && g.pw == g.KW / 2 && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2);
 }
 
@@ -162,10 +163,11 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     if (g.B == 0)
         return DLP_OK;
     DwArgs a;
-    a.x = (const float *)x;
-    a.w = (const float *)w;
+    a.x = x;
+    a.w = w;
     a.bias = ep.bias;
-    a.y = (float *)y;
+    a.y = y;
+    const bool bf16 = g.dtype == DLP_BFLOAT16;
     a.planes = g.B * g.Cin;
     a.C = g.Cin;
     a.H = g.H;
@@ -183,16 +185,23 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         const long long blocks = (waves + 3) / 4;
         if (blocks > 0x7fffffffLL)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
-        if (g.sh == 1)
-            hipLaunchKernelGGL(depthwise3x3_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        if (g.sh == 1 && !bf16)
+            hipLaunchKernelGGL((depthwise3x3_kernel<float, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        else if (g.sh == 1)
+            hipLaunchKernelGGL((depthwise3x3_kernel<bf16_t, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        else if (!bf16)
+            hipLaunchKernelGGL((depthwise3x3_kernel<float, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         else
-            hipLaunchKernelGGL(depthwise3x3_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL((depthwise3x3_kernel<bf16_t, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
     } else {
         const long long total = (long long)a.planes * g.OH * g.OW;
         const long long blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffLL)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
-        hipLaunchKernelGGL(depthwise_direct_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
+        if (bf16)
+            hipLaunchKernelGGL(depthwise_direct_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
+        else
+            hipLaunchKernelGGL(depthwise_direct_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;

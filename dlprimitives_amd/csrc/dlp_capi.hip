@@ -290,7 +290,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     DLP_REQUIRE(valid_activation(activation), "unknown activation");
     // The reference checks dtype == float_data (src/gemm.cpp:593).  Here bfloat16_data is
     // also accepted: x, w, y are stored as bf16, bias stays fp32, all arithmetic is fp32
-    // (the implicit-GEMM and Winograd algorithms serve it; depthwise requests fall back to gemm).
+    // (all three algorithms serve it).
     if (cfg->dtype != DLP_FLOAT && cfg->dtype != DLP_BFLOAT16)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "Conv2DForward: float_data and bfloat16_data are implemented");
     std::string al = algo ? algo : "";

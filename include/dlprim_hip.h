@@ -166,9 +166,11 @@ int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float c
  * src/gemm.cpp:577,593).  DLP_BFLOAT16 (an extension): x, w, y of Conv2DForward and
  * IPForward and the tensors of the glue operators are stored as bfloat16; bias stays
  * fp32; products are accumulated in fp32 on the matrix cores and the epilogue runs in
- * fp32 before one round-to-nearest-even conversion of the result ("gemm" and "winograd";
- * the Winograd transforms also run in fp32).  The "depthwise_separable" algorithm serves
- * DLP_FLOAT only; a DLP_BFLOAT16 request for it runs as "gemm". */
+ * fp32 before one round-to-nearest-even conversion of the result.  All three algorithms
+ * serve it: "gemm" multiplies bf16 operands on the bf16 matrix instruction (products of bf16
+ * values are exact in fp32), "winograd" transforms in fp32 and multiplies on the fp32 matrix
+ * instruction, "depthwise_separable" computes in fp32.  With algo "" / "auto" a bf16
+ * convolution runs "gemm" where the reference rule would pick "winograd". */
 
 #ifdef __cplusplus
 }

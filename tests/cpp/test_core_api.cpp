@@ -7,6 +7,7 @@
 //   test_core_api <dev>  : the device checks on HIP device <dev> (default 0)
 #include <dlprim/core/conv.hpp>
 #include <dlprim/core/ip.hpp>
+#include <dlprim/core/pool.hpp>
 
 #include <cmath>
 #include <cstdio>
@@ -167,6 +168,57 @@ static void ip_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int in, in
     EXPECT(worst < 1e-4);
 }
 
+// Pooling2DForward the way src/ops/pooling.cpp:250-279 drives it: max 3x3 stride 2 pad 1 and global average
+static void pool_case(dp::Context &ctx, dp::ExecutionContext &q)
+{
+    const int B = 2, C = 5, H = 9, W = 11;
+    int k[2] = {3, 3}, p[2] = {1, 1}, s[2] = {2, 2};
+    const int OH = dp::core::calc_pooling_output_size(H, 3, 1, 2, false), OW = dp::core::calc_pooling_output_size(W, 3, 1, 2, false);
+    EXPECT(OH == 5 && OW == 6);
+    EXPECT(dp::core::calc_pooling_output_size(7, 3, 1, 3, true) == 3 && dp::core::calc_pooling_output_size(5, 2, 0, 2, true) == 3);
+    std::mt19937 rng(7);
+    dp::Tensor X(ctx, dp::Shape(B, C, H, W)), Y(ctx, dp::Shape(B, C, OH, OW)), G(ctx, dp::Shape(B, C, 1, 1));
+    fill(X, rng, -1, 1);
+    X.to_device(q);
+    auto mp = dp::core::Pooling2DForward::create_max_pooling(ctx, k, p, s);
+    auto gp = dp::core::Pooling2DForward::create_global_avg_pooling(ctx, X.shape());
+    EXPECT(mp->workspace() == 0);
+    mp->enqueue(X, Y, q);
+    gp->enqueue(X, G, q);
+    Y.to_host(q);
+    G.to_host(q);
+    q.finish();
+    double worst = 0;
+    for (int bc = 0; bc < B * C; bc++) {
+        const float *x = X.data<float>() + size_t(bc) * H * W;
+        double sum = 0;
+        for (int i = 0; i < H * W; i++)
+            sum += x[i];
+        worst = std::fmax(worst, std::fabs(sum / (H * W) - G.data<float>()[bc]));
+        for (int oy = 0; oy < OH; oy++)
+            for (int ox = 0; ox < OW; ox++) {
+                float m = -INFINITY;
+                for (int dy = 0; dy < 3; dy++)
+                    for (int dx = 0; dx < 3; dx++) {
+                        int yy = oy * 2 - 1 + dy, xx = ox * 2 - 1 + dx;
+                        if (yy >= 0 && yy < H && xx >= 0 && xx < W)
+                            m = std::fmax(m, x[yy * W + xx]);
+                    }
+                worst = std::fmax(worst, std::fabs(double(m) - Y.data<float>()[(size_t(bc) * OH + oy) * OW + ox]));
+            }
+    }
+    std::printf("pooling max 3x3/2 + global avg : max err %.2e\n", worst);
+    EXPECT(worst < 1e-6);
+    bool thrown = false;
+    try {
+        dp::Tensor bad(ctx, dp::Shape(B, C, OH + 1, OW));
+        mp->enqueue(X, bad, q);
+    } catch (dp::ValidationError const &) {
+        thrown = true;
+    }
+    EXPECT(thrown);
+}
+
 int main(int argc, char **argv)
 {
     std::string dev = argc > 1 ? argv[1] : "0";
@@ -183,6 +235,7 @@ int main(int argc, char **argv)
             conv_case(ctx, q, 3, 24, 24, 9, 3, 2, 1, 24, true, A::relu6, "", "depthwise_separable", 0.0f);
             conv_case(ctx, q, 1, 8, 6, 5, 1, 1, 0, 2, true, A::sigmoid, "winograd", "gemm", 0.0f); // incompatible request -> gemm
             ip_case(ctx, q, 5, 64, 10);
+            pool_case(ctx, q);
             // sub-tensor views share memory: run on the second image of a batch-2 tensor
             dp::Tensor big(ctx, dp::Shape(2, 4, 6, 6));
             dp::Tensor second = big.sub_tensor(4 * 6 * 6, dp::Shape(1, 4, 6, 6));

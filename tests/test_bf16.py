@@ -22,7 +22,7 @@ def run_conv_bf16(c, x, w, bias, algo="", factor=0.0, y_init=None):
 
     st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
     op = dlp.Conv2DForward.create(st, bias is not None, c["activation"], algo)
-    assert op.algo() == (algo if algo in ("gemm", "winograd") else "gemm")
+    assert op.algo() == (algo if algo else "gemm")
     y = _bf(y_init) if y_init is not None else torch.full(dlp.conv2d_output_shape(st, x.shape), float("nan"), dtype=torch.bfloat16, device="cuda:0")
     ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
     bd = torch.from_numpy(bias).cuda() if bias is not None else None
@@ -39,7 +39,7 @@ CASES = [
     (case(3, 1, 2, 1, 128, 128, True, 1, True), (2, 56, 56)),
     (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),      # split-K path
     (case((3, 5), (1, 2), (2, 3), (3, 2), 3, 8, False, 1, False), (2, 19, 19)),
-    (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise geometry, served by gemm
+    (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise geometry through gemm (channel-major K, one channel per group)
     # bf16 matrix instruction, pixel-pair loader ("same" stride-1 convolutions with Cin/groups % 32 == 0)
     (case(1, 0, 1, 1, 64, 256, True, 1, True), (5, 7, 7)),       # odd pixel count per image: padded column numbering
     (case(1, 0, 1, 1, 2048, 512, True, 1, True), (3, 7, 7)),     # long K, split over workgroups
@@ -78,6 +78,19 @@ def test_bf16_winograd_vs_fp32_reference(oracle_mod, cin, cout, bhw):
     assert np.abs(got - want).max() <= 1e-2 * scale
     want_r = oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, "relu", threads=8)
     np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=2e-4 * scale)
+
+
+@pytest.mark.parametrize("ch,hw,stride,k", [(144, 56, 1, 3), (192, 28, 2, 3), (40, 9, 1, 3), (24, 11, 2, 3), (16, 12, 1, 5)])
+def test_bf16_depthwise_vs_fp32_reference(oracle_mod, ch, hw, stride, k):
+    c = case(k, k // 2, stride, 1, ch, ch, True, ch, False)
+    c = dict(c, activation="relu6")
+    x, w, bias = make_tensors(c, (2, hw, hw), seed=23)
+    got = run_conv_bf16(c, x, w, bias, algo="depthwise_separable")
+    cfg = oracle_mod.make_cfg(ch, ch, k, stride, 1, k // 2, ch)
+    want_r = oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, "relu6", threads=8)
+    np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=1e-3)
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, "relu6", threads=8)
+    assert np.abs(got - want).max() <= 1e-2 * max(np.abs(want).max(), 1.0)
 
 
 def test_bf16_factor_contract(oracle_mod):
