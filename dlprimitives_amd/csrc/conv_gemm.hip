@@ -493,10 +493,16 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 // The sum over k is accumulated in fp32 exactly as in the fp32 kernel (products of bf16 values
 // are exact in fp32), only in a different order.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+// Register sets of tiles in flight (2 or 4).  Measured: 4 sets (two more K steps of load latency
+// hidden, 148 instead of 102 VGPRs) are not faster -- the kernel is bound by the vector-memory
+// access rate, not by latency -- so 2 sets and three workgroups per CU it is.
+#ifndef DLP_BF16_NSET
+#define DLP_BF16_NSET 2
+#endif
 constexpr int BK2 = 32;
 constexpr int LDK = BK2 + 8;
 
-template <int BM, int BN, int WM, int WN, int ORDER, int ACT>
+template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -583,9 +589,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     const uint32_t a_tile_bytes = BM * BK2 * 2;
     const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
 
-    u32x4 ra[2][A_LD];
-    uint32_t rb[2][B_LD]; // one bf16 each, zero extended
-    uint32_t vsel[2] = {kOutOfRange, kOutOfRange};
+    // NSET register sets hold the tiles in flight: at K step i they hold tiles i+1 .. i+NSET; the
+    // step stores tile i+1 to LDS and at once reuses that set for the loads of tile i+NSET+1, so a
+    // load has NSET K steps to land (one step is only a few hundred matrix cycles here).
+    u32x4 ra[NSET][A_LD];
+    uint32_t rb[NSET][B_LD]; // one bf16 each, zero extended
+    uint32_t vsel[NSET];
 
     auto load_half = [&](auto set, int kt, auto half_c) {
         constexpr int S = decltype(set)::value;
@@ -651,10 +660,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
 
-    // K step on tile kt in LDS[BUF]: set_next (tile kt+1) -> LDS[BUF^1], tile kt+2 -> set_load
-    auto k_step = [&](auto buf_c, auto set_next, auto set_load, int kt) {
-        constexpr int BUF = decltype(buf_c)::value;
+    // K step i (compile-time residue mod NSET) on tile kt = kt_begin + i, resident in LDS[i % 2]
+    auto k_step = [&](auto step_c, int kt) {
+        constexpr int STEP = decltype(step_c)::value;
+        constexpr int BUF = STEP & 1;
         using NextBuf = std::integral_constant<int, BUF ^ 1>;
+        const std::integral_constant<int, (STEP + 1) % NSET> set{};
         bf16x8 fa[2][TM], fb[2][TN];
 #pragma unroll
         for (int s = 0; s < 2; s++) {
@@ -665,15 +676,15 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             for (int j = 0; j < TN; j++)
                 fb[s][j] = *(const bf16x8 *)&Bs[BUF][wn * WTN + j * 32 + l32][s * 16 + h * 8];
         }
-        store_half(set_next, NextBuf{}, std::integral_constant<int, 0>{});
-        load_half(set_load, kt + 2, std::integral_constant<int, 0>{});
+        store_half(set, NextBuf{}, std::integral_constant<int, 0>{});
+        load_half(set, kt + NSET + 1, std::integral_constant<int, 0>{});
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
-        store_half(set_next, NextBuf{}, std::integral_constant<int, 1>{});
-        load_half(set_load, kt + 2, std::integral_constant<int, 1>{});
+        store_half(set, NextBuf{}, std::integral_constant<int, 1>{});
+        load_half(set, kt + NSET + 1, std::integral_constant<int, 1>{});
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -684,20 +695,41 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    static_assert(NSET == 2 || NSET == 4, "the K loop is unrolled NSET times");
     load_half(I0{}, kt_begin, I0{});
     load_half(I0{}, kt_begin, I1{});
     load_half(I1{}, kt_begin + 1, I0{});
     load_half(I1{}, kt_begin + 1, I1{});
+    if constexpr (NSET == 4) {
+        load_half(I2{}, kt_begin + 2, I0{});
+        load_half(I2{}, kt_begin + 2, I1{});
+        load_half(I3{}, kt_begin + 3, I0{});
+        load_half(I3{}, kt_begin + 3, I1{});
+    }
     store_half(I0{}, I0{}, I0{});
     store_half(I0{}, I0{}, I1{});
+    load_half(I0{}, kt_begin + NSET, I0{});
+    load_half(I0{}, kt_begin + NSET, I1{});
     __syncthreads();
     int kt = kt_begin;
-    for (; kt + 1 < kt_end; kt += 2) {
-        k_step(I0{}, I1{}, I0{}, kt);
-        k_step(I1{}, I0{}, I1{}, kt + 1);
+    for (; kt + NSET - 1 < kt_end; kt += NSET) {
+        k_step(I0{}, kt);
+        k_step(I1{}, kt + 1);
+        if constexpr (NSET == 4) {
+            k_step(I2{}, kt + 2);
+            k_step(I3{}, kt + 3);
+        }
     }
     if (kt < kt_end)
-        k_step(I0{}, I1{}, I0{}, kt);
+        k_step(I0{}, kt);
+    if constexpr (NSET == 4) {
+        if (kt + 1 < kt_end)
+            k_step(I1{}, kt + 1);
+        if (kt + 2 < kt_end)
+            k_step(I2{}, kt + 2);
+    }
 
     if (a.splitk > 1) {
         if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
@@ -989,10 +1021,10 @@ int launch_bf16_mfma(const ConvGeom &g, int order, GemmArgs &a, hipStream_t stre
     {
         TimingScope ts("conv_gemm", stream);
         if (order == GEMM_ORDER_TAP_BF16)
-            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0,
+            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET>), dim3((unsigned)blocks), dim3(kThreads), 0,
                                stream, a);
         else
-            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP>), dim3((unsigned)blocks),
+            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2>), dim3((unsigned)blocks),
                                dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
