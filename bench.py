@@ -42,8 +42,9 @@ BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 imag
 # scaled by what the same counter reads for a plain copy of known size: x2.0 / x1.0).
 # Measured offline (a benchmark run cannot collect counters on itself); keyed by (workload, kernel).
 MEASURED_TRAFFIC_BYTES = {
-    ("resnet18", "conv_gemm_f32_kernel<float, 64, 64, 2, 2, 1, 1, 0>"): (17849.2 * 2.0 + 27428.2) * 1024,
-    ("winograd", "wino_fused_kernel<float, ...>"): ((16818.7 + 40712.3) / 2 * 2.0 + (25373.0 + 12838.7) / 2) * 1024,
+    ("resnet18", "conv_gemm_f32_kernel<float, 64, 64, 2, 2, 1, 1, 0>"): (17948.0 * 2.0 + 27441.7) * 1024,
+    ("winograd", "wino_fused_kernel<float, ...>"): ((16817.5 + 40712.4) / 2 * 2.0 + (25377.0 + 12838.6) / 2) * 1024,
+    ("mobilenet", "depthwise3x3_kernel<float, 1>"): (27364.9 * 2.0 + 45795.7) * 1024,
 }
 
 
@@ -109,7 +110,7 @@ def kernel_class(L, bf16=False):
     small = L["kernel"] ** 2 <= 31
     if bf16 and L["activation"] not in ("tanh", "sigmoid"):
         order = 2 if (small and cin_g % 32 == 0) else 3  # one tap x 32 channels per K tile, or the per-element table
-        return "conv_gemm_bf16_kernel<%s, %d, 0>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4", order)
+        return "conv_gemm_bf16_kernel<%s, %d, 0, 2>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4", order)
     tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     order = 1 if (small and cin_g % 16 == 0) else 0
     mask = 1 if small else 2
