@@ -49,6 +49,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int BK = 16;
 constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
+constexpr int kPatchPitch = 192;               // LDS patch rows of conv_patch_f32_kernel
 
 enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
@@ -131,6 +132,10 @@ __device__ __forceinline__ void static_for_all(F &&f)
     f(std::integral_constant<int, 6>{});
     f(std::integral_constant<int, 7>{});
 }
+
+template <class T, int BM, int BN, int WM, int WN, int ACT>
+__device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
+                                                 int g, int slice, int wm, int wn, int h, int l32, int tid);
 
 template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
@@ -362,6 +367,18 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     if (kt < kt_end)
         k_step(I0{}, I1{}, I0{}, kt);
 
+    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, wm, wn, h, l32, tid);
+}
+
+// What a workgroup does with its finished accumulator tile: the split-K partial store, or the
+// epilogue (bias, activation, factor) and the NCHW store.  `lds` is LDS that is free after the
+// last barrier of the main loop (at least BM floats).
+template <class T, int BM, int BN, int WM, int WN, int ACT>
+__device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
+                                                 int g, int slice, int wm, int wn, int h, int l32, int tid)
+{
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
     // ---- split-K: raw partial sums to the workspace, reduced by a second kernel ----
     if (a.splitk > 1) {
         if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
@@ -407,7 +424,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // through LDS (free after the last barrier) and the stores are buffer stores whose row offset
     // is scalar, instead of a bias load and 64-bit address arithmetic per value.
     if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
-        float *bias_s = &As[0][0][0];
+        float *bias_s = lds;
         if (tid < BM)
             bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
         __syncthreads();
@@ -475,6 +492,220 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             }
         }
     }
+}
+
+// ---- stride-1 "same" convolutions: the input patch of a tile goes through LDS once ----------
+// For stride 1, dilation 1 and output size == input size, the pixels that the KH*KW taps of a
+// run of 64 output pixels read are one run of 64 + 2*(ph*W + pw) consecutive pixels of each
+// input channel plane (one such run per image when the tile crosses an image boundary).  A K
+// stage = 16 input channels: its patch [16][PITCH] is loaded once, with coalesced loads and no
+// masks, and serves all KH*KW K tiles of the stage.  An MFMA B operand is then a ds_read at
+// (lane's patch row + tap shift); padding taps read a row that is always zero.  Every
+// address is fixed before the main loop, which is left with MFMAs, LDS reads with immediate
+// offsets and the loads of the next stage: no vector-ALU work at all.
+// Weights: the same packed tap-major tiles as the gathering kernel (K tile = stage * KH*KW + tap).
+template <int N, class F, int... I>
+__device__ __forceinline__ void static_for_seq(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for_n(F &&f)
+{
+    static_for_seq<N>(f, std::make_integer_sequence<int, N>{});
+}
+
+template <class T, int KH, int KW, int PITCH, int ACT>
+__global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
+{
+    constexpr int BM = 64, BN = 64, WM = 2, WN = 2, KHW = KH * KW;
+    constexpr int QS = PITCH / 64;  // patch rows per lane
+    constexpr int CPW = BK / 4;     // channels of a stage per wavefront
+    constexpr int NPL = QS * CPW;   // patch loads per lane and stage
+    constexpr int MAXSEG = 3;       // images a tile may touch (H*W >= 32)
+    constexpr int ZERO_ROW = PITCH - 1; // never loaded: reads 0 in every channel
+    static_assert(PITCH % 64 == 0 && BK == 16, "patch shape");
+
+    __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
+    __shared__ float Ps[2][BK][PITCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+
+    int t; // XCD-contiguous tile numbering, as in conv_gemm_f32_kernel
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, r = nb & 7;
+        const int xcd = bid & 7, slot = bid >> 3;
+        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    }
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    t /= a.ntiles;
+    const int g = t % a.groups;
+    const int slice = t / a.groups;
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int ncb = a.nkt / KHW;                  // stages in K
+    const int cb_per = a.kt_per_slice / KHW;      // the host makes kt_per_slice a multiple of KHW
+    const int cb_begin = slice * cb_per;
+    const int cb_end = min(cb_begin + cb_per, ncb);
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
+
+    // ---- the tile's patch: one segment of consecutive plane pixels per image (wavefront-uniform) ----
+    const int HW = a.OHW;
+    const int halo = a.ph * a.W + a.pw;
+    const int n_last = min(n0 + BN, a.N) - 1;
+    const int b0 = (int)fast_div((uint32_t)n0, a.ohw_magic, a.ohw_shift);
+    int seg_row[MAXSEG], seg_a[MAXSEG], seg_len[MAXSEG];
+    {
+        int row = 0;
+#pragma unroll
+        for (int s = 0; s < MAXSEG; s++) {
+            const int base = (b0 + s) * HW;
+            const int first = max(n0, base), last = min(n_last, base + HW - 1);
+            int as = 0, len = 0;
+            if (first <= last) {
+                as = max(0, first - base - halo);
+                len = min(HW, last - base + 1 + halo) - as;
+            }
+            seg_row[s] = row;
+            seg_a[s] = as;
+            seg_len[s] = len;
+            row += len;
+        }
+    }
+    // patch rows lane, lane + 64, ...: byte offset of the pixel in channel 0 of the group (or out of range)
+    uint32_t pvoff[QS];
+#pragma unroll
+    for (int q = 0; q < QS; q++) {
+        const int rho = lane + 64 * q;
+        uint32_t v = kOutOfRange;
+#pragma unroll
+        for (int s = 0; s < MAXSEG; s++) {
+            const int d = rho - seg_row[s];
+            if (d >= 0 && d < seg_len[s])
+                v = (uint32_t)((((b0 + s) * a.Cin + g * a.Cin_g) * HW + seg_a[s] + d) * (int)sizeof(T));
+        }
+        pvoff[q] = v;
+    }
+    // this lane's B operand (k = h, column l32 of the wavefront tile) per tap: byte offset in a patch buffer
+    uint32_t baddr[KHW];
+    {
+        const int n = n0 + wn * 32 + l32;
+        const bool vn = n < a.N;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * HW;
+        const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+        const int ox = pix - oy * a.OW;
+        const int s = b - b0;
+        const int row = pix + (s == 0 ? seg_row[0] - seg_a[0] : s == 1 ? seg_row[1] - seg_a[1] : seg_row[2] - seg_a[2]);
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) {
+                const int yy = oy + ky - a.ph, xx = ox + kx - a.pw;
+                const bool ok = vn && yy >= 0 && yy < a.H && xx >= 0 && xx < a.W;
+                const int r = ok ? row + (ky - a.ph) * a.W + (kx - a.pw) : ZERO_ROW;
+                baddr[ky * KW + kx] = (uint32_t)((h * PITCH + r) * 4);
+            }
+    }
+
+    const uint32_t a_tile_bytes = BK * BM * 4;
+    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
+
+    f32x4 ra[2];      // packed A tiles in flight (distance two, as in conv_gemm_f32_kernel)
+    float preg[NPL];  // patch of the next stage
+    f32x16 acc[1][1];
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        acc[0][0][r] = 0.0f;
+
+    auto load_a = [&](auto set, int kt) {
+        ra[decltype(set)::value] = buf_load4(wr, (uint32_t)(tid * 16), a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes);
+    };
+    auto store_a = [&](auto set, auto buf_c) {
+        *(f32x4 *)&As[decltype(buf_c)::value][tid / (BM / 4)][(tid % (BM / 4)) * 4] = ra[decltype(set)::value];
+    };
+    auto load_patch = [&](int j, uint32_t stage_soff) { // j = channel-in-wavefront * QS + row slot
+        preg[j] = buf_load<T>(xr, pvoff[j % QS], stage_soff + (uint32_t)(j / QS) * a.hw4);
+    };
+    auto store_patch = [&](auto buf_c, int j) { Ps[decltype(buf_c)::value][wave * CPW + j / QS][lane + 64 * (j % QS)] = preg[j]; };
+
+    // One stage: KHW K tiles on patch buffer P; the patch of stage cb + 1 is requested during
+    // the first tile and goes to the other buffer during the last one.
+    auto stage = [&](auto par, int cb) {
+        constexpr int P = decltype(par)::value;
+        using OtherP = std::integral_constant<int, P ^ 1>;
+        const uint32_t next_soff = (uint32_t)(min(cb + 1, ncb - 1) * BK + wave * CPW) * a.hw4;
+        static_for_n<KHW>([&](auto tau_c) {
+            constexpr int TAU = decltype(tau_c)::value;
+            constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2 drives the A buffers and register sets
+            constexpr int BUF = IDX & 1;
+            using NextBuf = std::integral_constant<int, BUF ^ 1>;
+            using SetNext = std::integral_constant<int, (IDX + 1) & 1>;
+            using SetLoad = std::integral_constant<int, IDX & 1>;
+            const int kt = cb * KHW + TAU;
+            const float *arow = &As[BUF][h][wm * 32 + l32];
+            const char *prow = reinterpret_cast<const char *>(&Ps[P][0][0]) + baddr[TAU];
+            float fa[2], fb[2];
+            fa[0] = arow[0];
+            fb[0] = *reinterpret_cast<const float *>(prow);
+#pragma unroll
+            for (int kk = 0; kk < BK / 2; kk++) {
+                const int cur = kk & 1;
+                if (kk + 1 < BK / 2) {
+                    fa[cur ^ 1] = arow[2 * (kk + 1) * BM];
+                    fb[cur ^ 1] = *reinterpret_cast<const float *>(prow + 2 * (kk + 1) * PITCH * 4);
+                }
+                if (kk == 0)
+                    store_a(SetNext{}, NextBuf{});
+                if (kk == 1)
+                    load_a(SetLoad{}, kt + 2);
+#pragma unroll
+                for (int j = 0; j < NPL; j++)
+                    if (j % (BK / 2) == kk) {
+                        if (TAU == 0)
+                            load_patch(j, next_soff);
+                        if (TAU == KHW - 1)
+                            store_patch(OtherP{}, j);
+                    }
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur], fb[cur], acc[0][0], 0, 0, 0);
+            }
+            __syncthreads();
+        });
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    {
+        const uint32_t soff0 = (uint32_t)(cb_begin * BK + wave * CPW) * a.hw4;
+#pragma unroll
+        for (int j = 0; j < NPL; j++)
+            load_patch(j, soff0);
+        load_a(I0{}, cb_begin * KHW);
+        load_a(I1{}, cb_begin * KHW + 1);
+#pragma unroll
+        for (int j = 0; j < NPL; j++)
+            store_patch(I0{}, j);
+        store_a(I0{}, I0{});
+        __syncthreads();
+    }
+    int cb = cb_begin;
+    for (; cb + 1 < cb_end; cb += 2) {
+        stage(I0{}, cb);
+        stage(I1{}, cb + 1);
+    }
+    if (cb < cb_end)
+        stage(I0{}, cb);
+
+    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, wm, wn, h, l32, tid);
 }
 
 // ---- bfloat16 storage on the bf16 matrix instruction ------------------------------------
@@ -947,6 +1178,73 @@ __global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int 
     out[idx] = v;
 }
 
+// Tap-major K orders: the same packed layouts as the two kernels above, written through an LDS
+// transpose.  One workgroup takes 16 filters x one block of KB channels: that is 16 runs of
+// KB*khw consecutive source elements (read coalesced), which it scatters into the khw K tiles
+// of the channel block, 16 consecutive filters ([k][m] tiles) or KB consecutive channels
+// ([m][k] tiles) at a time.  Dynamic LDS: 16 * (KB*khw + 1) elements of TI.
+template <class TI, class TO, int KB, bool M_MAJOR>
+__global__ __launch_bounds__(256) void pack_weights_tap_kernel(GemmPlan p, int ncb, int khw, const TI *__restrict__ w,
+                                                               TO *__restrict__ out)
+{
+    extern __shared__ __align__(16) unsigned char pack_smem[];
+    TI *lds = reinterpret_cast<TI *>(pack_smem);
+    const int run = KB * khw, ld = run + 1;
+    const int mchunks = p.BM / 16;
+    int bid = (int)blockIdx.x;
+    const int mc = bid % mchunks;
+    bid /= mchunks;
+    const int cb = bid % ncb;
+    bid /= ncb;
+    const int mt = bid % p.mtiles;
+    const int g = bid / p.mtiles;
+    const int m_base = mt * p.BM + mc * 16;
+    const int col0 = cb * run;
+    const int total = 16 * run;
+    // each wavefront reads four filter rows, 16 bytes per lane, all four loads in flight at once
+    // (the source rows start on 16-byte boundaries: K is a multiple of KB and the host checks w)
+    constexpr int VEC = 16 / (int)sizeof(TI);
+    struct alignas(16) Vec {
+        TI e[VEC];
+    };
+    const int wv = (int)threadIdx.x >> 6;
+    for (int j = ((int)threadIdx.x & 63) * VEC; j < run; j += 64 * VEC) {
+        Vec v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int m = m_base + wv + 4 * q;
+            v[q] = Vec();
+            if (m < p.M)
+                v[q] = *reinterpret_cast<const Vec *>(w + ((size_t)g * p.M + m) * p.K + col0 + j);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                lds[(wv + 4 * q) * ld + j + e] = v[q].e[e];
+    }
+    __syncthreads();
+    TO *tile0 = out + ((size_t)(g * p.mtiles + mt) * p.nkt + (size_t)cb * khw) * (KB * p.BM);
+#pragma unroll 4
+    for (int idx = (int)threadIdx.x; idx < total; idx += 256) {
+        int r, k;
+        if (M_MAJOR) {
+            k = idx % KB;
+            r = (idx / KB) % 16;
+        } else {
+            r = idx % 16;
+            k = (idx / 16) % KB;
+        }
+        const int tap = idx / (16 * KB);
+        const TI v = lds[r * ld + k * khw + tap];
+        TO *dst = tile0 + (size_t)tap * (KB * p.BM) + (M_MAJOR ? (mc * 16 + r) * KB + k : k * p.BM + mc * 16 + r);
+        if constexpr (sizeof(TO) == sizeof(TI))
+            *dst = v;
+        else
+            *dst = to_float(v);
+    }
+}
+
 bool bf16_mfma_order(int order) { return order == GEMM_ORDER_TAP_BF16 || order == GEMM_ORDER_CHANNEL_BF16; }
 
 // Split-K factor for a launch of `tiles` output tiles over `nkt` K tiles.
@@ -989,6 +1287,10 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
     if (s > 1 && (!have_ws || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
+    if (p.patch) { // whole stages of KH*KW tiles
+        const int khw = a.KH * a.KW, stages = a.nkt / khw;
+        a.kt_per_slice = (stages + s - 1) / s * khw;
+    }
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
 }
 
@@ -1032,6 +1334,25 @@ int launch_bf16_mfma(const ConvGeom &g, int order, GemmArgs &a, hipStream_t stre
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
         hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+int launch_patch(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+{
+    long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
+    if (blocks > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    {
+        TimingScope ts("conv_gemm", stream);
+        hipLaunchKernelGGL((conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    }
+    if (a.splitk > 1) {
+        TimingScope ts("splitk_reduce", stream);
+        if (a.Cout > 65535)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
+        hipLaunchKernelGGL((splitk_reduce_kernel<float, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
@@ -1086,6 +1407,9 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
     }
     p.tile = tile_choice(p.M);
+    // stride-1 3x3 "same" convolutions whose 64-pixel patch fits the LDS rows (W <= 62): LDS-patch kernel
+    p.patch = g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && p.tile == 0 && g.KH == 3 && g.KW == 3 && g.sh == 1 && g.sw == 1 &&
+              g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 && g.H * g.W >= 32 && 64 + 2 * (g.W + 1) < kPatchPitch;
     if (g.dtype == DLP_BFLOAT16 && !generic_act(activation)) { // bf16 matrix instruction
         const bool tap_major = small_kernel && cin_g % BK2 == 0;
         p.order = tap_major ? GEMM_ORDER_TAP_BF16 : GEMM_ORDER_CHANNEL_BF16;
@@ -1169,7 +1493,20 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
     TimingScope ts("pack_weights", stream);
-    if (bf16_mfma_order(p.order))
+    const int khw = g.KH * g.KW;
+    if ((p.order == GEMM_ORDER_TAP || p.order == GEMM_ORDER_TAP_BF16) && ((uintptr_t)w & 15) == 0) {
+        const int ncb = p.nkt / khw;
+        const dim3 grid((unsigned)((long long)g.groups * p.mtiles * ncb * (p.BM / 16)));
+        if (p.order == GEMM_ORDER_TAP_BF16)
+            hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, bf16_t, BK2, true>), grid, dim3(256),
+                               16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked);
+        else if (g.dtype == DLP_BFLOAT16)
+            hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, float, BK, false>), grid, dim3(256),
+                               16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked);
+        else
+            hipLaunchKernelGGL((pack_weights_tap_kernel<float, float, BK, false>), grid, dim3(256),
+                               16 * (BK * khw + 1) * sizeof(float), stream, p, ncb, khw, (const float *)w, (float *)wpacked);
+    } else if (bf16_mfma_order(p.order))
         hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
                            g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked);
     else if (g.dtype == DLP_BFLOAT16)
@@ -1246,6 +1583,8 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
 
     if (bf16_mfma_order(p.order))
         return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, p.order, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, p.order, a, stream);
+    if (p.patch)
+        return launch_patch(g, a, stream);
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)
             return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);

@@ -153,6 +153,7 @@ struct GemmPlan {
     int tile, BM, BN;   // workgroup tile
     int M, K, nkt;      // per group: rows, reduction length, K tiles of 16
     int mtiles;         // ceil(M / BM)
+    int patch;          // 1: stride-1 "same" convolution run by the LDS-patch kernel (tap-major packed weights)
     size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded
 };
 GemmPlan conv_gemm_plan(const ConvGeom &g, int activation);
