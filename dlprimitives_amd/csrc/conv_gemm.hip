@@ -63,6 +63,13 @@ struct GemmArgs {
     int mtiles, ntiles;
     int splitk, kt_per_slice; // K tiles are dealt to `splitk` slices of kt_per_slice (even) tiles
     float *part;              // split-K partial sums [slice][Cout][N]
+    int sk_units;             // stream-K (conv_patch_f32_kernel): tiles * stages
+    float *sk_part;           // two 64x64 accumulator images per workgroup
+    uint32_t sk_part_bytes;
+#ifdef DLP_PATCH_TRACE
+    long long *trace;
+#endif
+    int *sk_cnt;              // pieces arrived, per tile (zero at launch)
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -536,27 +543,37 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const int h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
 
-    int t; // XCD-contiguous tile numbering, as in conv_gemm_f32_kernel
+    // ---- stream-K: the K stages of all tiles, in tile order, are dealt evenly to the workgroups ----
+    // unit = (tile, stage); workgroup j (XCD-contiguous numbering, as in conv_gemm_f32_kernel) runs
+    // units [j*U/G, (j+1)*U/G): the tail of one tile, whole tiles, the head of another.
+    int j;
     {
         const int nb = gridDim.x, bid = blockIdx.x;
         const int q = nb >> 3, r = nb & 7;
         const int xcd = bid & 7, slot = bid >> 3;
-        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+        j = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
     }
-    const int mt = t % a.mtiles;
-    t /= a.mtiles;
-    const int nt = t % a.ntiles;
-    t /= a.ntiles;
-    const int g = t % a.groups;
-    const int slice = t / a.groups;
-    const int m0 = mt * BM, n0 = nt * BN;
-    const int ncb = a.nkt / KHW;                  // stages in K
-    const int cb_per = a.kt_per_slice / KHW;      // the host makes kt_per_slice a multiple of KHW
-    const int cb_begin = slice * cb_per;
-    const int cb_end = min(cb_begin + cb_per, ncb);
+    const int ncb = a.nkt / KHW; // stages per tile
+    const uint64_t U = (uint64_t)a.sk_units, G = gridDim.x;
+    const int u_begin = (int)((uint64_t)j * U / G), u_end = (int)((uint64_t)(j + 1) * U / G);
+#ifdef DLP_PATCH_TRACE
+    long long tr[4] = {(long long)wall_clock64(), 0, 0, 0};
+    const long long ck0 = (long long)clock64();
+#endif
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
+
+    for (int u = u_begin; u < u_end;) {
+    int t = u / ncb; // tile: m tile fastest, then n tile, then group
+    const int tile = t;
+    const int cb_begin = u - t * ncb;
+    const int cb_end = min(ncb, cb_begin + (u_end - u));
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    const int g = t / a.ntiles;
+    const int m0 = mt * BM, n0 = nt * BN;
 
     // ---- the tile's patch: one segment of consecutive plane pixels per image (wavefront-uniform) ----
     const int HW = a.OHW;
@@ -620,8 +637,10 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const uint32_t a_tile_bytes = BK * BM * 4;
     const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
 
-    f32x4 ra[2];      // packed A tiles in flight (distance two, as in conv_gemm_f32_kernel)
+    static_assert((2 * KHW) % 3 == 0, "three A register sets rotate with period 3 inside a pair of stages");
+    f32x4 ra[3];      // packed A tiles in flight: tile kt + 3 is requested while tile kt is multiplied
     float preg[NPL];  // patch of the next stage
+    float fa[2][BK / 2], fb[2][BK / 2]; // MFMA operands of this K tile and of the next one
     f32x16 acc[1][1];
 #pragma unroll
     for (int r = 0; r < 16; r++)
@@ -637,66 +656,84 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         preg[j] = buf_load<T>(xr, pvoff[j % QS], stage_soff + (uint32_t)(j / QS) * a.hw4);
     };
     auto store_patch = [&](auto buf_c, int j) { Ps[decltype(buf_c)::value][wave * CPW + j / QS][lane + 64 * (j % QS)] = preg[j]; };
+    // operands kk of the K tile (A buffer ABUF, patch buffer PB, tap TAP) into operand set OS
+    auto read_operands = [&](auto os_c, auto abuf_c, auto pb_c, auto tap_c, int kk) {
+        constexpr int OS = decltype(os_c)::value;
+        fa[OS][kk] = As[decltype(abuf_c)::value][2 * kk + h][wm * 32 + l32];
+        fb[OS][kk] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(&Ps[decltype(pb_c)::value][0][0]) +
+                                                      baddr[decltype(tap_c)::value] + 2 * kk * PITCH * 4);
+    };
 
     // One stage: KHW K tiles on patch buffer P; the patch of stage cb + 1 is requested during
-    // the first tile and goes to the other buffer during the last one.
+    // the first tile and goes to the other buffer during the last one.  One barrier per K tile,
+    // in its middle: before it, the next tile's A (and patch) go to the LDS buffers nobody reads
+    // any more; after it, the next tile's operands are read while this tile's MFMAs still run,
+    // so a wavefront that is alone on its SIMD does not wait for LDS at the start of a tile.
     auto stage = [&](auto par, int cb) {
         constexpr int P = decltype(par)::value;
         using OtherP = std::integral_constant<int, P ^ 1>;
         const uint32_t next_soff = (uint32_t)(min(cb + 1, ncb - 1) * BK + wave * CPW) * a.hw4;
         static_for_n<KHW>([&](auto tau_c) {
             constexpr int TAU = decltype(tau_c)::value;
-            constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2 drives the A buffers and register sets
+            constexpr int IDX = P * KHW + TAU; // K tile counter: modulo 2 for LDS buffers and operand sets, modulo 3 for A registers
             constexpr int BUF = IDX & 1;
             using NextBuf = std::integral_constant<int, BUF ^ 1>;
-            using SetNext = std::integral_constant<int, (IDX + 1) & 1>;
-            using SetLoad = std::integral_constant<int, IDX & 1>;
+            using SetNext = std::integral_constant<int, (IDX + 1) % 3>;
+            using SetLoad = std::integral_constant<int, IDX % 3>;
+            using NextOps = std::integral_constant<int, BUF ^ 1>;
+            using NextTap = std::integral_constant<int, (TAU + 1) % KHW>;
+            using NextPatch = std::integral_constant<int, (TAU + 1 < KHW) ? P : (P ^ 1)>;
             const int kt = cb * KHW + TAU;
-            const float *arow = &As[BUF][h][wm * 32 + l32];
-            const char *prow = reinterpret_cast<const char *>(&Ps[P][0][0]) + baddr[TAU];
-            float fa[2], fb[2];
-            fa[0] = arow[0];
-            fb[0] = *reinterpret_cast<const float *>(prow);
 #pragma unroll
             for (int kk = 0; kk < BK / 2; kk++) {
-                const int cur = kk & 1;
-                if (kk + 1 < BK / 2) {
-                    fa[cur ^ 1] = arow[2 * (kk + 1) * BM];
-                    fb[cur ^ 1] = *reinterpret_cast<const float *>(prow + 2 * (kk + 1) * PITCH * 4);
-                }
                 if (kk == 0)
                     store_a(SetNext{}, NextBuf{});
                 if (kk == 1)
-                    load_a(SetLoad{}, kt + 2);
+                    load_a(SetLoad{}, kt + 3);
 #pragma unroll
-                for (int j = 0; j < NPL; j++)
-                    if (j % (BK / 2) == kk) {
-                        if (TAU == 0)
-                            load_patch(j, next_soff);
-                        if (TAU == KHW - 1)
-                            store_patch(OtherP{}, j);
-                    }
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur], fb[cur], acc[0][0], 0, 0, 0);
+                for (int j = 0; j < NPL; j++) {
+                    if (TAU == 0 && j % (BK / 2) == kk)
+                        load_patch(j, next_soff);
+                    if (TAU == KHW - 1 && j / 4 == kk) // before the barrier
+                        store_patch(OtherP{}, j);
+                }
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[BUF][kk], fb[BUF][kk], acc[0][0], 0, 0, 0);
+                if (kk == 3)
+                    __syncthreads();
+                if (kk >= 4) {
+                    read_operands(NextOps{}, NextBuf{}, NextPatch{}, NextTap{}, 2 * (kk - 4));
+                    read_operands(NextOps{}, NextBuf{}, NextPatch{}, NextTap{}, 2 * (kk - 4) + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0); // keep this order: the scheduler would sink the operand reads to their uses
             }
-            __syncthreads();
         });
     };
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
     {
+        static_assert(NPL <= 12, "patch stores of the last tile fit before its barrier");
         const uint32_t soff0 = (uint32_t)(cb_begin * BK + wave * CPW) * a.hw4;
 #pragma unroll
         for (int j = 0; j < NPL; j++)
             load_patch(j, soff0);
         load_a(I0{}, cb_begin * KHW);
         load_a(I1{}, cb_begin * KHW + 1);
+        load_a(I2{}, cb_begin * KHW + 2);
 #pragma unroll
         for (int j = 0; j < NPL; j++)
             store_patch(I0{}, j);
         store_a(I0{}, I0{});
         __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK / 2; kk++)
+            read_operands(I0{}, I0{}, I0{}, I0{}, kk);
     }
+#ifdef DLP_PATCH_TRACE
+    if (u == u_begin)
+        tr[1] = (long long)wall_clock64();
+#endif
     int cb = cb_begin;
     for (; cb + 1 < cb_end; cb += 2) {
         stage(I0{}, cb);
@@ -705,7 +742,63 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     if (cb < cb_end)
         stage(I0{}, cb);
 
-    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, wm, wn, h, l32, tid);
+#ifdef DLP_PATCH_TRACE
+    if (u == u_begin)
+        tr[2] = (long long)wall_clock64();
+#endif
+    bool output = true;
+    if (cb_begin != 0 || cb_end != ncb) {
+        // A piece of a tile: its accumulators go to this workgroup's first or second slot (register
+        // image, [r][thread]); the workgroup that arrives last at the tile's counter adds up all the
+        // pieces, in workgroup order whoever it is, and writes the tile.  Nobody waits for anybody.
+        // Pieces bypass the caches in both directions (write-through stores, uncached loads): a
+        // device-wide fence would write back and invalidate a whole L2 per piece.
+        constexpr int kThrough = 17; // sc0 | sc1
+        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.sk_part, 0, a.sk_part_bytes, 0x00020000);
+        const uint32_t piece_bytes = BM * BN * 4;
+        {
+            const uint32_t soff = (uint32_t)(2 * j + (u == u_begin ? 0 : 1)) * piece_bytes;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float v = acc[0][0][r];
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, (uint32_t)(r * kThreads + tid) * 4u, soff, kThrough);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this thread's piece has been written through
+        __syncthreads();
+        int *arrived_s = reinterpret_cast<int *>(&As[1][0][0]); // free after the last barrier of the main loop
+        if (tid == 0)
+            *arrived_s = atomicAdd(a.sk_cnt + tile, 1);
+        __syncthreads();
+        const int arrived = __builtin_amdgcn_readfirstlane(*arrived_s);
+        const uint64_t ut0 = (uint64_t)tile * ncb;
+        const int j_first = (int)(((ut0 + 1) * G - 1) / U), j_last = (int)(((ut0 + ncb) * G - 1) / U);
+        output = arrived == j_last - j_first;
+        if (output) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[0][0][r] = 0.0f;
+            for (int jj = j_first; jj <= j_last; jj++) {
+                const int first_tile = (int)((uint64_t)jj * U / G) / ncb; // tile of jj's first piece
+                const uint32_t soff = (uint32_t)(2 * jj + (first_tile == tile ? 0 : 1)) * piece_bytes;
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[0][0][r] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pr, (uint32_t)(r * kThreads + tid) * 4u, soff, kThrough));
+            }
+        }
+    }
+    if (output)
+        gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, 0, wm, wn, h, l32, tid);
+    __syncthreads(); // LDS is reused by the next piece
+    u += cb_end - cb_begin;
+    }
+#ifdef DLP_PATCH_TRACE
+    tr[3] = (long long)wall_clock64();
+    tr[2] = (long long)clock64() - ck0;
+    if (tid == 0 && a.trace)
+        for (int i = 0; i < 4; i++)
+            a.trace[j * 4 + i] = tr[i];
+#endif
 }
 
 // ---- bfloat16 storage on the bf16 matrix instruction ------------------------------------
@@ -1185,8 +1278,11 @@ __global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int 
 // ([m][k] tiles) at a time.  Dynamic LDS: 16 * (KB*khw + 1) elements of TI.
 template <class TI, class TO, int KB, bool M_MAJOR>
 __global__ __launch_bounds__(256) void pack_weights_tap_kernel(GemmPlan p, int ncb, int khw, const TI *__restrict__ w,
-                                                               TO *__restrict__ out)
+                                                               TO *__restrict__ out, int *__restrict__ zero, int nzero)
 {
+    // side job: clear the tile counters of the stream-K launch that follows on the stream
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < nzero; i += (int)gridDim.x * 256)
+        zero[i] = 0;
     extern __shared__ __align__(16) unsigned char pack_smem[];
     TI *lds = reinterpret_cast<TI *>(pack_smem);
     const int run = KB * khw, ld = run + 1;
@@ -1287,10 +1383,6 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
     if (s > 1 && (!have_ws || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
-    if (p.patch) { // whole stages of KH*KW tiles
-        const int khw = a.KH * a.KW, stages = a.nkt / khw;
-        a.kt_per_slice = (stages + s - 1) / s * khw;
-    }
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
 }
 
@@ -1339,21 +1431,71 @@ int launch_bf16_mfma(const ConvGeom &g, int order, GemmArgs &a, hipStream_t stre
     return DLP_OK;
 }
 
-int launch_patch(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+// Stream-K launch shape of the LDS-patch kernel: three workgroups per CU (measured best of 1..4:
+// one wavefront per SIMD already keeps its matrix pipe ~90 % busy, the others cover barriers and
+// the prologue), every one with the same number of (tile, stage) units, but no fewer than 4
+// stages per workgroup.
+constexpr int kPatchWgsPerCu = 3;
+int device_cu_count()
 {
-    long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
-    if (blocks > 0x7fffffffLL)
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+struct PatchShape {
+    long long tiles, units;
+    int grid;
+    size_t cnt_bytes, ws_bytes; // tile counters | two 64x64 fp32 pieces per workgroup
+};
+PatchShape patch_shape(const ConvGeom &g, const GemmPlan &p, long long N)
+{
+    PatchShape ps;
+    ps.tiles = (long long)p.mtiles * ((N + 63) / 64) * g.groups;
+    ps.units = ps.tiles * (p.nkt / (g.KH * g.KW));
+    long long grid = ps.units / 4;
+    const long long slots = (long long)device_cu_count() * kPatchWgsPerCu;
+    grid = grid < 1 ? 1 : grid > slots ? slots : grid;
+    ps.grid = (int)grid;
+    ps.cnt_bytes = (size_t)((ps.tiles * sizeof(int) + 255) / 256 * 256);
+    ps.ws_bytes = ps.cnt_bytes + (size_t)ps.grid * 2 * 64 * 64 * sizeof(float);
+    return ps;
+}
+
+int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t stream, void *part_ws, size_t part_bytes)
+{
+    a.mtiles = p.mtiles;
+    a.ntiles = (a.N + p.BN - 1) / p.BN;
+    a.splitk = 1;
+    a.kt_per_slice = a.nkt;
+    a.part = nullptr;
+    a.part_bytes = 0;
+    const PatchShape ps = patch_shape(g, p, a.N);
+    if (ps.units > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
-    {
-        TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL((conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+    a.sk_units = (int)ps.units;
+    int grid = ps.grid;
+    // same test as in conv_gemm_pack_weights, which clears the counters
+    if (part_ws != nullptr && part_bytes >= patch_shape(g, p, (long long)g.B * g.OH * g.OW).ws_bytes && part_bytes >= ps.ws_bytes) {
+        a.sk_cnt = (int *)part_ws; // zeroed by conv_gemm_pack_weights, which is handed the same workspace
+        a.sk_part = (float *)((char *)part_ws + ps.cnt_bytes);
+        a.sk_part_bytes = (uint32_t)(ps.ws_bytes - ps.cnt_bytes);
+    } else { // no room for pieces: one whole tile per workgroup
+        a.sk_cnt = nullptr;
+        a.sk_part = nullptr;
+        a.sk_part_bytes = 0;
+        grid = (int)ps.tiles;
     }
-    if (a.splitk > 1) {
-        TimingScope ts("splitk_reduce", stream);
-        if (a.Cout > 65535)
-            return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
-        hipLaunchKernelGGL((splitk_reduce_kernel<float, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
-    }
+#ifdef DLP_PATCH_TRACE
+    a.trace = (part_ws != nullptr && part_bytes >= ps.ws_bytes + (size_t)grid * 32 + (1u << 20)) ? (long long *)((char *)part_ws + part_bytes - (1u << 20)) : nullptr;
+#endif
+    TimingScope ts("conv_gemm", stream);
+    hipLaunchKernelGGL((conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -1479,6 +1621,8 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     if (g.B <= 0)
         return 0;
     const GemmPlan p = conv_gemm_plan(g, activation);
+    if (p.patch)
+        return p.wpack_bytes + patch_shape(g, p, (long long)g.B * g.OH * g.OW).ws_bytes;
     GemmArgs a;
     a.N = g.B * g.OH * g.OW;
     a.Cout = g.Cout;
@@ -1487,8 +1631,18 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     return p.wpack_bytes + (a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0);
 }
 
-int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream)
+int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
+                           size_t part_bytes)
 {
+    int *zero = nullptr; // tile counters of the stream-K launch that follows
+    int nzero = 0;
+    if (p.patch && part_ws != nullptr) {
+        const PatchShape ps = patch_shape(g, p, (long long)g.B * g.OH * g.OW);
+        if (part_bytes >= ps.ws_bytes && ps.tiles <= 0x7fffffffLL) {
+            zero = (int *)part_ws;
+            nzero = (int)ps.tiles;
+        }
+    }
     const long long total = (long long)g.groups * p.mtiles * p.nkt * (bf16_mfma_order(p.order) ? BK2 : BK) * p.BM;
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
@@ -1499,13 +1653,13 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
         const dim3 grid((unsigned)((long long)g.groups * p.mtiles * ncb * (p.BM / 16)));
         if (p.order == GEMM_ORDER_TAP_BF16)
             hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, bf16_t, BK2, true>), grid, dim3(256),
-                               16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked);
+                               16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked, (int *)nullptr, 0);
         else if (g.dtype == DLP_BFLOAT16)
             hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, float, BK, false>), grid, dim3(256),
-                               16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked);
+                               16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked, (int *)nullptr, 0);
         else
             hipLaunchKernelGGL((pack_weights_tap_kernel<float, float, BK, false>), grid, dim3(256),
-                               16 * (BK * khw + 1) * sizeof(float), stream, p, ncb, khw, (const float *)w, (float *)wpacked);
+                               16 * (BK * khw + 1) * sizeof(float), stream, p, ncb, khw, (const float *)w, (float *)wpacked, zero, nzero);
     } else if (bf16_mfma_order(p.order))
         hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
                            g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked);
@@ -1575,6 +1729,8 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     if (ep.activation == DLP_ACT_RELU6)
         a.clamp_hi = 6.0f;
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
+    if (p.patch)
+        return launch_patch(g, p, a, stream, part_ws, part_bytes);
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
     {
         const size_t used = (size_t)a.splitk * a.Cout * a.N * sizeof(float);
@@ -1583,8 +1739,6 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
 
     if (bf16_mfma_order(p.order))
         return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, p.order, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, p.order, a, stream);
-    if (p.patch)
-        return launch_patch(g, a, stream);
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)
             return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);

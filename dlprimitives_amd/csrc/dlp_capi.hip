@@ -389,11 +389,11 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
         // workspace = packed weights | split-K partial sums
         const GemmPlan plan = conv_gemm_plan(g, op->activation);
         DLP_REQUIRE(ws != nullptr && ws_bytes >= plan.wpack_bytes, "workspace smaller than workspace()");
-        rc = conv_gemm_pack_weights(g, plan, w, ws, s);
-        if (rc != DLP_OK)
-            return rc;
         const size_t used = round256(plan.wpack_bytes);
         void *part = ws_bytes > used ? (char *)ws + used : nullptr;
+        rc = conv_gemm_pack_weights(g, plan, w, ws, s, part, part ? ws_bytes - used : 0);
+        if (rc != DLP_OK)
+            return rc;
         return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0);
     }
     }

@@ -164,7 +164,10 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *host_tab)
 // split-K partial sums when there are too few output tiles to fill the chip.
 size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation);
 // Repack [Cout][Cin/groups][KH][KW] weights into the tile order the kernel loads.
-int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream);
+// part_ws/part_bytes: the workspace behind the packed weights that conv_gemm_launch will be given
+// (the packing kernel clears the counters the launch keeps there).
+int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream,
+                           void *part_ws = nullptr, size_t part_bytes = 0);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 // part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,

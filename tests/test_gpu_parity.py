@@ -98,6 +98,68 @@ def test_split_k_through_workspace(gpu, oracle_mod):
     np.testing.assert_allclose(y.cpu().numpy(), oracle_mod.apply_factor(want, old, 0.25), **TOL)
 
 
+# Stride-1 3x3 "same" convolutions with Cin/groups % 16 == 0 and Cout/groups > 32 run the LDS-patch
+# kernel, whose K stages are dealt evenly to the workgroups (stream-K): a tile is in general
+# computed in pieces that meet through the workspace.  (batch, cin, cout, groups, H, W)
+PATCH_SHAPES = [
+    (3, 64, 64, 1, 56, 56),    # whole tiles
+    (18, 64, 64, 1, 56, 56),   # more tiles than workgroups: pieces of 4-stage tiles
+    (5, 128, 128, 1, 28, 28),  # 8 stages per tile, tiles cross image rows
+    (7, 256, 256, 1, 14, 14),  # tiles cross images, N tail
+    (5, 512, 512, 1, 7, 7),    # up to three images per tile, 32 stages per tile
+    (3, 64, 128, 2, 9, 11),    # groups, odd width
+    (2, 48, 80, 1, 6, 62),     # widest supported row; 3 stages (odd), Cout off the tile size
+    (2, 48, 80, 1, 6, 63),     # one pixel wider: the gathering kernel
+    (4, 32, 64, 1, 5, 6),      # plane below 32 pixels: the gathering kernel
+    (1, 16, 40, 1, 40, 40),    # one stage per tile
+]
+
+
+@pytest.mark.parametrize("shape", PATCH_SHAPES, ids=lambda s: "b%d_%dto%d_g%d_%dx%d" % s)
+def test_patch_kernel_stream_k(gpu, oracle_mod, shape):
+    b, cin, cout, groups, h, w_ = shape
+    c = case(3, 1, 1, 1, cin, cout, True, groups, True)
+    x, w, bias = make_tensors(c, (b, h, w_), seed=b * 1000 + cin + h)
+    print("patch case", shape, flush=True)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+    # pieces are added in a fixed order: a second run gives the same bits
+    again, _ = gpu.run_conv(c, x, w, bias, algo="gemm")
+    assert np.array_equal(got, again)
+    # factor contract on the same path
+    old = np.random.default_rng(5).standard_normal(want.shape).astype(np.float32)
+    got_f, _ = gpu.run_conv(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got_f, oracle_mod.apply_factor(want, old, 0.5), **TOL)
+
+
+def test_patch_kernel_integer_exact_and_small_workspace(gpu):
+    # integer-valued tensors: every summation order gives the same fp32 result, so pieces that
+    # were mis-addressed, dropped or added twice cannot hide behind a tolerance.  The same op is
+    # then run with a workspace sized for batch 1: too small for the pieces, so every workgroup
+    # takes whole tiles, and the result must not change.
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(11)
+    c = case(3, 1, 1, 1, 128, 192, True, 1, False)
+    x = np.round(rng.standard_normal((6, 128, 14, 14)) * 2).astype(np.float32)
+    w = np.round(rng.standard_normal((192, 128, 3, 3)) * 2).astype(np.float32)
+    bias = np.round(rng.standard_normal(192) * 3).astype(np.float32)
+    want = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(bias).double(),
+                                      stride=1, padding=1).numpy()
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    assert np.array_equal(got.astype(np.float64), want)
+    op_small = dlp.Conv2DForward.create(gpu.settings_of(c, (1, 128, 14, 14)), True, "identity", "gemm")
+    op_full = dlp.Conv2DForward.create(gpu.settings_of(c, x.shape), True, "identity", "gemm")
+    assert 0 < op_small.workspace() < op_full.workspace()
+    y = torch.full(want.shape, float("nan"), dtype=torch.float32, device="cuda:0")
+    op_full.enqueue(gpu.dev(x), gpu.dev(w), gpu.dev(bias), y, torch.empty(op_small.workspace(), dtype=torch.uint8, device="cuda:0"), 0.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
+
+
 def test_gemm_integer_exact(gpu):
     # integer-valued inputs: fp32 sums are exact in any order, so the MFMA result must
     # EQUAL the integer result -- catches any indexing/layout slip that a tolerance could hide
