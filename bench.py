@@ -113,6 +113,9 @@ def kernel_class(L, bf16=False):
         return "conv_gemm_bf16_kernel<%s, %d, 0, 2>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4", order)
     tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     order = 1 if (small and cin_g % 16 == 0) else 0
+    if (not bf16 and order == 1 and m > 32 and L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
+            and L["hw"] * L["hw"] >= 32 and 64 + 2 * (L["hw"] + 1) < 192 and L["activation"] not in ("tanh", "sigmoid")):
+        return "conv_patch_f32_kernel<float, 3, 3, 192, 0>"  # stride-1 3x3: input patch through LDS, stream-K
     mask = 1 if small else 2
     return "conv_gemm_f32_kernel<%s, %s, %d, %d, 0>" % ("bf16_t" if bf16 else "float", tile, order, mask)
 

@@ -354,6 +354,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0); // keep the operand reads one step ahead of their MFMAs
         }
         __syncthreads();
     };
