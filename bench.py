@@ -42,7 +42,7 @@ BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 imag
 # scaled by what the same counter reads for a plain copy of known size: x2.0 / x1.0).
 # Measured offline (a benchmark run cannot collect counters on itself); keyed by (workload, kernel).
 MEASURED_TRAFFIC_BYTES = {
-    ("resnet18", "conv_gemm_f32_kernel<float, 64, 64, 2, 2, 1, 1, 0>"): (17948.0 * 2.0 + 27441.7) * 1024,
+    ("resnet18", "conv_patch_f32_kernel<float, 3, 3, 192, 0>"): (32886.5 * 2.0 + 46377.9) * 1024,
     ("winograd", "wino_fused_kernel<float, ...>"): ((16817.5 + 40712.4) / 2 * 2.0 + (25377.0 + 12838.6) / 2) * 1024,
     ("mobilenet", "depthwise3x3_kernel<float, 1>"): (27364.9 * 2.0 + 45795.7) * 1024,
 }

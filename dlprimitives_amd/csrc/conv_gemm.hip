@@ -36,6 +36,7 @@
 //    fixed order by a second kernel (deterministic).
 #include "dlp_internal.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace dlp {
@@ -70,6 +71,7 @@ struct GemmArgs {
     long long *trace;
 #endif
     int *sk_cnt;              // pieces arrived, per tile (zero at launch)
+    int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -570,10 +572,36 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const int tile = t;
     const int cb_begin = u - t * ncb;
     const int cb_end = min(ncb, cb_begin + (u_end - u));
-    const int mt = t % a.mtiles;
-    t /= a.mtiles;
-    const int nt = t % a.ntiles;
-    const int g = t / a.ntiles;
+    // Which (group, m tile, n tile) the tile-th tile of the stream is -- any bijection is correct; this
+    // one is chosen for the L2 of the XCD that runs it.  (1) Each eighth of the stream (one XCD's
+    // share) is read transposed, sk_tpw tiles (one workgroup's share) per column: at any time the
+    // workgroups of an XCD then work on neighbouring tiles instead of tiles sk_tpw apart, so the halo
+    // rows that neighbouring pixel tiles share are fetched once.  (2) Neighbouring tiles are the
+    // sk_mb m tiles of one pixel tile, then the next pixel tile: an XCD's share covers few m tiles
+    // (little of the weights) and a compact range of pixels.
+    {
+        const int NT = (int)(U / (uint64_t)ncb);
+        int c = (int)(((int64_t)t * 8) / NT);
+        int lo = (int)(((int64_t)c * NT) / 8), hi = (int)(((int64_t)(c + 1) * NT) / 8);
+        if (t >= hi) {
+            c++;
+            lo = hi;
+            hi = (int)(((int64_t)(c + 1) * NT) / 8);
+        }
+        const int L = hi - lo, i = t - lo;
+        const int q = L / a.sk_tpw, r = L - q * a.sk_tpw;
+        const int col = i / a.sk_tpw, row = i - col * a.sk_tpw;
+        // rows 0..r-1 of the ragged L = q*tpw + r layout hold q+1 tiles, the others q; a column index
+        // past a short row's end only happens in the last (partial) column, which holds rows < r
+        t = lo + row * q + min(row, r) + col;
+    }
+    const int per_group = a.mtiles * a.ntiles;
+    const int g = t / per_group;
+    t -= g * per_group;
+    const int mblk = t / (a.sk_mb * a.ntiles);
+    t -= mblk * a.sk_mb * a.ntiles;
+    const int nt = t / a.sk_mb;
+    const int mt = mblk * a.sk_mb + (t - nt * a.sk_mb);
     const int m0 = mt * BM, n0 = nt * BN;
 
     // ---- the tile's patch: one segment of consecutive plane pixels per image (wavefront-uniform) ----
@@ -1491,6 +1519,24 @@ int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t 
         a.sk_part = nullptr;
         a.sk_part_bytes = 0;
         grid = (int)ps.tiles;
+    }
+    // tile order (see the kernel): tiles per workgroup, and how many m tiles run side by side --
+    // the divisor of mtiles for which one XCD's share of the tiles touches the fewest bytes
+    // (mb m tiles of weights + its pixel tiles of input)
+    a.sk_tpw = (int)std::max<long long>(1, (ps.tiles + grid / 2) / grid);
+    {
+        const double a_bytes = 64.0 * a.K * 4, x_bytes = 64.0 * a.Cin_g * 4, share = (double)ps.tiles / 8;
+        double best = 0;
+        a.sk_mb = 1;
+        for (int mb = 1; mb <= p.mtiles; mb++) {
+            if (p.mtiles % mb)
+                continue;
+            const double cost = mb * a_bytes + share / mb * x_bytes;
+            if (mb == 1 || cost < best) {
+                best = cost;
+                a.sk_mb = mb;
+            }
+        }
     }
 #ifdef DLP_PATCH_TRACE
     a.trace = (part_ws != nullptr && part_bytes >= ps.ws_bytes + (size_t)grid * 32 + (1u << 20)) ? (long long *)((char *)part_ws + part_bytes - (1u << 20)) : nullptr;
