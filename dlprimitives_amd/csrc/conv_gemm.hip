@@ -44,6 +44,7 @@ namespace dlp {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 namespace {
 
@@ -72,6 +73,7 @@ struct GemmArgs {
 #endif
     int *sk_cnt;              // pieces arrived, per tile (zero at launch)
     int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
+    int pxv;                  // bf16 matrix-instruction kernel: pixels per output store (0 = one element per store)
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -855,9 +857,19 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int BK2 = 32;
 constexpr int LDK = BK2 + 8;
 
-template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET>
+// PXL > 0 selects the dense loader (1x1, stride 1, no padding: a plain GEMM W * X per image):
+// a lane loads PXL consecutive pixels of 8 consecutive channels with 8- or 16-byte loads (the
+// texture path handles four lanes per clock whatever the width of the load, so a 16-bit load per
+// element is an eighth of its rate), transposes the 8 x PXL block in registers (one v_perm per
+// dword) and stores each pixel's 8 channels as one 16-byte piece.  The B tile is then kept as
+// [8-channel group][pixel][8 channels] with the pixel index XOR-swizzled (pixel ^ (pixel / 8 % 8))
+// so that both these stores (pixels PXL apart across lanes) and the operand reads (consecutive
+// pixels across lanes) are free of bank conflicts.  64 * 4 / PXL lanes suffice for a tile, so the
+// B tiles are dealt to the wavefronts in turn (LW wavefronts per tile).
+template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
+    static_assert(PXL == 0 || ((PXL == 4 || PXL == 8) && ORDER == GEMM_ORDER_TAP_BF16 && NSET == 2), "dense loader variants");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -870,8 +882,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     static_assert(A_V4 % kThreads == 0, "A loader shape");
     constexpr int A_LD = A_V4 / kThreads;
 
-    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM][LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN][LDK];
+    constexpr int A_TILE_BYTES = BM * LDK * 2, B_TILE_BYTES = BN * LDK * 2;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * A_TILE_BYTES + 2 * B_TILE_BYTES];
+    auto As = reinterpret_cast<uint16_t(*)[BM][LDK]>(smem);
+    auto Bs = reinterpret_cast<uint16_t(*)[BN][LDK]>(smem + 2 * A_TILE_BYTES);
+    unsigned char *const bs_bytes = smem + 2 * A_TILE_BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -942,6 +957,70 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     const uint32_t a_tile_bytes = BM * BK2 * 2;
     const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
 
+    // ---- dense loader state: block = 8 channels x PXL pixels; blocks of a tile = 4 * BN / PXL ----
+    constexpr int PXN = PXL ? PXL : 1;
+    constexpr int NPQ = BN / PXN;                  // pixel groups of a tile
+    constexpr int LW = PXL ? 4 * NPQ / 64 : 4;     // wavefronts that load one B tile
+    constexpr int NSETB = (LW == 4) ? 2 : 1;       // a wavefront that loads every 4/LW-th tile needs one register set
+    constexpr int DW = PXL ? PXL / 2 : 1;          // dwords per load
+    static_assert(LW == 1 || LW == 2 || LW == 4, "loader wavefronts");
+    uint32_t dvoff = kOutOfRange; // byte offset of (first channel of the block, first pixel) in x
+    uint32_t dslot[PXN];          // LDS byte offsets of the block's pixels inside a B tile
+    uint32_t brd[TN];             // LDS byte offset of this lane's operand pixel (channel group h)
+    uint32_t rbw[NSETB][8][DW];
+    const int my_turn = wave / LW; // tile T is loaded by this wavefront when T % (4 / LW) == my_turn
+    if constexpr (PXL > 0) {
+        const int blk = (wave % LW) * 64 + lane;
+        const int oct = blk / NPQ, pq = blk % NPQ;
+        const int n = n0 + pq * PXL; // PXL divides OH*OW: the run stays inside one image
+        if (n < a.N) {
+            const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+            const int pix = n - b * a.OHW;
+            dvoff = (uint32_t)(b * a.Cin + g * a.Cin_g + oct * 8) * a.hw4 + (uint32_t)pix * 2u;
+        }
+#pragma unroll
+        for (int q = 0; q < PXN; q++) {
+            const int x = pq * PXL + q;
+            dslot[q] = (uint32_t)((oct * BN + (x ^ ((x >> 3) & 7))) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int x = wn * WTN + j * 32 + l32;
+            brd[j] = (uint32_t)((h * BN + (x ^ ((x >> 3) & 7))) * 16);
+        }
+    }
+    auto my_tile = [&](int kt) { return LW == 4 || (kt & (4 / LW - 1)) == my_turn; };
+    auto load_b = [&](auto set, int kt) {
+        constexpr int S = decltype(set)::value % NSETB;
+        const uint32_t soff = (uint32_t)(min(kt, a.nkt - 1) * BK2) * a.hw4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if constexpr (PXL == 8) {
+                const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, dvoff, soff + (uint32_t)i * a.hw4, 0));
+#pragma unroll
+                for (int d = 0; d < DW; d++)
+                    rbw[S][i][d] = v[d];
+            } else if constexpr (PXL == 4) {
+                const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(xr, dvoff, soff + (uint32_t)i * a.hw4, 0));
+#pragma unroll
+                for (int d = 0; d < DW; d++)
+                    rbw[S][i][d] = v[d];
+            }
+        }
+    };
+    auto store_b = [&](auto set, auto buf_c) {
+        constexpr int S = decltype(set)::value % NSETB;
+        constexpr int BUF = decltype(buf_c)::value;
+#pragma unroll
+        for (int q = 0; q < PXN; q++) {
+            u32x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; j++) // channels 2j (low half) and 2j+1 of pixel q
+                v[j] = __builtin_amdgcn_perm(rbw[S][2 * j + 1][q / 2], rbw[S][2 * j][q / 2], (q & 1) ? 0x07060302u : 0x05040100u);
+            *(u32x4 *)(bs_bytes + BUF * B_TILE_BYTES + dslot[q]) = v;
+        }
+    };
+
     // NSET register sets hold the tiles in flight: at K step i they hold tiles i+1 .. i+NSET; the
     // step stores tile i+1 to LDS and at once reuses that set for the loads of tile i+NSET+1, so a
     // load has NSET K steps to land (one step is only a few hundred matrix cycles here).
@@ -958,7 +1037,10 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             for (int j = 0; j < A_LD; j++)
                 ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
         }
-        if (ORDER == GEMM_ORDER_TAP_BF16) {
+        if constexpr (PXL > 0) {
+            if (Q == 1 && my_tile(kt))
+                load_b(set, kt);
+        } else if (ORDER == GEMM_ORDER_TAP_BF16) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
             const uint32_t xoff = (uint32_t)e[0], tap = (uint32_t)e[1];
@@ -982,7 +1064,8 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             }
         }
     };
-    auto store_half = [&](auto set, auto buf_c, auto half_c) {
+    // kt = the tile that set S holds
+    auto store_half = [&](auto set, auto buf_c, auto half_c, int kt) {
         constexpr int S = decltype(set)::value;
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int Q = decltype(half_c)::value;
@@ -992,6 +1075,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
                 const int idx = tid + j * kThreads; // 16-byte piece of the [BM][32] tile: row idx/4, piece idx%4
                 *(u32x4 *)&As[BUF][idx >> 2][(idx & 3) * 8] = ra[S][j];
             }
+        }
+        if constexpr (PXL > 0) {
+            if (Q == 0 && my_tile(kt))
+                store_b(set, buf_c);
+            return;
         }
 #pragma unroll
         for (int q = Q * (B_LD / 16); q < (Q + 1) * (B_LD / 16); q++) {
@@ -1026,17 +1114,21 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             for (int i = 0; i < TM; i++)
                 fa[s][i] = *(const bf16x8 *)&As[BUF][wm * WTM + i * 32 + l32][s * 16 + h * 8];
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-                fb[s][j] = *(const bf16x8 *)&Bs[BUF][wn * WTN + j * 32 + l32][s * 16 + h * 8];
+            for (int j = 0; j < TN; j++) {
+                if constexpr (PXL > 0)
+                    fb[s][j] = *(const bf16x8 *)(bs_bytes + BUF * B_TILE_BYTES + brd[j] + s * (2 * BN * 16));
+                else
+                    fb[s][j] = *(const bf16x8 *)&Bs[BUF][wn * WTN + j * 32 + l32][s * 16 + h * 8];
+            }
         }
-        store_half(set, NextBuf{}, std::integral_constant<int, 0>{});
+        store_half(set, NextBuf{}, std::integral_constant<int, 0>{}, kt + 1);
         load_half(set, kt + NSET + 1, std::integral_constant<int, 0>{});
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
-        store_half(set, NextBuf{}, std::integral_constant<int, 1>{});
+        store_half(set, NextBuf{}, std::integral_constant<int, 1>{}, kt + 1);
         load_half(set, kt + NSET + 1, std::integral_constant<int, 1>{});
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -1061,8 +1153,8 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         load_half(I3{}, kt_begin + 3, I0{});
         load_half(I3{}, kt_begin + 3, I1{});
     }
-    store_half(I0{}, I0{}, I0{});
-    store_half(I0{}, I0{}, I1{});
+    store_half(I0{}, I0{}, I0{}, kt_begin);
+    store_half(I0{}, I0{}, I1{}, kt_begin);
     load_half(I0{}, kt_begin + NSET, I0{});
     load_half(I0{}, kt_begin + NSET, I1{});
     __syncthreads();
@@ -1127,6 +1219,69 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     // tile's rows goes through LDS (free after the last barrier), the result is rounded by the
     // hardware conversion and stored with buffer stores whose row offset is scalar: a handful of
     // VALU operations per value instead of 64-bit address arithmetic and a bias load each. ----
+    // Wide stores (a.pxv = 2, 4 or 8 pixels per store; the host sets it when there is no factor, y is
+    // 4-byte aligned and below 2 GiB, and pxv divides OH*OW): the tile goes to LDS as bf16 [m][n]
+    // (rows padded by 16 bytes: the two half-waves, four rows apart, hit different banks) and is
+    // stored to y in runs of pxv pixels per lane, consecutive lanes on consecutive runs of a row --
+    // a store instruction costs the same whatever its width, so this is pxv times fewer of them.
+    if (a.pxv != 0) {
+        constexpr int PITCH = BN * 2 + 16;
+        static_assert(BM * PITCH + BM * 4 <= 2 * A_TILE_BYTES + 2 * B_TILE_BYTES, "the staged tile fits the operand buffers");
+        float *bias_s = (float *)(smem + BM * PITCH);
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            unsigned char *col = smem + (wn * WTN + j * 32 + l32) * 2 + (wm * WTM + 4 * h) * PITCH;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const f32x4 bv = *(const f32x4 *)&bias_s[wm * WTM + i * 32 + 8 * rq + 4 * h];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp)
+                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                        } else
+                            v = apply_act(v, a.act);
+                        *(uint16_t *)(col + (i * 32 + 8 * rq + rr) * PITCH) = to_bf16(v).bits;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        auto store_runs = [&](auto pxv_c) {
+            constexpr int PXV = decltype(pxv_c)::value;
+            constexpr int RUNS = BN / PXV; // per row
+#pragma unroll 4
+            for (int q = tid; q < BM * RUNS; q += kThreads) {
+                const int row = q / RUNS, cp = q % RUNS;
+                const int n = n0 + cp * PXV, m = m0 + row;
+                const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+                const int pix = n - b * a.OHW;
+                const uint32_t voff = (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
+                const unsigned char *src = smem + row * PITCH + cp * (PXV * 2);
+                if constexpr (PXV == 8)
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
+                else if constexpr (PXV == 4)
+                    __builtin_amdgcn_raw_buffer_store_b64(*(const u32x2 *)src, yr, voff, 0, 0);
+                else
+                    __builtin_amdgcn_raw_buffer_store_b32(*(const uint32_t *)src, yr, voff, 0, 0);
+            }
+        };
+        if (a.pxv == 8)
+            store_runs(std::integral_constant<int, 8>{});
+        else if (a.pxv == 4)
+            store_runs(std::integral_constant<int, 4>{});
+        else
+            store_runs(std::integral_constant<int, 2>{});
+        return;
+    }
     if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
         float *bias_s = (float *)&As[0][0][0];
         if (tid < BM)
@@ -1241,8 +1396,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
 // Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
 template <class T>
 __global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int groups, int cin_g, int khw, const T *__restrict__ w,
-                                                           float *__restrict__ out)
+                                                           float *__restrict__ out, int *__restrict__ zero, int nzero)
 {
+    // side job: clear the tile counters of the stream launch that follows on the stream
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < nzero; i += (int)gridDim.x * 256)
+        zero[i] = 0;
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long total = (long long)groups * p.mtiles * p.nkt * BK * p.BM;
     if (idx >= total)
@@ -1271,8 +1429,10 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(GemmPlan p, int group
 
 // bf16 matrix-instruction path: packed[group][m tile][K tile][m in tile][32 channels of one tap], bf16
 __global__ __launch_bounds__(256) void pack_weights_bf16_kernel(GemmPlan p, int groups, int cin_g, int khw, const bf16_t *__restrict__ w,
-                                                                bf16_t *__restrict__ out)
+                                                                bf16_t *__restrict__ out, int *__restrict__ zero, int nzero)
 {
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < nzero; i += (int)gridDim.x * 256)
+        zero[i] = 0; // as in pack_weights_kernel
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long total = (long long)groups * p.mtiles * p.nkt * p.BM * BK2;
     if (idx >= total)
@@ -1435,20 +1595,31 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     return DLP_OK;
 }
 
+typedef void (*Bf16Kernel)(GemmArgs);
 template <int BM, int BN, int WM, int WN>
-int launch_bf16_mfma(const ConvGeom &g, int order, GemmArgs &a, hipStream_t stream)
+Bf16Kernel bf16_kernel_of_tile(int order, int pxl)
+{
+    if (order == GEMM_ORDER_TAP_BF16 && pxl == 8)
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, 2, 8>;
+    if (order == GEMM_ORDER_TAP_BF16 && pxl == 4)
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, 2, 4>;
+    if (order == GEMM_ORDER_TAP_BF16)
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET, 0>;
+    return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2, 0>;
+}
+Bf16Kernel bf16_kernel(int tile, int order, int pxl)
+{
+    return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl);
+}
+
+int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a, hipStream_t stream)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     {
         TimingScope ts("conv_gemm", stream);
-        if (order == GEMM_ORDER_TAP_BF16)
-            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                               stream, a);
-        else
-            hipLaunchKernelGGL((conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2>), dim3((unsigned)blocks),
-                               dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL(bf16_kernel(p.tile, p.order, pxl), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
@@ -1583,6 +1754,7 @@ int with_tile(int choice, F &&f)
 GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
 {
     GemmPlan p;
+    p.dense_pxl = 0;
     const int cin_g = g.Cin / g.groups;
     p.M = g.Cout / g.groups;
     p.K = cin_g * g.KH * g.KW;
@@ -1605,6 +1777,8 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = tap_major ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
         p.nkt = (p.K + BK2 - 1) / BK2;
         p.tile = p.M > 64 ? 2 : 3;
+        if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.H * g.W) % 4 == 0)
+            p.dense_pxl = (g.H * g.W) % 8 == 0 ? 8 : 4;
     }
     p.BM = 64;
     p.BN = 64;
@@ -1700,7 +1874,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
         const dim3 grid((unsigned)((long long)g.groups * p.mtiles * ncb * (p.BM / 16)));
         if (p.order == GEMM_ORDER_TAP_BF16)
             hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, bf16_t, BK2, true>), grid, dim3(256),
-                               16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked, (int *)nullptr, 0);
+                               16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked, zero, nzero);
         else if (g.dtype == DLP_BFLOAT16)
             hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, float, BK, false>), grid, dim3(256),
                                16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked, (int *)nullptr, 0);
@@ -1709,13 +1883,13 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                                16 * (BK * khw + 1) * sizeof(float), stream, p, ncb, khw, (const float *)w, (float *)wpacked, zero, nzero);
     } else if (bf16_mfma_order(p.order))
         hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
-                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked);
+                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked, zero, nzero);
     else if (g.dtype == DLP_BFLOAT16)
         hipLaunchKernelGGL(pack_weights_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
-                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked);
+                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked, (int *)nullptr, 0);
     else
         hipLaunchKernelGGL(pack_weights_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
-                           g.Cin / g.groups, g.KH * g.KW, (const float *)w, (float *)wpacked);
+                           g.Cin / g.groups, g.KH * g.KW, (const float *)w, (float *)wpacked, zero, nzero);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -1784,8 +1958,15 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         a.part_bytes = (a.splitk > 1 && used < kOutOfRange) ? (uint32_t)used : 0;
     }
 
-    if (bf16_mfma_order(p.order))
-        return p.tile == 2 ? launch_bf16_mfma<128, 128, 2, 2>(g, p.order, a, stream) : launch_bf16_mfma<64, 256, 1, 4>(g, p.order, a, stream);
+    a.pxv = 0;
+    if (bf16_mfma_order(p.order)) {
+        // wide output stores: runs of 8, 4 or 2 pixels that stay inside one image, dword aligned
+        if (ep.factor == 0.0f && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1)
+            a.pxv = a.OHW % 8 == 0 ? 8 : a.OHW % 4 == 0 ? 4 : a.OHW % 2 == 0 ? 2 : 0;
+        // dense loader (1x1, stride 1, no padding): runs of 8 or 4 input pixels, dword aligned
+        const int pxl = ((uintptr_t)x & 3) == 0 ? p.dense_pxl : 0;
+        return launch_bf16_mfma(g, p, pxl, a, stream);
+    }
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)
             return launch_tile<bf16_t, decltype(bm)::value, decltype(bn)::value, decltype(wm)::value, decltype(wn)::value>(g, p, a, act, stream);

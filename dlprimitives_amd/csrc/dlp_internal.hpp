@@ -154,6 +154,7 @@ struct GemmPlan {
     int M, K, nkt;      // per group: rows, reduction length, K tiles of 16
     int mtiles;         // ceil(M / BM)
     int patch;          // 1: stride-1 "same" convolution run by the LDS-patch kernel (tap-major packed weights)
+    int dense_pxl;      // bf16 matrix-instruction path, 1x1 stride 1 pad 0: input pixels per load of the dense loader (8, 4; 0 = gather)
     size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded
 };
 GemmPlan conv_gemm_plan(const ConvGeom &g, int activation);

@@ -40,13 +40,22 @@ CASES = [
     (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),      # split-K path
     (case((3, 5), (1, 2), (2, 3), (3, 2), 3, 8, False, 1, False), (2, 19, 19)),
     (case(3, 1, 1, 1, 8, 8, True, 8, False), (2, 10, 10)),       # depthwise geometry through gemm (channel-major K, one channel per group)
-    # bf16 matrix instruction, pixel-pair loader ("same" stride-1 convolutions with Cin/groups % 32 == 0)
+    # bf16 matrix instruction, tap-major K order (Cin/groups % 32 == 0)
     (case(1, 0, 1, 1, 64, 256, True, 1, True), (5, 7, 7)),       # odd pixel count per image: padded column numbering
     (case(1, 0, 1, 1, 2048, 512, True, 1, True), (3, 7, 7)),     # long K, split over workgroups
     (case(3, 2, 1, 2, 64, 64, True, 1, True), (2, 13, 13)),      # dilated, odd width
     (case(3, 1, 1, 1, 64, 96, False, 2, True), (3, 9, 12)),      # two groups, Cout off the tile sizes
     (case(5, 2, 1, 1, 32, 48, True, 1, False), (2, 9, 9)),       # 25 taps
     (case((3, 1), (1, 0), 1, 1, 32, 32, True, 1, False), (1, 1, 1)),  # a single pixel: both ends of the tensor in one pair
+    # dense loader (1x1, stride 1, no padding, H*W % 4 == 0: wide loads + register transpose) and wide output stores
+    (case(1, 0, 1, 1, 64, 256, True, 1, True), (2, 56, 56)),     # 8-pixel runs, 128x128 tiles, two K tiles
+    (case(1, 0, 1, 1, 1024, 256, True, 1, True), (3, 14, 14)),   # 4-pixel runs, tiles crossing images, pixel tail
+    (case(1, 0, 1, 1, 256, 64, False, 1, False), (3, 14, 14)),   # 4-pixel runs, 64x256 tiles: every wavefront loads every tile
+    (case(1, 0, 1, 1, 64, 80, True, 1, True), (3, 8, 8)),        # Cout off the tile size
+    (case(1, 0, 1, 1, 128, 96, True, 2, False), (3, 6, 6)),      # two groups
+    (case(1, 0, 1, 1, 2048, 512, True, 1, True), (2, 8, 8)),     # long K: split-K slices start in the middle of the loader rotation
+    (case(1, 0, 1, 1, 160, 64, True, 1, True), (5, 4, 10)),      # five K tiles, 8-pixel runs, 64x256 tiles
+    (case(3, 1, 1, 1, 64, 64, True, 1, True), (2, 13, 14)),      # 2-pixel output runs
     # per-pixel loader (strided or size-changing)
     (case(3, 0, 1, 1, 32, 64, True, 1, True), (2, 12, 12)),
     (case(3, 1, 2, 1, 256, 256, True, 1, True), (2, 28, 28)),
@@ -65,6 +74,23 @@ def test_bf16_conv_vs_fp32_reference(oracle_mod, c, bhw):
     # and against the oracle fed the same bf16-rounded operands only the output rounding (2^-9) remains
     want_r = oracle_mod.conv2d_forward(oracle_mod.bf16_round(x), oracle_mod.bf16_round(w), bias, cfg, c["activation"], threads=8)
     np.testing.assert_allclose(got, want_r, rtol=2 ** -8, atol=1e-4 * scale)
+
+
+# ResNet-50 layer shapes at the full batch of configuration 5 (many tiles, images crossing tiles)
+FULL_BATCH_CASES = [
+    (case(1, 0, 1, 1, 128, 128, True, 1, True), (128, 28, 28)),
+    (case(1, 0, 1, 1, 160, 128, True, 1, True), (127, 28, 28)),   # odd number of K tiles, partial last tile
+]
+
+
+@pytest.mark.parametrize("c,bhw", FULL_BATCH_CASES, ids=case_id)
+def test_bf16_full_batch(oracle_mod, c, bhw):
+    x, w, bias = make_tensors(c, bhw, seed=31)
+    x, w = oracle_mod.bf16_round(x), oracle_mod.bf16_round(w)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm")
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8)
+    np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-4 * np.abs(want).max())
 
 
 @pytest.mark.parametrize("cin,cout,bhw", [(64, 64, (2, 56, 56)), (24, 40, (3, 13, 9)), (128, 128, (4, 28, 28)), (512, 512, (3, 7, 7))])
