@@ -110,7 +110,16 @@ def kernel_class(L, bf16=False):
     small = L["kernel"] ** 2 <= 31
     if bf16 and L["activation"] not in ("tanh", "sigmoid"):
         order = 2 if (small and cin_g % 32 == 0) else 3  # one tap x 32 channels per K tile, or the per-element table
-        return "conv_gemm_bf16_kernel<%s, %d, 0, 2>" % ("128, 128, 2, 2" if m > 64 else "64, 256, 1, 4", order)
+        tile = "128, 128, 2, 2" if m > 64 else "64, 256, 1, 4"
+        hw = L["hw"] * L["hw"]
+        same3 = L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
+        if order == 2 and same3 and hw % 4 == 0 and hw >= (128 if m > 64 else 254):
+            # stride-1 3x3: input patch through LDS (the library falls back to the gather when the patch does not fit)
+            return "conv_patch_bf16_kernel<%s, %d, %d, 0>" % (tile, 320 if m > 64 else 448, 8 if hw % 8 == 0 else 4)
+        pxl = 0
+        if order == 2 and L["kernel"] == 1 and L["stride"] == 1 and L["pad"] == 0 and hw % 4 == 0:
+            pxl = 8 if hw % 8 == 0 else 4  # dense loader: 8 or 4 pixels per load
+        return "conv_gemm_bf16_kernel<%s, %d, 0, 2, %d>" % (tile, order, pxl)
     tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     order = 1 if (small and cin_g % 16 == 0) else 0
     if (not bf16 and order == 1 and m > 32 and L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
@@ -121,7 +130,7 @@ def kernel_class(L, bf16=False):
 
 
 def matrix_peak_tflops(kernel_name):
-    return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith("conv_gemm_bf16_kernel") else FP32_MATRIX_PEAK_TFLOPS
+    return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith(("conv_gemm_bf16_kernel", "conv_patch_bf16_kernel")) else FP32_MATRIX_PEAK_TFLOPS
 
 
 MAIN_SECTION = {"gemm": "conv_gemm", "winograd": "winograd_fused", "depthwise_separable": "sep_conv"}

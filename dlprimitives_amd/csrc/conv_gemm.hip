@@ -52,6 +52,8 @@ constexpr int kThreads = 256;
 constexpr int BK = 16;
 constexpr uint32_t kOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
 constexpr int kPatchPitch = 192;               // LDS patch rows of conv_patch_f32_kernel
+constexpr int kPatchPitchBf16_128 = 320;       // ... of conv_patch_bf16_kernel with 128-pixel tiles
+constexpr int kPatchPitchBf16_256 = 448;       // ... with 256-pixel tiles
 
 enum { ACT_CLAMP = 0, ACT_GENERIC = 1 };
 
@@ -73,7 +75,8 @@ struct GemmArgs {
 #endif
     int *sk_cnt;              // pieces arrived, per tile (zero at launch)
     int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
-    int pxv;                  // bf16 matrix-instruction kernel: pixels per output store (0 = one element per store)
+    int pxv;                  // bf16 matrix-instruction kernels: pixels per output store (0 = one element per store)
+    int pp_nbr;               // conv_patch_bf16_kernel: blocks of PXP rows in the largest patch of the launch
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -854,8 +857,191 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 #ifndef DLP_BF16_NSET
 #define DLP_BF16_NSET 2
 #endif
+#ifndef DLP_DENSE_NSET
+#define DLP_DENSE_NSET 2
+#endif
 constexpr int BK2 = 32;
 constexpr int LDK = BK2 + 8;
+
+// What a workgroup of the bf16 kernels does with its finished accumulator tile: the split-K partial
+// store, or the epilogue (bias, activation, factor) and the store to y.  `smem` is the kernel's LDS
+// (at least BM * (BN * 2 + 16) + BM * 4 bytes), free after the last barrier of the main loop.
+template <int BM, int BN, int WM, int WN, int ACT>
+__device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], unsigned char *smem, int smem_bytes,
+                                                 int m0, int n0, int g, int slice, int wm, int wn, int h, int l32, int tid)
+{
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    if (a.splitk > 1) {
+        if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
+            const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + wn * WTN + j * 32 + l32;
+                const uint32_t voff =
+                    n < a.N ? (uint32_t)((slice * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.N + n) * 4u : kOutOfRange;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int mrow = i * 32 + 8 * (r >> 2) + (r & 3);
+                        const float v = acc[i][j][r]; // a copy: bit_cast of a vector element reads element 0
+                        if (m0 + wm * WTM + mrow < a.M)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, voff, (uint32_t)(mrow * a.N) * 4u, 0);
+                    }
+            }
+            return;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            if (n >= a.N)
+                continue;
+            float *pb = a.part + ((size_t)slice * a.Cout + (size_t)g * a.M) * a.N + n;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < a.M)
+                        pb[(size_t)m * a.N] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- epilogue.  Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the
+    // tile's rows goes through LDS (free after the last barrier), the result is rounded by the
+    // hardware conversion and stored with buffer stores whose row offset is scalar: a handful of
+    // VALU operations per value instead of 64-bit address arithmetic and a bias load each. ----
+    // Wide stores (a.pxv = 2, 4 or 8 pixels per store; the host sets it when there is no factor, y is
+    // 4-byte aligned and below 2 GiB, and pxv divides OH*OW): the tile goes to LDS as bf16 [m][n]
+    // (rows padded by 16 bytes: the two half-waves, four rows apart, hit different banks) and is
+    // stored to y in runs of pxv pixels per lane, consecutive lanes on consecutive runs of a row --
+    // a store instruction costs the same whatever its width, so this is pxv times fewer of them.
+    if (a.pxv != 0) {
+        constexpr int PITCH = BN * 2 + 16;
+        (void)smem_bytes; // the callers check BM * PITCH + BM * 4 <= their LDS
+        float *bias_s = (float *)(smem + BM * PITCH);
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            unsigned char *col = smem + (wn * WTN + j * 32 + l32) * 2 + (wm * WTM + 4 * h) * PITCH;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const f32x4 bv = *(const f32x4 *)&bias_s[wm * WTM + i * 32 + 8 * rq + 4 * h];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp)
+                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                        } else
+                            v = apply_act(v, a.act);
+                        *(uint16_t *)(col + (i * 32 + 8 * rq + rr) * PITCH) = to_bf16(v).bits;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        auto store_runs = [&](auto pxv_c) {
+            constexpr int PXV = decltype(pxv_c)::value;
+            constexpr int RUNS = BN / PXV; // per row
+#pragma unroll 4
+            for (int q = tid; q < BM * RUNS; q += kThreads) {
+                const int row = q / RUNS, cp = q % RUNS;
+                const int n = n0 + cp * PXV, m = m0 + row;
+                const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+                const int pix = n - b * a.OHW;
+                const uint32_t voff = (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
+                const unsigned char *src = smem + row * PITCH + cp * (PXV * 2);
+                if constexpr (PXV == 8)
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
+                else if constexpr (PXV == 4)
+                    __builtin_amdgcn_raw_buffer_store_b64(*(const u32x2 *)src, yr, voff, 0, 0);
+                else
+                    __builtin_amdgcn_raw_buffer_store_b32(*(const uint32_t *)src, yr, voff, 0, 0);
+            }
+        };
+        if (a.pxv == 8)
+            store_runs(std::integral_constant<int, 8>{});
+        else if (a.pxv == 4)
+            store_runs(std::integral_constant<int, 4>{});
+        else
+            store_runs(std::integral_constant<int, 2>{});
+        return;
+    }
+    if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
+        float *bias_s = (float *)smem;
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WTN + j * 32 + l32;
+            const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+            const int pix = n - b * a.OHW;
+            const uint32_t voff = n < a.N ? (uint32_t)(((b * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.OHW + pix) * 2) : kOutOfRange;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int mrow = wm * WTM + i * 32 + 8 * rq; // + 4*h + (r & 3); uniform part
+                    if (m0 + mrow >= a.M)
+                        continue;
+                    const f32x4 bv = *(const f32x4 *)&bias_s[mrow + 4 * h];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp)
+                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                        } else
+                            v = apply_act(v, a.act);
+                        __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * 2), 0);
+                    }
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + l32;
+        if (n >= a.N)
+            continue;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * a.OHW;
+        bf16_t *yb = (bf16_t *)a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < a.M) {
+                    float v = acc[i][j][r];
+                    if (a.bias)
+                        v += a.bias[g * a.M + m];
+                    if (ACT == ACT_CLAMP) {
+                        if (a.act != DLP_ACT_IDENTITY)
+                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                    } else
+                        v = apply_act(v, a.act);
+                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
+                }
+            }
+        }
+    }
+}
 
 // PXL > 0 selects the dense loader (1x1, stride 1, no padding: a plain GEMM W * X per image):
 // a lane loads PXL consecutive pixels of 8 consecutive channels with 8- or 16-byte loads (the
@@ -869,7 +1055,7 @@ constexpr int LDK = BK2 + 8;
 template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
-    static_assert(PXL == 0 || ((PXL == 4 || PXL == 8) && ORDER == GEMM_ORDER_TAP_BF16 && NSET == 2), "dense loader variants");
+    static_assert(PXL == 0 || ((PXL == 4 || PXL == 8) && ORDER == GEMM_ORDER_TAP_BF16), "dense loader variants");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -961,7 +1147,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     constexpr int PXN = PXL ? PXL : 1;
     constexpr int NPQ = BN / PXN;                  // pixel groups of a tile
     constexpr int LW = PXL ? 4 * NPQ / 64 : 4;     // wavefronts that load one B tile
-    constexpr int NSETB = (LW == 4) ? 2 : 1;       // a wavefront that loads every 4/LW-th tile needs one register set
+    constexpr int NSETB = NSET * LW / 4 ? NSET * LW / 4 : 1; // a wavefront loads every 4/LW-th tile: that many fewer register sets
     constexpr int DW = PXL ? PXL / 2 : 1;          // dwords per load
     static_assert(LW == 1 || LW == 2 || LW == 4, "loader wavefronts");
     uint32_t dvoff = kOutOfRange; // byte offset of (first channel of the block, first pixel) in x
@@ -991,7 +1177,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     }
     auto my_tile = [&](int kt) { return LW == 4 || (kt & (4 / LW - 1)) == my_turn; };
     auto load_b = [&](auto set, int kt) {
-        constexpr int S = decltype(set)::value % NSETB;
+        constexpr int S = (decltype(set)::value * LW / 4) % NSETB;
         const uint32_t soff = (uint32_t)(min(kt, a.nkt - 1) * BK2) * a.hw4;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -1009,7 +1195,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         }
     };
     auto store_b = [&](auto set, auto buf_c) {
-        constexpr int S = decltype(set)::value % NSETB;
+        constexpr int S = (decltype(set)::value * LW / 4) % NSETB;
         constexpr int BUF = decltype(buf_c)::value;
 #pragma unroll
         for (int q = 0; q < PXN; q++) {
@@ -1176,175 +1362,259 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             k_step(I2{}, kt + 2);
     }
 
-    if (a.splitk > 1) {
-        if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
-            const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int n = n0 + wn * WTN + j * 32 + l32;
-                const uint32_t voff =
-                    n < a.N ? (uint32_t)((slice * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.N + n) * 4u : kOutOfRange;
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int mrow = i * 32 + 8 * (r >> 2) + (r & 3);
-                        const float v = acc[i][j][r]; // a copy: bit_cast of a vector element reads element 0
-                        if (m0 + wm * WTM + mrow < a.M)
-                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, voff, (uint32_t)(mrow * a.N) * 4u, 0);
-                    }
-            }
-            return;
-        }
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + wn * WTN + j * 32 + l32;
-            if (n >= a.N)
-                continue;
-            float *pb = a.part + ((size_t)slice * a.Cout + (size_t)g * a.M) * a.N + n;
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < a.M)
-                        pb[(size_t)m * a.N] = acc[i][j][r];
-                }
-            }
-        }
-        return;
-    }
+    static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
+    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, slice, wm, wn, h, l32, tid);
+}
 
-    // ---- epilogue.  Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the
-    // tile's rows goes through LDS (free after the last barrier), the result is rounded by the
-    // hardware conversion and stored with buffer stores whose row offset is scalar: a handful of
-    // VALU operations per value instead of 64-bit address arithmetic and a bias load each. ----
-    // Wide stores (a.pxv = 2, 4 or 8 pixels per store; the host sets it when there is no factor, y is
-    // 4-byte aligned and below 2 GiB, and pxv divides OH*OW): the tile goes to LDS as bf16 [m][n]
-    // (rows padded by 16 bytes: the two half-waves, four rows apart, hit different banks) and is
-    // stored to y in runs of pxv pixels per lane, consecutive lanes on consecutive runs of a row --
-    // a store instruction costs the same whatever its width, so this is pxv times fewer of them.
-    if (a.pxv != 0) {
-        constexpr int PITCH = BN * 2 + 16;
-        static_assert(BM * PITCH + BM * 4 <= 2 * A_TILE_BYTES + 2 * B_TILE_BYTES, "the staged tile fits the operand buffers");
-        float *bias_s = (float *)(smem + BM * PITCH);
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
-        const bool clamp = a.act != DLP_ACT_IDENTITY;
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            unsigned char *col = smem + (wn * WTN + j * 32 + l32) * 2 + (wm * WTM + 4 * h) * PITCH;
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const f32x4 bv = *(const f32x4 *)&bias_s[wm * WTM + i * 32 + 8 * rq + 4 * h];
-#pragma unroll
-                    for (int rr = 0; rr < 4; rr++) {
-                        float v = acc[i][j][4 * rq + rr] + bv[rr];
-                        if (ACT == ACT_CLAMP) {
-                            if (clamp)
-                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
-                        } else
-                            v = apply_act(v, a.act);
-                        *(uint16_t *)(col + (i * 32 + 8 * rq + rr) * PITCH) = to_bf16(v).bits;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
-        auto store_runs = [&](auto pxv_c) {
-            constexpr int PXV = decltype(pxv_c)::value;
-            constexpr int RUNS = BN / PXV; // per row
-#pragma unroll 4
-            for (int q = tid; q < BM * RUNS; q += kThreads) {
-                const int row = q / RUNS, cp = q % RUNS;
-                const int n = n0 + cp * PXV, m = m0 + row;
-                const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
-                const int pix = n - b * a.OHW;
-                const uint32_t voff = (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
-                const unsigned char *src = smem + row * PITCH + cp * (PXV * 2);
-                if constexpr (PXV == 8)
-                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
-                else if constexpr (PXV == 4)
-                    __builtin_amdgcn_raw_buffer_store_b64(*(const u32x2 *)src, yr, voff, 0, 0);
-                else
-                    __builtin_amdgcn_raw_buffer_store_b32(*(const uint32_t *)src, yr, voff, 0, 0);
-            }
-        };
-        if (a.pxv == 8)
-            store_runs(std::integral_constant<int, 8>{});
-        else if (a.pxv == 4)
-            store_runs(std::integral_constant<int, 4>{});
-        else
-            store_runs(std::integral_constant<int, 2>{});
-        return;
+// ---- stride-1 3x3 "same" convolutions on the bf16 matrix instruction: the input patch goes through LDS once ----
+// The bf16 counterpart of conv_patch_f32_kernel.  A K stage = 32 input channels: the pixels that the
+// nine taps of the tile's BN output pixels read -- one run of consecutive plane pixels per image the
+// tile touches, BN + 2*(W+1) in all -- are loaded once per stage with 8- or 16-byte loads (PXP pixels
+// of 8 channels per lane), transposed in registers like the dense loader's blocks, and kept in LDS as
+// [8-channel group][patch row][8 channels] with the row index XOR-swizzled.  The B operand of tap
+// (ky,kx) is then a 16-byte LDS read at (lane's patch row + (ky-1)*W + (kx-1)); taps that fall into
+// the padding read a row that is always zero.  Compared with gathering every tap from memory with
+// 16-bit loads this is 9 * 8 times fewer trips through the texture path, which is what bounds that
+// kernel.  Runs start on multiples of PXP pixels of their plane (H*W % PXP == 0), so every load is
+// dword aligned.  Weights: the packed tap-major tiles of conv_gemm_bf16_kernel (K tile = stage * 9 + tap).
+template <int BM, int BN, int WM, int WN, int PITCH, int PXP, int ACT>
+__global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
+{
+    constexpr int KHW = 9;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_V4 = BM * BK2 * 2 / 16; // 16-byte pieces of a packed A tile
+    static_assert(A_V4 % kThreads == 0, "A loader shape");
+    constexpr int A_LD = A_V4 / kThreads;
+    constexpr int A_TILE_BYTES = BM * LDK * 2;
+    constexpr int P_BUF_BYTES = 4 * PITCH * 16;
+    constexpr int MAXSEG = 3;           // images a tile may touch (H*W >= BN / 2 + 1 is checked by the host)
+    constexpr int DW = PXP / 2;         // dwords per load
+    constexpr int ZERO_ROW = PITCH - 1; // its aligned group of 8 rows is never loaded
+    static_assert(PITCH % 8 == 0 && (PXP == 4 || PXP == 8), "patch shape");
+
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * A_TILE_BYTES + 2 * P_BUF_BYTES];
+    auto As = reinterpret_cast<uint16_t(*)[BM][LDK]>(smem);
+    unsigned char *const ps_bytes = smem + 2 * A_TILE_BYTES;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+
+    int t; // XCD-aware renumbering, as in the other kernels
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, r = nb & 7;
+        const int xcd = bid & 7, slot = bid >> 3;
+        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
     }
-    if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
-        float *bias_s = (float *)&As[0][0][0];
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
-        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
-        const bool clamp = a.act != DLP_ACT_IDENTITY;
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    const int g = t / a.ntiles;
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int ncb = a.nkt / KHW; // stages
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
+    auto swz = [](int row) { return row ^ ((row >> 3) & 7); };
+
+    // ---- the tile's patch: one segment of consecutive plane pixels per image, PXP-aligned at both ends ----
+    const int HW = a.OHW;
+    const int halo = a.W + 1;
+    const int n_last = min(n0 + BN, a.N) - 1;
+    const int b0 = (int)fast_div((uint32_t)n0, a.ohw_magic, a.ohw_shift);
+    int seg_row[MAXSEG], seg_a[MAXSEG], seg_len[MAXSEG];
+    {
+        int row = 0;
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + wn * WTN + j * 32 + l32;
-            const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
-            const int pix = n - b * a.OHW;
-            const uint32_t voff = n < a.N ? (uint32_t)(((b * a.Cout + g * a.M + m0 + wm * WTM + 4 * h) * a.OHW + pix) * 2) : kOutOfRange;
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int mrow = wm * WTM + i * 32 + 8 * rq; // + 4*h + (r & 3); uniform part
-                    if (m0 + mrow >= a.M)
-                        continue;
-                    const f32x4 bv = *(const f32x4 *)&bias_s[mrow + 4 * h];
-#pragma unroll
-                    for (int rr = 0; rr < 4; rr++) {
-                        float v = acc[i][j][4 * rq + rr] + bv[rr];
-                        if (ACT == ACT_CLAMP) {
-                            if (clamp)
-                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
-                        } else
-                            v = apply_act(v, a.act);
-                        __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * 2), 0);
-                    }
-                }
+        for (int s = 0; s < MAXSEG; s++) {
+            const int base = (b0 + s) * HW;
+            const int first = max(n0, base), last = min(n_last, base + HW - 1);
+            int as = 0, len = 0;
+            if (first <= last) {
+                as = max(0, first - base - halo) & ~(PXP - 1);
+                len = ((min(HW, last - base + 1 + halo) + PXP - 1) & ~(PXP - 1)) - as;
             }
+            seg_row[s] = row;
+            seg_a[s] = as;
+            seg_len[s] = len;
+            row += len;
         }
-        return;
     }
+    // loader: this lane's block = 8 channels (group oct) x patch rows [rho0, rho0 + PXP)
+    const int nbr = a.pp_nbr; // row blocks of the largest patch of this launch
+    const bool loader = tid < 4 * nbr;
+    const int oct = tid / nbr, rho0 = (tid - oct * nbr) * PXP;
+    uint32_t pvoff = kOutOfRange;
+    uint32_t dslot[PXP];
+    if (loader) {
+#pragma unroll
+        for (int s = 0; s < MAXSEG; s++) {
+            const int d = rho0 - seg_row[s];
+            if (d >= 0 && d < seg_len[s])
+                pvoff = (uint32_t)((b0 + s) * a.Cin + g * a.Cin_g + oct * 8) * a.hw4 + (uint32_t)(seg_a[s] + d) * 2u;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < PXP; q++)
+        dslot[q] = (uint32_t)(((oct & 3) * PITCH + swz(rho0 + q)) * 16);
+    // this lane's B operands (channel group h of a k step, pixel l32 of block j) per tap: byte offset in a patch buffer
+    uint32_t baddr[TN][KHW];
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int n = n0 + wn * WTN + j * 32 + l32;
-        if (n >= a.N)
-            continue;
+        const bool vn = n < a.N;
         const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
-        const int pix = n - b * a.OHW;
-        bf16_t *yb = (bf16_t *)a.y + ((size_t)b * a.Cout + (size_t)g * a.M) * a.OHW + pix;
+        const int pix = n - b * HW;
+        const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+        const int ox = pix - oy * a.OW;
+        const int s = b - b0;
+        const int row = pix + (s == 0 ? seg_row[0] - seg_a[0] : s == 1 ? seg_row[1] - seg_a[1] : seg_row[2] - seg_a[2]);
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
+        for (int ky = 0; ky < 3; ky++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (m < a.M) {
-                    float v = acc[i][j][r];
-                    if (a.bias)
-                        v += a.bias[g * a.M + m];
-                    if (ACT == ACT_CLAMP) {
-                        if (a.act != DLP_ACT_IDENTITY)
-                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
-                    } else
-                        v = apply_act(v, a.act);
-                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
-                }
+            for (int kx = 0; kx < 3; kx++) {
+                const int yy = oy + ky - 1, xx = ox + kx - 1;
+                const bool ok = vn && yy >= 0 && yy < a.H && xx >= 0 && xx < a.W;
+                const int r = ok ? row + (ky - 1) * a.W + (kx - 1) : ZERO_ROW;
+                baddr[j][ky * 3 + kx] = (uint32_t)((h * PITCH + swz(r)) * 16);
+            }
+    }
+    if (tid < 8) { // the zero row of both buffers, all four channel groups
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        *(u32x4 *)(ps_bytes + (tid >> 2) * P_BUF_BYTES + ((tid & 3) * PITCH + swz(ZERO_ROW)) * 16) = z;
+    }
+
+    const uint32_t a_tile_bytes = BM * BK2 * 2;
+    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
+    u32x4 ra[2][A_LD];
+    uint32_t rbw[8][DW];
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    auto load_a = [&](auto set, int kt) {
+        constexpr int S = decltype(set)::value;
+        const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
+#pragma unroll
+        for (int j = 0; j < A_LD; j++)
+            ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
+    };
+    auto store_a = [&](auto set, auto buf_c) {
+        constexpr int S = decltype(set)::value;
+        constexpr int BUF = decltype(buf_c)::value;
+#pragma unroll
+        for (int j = 0; j < A_LD; j++) {
+            const int idx = tid + j * kThreads;
+            *(u32x4 *)&As[BUF][idx >> 2][(idx & 3) * 8] = ra[S][j];
+        }
+    };
+    auto load_patch = [&](int cb) {
+        if (!loader)
+            return;
+        const uint32_t soff = (uint32_t)(cb * BK2) * a.hw4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if constexpr (PXP == 8) {
+                const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, pvoff, soff + (uint32_t)i * a.hw4, 0));
+#pragma unroll
+                for (int d = 0; d < DW; d++)
+                    rbw[i][d] = v[d];
+            } else {
+                const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(xr, pvoff, soff + (uint32_t)i * a.hw4, 0));
+#pragma unroll
+                for (int d = 0; d < DW; d++)
+                    rbw[i][d] = v[d];
             }
         }
+    };
+    auto store_patch = [&](auto buf_c) {
+        constexpr int PB = decltype(buf_c)::value;
+        if (!loader)
+            return;
+#pragma unroll
+        for (int q = 0; q < PXP; q++) {
+            u32x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; j++) // channels 2j (low half) and 2j+1 of patch row rho0 + q
+                v[j] = __builtin_amdgcn_perm(rbw[2 * j + 1][q / 2], rbw[2 * j][q / 2], (q & 1) ? 0x07060302u : 0x05040100u);
+            *(u32x4 *)(ps_bytes + PB * P_BUF_BYTES + dslot[q]) = v;
+        }
+    };
+
+    // One stage: nine K tiles (taps) on patch buffer P.  The patch of the next stage is requested during
+    // the first tap and goes to the other buffer during the last one; the A tiles run through two
+    // register sets and two LDS buffers as in conv_gemm_bf16_kernel (tile kt+1 stored, tile kt+3
+    // requested while tile kt is multiplied); one barrier per K tile.
+    auto stage = [&](auto par, int cb) {
+        constexpr int P = decltype(par)::value;
+        using OtherP = std::integral_constant<int, P ^ 1>;
+        const bool has_next = cb + 1 < ncb;
+        static_for_n<KHW>([&](auto tau_c) {
+            constexpr int TAU = decltype(tau_c)::value;
+            constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2
+            constexpr int BUF = IDX & 1;
+            using NextBuf = std::integral_constant<int, BUF ^ 1>;
+            using Set = std::integral_constant<int, (IDX + 1) & 1>;
+            const int kt = cb * KHW + TAU;
+            bf16x8 fa[2][TM], fb[2][TN];
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+                    fa[s][i] = *(const bf16x8 *)&As[BUF][wm * WTM + i * 32 + l32][s * 16 + h * 8];
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    fb[s][j] = *(const bf16x8 *)(ps_bytes + P * P_BUF_BYTES + baddr[j][TAU] + s * (2 * PITCH * 16));
+            }
+            store_a(Set{}, NextBuf{});
+            load_a(Set{}, kt + 3);
+            if (TAU == 0 && has_next)
+                load_patch(cb + 1);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+            if (TAU == KHW - 1 && has_next)
+                store_patch(OtherP{});
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+            __syncthreads();
+        });
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    load_patch(0);
+    load_a(I0{}, 0);
+    load_a(I1{}, 1);
+    store_patch(I0{});
+    store_a(I0{}, I0{});
+    load_a(I0{}, 2);
+    __syncthreads();
+    int cb = 0;
+    for (; cb + 1 < ncb; cb += 2) {
+        stage(I0{}, cb);
+        stage(I1{}, cb + 1);
     }
+    if (cb < ncb)
+        stage(I0{}, cb);
+
+    static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
+    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
 }
 
 // Sums the split-K slices in slice order (deterministic) and applies the epilogue.
@@ -1600,9 +1870,9 @@ template <int BM, int BN, int WM, int WN>
 Bf16Kernel bf16_kernel_of_tile(int order, int pxl)
 {
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 8)
-        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, 2, 8>;
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 8>;
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 4)
-        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, 2, 4>;
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 4>;
     if (order == GEMM_ORDER_TAP_BF16)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET, 0>;
     return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2, 0>;
@@ -1610,6 +1880,65 @@ Bf16Kernel bf16_kernel_of_tile(int order, int pxl)
 Bf16Kernel bf16_kernel(int tile, int order, int pxl)
 {
     return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl);
+}
+
+// Largest number of patch rows any pixel tile of conv_patch_bf16_kernel needs (same arithmetic as the kernel).
+int bf16_patch_rows(const ConvGeom &g, int BN, int pxp)
+{
+    const long long N = (long long)g.B * g.OH * g.OW;
+    const int HW = g.OH * g.OW, halo = g.W + 1;
+    const long long ntiles = (N + BN - 1) / BN;
+    int most = 0;
+    // the offset of a tile inside its image repeats after HW / gcd(BN, HW) tiles; the last tile may be short
+    long long period = HW;
+    for (long long x = BN, y = HW; y != 0;) {
+        const long long r = x % y;
+        x = y;
+        y = r;
+        period = HW / x;
+    }
+    for (long long i = 0; i < std::min(ntiles, period + 1); i++) {
+        const long long nt = i < period ? i : ntiles - 1;
+        const long long n0 = nt * BN, n_last = std::min(n0 + BN, N) - 1;
+        const long long b0 = n0 / HW;
+        int rows = 0;
+        for (int s = 0; s < 3; s++) {
+            const long long base = (b0 + s) * HW;
+            const long long first = std::max(n0, base), last = std::min(n_last, base + HW - 1);
+            if (first <= last) {
+                const int as = (int)std::max<long long>(0, first - base - halo) & ~(pxp - 1);
+                rows += (((int)std::min<long long>(HW, last - base + 1 + halo) + pxp - 1) & ~(pxp - 1)) - as;
+            }
+        }
+        most = std::max(most, rows);
+    }
+    return most;
+}
+
+int launch_patch_bf16(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t stream)
+{
+    a.mtiles = p.mtiles;
+    a.ntiles = (a.N + p.BN - 1) / p.BN;
+    a.splitk = 1;
+    a.kt_per_slice = a.nkt;
+    a.part = nullptr;
+    a.part_bytes = 0;
+    a.pp_nbr = p.pp_nbr;
+    const long long blocks = (long long)a.mtiles * a.ntiles * g.groups;
+    if (blocks > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    TimingScope ts("conv_gemm", stream);
+    const dim3 grid((unsigned)blocks), block(kThreads);
+    if (p.tile == 2 && p.patch_bf16 == 8)
+        hipLaunchKernelGGL((conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+    else if (p.tile == 2)
+        hipLaunchKernelGGL((conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+    else if (p.patch_bf16 == 8)
+        hipLaunchKernelGGL((conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
 }
 
 int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a, hipStream_t stream)
@@ -1755,6 +2084,8 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
 {
     GemmPlan p;
     p.dense_pxl = 0;
+    p.patch_bf16 = 0;
+    p.pp_nbr = 0;
     const int cin_g = g.Cin / g.groups;
     p.M = g.Cout / g.groups;
     p.K = cin_g * g.KH * g.KW;
@@ -1779,6 +2110,17 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.tile = p.M > 64 ? 2 : 3;
         if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.H * g.W) % 4 == 0)
             p.dense_pxl = (g.H * g.W) % 8 == 0 ? 8 : 4;
+        // stride-1 3x3 "same" convolutions whose largest patch fits the LDS rows and one block per lane: LDS-patch kernel
+        if (tap_major && g.KH == 3 && g.KW == 3 && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 &&
+            (g.H * g.W) % 4 == 0 && g.B > 0) {
+            const int pxp = (g.H * g.W) % 8 == 0 ? 8 : 4;
+            const int BN = p.tile == 2 ? 128 : 256, pitch = p.tile == 2 ? kPatchPitchBf16_128 : kPatchPitchBf16_256;
+            const int rows = bf16_patch_rows(g, BN, pxp), nbr = (rows + pxp - 1) / pxp;
+            if ((BN - 2) / (g.H * g.W) + 2 <= 3 && nbr * pxp <= pitch - 8 && 4 * nbr <= kThreads) {
+                p.patch_bf16 = pxp;
+                p.pp_nbr = nbr;
+            }
+        }
     }
     p.BM = 64;
     p.BN = 64;
@@ -1964,6 +2306,8 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         if (ep.factor == 0.0f && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1)
             a.pxv = a.OHW % 8 == 0 ? 8 : a.OHW % 4 == 0 ? 4 : a.OHW % 2 == 0 ? 2 : 0;
         // dense loader (1x1, stride 1, no padding): runs of 8 or 4 input pixels, dword aligned
+        if (p.patch_bf16 && ((uintptr_t)x & 3) == 0)
+            return launch_patch_bf16(g, p, a, stream);
         const int pxl = ((uintptr_t)x & 3) == 0 ? p.dense_pxl : 0;
         return launch_bf16_mfma(g, p, pxl, a, stream);
     }

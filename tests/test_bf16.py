@@ -56,6 +56,14 @@ CASES = [
     (case(1, 0, 1, 1, 2048, 512, True, 1, True), (2, 8, 8)),     # long K: split-K slices start in the middle of the loader rotation
     (case(1, 0, 1, 1, 160, 64, True, 1, True), (5, 4, 10)),      # five K tiles, 8-pixel runs, 64x256 tiles
     (case(3, 1, 1, 1, 64, 64, True, 1, True), (2, 13, 14)),      # 2-pixel output runs
+    # LDS-patch kernel (stride-1 3x3 "same", H*W % 4 == 0): the tile's input patch is loaded once per 32 channels
+    (case(3, 1, 1, 1, 128, 128, True, 1, True), (3, 28, 28)),    # 128-pixel tiles, 8-pixel loads, pixel tail
+    (case(3, 1, 1, 1, 256, 256, True, 1, True), (5, 14, 14)),    # 4-pixel loads, tiles crossing an image boundary
+    (case(3, 1, 1, 1, 64, 64, False, 1, False), (4, 14, 14)),    # 256-pixel tiles over three images
+    (case(3, 1, 1, 1, 96, 128, True, 1, True), (2, 16, 16)),     # three stages (odd)
+    (case(3, 1, 1, 1, 64, 256, True, 2, True), (2, 12, 12)),     # two groups of 32 channels: a single stage
+    (case(3, 1, 1, 1, 32, 128, True, 1, True), (5, 8, 8)),       # images smaller than a tile: three segments
+    (case(3, 1, 1, 1, 64, 64, True, 1, True), (1, 4, 60)),       # wide, flat image
     # per-pixel loader (strided or size-changing)
     (case(3, 0, 1, 1, 32, 64, True, 1, True), (2, 12, 12)),
     (case(3, 1, 2, 1, 256, 256, True, 1, True), (2, 28, 28)),
@@ -80,6 +88,8 @@ def test_bf16_conv_vs_fp32_reference(oracle_mod, c, bhw):
 FULL_BATCH_CASES = [
     (case(1, 0, 1, 1, 128, 128, True, 1, True), (128, 28, 28)),
     (case(1, 0, 1, 1, 160, 128, True, 1, True), (127, 28, 28)),   # odd number of K tiles, partial last tile
+    (case(3, 1, 1, 1, 128, 128, True, 1, True), (64, 28, 28)),    # LDS-patch kernel, 392 tiles
+    (case(3, 1, 1, 1, 64, 64, True, 1, True), (8, 56, 56)),       # LDS-patch kernel, 256-pixel tiles
 ]
 
 
