@@ -1366,14 +1366,18 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, slice, wm, wn, h, l32, tid);
 }
 
+#ifndef DLP_PATCH_BF16_NA
+#define DLP_PATCH_BF16_NA 3
+#endif
 // ---- stride-1 3x3 "same" convolutions on the bf16 matrix instruction: the input patch goes through LDS once ----
 // The bf16 counterpart of conv_patch_f32_kernel.  A K stage = 32 input channels: the pixels that the
 // nine taps of the tile's BN output pixels read -- one run of consecutive plane pixels per image the
 // tile touches, BN + 2*(W+1) in all -- are loaded once per stage with 8- or 16-byte loads (PXP pixels
 // of 8 channels per lane), transposed in registers like the dense loader's blocks, and kept in LDS as
-// [8-channel group][patch row][8 channels] with the row index XOR-swizzled.  The B operand of tap
-// (ky,kx) is then a 16-byte LDS read at (lane's patch row + (ky-1)*W + (kx-1)); taps that fall into
-// the padding read a row that is always zero.  Compared with gathering every tap from memory with
+// [8-channel group][patch row][8 channels] (rows in order: the reads of consecutive lanes are then
+// consecutive 16-byte pieces whatever the tap's shift, free of bank conflicts; the few stores per
+// stage, 8 rows apart across lanes, are not).  The B operand of tap (ky,kx) is a 16-byte LDS read at
+// (lane's patch row + (ky-1)*W + (kx-1)); taps that fall into the padding read a row that is always zero.  Compared with gathering every tap from memory with
 // 16-bit loads this is 9 * 8 times fewer trips through the texture path, which is what bounds that
 // kernel.  Runs start on multiples of PXP pixels of their plane (H*W % PXP == 0), so every load is
 // dword aligned.  Weights: the packed tap-major tiles of conv_gemm_bf16_kernel (K tile = stage * 9 + tap).
@@ -1392,6 +1396,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     constexpr int DW = PXP / 2;         // dwords per load
     constexpr int ZERO_ROW = PITCH - 1; // its aligned group of 8 rows is never loaded
     static_assert(PITCH % 8 == 0 && (PXP == 4 || PXP == 8), "patch shape");
+    constexpr int NA = DLP_PATCH_BF16_NA; // register sets of A tiles
+    static_assert((2 * KHW) % NA == 0, "the A register sets rotate with a period that divides a pair of stages");
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * A_TILE_BYTES + 2 * P_BUF_BYTES];
     auto As = reinterpret_cast<uint16_t(*)[BM][LDK]>(smem);
@@ -1420,7 +1426,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
-    auto swz = [](int row) { return row ^ ((row >> 3) & 7); };
 
     // ---- the tile's patch: one segment of consecutive plane pixels per image, PXP-aligned at both ends ----
     const int HW = a.OHW;
@@ -1461,7 +1466,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     }
 #pragma unroll
     for (int q = 0; q < PXP; q++)
-        dslot[q] = (uint32_t)(((oct & 3) * PITCH + swz(rho0 + q)) * 16);
+        dslot[q] = (uint32_t)(((oct & 3) * PITCH + rho0 + q) * 16);
     // this lane's B operands (channel group h of a k step, pixel l32 of block j) per tap: byte offset in a patch buffer
     uint32_t baddr[TN][KHW];
 #pragma unroll
@@ -1481,17 +1486,17 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
                 const int yy = oy + ky - 1, xx = ox + kx - 1;
                 const bool ok = vn && yy >= 0 && yy < a.H && xx >= 0 && xx < a.W;
                 const int r = ok ? row + (ky - 1) * a.W + (kx - 1) : ZERO_ROW;
-                baddr[j][ky * 3 + kx] = (uint32_t)((h * PITCH + swz(r)) * 16);
+                baddr[j][ky * 3 + kx] = (uint32_t)((h * PITCH + r) * 16);
             }
     }
     if (tid < 8) { // the zero row of both buffers, all four channel groups
         const u32x4 z = {0u, 0u, 0u, 0u};
-        *(u32x4 *)(ps_bytes + (tid >> 2) * P_BUF_BYTES + ((tid & 3) * PITCH + swz(ZERO_ROW)) * 16) = z;
+        *(u32x4 *)(ps_bytes + (tid >> 2) * P_BUF_BYTES + ((tid & 3) * PITCH + ZERO_ROW) * 16) = z;
     }
 
     const uint32_t a_tile_bytes = BM * BK2 * 2;
     const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
-    u32x4 ra[2][A_LD];
+    u32x4 ra[NA][A_LD]; // packed A tiles in flight: tile kt + 1 + NA is requested while tile kt is multiplied
     uint32_t rbw[8][DW];
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -1551,10 +1556,28 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         }
     };
 
+    // operands of a K tile (A buffer ABUF, patch buffer PB, tap TAP) into operand set OS
+    bf16x8 fa[2][2][TM], fb[2][2][TN];
+    auto read_operands = [&](auto os_c, auto abuf_c, auto pb_c, auto tap_c) {
+        constexpr int OS = decltype(os_c)::value;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                fa[OS][s][i] = *(const bf16x8 *)&As[decltype(abuf_c)::value][wm * WTM + i * 32 + l32][s * 16 + h * 8];
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                fb[OS][s][j] = *(const bf16x8 *)(ps_bytes + decltype(pb_c)::value * P_BUF_BYTES + baddr[j][decltype(tap_c)::value] + s * (2 * PITCH * 16));
+        }
+    };
+
     // One stage: nine K tiles (taps) on patch buffer P.  The patch of the next stage is requested during
     // the first tap and goes to the other buffer during the last one; the A tiles run through two
-    // register sets and two LDS buffers as in conv_gemm_bf16_kernel (tile kt+1 stored, tile kt+3
-    // requested while tile kt is multiplied); one barrier per K tile.
+    // register sets and two LDS buffers (tile kt+1 stored, tile kt+3 requested while tile kt is
+    // multiplied).  One barrier per K tile, in its middle: before it, the next tile's A (and patch) go
+    // to the LDS buffers nobody reads any more; after it, the next tile's operands are read while the
+    // second half of this tile's matrix instructions runs, so a wavefront that is alone on its SIMD
+    // does not wait for LDS at the start of a tile.
     auto stage = [&](auto par, int cb) {
         constexpr int P = decltype(par)::value;
         using OtherP = std::integral_constant<int, P ^ 1>;
@@ -1562,49 +1585,43 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         static_for_n<KHW>([&](auto tau_c) {
             constexpr int TAU = decltype(tau_c)::value;
             constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2
-            constexpr int BUF = IDX & 1;
+            constexpr int BUF = IDX & 1;       // A buffer and operand set of this tile
             using NextBuf = std::integral_constant<int, BUF ^ 1>;
-            using Set = std::integral_constant<int, (IDX + 1) & 1>;
+            using Set = std::integral_constant<int, (IDX + 1) % NA>;
+            using NextTap = std::integral_constant<int, (TAU + 1) % KHW>;
+            using NextPatch = std::integral_constant<int, (TAU + 1 < KHW) ? P : (P ^ 1)>;
             const int kt = cb * KHW + TAU;
-            bf16x8 fa[2][TM], fb[2][TN];
-#pragma unroll
-            for (int s = 0; s < 2; s++) {
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-                    fa[s][i] = *(const bf16x8 *)&As[BUF][wm * WTM + i * 32 + l32][s * 16 + h * 8];
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    fb[s][j] = *(const bf16x8 *)(ps_bytes + P * P_BUF_BYTES + baddr[j][TAU] + s * (2 * PITCH * 16));
-            }
             store_a(Set{}, NextBuf{});
-            load_a(Set{}, kt + 3);
-            if (TAU == 0 && has_next)
-                load_patch(cb + 1);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
             if (TAU == KHW - 1 && has_next)
                 store_patch(OtherP{});
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[BUF][0][i], fb[BUF][0][j], acc[i][j], 0, 0, 0);
             __syncthreads();
+            read_operands(NextBuf{}, NextBuf{}, NextPatch{}, NextTap{});
+            load_a(Set{}, kt + 1 + NA);
+            if (TAU == 0 && has_next)
+                load_patch(cb + 1);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[BUF][1][i], fb[BUF][1][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0); // keep this order: the scheduler would sink the operand reads to their uses
         });
     };
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     load_patch(0);
-    load_a(I0{}, 0);
-    load_a(I1{}, 1);
+    static_for_n<NA>([&](auto set) { load_a(set, decltype(set)::value); });
     store_patch(I0{});
     store_a(I0{}, I0{});
-    load_a(I0{}, 2);
+    load_a(I0{}, NA);
     __syncthreads();
+    read_operands(I0{}, I0{}, I0{}, I0{});
     int cb = 0;
     for (; cb + 1 < ncb; cb += 2) {
         stage(I0{}, cb);
@@ -1612,6 +1629,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     }
     if (cb < ncb)
         stage(I0{}, cb);
+    __syncthreads(); // the operand reads issued after the last barrier are done before LDS is reused
 
     static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
