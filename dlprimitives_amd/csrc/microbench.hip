@@ -54,6 +54,31 @@ __global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, f
         dst[i] = src[i];
 }
 
+__global__ __launch_bounds__(256) void read_f4(const float4 *__restrict__ src, float *out, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    float4 s = {0, 0, 0, 0};
+    for (; i < n; i += stride) {
+        const float4 v = src[i];
+        s.x += v.x;
+        s.y += v.y;
+        s.z += v.z;
+        s.w += v.w;
+    }
+    if (s.x + s.y + s.z + s.w == 12345.678f) // never true for the probe's data
+        out[0] = 1.0f;
+}
+
+__global__ __launch_bounds__(256) void write_f4(float4 *__restrict__ dst, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    const float4 v = {1, 2, 3, 4};
+    for (; i < n; i += stride)
+        dst[i] = v;
+}
+
 static float time_ms(hipStream_t s, hipEvent_t e0, hipEvent_t e1)
 {
     float ms = 0;
@@ -144,6 +169,38 @@ int dlp_probe_copy(int mbytes, double *gbs)
     (void)hipEventDestroy(e1);
     (void)hipFree(a);
     (void)hipFree(b);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// read-only (write != 0: write-only) streaming bandwidth in GB/s over `mbytes` MiB
+int dlp_probe_stream(int mbytes, int write, double *gbs)
+{
+    size_t bytes = (size_t)mbytes << 20;
+    float4 *a = nullptr;
+    float *o = nullptr;
+    if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&o, 4) != hipSuccess)
+        return 1;
+    (void)hipMemset(a, 1, bytes);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    size_t n = bytes / 16;
+    const int reps = 10;
+    for (int r = 0; r <= reps; r++) {
+        if (r == 1)
+            (void)hipEventRecord(e0, 0);
+        if (write)
+            write_f4<<<256 * 16, 256>>>(a, n);
+        else
+            read_f4<<<256 * 16, 256>>>(a, o, n);
+    }
+    (void)hipEventRecord(e1, 0);
+    float ms = time_ms(0, e0, e1);
+    *gbs = 1.0 * bytes * reps / (ms * 1e-3) / 1e9;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(a);
+    (void)hipFree(o);
     return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 }

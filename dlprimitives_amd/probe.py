@@ -32,6 +32,15 @@ def main():
         raise SystemExit("copy probe failed")
     out["copy_gbs_read_plus_write"] = round(v.value, 1)
     out["copy_bytes_per_launch_each_direction"] = args.copy_mb << 20
+    if not args.no_mfma:
+        # tensors far above the 256 MB last-level cache: what HBM itself sustains
+        big = 2048
+        if lib.dlp_probe_copy(big, ctypes.byref(v)) == 0:
+            out["copy_gbs_%dmb" % big] = round(v.value, 1)
+        if lib.dlp_probe_stream(big, 0, ctypes.byref(v)) == 0:
+            out["read_gbs_%dmb" % big] = round(v.value, 1)
+        if lib.dlp_probe_stream(big, 1, ctypes.byref(v)) == 0:
+            out["write_gbs_%dmb" % big] = round(v.value, 1)
     print(json.dumps(out))
 
 
