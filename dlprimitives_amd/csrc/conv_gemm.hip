@@ -1052,10 +1052,13 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
 // so that both these stores (pixels PXL apart across lanes) and the operand reads (consecutive
 // pixels across lanes) are free of bank conflicts.  64 * 4 / PXL lanes suffice for a tile, so the
 // B tiles are dealt to the wavefronts in turn (LW wavefronts per tile).
-template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL>
+// SX = 2: the same for 1x1 stride-2 convolutions whose output width is a multiple of PXL: a lane
+// loads 2 * PXL consecutive input pixels of an even input row and keeps the even ones.
+template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL, int SX = 1>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
-    static_assert(PXL == 0 || ((PXL == 4 || PXL == 8) && ORDER == GEMM_ORDER_TAP_BF16), "dense loader variants");
+    static_assert(PXL == 0 || ((PXL == 2 || PXL == 4 || PXL == 8) && PXL * SX >= 4 && PXL * SX <= 8 && ORDER == GEMM_ORDER_TAP_BF16),
+                  "dense loader variants: loads of 8 or 16 bytes");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -1148,7 +1151,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     constexpr int NPQ = BN / PXN;                  // pixel groups of a tile
     constexpr int LW = PXL ? 4 * NPQ / 64 : 4;     // wavefronts that load one B tile
     constexpr int NSETB = NSET * LW / 4 ? NSET * LW / 4 : 1; // a wavefront loads every 4/LW-th tile: that many fewer register sets
-    constexpr int DW = PXL ? PXL / 2 : 1;          // dwords per load
+    constexpr int DW = PXL ? PXL * SX / 2 : 1;     // dwords per load
     static_assert(LW == 1 || LW == 2 || LW == 4, "loader wavefronts");
     uint32_t dvoff = kOutOfRange; // byte offset of (first channel of the block, first pixel) in x
     uint32_t dslot[PXN];          // LDS byte offsets of the block's pixels inside a B tile
@@ -1158,11 +1161,16 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     if constexpr (PXL > 0) {
         const int blk = (wave % LW) * 64 + lane;
         const int oct = blk / NPQ, pq = blk % NPQ;
-        const int n = n0 + pq * PXL; // PXL divides OH*OW: the run stays inside one image
+        const int n = n0 + pq * PXL; // PXL divides OH*OW (stride 2: OW): the run stays inside one image (one row)
         if (n < a.N) {
             const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
             const int pix = n - b * a.OHW;
-            dvoff = (uint32_t)(b * a.Cin + g * a.Cin_g + oct * 8) * a.hw4 + (uint32_t)pix * 2u;
+            uint32_t in_pix = (uint32_t)pix;
+            if (SX == 2) {
+                const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+                in_pix = (uint32_t)(oy * 2 * a.W + (pix - oy * a.OW) * 2);
+            }
+            dvoff = (uint32_t)(b * a.Cin + g * a.Cin_g + oct * 8) * a.hw4 + in_pix * 2u;
         }
 #pragma unroll
         for (int q = 0; q < PXN; q++) {
@@ -1181,12 +1189,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         const uint32_t soff = (uint32_t)(min(kt, a.nkt - 1) * BK2) * a.hw4;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            if constexpr (PXL == 8) {
+            if constexpr (DW == 4) {
                 const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, dvoff, soff + (uint32_t)i * a.hw4, 0));
 #pragma unroll
                 for (int d = 0; d < DW; d++)
                     rbw[S][i][d] = v[d];
-            } else if constexpr (PXL == 4) {
+            } else if constexpr (DW == 2) {
                 const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(xr, dvoff, soff + (uint32_t)i * a.hw4, 0));
 #pragma unroll
                 for (int d = 0; d < DW; d++)
@@ -1201,8 +1209,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         for (int q = 0; q < PXN; q++) {
             u32x4 v;
 #pragma unroll
-            for (int j = 0; j < 4; j++) // channels 2j (low half) and 2j+1 of pixel q
-                v[j] = __builtin_amdgcn_perm(rbw[S][2 * j + 1][q / 2], rbw[S][2 * j][q / 2], (q & 1) ? 0x07060302u : 0x05040100u);
+            for (int j = 0; j < 4; j++) { // channels 2j (low half) and 2j+1 of pixel q
+                if constexpr (SX == 2) // pixel q is the low half of dword q
+                    v[j] = __builtin_amdgcn_perm(rbw[S][2 * j + 1][q], rbw[S][2 * j][q], 0x05040100u);
+                else
+                    v[j] = __builtin_amdgcn_perm(rbw[S][2 * j + 1][q / 2], rbw[S][2 * j][q / 2], (q & 1) ? 0x07060302u : 0x05040100u);
+            }
             *(u32x4 *)(bs_bytes + BUF * B_TILE_BYTES + dslot[q]) = v;
         }
     };
@@ -1885,8 +1897,14 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
 
 typedef void (*Bf16Kernel)(GemmArgs);
 template <int BM, int BN, int WM, int WN>
-Bf16Kernel bf16_kernel_of_tile(int order, int pxl)
+Bf16Kernel bf16_kernel_of_tile(int order, int pxl, int sx)
 {
+    if (order == GEMM_ORDER_TAP_BF16 && sx == 2 && pxl == 4)
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 4, 2>;
+    if constexpr (BN == 128) {
+        if (order == GEMM_ORDER_TAP_BF16 && sx == 2 && pxl == 2)
+            return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 2, 2>;
+    }
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 8)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 8>;
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 4)
@@ -1895,9 +1913,9 @@ Bf16Kernel bf16_kernel_of_tile(int order, int pxl)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET, 0>;
     return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2, 0>;
 }
-Bf16Kernel bf16_kernel(int tile, int order, int pxl)
+Bf16Kernel bf16_kernel(int tile, int order, int pxl, int sx)
 {
-    return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl);
+    return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl, sx) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl, sx);
 }
 
 // Largest number of patch rows any pixel tile of conv_patch_bf16_kernel needs (same arithmetic as the kernel).
@@ -1966,7 +1984,7 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     {
         TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL(bf16_kernel(p.tile, p.order, pxl), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL(bf16_kernel(p.tile, p.order, pxl, p.dense_sx), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
@@ -2102,6 +2120,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
 {
     GemmPlan p;
     p.dense_pxl = 0;
+    p.dense_sx = 1;
     p.patch_bf16 = 0;
     p.pp_nbr = 0;
     const int cin_g = g.Cin / g.groups;
@@ -2128,6 +2147,14 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.tile = p.M > 64 ? 2 : 3;
         if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.H * g.W) % 4 == 0)
             p.dense_pxl = (g.H * g.W) % 8 == 0 ? 8 : 4;
+        // 1x1 stride 2 on even-sized images: runs of 4 (2) output pixels of a row = 8 (4) consecutive input pixels
+        if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.W % 2 == 0 && g.H % 2 == 0) {
+            const int pxl = g.OW % 4 == 0 ? 4 : (g.OW % 2 == 0 && p.tile == 2) ? 2 : 0;
+            if (pxl) {
+                p.dense_pxl = pxl;
+                p.dense_sx = 2;
+            }
+        }
         // stride-1 3x3 "same" convolutions whose largest patch fits the LDS rows and one block per lane: LDS-patch kernel
         if (tap_major && g.KH == 3 && g.KW == 3 && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 &&
             (g.H * g.W) % 4 == 0 && g.B > 0) {

@@ -155,6 +155,7 @@ struct GemmPlan {
     int mtiles;         // ceil(M / BM)
     int patch;          // 1: stride-1 "same" convolution run by the LDS-patch kernel (tap-major packed weights)
     int dense_pxl;      // bf16 matrix-instruction path, 1x1 stride 1 pad 0: input pixels per load of the dense loader (8, 4; 0 = gather)
+    int dense_sx;       // ... 2: the dense loader on a 1x1 stride-2 convolution (dense_pxl output pixels = 2 * dense_pxl loaded)
     int patch_bf16;     // bf16 matrix-instruction path, stride-1 3x3 "same": pixels per load of the LDS-patch kernel (8, 4; 0 = gather)
     int pp_nbr;         // ... and the blocks of that many patch rows in its largest patch
     size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded

@@ -56,6 +56,11 @@ CASES = [
     (case(1, 0, 1, 1, 2048, 512, True, 1, True), (2, 8, 8)),     # long K: split-K slices start in the middle of the loader rotation
     (case(1, 0, 1, 1, 160, 64, True, 1, True), (5, 4, 10)),      # five K tiles, 8-pixel runs, 64x256 tiles
     (case(3, 1, 1, 1, 64, 64, True, 1, True), (2, 13, 14)),      # 2-pixel output runs
+    # dense loader on 1x1 stride-2 convolutions (even image sizes): every other pixel of every other row
+    (case(1, 0, 2, 1, 64, 128, True, 1, True), (3, 28, 28)),     # output width 14: runs of 2 output pixels
+    (case(1, 0, 2, 1, 64, 64, True, 1, False), (2, 16, 16)),     # 64x256 tiles, runs of 4
+    (case(1, 0, 2, 1, 96, 160, False, 1, True), (2, 12, 20)),    # not square, Cout off the tile size, three K tiles
+    (case(1, 0, 2, 1, 32, 64, True, 1, True), (2, 14, 14)),      # odd output width: the gather loader
     # LDS-patch kernel (stride-1 3x3 "same", H*W % 4 == 0): the tile's input patch is loaded once per 32 channels
     (case(3, 1, 1, 1, 128, 128, True, 1, True), (3, 28, 28)),    # 128-pixel tiles, 8-pixel loads, pixel tail
     (case(3, 1, 1, 1, 256, 256, True, 1, True), (5, 14, 14)),    # 4-pixel loads, tiles crossing an image boundary
