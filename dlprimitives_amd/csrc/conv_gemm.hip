@@ -346,6 +346,9 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     auto k_step = [&](auto buf_c, auto set_next, auto set_load, int kt) {
         constexpr int BUF = decltype(buf_c)::value;
         using NextBuf = std::integral_constant<int, BUF ^ 1>;
+        // channel-major order: K need not be a multiple of the K tile; the MFMA steps of the last tile
+        // whose two k rows are both padding are skipped (the 7x7x3 stem: 147 = 9 tiles + 3 rows)
+        const int kk_valid = (ORDER == GEMM_ORDER_CHANNEL) ? (min(BK, a.K - kt * BK) + 1) >> 1 : BK / 2;
         read_operands(buf_c, 0, 0);
 #pragma unroll
         for (int kk = 0; kk < BK / 2; kk++) {
@@ -356,11 +359,13 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 store_slice(set_next, NextBuf{}, q);
                 load_slice(set_load, kt + 2, q);
             });
+            if (ORDER != GEMM_ORDER_CHANNEL || kk < kk_valid) {
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+                for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0); // keep the operand reads one step ahead of their MFMAs
         }
         __syncthreads();
