@@ -6,6 +6,8 @@
 // fallback: every compute entry launches a device kernel or fails.
 #include "dlp_internal.hpp"
 
+#include <algorithm>
+
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -87,6 +89,8 @@ struct dlp_ip_fwd {
     KTabEntry *ktab;
     GemmPlan plan;
     void *wpacked; // op-owned: IPForward::enqueue has no workspace argument
+    void *scratch; // direct kernel: tile counters + K-slice partial sums, grown to the largest batch seen
+    size_t scratch_bytes, scratch_cnt_bytes;
 };
 
 static int upload_ktab(const ConvGeom &g, int activation, KTabEntry **out)
@@ -429,6 +433,8 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
     const ConvGeom g1 = ip_gemm_geom(1, cfg->inputs, cfg->outputs, cfg->dtype);
     op->plan = conv_gemm_plan(g1, activation);
     op->wpacked = nullptr;
+    op->scratch = nullptr;
+    op->scratch_bytes = op->scratch_cnt_bytes = 0;
     int rc = upload_ktab(g1, activation, &op->ktab);
     if (rc == DLP_OK && hipMalloc(&op->wpacked, op->plan.wpack_bytes) != hipSuccess)
         rc = fail(DLP_ERR_RUNTIME, "hipMalloc(packed weights) failed");
@@ -454,6 +460,28 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
     ep.bias = (const float *)bias;
     ep.factor = 0.0f; // src/core/ip.cpp:38
     ep.activation = op->activation;
+    if (ip_direct_supported(op->cfg.inputs, op->cfg.dtype, x, w)) {
+        IpPlan ip;
+        const size_t need = ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
+        (void)need;
+        // op-owned scratch = [counters | partial sums]; both regions only ever grow, and the counter region keeps
+        // its place so that no partial sum is ever written where a later, larger batch expects zeroed counters
+        if (ip.cnt_bytes > op->scratch_cnt_bytes || ip.part_bytes > op->scratch_bytes - op->scratch_cnt_bytes) {
+            // first call, or a larger batch than any before: hipFree waits for the kernels that use the old buffer
+            const size_t cnt_bytes = std::max(ip.cnt_bytes, op->scratch_cnt_bytes);
+            const size_t part_bytes = std::max(ip.part_bytes, op->scratch_bytes - op->scratch_cnt_bytes);
+            if (op->scratch)
+                (void)hipFree(op->scratch);
+            op->scratch = nullptr;
+            op->scratch_bytes = op->scratch_cnt_bytes = 0;
+            DLP_HIP_TRY(hipMalloc(&op->scratch, cnt_bytes + part_bytes));
+            DLP_HIP_TRY(hipMemset(op->scratch, 0, cnt_bytes));
+            op->scratch_bytes = cnt_bytes + part_bytes;
+            op->scratch_cnt_bytes = cnt_bytes;
+        }
+        return ip_direct_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, (int *)op->scratch,
+                                (float *)((char *)op->scratch + op->scratch_cnt_bytes), (hipStream_t)stream);
+    }
     const ConvGeom g = ip_gemm_geom(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype);
     int rc = conv_gemm_pack_weights(g, op->plan, w, op->wpacked, (hipStream_t)stream);
     if (rc != DLP_OK)
@@ -469,6 +497,8 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op)
         (void)hipFree(op->ktab);
     if (op->wpacked)
         (void)hipFree(op->wpacked);
+    if (op->scratch)
+        (void)hipFree(op->scratch);
     delete op;
 }
 

@@ -197,5 +197,17 @@ int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, cons
 
 // ---- InnerProduct GEMM (ip_gemm.hip) ------------------------------------------
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype);
+// Launch shape of the direct kernel (operands loaded from memory straight into matrix-instruction registers)
+struct IpPlan {
+    int nb;               // blocks of 32 batch rows per wavefront (1, 2, 4)
+    int mblocks, nchunks; // tiles: blocks of 32 outputs x chunks of nb * 32 batch rows
+    int ngroups, gps, S;  // groups of 8 (fp32) / 16 (bf16) k: in all, per K slice; K slices
+    size_t cnt_bytes, part_bytes; // op-owned scratch: tile counters | partial sums
+};
+size_t ip_direct_scratch_bytes(int batch, int inputs, int outputs, int dtype, IpPlan *plan);
+bool ip_direct_supported(int inputs, int dtype, const void *x, const void *w);
+// counters: cnt_bytes of zeros (they are left zero); partials: part_bytes
+int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
+                     float *partials, hipStream_t stream);
 
 } // namespace dlp

@@ -3,15 +3,332 @@
 // Replaces the reference's IPForwardImpl / StandardSGEMM path
 // (src/core/ip.cpp:15-50, src/gemm.cpp:240-345):
 //   y[B x Out] = act(x[B x In] * w[Out x In]^T + bias[Out])
-// This is the same GEMM as a 1x1 convolution over 1x1 images with
-// Cin = In, Cout = Out and one "pixel" per batch row:
-//   x[b][c] sits at element b*In + c      = NCHW [B, In, 1, 1]
-//   y[b][o] sits at element b*Out + o     = NCHW [B, Out, 1, 1]
-// so it runs through the implicit-GEMM kernel with that geometry; the bias is
-// per output feature, which is the per-row (bias_M) epilogue of the conv form.
+//
+// Both operands are stored with the reduction index innermost, which is exactly what a matrix
+// instruction wants in a lane: ip_direct_kernel loads them straight from memory into operand
+// registers -- no LDS, no repacking of the weights, no barriers.
+//  * A wavefront owns 32 outputs x up to 128 batch rows (NB blocks of 32) over one slice of K.
+//    A lane (row = lane % 32, half = lane / 32) loads 16 bytes of its weight row and of its NB
+//    batch rows per step: 4 consecutive k in fp32 (half h takes k = 8t + 4h .. +3; the four
+//    v_mfma_f32_32x32x2_f32 of the step pair element e of half 0 with element e of half 1 --
+//    the sum over k is order free as long as both operands use the same pairing), or the 8
+//    consecutive k of one v_mfma_f32_32x32x16_bf16 operand for bf16 tensors.
+//  * The layer is bound by reading w once from HBM, so K is split over enough wavefronts to have
+//    the whole chip loading; the slices of a tile leave their partial sums in an op-owned buffer
+//    (write-through) and the wavefront that arrives last at the tile's counter adds them up in
+//    slice order (deterministic), applies bias and activation, writes y and resets the counter.
+//    Nobody waits for anybody.
+// The reduction over k is accumulated in fp32 in a different order than the reference's sgemm.
+//
+// Shapes the direct kernel does not take (bf16 rows that are not dword aligned) run as a 1x1
+// convolution over 1x1 images through the implicit-GEMM kernel:
+//   x[b][c] sits at element b*In + c = NCHW [B, In, 1, 1],  y[b][o] at b*Out + o = NCHW [B, Out, 1, 1].
 #include "dlp_internal.hpp"
 
+#include <algorithm>
+#include <type_traits>
+
 namespace dlp {
+
+typedef float ip_f32x16 __attribute__((ext_vector_type(16)));
+typedef float ip_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t ip_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 ip_bf16x8 __attribute__((ext_vector_type(8)));
+
+namespace {
+
+constexpr uint32_t kIpOutOfRange = 0x80000000u;
+
+struct IpArgs {
+    const void *x, *w;
+    const float *bias;
+    void *y;
+    float *part; // [tile][slice][NB*16][64] partial sums (register images)
+    int *cnt;    // slices arrived, per tile; zero between launches
+    int B, In, Out;
+    int S;                // K slices
+    int ngroups, gps;     // groups of KG k in all, per slice
+    int mblocks, nchunks; // tiles = mblocks * nchunks; a chunk = NB * 32 batch rows
+    int act;
+    uint32_t x_bytes, w_bytes, part_bytes;
+};
+
+// 16 bytes of a row: elements [k0, k0 + 16 / sizeof(T)), k0 = group offset (scalar, through soff) + the
+// lane's half (in row_off).  With `tail` set (In is not a multiple of the group), a piece that reaches
+// past the end of the row is read dword by dword and only up to the row's end: what follows belongs to
+// the next row, or lies outside the tensor.  (bf16 rows have an even length: a dword is all in or all out.)
+// WIDE: rows start on 16-byte boundaries, a whole piece is one 16-byte load (which wants that alignment).
+template <class T, bool WIDE>
+__device__ __forceinline__ ip_u32x4 load_piece(__amdgpu_buffer_rsrc_t r, uint32_t row_off, uint32_t soff, int k0, int In, bool tail)
+{
+    constexpr int E = 16 / (int)sizeof(T);
+    constexpr int EPD = 4 / (int)sizeof(T); // elements per dword
+    if (!WIDE || (tail && k0 + E > In)) {
+        ip_u32x4 v;
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+            v[d] = (k0 + d * EPD < In) ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, row_off + 4u * (uint32_t)d, soff, 0) : 0u;
+        return v;
+    }
+    return __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, row_off, soff, 0));
+}
+
+template <class T, int NB, bool WIDE>
+__global__ __launch_bounds__(256) void ip_direct_kernel(IpArgs a)
+{
+    constexpr int KG = 32 / (int)sizeof(T); // k per step: 8 (fp32: four MFMAs) or 16 (bf16: one)
+    constexpr int KH = KG / 2;              // k per lane and step
+    const int lane = threadIdx.x & 63;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int gw = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6); // wavefront = work item; no LDS, no barriers
+    const int items = a.mblocks * a.nchunks * a.S;
+    if (gw >= items)
+        return;
+    const int nc = gw % a.nchunks;
+    const int slice = (gw / a.nchunks) % a.S;
+    const int mb = gw / (a.nchunks * a.S);
+    const int tile = mb * a.nchunks + nc;
+    const int m0 = mb * 32, n0 = nc * (NB * 32);
+
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    // rows past the end are clamped to the last one (valid memory); their results are never stored
+    // (byte offsets of the lane's row + its half of a group; the group goes through the scalar offset)
+    const uint32_t half_off = (uint32_t)(h * KH * (int)sizeof(T));
+    const uint32_t a_off = (uint32_t)min(m0 + l32, a.Out - 1) * (uint32_t)a.In * (uint32_t)sizeof(T) + half_off;
+    uint32_t b_off[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+        b_off[j] = (uint32_t)min(n0 + j * 32 + l32, a.B - 1) * (uint32_t)a.In * (uint32_t)sizeof(T) + half_off;
+    const bool tail = a.In % KG != 0;
+
+    ip_f32x16 acc[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            acc[j][r] = 0.0f;
+
+    const int g_begin = slice * a.gps, g_end = min(g_begin + a.gps, a.ngroups);
+    auto load_group = [&](int g, ip_u32x4 &fa, ip_u32x4 (&fb)[NB]) {
+        const int k0 = g * KG + h * KH;
+        const uint32_t soff = (uint32_t)(g * KG * (int)sizeof(T));
+        fa = load_piece<T, WIDE>(wr, a_off, soff, k0, a.In, tail);
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+            fb[j] = load_piece<T, WIDE>(xr, b_off[j], soff, k0, a.In, tail);
+    };
+    auto multiply = [&](const ip_u32x4 &fa, const ip_u32x4 (&fb)[NB]) {
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t ae = fa[e]; // copies: bit_cast applied to a vector element reads element 0
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const uint32_t be = fb[j][e];
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, ae), __builtin_bit_cast(float, be), acc[j], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ip_bf16x8, fa), __builtin_bit_cast(ip_bf16x8, fb[j]), acc[j], 0, 0, 0);
+        }
+    };
+    // four groups (a 128-byte line of every row) in flight per wavefront
+    constexpr int DEPTH = 4;
+    ip_u32x4 fa[DEPTH], fb[DEPTH][NB];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+        if (g_begin + d < g_end)
+            load_group(g_begin + d, fa[d], fb[d]);
+    for (int g = g_begin; g < g_end; g += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (g + d < g_end) {
+                multiply(fa[d], fb[d]);
+                if (g + d + DEPTH < g_end)
+                    load_group(g + d + DEPTH, fa[d], fb[d]);
+            }
+        }
+    }
+
+    if (a.S > 1) {
+        constexpr int kThrough = 17; // sc0 | sc1: past the caches in both directions
+        constexpr uint32_t image_bytes = NB * 16 * 64 * 4;
+        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
+        const uint32_t base = (uint32_t)(tile * a.S) * image_bytes;
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float v = acc[j][r];
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, (uint32_t)lane * 4u,
+                                                      base + (uint32_t)slice * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough);
+            }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the partial sums have been written through
+        int arrived = 0;
+        if (lane == 0)
+            arrived = atomicAdd(a.cnt + tile, 1);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != a.S - 1)
+            return;
+        if (lane == 0)
+            atomicExch(a.cnt + tile, 0); // ready for the next launch on the stream
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[j][r] = 0.0f;
+            // four slices (64 loads) in flight at a time: these loads come from memory, not from a cache
+            for (int s0 = 0; s0 < a.S; s0 += 4) {
+                float p[4][16];
+#pragma unroll
+                for (int ds = 0; ds < 4; ds++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        p[ds][r] = (s0 + ds < a.S) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                         pr, (uint32_t)lane * 4u,
+                                                         base + (uint32_t)(s0 + ds) * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough))
+                                                   : 0.0f;
+#pragma unroll
+                for (int ds = 0; ds < 4; ds++) // slice order
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        acc[j][r] += p[ds][r];
+            }
+        }
+    }
+
+    // epilogue: accumulator register r of a block holds output m0 + 8*(r/4) + 4*h + r%4 of batch row n0 + 32*j + l32
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const int n = n0 + j * 32 + l32;
+        if (n >= a.B)
+            continue;
+        T *yrow = (T *)a.y + (size_t)n * a.Out;
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            const int mq = m0 + 8 * rq + 4 * h; // four consecutive outputs
+            float v[4];
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                v[rr] = acc[j][4 * rq + rr];
+                if (a.bias && mq + rr < a.Out)
+                    v[rr] += a.bias[mq + rr];
+                v[rr] = apply_act(v[rr], a.act);
+            }
+            if (sizeof(T) == 4 && (a.Out & 3) == 0 && ((uintptr_t)a.y & 15) == 0) {
+                if (mq < a.Out)
+                    *(ip_f32x4 *)((float *)yrow + mq) = ip_f32x4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++)
+                    if (mq + rr < a.Out)
+                        store_plain(yrow + mq + rr, v[rr]);
+            }
+        }
+    }
+}
+
+} // namespace
+
+size_t ip_direct_scratch_bytes(int batch, int inputs, int outputs, int dtype, IpPlan *plan)
+{
+    IpPlan p;
+    const int kg = dtype == DLP_FLOAT ? 8 : 16;
+    // One block of 32 batch rows per wavefront: the wavefronts of a workgroup are the batch chunks of one
+    // (output block, K slice), so they share its weights through the L1 and the work spreads over 4x the
+    // SIMDs (the fp32 matrix instruction is slow: 64 clocks per 32x32x2 block).
+    p.nb = 1;
+    p.mblocks = (outputs + 31) / 32;
+    p.nchunks = (batch + p.nb * 32 - 1) / (p.nb * 32);
+    p.ngroups = (inputs + kg - 1) / kg;
+    // K slices: about one wavefront per SIMD (1024), slices of at least 8 steps, at most 16 slices, and
+    // partial sums (4 KB per tile and slice, written and read once) that stay below half the bytes of w.
+    // Measured on 25088 -> 4096 at batch 16 (411 MB of weights): 155 us = 2.7 TB/s this way; 4096
+    // wavefronts with eight groups in flight each: 195 us.
+    const long long tiles = (long long)p.mblocks * p.nchunks;
+    const long long w_bytes = (long long)outputs * inputs * (dtype == DLP_FLOAT ? 4 : 2);
+    long long s = (1024 + tiles - 1) / tiles;
+    s = std::min<long long>(s, p.ngroups / 8);
+    s = std::min<long long>(s, w_bytes / (8192 * tiles));
+    s = std::max<long long>(1, std::min<long long>(s, 16));
+    p.gps = (int)((p.ngroups + s - 1) / s);
+    p.S = (p.ngroups + p.gps - 1) / p.gps;
+    p.cnt_bytes = (size_t)((tiles * sizeof(int) + 255) / 256 * 256);
+    p.part_bytes = p.S > 1 ? (size_t)tiles * p.S * p.nb * 16 * 64 * sizeof(float) : 0;
+    if (plan)
+        *plan = p;
+    return p.cnt_bytes + p.part_bytes;
+}
+
+bool ip_direct_supported(int inputs, int dtype, const void *x, const void *w)
+{
+    if (dtype == DLP_FLOAT)
+        return true; // rows are dword aligned
+    return dtype == DLP_BFLOAT16 && inputs % 2 == 0 && (((uintptr_t)x | (uintptr_t)w) & 3) == 0;
+}
+
+int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
+                     float *partials, hipStream_t stream)
+{
+    IpPlan p;
+    ip_direct_scratch_bytes(batch, inputs, outputs, dtype, &p);
+    const size_t esize = dtype_size(dtype);
+    const size_t x_bytes = (size_t)batch * inputs * esize, w_bytes = (size_t)outputs * inputs * esize;
+    if (x_bytes >= kIpOutOfRange || w_bytes >= kIpOutOfRange || p.part_bytes >= kIpOutOfRange)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
+    IpArgs a;
+    a.x = x;
+    a.w = w;
+    a.bias = ep.bias;
+    a.y = y;
+    a.cnt = counters;
+    a.part = partials;
+    a.B = batch;
+    a.In = inputs;
+    a.Out = outputs;
+    a.S = p.S;
+    a.ngroups = p.ngroups;
+    a.gps = p.gps;
+    a.mblocks = p.mblocks;
+    a.nchunks = p.nchunks;
+    a.act = ep.activation;
+    a.x_bytes = (uint32_t)x_bytes;
+    a.w_bytes = (uint32_t)w_bytes;
+    a.part_bytes = (uint32_t)p.part_bytes;
+    const long long items = (long long)p.mblocks * p.nchunks * p.S;
+    if (items > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "inner product too large for a single launch");
+    const dim3 grid((unsigned)((items + 3) / 4)), block(256);
+    TimingScope ts("ip_direct", stream);
+    // 16-byte loads when every row of x and w starts on a 16-byte boundary, dword loads otherwise
+    const bool wide = (inputs * esize) % 16 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
+    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, a); };
+    auto pick = [&](auto type_tag, auto nb_c) {
+        using T = decltype(type_tag);
+        constexpr int NBV = decltype(nb_c)::value;
+        if (wide)
+            launch(ip_direct_kernel<T, NBV, true>);
+        else
+            launch(ip_direct_kernel<T, NBV, false>);
+    };
+    auto pick_nb = [&](auto type_tag) {
+        if (p.nb == 1)
+            pick(type_tag, std::integral_constant<int, 1>{});
+        else if (p.nb == 2)
+            pick(type_tag, std::integral_constant<int, 2>{});
+        else
+            pick(type_tag, std::integral_constant<int, 4>{});
+    };
+    if (dtype == DLP_BFLOAT16)
+        pick_nb(bf16_t{});
+    else
+        pick_nb(float{});
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
 
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype)
 {

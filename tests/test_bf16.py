@@ -174,6 +174,17 @@ def test_bf16_glue_and_inner_product(oracle_mod):
     torch.cuda.synchronize()
     want = oracle_mod.ip_forward(xi, wi, bi)
     assert np.abs(yi.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
+    # a partial last group of k (In % 16 != 0), Out and batch off the block sizes; and an odd In (rows not dword aligned:
+    # the implicit-GEMM fallback)
+    for (B, I, O) in ((37, 1000 + 6, 75), (5, 333, 20)):
+        xi = oracle_mod.bf16_round(rng.uniform(-1, 1, (B, I)).astype(np.float32))
+        wi = oracle_mod.bf16_round((rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32))
+        bi = rng.uniform(-0.1, 0.1, O).astype(np.float32)
+        ip = dlp.IPForward.create(dlp.IPSettings(I, O, B, dtype=BFLOAT16_DATA), True, "relu")
+        yi = torch.full((B, O), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        ip.enqueue(_bf(xi), _bf(wi), torch.from_numpy(bi).cuda(), yi)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(yi.float().cpu().numpy(), oracle_mod.ip_forward(xi, wi, bi, "relu"), rtol=2 ** -8, atol=1e-3)
 
 
 def test_resnet50_bf16_logits_vs_fp32_reference(oracle_mod):

@@ -331,7 +331,8 @@ def test_inner_product_reference_goldens(gpu):
     assert n == 28
 
 
-@pytest.mark.parametrize("bio", [(128, 2048, 1000), (1, 512, 1000), (8, 1024, 1024), (50, 333, 77), (2, 1, 1)], ids=lambda v: "b%d_%dto%d" % v)
+@pytest.mark.parametrize("bio", [(128, 2048, 1000), (1, 512, 1000), (8, 1024, 1024), (50, 333, 77), (2, 1, 1), (3, 1030, 70), (200, 512, 64),
+                                 (33, 4100, 31), (16, 25088, 96)], ids=lambda v: "b%d_%dto%d" % v)
 @pytest.mark.parametrize("bias", [True, False])
 def test_inner_product_vs_oracle(gpu, oracle_mod, bio, bias):
     B, I, O = bio
@@ -340,6 +341,44 @@ def test_inner_product_vs_oracle(gpu, oracle_mod, bio, bias):
     w = (rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
     b = rng.uniform(-0.1, 0.1, O).astype(np.float32) if bias else None
     np.testing.assert_allclose(gpu.run_ip(x, w, b, "relu"), oracle_mod.ip_forward(x, w, b, "relu"), **TOL)
+
+
+def test_inner_product_same_op_many_calls(gpu, oracle_mod):
+    """One op object, batches that grow and shrink: the op-owned partial-sum buffer is regrown, the tile
+    counters return to zero after every call, and the result does not depend on the call history."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(5)
+    I, O = 2048, 1000
+    w = (rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, O).astype(np.float32)
+    op = dlp.IPForward.create(dlp.IPSettings(I, O, 8), True, "identity")
+    wd, bd = gpu.dev(w), gpu.dev(b)
+    first = {}
+    for B in (8, 128, 8, 40, 128, 1):
+        x = rng.uniform(-1, 1, (B, I)).astype(np.float32) if B not in first else first[B][0]
+        yd = torch.full((B, O), float("nan"), dtype=torch.float32, device="cuda:0")
+        op.enqueue(gpu.dev(x), wd, bd, yd)
+        op.enqueue(gpu.dev(x), wd, bd, yd)  # back to back on the stream
+        torch.cuda.synchronize()
+        got = yd.cpu().numpy()
+        np.testing.assert_allclose(got, oracle_mod.ip_forward(x, w, b), **TOL)
+        if B in first:
+            assert np.array_equal(got, first[B][1])  # slices are added in a fixed order
+        first[B] = (x, got)
+
+
+def test_inner_product_integer_exact(gpu):
+    # integer-valued operands: every partial sum is exact in fp32, so the split over K slices and the
+    # pairing of k inside a matrix instruction must reproduce the integer result exactly
+    rng = np.random.default_rng(9)
+    x = rng.integers(-3, 4, (70, 1203)).astype(np.float32)
+    w = rng.integers(-3, 4, (45, 1203)).astype(np.float32)
+    b = rng.integers(-5, 6, 45).astype(np.float32)
+    want = (x.astype(np.int64) @ w.astype(np.int64).T + b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(gpu.run_ip(x, w, b), want)
 
 
 def test_inner_product_flattens_trailing_dims(gpu, oracle_mod):
