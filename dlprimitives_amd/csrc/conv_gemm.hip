@@ -77,6 +77,7 @@ struct GemmArgs {
     int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
     int pxv;                  // bf16 matrix-instruction kernels: pixels per output store (0 = one element per store)
     int pp_nbr;               // conv_patch_bf16_kernel: blocks of PXP rows in the largest patch of the launch
+    int wdirect;              // conv_gemm_bf16_kernel: wp is the weight tensor itself (1x1 convolution), not packed tiles
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -1148,8 +1149,23 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         }
     }
 
-    const uint32_t a_tile_bytes = BM * BK2 * 2;
-    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
+    // A loader: 16-byte pieces of the packed tile, in tile order -- or, for 1x1 convolutions, of the weight
+    // matrix itself ([Cout][Cin] has k innermost already: a tile row is 64 bytes of a matrix row, a.wp is w)
+    uint32_t a_tile_bytes = BM * BK2 * 2;
+    uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
+    uint32_t a_voff[A_LD];
+#pragma unroll
+    for (int j = 0; j < A_LD; j++)
+        a_voff[j] = (uint32_t)(tid + j * kThreads) * 16u;
+    if (a.wdirect) {
+        a_tile_bytes = BK2 * 2;
+        a_row_base = 0;
+#pragma unroll
+        for (int j = 0; j < A_LD; j++) {
+            const int idx = tid + j * kThreads, m = m0 + (idx >> 2);
+            a_voff[j] = m < a.M ? (uint32_t)(g * a.M + m) * (uint32_t)a.K * 2u + (uint32_t)(idx & 3) * 16u : kOutOfRange;
+        }
+    }
 
     // ---- dense loader state: block = 8 channels x PXL pixels; blocks of a tile = 4 * BN / PXL ----
     constexpr int PXN = PXL ? PXL : 1;
@@ -1238,7 +1254,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
 #pragma unroll
             for (int j = 0; j < A_LD; j++)
-                ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
+                ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, a_voff[j], a_soff, 0));
         }
         if constexpr (PXL > 0) {
             if (Q == 1 && my_tile(kt))
@@ -2124,6 +2140,7 @@ int with_tile(int choice, F &&f)
 GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
 {
     GemmPlan p;
+    p.wdirect = 0;
     p.dense_pxl = 0;
     p.dense_sx = 1;
     p.patch_bf16 = 0;
@@ -2150,6 +2167,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = tap_major ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
         p.nkt = (p.K + BK2 - 1) / BK2;
         p.tile = p.M > 64 ? 2 : 3;
+        p.wdirect = tap_major && g.KH == 1 && g.KW == 1; // [Cout][Cin] is read in place (when w is 16-byte aligned)
         if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.H * g.W) % 4 == 0)
             p.dense_pxl = (g.H * g.W) % 8 == 0 ? 8 : 4;
         // 1x1 stride 2 on even-sized images: runs of 4 (2) output pixels of a row = 8 (4) consecutive input pixels
@@ -2247,6 +2265,8 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
                            size_t part_bytes)
 {
+    if (p.wdirect && ((uintptr_t)w & 15) == 0)
+        return DLP_OK; // conv_gemm_launch reads w in place
     int *zero = nullptr; // tile counters of the stream-K launch that follows
     int nzero = 0;
     if (p.patch && part_ws != nullptr) {
@@ -2287,7 +2307,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 }
 
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes)
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes, const void *w)
 {
     if (g.dtype != DLP_FLOAT && g.dtype != DLP_BFLOAT16)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: float_data and bfloat16_data are implemented");
@@ -2328,6 +2348,12 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     a.KH = g.KH; a.KW = g.KW;
     a.x_bytes = (uint32_t)(x_elems * esize);
     a.wp_bytes = (uint32_t)p.wpack_bytes;
+    a.wdirect = 0;
+    if (p.wdirect && w != nullptr && ((uintptr_t)w & 15) == 0) { // same test as in conv_gemm_pack_weights
+        a.wdirect = 1;
+        a.wp = (const float *)w;
+        a.wp_bytes = (uint32_t)((size_t)g.Cout * p.K * esize);
+    }
     a.y_bytes = y_elems * esize < kOutOfRange ? (uint32_t)(y_elems * esize) : 0;
     a.x_shift = (uint32_t)x_shift;
     a.hw4 = (uint32_t)(g.H * g.W * esize);

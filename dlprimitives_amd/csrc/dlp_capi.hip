@@ -398,7 +398,7 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
         rc = conv_gemm_pack_weights(g, plan, w, ws, s, part, part ? ws_bytes - used : 0);
         if (rc != DLP_OK)
             return rc;
-        return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0);
+        return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0, w);
     }
     }
 }
@@ -486,7 +486,7 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
     int rc = conv_gemm_pack_weights(g, op->plan, w, op->wpacked, (hipStream_t)stream);
     if (rc != DLP_OK)
         return rc;
-    return conv_gemm_launch(g, op->plan, op->ktab, x, op->wpacked, y, ep, (hipStream_t)stream);
+    return conv_gemm_launch(g, op->plan, op->ktab, x, op->wpacked, y, ep, (hipStream_t)stream, -1, nullptr, 0, w);
 }
 
 void dlp_ip_fwd_destroy(dlp_ip_fwd *op)

@@ -154,6 +154,7 @@ struct GemmPlan {
     int M, K, nkt;      // per group: rows, reduction length, K tiles of 16
     int mtiles;         // ceil(M / BM)
     int patch;          // 1: stride-1 "same" convolution run by the LDS-patch kernel (tap-major packed weights)
+    int wdirect;        // bf16 matrix-instruction path, 1x1: the kernel reads the weight tensor in place, nothing is packed
     int dense_pxl;      // bf16 matrix-instruction path, 1x1 stride 1 pad 0: input pixels per load of the dense loader (8, 4; 0 = gather)
     int dense_sx;       // ... 2: the dense loader on a 1x1 stride-2 convolution (dense_pxl output pixels = 2 * dense_pxl loaded)
     int patch_bf16;     // bf16 matrix-instruction path, stride-1 3x3 "same": pixels per load of the LDS-patch kernel (8, 4; 0 = gather)
@@ -174,9 +175,10 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                            void *part_ws = nullptr, size_t part_bytes = 0);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 // part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.
+// w: the weight tensor as the caller gave it (plans with wdirect read it in place when it is 16-byte aligned).
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
                      void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *part_ws = nullptr,
-                     size_t part_bytes = 0);
+                     size_t part_bytes = 0, const void *w = nullptr);
 
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);
