@@ -62,6 +62,79 @@ __global__ __launch_bounds__(256) void pool2d_kernel(PoolArgs a)
     store_plain((T *)a.y + idx, val);
 }
 
+// Max pooling 3x3, stride 2, padding 1 (the ResNet stem): lanes own output columns of a strip of
+// kMaxStrip output rows, as in the stride-2 depthwise kernel.  A lane loads the two input columns it
+// owns (2*ox, 2*ox + 1: one 8- or 4-byte load when the row is aligned for it) of every input row of
+// the strip before it consumes any, takes column 2*ox - 1 from the lane to its left (lane 0 of a
+// wavefront is a halo lane that stores nothing; adjacent wavefronts overlap by it), and reuses the
+// row shared by consecutive output rows from registers: every input element is read once (plus
+// one halo row per strip) instead of 2.25 times.  Padding is ignored by max, as in the reference.
+constexpr int kMaxStrip = 7;
+
+template <class T>
+__global__ __launch_bounds__(256) void maxpool3x3s2p1_kernel(PoolArgs a, int nstrips, long long total_cols, int pairs)
+{
+    constexpr int NIN = 2 * kMaxStrip + 1;
+    constexpr float kLowest = -3.402823466e+38f;
+    const int lane = threadIdx.x & 63;
+    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long f = wave * 63 + lane - 1; // flat (plane, strip, ox) index
+    const bool in_range = f >= 0 && f < total_cols;
+    const long long ps = in_range ? f / a.OW : 0;
+    const int ox = in_range ? (int)(f - ps * a.OW) : 0;
+    const long long plane = ps / nstrips;
+    const int strip = (int)(ps - plane * nstrips);
+    const int oy0 = strip * kMaxStrip;
+    const T *xp = (const T *)a.x + plane * a.H * a.W;
+    const int x0 = 2 * ox;
+    const bool v0 = in_range && x0 < a.W, v1 = in_range && x0 + 1 < a.W;
+    const bool has_left = ox > 0;
+
+    float c0[NIN], c1[NIN];
+    const int iy0 = 2 * oy0 - 1;
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+        const int yy = iy0 + r;
+        const bool vy = yy >= 0 && yy < a.H;
+        const T *p = xp + (size_t)(vy ? yy : 0) * a.W + x0;
+        c0[r] = kLowest;
+        c1[r] = kLowest;
+        if (pairs) { // even W, aligned base: both columns exist and sit in one aligned pair
+            if (vy && v0) {
+                if constexpr (sizeof(T) == 4) {
+                    const float2 v = *(const float2 *)p;
+                    c0[r] = v.x;
+                    c1[r] = v.y;
+                } else {
+                    const uint32_t v = *(const uint32_t *)p;
+                    c0[r] = __builtin_bit_cast(float, v << 16);
+                    c1[r] = __builtin_bit_cast(float, v & 0xffff0000u);
+                }
+            }
+        } else {
+            if (vy && v0)
+                c0[r] = to_float(p[0]);
+            if (vy && v1)
+                c1[r] = to_float(p[1]);
+        }
+    }
+    float m[NIN]; // maximum over the row's three window columns
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+        const float l = __shfl_up(c1[r], 1); // the left lane's odd column = 2*ox - 1
+        m[r] = fmaxf(fmaxf(has_left ? l : kLowest, c0[r]), c1[r]);
+    }
+    if (!in_range || lane == 0)
+        return;
+    T *yp = (T *)a.y + plane * a.OH * a.OW + ox;
+#pragma unroll
+    for (int j = 0; j < kMaxStrip; j++) {
+        const int oy = oy0 + j;
+        if (oy < a.OH)
+            store_plain(yp + (size_t)oy * a.OW, fmaxf(fmaxf(m[2 * j], m[2 * j + 1]), m[2 * j + 2]));
+    }
+}
+
 // one wavefront per plane: lanes stride over the plane, then a shuffle reduction.
 // The average is accumulated per lane in ascending index order and combined pairwise,
 // so it differs from the reference's single running sum only by fp32 rounding.
@@ -255,7 +328,17 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         const long long total = planes * a.OH * a.OW;
         DLP_REQUIRE(planes < 0x7fffffffLL && total < 0x7fffffffLL * 256, "tensor too large");
         TimingScope ts("pooling", s);
-        if (op->dtype == DLP_BFLOAT16)
+        if (a.mode == 0 && a.kh == 3 && a.kw == 3 && a.sh == 2 && a.sw == 2 && a.ph == 1 && a.pw == 1) {
+            const int nstrips = (a.OH + kMaxStrip - 1) / kMaxStrip;
+            const long long total_cols = planes * nstrips * a.OW;
+            const long long blocks = ((total_cols + 62) / 63 + 3) / 4;
+            const size_t esize = dtype_size(op->dtype);
+            const int pairs = a.W % 2 == 0 && ((uintptr_t)x & (2 * esize - 1)) == 0;
+            if (op->dtype == DLP_BFLOAT16)
+                hipLaunchKernelGGL(maxpool3x3s2p1_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, s, a, nstrips, total_cols, pairs);
+            else
+                hipLaunchKernelGGL(maxpool3x3s2p1_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, a, nstrips, total_cols, pairs);
+        } else if (op->dtype == DLP_BFLOAT16)
             hipLaunchKernelGGL(pool2d_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
         else
             hipLaunchKernelGGL(pool2d_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);

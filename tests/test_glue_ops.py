@@ -133,6 +133,34 @@ def test_gpu_pooling_large_shapes_vs_oracle(oracle_mod):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_maxpool_3x3_stride2_pad1_shapes(oracle_mod, dtype):
+    """The strip kernel behind max pooling 3x3 / stride 2 / pad 1: odd and even sizes, planes smaller than a
+    strip, rows shorter than a wavefront, ceil-mode output sizes; a maximum of stored values is exact."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA
+
+    rng = np.random.default_rng(3)
+    tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    for (b, c, h, w, ceil_mode) in [(2, 3, 112, 112, 0), (1, 5, 7, 7, 0), (3, 2, 13, 9, 1), (2, 4, 30, 31, 0), (1, 1, 2, 2, 0), (2, 7, 15, 64, 1),
+                                    (1, 2, 57, 130, 0)]:
+        x = rng.standard_normal((b, c, h, w)).astype(np.float32)
+        if dtype == "bfloat16":
+            x = oracle_mod.bf16_round(x)
+        oh = dlp.pool2d_output_size(h, 3, 1, 2, ceil_mode)
+        ow = dlp.pool2d_output_size(w, 3, 1, 2, ceil_mode)
+        y = torch.full((b, c, oh, ow), float("nan"), dtype=tdt, device="cuda:0")
+        op = dlp.Pooling2DForward.create_max_pooling(3, 1, 2, dtype=BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA)
+        op.enqueue(torch.from_numpy(x).cuda().to(tdt), y)
+        torch.cuda.synchronize()
+        want = oracle_mod.pool2d_forward(x, 3, 1, 2, "max", ceil_mode=ceil_mode)
+        assert want.shape == (b, c, oh, ow)
+        assert np.array_equal(y.float().cpu().numpy(), want), (b, c, h, w, ceil_mode)
+
+
+@pytest.mark.gpu
 def test_gpu_global_pooling(oracle_mod):
     import torch
 
