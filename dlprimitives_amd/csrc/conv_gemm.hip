@@ -400,8 +400,52 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
 {
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    // ---- split-K: raw partial sums to the workspace, reduced by a second kernel ----
-    if (a.splitk > 1) {
+    // ---- split-K, reduced in place: the slice's accumulators go to the workspace as a register image
+    // ([r][thread], write-through); the workgroup that arrives last at the tile's counter adds up all
+    // slices in slice order (deterministic), whoever it is, and goes on to the epilogue.  Nobody waits. ----
+    if (a.splitk > 1 && a.sk_cnt != nullptr) {
+        static_assert(TM == 1 && TN == 1, "one MFMA block per wavefront");
+        constexpr int kThrough = 17; // sc0 | sc1: past the caches in both directions
+        constexpr uint32_t image_bytes = BM * BN * 4;
+        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.sk_part, 0, a.sk_part_bytes, 0x00020000);
+        const int tile = (g * a.ntiles + n0 / BN) * a.mtiles + m0 / BM;
+        const uint32_t base = (uint32_t)(tile * a.splitk) * image_bytes;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float v = acc[0][0][r];
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, (uint32_t)tid * 4u,
+                                                  base + (uint32_t)slice * image_bytes + (uint32_t)(r * kThreads * 4), kThrough);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this thread's part has been written through
+        __syncthreads();
+        int *arrived_s = reinterpret_cast<int *>(lds);
+        if (tid == 0)
+            *arrived_s = atomicAdd(a.sk_cnt + tile, 1);
+        __syncthreads();
+        const int arrived = __builtin_amdgcn_readfirstlane(*arrived_s);
+        __syncthreads(); // lds is reused by the epilogue
+        if (arrived != a.splitk - 1)
+            return;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            acc[0][0][r] = 0.0f;
+        for (int s0 = 0; s0 < a.splitk; s0 += 4) { // four slices (64 loads) in flight at a time
+            float p[4][16];
+#pragma unroll
+            for (int ds = 0; ds < 4; ds++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    p[ds][r] = (s0 + ds < a.splitk) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                          pr, (uint32_t)tid * 4u,
+                                                          base + (uint32_t)(s0 + ds) * image_bytes + (uint32_t)(r * kThreads * 4), kThrough))
+                                                    : 0.0f;
+#pragma unroll
+            for (int ds = 0; ds < 4; ds++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[0][0][r] += p[ds][r];
+        }
+    } else if (a.splitk > 1) { // raw partial sums in output order, reduced by splitk_reduce_kernel
         if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
             const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
 #pragma unroll
@@ -1858,6 +1902,9 @@ bool bf16_mfma_order(int order) { return order == GEMM_ORDER_TAP_BF16 || order =
 // kernel needs on the order of 1200 workgroups in flight to keep the matrix pipes of
 // 256 CUs busy, and a split only pays when every slice still has a long K loop
 // (the partial sums cost one extra pass over the output per slice).
+#ifndef DLP_SPLITK_MIN_KT
+#define DLP_SPLITK_MIN_KT 24
+#endif
 int choose_splitk(long long tiles, int nkt, int order)
 {
     if (bf16_mfma_order(order)) {
@@ -1875,7 +1922,7 @@ int choose_splitk(long long tiles, int nkt, int order)
     if (tiles >= 1000)
         return 1;
     long long s = (1200 + tiles / 2) / tiles; // round(1200 / tiles)
-    const long long max_by_k = nkt / 24;
+    const long long max_by_k = nkt / DLP_SPLITK_MIN_KT;
     if (s > max_by_k)
         s = max_by_k;
     if (s > 16)
@@ -1885,12 +1932,26 @@ int choose_splitk(long long tiles, int nkt, int order)
 
 bool generic_act(int activation) { return activation == DLP_ACT_TANH || activation == DLP_ACT_SIGMOID; }
 
+// Workspace of a split launch.  fp32-instruction kernels reduce in place: one counter per tile (256-byte
+// rounded) | one BM x BN accumulator image per tile and slice.  bf16-instruction kernels: partial sums
+// in output order, [slice][Cout][N], for splitk_reduce_kernel.
+size_t split_counter_bytes(long long tiles) { return (size_t)((tiles * sizeof(int) + 255) / 256 * 256); }
+size_t split_workspace_bytes(const GemmPlan &p, const GemmArgs &a, int groups, int s)
+{
+    if (s <= 1)
+        return 0;
+    if (bf16_mfma_order(p.order))
+        return (size_t)s * a.Cout * a.N * sizeof(float);
+    const long long tiles = (long long)a.mtiles * a.ntiles * groups;
+    return split_counter_bytes(tiles) + (size_t)tiles * s * p.BM * p.BN * sizeof(float);
+}
+
 void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t ws_bytes)
 {
     a.mtiles = p.mtiles;
     a.ntiles = (a.N + p.BN - 1) / p.BN;
     int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt, p.order);
-    if (s > 1 && (!have_ws || ws_bytes < (size_t)s * a.Cout * a.N * sizeof(float)))
+    if (s > 1 && (!have_ws || ws_bytes < split_workspace_bytes(p, a, groups, s)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
@@ -1906,7 +1967,7 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
         TimingScope ts("conv_gemm", stream);
         hipLaunchKernelGGL((conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
-    if (a.splitk > 1) {
+    if (a.splitk > 1 && a.sk_cnt == nullptr) {
         TimingScope ts("splitk_reduce", stream);
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
@@ -2259,7 +2320,7 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     a.Cout = g.Cout;
     a.nkt = p.nkt;
     plan_split(p, a, g.groups, true, (size_t)-1);
-    return p.wpack_bytes + (a.splitk > 1 ? (size_t)a.splitk * a.Cout * a.N * sizeof(float) : 0);
+    return p.wpack_bytes + split_workspace_bytes(p, a, g.groups, a.splitk);
 }
 
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
@@ -2276,6 +2337,17 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
             nzero = (int)ps.tiles;
         }
     }
+    if (!p.patch && !bf16_mfma_order(p.order) && part_ws != nullptr) { // counters of the in-place split-K reduction
+        GemmArgs a;
+        a.N = g.B * g.OH * g.OW;
+        a.Cout = g.Cout;
+        a.nkt = p.nkt;
+        plan_split(p, a, g.groups, true, part_bytes);
+        if (a.splitk > 1) {
+            zero = (int *)part_ws;
+            nzero = (int)((long long)a.mtiles * a.ntiles * g.groups);
+        }
+    }
     const long long total = (long long)g.groups * p.mtiles * p.nkt * (bf16_mfma_order(p.order) ? BK2 : BK) * p.BM;
     if (total >= 0x7fffffffLL * 256)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "weight tensor too large");
@@ -2289,7 +2361,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                                16 * (BK2 * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (bf16_t *)wpacked, zero, nzero);
         else if (g.dtype == DLP_BFLOAT16)
             hipLaunchKernelGGL((pack_weights_tap_kernel<bf16_t, float, BK, false>), grid, dim3(256),
-                               16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked, (int *)nullptr, 0);
+                               16 * (BK * khw + 1) * sizeof(bf16_t), stream, p, ncb, khw, (const bf16_t *)w, (float *)wpacked, zero, nzero);
         else
             hipLaunchKernelGGL((pack_weights_tap_kernel<float, float, BK, false>), grid, dim3(256),
                                16 * (BK * khw + 1) * sizeof(float), stream, p, ncb, khw, (const float *)w, (float *)wpacked, zero, nzero);
@@ -2298,7 +2370,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                            g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (bf16_t *)wpacked, zero, nzero);
     else if (g.dtype == DLP_BFLOAT16)
         hipLaunchKernelGGL(pack_weights_kernel<bf16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
-                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked, (int *)nullptr, 0);
+                           g.Cin / g.groups, g.KH * g.KW, (const bf16_t *)w, (float *)wpacked, zero, nzero);
     else
         hipLaunchKernelGGL(pack_weights_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, g.groups,
                            g.Cin / g.groups, g.KH * g.KW, (const float *)w, (float *)wpacked, zero, nzero);
@@ -2371,9 +2443,20 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     if (p.patch)
         return launch_patch(g, p, a, stream, part_ws, part_bytes);
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
-    {
+    a.sk_cnt = nullptr;
+    a.part_bytes = 0;
+    if (a.splitk > 1 && !bf16_mfma_order(p.order)) {
+        // reduced in place; the counters were cleared by conv_gemm_pack_weights (same workspace, a batch at least as large)
+        const long long tiles = (long long)a.mtiles * a.ntiles * g.groups;
+        const size_t images = split_workspace_bytes(p, a, g.groups, a.splitk) - split_counter_bytes(tiles);
+        if (images >= kOutOfRange)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K workspace of 2 GiB or more");
+        a.sk_cnt = (int *)part_ws;
+        a.sk_part = (float *)((char *)part_ws + split_counter_bytes(tiles));
+        a.sk_part_bytes = (uint32_t)images;
+    } else if (a.splitk > 1) {
         const size_t used = (size_t)a.splitk * a.Cout * a.N * sizeof(float);
-        a.part_bytes = (a.splitk > 1 && used < kOutOfRange) ? (uint32_t)used : 0;
+        a.part_bytes = used < kOutOfRange ? (uint32_t)used : 0;
     }
 
     a.pxv = 0;
