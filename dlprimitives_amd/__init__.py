@@ -16,7 +16,9 @@ from .capi import (  # noqa: F401
     NotImplementedErrorDlprim,
     Pooling2DForward,
     ValidationError,
+    activation_forward,
     build_library,
+    channel_affine_forward,
     conv2d_output_shape,
     eltwise_forward,
     lib,

@@ -329,3 +329,21 @@ def eltwise_forward(a, b, c, operation="sum", coef1=1.0, coef2=1.0, activation="
                                                     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     _check(lib().dlp_eltwise_fwd_enqueue_dtype(torch_dtype_code(a), ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation),
                                                a.numel(), _ptr(a), _ptr(b), _ptr(c), _stream(stream)))
+
+
+def activation_forward(x, y, activation, stream=None):
+    """Activation::forward: y = act(x); y may be x"""
+    lib().dlp_activation_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    _check(lib().dlp_activation_fwd_enqueue(torch_dtype_code(x), _act(activation), x.numel(), _ptr(x), _ptr(y), _stream(stream)))
+
+
+def channel_affine_forward(x, scale, shift, y, activation="identity", stream=None):
+    """BatchNorm::forward with fixed statistics: y[b,c,...] = act(x[b,c,...] * scale[c] + shift[c]); scale and shift are float32"""
+    if x.dim() < 2 or scale.numel() != x.shape[1] or shift.numel() != x.shape[1]:
+        raise ValidationError("channel_affine: scale/shift need one value per channel")
+    batch, channels = int(x.shape[0]), int(x.shape[1])
+    plane = x.numel() // max(batch * channels, 1)
+    lib().dlp_channel_affine_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    _check(lib().dlp_channel_affine_fwd_enqueue(torch_dtype_code(x), _act(activation), batch, channels, plane, _ptr(x), _ptr(scale), _ptr(shift),
+                                                _ptr(y), _stream(stream)))

@@ -210,6 +210,53 @@ __global__ __launch_bounds__(256) void eltwise_scalar_kernel(size_t n, int op, f
 }
 
 } // namespace
+
+// y = act(x): 16 bytes per thread and step over the aligned body, the tail one by one.
+template <class T>
+__global__ __launch_bounds__(256) void activation_kernel(size_t n, int act, const T *__restrict__ x, T *__restrict__ y, int vec_ok)
+{
+    constexpr int VEC = 16 / (int)sizeof(T);
+    struct alignas(16) Pack {
+        T v[VEC];
+    };
+    const size_t n16 = vec_ok ? n / VEC : 0;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = i; k < n16; k += stride) {
+        const Pack px = ((const Pack *)x)[k];
+        Pack py;
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            store_plain(&py.v[e], apply_act(to_float(px.v[e]), act));
+        ((Pack *)y)[k] = py;
+    }
+    for (size_t k = n16 * VEC + i; k < n; k += stride)
+        store_plain(y + k, apply_act(to_float(x[k]), act));
+}
+
+// y[b][c][i] = act(x[b][c][i] * scale[c] + shift[c]): batch normalisation with fixed statistics.
+// VEC elements per thread and step; with VEC > 1 the host guarantees plane % VEC == 0 (a pack never
+// straddles two channels) and 16-byte aligned tensors.
+template <class T, int VEC>
+__global__ __launch_bounds__(256) void channel_affine_kernel(size_t packs, int C, int plane_packs, int act, const T *__restrict__ x,
+                                                             const float *__restrict__ scale, const float *__restrict__ shift, T *__restrict__ y)
+{
+    struct alignas(VEC * sizeof(T)) Pack {
+        T v[VEC];
+    };
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < packs; k += stride) {
+        const int c = (int)((k / (size_t)plane_packs) % (size_t)C);
+        const float sc = scale[c], sh = shift[c];
+        const Pack px = ((const Pack *)x)[k];
+        Pack py;
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            store_plain(&py.v[e], apply_act(fmaf(to_float(px.v[e]), sc, sh), act));
+        ((Pack *)y)[k] = py;
+    }
+}
+
 } // namespace dlp
 
 using namespace dlp;
@@ -362,6 +409,67 @@ int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float c
                                   const void *b, void *c, void *stream)
 {
     return eltwise_launch(dtype, operation, coef1, coef2, activation, n, a, b, c, stream);
+}
+
+
+int dlp_activation_fwd_enqueue(int dtype, int activation, size_t n, const void *x, void *y, void *stream)
+{
+    DLP_REQUIRE(dtype == DLP_FLOAT || dtype == DLP_BFLOAT16, "float_data and bfloat16_data are implemented");
+    DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
+    if (n == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && y != nullptr, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int vec_ok = (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
+    const size_t per_block = 256 * (16 / dtype_size(dtype));
+    size_t blocks = (n + per_block - 1) / per_block;
+    if (blocks > 65536)
+        blocks = 65536;
+    TimingScope ts("activation", st);
+    if (dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(activation_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, n, activation, (const bf16_t *)x, (bf16_t *)y, vec_ok);
+    else
+        hipLaunchKernelGGL(activation_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, n, activation, (const float *)x, (float *)y, vec_ok);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale,
+                                   const float *shift, void *y, void *stream)
+{
+    DLP_REQUIRE(dtype == DLP_FLOAT || dtype == DLP_BFLOAT16, "float_data and bfloat16_data are implemented");
+    DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
+    DLP_REQUIRE(batch >= 0 && channels > 0 && plane > 0, "shape");
+    if (batch == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && y != nullptr && scale != nullptr && shift != nullptr, "null tensor pointer");
+    const size_t n = (size_t)batch * channels * plane;
+    hipStream_t st = (hipStream_t)stream;
+    const int vec = 16 / (dtype == DLP_BFLOAT16 ? 2 : 4);
+    const bool wide = plane % vec == 0 && (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
+    const size_t packs = wide ? n / vec : n;
+    const int plane_packs = wide ? plane / vec : plane;
+    size_t blocks = (packs + 255) / 256;
+    if (blocks > 256 * 32)
+        blocks = 256 * 32;
+    TimingScope ts("channel_affine", st);
+    if (dtype == DLP_BFLOAT16) {
+        if (wide)
+            hipLaunchKernelGGL((channel_affine_kernel<bf16_t, 8>), dim3((unsigned)blocks), dim3(256), 0, st, packs, channels, plane_packs,
+                               activation, (const bf16_t *)x, scale, shift, (bf16_t *)y);
+        else
+            hipLaunchKernelGGL((channel_affine_kernel<bf16_t, 1>), dim3((unsigned)blocks), dim3(256), 0, st, packs, channels, plane_packs,
+                               activation, (const bf16_t *)x, scale, shift, (bf16_t *)y);
+    } else {
+        if (wide)
+            hipLaunchKernelGGL((channel_affine_kernel<float, 4>), dim3((unsigned)blocks), dim3(256), 0, st, packs, channels, plane_packs,
+                               activation, (const float *)x, scale, shift, (float *)y);
+        else
+            hipLaunchKernelGGL((channel_affine_kernel<float, 1>), dim3((unsigned)blocks), dim3(256), 0, st, packs, channels, plane_packs,
+                               activation, (const float *)x, scale, shift, (float *)y);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
 }
 
 } // extern "C"

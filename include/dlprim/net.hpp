@@ -1,0 +1,699 @@
+// dlprim::Net, forward (predict) part, over the HIP operators of this library.
+//
+// Mirrors what dlprimitives' Net does for inference (include/dlprim/net.hpp:21-294, src/net.cpp):
+// it loads a network in the JSON format of docs/network_json_format.md (inputs / outputs / operators
+// with name, type, inputs, outputs, params, options), loads parameters from a DLPW file
+// (src/net.cpp:63-101 writer, :204-305 reader: "DLPW", big-endian header length, JSON header
+// {"tensors": {name: {dtype, shape, size, start}}}, raw data), infers shapes, plans tensor memory by
+// liveness (src/net.cpp:585-654: intermediate tensors share chunks unless keep_intermediate_tensors),
+// and runs the operators in order on one ExecutionContext with one shared workspace
+// (src/net.cpp:836-851).  Operator types: Convolution2D, BatchNorm, Activation, Pooling2D,
+// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- with the option
+// names of the reference's *Config::from_json functions.
+//
+// In predict mode two graph rewrites are applied at setup (fuse(true), the default):
+//  * a BatchNorm that is the only consumer of a Convolution2D / InnerProduct output is folded into its
+//    weights and bias: W' = W * gamma / sqrt(var + eps) per output channel, b' = beta + (b - mean) * scale
+//    (closed form of src/ops/batch_normalization.cpp:210-232);
+//  * an Activation that is the next user of the output of an operator with a fused activation slot
+//    (Convolution2D, InnerProduct, Elementwise, BatchNorm) whose activation is identity moves into that
+//    slot (the reference's ONNX importer does the same merge, src/importers/onnx.cpp:531-580).
+// Training, gradients and the other operator types are not part of this library.
+#pragma once
+#include <algorithm>
+#include <cmath>
+#include <fstream>
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "core/conv.hpp"
+#include "core/ip.hpp"
+#include "core/pool.hpp"
+#include "json.hpp"
+
+namespace dlprim {
+
+enum class CalculationsMode { train, predict };
+
+class Net {
+public:
+    explicit Net(Context &ctx) : ctx_(ctx) {}
+    Net(Net const &) = delete;
+    Net &operator=(Net const &) = delete;
+
+    void load_from_json_file(std::string const &name)
+    {
+        std::ifstream f(name);
+        if (!f)
+            throw ValidationError("Failed to open file " + name);
+        load_from_json(json::value::load(f));
+    }
+    void load_from_json(json::value const &v)
+    {
+        for (auto const &in : v["inputs"].array()) {
+            std::string dt = in.get("dtype", "float");
+            if (dt != "float")
+                throw NotImplementedError("input dtype " + dt);
+            std::vector<int> dims = in.get<std::vector<int>>("shape");
+            add_input_tensor(in.get<std::string>("name"), shape_of(dims));
+        }
+        for (auto const &op : v["operators"].array()) {
+            Node n;
+            n.name = op.get<std::string>("name");
+            n.type = op.get<std::string>("type");
+            n.inputs = op.get<std::vector<std::string>>("inputs");
+            n.outputs = op.get<std::vector<std::string>>("outputs");
+            if (!op.find("params").is_undefined())
+                n.param_names = op.get<std::vector<std::string>>("params");
+            n.options = op.find("options");
+            nodes_.push_back(std::move(n));
+        }
+        for (auto const &out : v["outputs"].array())
+            mark_output_tensor(out.type() == json::is_string ? out.str() : out.get<std::string>("name"));
+    }
+    void add_input_tensor(std::string const &name, Shape const &s)
+    {
+        input_names_.push_back(name);
+        specs_[name] = s;
+    }
+    void mark_output_tensor(std::string const &name) { output_names_.push_back(name); }
+
+    void mode(CalculationsMode m)
+    {
+        if (m != CalculationsMode::predict)
+            throw NotImplementedError("only CalculationsMode::predict is implemented");
+    }
+    CalculationsMode mode() const { return CalculationsMode::predict; }
+    // keep every tensor in memory of its own (no sharing between intermediate tensors)
+    void keep_intermediate_tensors(bool keep) { keep_intermediate_ = keep; }
+    bool keep_intermediate_tensors() const { return keep_intermediate_; }
+    // fold BatchNorm into the preceding convolution / inner product and merge activations (default on)
+    void fuse(bool on) { fuse_ = on; }
+
+    // shapes, rewrites, operators, memory; parameters are allocated (zero on the host) and wait for load_parameters
+    void setup()
+    {
+        infer_and_create_params();
+        if (fuse_)
+            rewrite_graph();
+        create_operators();
+        allocate_tensors();
+        ready_ = true;
+    }
+
+    void load_parameters(std::string const &file, bool allow_missing = false)
+    {
+        std::ifstream f(file, std::ios::binary);
+        if (!f)
+            throw ValidationError("Failed to open file " + file);
+        load_parameters(f, allow_missing);
+    }
+    void load_parameters(std::istream &f, bool allow_missing = false)
+    {
+        DLPRIM_CHECK(ready_);
+        char magic[4] = {0, 0, 0, 0};
+        unsigned char len_bytes[4] = {0, 0, 0, 0};
+        f.read(magic, 4);
+        f.read(reinterpret_cast<char *>(len_bytes), 4);
+        if (!f || std::string(magic, 4) != "DLPW")
+            throw ValidationError("Not a DLPW parameters file");
+        size_t len = (size_t(len_bytes[0]) << 24) | (size_t(len_bytes[1]) << 16) | (size_t(len_bytes[2]) << 8) | size_t(len_bytes[3]);
+        std::string header(len, '\0');
+        f.read(&header[0], (std::streamsize)len);
+        if (!f)
+            throw ValidationError("Truncated DLPW header");
+        json::value h = json::value::parse(header);
+        std::streamoff data_start = f.tellg();
+        std::set<std::string> loaded;
+        for (auto const &kv : h["tensors"].object()) {
+            auto p = params_.find(kv.first);
+            if (p == params_.end())
+                continue; // the file may hold more than this network uses
+            json::value const &ts = kv.second;
+            if (ts.get("dtype", "float") != "float")
+                throw NotImplementedError("parameter dtype of " + kv.first);
+            std::vector<int> dims = ts.get<std::vector<int>>("shape");
+            if (shape_of(dims).total_size() != p->second.shape().total_size())
+                throw ValidationError("Parameter " + kv.first + " has a different size in the file");
+            size_t bytes = ts.get<size_t>("size");
+            DLPRIM_CHECK(bytes == p->second.memory_size());
+            f.seekg(data_start + (std::streamoff)ts.get<size_t>("start"));
+            f.read(static_cast<char *>(p->second.host_data()), (std::streamsize)bytes);
+            if (!f)
+                throw ValidationError("Truncated DLPW data for " + kv.first);
+            loaded.insert(kv.first);
+        }
+        if (!allow_missing)
+            for (auto const &p : params_)
+                if (!loaded.count(p.first))
+                    throw ValidationError("No parameter " + p.first + " in the file");
+        copy_parameters_to_device();
+    }
+    void save_parameters(std::string const &file)
+    {
+        json::value header;
+        json::value &tensors = header["tensors"];
+        tensors.object();
+        size_t start = 0;
+        for (auto &p : params_) {
+            json::value &ts = tensors[p.first];
+            ts["dtype"] = json::value("float");
+            for (int i = 0; i < p.second.shape().size(); i++)
+                ts["shape"][size_t(i)] = json::value((size_t)p.second.shape()[i]);
+            ts["size"] = json::value(p.second.memory_size());
+            ts["start"] = json::value(start);
+            start += p.second.memory_size();
+        }
+        std::string text = header.save();
+        std::ofstream f(file, std::ios::binary);
+        f << "DLPW";
+        for (int i = 0; i < 4; i++)
+            f << (char)(0xFF & (text.size() >> (24 - i * 8)));
+        f << text;
+        for (auto &p : params_)
+            f.write(static_cast<char *>(p.second.host_data()), (std::streamsize)p.second.memory_size());
+        if (!f)
+            throw ValidationError("I/O error in saving to " + file);
+    }
+
+    // host copies of the parameters -> device (with the folded / derived forms the operators read)
+    void copy_parameters_to_device()
+    {
+        DLPRIM_CHECK(ready_);
+        ExecutionContext e = ctx_.make_execution_context();
+        for (auto &p : params_)
+            p.second.to_device(e);
+        for (auto &n : nodes_)
+            if (!n.skipped)
+                prepare_derived_parameters(n, e);
+        e.finish();
+    }
+
+    std::map<std::string, Tensor> &tensors() { return tensors_; }
+    std::map<std::string, Tensor> &params() { return params_; }
+    Tensor &tensor(std::string const &name)
+    {
+        auto p = tensors_.find(name);
+        if (p == tensors_.end())
+            throw ValidationError("Unknown tensor name:" + name);
+        return p->second;
+    }
+    Tensor &param(std::string const &name)
+    {
+        auto p = params_.find(name);
+        if (p == params_.end())
+            throw ValidationError("Unknown parameter name:" + name);
+        return p->second;
+    }
+    std::vector<std::string> const &input_names() { return input_names_; }
+    std::vector<std::string> const &output_names() { return output_names_; }
+    Tensor &input(unsigned id) { return tensor(input_names_.at(id)); }
+    Tensor &output(unsigned id) { return tensor(output_names_.at(id)); }
+
+    void forward(ExecutionContext const &e, bool sync = false)
+    {
+        DLPRIM_CHECK(ready_);
+        if (ctx_.is_cpu_context())
+            throw NotImplementedError("Net::forward needs a device context");
+        for (auto &n : nodes_)
+            if (!n.skipped)
+                run(n, e);
+        if (sync)
+            e.finish();
+    }
+
+    // bytes of device memory behind the tensors (after planning) and operators that run (after the rewrites)
+    size_t tensor_memory() const { return tensor_memory_; }
+    size_t operators_run() const
+    {
+        size_t c = 0;
+        for (auto const &n : nodes_)
+            c += n.skipped ? 0 : 1;
+        return c;
+    }
+
+private:
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip };
+    struct Node {
+        std::string name, type;
+        std::vector<std::string> inputs, outputs, param_names;
+        json::value options;
+        Kind kind = k_conv;
+        bool skipped = false;
+        StandardActivations activation = StandardActivations::identity;
+        // Convolution2D / InnerProduct
+        Convolution2DConfigBase conv;
+        bool bias = false;
+        std::string algo;
+        int ip_inputs = -1, ip_outputs = -1;
+        Node *folded_bn = nullptr; // BatchNorm folded into this operator
+        std::unique_ptr<core::Conv2DForward> conv_op;
+        std::unique_ptr<core::IPForward> ip_op;
+        Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
+        // BatchNorm
+        float eps = 1e-5f;
+        bool affine = true;
+        Tensor scale, shift;
+        // Pooling2D / GlobalPooling
+        int kernel[2] = {1, 1}, stride[2] = {1, 1}, pad[2] = {0, 0};
+        bool max_mode = true, count_include_pad = false, ceil_mode = false;
+        std::unique_ptr<core::Pooling2DForward> pool_op;
+        // Elementwise
+        int eltwise_op = DLP_ELTWISE_SUM;
+        float coef[2] = {1.0f, 1.0f};
+    };
+
+    static Shape shape_of(std::vector<int> const &d)
+    {
+        switch (d.size()) {
+        case 1: return Shape(size_t(d[0]));
+        case 2: return Shape(size_t(d[0]), d[1]);
+        case 3: return Shape(size_t(d[0]), d[1], d[2]);
+        case 4: return Shape(size_t(d[0]), d[1], d[2], d[3]);
+        default: throw NotImplementedError("tensors of rank " + std::to_string(d.size()));
+        }
+    }
+    static void pair_option(json::value const &o, char const *key, int (&dst)[2], bool required = false)
+    {
+        json::value const &v = o.find(key);
+        if (v.is_undefined()) {
+            if (required)
+                throw ValidationError(std::string("Missing option ") + key);
+            return;
+        }
+        if (v.type() == json::is_array) {
+            DLPRIM_CHECK(v.size() == 2);
+            dst[0] = (int)v[size_t(0)].number();
+            dst[1] = (int)v[size_t(1)].number();
+        } else
+            dst[0] = dst[1] = (int)v.number();
+    }
+    Shape const &spec(std::string const &name) const
+    {
+        auto p = specs_.find(name);
+        if (p == specs_.end())
+            throw ValidationError("Tensor " + name + " is used before it is produced");
+        return p->second;
+    }
+    std::string param_name(Node &n, size_t i)
+    {
+        if (n.param_names.size() <= i)
+            n.param_names.resize(i + 1);
+        if (n.param_names[i].empty())
+            n.param_names[i] = n.name + "." + std::to_string(i); // the reference's default naming
+        return n.param_names[i];
+    }
+    void make_param(Node &n, size_t i, Shape const &s)
+    {
+        std::string name = param_name(n, i);
+        auto p = params_.find(name);
+        if (p != params_.end()) { // shared parameter
+            DLPRIM_CHECK(p->second.shape() == s);
+            return;
+        }
+        Tensor t(ctx_, s);
+        std::fill(t.data<float>(), t.data<float>() + s.total_size(), 0.0f);
+        params_[name] = t;
+    }
+
+    void infer_and_create_params()
+    {
+        for (auto &n : nodes_) {
+            json::value const &o = n.options;
+            std::string act = o.type() == json::is_object ? o.get("activation", "identity") : "identity";
+            n.activation = activation_from_name(act);
+            if (n.type == "Convolution2D") {
+                n.kind = k_conv;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() == 4);
+                n.conv.channels_in = o.get("channels_in", int(in[1]));
+                n.conv.channels_out = o.get<int>("channels_out");
+                pair_option(o, "kernel", n.conv.kernel, true);
+                pair_option(o, "stride", n.conv.stride);
+                pair_option(o, "dilate", n.conv.dilate);
+                pair_option(o, "pad", n.conv.pad);
+                n.conv.groups = o.get("groups", 1);
+                n.bias = o.get("bias", true);
+                n.algo = o.get("fwd_algo", "auto");
+                if (n.algo == "auto")
+                    n.algo = "";
+                DLPRIM_CHECK(n.conv.channels_in == int(in[1]));
+                specs_[n.outputs[0]] = core::Conv2DBase::get_output_shape(n.conv, in);
+                make_param(n, 0, Shape(size_t(n.conv.channels_out), n.conv.channels_in / n.conv.groups, n.conv.kernel[0], n.conv.kernel[1]));
+                if (n.bias)
+                    make_param(n, 1, Shape(size_t(n.conv.channels_out)));
+            } else if (n.type == "InnerProduct") {
+                n.kind = k_ip;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                n.ip_inputs = o.get("inputs", int(in.size_no_batch()));
+                n.ip_outputs = o.get<int>("outputs");
+                n.bias = o.get("bias", true);
+                DLPRIM_CHECK(size_t(n.ip_inputs) == in.size_no_batch());
+                specs_[n.outputs[0]] = Shape(in[0], n.ip_outputs);
+                make_param(n, 0, Shape(size_t(n.ip_outputs), n.ip_inputs));
+                if (n.bias)
+                    make_param(n, 1, Shape(size_t(n.ip_outputs)));
+            } else if (n.type == "BatchNorm") {
+                n.kind = k_bn;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() >= 2);
+                int features = o.get("features", -1);
+                DLPRIM_CHECK(features == -1 || features == int(in[1]));
+                n.eps = o.get("eps", 1e-5f);
+                n.affine = o.get("affine", true);
+                specs_[n.outputs[0]] = in;
+                for (size_t i = 0; i < (n.affine ? 4u : 2u); i++) // running mean, running variance, gamma, beta
+                    make_param(n, i, Shape(in[1]));
+            } else if (n.type == "Activation") {
+                n.kind = k_act;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                specs_[n.outputs[0]] = spec(n.inputs[0]);
+            } else if (n.type == "Pooling2D") {
+                n.kind = k_pool;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() == 4);
+                pair_option(o, "kernel", n.kernel, true);
+                pair_option(o, "stride", n.stride);
+                pair_option(o, "pad", n.pad);
+                std::string mode = o.get("mode", "max");
+                DLPRIM_CHECK(mode == "max" || mode == "avg");
+                n.max_mode = mode == "max";
+                n.ceil_mode = o.get("ceil_mode", false);
+                n.count_include_pad = o.get("count_include_pad", false);
+                specs_[n.outputs[0]] = Shape(in[0], in[1], core::calc_pooling_output_size(int(in[2]), n.kernel[0], n.pad[0], n.stride[0], n.ceil_mode),
+                                             core::calc_pooling_output_size(int(in[3]), n.kernel[1], n.pad[1], n.stride[1], n.ceil_mode));
+            } else if (n.type == "GlobalPooling") {
+                n.kind = k_gpool;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() == 4);
+                std::string mode = o.get("mode", "max");
+                DLPRIM_CHECK(mode == "max" || mode == "avg");
+                n.max_mode = mode == "max";
+                specs_[n.outputs[0]] = Shape(in[0], in[1], 1, 1);
+            } else if (n.type == "Elementwise") {
+                n.kind = k_eltwise;
+                DLPRIM_CHECK(n.inputs.size() == 2 && n.outputs.size() == 1);
+                if (spec(n.inputs[0]) != spec(n.inputs[1]))
+                    throw NotImplementedError("Elementwise with broadcasting (" + n.name + ")");
+                std::string op = o.get("operation", "sum");
+                if (op == "sum")
+                    n.eltwise_op = DLP_ELTWISE_SUM;
+                else if (op == "prod")
+                    n.eltwise_op = DLP_ELTWISE_PROD;
+                else if (op == "max")
+                    n.eltwise_op = DLP_ELTWISE_MAX;
+                else
+                    throw ValidationError("Unsupported Elementwise operation " + op);
+                n.coef[0] = o.get("coef1", 1.0f);
+                n.coef[1] = o.get("coef2", 1.0f);
+                specs_[n.outputs[0]] = spec(n.inputs[0]);
+            } else
+                throw NotImplementedError("Operator type " + n.type + " (" + n.name + ")");
+        }
+        for (auto const &name : output_names_)
+            spec(name);
+    }
+
+    // index of the next node after `from` that reads or writes tensor `t`, or -1
+    int next_user(size_t from, std::string const &t) const
+    {
+        for (size_t i = from + 1; i < nodes_.size(); i++) {
+            if (nodes_[i].skipped)
+                continue;
+            for (auto const &s : nodes_[i].inputs)
+                if (s == t)
+                    return int(i);
+            for (auto const &s : nodes_[i].outputs)
+                if (s == t)
+                    return int(i);
+        }
+        return -1;
+    }
+    int readers_after(size_t from, std::string const &t) const
+    {
+        int c = 0;
+        for (size_t i = from + 1; i < nodes_.size(); i++) {
+            if (nodes_[i].skipped)
+                continue;
+            for (auto const &s : nodes_[i].inputs)
+                if (s == t)
+                    c++;
+            bool rewritten = false;
+            for (auto const &s : nodes_[i].outputs)
+                if (s == t && std::find(nodes_[i].inputs.begin(), nodes_[i].inputs.end(), t) == nodes_[i].inputs.end())
+                    rewritten = true;
+            if (rewritten)
+                break; // a new value under the same name
+        }
+        return c;
+    }
+    bool is_net_output(std::string const &t) const { return std::find(output_names_.begin(), output_names_.end(), t) != output_names_.end(); }
+
+    void rewrite_graph()
+    {
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            Node &p = nodes_[i];
+            if (p.skipped)
+                continue;
+            // BatchNorm into the convolution / inner product that feeds only it
+            if ((p.kind == k_conv || p.kind == k_ip) && p.activation == StandardActivations::identity && !p.folded_bn) {
+                std::string const &t = p.outputs[0];
+                int u = next_user(i, t);
+                if (u >= 0 && nodes_[u].kind == k_bn && nodes_[u].inputs[0] == t && !is_net_output(t) &&
+                    (nodes_[u].outputs[0] == t || readers_after(i, t) == 1)) {
+                    Node &bn = nodes_[u];
+                    p.folded_bn = &bn;
+                    p.activation = bn.activation;
+                    p.outputs[0] = bn.outputs[0];
+                    bn.skipped = true;
+                }
+            }
+            // Activation into the fused slot of its producer
+            if ((p.kind == k_conv || p.kind == k_ip || p.kind == k_eltwise || p.kind == k_bn) && p.activation == StandardActivations::identity) {
+                std::string const &t = p.outputs[0];
+                int u = next_user(i, t);
+                if (u >= 0 && nodes_[u].kind == k_act && nodes_[u].inputs[0] == t &&
+                    (nodes_[u].outputs[0] == t || (!is_net_output(t) && readers_after(i, t) == 1))) {
+                    Node &a = nodes_[u];
+                    p.activation = a.activation;
+                    p.outputs[0] = a.outputs[0];
+                    a.skipped = true;
+                }
+            }
+        }
+    }
+
+    void create_operators()
+    {
+        workspace_bytes_ = 0;
+        if (ctx_.is_cpu_context())
+            return; // shapes and the memory plan only: the operators exist on a device
+        for (auto &n : nodes_) {
+            if (n.skipped)
+                continue;
+            Shape const &in = spec(n.inputs[0]);
+            switch (n.kind) {
+            case k_conv: {
+                core::Conv2DSettings cfg(n.conv, in, float_data);
+                n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
+                workspace_bytes_ = std::max(workspace_bytes_, n.conv_op->workspace());
+                break;
+            }
+            case k_ip: {
+                core::IPSettings cfg;
+                cfg.inputs = n.ip_inputs;
+                cfg.outputs = n.ip_outputs;
+                cfg.optimal_batch_size = int(in[0]);
+                n.ip_op = core::IPForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation);
+                break;
+            }
+            case k_pool:
+                n.pool_op = n.max_mode ? core::Pooling2DForward::create_max_pooling(ctx_, n.kernel, n.pad, n.stride)
+                                       : core::Pooling2DForward::create_avg_pooling(ctx_, n.kernel, n.pad, n.stride, n.count_include_pad);
+                break;
+            case k_gpool:
+                n.pool_op = n.max_mode ? core::Pooling2DForward::create_global_max_pooling(ctx_, in)
+                                       : core::Pooling2DForward::create_global_avg_pooling(ctx_, in);
+                break;
+            default: break;
+            }
+        }
+        if (workspace_bytes_ > 0)
+            workspace_ = Tensor(ctx_, Shape(workspace_bytes_), uint8_data);
+    }
+
+    // Tensor memory.  Network inputs and outputs own their memory; an intermediate tensor takes the
+    // smallest free chunk that fits when its producer runs and gives it back after its last reader
+    // (an operator's outputs are placed before its inputs are released, so they never alias).
+    void allocate_tensors()
+    {
+        std::map<std::string, int> last_use;
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            if (nodes_[i].skipped)
+                continue;
+            for (auto const &t : nodes_[i].inputs)
+                last_use[t] = int(i);
+            for (auto const &t : nodes_[i].outputs)
+                last_use[t] = std::max(last_use.count(t) ? last_use[t] : -1, int(i));
+        }
+        tensor_memory_ = 0;
+        auto own = [&](std::string const &name) {
+            tensors_[name] = Tensor(ctx_, spec(name));
+            tensor_memory_ += tensors_[name].memory_size();
+        };
+        for (auto const &name : input_names_)
+            own(name);
+        struct Chunk {
+            Tensor mem;
+            size_t bytes;
+        };
+        std::vector<Chunk> free_chunks;
+        std::map<std::string, Chunk> held;
+        for (size_t i = 0; i < nodes_.size(); i++) {
+            Node &n = nodes_[i];
+            if (n.skipped)
+                continue;
+            for (auto const &t : n.outputs) {
+                if (tensors_.count(t))
+                    continue; // in place, or written before
+                if (keep_intermediate_ || is_net_output(t)) {
+                    own(t);
+                    continue;
+                }
+                const size_t bytes = spec(t).total_size() * sizeof(float);
+                int best = -1;
+                for (size_t c = 0; c < free_chunks.size(); c++)
+                    if (free_chunks[c].bytes >= bytes && (best < 0 || free_chunks[c].bytes < free_chunks[size_t(best)].bytes))
+                        best = int(c);
+                Chunk ch;
+                if (best >= 0) {
+                    ch = free_chunks[size_t(best)];
+                    free_chunks.erase(free_chunks.begin() + best);
+                } else {
+                    ch.mem = Tensor(ctx_, Shape(bytes), uint8_data);
+                    ch.bytes = bytes;
+                    tensor_memory_ += bytes;
+                }
+                tensors_[t] = ch.mem.sub_tensor(0, spec(t), float_data);
+                held[t] = ch;
+            }
+            std::set<std::string> touched(n.inputs.begin(), n.inputs.end());
+            touched.insert(n.outputs.begin(), n.outputs.end());
+            for (auto const &t : touched) {
+                auto h = held.find(t);
+                if (h != held.end() && last_use[t] == int(i)) {
+                    free_chunks.push_back(h->second);
+                    held.erase(h);
+                }
+            }
+        }
+        for (auto const &name : output_names_)
+            if (!tensors_.count(name))
+                throw ValidationError("Output tensor " + name + " is not produced by any operator");
+    }
+
+    void prepare_derived_parameters(Node &n, ExecutionContext const &e)
+    {
+        auto bn_scale_shift = [&](Node &bn, std::vector<float> &scale, std::vector<float> &shift) {
+            Tensor &mean = param(bn.param_names[0]), &var = param(bn.param_names[1]);
+            const size_t c = mean.shape().total_size();
+            scale.resize(c);
+            shift.resize(c);
+            for (size_t i = 0; i < c; i++) { // the order of operations of src/ops/batch_normalization.cpp:218-226
+                float alpha = 1.0f / std::sqrt(var.data<float>()[i] + bn.eps);
+                float beta = -mean.data<float>()[i] * alpha;
+                if (bn.affine) {
+                    const float g = param(bn.param_names[2]).data<float>()[i];
+                    alpha *= g;
+                    beta = g * beta + param(bn.param_names[3]).data<float>()[i];
+                }
+                scale[i] = alpha;
+                shift[i] = beta;
+            }
+        };
+        if (n.kind == k_bn) {
+            std::vector<float> scale, shift;
+            bn_scale_shift(n, scale, shift);
+            n.scale = Tensor(ctx_, Shape(scale.size()));
+            n.shift = Tensor(ctx_, Shape(shift.size()));
+            std::copy(scale.begin(), scale.end(), n.scale.data<float>());
+            std::copy(shift.begin(), shift.end(), n.shift.data<float>());
+            n.scale.to_device(e);
+            n.shift.to_device(e);
+        } else if ((n.kind == k_conv || n.kind == k_ip) && n.folded_bn) {
+            std::vector<float> scale, shift;
+            bn_scale_shift(*n.folded_bn, scale, shift);
+            Tensor &w = param(n.param_names[0]);
+            const size_t cout = scale.size(), per = w.shape().total_size() / cout;
+            n.w_dev = Tensor(ctx_, w.shape());
+            n.b_dev = Tensor(ctx_, Shape(cout));
+            for (size_t c = 0; c < cout; c++) {
+                for (size_t i = 0; i < per; i++)
+                    n.w_dev.data<float>()[c * per + i] = w.data<float>()[c * per + i] * scale[c];
+                const float b = n.bias ? param(n.param_names[1]).data<float>()[c] : 0.0f;
+                n.b_dev.data<float>()[c] = shift[c] + b * scale[c];
+            }
+            n.w_dev.to_device(e);
+            n.b_dev.to_device(e);
+        }
+    }
+
+    void run(Node &n, ExecutionContext const &e)
+    {
+        Tensor &x = tensor(n.inputs[0]);
+        Tensor &y = tensor(n.outputs[0]);
+        switch (n.kind) {
+        case k_conv: {
+            Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
+            Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
+            n.conv_op->enqueue(x, w, b, y, workspace_, 0.0f, e);
+            break;
+        }
+        case k_ip: {
+            Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
+            Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
+            n.ip_op->enqueue(x, w, b, y, e);
+            break;
+        }
+        case k_bn: {
+            Shape const &s = x.shape();
+            details::check_status(dlp_channel_affine_fwd_enqueue(int(float_data), int(n.activation), int(s[0]), int(s[1]),
+                                                                 int(s.total_size() / (s[0] * s[1])), x.device_ptr(),
+                                                                 static_cast<const float *>(n.scale.device_ptr()),
+                                                                 static_cast<const float *>(n.shift.device_ptr()), y.device_ptr(), e.stream()));
+            break;
+        }
+        case k_act:
+            details::check_status(dlp_activation_fwd_enqueue(int(float_data), int(n.activation), x.shape().total_size(), x.device_ptr(), y.device_ptr(),
+                                                             e.stream()));
+            break;
+        case k_pool:
+        case k_gpool: n.pool_op->enqueue(x, y, e); break;
+        case k_eltwise: {
+            Tensor &x1 = tensor(n.inputs[1]);
+            details::check_status(dlp_eltwise_fwd_enqueue(n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),
+                                                          x1.device_ptr(), y.device_ptr(), e.stream()));
+            break;
+        }
+        }
+    }
+
+    Context ctx_;
+    std::vector<Node> nodes_;
+    std::vector<std::string> input_names_, output_names_;
+    std::map<std::string, Shape> specs_;
+    std::map<std::string, Tensor> tensors_, params_;
+    Tensor workspace_;
+    size_t workspace_bytes_ = 0, tensor_memory_ = 0;
+    bool keep_intermediate_ = false, fuse_ = true, ready_ = false;
+};
+
+} // namespace dlprim

@@ -161,6 +161,16 @@ int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activat
 int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a,
                                   const void *b, void *c, void *stream);
 
+/* Activation::forward, src/ops/activation.cpp (cpu::apply_activation, include/dlprim/cpu/cpu_ops.hpp:17-53):
+ * y = act(x) over n elements stored as `dtype`; x == y (in place) is allowed. */
+int dlp_activation_fwd_enqueue(int dtype, int activation, size_t n, const void *x, void *y, void *stream);
+
+/* BatchNorm::forward with fixed statistics (predict mode / use_global_stats), src/ops/batch_normalization.cpp:161-232:
+ * y[b][c][i] = act(x[b][c][i] * scale[c] + shift[c]) with scale = gamma / sqrt(var + eps), shift = beta - mean * scale
+ * computed by the caller (fp32 device arrays of `channels` values); plane = H * W; x == y is allowed. */
+int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale,
+                                   const float *shift, void *y, void *stream);
+
 /* ===== data types ==================================================================
  * DLP_FLOAT: everything fp32, as in the reference (its conv/GEMM reject other types,
  * src/gemm.cpp:577,593).  DLP_BFLOAT16 (an extension): x, w, y of Conv2DForward and

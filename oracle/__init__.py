@@ -253,6 +253,23 @@ def eltwise_forward(a, b, op="sum", coef1=1.0, coef2=1.0, activation="identity")
     return c
 
 
+def batch_norm_forward(x, mean, var, gamma=None, beta=None, eps=1e-5, activation="identity"):
+    """BatchNorm::forward_cpu with fixed statistics (src/ops/batch_normalization.cpp:176-181): per channel
+    alpha = 1/sqrt(var + eps), beta' = -mean * alpha, with gamma/beta alpha *= gamma, beta' = gamma * beta' + beta
+    (compute_conv_parameters, :210-227), then y = alpha * x + beta' (cpu_forward_data, :196-206), all in float32,
+    and the operator's activation.  Pinned against torch.nn.functional.batch_norm in tests/test_glue_ops.py."""
+    x = _f32(x)
+    one = np.float32(1.0)
+    alpha = one / np.sqrt(_f32(var) + np.float32(eps))
+    shift = -_f32(mean) * alpha
+    if gamma is not None:
+        alpha = alpha * _f32(gamma)
+        shift = _f32(gamma) * shift + _f32(beta)
+    shape = (1, -1) + (1,) * (x.ndim - 2)
+    y = alpha.reshape(shape) * x + shift.reshape(shape)
+    return apply_activation(y.astype(np.float32), activation).reshape(x.shape)
+
+
 def bf16_round(a):
     a = _f32(a).copy()
     lib().orc_bf16_round_array(_ptr(a), ctypes.c_size_t(a.size))

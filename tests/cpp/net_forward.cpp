@@ -1,0 +1,164 @@
+// Driver for dlprim::Net (include/dlprim/net.hpp), used by tests/test_net.py the way dlprimitives'
+// own tools drive a network (tools/image_predict.cpp, docs/network_json_format.md):
+//
+//   net_forward json <file.json>
+//       parse and print the document again (no GPU)
+//   net_forward plan <net.json> [keep] [nofuse]
+//       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
+//       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [resave=<file.dlpw>] [repeat=<n>]
+//       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
+//       network's input order), runs forward and writes the outputs (float32, in output order)
+//   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse]
+//       random parameters and inputs, ms per forward pass on HIP device 0 (what the reference's
+//       tools/benchmark.cpp reports for its docs/nets_for_benchmark files)
+#include <dlprim/net.hpp>
+
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <chrono>
+#include <iostream>
+#include <random>
+#include <sstream>
+
+namespace dp = dlprim;
+
+static int usage()
+{
+    std::fprintf(stderr, "usage: net_forward json <file> | plan <net.json> [keep] [nofuse] | run <net.json> <params> <in.bin> <out.bin> [keep] [nofuse] [resave=<file>] [repeat=<n>] | time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse]\n");
+    return 2;
+}
+
+int main(int argc, char **argv)
+{
+    if (argc < 3)
+        return usage();
+    std::string cmd = argv[1];
+    try {
+        if (cmd == "json") {
+            std::ifstream f(argv[2]);
+            if (!f)
+                throw dp::ValidationError(std::string("cannot open ") + argv[2]);
+            dp::json::value v = dp::json::value::load(f);
+            std::cout << v.save() << std::endl;
+            return 0;
+        }
+        bool keep = false, fuse = true;
+        std::string resave;
+        int repeat = 1, warmup = 5, iters = 20;
+        const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
+        for (int i = first_flag; i < argc; i++) {
+            std::string a = argv[i];
+            if (a == "keep")
+                keep = true;
+            else if (a == "nofuse")
+                fuse = false;
+            else if (a.compare(0, 7, "resave=") == 0)
+                resave = a.substr(7);
+            else if (a.compare(0, 7, "repeat=") == 0)
+                repeat = std::atoi(a.c_str() + 7);
+            else if (a.compare(0, 7, "warmup=") == 0)
+                warmup = std::atoi(a.c_str() + 7);
+            else if (a.compare(0, 6, "iters=") == 0)
+                iters = std::atoi(a.c_str() + 6);
+            else
+                return usage();
+        }
+        if (cmd == "plan") {
+            dp::Context ctx(dp::Context::cpu);
+            dp::Net net(ctx);
+            net.keep_intermediate_tensors(keep);
+            net.fuse(fuse);
+            net.load_from_json_file(argv[2]);
+            net.setup();
+            std::printf("operators %zu tensor_memory %zu\n", net.operators_run(), net.tensor_memory());
+            for (auto const &name : net.output_names()) {
+                dp::Shape const &s = net.tensor(name).shape();
+                std::printf("tensor %s", name.c_str());
+                for (int i = 0; i < s.size(); i++)
+                    std::printf(" %zu", s[i]);
+                std::printf("\n");
+            }
+            return 0;
+        }
+        if (cmd == "time") {
+            dp::Context ctx(dp::Context::hip, 0, 0);
+            dp::Net net(ctx);
+            net.keep_intermediate_tensors(keep);
+            net.fuse(fuse);
+            net.load_from_json_file(argv[2]);
+            net.setup();
+            std::mt19937 rng(1);
+            for (auto &p : net.params()) {
+                dp::Shape const &s = p.second.shape();
+                const size_t n = s.total_size();
+                const bool variance = p.first.find("running_var") != std::string::npos;
+                // keeps activations of order one: weights scaled by fan-in, variances near one
+                const float range = s.size() > 1 ? std::sqrt(6.0f / float(n / s[0])) : 0.5f;
+                std::uniform_real_distribution<float> d(variance ? 0.5f : -range, variance ? 1.5f : range);
+                float *v = p.second.data<float>();
+                for (size_t i = 0; i < n; i++)
+                    v[i] = d(rng);
+            }
+            net.copy_parameters_to_device();
+            dp::ExecutionContext e = ctx.make_execution_context();
+            std::uniform_real_distribution<float> d(-1.0f, 1.0f);
+            for (unsigned i = 0; i < net.input_names().size(); i++) {
+                dp::Tensor &t = net.input(i);
+                float *v = t.data<float>();
+                for (size_t j = 0; j < t.shape().total_size(); j++)
+                    v[j] = d(rng);
+                t.to_device(e);
+            }
+            for (int i = 0; i < warmup; i++)
+                net.forward(e, false);
+            e.finish();
+            auto t0 = std::chrono::steady_clock::now();
+            for (int i = 0; i < iters; i++)
+                net.forward(e, false);
+            e.finish();
+            const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / iters;
+            const size_t batch = net.input(0).shape()[0];
+            std::printf("operators %zu tensor_memory %zu ms_per_forward %.4f images_per_s %.1f\nok\n", net.operators_run(), net.tensor_memory(), ms,
+                        batch * 1000.0 / ms);
+            return 0;
+        }
+        if (cmd != "run" || argc < 6)
+            return usage();
+        dp::Context ctx(dp::Context::hip, 0, 0);
+        dp::Net net(ctx);
+        net.keep_intermediate_tensors(keep);
+        net.fuse(fuse);
+        net.mode(dp::CalculationsMode::predict);
+        net.load_from_json_file(argv[2]);
+        net.setup();
+        net.load_parameters(argv[3]);
+        if (!resave.empty())
+            net.save_parameters(resave);
+        dp::ExecutionContext e = ctx.make_execution_context();
+        std::ifstream in(argv[4], std::ios::binary);
+        if (!in)
+            throw dp::ValidationError(std::string("cannot open ") + argv[4]);
+        for (unsigned i = 0; i < net.input_names().size(); i++) {
+            dp::Tensor &t = net.input(i);
+            in.read(static_cast<char *>(t.host_data()), (std::streamsize)t.memory_size());
+            if (!in)
+                throw dp::ValidationError("input file is too short");
+            t.to_device(e);
+        }
+        for (int r = 0; r < repeat; r++) // later passes must give what the first one gave: shared chunks are rewritten
+            net.forward(e, true);
+        std::ofstream out(argv[5], std::ios::binary);
+        for (unsigned i = 0; i < net.output_names().size(); i++) {
+            dp::Tensor &t = net.output(i);
+            t.to_host(e);
+            out.write(static_cast<char *>(t.host_data()), (std::streamsize)t.memory_size());
+        }
+        std::printf("operators %zu tensor_memory %zu\nok\n", net.operators_run(), net.tensor_memory());
+        return 0;
+    } catch (std::exception const &ex) {
+        std::fprintf(stderr, "error: %s\n", ex.what());
+        return 1;
+    }
+}

@@ -219,3 +219,70 @@ def test_gpu_eltwise_alignments_and_tails(oracle_mod, dtype):
         torch.cuda.synchronize()
         want = oracle_mod.eltwise_forward(a[off:], b[off:], "sum", 1.0, 1.0, "relu")
         np.testing.assert_allclose(c.float().cpu().numpy(), want, rtol=2 ** -8 if dtype == "bfloat16" else 1e-6, atol=1e-6)
+
+
+def test_oracle_batch_norm_matches_torch(oracle_mod):
+    """The oracle's fixed-statistics batch normalisation against torch's library routine (eval mode)."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((3, 7, 5, 4)).astype(np.float32)
+    mean, var = rng.standard_normal(7).astype(np.float32), rng.uniform(0.2, 3.0, 7).astype(np.float32)
+    gamma, beta = rng.standard_normal(7).astype(np.float32), rng.standard_normal(7).astype(np.float32)
+    for eps in (1e-5, 1e-2):
+        want = F.batch_norm(torch.from_numpy(x).double(), torch.from_numpy(mean).double(), torch.from_numpy(var).double(),
+                            torch.from_numpy(gamma).double(), torch.from_numpy(beta).double(), False, 0.0, eps).numpy()
+        np.testing.assert_allclose(oracle_mod.batch_norm_forward(x, mean, var, gamma, beta, eps), want, rtol=1e-5, atol=1e-5)
+        want = F.batch_norm(torch.from_numpy(x).double(), torch.from_numpy(mean).double(), torch.from_numpy(var).double(), None, None, False, 0.0, eps).numpy()
+        np.testing.assert_allclose(oracle_mod.batch_norm_forward(x, mean, var, eps=eps, activation="relu"), np.maximum(want, 0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_activation_forward(oracle_mod, dtype):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(12)
+    for n, off in [(1, 0), (4099, 0), (4099, 1), (37, 3), (1 << 20, 0)]:
+        x = oracle_mod.bf16_round(rng.uniform(-8, 8, n + off).astype(np.float32))
+        for act in ("identity", "relu", "tanh", "sigmoid", "relu6"):
+            tx = _dev(x).to(tdt)[off:]
+            y = torch.full((n + off,), float("nan"), device="cuda:0", dtype=tdt)[off:]
+            dlp.activation_forward(tx, y, act)
+            want = oracle_mod.apply_activation(x[off:], act)
+            np.testing.assert_allclose(y.float().cpu().numpy(), want, rtol=2 ** -8 if dtype == "bfloat16" else 1e-6, atol=1e-6)
+            dlp.activation_forward(tx, tx, act)  # in place
+            np.testing.assert_array_equal(tx.float().cpu().numpy(), y.float().cpu().numpy())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_channel_affine_is_batch_norm_with_fixed_statistics(oracle_mod, dtype):
+    """Planes that are and are not a multiple of the vector width, one-element planes (after global
+    pooling / inner product), more than 65535 planes, unaligned tensors, in place."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(13)
+    for shape, off, act in [((2, 5, 7, 9), 0, "relu"), ((3, 16, 8, 8), 0, "identity"), ((3, 16, 8, 8), 1, "relu6"), ((4, 9), 0, "tanh"),
+                            ((64, 2048, 2, 2), 0, "relu"), ((2, 3, 1, 24), 4, "sigmoid"), ((1, 1, 3, 1), 0, "identity")]:
+        n = int(np.prod(shape))
+        c = shape[1]
+        x = oracle_mod.bf16_round(rng.standard_normal(n + off).astype(np.float32))
+        mean, var = rng.standard_normal(c).astype(np.float32), rng.uniform(0.3, 2.0, c).astype(np.float32)
+        gamma, beta = rng.uniform(0.5, 1.5, c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+        alpha = (np.float32(1) / np.sqrt(var + np.float32(1e-5))) * gamma
+        shift = gamma * (-mean * (np.float32(1) / np.sqrt(var + np.float32(1e-5)))) + beta
+        tx = _dev(x).to(tdt)[off:].view(shape)
+        y = torch.full((n + off,), float("nan"), device="cuda:0", dtype=tdt)[off:].view(shape)
+        dlp.channel_affine_forward(tx, _dev(alpha), _dev(shift), y, act)
+        want = oracle_mod.batch_norm_forward(x[off:].reshape(shape), mean, var, gamma, beta, 1e-5, act)
+        np.testing.assert_allclose(y.float().cpu().numpy(), want, rtol=2 ** -7 if dtype == "bfloat16" else 1e-5, atol=2 ** -7 if dtype == "bfloat16" else 1e-5)
+        dlp.channel_affine_forward(tx, _dev(alpha), _dev(shift), tx, act)
+        np.testing.assert_array_equal(tx.float().cpu().numpy(), y.float().cpu().numpy())

@@ -1,0 +1,323 @@
+"""dlprim::Net (include/dlprim/net.hpp) through its driver tests/cpp/net_forward.cpp.
+
+CPU: the JSON reader/writer on documents python's json module writes and reads, the DLPW writer and
+reader of dlprimitives_amd.netfile, and shape inference + graph rewrites + the memory plan on a CPU
+context, for generated networks and (where the reference tree is present) for the reference's own
+docs/nets_for_benchmark/*.js.
+
+GPU: networks written in the reference's JSON + DLPW formats run through Net::forward and are compared
+with a float64 torch evaluation of the same operator list (BatchNorm unfused there), to 1e-4 of the
+output's largest magnitude; with and without the graph rewrites, with and without shared memory.
+"""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from dlprimitives_amd import netfile
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "bin", "net_forward")
+REF_NETS = "/root/reference/docs/nets_for_benchmark"
+
+
+def tool(*args, ok=True):
+    if not os.path.exists(BIN):
+        pytest.fail("tests/bin/net_forward is not built: run `make -C tests/cpp` (or __graft_entry__.build())")
+    r = subprocess.run([BIN] + [str(a) for a in args], capture_output=True, text=True, timeout=300)
+    if ok:
+        assert r.returncode == 0, r.stdout + r.stderr
+    return r
+
+
+# ---------------------------------------------------------------- json
+
+JSON_DOCS = [
+    {"a": 1, "b": [1, 2.5, -3e-7, 1e21, 0.1], "c": {"d": None, "e": True, "f": False}, "g": "text"},
+    {"esc": "quote\" backslash\\ slash/ tab\t nl\n cr\r bs\b ff\f", "uni": "é中\U0001F600", "ctl": "\u0001"},
+    [[], {}, [[]], [{}], "", 0, -0.0, 123456789012, 9.999999747378752e-06, 0.10000002384185791],
+    {"zeta": 1, "alpha": 2, "mid": 3},
+]
+
+
+@pytest.mark.parametrize("doc", JSON_DOCS, ids=range(len(JSON_DOCS)))
+@pytest.mark.parametrize("ascii_only", [True, False])
+def test_json_round_trip(tmp_path, doc, ascii_only):
+    p = tmp_path / "d.json"
+    p.write_text(json.dumps(doc, ensure_ascii=ascii_only, indent=2 if ascii_only else None), encoding="utf-8")
+    out = tool("json", p).stdout
+    back = json.loads(out)
+    assert back == doc
+    if isinstance(doc, dict):
+        assert list(back.keys()) == list(doc.keys())  # objects keep the order of their keys
+
+
+@pytest.mark.parametrize("text", ["{", "[1,]", '{"a" 1}', '{"a": tru}', '"open', "[1] x", "", '{"a": 1e}', '"\\u12"', "nul"])
+def test_json_rejects_malformed(tmp_path, text):
+    p = tmp_path / "bad.json"
+    p.write_text(text)
+    r = tool("json", p, ok=False)
+    assert r.returncode == 1 and "json" in r.stderr
+
+
+# ---------------------------------------------------------------- DLPW (python side)
+
+
+def test_dlpw_round_trip(tmp_path):
+    rng = np.random.default_rng(0)
+    tensors = {"w": rng.standard_normal((4, 3, 3, 3)).astype(np.float32), "b": rng.standard_normal(4).astype(np.float32), "s": np.float32([7])}
+    p = tmp_path / "t.dlpw"
+    netfile.save_dlpw(p, tensors)
+    raw = p.read_bytes()
+    assert raw[:4] == b"DLPW"
+    n = int.from_bytes(raw[4:8], "big")
+    header = json.loads(raw[8 : 8 + n])
+    assert list(header["tensors"]) == ["w", "b", "s"]
+    assert header["tensors"]["b"] == {"dtype": "float", "shape": [4], "size": 16, "start": 432}
+    assert len(raw) == 8 + n + sum(t.nbytes for t in tensors.values())
+    back = netfile.load_dlpw(p)
+    for k in tensors:
+        np.testing.assert_array_equal(back[k], tensors[k])
+
+
+# ---------------------------------------------------------------- plan (CPU context)
+
+
+def parse_plan(out):
+    lines = out.strip().splitlines()
+    head = lines[0].split()
+    info = {"operators": int(head[1]), "tensor_memory": int(head[3]), "tensors": {}}
+    for ln in lines[1:]:
+        parts = ln.split()
+        if parts[0] == "tensor":
+            info["tensors"][parts[1]] = tuple(int(v) for v in parts[2:])
+    return info
+
+
+def write_net(tmp_path, builder, name="net"):
+    p = tmp_path / (name + ".json")
+    p.write_text(json.dumps(builder.doc, indent=1))
+    return p
+
+
+def test_plan_resnet18_rewrites_and_memory(tmp_path):
+    b = netfile.resnet18(4, 64, 10)
+    p = write_net(tmp_path, b)
+    fused = parse_plan(tool("plan", p).stdout)
+    plain = parse_plan(tool("plan", p, "nofuse").stdout)
+    keep = parse_plan(tool("plan", p, "keep").stdout)
+    n_ops = len(b.doc["operators"])
+    assert plain["operators"] == n_ops == 20 + 20 + 9 + 1 + 8 + 1 + 1
+    # 20 BatchNorm folded, 9 Activation merged
+    assert fused["operators"] == 20 + 1 + 8 + 1 + 1
+    assert fused["tensors"] == {"loss": (4, 10)} == plain["tensors"]
+    # every tensor in memory of its own: the sum over all tensors the fused graph produces
+    names = {"data"}
+    for op in b.doc["operators"]:
+        names.update(op["outputs"])
+    all_bytes = sum(4 * int(np.prod(b.shapes[t])) for t in names)
+    assert keep["tensor_memory"] < all_bytes  # folded BatchNorm outputs are never materialised
+    # shared chunks: input + output + at most 3 live activations of the largest size
+    biggest = 4 * 4 * 64 * 32 * 32
+    assert fused["tensor_memory"] <= 4 * int(np.prod(b.shapes["data"])) + 4 * 4 * 10 + 3 * biggest
+    assert fused["tensor_memory"] < keep["tensor_memory"] / 2
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_NETS), reason="reference tree not present")
+@pytest.mark.parametrize("name", ["resnet18", "resnet50", "mobilenet_v2"])
+def test_builders_write_the_reference_operator_lists(name):
+    """Same operator types, in the same order, with the same options, as the reference's file."""
+    ref = json.load(open(os.path.join(REF_NETS, name + "-b16.js")))
+    mine = getattr(netfile, name)(16).doc
+    assert [i["shape"] for i in mine["inputs"]] == [i["shape"] for i in ref["inputs"]]
+    assert len(mine["operators"]) == len(ref["operators"])
+    for a, r in zip(mine["operators"], ref["operators"]):
+        assert a["type"] == r["type"], (a["name"], r["name"])
+        assert len(a["inputs"]) == len(r["inputs"]) and (a["inputs"] == a["outputs"]) == (r["inputs"] == r["outputs"])
+        for key in ("kernel", "stride", "pad", "groups", "channels_in", "channels_out", "bias", "mode", "activation", "operation", "inputs", "outputs"):
+            assert a["options"].get(key) == r["options"].get(key), (a["name"], r["name"], key)
+
+
+def test_plan_rejects_bad_networks(tmp_path):
+    b = netfile.NetBuilder("data", (1, 3, 8, 8))
+    b.conv("data", "c", 4, 3)
+    b.output("nothing")
+    r = tool("plan", write_net(tmp_path, b, "a"), ok=False)
+    assert r.returncode == 1 and "nothing" in r.stderr
+    b = netfile.NetBuilder("data", (1, 3, 8, 8))
+    b.conv("data", "c", 4, 3)
+    b.doc["operators"][0]["type"] = "Convolution3D"
+    b.output("c")
+    r = tool("plan", write_net(tmp_path, b, "b"), ok=False)
+    assert r.returncode == 1 and "Convolution3D" in r.stderr
+    b = netfile.NetBuilder("data", (1, 3, 8, 8))
+    b.conv("data", "c", 4, 3)
+    b.doc["operators"][0]["options"]["channels_in"] = 5
+    b.output("c")
+    assert tool("plan", write_net(tmp_path, b, "c"), ok=False).returncode == 1
+    b = netfile.NetBuilder("data", (1, 3, 8, 8))
+    b.conv("data", "c", 4, 3)
+    b.doc["operators"][0]["options"]["activation"] = "swish"
+    b.output("c")
+    assert tool("plan", write_net(tmp_path, b, "d"), ok=False).returncode == 1
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_NETS), reason="reference tree not present")
+@pytest.mark.parametrize(
+    "name,ops_fused",
+    [
+        ("resnet18-b16", 20 + 1 + 8 + 1 + 1),
+        ("resnet50-b16", 53 + 1 + 16 + 1 + 1),
+        ("mobilenet_v2-b16", 52 + 10 + 1 + 1),
+        ("alexnet-b16", 5 + 4 + 3),
+        ("vgg16-b16", 13 + 6 + 3),
+    ],
+)
+def test_plan_reference_benchmark_nets(name, ops_fused):
+    path = os.path.join(REF_NETS, name + ".js")
+    doc = json.load(open(path))
+    fused = parse_plan(tool("plan", path).stdout)
+    plain = parse_plan(tool("plan", path, "nofuse").stdout)
+    assert plain["operators"] == len(doc["operators"])
+    assert fused["operators"] == ops_fused
+    assert fused["tensors"] == {"loss": (16, 1000)}
+
+
+# ---------------------------------------------------------------- forward on the GPU
+
+
+def torch_forward(doc, params, inputs):
+    """float64 evaluation of the operator list, one torch call per operator, nothing fused."""
+    import torch
+    import torch.nn.functional as F
+
+    acts = {"identity": lambda v: v, "relu": torch.relu, "relu6": lambda v: torch.clamp(v, 0, 6), "tanh": torch.tanh, "sigmoid": torch.sigmoid}
+    t = {k: torch.from_numpy(np.asarray(v, dtype=np.float64)) for k, v in inputs.items()}
+    P = lambda n: torch.from_numpy(params[n].astype(np.float64))
+
+    def pair(v, d):
+        if v is None:
+            return d
+        return (v, v) if isinstance(v, int) else tuple(v)
+
+    for op in doc["operators"]:
+        o = op.get("options", {})
+        x = t[op["inputs"][0]]
+        kind = op["type"]
+        names = op.get("params", [])
+        if kind == "Convolution2D":
+            y = F.conv2d(x, P(names[0]), P(names[1]) if o.get("bias", True) else None, pair(o.get("stride"), (1, 1)), pair(o.get("pad"), (0, 0)),
+                         pair(o.get("dilate"), (1, 1)), o.get("groups", 1))
+        elif kind == "InnerProduct":
+            y = F.linear(x.reshape(x.shape[0], -1), P(names[0]), P(names[1]) if o.get("bias", True) else None)
+        elif kind == "BatchNorm":
+            affine = o.get("affine", True)
+            y = F.batch_norm(x, P(names[0]), P(names[1]), P(names[2]) if affine else None, P(names[3]) if affine else None, False, 0.0, o.get("eps", 1e-5))
+        elif kind == "Activation":
+            y = x
+        elif kind == "Pooling2D":
+            k, s, p = pair(o["kernel"], None), pair(o.get("stride"), (1, 1)), pair(o.get("pad"), (0, 0))
+            if o.get("mode", "max") == "max":
+                y = F.max_pool2d(x, k, s, p, ceil_mode=bool(o.get("ceil_mode", False)))
+            else:
+                y = F.avg_pool2d(x, k, s, p, ceil_mode=bool(o.get("ceil_mode", False)), count_include_pad=bool(o.get("count_include_pad", False)))
+        elif kind == "GlobalPooling":
+            y = x.amax((2, 3), keepdim=True) if o.get("mode", "max") == "max" else x.mean((2, 3), keepdim=True)
+        elif kind == "Elementwise":
+            a, b = x * o.get("coef1", 1.0), t[op["inputs"][1]] * o.get("coef2", 1.0)
+            y = {"sum": a + b, "prod": a * b, "max": torch.maximum(a, b)}[o.get("operation", "sum")]
+        else:
+            raise AssertionError(kind)
+        t[op["outputs"][0]] = acts[o.get("activation", "identity")](y)
+    return [t[n].numpy() for n in doc["outputs"]]
+
+
+def mixed_net():
+    """Every operator type and option form: scalar and pair options, bias and no bias, fused and
+    separate activations (in place and not), BatchNorm that folds and BatchNorm that cannot
+    (after pooling; feeding two readers; without affine), a dilated and a grouped convolution,
+    avg pooling with ceil mode, all three elementwise operations with coefficients, two inputs
+    and two outputs."""
+    b = netfile.NetBuilder("data", (3, 5, 23, 19))
+    b.input("side", (3, 12, 12, 10))
+    t = b.conv("data", "c0", 12, 3, 2, 1, bias=True, scalar_options=True)
+    t = b.bn(t, "c0n")  # folds
+    t = b.act(t, "relu", dst="c0a")  # separate output name, merges
+    u = b.eltwise(t, "side", "e0", "prod", coef1=0.5, coef2=-1.5, activation="tanh")
+    v = b.pool(u, "p0", "avg", 3, 2, 1, ceil_mode=True)
+    v = b.bn(v, "p0n", eps=1e-3, affine=False)  # stands alone (follows a pooling)
+    v = b.act(v, "sigmoid")  # merges into the BatchNorm's slot
+    w = b.conv(v, "c1", 12, (3, 1), 1, (2, 0), groups=3, dilate=(2, 1), activation="relu6")
+    w2 = b.bn(w, "c1n")  # cannot fold: the convolution has an activation
+    x = b.conv(v, "c2", 12, 1, bias=True)
+    xn = b.bn(x, "c2n")  # cannot fold: c2 has a second reader
+    m = b.eltwise(x, xn, "e1", "max")
+    s = b.eltwise(m, w2, "e2", "sum", coef2=0.25)
+    s = b.act(s, "relu")
+    q = b.pool(s, "p1", "max", 2, 2)
+    g = b.global_pool(q, "g0", "max")
+    h = b.global_pool(q, "g1", "avg")
+    gh = b.eltwise(g, h, "e3", "sum")
+    f = b.ip(q, "f0", 17, activation="relu")
+    f = b.ip(f, "f1", 9, bias=False)
+    f = b.bn(f, "f1n")  # folds into the inner product
+    b.output("f1n")
+    b.output("e3")
+    return b
+
+
+NETS = {
+    "mixed": (mixed_net, 5),
+    "resnet18_b2_64": (lambda: netfile.resnet18(2, 64, 10), 6),
+    "resnet50_b2_64": (lambda: netfile.resnet50(2, 64, 10), 8),
+    "mobilenet_v2_b3_64": (lambda: netfile.mobilenet_v2(3, 64, 10), 7),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("flags", [(), ("nofuse",), ("keep",), ("nofuse", "keep")], ids=["default", "nofuse", "keep", "nofuse_keep"])
+@pytest.mark.parametrize("net", list(NETS))
+def test_gpu_net_forward_matches_torch(tmp_path, net, flags):
+    make, seed = NETS[net]
+    b = make()
+    p = write_net(tmp_path, b)
+    params = b.random_parameters(seed)
+    netfile.save_dlpw(tmp_path / "w.dlpw", params)
+    rng = np.random.default_rng(seed + 100)
+    inputs = {i["name"]: rng.uniform(-1, 1, i["shape"]).astype(np.float32) for i in b.doc["inputs"]}
+    with open(tmp_path / "in.bin", "wb") as f:
+        for i in b.doc["inputs"]:
+            f.write(inputs[i["name"]].tobytes())
+    r = tool("run", p, tmp_path / "w.dlpw", tmp_path / "in.bin", tmp_path / "out.bin", "repeat=3", "resave=" + str(tmp_path / "again.dlpw"), *flags)
+    assert "ok" in r.stdout
+    want = torch_forward(b.doc, params, inputs)
+    got = np.fromfile(tmp_path / "out.bin", dtype=np.float32)
+    assert got.size == sum(w.size for w in want)
+    off = 0
+    for name, w in zip(b.doc["outputs"], want):
+        g = got[off : off + w.size].reshape(w.shape)
+        off += w.size
+        scale = np.abs(w).max()
+        assert scale > 1e-3, name
+        err = np.abs(g - w).max() / scale
+        print(net, flags, name, "max err / max |y| = %.3g" % err)
+        assert err < 1e-4, (name, err)
+    # the parameters the network wrote back are the ones it was given
+    again = netfile.load_dlpw(tmp_path / "again.dlpw")
+    assert set(again) == set(params)
+    for k in params:
+        np.testing.assert_array_equal(again[k].reshape(-1), params[k].reshape(-1))
+
+
+@pytest.mark.gpu
+def test_gpu_net_missing_parameter_is_an_error(tmp_path):
+    b = netfile.resnet18(1, 32, 4)
+    p = write_net(tmp_path, b)
+    params = b.random_parameters(1)
+    del params["fc.bias"]
+    netfile.save_dlpw(tmp_path / "w.dlpw", params)
+    np.zeros((1, 3, 32, 32), np.float32).tofile(tmp_path / "in.bin")
+    r = tool("run", p, tmp_path / "w.dlpw", tmp_path / "in.bin", tmp_path / "out.bin", ok=False)
+    assert r.returncode == 1 and "fc.bias" in r.stderr
