@@ -8,6 +8,8 @@ ctypes front end of the same C ABI, operating on torch device tensors.
 """
 from .capi import (  # noqa: F401
     ACTIVATIONS,
+    Conv2DBackwardData,
+    Conv2DBackwardFilter,
     Conv2DForward,
     Conv2DSettings,
     DlprimError,
@@ -17,6 +19,7 @@ from .capi import (  # noqa: F401
     Pooling2DForward,
     ValidationError,
     activation_forward,
+    bias_backward,
     build_library,
     channel_affine_forward,
     conv2d_output_shape,

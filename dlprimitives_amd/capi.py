@@ -85,6 +85,19 @@ def lib():
                                              ctypes.c_void_p]
         L.dlp_conv2d_fwd_destroy.argtypes = [ctypes.c_void_p]
         L.dlp_conv2d_fwd_destroy.restype = None
+        for kind in ("data", "filter"):
+            pre = "dlp_conv2d_bwd_%s_" % kind
+            getattr(L, pre + "create").argtypes = [ctypes.POINTER(_Settings), ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
+            getattr(L, pre + "algo").restype = ctypes.c_char_p
+            getattr(L, pre + "algo").argtypes = [ctypes.c_void_p]
+            getattr(L, pre + "workspace").restype = ctypes.c_size_t
+            getattr(L, pre + "workspace").argtypes = [ctypes.c_void_p]
+            getattr(L, pre + "enqueue").argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                    ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_void_p]
+            getattr(L, pre + "destroy").argtypes = [ctypes.c_void_p]
+            getattr(L, pre + "destroy").restype = None
+        L.dlp_bias_bwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float,
+                                           ctypes.c_void_p]
         L.dlp_conv2d_output_shape.argtypes = [ctypes.POINTER(_Settings), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.dlp_ip_fwd_create.argtypes = [ctypes.POINTER(_IPSettings), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
         L.dlp_ip_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -214,6 +227,63 @@ class Conv2DForward:
         if getattr(self, "_h", None):
             lib().dlp_conv2d_fwd_destroy(self._h)
             self._h = None
+
+
+class _Conv2DBackward:
+    _kind = None
+
+    def __init__(self, handle, settings):
+        self._h = handle
+        self.settings = settings
+
+    @classmethod
+    def create(cls, settings, algo=""):
+        h = ctypes.c_void_p()
+        c = settings._c()
+        _check(getattr(lib(), "dlp_conv2d_bwd_%s_create" % cls._kind)(ctypes.byref(c), (algo or "").encode(), ctypes.byref(h)))
+        return cls(h, settings)
+
+    def algo(self):
+        return getattr(lib(), "dlp_conv2d_bwd_%s_algo" % self._kind)(self._h).decode()
+
+    def workspace(self):
+        return int(getattr(lib(), "dlp_conv2d_bwd_%s_workspace" % self._kind)(self._h))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            getattr(lib(), "dlp_conv2d_bwd_%s_destroy" % self._kind)(self._h)
+            self._h = None
+
+
+class Conv2DBackwardData(_Conv2DBackward):
+    """core::Conv2DBackwardData"""
+
+    _kind = "data"
+
+    def enqueue(self, dx, w, dy, ws=None, factor=0.0, stream=None):
+        """dx = factor * dx + gradient with respect to x; ws: uint8 tensor of >= workspace() bytes"""
+        xs = (ctypes.c_int * 4)(*dx.shape)
+        ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
+        _check(lib().dlp_conv2d_bwd_data_enqueue(self._h, xs, _ptr(dx), _ptr(w), _ptr(dy), _ptr(ws), ws_bytes, float(factor), _stream(stream)))
+
+
+class Conv2DBackwardFilter(_Conv2DBackward):
+    """core::Conv2DBackwardFilter"""
+
+    _kind = "filter"
+
+    def enqueue(self, x, dw, dy, ws=None, factor=0.0, stream=None):
+        """dw = factor * dw + gradient with respect to the filter"""
+        xs = (ctypes.c_int * 4)(*x.shape)
+        ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
+        _check(lib().dlp_conv2d_bwd_filter_enqueue(self._h, xs, _ptr(x), _ptr(dw), _ptr(dy), _ptr(ws), ws_bytes, float(factor), _stream(stream)))
+
+
+def bias_backward(dy, db, beta=0.0, stream=None):
+    """core::BiasBackwardFilter::enqueue: db[f] = beta * db[f] + sum of dy[:, f] over batch and plane"""
+    batch, features = int(dy.shape[0]), int(dy.shape[1])
+    plane = dy.numel() // max(batch * features, 1) if batch else 1
+    _check(lib().dlp_bias_bwd_enqueue(torch_dtype_code(dy), batch, features, max(plane, 1), _ptr(dy), _ptr(db), float(beta), _stream(stream)))
 
 
 class IPSettings:

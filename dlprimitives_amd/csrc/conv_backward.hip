@@ -1,0 +1,561 @@
+// Gradients of the 2D convolution: with respect to the input (backward data), the filter
+// (backward filter) and the bias.
+//
+// Replaces core::Conv2DBackwardData / core::Conv2DBackwardFilter (include/dlprim/core/conv.hpp:60-80,
+// src/core/conv.cpp:113-220,299-434,512-669) and core::BiasBackwardFilter (src/core/bias.cpp) of
+// dlprimitives; the arithmetic contract is the CPU one, src/ops/conv2d.cpp:411-435,475-498 and
+// src/ops/bwd_bias.cpp:34-60: result = factor * old + gradient.
+//
+//  * backward data is a forward convolution of dy with the filter transposed within its group and
+//    flipped in both axes, stride 1, padding dilate * (kernel - 1) - pad; it runs on the forward
+//    operator of this library (every algorithm and tile shape of the forward path serves it).  For
+//    stride > 1, dy is first spread out with zeros between its elements (workspace), so that the same
+//    stride-1 convolution applies; the matrix cores then multiply the inserted zeros as well.
+//  * backward filter is a GEMM of its own: dW[Cout_g x Cin_g*KH*KW] = dy[Cout_g x B*OH*OW] *
+//    cols[B*OH*OW x Cin_g*KH*KW], reduction over the pixels of all images.  Both operands are
+//    contiguous along the reduction index in memory, so a workgroup stages 64 pixels of BM dy rows and
+//    BN gathered x rows in LDS (lane = pixel: coalesced loads, conflict-free stores) and every lane
+//    fetches its four k values of a row with one 16-byte LDS read.  The reduction is cut into slices
+//    across workgroups; the slices' partial tiles go to the workspace in output order and one small
+//    kernel adds them up in slice order (deterministic).
+#include <algorithm>
+#include <new>
+#include <string>
+
+#include "dlp_internal.hpp"
+
+namespace dlp {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int KC = 64;        // pixels per staged chunk (one per lane)
+constexpr int PITCH = KC + 4; // LDS row pitch in floats: 16-byte reads of 8 consecutive lanes cover all banks
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+struct WgradArgs {
+    const float *x, *dy;
+    float *out; // dW itself (one slice) or the partial sums [slice][Cout][Ncol]
+    int Cin, Cin_g, Cout, Cout_g, groups, H, W, OW, OHW, KH, KW, sh, sw, ph, pw, dh, dw;
+    int Ncol; // Cin_g * KH * KW
+    int mtiles, ntiles, slices, chunks, cpi, cps; // chunks in all, per image, per slice
+    uint32_t x_bytes, dy_bytes;
+    uint32_t ow_magic, ow_shift, khw_magic, khw_shift, kw_magic, kw_shift, cpi_magic, cpi_shift;
+    float factor;
+};
+
+// dW tile of BM filters x BN (channel, tap) columns over the chunks of one slice.
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
+{
+    constexpr int TM = BM / 64, TN = BN / 64; // 32x32 MFMA blocks per wavefront (wavefronts 2 x 2)
+    constexpr int RA = BM / 4, RB = BN / 4;   // rows each wavefront stages
+    __shared__ __attribute__((aligned(16))) float As[BM * PITCH];
+    __shared__ __attribute__((aligned(16))) float Bs[BN * PITCH];
+    __shared__ __attribute__((aligned(16))) int rowtab[BN * 4]; // per column: x offset of the tap, dy, dx, valid
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    int t = blockIdx.x; // tile fastest: workgroups that share a slice (the same dy / x data) are neighbours
+    const int mt = t % a.mtiles;
+    t /= a.mtiles;
+    const int nt = t % a.ntiles;
+    t /= a.ntiles;
+    const int g = t % a.groups;
+    const int slice = t / a.groups;
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int ck_begin = slice * a.cps;
+    const int ck_end = min(ck_begin + a.cps, a.chunks);
+
+    if (tid < BN) {
+        const int n = n0 + tid;
+        const uint32_t c = fast_div((uint32_t)n, a.khw_magic, a.khw_shift);
+        const int rs = n - (int)c * a.KH * a.KW;
+        const int r = (int)fast_div((uint32_t)rs, a.kw_magic, a.kw_shift);
+        const int s = rs - r * a.KW;
+        const int dr = r * a.dh - a.ph, ds = s * a.dw - a.pw;
+        rowtab[tid * 4 + 0] = ((int)c * a.H + dr) * a.W + ds;
+        rowtab[tid * 4 + 1] = dr;
+        rowtab[tid * 4 + 2] = ds;
+        rowtab[tid * 4 + 3] = n < a.Ncol ? 1 : 0;
+    }
+    __syncthreads();
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void *)a.dy, 0, a.dy_bytes, 0x00020000);
+
+    float ra[RA], rb[RB];
+    // one chunk: 64 pixels (this lane's is pix0 + lane) of image b; rows wave, wave + 4, ...
+    auto fetch = [&](int ck) {
+        const int b = (int)fast_div((uint32_t)ck, a.cpi_magic, a.cpi_shift);
+        const int pix = (ck - b * a.cpi) * KC + lane;
+        const bool pv = pix < a.OHW;
+        const int oh = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+        const int ow = pix - oh * a.OW;
+        const int ohs = oh * a.sh, ows = ow * a.sw;
+        const uint32_t ybase = (uint32_t)((b * a.Cout + g * a.Cout_g + m0 + wave) * a.OHW + pix) * 4u;
+#pragma unroll
+        for (int i = 0; i < RA; i++) {
+            const bool ok = pv && (m0 + wave + 4 * i < a.Cout_g);
+            ra[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, ok ? ybase : kOutOfRange, (uint32_t)(4 * i * a.OHW) * 4u, 0));
+        }
+        const int xbase = (b * a.Cin + g * a.Cin_g) * a.H * a.W + ohs * a.W + ows;
+#pragma unroll
+        for (int i = 0; i < RB; i++) {
+            const int4 rt = *reinterpret_cast<const int4 *>(&rowtab[(wave + 4 * i) * 4]);
+            const bool ok = pv && rt.w != 0 && (unsigned)(ohs + rt.y) < (unsigned)a.H && (unsigned)(ows + rt.z) < (unsigned)a.W;
+            rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? (uint32_t)(xbase + rt.x) * 4u : kOutOfRange, 0, 0));
+        }
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    if (ck_begin < ck_end)
+        fetch(ck_begin);
+    for (int ck = ck_begin; ck < ck_end; ck++) {
+        __syncthreads(); // the previous chunk has been read
+#pragma unroll
+        for (int i = 0; i < RA; i++)
+            As[(wave + 4 * i) * PITCH + lane] = ra[i];
+#pragma unroll
+        for (int i = 0; i < RB; i++)
+            Bs[(wave + 4 * i) * PITCH + lane] = rb[i];
+        __syncthreads();
+        if (ck + 1 < ck_end)
+            fetch(ck + 1); // lands while this chunk is multiplied
+        // k order inside a chunk: MFMA step 4*kq + e takes pixel 8*kq + e from the lower half-wave and
+        // 8*kq + 4 + e from the upper one, for both operands alike
+#pragma unroll
+        for (int kq = 0; kq < KC / 8; kq++) {
+            f32x4 av[TM], bv[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                av[i] = *reinterpret_cast<const f32x4 *>(&As[(wm * (BM / 2) + i * 32 + l32) * PITCH + kq * 8 + h * 4]);
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                bv[j] = *reinterpret_cast<const f32x4 *>(&Bs[(wn * (BN / 2) + j * 32 + l32) * PITCH + kq * 8 + h * 4]);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // accumulator element r of block (i, j): row 8 * (r / 4) + r % 4 + 4 * h, column l32
+    const bool direct = a.slices == 1;
+    float *dst = a.out + (direct ? (size_t)0 : (size_t)slice * a.Cout * a.Ncol);
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * (BN / 2) + j * 32 + l32;
+        if (n >= a.Ncol)
+            continue;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + (r & 3) + 4 * h;
+                if (m < a.Cout_g) {
+                    float *p = dst + (size_t)(g * a.Cout_g + m) * a.Ncol + n;
+                    const float v = acc[i][j][r];
+                    if (direct && a.factor != 0.0f)
+                        *p = fmaf(*p, a.factor, v);
+                    else
+                        *p = v;
+                }
+            }
+    }
+}
+
+// out[i] = factor * out[i] + sum over slices, in slice order
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ out, size_t n, int slices, float factor)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float s = 0.0f;
+        int k = 0;
+        for (; k + 4 <= slices; k += 4) {
+            const float v0 = part[(size_t)k * n + i], v1 = part[(size_t)(k + 1) * n + i], v2 = part[(size_t)(k + 2) * n + i],
+                        v3 = part[(size_t)(k + 3) * n + i];
+            s = (((s + v0) + v1) + v2) + v3;
+        }
+        for (; k < slices; k++)
+            s += part[(size_t)k * n + i];
+        out[i] = factor != 0.0f ? fmaf(out[i], factor, s) : s;
+    }
+}
+
+// wt[g][c][k][KH-1-r][KW-1-s] = w[g][k][c][r][s]: the filter of the stride-1 convolution that maps dy to dx
+__global__ __launch_bounds__(256) void filter_transpose_flip_kernel(const float *__restrict__ w, float *__restrict__ wt, int groups, int cout_g, int cin_g,
+                                                                    int khw)
+{
+    const size_t n = (size_t)groups * cout_g * cin_g * khw;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const int rs = (int)(i % khw);
+        size_t q = i / khw;
+        const int c = (int)(q % cin_g);
+        q /= cin_g;
+        const int k = (int)(q % cout_g);
+        const int g = (int)(q / cout_g);
+        wt[(((size_t)g * cin_g + c) * cout_g + k) * khw + (khw - 1 - rs)] = w[i];
+    }
+}
+
+// up[p][hu][wu] = dy[p][hu / sh][wu / sw] where both divide and the quotient is inside dy, else 0
+__global__ __launch_bounds__(256) void spread_with_zeros_kernel(const float *__restrict__ dy, float *__restrict__ up, size_t planes, int OH, int OW, int Hu,
+                                                                int Wu, int sh, int sw)
+{
+    const size_t n = planes * Hu * Wu;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const int wu = (int)(i % Wu);
+        const size_t q = i / Wu;
+        const int hu = (int)(q % Hu);
+        const size_t p = q / Hu;
+        const int oh = hu / sh, ow = wu / sw;
+        float v = 0.0f;
+        if (oh * sh == hu && ow * sw == wu && oh < OH && ow < OW)
+            v = dy[(p * OH + oh) * OW + ow];
+        up[i] = v;
+    }
+}
+
+// db[f] = beta * db[f] + sum over batch and plane of dy[b][f][:]; one workgroup per feature
+__global__ __launch_bounds__(256) void bias_backward_kernel(const float *__restrict__ dy, float *__restrict__ db, int batch, int features, int plane, float beta)
+{
+    __shared__ float partial[4];
+    const int f = blockIdx.x;
+    float s = 0.0f;
+    for (int b = 0; b < batch; b++) {
+        const float *p = dy + ((size_t)b * features + f) * plane;
+        for (int i = threadIdx.x; i < plane; i += 256)
+            s += p[i];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+        s += __shfl_down(s, off);
+    if ((threadIdx.x & 63) == 0)
+        partial[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float v = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+        db[f] = beta != 0.0f ? fmaf(db[f], beta, v) : v;
+    }
+}
+
+size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+unsigned grid_for(size_t n)
+{
+    size_t blocks = (n + 255) / 256;
+    return (unsigned)std::min<size_t>(std::max<size_t>(blocks, 1), 256 * 32);
+}
+
+struct WgradPlan {
+    int BM, BN, mtiles, ntiles, cpi, chunks, cps, slices;
+    size_t part_bytes;
+};
+
+// Slices: enough workgroups for four per compute unit, at least two chunks each.
+WgradPlan wgrad_plan(const dlp_conv2d_settings &c, int batch, int OH, int OW)
+{
+    WgradPlan p;
+    const int cout_g = c.channels_out / c.groups, ncol = c.channels_in / c.groups * c.kernel[0] * c.kernel[1];
+    p.BM = cout_g > 64 ? 128 : 64;
+    p.BN = ncol > 64 ? 128 : 64;
+    p.mtiles = (cout_g + p.BM - 1) / p.BM;
+    p.ntiles = (ncol + p.BN - 1) / p.BN;
+    p.cpi = (OH * OW + KC - 1) / KC;
+    p.chunks = batch * p.cpi;
+    const long long tiles = (long long)p.mtiles * p.ntiles * c.groups;
+    long long want = std::max<long long>(1, 1024 / tiles);
+    want = std::min<long long>(want, std::max(1, p.chunks / 2));
+    p.cps = (int)((p.chunks + want - 1) / want);
+    p.slices = (p.chunks + p.cps - 1) / p.cps;
+    p.part_bytes = p.slices > 1 ? (size_t)p.slices * c.channels_out * ncol * sizeof(float) : 0;
+    return p;
+}
+
+} // namespace
+} // namespace dlp
+
+using namespace dlp;
+
+struct dlp_conv2d_bwd_data {
+    dlp_conv2d_settings cfg;
+    dlp_conv2d_fwd *fwd; // the stride-1 convolution dy -> dx
+    int OH, OW, Hu, Wu;  // dy, and dy spread out by the stride (== dy for stride 1)
+    bool spread;
+    size_t wt_bytes, fwd_ws;
+};
+
+struct dlp_conv2d_bwd_filter {
+    dlp_conv2d_settings cfg;
+    int OH, OW;
+};
+
+static int check_settings(const dlp_conv2d_settings *cfg, int out[4])
+{
+    DLP_REQUIRE(cfg != nullptr, "null argument");
+    DLP_REQUIRE(cfg->channels_in > 0 && cfg->channels_out > 0 && cfg->groups > 0, "channels/groups must be positive");
+    DLP_REQUIRE(cfg->channels_in % cfg->groups == 0 && cfg->channels_out % cfg->groups == 0, "channels not divisible by groups");
+    if (cfg->dtype != DLP_FLOAT)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution gradients: float_data is implemented");
+    return dlp_conv2d_output_shape(cfg, cfg->shape, out);
+}
+
+extern "C" {
+
+int dlp_conv2d_bwd_data_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_data **out)
+{
+    DLP_REQUIRE(out != nullptr, "null argument");
+    *out = nullptr;
+    int oshape[4];
+    int rc = check_settings(cfg, oshape);
+    if (rc != DLP_OK)
+        return rc;
+    dlp_conv2d_settings t = *cfg;
+    t.channels_in = cfg->channels_out;
+    t.channels_out = cfg->channels_in;
+    bool spread = false;
+    for (int i = 0; i < 2; i++) {
+        t.stride[i] = 1;
+        t.pad[i] = cfg->dilate[i] * (cfg->kernel[i] - 1) - cfg->pad[i];
+        if (t.pad[i] < 0)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "backward data: padding larger than dilate * (kernel - 1)");
+        // size of dy spread by the stride, with the rows/columns the forward window never reached
+        t.shape[2 + i] = cfg->shape[2 + i] + 2 * cfg->pad[i] - cfg->dilate[i] * (cfg->kernel[i] - 1);
+        spread = spread || cfg->stride[i] != 1;
+    }
+    t.shape[1] = cfg->channels_out;
+    dlp_conv2d_bwd_data *op = new (std::nothrow) dlp_conv2d_bwd_data();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *cfg;
+    op->OH = oshape[2];
+    op->OW = oshape[3];
+    op->Hu = t.shape[2];
+    op->Wu = t.shape[3];
+    op->spread = spread;
+    op->fwd = nullptr;
+    rc = dlp_conv2d_fwd_create(&t, 0, DLP_ACT_IDENTITY, algo, &op->fwd);
+    if (rc != DLP_OK) {
+        delete op;
+        return rc;
+    }
+    op->wt_bytes = round256((size_t)cfg->channels_out * (cfg->channels_in / cfg->groups) * cfg->kernel[0] * cfg->kernel[1] * sizeof(float));
+    op->fwd_ws = round256(dlp_conv2d_fwd_workspace(op->fwd));
+    *out = op;
+    return DLP_OK;
+}
+
+const char *dlp_conv2d_bwd_data_algo(const dlp_conv2d_bwd_data *op) { return op ? dlp_conv2d_fwd_algo(op->fwd) : ""; }
+
+static size_t bwd_data_spread_bytes(const dlp_conv2d_bwd_data *op, int batch)
+{
+    return op->spread ? round256((size_t)batch * op->cfg.channels_out * op->Hu * op->Wu * sizeof(float)) : 0;
+}
+
+size_t dlp_conv2d_bwd_data_workspace(const dlp_conv2d_bwd_data *op)
+{
+    return op ? op->wt_bytes + bwd_data_spread_bytes(op, std::max(op->cfg.shape[0], 1)) + op->fwd_ws : 0;
+}
+
+int dlp_conv2d_bwd_data_enqueue(dlp_conv2d_bwd_data *op, const int x_shape[4], void *dx, const void *w, const void *dy, void *ws, size_t ws_bytes,
+                                float factor, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[1] == op->cfg.channels_in && x_shape[2] == op->cfg.shape[2] && x_shape[3] == op->cfg.shape[3],
+                "the operator was created for another input shape");
+    const int batch = x_shape[0];
+    DLP_REQUIRE(batch >= 0, "negative batch");
+    if (batch == 0)
+        return DLP_OK;
+    DLP_REQUIRE(dx != nullptr && w != nullptr && dy != nullptr, "null tensor pointer");
+    const size_t spread_bytes = bwd_data_spread_bytes(op, batch);
+    const size_t need = op->wt_bytes + spread_bytes + op->fwd_ws;
+    DLP_REQUIRE(ws != nullptr && ws_bytes >= need, "workspace smaller than workspace() for this batch");
+    hipStream_t st = (hipStream_t)stream;
+    const dlp_conv2d_settings &c = op->cfg;
+    float *wt = (float *)ws;
+    float *up = (float *)((char *)ws + op->wt_bytes);
+    void *fws = (char *)ws + op->wt_bytes + spread_bytes;
+    const int cout_g = c.channels_out / c.groups, cin_g = c.channels_in / c.groups, khw = c.kernel[0] * c.kernel[1];
+    {
+        TimingScope ts("bwd_data_filter_transpose", st);
+        hipLaunchKernelGGL(filter_transpose_flip_kernel, dim3(grid_for((size_t)c.channels_out * cin_g * khw)), dim3(256), 0, st, (const float *)w, wt,
+                           c.groups, cout_g, cin_g, khw);
+    }
+    const void *src = dy;
+    if (op->spread) {
+        const size_t planes = (size_t)batch * c.channels_out;
+        DLP_REQUIRE(planes * op->Hu * op->Wu < (1ull << 31) / 4, "tensor of 2 GiB or more");
+        TimingScope ts("bwd_data_spread", st);
+        hipLaunchKernelGGL(spread_with_zeros_kernel, dim3(grid_for(planes * op->Hu * op->Wu)), dim3(256), 0, st, (const float *)dy, up, planes, op->OH,
+                           op->OW, op->Hu, op->Wu, c.stride[0], c.stride[1]);
+        src = up;
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    const int in_shape[4] = {batch, c.channels_out, op->Hu, op->Wu};
+    return dlp_conv2d_fwd_enqueue(op->fwd, in_shape, src, wt, nullptr, dx, op->fwd_ws ? fws : nullptr, op->fwd_ws, factor, stream);
+}
+
+void dlp_conv2d_bwd_data_destroy(dlp_conv2d_bwd_data *op)
+{
+    if (!op)
+        return;
+    dlp_conv2d_fwd_destroy(op->fwd);
+    delete op;
+}
+
+int dlp_conv2d_bwd_filter_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_filter **out)
+{
+    DLP_REQUIRE(out != nullptr, "null argument");
+    *out = nullptr;
+    int oshape[4];
+    int rc = check_settings(cfg, oshape);
+    if (rc != DLP_OK)
+        return rc;
+    const std::string al = algo ? algo : "";
+    DLP_REQUIRE(al == "" || al == "auto" || al == "gemm" || al == "winograd" || al == "depthwise_separable", "unknown algorithm name");
+    DLP_REQUIRE(cfg->kernel[0] <= 31 && cfg->kernel[1] <= 31, "kernel extent above 31");
+    dlp_conv2d_bwd_filter *op = new (std::nothrow) dlp_conv2d_bwd_filter();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *cfg;
+    op->OH = oshape[2];
+    op->OW = oshape[3];
+    *out = op;
+    return DLP_OK;
+}
+
+const char *dlp_conv2d_bwd_filter_algo(const dlp_conv2d_bwd_filter *) { return "gemm"; }
+
+size_t dlp_conv2d_bwd_filter_workspace(const dlp_conv2d_bwd_filter *op)
+{
+    return op ? round256(wgrad_plan(op->cfg, std::max(op->cfg.shape[0], 1), op->OH, op->OW).part_bytes) : 0;
+}
+
+int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4], const void *x, void *dw, const void *dy, void *ws, size_t ws_bytes,
+                                  float factor, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    const dlp_conv2d_settings &c = op->cfg;
+    DLP_REQUIRE(x_shape[1] == c.channels_in && x_shape[2] == c.shape[2] && x_shape[3] == c.shape[3], "the operator was created for another input shape");
+    const int batch = x_shape[0];
+    DLP_REQUIRE(batch >= 0, "negative batch");
+    DLP_REQUIRE(dw != nullptr, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int cin_g = c.channels_in / c.groups, cout_g = c.channels_out / c.groups;
+    const int ncol = cin_g * c.kernel[0] * c.kernel[1];
+    const size_t n_out = (size_t)c.channels_out * ncol;
+    if (batch == 0) { // the gradient is zero: dw = factor * dw
+        TimingScope ts("wgrad_reduce", st);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)dw, (float *)dw, n_out, 0, factor);
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
+    DLP_REQUIRE(x != nullptr && dy != nullptr, "null tensor pointer");
+    const size_t x_elems = (size_t)batch * c.channels_in * c.shape[2] * c.shape[3];
+    const size_t y_elems = (size_t)batch * c.channels_out * op->OH * op->OW;
+    if (x_elems >= (1ull << 31) / 4 || y_elems >= (1ull << 31) / 4)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "tensor of 2 GiB or more");
+    WgradPlan p = wgrad_plan(c, batch, op->OH, op->OW);
+    if (p.slices > 1) {
+        // fewer slices when the caller's workspace was sized for a smaller batch
+        const size_t per_slice = n_out * sizeof(float);
+        const int fit = (int)std::min<size_t>(ws ? ws_bytes / per_slice : 0, (size_t)p.slices);
+        if (fit < p.slices) {
+            const int want = std::max(fit, 1);
+            p.cps = (p.chunks + want - 1) / want;
+            p.slices = (p.chunks + p.cps - 1) / p.cps;
+        }
+        DLP_REQUIRE(p.slices == 1 || (ws != nullptr && (size_t)p.slices * per_slice <= ws_bytes), "workspace smaller than workspace()");
+    }
+    WgradArgs a;
+    a.x = (const float *)x;
+    a.dy = (const float *)dy;
+    a.out = p.slices > 1 ? (float *)ws : (float *)dw;
+    a.Cin = c.channels_in;
+    a.Cin_g = cin_g;
+    a.Cout = c.channels_out;
+    a.Cout_g = cout_g;
+    a.groups = c.groups;
+    a.H = c.shape[2];
+    a.W = c.shape[3];
+    a.OW = op->OW;
+    a.OHW = op->OH * op->OW;
+    a.KH = c.kernel[0];
+    a.KW = c.kernel[1];
+    a.sh = c.stride[0];
+    a.sw = c.stride[1];
+    a.ph = c.pad[0];
+    a.pw = c.pad[1];
+    a.dh = c.dilate[0];
+    a.dw = c.dilate[1];
+    a.Ncol = ncol;
+    a.mtiles = p.mtiles;
+    a.ntiles = p.ntiles;
+    a.slices = p.slices;
+    a.chunks = p.chunks;
+    a.cpi = p.cpi;
+    a.cps = p.cps;
+    a.x_bytes = (uint32_t)(x_elems * 4);
+    a.dy_bytes = (uint32_t)(y_elems * 4);
+    make_magic((uint32_t)a.OW, a.ow_magic, a.ow_shift);
+    make_magic((uint32_t)(a.KH * a.KW), a.khw_magic, a.khw_shift);
+    make_magic((uint32_t)a.KW, a.kw_magic, a.kw_shift);
+    make_magic((uint32_t)a.cpi, a.cpi_magic, a.cpi_shift);
+    a.factor = factor;
+    const long long wgs = (long long)p.mtiles * p.ntiles * c.groups * p.slices;
+    DLP_REQUIRE(wgs < (1ll << 31), "too many workgroups");
+    {
+        TimingScope ts("wgrad", st);
+        const dim3 grid((unsigned)wgs), block(256);
+        if (p.BM == 128 && p.BN == 128)
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<128, 128>), grid, block, 0, st, a);
+        else if (p.BM == 128)
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<128, 64>), grid, block, 0, st, a);
+        else if (p.BN == 128)
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<64, 128>), grid, block, 0, st, a);
+        else
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<64, 64>), grid, block, 0, st, a);
+    }
+    if (p.slices > 1) {
+        TimingScope ts("wgrad_reduce", st);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
+    }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+void dlp_conv2d_bwd_filter_destroy(dlp_conv2d_bwd_filter *op) { delete op; }
+
+int dlp_bias_bwd_enqueue(int dtype, int batch, int features, int plane, const void *dy, float *db, float beta, void *stream)
+{
+    if (dtype != DLP_FLOAT)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "bias gradient: float_data is implemented");
+    DLP_REQUIRE(batch >= 0 && features > 0 && plane > 0, "shape");
+    DLP_REQUIRE(db != nullptr && (batch == 0 || dy != nullptr), "null tensor pointer");
+    TimingScope ts("bias_backward", (hipStream_t)stream);
+    hipLaunchKernelGGL(bias_backward_kernel, dim3((unsigned)features), dim3(256), 0, (hipStream_t)stream, (const float *)dy, db, batch, features, plane, beta);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+} // extern "C"

@@ -1,5 +1,5 @@
-// dlprim::core::Conv2DForward on the MI355X: same interface as dlprimitives'
-// include/dlprim/core/conv.hpp:17-58, implemented over the C ABI in dlprim_hip.h.
+// dlprim::core::Conv2DForward / Conv2DBackwardData / Conv2DBackwardFilter on the MI355X: same interface
+// as dlprimitives' include/dlprim/core/conv.hpp:17-80, implemented over the C ABI in dlprim_hip.h.
 #pragma once
 #include <memory>
 #include <string>
@@ -97,6 +97,97 @@ private:
     dlp_conv2d_fwd *op_ = nullptr;
 };
 } // namespace details
+
+// dx = factor * dx + gradient with respect to x (include/dlprim/core/conv.hpp:60-68 in the reference)
+class Conv2DBackwardData : public Conv2DBase {
+public:
+    virtual ~Conv2DBackwardData() {}
+    virtual void enqueue(Tensor &dx, Tensor &w, Tensor &dy, Tensor &ws, float factor, ExecutionContext const &e) = 0;
+    static std::unique_ptr<Conv2DBackwardData> create(Context &ctx, Conv2DSettings const &config, std::string const &algo = std::string());
+};
+
+// dw = factor * dw + gradient with respect to the filter (include/dlprim/core/conv.hpp:70-78 in the reference)
+class Conv2DBackwardFilter : public Conv2DBase {
+public:
+    virtual ~Conv2DBackwardFilter() {}
+    virtual void enqueue(Tensor &x, Tensor &dw, Tensor &dy, Tensor &ws, float factor, ExecutionContext const &e) = 0;
+    static std::unique_ptr<Conv2DBackwardFilter> create(Context &ctx, Conv2DSettings const &config, std::string const &algo = std::string());
+};
+
+namespace details {
+inline void shape4(Shape const &s, int (&out)[4])
+{
+    DLPRIM_CHECK(s.size() == 4);
+    for (int i = 0; i < 4; i++)
+        out[i] = int(s[i]);
+}
+
+class Conv2DBackwardDataHip : public Conv2DBackwardData {
+public:
+    Conv2DBackwardDataHip(Context &ctx, Conv2DSettings const &config, std::string const &algo)
+    {
+        if (!ctx.is_hip_context())
+            throw ValidationError("core::Conv2DBackwardData needs a device context");
+        ctx.select();
+        dlp_conv2d_settings s = to_c(config, config.shape, config.dtype);
+        dlprim::details::check_status(dlp_conv2d_bwd_data_create(&s, algo.c_str(), &op_));
+    }
+    ~Conv2DBackwardDataHip() { dlp_conv2d_bwd_data_destroy(op_); }
+    Conv2DBackwardDataHip(Conv2DBackwardDataHip const &) = delete;
+    void operator=(Conv2DBackwardDataHip const &) = delete;
+    char const *algo() const override { return dlp_conv2d_bwd_data_algo(op_); }
+    size_t workspace() override { return dlp_conv2d_bwd_data_workspace(op_); }
+    void enqueue(Tensor &dx, Tensor &w, Tensor &dy, Tensor &ws, float factor, ExecutionContext const &e) override
+    {
+        int xs[4];
+        shape4(dx.shape(), xs);
+        const size_t ws_bytes = workspace() ? ws.memory_size() : 0;
+        dlprim::details::check_status(dlp_conv2d_bwd_data_enqueue(op_, xs, dx.device_ptr(), w.device_ptr(), dy.device_ptr(),
+                                                                  ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, factor, e.stream()));
+    }
+
+private:
+    dlp_conv2d_bwd_data *op_ = nullptr;
+};
+
+class Conv2DBackwardFilterHip : public Conv2DBackwardFilter {
+public:
+    Conv2DBackwardFilterHip(Context &ctx, Conv2DSettings const &config, std::string const &algo)
+    {
+        if (!ctx.is_hip_context())
+            throw ValidationError("core::Conv2DBackwardFilter needs a device context");
+        ctx.select();
+        dlp_conv2d_settings s = to_c(config, config.shape, config.dtype);
+        dlprim::details::check_status(dlp_conv2d_bwd_filter_create(&s, algo.c_str(), &op_));
+    }
+    ~Conv2DBackwardFilterHip() { dlp_conv2d_bwd_filter_destroy(op_); }
+    Conv2DBackwardFilterHip(Conv2DBackwardFilterHip const &) = delete;
+    void operator=(Conv2DBackwardFilterHip const &) = delete;
+    char const *algo() const override { return dlp_conv2d_bwd_filter_algo(op_); }
+    size_t workspace() override { return dlp_conv2d_bwd_filter_workspace(op_); }
+    void enqueue(Tensor &x, Tensor &dw, Tensor &dy, Tensor &ws, float factor, ExecutionContext const &e) override
+    {
+        int xs[4];
+        shape4(x.shape(), xs);
+        const size_t ws_bytes = workspace() ? ws.memory_size() : 0;
+        dlprim::details::check_status(dlp_conv2d_bwd_filter_enqueue(op_, xs, x.device_ptr(), dw.device_ptr(), dy.device_ptr(),
+                                                                    ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, factor, e.stream()));
+    }
+
+private:
+    dlp_conv2d_bwd_filter *op_ = nullptr;
+};
+} // namespace details
+
+inline std::unique_ptr<Conv2DBackwardData> Conv2DBackwardData::create(Context &ctx, Conv2DSettings const &config, std::string const &algo)
+{
+    return std::unique_ptr<Conv2DBackwardData>(new details::Conv2DBackwardDataHip(ctx, config, algo));
+}
+
+inline std::unique_ptr<Conv2DBackwardFilter> Conv2DBackwardFilter::create(Context &ctx, Conv2DSettings const &config, std::string const &algo)
+{
+    return std::unique_ptr<Conv2DBackwardFilter>(new details::Conv2DBackwardFilterHip(ctx, config, algo));
+}
 
 inline std::unique_ptr<Conv2DForward> Conv2DForward::create(Context &ctx, Conv2DSettings const &config, bool bias,
                                                             StandardActivations activation, std::string const &algo)

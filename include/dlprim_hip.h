@@ -122,6 +122,38 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4],
 
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
+/* ---- core::Conv2DBackwardData, include/dlprim/core/conv.hpp:60-68, src/core/conv.cpp:113-163,299-367,
+ *      512-590 (CPU contract: src/ops/conv2d.cpp:426-430,485-498):
+ *      dx [B,Cin,H,W] = factor * dx + gradient of the convolution with respect to x, from
+ *      w [Cout,Cin/groups,KH,KW] and dy [B,Cout,OH,OW].  `cfg` is the forward convolution's settings
+ *      (shape = shape of x); algo as for the forward operator.  float_data only.
+ *      ws >= workspace() bytes (sized for the batch in cfg->shape; a larger batch needs more when
+ *      stride > 1).  Asynchronous on `stream`. ---------------------------------------------------- */
+typedef struct dlp_conv2d_bwd_data dlp_conv2d_bwd_data;
+int dlp_conv2d_bwd_data_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_data **out);
+const char *dlp_conv2d_bwd_data_algo(const dlp_conv2d_bwd_data *op);
+size_t dlp_conv2d_bwd_data_workspace(const dlp_conv2d_bwd_data *op);
+int dlp_conv2d_bwd_data_enqueue(dlp_conv2d_bwd_data *op, const int x_shape[4], void *dx, const void *w,
+                                const void *dy, void *ws, size_t ws_bytes, float factor, void *stream);
+void dlp_conv2d_bwd_data_destroy(dlp_conv2d_bwd_data *op);
+
+/* ---- core::Conv2DBackwardFilter, include/dlprim/core/conv.hpp:70-78, src/core/conv.cpp:165-220,
+ *      369-434,592-669 (CPU contract: src/ops/conv2d.cpp:431-435,475-484):
+ *      dw [Cout,Cin/groups,KH,KW] = factor * dw + gradient with respect to the filter, from
+ *      x [B,Cin,H,W] and dy [B,Cout,OH,OW].  float_data only; ws >= workspace() bytes. ------------- */
+typedef struct dlp_conv2d_bwd_filter dlp_conv2d_bwd_filter;
+int dlp_conv2d_bwd_filter_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_filter **out);
+const char *dlp_conv2d_bwd_filter_algo(const dlp_conv2d_bwd_filter *op);
+size_t dlp_conv2d_bwd_filter_workspace(const dlp_conv2d_bwd_filter *op);
+int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4], const void *x, void *dw,
+                                  const void *dy, void *ws, size_t ws_bytes, float factor, void *stream);
+void dlp_conv2d_bwd_filter_destroy(dlp_conv2d_bwd_filter *op);
+
+/* ---- core::BiasBackwardFilter::enqueue, include/dlprim/core/bias.hpp:16-35, src/core/bias.cpp (CPU contract:
+ *      BWBias::backward_cpu, src/ops/bwd_bias.cpp:34-60): db[f] = beta * db[f] + sum over b, plane of
+ *      dy[b][f][plane] ---------------------------------------------------------------------------- */
+int dlp_bias_bwd_enqueue(int dtype, int batch, int features, int plane, const void *dy, float *db, float beta, void *stream);
+
 /* ---- core::IPForward::create / enqueue, include/dlprim/core/ip.hpp:30-45,
  *      src/core/ip.cpp:15-50: y[B,Out] = act(x[B,In] * w[Out,In]^T + bias[Out]) */
 int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_ip_fwd **out);

@@ -128,6 +128,50 @@ def conv2d_forward(x, w, bias, cfg, activation="identity", threads=1):
     return y
 
 
+def conv2d_backward_data(dy, w, cfg, in_shape, dx_old=None, factor=0.0):
+    """Convolution2D::backward_data_cpu restated: returns factor * dx_old + gradient with respect to x."""
+    dy, w = _f32(dy), _f32(w)
+    ish = (ctypes.c_int * 4)(*in_shape)
+    dx = _f32(dx_old).copy() if dx_old is not None else np.zeros(tuple(in_shape), dtype=np.float32)
+    ws = np.empty(max(1, lib().orc_conv2d_workspace(ctypes.byref(cfg), ish) // 4), dtype=np.float32)
+    if lib().orc_conv2d_backward_data(ctypes.byref(cfg), ish, _ptr(dy), _ptr(w), _ptr(dx), _ptr(ws), ctypes.c_float(factor)) < 0:
+        raise ValueError("invalid convolution configuration")
+    return dx
+
+
+def conv2d_backward_filter(dy, x, cfg, dw_old=None, factor=0.0):
+    """Convolution2D::backward_filter_cpu restated: returns factor * dw_old + gradient with respect to w."""
+    dy, x = _f32(dy), _f32(x)
+    ish = (ctypes.c_int * 4)(*x.shape)
+    shape = (cfg.channels_out, cfg.channels_in // cfg.groups, cfg.kernel[0], cfg.kernel[1])
+    dw = _f32(dw_old).copy() if dw_old is not None else np.zeros(shape, dtype=np.float32)
+    ws = np.empty(max(1, lib().orc_conv2d_workspace(ctypes.byref(cfg), ish) // 4), dtype=np.float32)
+    if lib().orc_conv2d_backward_filter(ctypes.byref(cfg), ish, _ptr(dy), _ptr(x), _ptr(dw), _ptr(ws), ctypes.c_float(factor)) < 0:
+        raise ValueError("invalid convolution configuration")
+    return dw
+
+
+def bias_backward(dy, db_old=None, beta=0.0):
+    """BWBias::backward_cpu restated: db[f] = beta * db_old[f] + sum of dy over batch and plane."""
+    dy = _f32(dy)
+    features = dy.shape[1]
+    db = _f32(db_old).copy() if db_old is not None else np.zeros(features, dtype=np.float32)
+    lib().orc_bias_backward(int(dy.shape[0]), int(features), int(dy.size // max(dy.shape[0] * features, 1)), _ptr(dy), _ptr(db), ctypes.c_float(beta))
+    return db
+
+
+def sgemm(A, B, trans_a=False, trans_b=False, C=None, alpha=1.0, beta=0.0):
+    """The restated my_cblas products (nt, nn, tn), row-major, with the reference's loop orders."""
+    A, B = _f32(A), _f32(B)
+    M = A.shape[1] if trans_a else A.shape[0]
+    K = A.shape[0] if trans_a else A.shape[1]
+    N = B.shape[0] if trans_b else B.shape[1]
+    out = _f32(C).copy() if C is not None else np.zeros((M, N), dtype=np.float32)
+    fn = {(False, True): lib().orc_sgemm_nt, (False, False): lib().orc_sgemm_nn, (True, False): lib().orc_sgemm_tn}[(bool(trans_a), bool(trans_b))]
+    fn(M, N, K, ctypes.c_float(alpha), _ptr(A), int(A.shape[1]), _ptr(B), int(B.shape[1]), ctypes.c_float(beta), _ptr(out), N)
+    return out
+
+
 def conv2d_direct_f64(x, w, bias, cfg, activation="identity"):
     x, w = _f32(x), _f32(w)
     bias = _f32(bias) if bias is not None else None

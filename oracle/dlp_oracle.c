@@ -245,6 +245,141 @@ int orc_conv2d_forward_mt(const orc_conv2d_cfg *cfg, const int in_shape[4],
     return used;
 }
 
+/* src/my_blas/my_cblas.cpp:28-39 (beta), :41-51 (nn product: r, k, c loops) */
+void orc_sgemm_nn(int M, int N, int K, float alpha, const float *A, int lda,
+                  const float *B, int ldb, float beta, float *C, int ldc)
+{
+    for (int r = 0; r < M; r++) {
+        if (beta == 0.0f)
+            memset(C + (size_t)ldc * r, 0, sizeof(float) * (size_t)N);
+        else
+            for (int c = 0; c < N; c++)
+                C[(size_t)r * ldc + c] *= beta;
+    }
+    for (int r = 0; r < M; r++)
+        for (int k = 0; k < K; k++) {
+            float av = A[(size_t)r * lda + k] * alpha;
+            for (int c = 0; c < N; c++)
+                C[(size_t)r * ldc + c] += av * B[(size_t)k * ldb + c];
+        }
+}
+
+/* src/my_blas/my_cblas.cpp:28-39 (beta), :52-62 (tn product: k, r, c loops; A is K x M) */
+void orc_sgemm_tn(int M, int N, int K, float alpha, const float *A, int lda,
+                  const float *B, int ldb, float beta, float *C, int ldc)
+{
+    for (int r = 0; r < M; r++) {
+        if (beta == 0.0f)
+            memset(C + (size_t)ldc * r, 0, sizeof(float) * (size_t)N);
+        else
+            for (int c = 0; c < N; c++)
+                C[(size_t)r * ldc + c] *= beta;
+    }
+    for (int k = 0; k < K; k++)
+        for (int r = 0; r < M; r++) {
+            float av = A[r + (size_t)lda * k] * alpha;
+            for (int c = 0; c < N; c++)
+                C[(size_t)r * ldc + c] += av * B[(size_t)k * ldb + c];
+        }
+}
+
+/* Convolution2DBase::im2col<Col2ImOp>, src/ops/conv2d.cpp:262-278 (img += column entry, padding skipped)
+ * over the generic walk :376-409: the adjoint of orc_im2col */
+void orc_col2im(const orc_conv2d_cfg *cfg, int cin_g, int H, int W, int OH, int OW,
+                float *img, const float *mat)
+{
+    const int kh = cfg->kernel[0], kw = cfg->kernel[1];
+    const int width = cin_g * kh * kw;
+    for (int chan = 0; chan < cin_g; chan++) {
+        for (int r = 0; r < OH; r++) {
+            for (int c = 0; c < OW; c++) {
+                const float *m = mat + (size_t)(r * OW + c) * width + chan * kh * kw;
+                int y0 = r * cfg->stride[0] - cfg->pad[0];
+                int x0 = c * cfg->stride[1] - cfg->pad[1];
+                for (int ky = 0; ky < kh; ky++) {
+                    int y = y0 + ky * cfg->dilate[0];
+                    for (int kx = 0; kx < kw; kx++) {
+                        int x = x0 + kx * cfg->dilate[1];
+                        float v = *m++;
+                        if (y >= 0 && y < H && x >= 0 && x < W)
+                            img[((size_t)chan * H + y) * W + x] += v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* Convolution2DBase::scale_cpu, src/ops/conv2d.cpp:411-419 */
+static void scale_by(float *p, size_t n, float v)
+{
+    if (v == 0.0f)
+        memset(p, 0, n * sizeof(float));
+    else
+        for (size_t i = 0; i < n; i++)
+            p[i] *= v;
+}
+
+/* src/ops/conv2d.cpp:426-430 and the backward_data branch :485-498 */
+int orc_conv2d_backward_data(const orc_conv2d_cfg *cfg, const int in_shape[4],
+                             const float *dy, const float *w, float *dx, void *ws, float factor)
+{
+    int out[4];
+    if (conv_cfg_ok(cfg, in_shape, out) != 0)
+        return -1;
+    const int H = in_shape[2], W = in_shape[3], OH = out[2], OW = out[3];
+    const int cin_g = cfg->channels_in / cfg->groups, cout_g = cfg->channels_out / cfg->groups;
+    const int K = cin_g * cfg->kernel[0] * cfg->kernel[1];
+    const int plane = OH * OW;
+    const size_t in_img = (size_t)in_shape[1] * H * W, out_img = (size_t)out[1] * plane;
+    float *col = (float *)ws;
+    scale_by(dx, in_img * (size_t)in_shape[0], factor);
+    for (int b = 0; b < in_shape[0]; b++)
+        for (int g = 0; g < cfg->groups; g++) {
+            float *img = dx + b * in_img + (size_t)g * cin_g * H * W;
+            const float *omg = dy + b * out_img + (size_t)g * cout_g * plane;
+            /* col[plane x K] = omg^T[plane x cout_g] * kernel[cout_g x K] */
+            orc_sgemm_tn(plane, K, cout_g, 1.0f, omg, plane, w + (size_t)g * cout_g * K, K, 0.0f, col, K);
+            orc_col2im(cfg, cin_g, H, W, OH, OW, img, col);
+        }
+    return 0;
+}
+
+/* src/ops/conv2d.cpp:431-435 and the backward_filter branch :475-484 */
+int orc_conv2d_backward_filter(const orc_conv2d_cfg *cfg, const int in_shape[4],
+                               const float *dy, const float *x, float *dw, void *ws, float factor)
+{
+    int out[4];
+    if (conv_cfg_ok(cfg, in_shape, out) != 0)
+        return -1;
+    const int H = in_shape[2], W = in_shape[3], OH = out[2], OW = out[3];
+    const int cin_g = cfg->channels_in / cfg->groups, cout_g = cfg->channels_out / cfg->groups;
+    const int K = cin_g * cfg->kernel[0] * cfg->kernel[1];
+    const int plane = OH * OW;
+    const size_t in_img = (size_t)in_shape[1] * H * W, out_img = (size_t)out[1] * plane;
+    float *col = (float *)ws;
+    scale_by(dw, (size_t)cfg->channels_out * K, factor);
+    for (int b = 0; b < in_shape[0]; b++)
+        for (int g = 0; g < cfg->groups; g++) {
+            const float *img = x + b * in_img + (size_t)g * cin_g * H * W;
+            const float *omg = dy + b * out_img + (size_t)g * cout_g * plane;
+            orc_im2col(cfg, cin_g, H, W, OH, OW, img, col);
+            /* dK[cout_g x K] += omg[cout_g x plane] * col[plane x K] */
+            orc_sgemm_nn(cout_g, K, plane, 1.0f, omg, plane, col, K, 1.0f, dw + (size_t)g * cout_g * K, K);
+        }
+    return 0;
+}
+
+/* BWBias::backward_cpu, src/ops/bwd_bias.cpp:34-60 */
+void orc_bias_backward(int batch, int features, int plane, const float *dy, float *db, float beta)
+{
+    scale_by(db, (size_t)features, beta);
+    for (int b = 0; b < batch; b++)
+        for (int f = 0; f < features; f++)
+            for (int p = 0; p < plane; p++)
+                db[f] += *dy++;
+}
+
 /* src/kernels/sgemm.cl:707-710 (also winograd_fwd.cl:216-222,
  * depthwise_separable_conv.cl:96-101) */
 void orc_apply_factor(float *y, const float *y_old, size_t n, float factor)

@@ -71,6 +71,27 @@ int orc_conv2d_forward_mt(const orc_conv2d_cfg *cfg, const int in_shape[4],
                           const float *x, const float *w, const float *bias,
                           float *y, int activation, int threads);
 
+/* my_cblas::cblas_sgemm NoTrans x NoTrans and Trans x NoTrans, src/my_blas/my_cblas.cpp:41-62,88-103 */
+void orc_sgemm_nn(int M, int N, int K, float alpha, const float *A, int lda,
+                  const float *B, int ldb, float beta, float *C, int ldc);
+void orc_sgemm_tn(int M, int N, int K, float alpha, const float *A, int lda,
+                  const float *B, int ldb, float beta, float *C, int ldc);
+
+/* Convolution2DBase::im2col<Col2ImOp>, src/ops/conv2d.cpp:262-278,376-409: img += the column matrix */
+void orc_col2im(const orc_conv2d_cfg *cfg, int cin_g, int H, int W, int OH, int OW,
+                float *img, const float *mat);
+
+/* Convolution2D::backward_data_cpu / backward_filter_cpu, src/ops/conv2d.cpp:411-419,426-435,475-498.
+ * dx = factor * dx + (gradient with respect to x); dw = factor * dw + (gradient with respect to w).
+ * ws: scratch of at least orc_conv2d_workspace() bytes.  Returns 0, or -1 on invalid configuration. */
+int orc_conv2d_backward_data(const orc_conv2d_cfg *cfg, const int in_shape[4],
+                             const float *dy, const float *w, float *dx, void *ws, float factor);
+int orc_conv2d_backward_filter(const orc_conv2d_cfg *cfg, const int in_shape[4],
+                               const float *dy, const float *x, float *dw, void *ws, float factor);
+
+/* BWBias::backward_cpu, src/ops/bwd_bias.cpp:34-60: db[f] = beta * db[f] + sum over batch and plane of dy */
+void orc_bias_backward(int batch, int features, int plane, const float *dy, float *db, float beta);
+
 /* The device-side `factor` contract, src/kernels/sgemm.cl:707-710:
  * y = factor != 0 ? y_old*factor + v : v, applied to an already activated v. */
 void orc_apply_factor(float *y, const float *y_old, size_t n, float factor);

@@ -5,10 +5,12 @@
 //
 //   test_core_api host   : everything that needs no GPU (shapes, exceptions)
 //   test_core_api <dev>  : the device checks on HIP device <dev> (default 0)
+#include <dlprim/core/bias.hpp>
 #include <dlprim/core/conv.hpp>
 #include <dlprim/core/ip.hpp>
 #include <dlprim/core/pool.hpp>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -135,6 +137,85 @@ static void conv_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int cin,
     EXPECT(worst < 1e-4);
 }
 
+// Gradients the way Convolution2D::backward calls them (src/ops/conv2d.cpp:504-555): bias, filter, data,
+// each accumulating with its own factor; checked against the definition of the gradients in double.
+static void conv_backward_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int cin, int cout, int hw, int k, int stride, int pad, int groups,
+                               float factor)
+{
+    dp::Convolution2DConfigBase c;
+    c.channels_in = cin;
+    c.channels_out = cout;
+    c.kernel[0] = c.kernel[1] = k;
+    c.stride[0] = c.stride[1] = stride;
+    c.pad[0] = c.pad[1] = pad;
+    c.groups = groups;
+    dp::Shape in(B, cin, hw, hw);
+    dp::core::Conv2DSettings cfg(c, in, dp::float_data);
+    dp::Shape os = dp::core::Conv2DBase::get_output_shape(c, in);
+    std::unique_ptr<dp::core::Conv2DBackwardData> bd = dp::core::Conv2DBackwardData::create(ctx, cfg);
+    std::unique_ptr<dp::core::Conv2DBackwardFilter> bf = dp::core::Conv2DBackwardFilter::create(ctx, cfg);
+    std::unique_ptr<dp::core::BiasBackwardFilter> bb = dp::core::BiasBackwardFilter::create(ctx, os);
+    const int cg = cin / groups, og = cout / groups, OH = int(os[2]), OW = int(os[3]);
+    dp::Tensor X(ctx, in), W(ctx, dp::Shape(cout, cg, k, k)), dY(ctx, os), dX(ctx, in), dW(ctx, dp::Shape(cout, cg, k, k)), dB(ctx, dp::Shape(cout));
+    size_t ws_size = std::max(std::max(bd->workspace(), bf->workspace()), bb->workspace());
+    dp::Tensor ws(ctx, dp::Shape(ws_size ? ws_size : 1), dp::uint8_data);
+    std::mt19937 rng(cin * 77 + cout + hw);
+    fill(X, rng, -1, 1);
+    fill(W, rng, -0.3f, 0.3f);
+    fill(dY, rng, -1, 1);
+    fill(dX, rng, -1, 1);
+    fill(dW, rng, -1, 1);
+    fill(dB, rng, -1, 1);
+    std::vector<double> want_dx(in.total_size()), want_dw(W.shape().total_size()), want_db(cout);
+    for (size_t i = 0; i < want_dx.size(); i++)
+        want_dx[i] = double(factor) * dX.data<float>()[i];
+    for (size_t i = 0; i < want_dw.size(); i++)
+        want_dw[i] = double(factor) * dW.data<float>()[i];
+    for (int i = 0; i < cout; i++)
+        want_db[i] = double(factor) * dB.data<float>()[i];
+    const float *x = X.data<float>(), *w = W.data<float>(), *dy = dY.data<float>();
+    for (int b = 0; b < B; b++)
+        for (int o = 0; o < cout; o++)
+            for (int oy = 0; oy < OH; oy++)
+                for (int ox = 0; ox < OW; ox++) {
+                    const double g = dy[((size_t(b) * cout + o) * OH + oy) * OW + ox];
+                    want_db[o] += g;
+                    const int grp = o / og;
+                    for (int ci = 0; ci < cg; ci++)
+                        for (int ky = 0; ky < k; ky++)
+                            for (int kx = 0; kx < k; kx++) {
+                                int iy = oy * stride - pad + ky, ix = ox * stride - pad + kx;
+                                if (iy < 0 || iy >= hw || ix < 0 || ix >= hw)
+                                    continue;
+                                const size_t xi = ((size_t(b) * cin + grp * cg + ci) * hw + iy) * hw + ix;
+                                const size_t wi = ((size_t(o) * cg + ci) * k + ky) * k + kx;
+                                want_dx[xi] += g * w[wi];
+                                want_dw[wi] += g * x[xi];
+                            }
+                }
+    for (dp::Tensor *t : {&X, &W, &dY, &dX, &dW, &dB})
+        t->to_device(q);
+    bb->enqueue(dY, dB, ws, factor, q);
+    bf->enqueue(X, dW, dY, ws, factor, q);
+    bd->enqueue(dX, W, dY, ws, factor, q);
+    dX.to_host(q);
+    dW.to_host(q);
+    dB.to_host(q);
+    q.finish();
+    auto worst = [](std::vector<double> const &want, const float *got) {
+        double scale = 1e-6, err = 0;
+        for (double v : want)
+            scale = std::max(scale, std::fabs(v));
+        for (size_t i = 0; i < want.size(); i++)
+            err = std::max(err, std::fabs(want[i] - got[i]) / scale);
+        return err;
+    };
+    const double ex = worst(want_dx, dX.data<float>()), ew = worst(want_dw, dW.data<float>()), eb = worst(want_db, dB.data<float>());
+    std::printf("conv backward (%s / %s) b%d %d->%d @%d k%d s%d g%d factor %.2f : max err dx %.2e dw %.2e db %.2e\n", bd->algo(), bf->algo(), B, cin, cout,
+                hw, k, stride, groups, factor, ex, ew, eb);
+    EXPECT(ex < 1e-4 && ew < 1e-4 && eb < 1e-4);
+}
+
 static void ip_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int in, int out)
 {
     dp::core::IPSettings cfg;
@@ -234,6 +315,10 @@ int main(int argc, char **argv)
             conv_case(ctx, q, 2, 3, 8, 20, 7, 2, 3, 1, false, A::identity, "", "gemm", 0.5f);
             conv_case(ctx, q, 3, 24, 24, 9, 3, 2, 1, 24, true, A::relu6, "", "depthwise_separable", 0.0f);
             conv_case(ctx, q, 1, 8, 6, 5, 1, 1, 0, 2, true, A::sigmoid, "winograd", "gemm", 0.0f); // incompatible request -> gemm
+            conv_backward_case(ctx, q, 2, 16, 32, 14, 3, 1, 1, 1, 0.0f);
+            conv_backward_case(ctx, q, 3, 6, 8, 13, 3, 2, 1, 2, 0.5f);
+            conv_backward_case(ctx, q, 2, 24, 24, 9, 3, 1, 1, 24, 1.0f);
+            conv_backward_case(ctx, q, 2, 3, 8, 20, 7, 2, 3, 1, 0.0f);
             ip_case(ctx, q, 5, 64, 10);
             pool_case(ctx, q);
             // sub-tensor views share memory: run on the second image of a batch-2 tensor

@@ -229,3 +229,76 @@ def test_bf16_round_matches_torch(oracle_mod):
     x = np.random.default_rng(9).standard_normal(10000).astype(np.float32) * 100
     want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
     assert np.array_equal(oracle_mod.bf16_round(x), want)
+
+
+# ---------------------------------------------------------------- backward (the gradient operators)
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("mnk", [(1, 1, 1), (3, 5, 7), (24, 50, 36), (17, 129, 33)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_sgemm_nn_tn_bit_exact_vs_compiled_reference(oracle_mod, mnk, beta, ta):
+    if oracle_mod.ref() is None:
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    M, N, K = mnk
+    rng = np.random.default_rng(M * 1000 + N * 10 + K)
+    A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    got = oracle_mod.sgemm(A, B, ta, False, C0, alpha=1.0, beta=beta)
+    want = oracle_mod.ref_sgemm(A, B, ta, False, C0, alpha=1.0, beta=beta)
+    assert np.array_equal(got, want)
+    np.testing.assert_allclose(got, (A.T if ta else A).astype(np.float64) @ B + beta * C0, rtol=1e-4, atol=1e-4)
+
+
+def torch_conv_grads(x, w, dy, c):
+    xt = torch.from_numpy(x).double().requires_grad_(True)
+    wt = torch.from_numpy(w).double().requires_grad_(True)
+    y = torch.nn.functional.conv2d(xt, wt, None, stride=c["stride"], padding=c["pad"], dilation=c["dilate"], groups=c["groups"])
+    y.backward(torch.from_numpy(dy).double())
+    return xt.grad.numpy(), wt.grad.numpy()
+
+
+@pytest.mark.parametrize("c,bhw", small_cases(), ids=case_id)
+def test_conv_backward_vs_torch_autograd(oracle_mod, c, bhw):
+    """Both gradient restatements against torch's autograd of the library convolution, and the
+    accumulate contract (result = factor * old + gradient) against the same."""
+    x, w, _ = make_tensors(c, bhw, seed=4321)
+    cfg = cfg_of(oracle_mod, c)
+    rng = np.random.default_rng(99)
+    dy = rng.standard_normal(oracle_mod.conv2d_output_shape(cfg, x.shape)).astype(np.float32)
+    want_dx, want_dw = torch_conv_grads(x, w, dy, c)
+    dx = oracle_mod.conv2d_backward_data(dy, w, cfg, x.shape)
+    dw = oracle_mod.conv2d_backward_filter(dy, x, cfg)
+    np.testing.assert_allclose(dx, want_dx, rtol=1e-4, atol=1e-4 * max(1.0, np.abs(want_dx).max()))
+    np.testing.assert_allclose(dw, want_dw, rtol=1e-4, atol=1e-4 * max(1.0, np.abs(want_dw).max()))
+    old_dx = rng.standard_normal(x.shape).astype(np.float32)
+    old_dw = rng.standard_normal(w.shape).astype(np.float32)
+    dx2 = oracle_mod.conv2d_backward_data(dy, w, cfg, x.shape, old_dx, 0.5)
+    dw2 = oracle_mod.conv2d_backward_filter(dy, x, cfg, old_dw, -2.0)
+    np.testing.assert_allclose(dx2, want_dx + 0.5 * old_dx, rtol=1e-4, atol=1e-4 * max(1.0, np.abs(want_dx).max()))
+    np.testing.assert_allclose(dw2, want_dw - 2.0 * old_dw, rtol=1e-4, atol=1e-4 * max(1.0, np.abs(want_dw).max()))
+
+
+def test_conv_backward_is_the_adjoint_of_forward(oracle_mod):
+    """<dy, conv(x, w)> = <backward_data(dy, w), x> = <backward_filter(dy, x), w>: the forward oracle is
+    pinned by the reference's goldens; the identities tie both gradients to it without any formula."""
+    rng = np.random.default_rng(5)
+    for (cin, cout, k, s, d, p, g, hw) in [(4, 6, 3, 2, 1, 1, 2, (9, 8)), (3, 5, (2, 3), (1, 2), (2, 1), (1, 2), 1, (7, 10)), (8, 8, 3, 1, 1, 1, 8, (6, 6))]:
+        cfg = oracle_mod.make_cfg(cin, cout, k, s, d, p, g)
+        kh, kw = (k, k) if isinstance(k, int) else k
+        x = np.round(rng.standard_normal((2, cin) + hw) * 4).astype(np.float32)
+        w = np.round(rng.standard_normal((cout, cin // g, kh, kw)) * 4).astype(np.float32)
+        y = oracle_mod.conv2d_forward(x, w, None, cfg)
+        dy = np.round(rng.standard_normal(y.shape) * 4).astype(np.float32)
+        lhs = float((dy.astype(np.float64) * y).sum())
+        # integer-valued tensors: every sum is exact in fp32, so the identities hold exactly
+        assert float((oracle_mod.conv2d_backward_data(dy, w, cfg, x.shape).astype(np.float64) * x).sum()) == lhs
+        assert float((oracle_mod.conv2d_backward_filter(dy, x, cfg).astype(np.float64) * w).sum()) == lhs
+
+
+def test_bias_backward_closed_form(oracle_mod):
+    rng = np.random.default_rng(6)
+    dy = np.round(rng.standard_normal((3, 5, 4, 7)) * 8).astype(np.float32)
+    old = np.round(rng.standard_normal(5) * 8).astype(np.float32)
+    assert np.array_equal(oracle_mod.bias_backward(dy), dy.sum((0, 2, 3)))
+    assert np.array_equal(oracle_mod.bias_backward(dy, old, 2.0), dy.sum((0, 2, 3)) + 2 * old)
+    assert np.array_equal(oracle_mod.bias_backward(dy[:, :, 0, 0]), dy[:, :, 0, 0].sum(0))
