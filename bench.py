@@ -13,6 +13,8 @@ Other workloads (same JSON contract, for the remaining configurations):
   --workload winograd       the two Winograd shapes, algo winograd
   --workload winograd-gemm  the same two shapes through the implicit GEMM
   --workload resnet18-full / resnet50-full   whole network forward incl. pooling, adds, GAP, IP
+  --workload resnet18-backward   gradients of the 20 ResNet-18 convolutions (backward filter for all,
+                            backward data for all but conv1, whose input needs none), fp32
 
 Prints ONE JSON line.  `value` = images/s of the whole workload; `gflops_per_s` is
 the same run expressed with the reference's flop accounting (tools/flops.cpp:660).
@@ -215,13 +217,77 @@ def run_graph_workload(args):
     print(json.dumps(out))
 
 
+def run_backward_workload(args):
+    """Backward data + backward filter of every layer of the ResNet-18 convolution stack; same JSON
+    contract; roofline for the backward-filter kernel (its flops = the forward convolution's)."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.workloads import RESNET18_CONVS, conv_flops
+
+    torch.manual_seed(2024)
+    layers = []
+    for L in RESNET18_CONVS:
+        st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], (args.batch, L["cin"], L["hw"], L["hw"]))
+        osh = dlp.conv2d_output_shape(st, st.shape)
+        e = dict(L=L, x=torch.randn(st.shape, device="cuda:0"),
+                 w=torch.randn(L["cout"], L["cin"] // L["groups"], L["kernel"], L["kernel"], device="cuda:0"),
+                 dy=torch.randn(osh, device="cuda:0"), bf=dlp.Conv2DBackwardFilter.create(st), bd=None if L["cin"] == 3 else dlp.Conv2DBackwardData.create(st))
+        e["dx"], e["dw"] = torch.empty_like(e["x"]), torch.empty_like(e["w"])
+        e["ws"] = torch.empty(max(e["bf"].workspace(), e["bd"].workspace() if e["bd"] else 0, 1), dtype=torch.uint8, device="cuda:0")
+        layers.append(e)
+
+    def step():
+        for e in layers:
+            e["bf"].enqueue(e["x"], e["dw"], e["dy"], e["ws"])
+            if e["bd"]:
+                e["bd"].enqueue(e["dx"], e["w"], e["dy"], e["ws"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    dlp.timing_reset()
+    dlp.timing_enable(True)
+    step()
+    torch.cuda.synchronize()
+    dlp.timing_enable(False)
+    sections = {}
+    for (section, ms) in dlp.timing_records():
+        sections[section] = round(sections.get(section, 0.0) + ms, 4)
+    dlp.timing_reset()
+    flops_f = sum(conv_flops(e["L"], args.batch) for e in layers)
+    flops_d = sum(conv_flops(e["L"], args.batch) for e in layers if e["bd"])
+    wgrad_ms = sections.get("wgrad", 0.0)
+    out = {
+        "metric": BASELINE_METRIC, "value": round(args.batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "gradients of the ResNet-18 convolution stack: backward filter of 20 layers, backward data of 19 (not conv1), "
+                               "fp32 NCHW, batch %d" % args.batch, "batch": args.batch,
+                   "gflop_per_step": round((flops_f + flops_d) / 1e9, 1)},
+        "gflops_per_s": round((flops_f + flops_d) / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac_of_fp32_matrix_peak": round((flops_f + flops_d) / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
+        "kernel_ms_by_section": sections,
+        "roofline": {"bound": "mfma", "kernel": "conv_wgrad_f32_kernel (20 launches)", "achieved": round(flops_f / (wgrad_ms * 1e-3) / 1e12, 2) if wgrad_ms else None,
+                     "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops_f / (wgrad_ms * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4) if wgrad_ms else None, "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full"])
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full", "resnet18-backward"])
     ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
@@ -244,6 +310,9 @@ def main():
     torch.cuda.set_device(0)
     if args.workload.endswith("-full"):
         run_graph_workload(args)
+        return
+    if args.workload == "resnet18-backward":
+        run_backward_workload(args)
         return
     layer_list, description = workload_layers(args.workload)
     if args.only:

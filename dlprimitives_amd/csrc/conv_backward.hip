@@ -13,9 +13,9 @@
 //    stride-1 convolution applies; the matrix cores then multiply the inserted zeros as well.
 //  * backward filter is a GEMM of its own: dW[Cout_g x Cin_g*KH*KW] = dy[Cout_g x B*OH*OW] *
 //    cols[B*OH*OW x Cin_g*KH*KW], reduction over the pixels of all images.  Both operands are
-//    contiguous along the reduction index in memory, so a workgroup stages 64 pixels of BM dy rows and
-//    BN gathered x rows in LDS (lane = pixel: coalesced loads, conflict-free stores) and every lane
-//    fetches its four k values of a row with one 16-byte LDS read.  The reduction is cut into slices
+//    contiguous along the reduction index in memory, so a workgroup stages 32 reduction indices of BM dy
+//    rows (16 bytes per lane) and BN gathered x rows (lane = pixel, the padding test one bit of a tap mask)
+//    in LDS and every lane fetches its four k values of a row with one 16-byte LDS read.  The reduction is cut into slices
 //    across workgroups; the slices' partial tiles go to the workspace in output order and one small
 //    kernel adds them up in slice order (deterministic).
 #include <algorithm>
@@ -30,7 +30,7 @@ namespace {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int KC = 64;        // pixels per staged chunk (one per lane)
+constexpr int KC = 32;        // reduction indices (pixels of the batch, image after image) per staged chunk
 constexpr int PITCH = KC + 4; // LDS row pitch in floats: 16-byte reads of 8 consecutive lanes cover all banks
 constexpr uint32_t kOutOfRange = 0x80000000u;
 
@@ -38,22 +38,26 @@ struct WgradArgs {
     const float *x, *dy;
     float *out; // dW itself (one slice) or the partial sums [slice][Cout][Ncol]
     int Cin, Cin_g, Cout, Cout_g, groups, H, W, OW, OHW, KH, KW, sh, sw, ph, pw, dh, dw;
-    int Ncol; // Cin_g * KH * KW
-    int mtiles, ntiles, slices, chunks, cpi, cps; // chunks in all, per image, per slice
+    int Ncol;   // Cin_g * KH * KW
+    int Ktotal; // B * OH * OW
+    int mtiles, ntiles, slices, chunks, cps; // chunks in all and per slice
     uint32_t x_bytes, dy_bytes;
-    uint32_t ow_magic, ow_shift, khw_magic, khw_shift, kw_magic, kw_shift, cpi_magic, cpi_shift;
+    uint32_t ow_magic, ow_shift, ohw_magic, ohw_shift, khw_magic, khw_shift, kw_magic, kw_shift;
     float factor;
 };
 
 // dW tile of BM filters x BN (channel, tap) columns over the chunks of one slice.
-template <int BM, int BN>
+// AVEC: OH * OW is a multiple of 4, dy rows are read 16 bytes per lane.
+// MASKED: KH * KW <= 31, the padding test of a gathered element is one bit of a per-lane tap mask.
+template <int BM, int BN, bool AVEC, bool MASKED>
 __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 MFMA blocks per wavefront (wavefronts 2 x 2)
-    constexpr int RA = BM / 4, RB = BN / 4;   // rows each wavefront stages
+    constexpr int RB = BN / 8;                // gathered rows per thread: two rows per wavefront load
+    constexpr int RA = AVEC ? BM / 32 : BM / 8;
     __shared__ __attribute__((aligned(16))) float As[BM * PITCH];
     __shared__ __attribute__((aligned(16))) float Bs[BN * PITCH];
-    __shared__ __attribute__((aligned(16))) int rowtab[BN * 4]; // per column: x offset of the tap, dy, dx, valid
+    __shared__ __attribute__((aligned(16))) int rowtab[BN * 4]; // per column: x offset of the tap, tap bit (or 31), row and column shift
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -79,37 +83,73 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
         const int r = (int)fast_div((uint32_t)rs, a.kw_magic, a.kw_shift);
         const int s = rs - r * a.KW;
         const int dr = r * a.dh - a.ph, ds = s * a.dw - a.pw;
-        rowtab[tid * 4 + 0] = ((int)c * a.H + dr) * a.W + ds;
-        rowtab[tid * 4 + 1] = dr;
-        rowtab[tid * 4 + 2] = ds;
-        rowtab[tid * 4 + 3] = n < a.Ncol ? 1 : 0;
+        const bool nv = n < a.Ncol;
+        rowtab[tid * 4 + 0] = nv ? ((int)c * a.H + dr) * a.W + ds : 0;
+        rowtab[tid * 4 + 1] = nv ? rs : 31; // bit 31 of a tap mask is never set
+        rowtab[tid * 4 + 2] = nv ? dr : -(1 << 28); // far outside the image for the comparing path
+        rowtab[tid * 4 + 3] = ds;
     }
     __syncthreads();
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void *)a.dy, 0, a.dy_bytes, 0x00020000);
 
-    float ra[RA], rb[RB];
-    // one chunk: 64 pixels (this lane's is pix0 + lane) of image b; rows wave, wave + 4, ...
+    float rb[RB];
+    float ra[AVEC ? 1 : RA];
+    f32x4 ra4[AVEC ? RA : 1];
+    const int brow = wave * 2 + h;                              // gathered rows brow + 8 * i, pixel l32 of the chunk
+    const int arow = AVEC ? wave * 8 + (lane >> 3) : brow;      // dy rows arow + 32 * i (16-byte pieces) or arow + 8 * i
     auto fetch = [&](int ck) {
-        const int b = (int)fast_div((uint32_t)ck, a.cpi_magic, a.cpi_shift);
-        const int pix = (ck - b * a.cpi) * KC + lane;
-        const bool pv = pix < a.OHW;
-        const int oh = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
-        const int ow = pix - oh * a.OW;
-        const int ohs = oh * a.sh, ows = ow * a.sw;
-        const uint32_t ybase = (uint32_t)((b * a.Cout + g * a.Cout_g + m0 + wave) * a.OHW + pix) * 4u;
+        {
+            const uint32_t kidx = (uint32_t)(ck * KC + l32);
+            const bool pv = kidx < (uint32_t)a.Ktotal;
+            const int b = (int)fast_div(kidx, a.ohw_magic, a.ohw_shift);
+            const int pix = (int)kidx - b * a.OHW;
+            const int oh = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+            const int ow = pix - oh * a.OW;
+            const int ohs = oh * a.sh, ows = ow * a.sw;
+            const int xbase = (b * a.Cin + g * a.Cin_g) * a.H * a.W + ohs * a.W + ows;
+            if (MASKED) {
+                uint32_t cols = 0, taps = 0;
+                for (int s = 0; s < a.KW; s++)
+                    cols |= ((unsigned)(ows + s * a.dw - a.pw) < (unsigned)a.W ? 1u : 0u) << s;
+                for (int r = 0; r < a.KH; r++)
+                    taps |= ((unsigned)(ohs + r * a.dh - a.ph) < (unsigned)a.H ? cols : 0u) << (r * a.KW);
+                const uint32_t bad = pv ? ~taps : 0xFFFFFFFFu;
 #pragma unroll
-        for (int i = 0; i < RA; i++) {
-            const bool ok = pv && (m0 + wave + 4 * i < a.Cout_g);
-            ra[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, ok ? ybase : kOutOfRange, (uint32_t)(4 * i * a.OHW) * 4u, 0));
+                for (int i = 0; i < RB; i++) {
+                    const int2 rt = *reinterpret_cast<const int2 *>(&rowtab[(brow + 8 * i) * 4]);
+                    const uint32_t off = ((uint32_t)(xbase + rt.x) << 2) | (((bad >> rt.y) & 1u) << 31);
+                    rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RB; i++) {
+                    const int4 rt = *reinterpret_cast<const int4 *>(&rowtab[(brow + 8 * i) * 4]);
+                    const bool ok = pv && (unsigned)(ohs + rt.z) < (unsigned)a.H && (unsigned)(ows + rt.w) < (unsigned)a.W;
+                    rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? (uint32_t)(xbase + rt.x) * 4u : kOutOfRange, 0, 0));
+                }
+            }
+            if (!AVEC) {
+                const uint32_t ybase = (uint32_t)((b * a.Cout + g * a.Cout_g + m0 + arow) * a.OHW + pix) * 4u;
+#pragma unroll
+                for (int i = 0; i < RA; i++) {
+                    const bool ok = pv && (m0 + arow + 8 * i < a.Cout_g);
+                    ra[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, ok ? ybase : kOutOfRange, (uint32_t)(8 * i * a.OHW) * 4u, 0));
+                }
+            }
         }
-        const int xbase = (b * a.Cin + g * a.Cin_g) * a.H * a.W + ohs * a.W + ows;
+        if (AVEC) { // four consecutive reduction indices of one dy row: never across two images, OH * OW being a multiple of 4
+            const uint32_t kidx = (uint32_t)(ck * KC + 4 * (lane & 7));
+            const bool pv = kidx < (uint32_t)a.Ktotal;
+            const int b = (int)fast_div(kidx, a.ohw_magic, a.ohw_shift);
+            const int pix = (int)kidx - b * a.OHW;
+            const uint32_t ybase = (uint32_t)((b * a.Cout + g * a.Cout_g + m0 + arow) * a.OHW + pix) * 4u;
 #pragma unroll
-        for (int i = 0; i < RB; i++) {
-            const int4 rt = *reinterpret_cast<const int4 *>(&rowtab[(wave + 4 * i) * 4]);
-            const bool ok = pv && rt.w != 0 && (unsigned)(ohs + rt.y) < (unsigned)a.H && (unsigned)(ows + rt.z) < (unsigned)a.W;
-            rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? (uint32_t)(xbase + rt.x) * 4u : kOutOfRange, 0, 0));
+            for (int i = 0; i < RA; i++) {
+                const bool ok = pv && (m0 + arow + 32 * i < a.Cout_g);
+                ra4[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(yr, ok ? ybase : kOutOfRange, (uint32_t)(32 * i * a.OHW) * 4u, 0));
+            }
         }
     };
 
@@ -126,16 +166,22 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
         fetch(ck_begin);
     for (int ck = ck_begin; ck < ck_end; ck++) {
         __syncthreads(); // the previous chunk has been read
+        if (AVEC) {
 #pragma unroll
-        for (int i = 0; i < RA; i++)
-            As[(wave + 4 * i) * PITCH + lane] = ra[i];
+            for (int i = 0; i < RA; i++)
+                *reinterpret_cast<f32x4 *>(&As[(arow + 32 * i) * PITCH + 4 * (lane & 7)]) = ra4[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < RA; i++)
+                As[(arow + 8 * i) * PITCH + l32] = ra[i];
+        }
 #pragma unroll
         for (int i = 0; i < RB; i++)
-            Bs[(wave + 4 * i) * PITCH + lane] = rb[i];
+            Bs[(brow + 8 * i) * PITCH + l32] = rb[i];
         __syncthreads();
         if (ck + 1 < ck_end)
             fetch(ck + 1); // lands while this chunk is multiplied
-        // k order inside a chunk: MFMA step 4*kq + e takes pixel 8*kq + e from the lower half-wave and
+        // k order inside a chunk: MFMA step 4*kq + e takes index 8*kq + e from the lower half-wave and
         // 8*kq + 4 + e from the upper one, for both operands alike
 #pragma unroll
         for (int kq = 0; kq < KC / 8; kq++) {
@@ -179,6 +225,55 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
                 }
             }
     }
+}
+
+// Depthwise 3x3 filter gradient (one input channel per group): every thread walks pixels of its
+// channel's planes, multiplies dy by the nine taps it meets and the workgroup adds the nine sums up.
+// Workgroup (k, slice) takes images slice, slice + slices, ...; partial sums [slice][Cout][9].
+__global__ __launch_bounds__(256) void depthwise_wgrad3x3_kernel(const float *__restrict__ x, const float *__restrict__ dy, float *__restrict__ part,
+                                                                int B, int Cin, int Cout, int mult, int H, int W, int OH, int OW, int sh, int sw, int ph,
+                                                                int pw, int dh, int dw)
+{
+    __shared__ float red[4][9];
+    const int k = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
+    const int c = k / mult;
+    const int ohw = OH * OW;
+    float acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; t++)
+        acc[t] = 0.0f;
+    for (int b = slice; b < B; b += slices) {
+        const float *xp = x + ((size_t)b * Cin + c) * H * W;
+        const float *yp = dy + ((size_t)b * Cout + k) * ohw;
+        for (int pix = threadIdx.x; pix < ohw; pix += 256) {
+            const float g = yp[pix];
+            const int oh = pix / OW, ow = pix - oh * OW;
+            const int ih0 = oh * sh - ph, iw0 = ow * sw - pw;
+#pragma unroll
+            for (int r = 0; r < 3; r++) {
+                const int ih = ih0 + r * dh;
+                const bool rv = (unsigned)ih < (unsigned)H;
+#pragma unroll
+                for (int q = 0; q < 3; q++) {
+                    const int iw = iw0 + q * dw;
+                    const float v = (rv && (unsigned)iw < (unsigned)W) ? xp[ih * W + iw] : 0.0f;
+                    acc[r * 3 + q] = fmaf(g, v, acc[r * 3 + q]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 9; t++) {
+        float v = acc[t];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1)
+            v += __shfl_down(v, off);
+        if ((threadIdx.x & 63) == 0)
+            red[threadIdx.x >> 6][t] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 9)
+        part[((size_t)slice * Cout + k) * 9 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
 // out[i] = factor * out[i] + sum over slices, in slice order
@@ -267,23 +362,32 @@ unsigned grid_for(size_t n)
 }
 
 struct WgradPlan {
-    int BM, BN, mtiles, ntiles, cpi, chunks, cps, slices;
+    int BM, BN, mtiles, ntiles, chunks, cps, slices;
+    bool depthwise; // depthwise_wgrad3x3_kernel: slices = workgroups per filter
     size_t part_bytes;
 };
 
-// Slices: enough workgroups for four per compute unit, at least two chunks each.
+constexpr int kWgradSlots = 256 * 3; // workgroups resident at once: three per compute unit
+
+// Slices: one full round of resident workgroups where the tiles allow it, at least two chunks each.
 WgradPlan wgrad_plan(const dlp_conv2d_settings &c, int batch, int OH, int OW)
 {
     WgradPlan p;
     const int cout_g = c.channels_out / c.groups, ncol = c.channels_in / c.groups * c.kernel[0] * c.kernel[1];
+    p.depthwise = c.channels_in == c.groups && c.kernel[0] == 3 && c.kernel[1] == 3 && cout_g <= 4;
+    if (p.depthwise) {
+        p.BM = p.BN = p.mtiles = p.ntiles = p.chunks = p.cps = 0;
+        p.slices = std::max(1, std::min(batch, (1024 + c.channels_out - 1) / c.channels_out));
+        p.part_bytes = (size_t)p.slices * c.channels_out * 9 * sizeof(float);
+        return p;
+    }
     p.BM = cout_g > 64 ? 128 : 64;
     p.BN = ncol > 64 ? 128 : 64;
     p.mtiles = (cout_g + p.BM - 1) / p.BM;
     p.ntiles = (ncol + p.BN - 1) / p.BN;
-    p.cpi = (OH * OW + KC - 1) / KC;
-    p.chunks = batch * p.cpi;
+    p.chunks = (int)(((long long)batch * OH * OW + KC - 1) / KC);
     const long long tiles = (long long)p.mtiles * p.ntiles * c.groups;
-    long long want = std::max<long long>(1, 1024 / tiles);
+    long long want = std::max<long long>(1, kWgradSlots / tiles);
     want = std::min<long long>(want, std::max(1, p.chunks / 2));
     p.cps = (int)((p.chunks + want - 1) / want);
     p.slices = (p.chunks + p.cps - 1) / p.cps;
@@ -476,6 +580,22 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
     if (x_elems >= (1ull << 31) / 4 || y_elems >= (1ull << 31) / 4)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensor of 2 GiB or more");
     WgradPlan p = wgrad_plan(c, batch, op->OH, op->OW);
+    if (p.depthwise) {
+        const size_t per_slice = n_out * sizeof(float);
+        p.slices = (int)std::min<size_t>(ws ? ws_bytes / per_slice : 0, (size_t)p.slices);
+        DLP_REQUIRE(p.slices >= 1, "workspace smaller than workspace()");
+        DLP_REQUIRE(c.channels_out <= 0x7FFFFFFF && p.slices <= 65535, "grid");
+        {
+            TimingScope ts("wgrad_depthwise", st);
+            hipLaunchKernelGGL(depthwise_wgrad3x3_kernel, dim3((unsigned)c.channels_out, (unsigned)p.slices), dim3(256), 0, st, (const float *)x,
+                               (const float *)dy, (float *)ws, batch, c.channels_in, c.channels_out, cout_g, c.shape[2], c.shape[3], op->OH, op->OW,
+                               c.stride[0], c.stride[1], c.pad[0], c.pad[1], c.dilate[0], c.dilate[1]);
+        }
+        TimingScope ts("wgrad_reduce", st);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
     if (p.slices > 1) {
         // fewer slices when the caller's workspace was sized for a smaller batch
         const size_t per_slice = n_out * sizeof(float);
@@ -512,29 +632,43 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
     a.mtiles = p.mtiles;
     a.ntiles = p.ntiles;
     a.slices = p.slices;
+    a.Ktotal = batch * op->OH * op->OW;
     a.chunks = p.chunks;
-    a.cpi = p.cpi;
     a.cps = p.cps;
     a.x_bytes = (uint32_t)(x_elems * 4);
     a.dy_bytes = (uint32_t)(y_elems * 4);
     make_magic((uint32_t)a.OW, a.ow_magic, a.ow_shift);
     make_magic((uint32_t)(a.KH * a.KW), a.khw_magic, a.khw_shift);
     make_magic((uint32_t)a.KW, a.kw_magic, a.kw_shift);
-    make_magic((uint32_t)a.cpi, a.cpi_magic, a.cpi_shift);
+    make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
     a.factor = factor;
     const long long wgs = (long long)p.mtiles * p.ntiles * c.groups * p.slices;
     DLP_REQUIRE(wgs < (1ll << 31), "too many workgroups");
     {
         TimingScope ts("wgrad", st);
         const dim3 grid((unsigned)wgs), block(256);
+        const bool avec = a.OHW % 4 == 0 && ((uintptr_t)dy & 15) == 0;
+        const bool masked = a.KH * a.KW <= 31;
+#define DLP_WGRAD_LAUNCH(BM_, BN_)                                                                             \
+    do {                                                                                                       \
+        if (avec && masked)                                                                                    \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, true, true>), grid, block, 0, st, a);          \
+        else if (avec)                                                                                         \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, true, false>), grid, block, 0, st, a);         \
+        else if (masked)                                                                                       \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, false, true>), grid, block, 0, st, a);         \
+        else                                                                                                   \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, false, false>), grid, block, 0, st, a);        \
+    } while (0)
         if (p.BM == 128 && p.BN == 128)
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<128, 128>), grid, block, 0, st, a);
+            DLP_WGRAD_LAUNCH(128, 128);
         else if (p.BM == 128)
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<128, 64>), grid, block, 0, st, a);
+            DLP_WGRAD_LAUNCH(128, 64);
         else if (p.BN == 128)
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<64, 128>), grid, block, 0, st, a);
+            DLP_WGRAD_LAUNCH(64, 128);
         else
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<64, 64>), grid, block, 0, st, a);
+            DLP_WGRAD_LAUNCH(64, 64);
+#undef DLP_WGRAD_LAUNCH
     }
     if (p.slices > 1) {
         TimingScope ts("wgrad_reduce", st);

@@ -108,6 +108,22 @@ def test_gpu_backward_accumulates_with_factor(oracle_mod, algo):
         _run_case(dlp, torch, oracle_mod, c, bhw, 6, factor_dx=1.0, factor_dw=1.0, algo=algo)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(6, 6, 1, 1, 1, (3, 9, 11)), (4, 8, 2, 1, 1, (2, 12, 7)), (5, 5, 1, 2, 1, (70, 8, 8)), (3, 12, 1, 1, 0, (1, 5, 5)),
+                                   (16, 16, (2, 1), (1, 2), (2, 0), (2, 17, 20))], ids=str)
+def test_gpu_depthwise_backward(oracle_mod, shape):
+    """One input channel per group (channel multiplier 1, 2, 4), strides, dilation, more images than slices."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from conv_cases import case
+
+    cin, cout, stride, dilate, pad, bhw = shape
+    c = case(3, pad, stride, dilate, cin, cout, False, cin, False)
+    _run_case(dlp, torch, oracle_mod, c, bhw, 21)
+    _run_case(dlp, torch, oracle_mod, c, bhw, 22, factor_dx=0.5, factor_dw=2.0)
+
+
 LAYERS = [  # ResNet-18 / MobileNet-v2 layer shapes: cin, cout, k, s, p, groups, H, batch
     (64, 64, 3, 1, 1, 1, 56, 16),
     (64, 128, 3, 2, 1, 1, 56, 16),
