@@ -9,8 +9,11 @@
 //  * backward data is a forward convolution of dy with the filter transposed within its group and
 //    flipped in both axes, stride 1, padding dilate * (kernel - 1) - pad; it runs on the forward
 //    operator of this library (every algorithm and tile shape of the forward path serves it).  For
-//    stride > 1, dy is first spread out with zeros between its elements (workspace), so that the same
-//    stride-1 convolution applies; the matrix cores then multiply the inserted zeros as well.
+//    stride > 1 the rows h = stride * i + a of dx (phase a) only meet the filter rows r with
+//    a + pad - r * dilate divisible by the stride; over those the pass is again a stride-1 convolution of
+//    dy (for a 3x3 filter at stride 2: filters of 1x1, 1x2, 2x1 and 2x2 taps), so every phase runs on the
+//    forward operator into the workspace and one kernel interleaves the phases into dx.  No multiply
+//    is spent on zeros.
 //  * backward filter is a GEMM of its own: dW[Cout_g x Cin_g*KH*KW] = dy[Cout_g x B*OH*OW] *
 //    cols[B*OH*OW x Cin_g*KH*KW], reduction over the pixels of all images.  Both operands are
 //    contiguous along the reduction index in memory, so a workgroup stages 32 reduction indices of BM dy
@@ -311,22 +314,56 @@ __global__ __launch_bounds__(256) void filter_transpose_flip_kernel(const float 
     }
 }
 
-// up[p][hu][wu] = dy[p][hu / sh][wu / sw] where both divide and the quotient is inside dy, else 0
-__global__ __launch_bounds__(256) void spread_with_zeros_kernel(const float *__restrict__ dy, float *__restrict__ up, size_t planes, int OH, int OW, int Hu,
-                                                                int Wu, int sh, int sw)
+// One phase of a strided backward-data pass.  dx rows h = sh * i + a only meet the filter rows r with
+// (a + ph - r * dh) divisible by sh; over those rows the pass is a stride-1 correlation of dy.
+// wt[g][c][k][jh][jw] = w[g][k][c][rh(nh - 1 - jh)][rw(nw - 1 - jw)], r(j) = r0 + j * rstep.
+struct PhaseFilterArgs {
+    int groups, cout_g, cin_g, KH, KW;
+    int nh, nw, rh0, rhstep, rw0, rwstep;
+};
+__global__ __launch_bounds__(256) void phase_filter_kernel(const float *__restrict__ w, float *__restrict__ wt, PhaseFilterArgs a)
 {
-    const size_t n = planes * Hu * Wu;
+    const int taps = a.nh * a.nw;
+    const size_t n = (size_t)a.groups * a.cin_g * a.cout_g * taps;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const int wu = (int)(i % Wu);
-        const size_t q = i / Wu;
-        const int hu = (int)(q % Hu);
-        const size_t p = q / Hu;
-        const int oh = hu / sh, ow = wu / sw;
+        const int jw = (int)(i % a.nw);
+        size_t q = i / a.nw;
+        const int jh = (int)(q % a.nh);
+        q /= a.nh;
+        const int k = (int)(q % a.cout_g);
+        q /= a.cout_g;
+        const int c = (int)(q % a.cin_g);
+        const int g = (int)(q / a.cin_g);
+        const int rh = a.rh0 + (a.nh - 1 - jh) * a.rhstep, rw = a.rw0 + (a.nw - 1 - jw) * a.rwstep;
+        wt[i] = w[((((size_t)g * a.cout_g + k) * a.cin_g + c) * a.KH + rh) * a.KW + rw];
+    }
+}
+
+// dx[p][sh * i + a][sw * j + b] = factor * dx + phase(a, b)[p][i + off_h][j + off_w] (0 for a phase without filter taps)
+constexpr int kMaxPhases = 16;
+struct InterleaveArgs {
+    const float *buf[kMaxPhases];
+    int out_h[kMaxPhases], out_w[kMaxPhases], off_h[kMaxPhases], off_w[kMaxPhases];
+    int H, W, sh, sw;
+    float factor;
+};
+__global__ __launch_bounds__(256) void phase_interleave_kernel(float *__restrict__ dx, size_t planes, InterleaveArgs a)
+{
+    const size_t n = planes * a.H * a.W;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+        const int w = (int)(e % a.W);
+        const size_t q = e / a.W;
+        const int h = (int)(q % a.H);
+        const size_t p = q / a.H;
+        const int i = h / a.sh, j = w / a.sw;
+        const int ph = (h - i * a.sh) * a.sw + (w - j * a.sw);
+        const float *buf = a.buf[ph];
         float v = 0.0f;
-        if (oh * sh == hu && ow * sw == wu && oh < OH && ow < OW)
-            v = dy[(p * OH + oh) * OW + ow];
-        up[i] = v;
+        if (buf)
+            v = buf[(p * a.out_h[ph] + i + a.off_h[ph]) * a.out_w[ph] + j + a.off_w[ph]];
+        dx[e] = a.factor != 0.0f ? fmaf(dx[e], a.factor, v) : v;
     }
 }
 
@@ -400,12 +437,27 @@ WgradPlan wgrad_plan(const dlp_conv2d_settings &c, int batch, int OH, int OW)
 
 using namespace dlp;
 
+// One axis of one phase: filter rows r0, r0 + rstep, ... (n of them), and the stride-1 convolution over dy
+// that computes the phase: kernel extent n, dilation dil, symmetric padding pad; its output has `out`
+// rows of which rows off .. off + len - 1 are the phase's rows of dx.
+struct PhaseAxis {
+    int n, r0, rstep, dil, pad, off, out, len;
+};
+
+struct BwdPhase {
+    PhaseAxis h, w;
+    dlp_conv2d_fwd *fwd;
+    size_t wt_bytes, fwd_ws;
+};
+
 struct dlp_conv2d_bwd_data {
     dlp_conv2d_settings cfg;
-    dlp_conv2d_fwd *fwd; // the stride-1 convolution dy -> dx
-    int OH, OW, Hu, Wu;  // dy, and dy spread out by the stride (== dy for stride 1)
-    bool spread;
-    size_t wt_bytes, fwd_ws;
+    int OH, OW;
+    bool strided;            // one stride-1 convolution per phase, then interleaved into dx
+    dlp_conv2d_fwd *fwd;     // stride 1: the convolution dy -> dx on the transposed, flipped filter
+    size_t wt_bytes, fwd_ws; // stride 1
+    BwdPhase phase[kMaxPhases];
+    int nphases;
 };
 
 struct dlp_conv2d_bwd_filter {
@@ -425,6 +477,46 @@ static int check_settings(const dlp_conv2d_settings *cfg, int out[4])
 
 extern "C" {
 
+static PhaseAxis phase_axis(int a, int size, int osize, int k, int stride, int dilate, int pad)
+{
+    PhaseAxis x = {0, 0, 1, 1, 0, 0, 0, 0};
+    x.len = a < size ? (size - a + stride - 1) / stride : 0;
+    int qmax = 0, qmin = 0, r1 = -1;
+    for (int r = 0; r < k; r++) {
+        const int v = a + pad - r * dilate;
+        if (((v % stride) + stride) % stride != 0)
+            continue;
+        const int q = (v - (((v % stride) + stride) % stride)) / stride; // exact
+        if (x.n == 0) {
+            x.r0 = r;
+            qmax = q;
+        } else if (x.n == 1)
+            r1 = r;
+        qmin = q;
+        x.n++;
+    }
+    if (x.n == 0 || x.len == 0) {
+        x.n = 0;
+        return x;
+    }
+    if (x.n > 1) {
+        x.rstep = r1 - x.r0;
+        x.dil = dilate * x.rstep / stride;
+    }
+    x.pad = std::max(0, std::max(-qmin, x.len + qmax - osize));
+    x.off = qmin + x.pad;
+    x.out = osize + 2 * x.pad - x.dil * (x.n - 1);
+    return x;
+}
+
+static void bwd_data_free(dlp_conv2d_bwd_data *op)
+{
+    dlp_conv2d_fwd_destroy(op->fwd);
+    for (int i = 0; i < op->nphases; i++)
+        dlp_conv2d_fwd_destroy(op->phase[i].fwd);
+    delete op;
+}
+
 int dlp_conv2d_bwd_data_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_data **out)
 {
     DLP_REQUIRE(out != nullptr, "null argument");
@@ -433,52 +525,109 @@ int dlp_conv2d_bwd_data_create(const dlp_conv2d_settings *cfg, const char *algo,
     int rc = check_settings(cfg, oshape);
     if (rc != DLP_OK)
         return rc;
-    dlp_conv2d_settings t = *cfg;
-    t.channels_in = cfg->channels_out;
-    t.channels_out = cfg->channels_in;
-    bool spread = false;
-    for (int i = 0; i < 2; i++) {
-        t.stride[i] = 1;
-        t.pad[i] = cfg->dilate[i] * (cfg->kernel[i] - 1) - cfg->pad[i];
-        if (t.pad[i] < 0)
-            return fail(DLP_ERR_NOT_IMPLEMENTED, "backward data: padding larger than dilate * (kernel - 1)");
-        // size of dy spread by the stride, with the rows/columns the forward window never reached
-        t.shape[2 + i] = cfg->shape[2 + i] + 2 * cfg->pad[i] - cfg->dilate[i] * (cfg->kernel[i] - 1);
-        spread = spread || cfg->stride[i] != 1;
-    }
-    t.shape[1] = cfg->channels_out;
     dlp_conv2d_bwd_data *op = new (std::nothrow) dlp_conv2d_bwd_data();
     if (!op)
         return fail(DLP_ERR_RUNTIME, "out of host memory");
     op->cfg = *cfg;
     op->OH = oshape[2];
     op->OW = oshape[3];
-    op->Hu = t.shape[2];
-    op->Wu = t.shape[3];
-    op->spread = spread;
     op->fwd = nullptr;
-    rc = dlp_conv2d_fwd_create(&t, 0, DLP_ACT_IDENTITY, algo, &op->fwd);
-    if (rc != DLP_OK) {
-        delete op;
-        return rc;
+    op->nphases = 0;
+    op->strided = cfg->stride[0] != 1 || cfg->stride[1] != 1;
+    dlp_conv2d_settings t = *cfg;
+    t.channels_in = cfg->channels_out;
+    t.channels_out = cfg->channels_in;
+    t.stride[0] = t.stride[1] = 1;
+    t.shape[1] = cfg->channels_out;
+    t.shape[2] = op->OH;
+    t.shape[3] = op->OW;
+    const size_t cin_g = cfg->channels_in / cfg->groups;
+    if (!op->strided) {
+        for (int i = 0; i < 2; i++) {
+            t.pad[i] = cfg->dilate[i] * (cfg->kernel[i] - 1) - cfg->pad[i];
+            if (t.pad[i] < 0) {
+                delete op;
+                return fail(DLP_ERR_NOT_IMPLEMENTED, "backward data: padding larger than dilate * (kernel - 1)");
+            }
+        }
+        rc = dlp_conv2d_fwd_create(&t, 0, DLP_ACT_IDENTITY, algo, &op->fwd);
+        if (rc != DLP_OK) {
+            delete op;
+            return rc;
+        }
+        op->wt_bytes = round256((size_t)cfg->channels_out * cin_g * cfg->kernel[0] * cfg->kernel[1] * sizeof(float));
+        op->fwd_ws = round256(dlp_conv2d_fwd_workspace(op->fwd));
+        *out = op;
+        return DLP_OK;
     }
-    op->wt_bytes = round256((size_t)cfg->channels_out * (cfg->channels_in / cfg->groups) * cfg->kernel[0] * cfg->kernel[1] * sizeof(float));
-    op->fwd_ws = round256(dlp_conv2d_fwd_workspace(op->fwd));
+    if (cfg->stride[0] * cfg->stride[1] > kMaxPhases) {
+        delete op;
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "backward data: more than 16 stride phases");
+    }
+    op->nphases = cfg->stride[0] * cfg->stride[1];
+    for (int i = 0; i < op->nphases; i++)
+        op->phase[i].fwd = nullptr;
+    for (int a = 0; a < cfg->stride[0]; a++)
+        for (int b = 0; b < cfg->stride[1]; b++) {
+            BwdPhase &ph = op->phase[a * cfg->stride[1] + b];
+            ph.h = phase_axis(a, cfg->shape[2], op->OH, cfg->kernel[0], cfg->stride[0], cfg->dilate[0], cfg->pad[0]);
+            ph.w = phase_axis(b, cfg->shape[3], op->OW, cfg->kernel[1], cfg->stride[1], cfg->dilate[1], cfg->pad[1]);
+            ph.wt_bytes = ph.fwd_ws = 0;
+            if (ph.h.n == 0 || ph.w.n == 0)
+                continue; // no filter tap meets this phase: its part of dx is zero
+            dlp_conv2d_settings u = t;
+            u.kernel[0] = ph.h.n;
+            u.kernel[1] = ph.w.n;
+            u.dilate[0] = ph.h.dil;
+            u.dilate[1] = ph.w.dil;
+            u.pad[0] = ph.h.pad;
+            u.pad[1] = ph.w.pad;
+            rc = dlp_conv2d_fwd_create(&u, 0, DLP_ACT_IDENTITY, algo, &ph.fwd);
+            if (rc != DLP_OK) {
+                bwd_data_free(op);
+                return rc;
+            }
+            ph.wt_bytes = round256((size_t)cfg->channels_out * cin_g * ph.h.n * ph.w.n * sizeof(float));
+            ph.fwd_ws = round256(dlp_conv2d_fwd_workspace(ph.fwd));
+        }
     *out = op;
     return DLP_OK;
 }
 
-const char *dlp_conv2d_bwd_data_algo(const dlp_conv2d_bwd_data *op) { return op ? dlp_conv2d_fwd_algo(op->fwd) : ""; }
-
-static size_t bwd_data_spread_bytes(const dlp_conv2d_bwd_data *op, int batch)
+const char *dlp_conv2d_bwd_data_algo(const dlp_conv2d_bwd_data *op)
 {
-    return op->spread ? round256((size_t)batch * op->cfg.channels_out * op->Hu * op->Wu * sizeof(float)) : 0;
+    if (!op)
+        return "";
+    if (!op->strided)
+        return dlp_conv2d_fwd_algo(op->fwd);
+    for (int i = 0; i < op->nphases; i++)
+        if (op->phase[i].fwd)
+            return dlp_conv2d_fwd_algo(op->phase[i].fwd);
+    return "gemm";
 }
 
-size_t dlp_conv2d_bwd_data_workspace(const dlp_conv2d_bwd_data *op)
+// strided: [phase filters][phase outputs for `batch` images][largest forward workspace]
+static size_t bwd_data_need(const dlp_conv2d_bwd_data *op, int batch, size_t *fwd_ws_out)
 {
-    return op ? op->wt_bytes + bwd_data_spread_bytes(op, std::max(op->cfg.shape[0], 1)) + op->fwd_ws : 0;
+    if (!op->strided) {
+        if (fwd_ws_out)
+            *fwd_ws_out = op->fwd_ws;
+        return op->wt_bytes + op->fwd_ws;
+    }
+    size_t total = 0, fws = 0;
+    for (int i = 0; i < op->nphases; i++) {
+        const BwdPhase &ph = op->phase[i];
+        if (!ph.fwd)
+            continue;
+        total += ph.wt_bytes + round256((size_t)batch * op->cfg.channels_in * ph.h.out * ph.w.out * sizeof(float));
+        fws = std::max(fws, ph.fwd_ws);
+    }
+    if (fwd_ws_out)
+        *fwd_ws_out = fws;
+    return total + fws;
 }
+
+size_t dlp_conv2d_bwd_data_workspace(const dlp_conv2d_bwd_data *op) { return op ? bwd_data_need(op, std::max(op->cfg.shape[0], 1), nullptr) : 0; }
 
 int dlp_conv2d_bwd_data_enqueue(dlp_conv2d_bwd_data *op, const int x_shape[4], void *dx, const void *w, const void *dy, void *ws, size_t ws_bytes,
                                 float factor, void *stream)
@@ -491,40 +640,75 @@ int dlp_conv2d_bwd_data_enqueue(dlp_conv2d_bwd_data *op, const int x_shape[4], v
     if (batch == 0)
         return DLP_OK;
     DLP_REQUIRE(dx != nullptr && w != nullptr && dy != nullptr, "null tensor pointer");
-    const size_t spread_bytes = bwd_data_spread_bytes(op, batch);
-    const size_t need = op->wt_bytes + spread_bytes + op->fwd_ws;
+    size_t fwd_ws = 0;
+    const size_t need = bwd_data_need(op, batch, &fwd_ws);
     DLP_REQUIRE(ws != nullptr && ws_bytes >= need, "workspace smaller than workspace() for this batch");
     hipStream_t st = (hipStream_t)stream;
     const dlp_conv2d_settings &c = op->cfg;
-    float *wt = (float *)ws;
-    float *up = (float *)((char *)ws + op->wt_bytes);
-    void *fws = (char *)ws + op->wt_bytes + spread_bytes;
     const int cout_g = c.channels_out / c.groups, cin_g = c.channels_in / c.groups, khw = c.kernel[0] * c.kernel[1];
-    {
-        TimingScope ts("bwd_data_filter_transpose", st);
-        hipLaunchKernelGGL(filter_transpose_flip_kernel, dim3(grid_for((size_t)c.channels_out * cin_g * khw)), dim3(256), 0, st, (const float *)w, wt,
-                           c.groups, cout_g, cin_g, khw);
+    const int in_shape[4] = {batch, c.channels_out, op->OH, op->OW};
+    if (!op->strided) {
+        float *wt = (float *)ws;
+        void *fws = (char *)ws + op->wt_bytes;
+        {
+            TimingScope ts("bwd_data_filter_transpose", st);
+            hipLaunchKernelGGL(filter_transpose_flip_kernel, dim3(grid_for((size_t)c.channels_out * cin_g * khw)), dim3(256), 0, st, (const float *)w, wt,
+                               c.groups, cout_g, cin_g, khw);
+        }
+        DLP_HIP_TRY(hipGetLastError());
+        return dlp_conv2d_fwd_enqueue(op->fwd, in_shape, dy, wt, nullptr, dx, op->fwd_ws ? fws : nullptr, op->fwd_ws, factor, stream);
     }
-    const void *src = dy;
-    if (op->spread) {
-        const size_t planes = (size_t)batch * c.channels_out;
-        DLP_REQUIRE(planes * op->Hu * op->Wu < (1ull << 31) / 4, "tensor of 2 GiB or more");
-        TimingScope ts("bwd_data_spread", st);
-        hipLaunchKernelGGL(spread_with_zeros_kernel, dim3(grid_for(planes * op->Hu * op->Wu)), dim3(256), 0, st, (const float *)dy, up, planes, op->OH,
-                           op->OW, op->Hu, op->Wu, c.stride[0], c.stride[1]);
-        src = up;
+    const size_t planes = (size_t)batch * c.channels_in;
+    DLP_REQUIRE(planes * c.shape[2] * c.shape[3] < (1ull << 31) / 4, "tensor of 2 GiB or more");
+    InterleaveArgs ia;
+    ia.H = c.shape[2];
+    ia.W = c.shape[3];
+    ia.sh = c.stride[0];
+    ia.sw = c.stride[1];
+    ia.factor = factor;
+    char *cursor = (char *)ws;
+    void *fws = (char *)ws + (need - fwd_ws);
+    for (int i = 0; i < kMaxPhases; i++) {
+        ia.buf[i] = nullptr;
+        ia.out_h[i] = ia.out_w[i] = 1;
+        ia.off_h[i] = ia.off_w[i] = 0;
+    }
+    for (int i = 0; i < op->nphases; i++) {
+        const BwdPhase &ph = op->phase[i];
+        if (!ph.fwd)
+            continue;
+        float *wt = (float *)cursor;
+        cursor += ph.wt_bytes;
+        float *outp = (float *)cursor;
+        cursor += round256(planes * ph.h.out * ph.w.out * sizeof(float));
+        PhaseFilterArgs fa = {c.groups, cout_g, cin_g, c.kernel[0], c.kernel[1], ph.h.n, ph.w.n, ph.h.r0, ph.h.rstep, ph.w.r0, ph.w.rstep};
+        {
+            TimingScope ts("bwd_data_phase_filter", st);
+            hipLaunchKernelGGL(phase_filter_kernel, dim3(grid_for((size_t)c.channels_out * cin_g * ph.h.n * ph.w.n)), dim3(256), 0, st, (const float *)w,
+                               wt, fa);
+        }
+        DLP_HIP_TRY(hipGetLastError());
+        int rc = dlp_conv2d_fwd_enqueue(ph.fwd, in_shape, dy, wt, nullptr, outp, ph.fwd_ws ? fws : nullptr, ph.fwd_ws, 0.0f, stream);
+        if (rc != DLP_OK)
+            return rc;
+        ia.buf[i] = outp;
+        ia.out_h[i] = ph.h.out;
+        ia.out_w[i] = ph.w.out;
+        ia.off_h[i] = ph.h.off;
+        ia.off_w[i] = ph.w.off;
+    }
+    {
+        TimingScope ts("bwd_data_interleave", st);
+        hipLaunchKernelGGL(phase_interleave_kernel, dim3(grid_for(planes * c.shape[2] * c.shape[3])), dim3(256), 0, st, (float *)dx, planes, ia);
     }
     DLP_HIP_TRY(hipGetLastError());
-    const int in_shape[4] = {batch, c.channels_out, op->Hu, op->Wu};
-    return dlp_conv2d_fwd_enqueue(op->fwd, in_shape, src, wt, nullptr, dx, op->fwd_ws ? fws : nullptr, op->fwd_ws, factor, stream);
+    return DLP_OK;
 }
 
 void dlp_conv2d_bwd_data_destroy(dlp_conv2d_bwd_data *op)
 {
-    if (!op)
-        return;
-    dlp_conv2d_fwd_destroy(op->fwd);
-    delete op;
+    if (op)
+        bwd_data_free(op);
 }
 
 int dlp_conv2d_bwd_filter_create(const dlp_conv2d_settings *cfg, const char *algo, dlp_conv2d_bwd_filter **out)

@@ -41,24 +41,32 @@ def test_backward_symbols_are_exported():
         assert hasattr(dlp.lib(), name)
 
 
-def test_backward_create_checks_arguments():
-    """No GPU needed: creation only plans."""
+def test_backward_create_rejects_bad_arguments():
+    """Rejected before anything touches a device."""
     import dlprimitives_amd as dlp
 
     s = dlp.Conv2DSettings(8, 16, 3, 2, 1, 1, 1, (4, 8, 17, 17))
-    d = dlp.Conv2DBackwardData.create(s)
-    f = dlp.Conv2DBackwardFilter.create(s)
-    assert f.algo() == "gemm" and d.algo() in ("gemm", "winograd", "depthwise_separable")
-    # dy spread by the stride: 4 x 16 x 17 x 17 floats, plus the transposed filter
-    assert d.workspace() >= 4 * 16 * 17 * 17 * 4 + 16 * 8 * 9 * 4
     with pytest.raises(dlp.ValidationError):
         dlp.Conv2DBackwardData.create(dlp.Conv2DSettings(8, 16, 3, 1, 1, 1, 3, (1, 8, 8, 8)))
     with pytest.raises(dlp.ValidationError):
         dlp.Conv2DBackwardFilter.create(s, "fft")
     with pytest.raises(dlp.NotImplementedErrorDlprim):
-        dlp.Conv2DBackwardData.create(dlp.Conv2DSettings(8, 16, 1, 1, 1, 1, 1, (1, 8, 8, 8)))  # pad > dilate * (kernel - 1)
+        dlp.Conv2DBackwardData.create(dlp.Conv2DSettings(8, 16, 1, 1, 1, 1, 1, (1, 8, 8, 8)))  # stride 1 with pad > dilate * (kernel - 1)
     with pytest.raises(dlp.NotImplementedErrorDlprim):
         dlp.Conv2DBackwardFilter.create(dlp.Conv2DSettings(8, 16, 3, 1, 1, 1, 1, (1, 8, 8, 8), dtype=dlp.capi.BFLOAT16_DATA))
+    f = dlp.Conv2DBackwardFilter.create(s)
+    assert f.algo() == "gemm" and f.workspace() > 0
+
+
+@pytest.mark.gpu
+def test_gpu_backward_data_workspace():
+    import dlprimitives_amd as dlp
+
+    s = dlp.Conv2DSettings(8, 16, 3, 2, 1, 1, 1, (4, 8, 17, 17))
+    d = dlp.Conv2DBackwardData.create(s)
+    assert d.algo() in ("gemm", "winograd", "depthwise_separable")
+    # the four stride phases of dx (4 x 8 x 17 x 17 floats in all) and their filters (16 x 8 x 9 taps in all)
+    assert d.workspace() >= 4 * 8 * 17 * 17 * 4 + 16 * 8 * 9 * 4
 
 
 def _run_case(dlp, torch, oracle_mod, c, bhw, seed, factor_dx=0.0, factor_dw=0.0, algo=""):
@@ -70,7 +78,8 @@ def _run_case(dlp, torch, oracle_mod, c, bhw, seed, factor_dx=0.0, factor_dw=0.0
     old_dw = rng.standard_normal(w.shape).astype(np.float32)
     s = _settings(dlp, c, x.shape)
     out = {}
-    if c["pad"][0] <= c["dilate"][0] * (c["kernel"][0] - 1) and c["pad"][1] <= c["dilate"][1] * (c["kernel"][1] - 1):
+    strided = c["stride"] != (1, 1)
+    if strided or (c["pad"][0] <= c["dilate"][0] * (c["kernel"][0] - 1) and c["pad"][1] <= c["dilate"][1] * (c["kernel"][1] - 1)):
         op = dlp.Conv2DBackwardData.create(s, algo)
         dx = _dev(old_dx) if factor_dx else torch.full(x.shape, float("nan"), device="cuda:0")
         op.enqueue(dx, _dev(w), _dev(dy), _ws(torch, op.workspace()), factor_dx)
@@ -122,6 +131,25 @@ def test_gpu_depthwise_backward(oracle_mod, shape):
     c = case(3, pad, stride, dilate, cin, cout, False, cin, False)
     _run_case(dlp, torch, oracle_mod, c, bhw, 21)
     _run_case(dlp, torch, oracle_mod, c, bhw, 22, factor_dx=0.5, factor_dw=2.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("geom", [(3, 2, 1, 1, 9), (3, 2, 1, 1, 10), (3, 2, 1, 0, 9), (1, 2, 1, 0, 9), (1, 2, 1, 0, 10), (5, 3, 1, 2, 11), (5, 2, 2, 3, 13),
+                                  (3, 3, 2, 5, 9), (4, 2, 1, 1, 8), (2, 4, 1, 0, 11), (7, 2, 1, 3, 20), ((3, 5), (2, 3), (3, 2), (1, 2), 17),
+                                  ((1, 3), (2, 1), (1, 1), (0, 1), 8), (3, (1, 2), 1, 1, 7)], ids=str)
+def test_gpu_strided_backward_data_phases(oracle_mod, geom):
+    """Strides, dilations and paddings that give phases with no, one and several taps, phases that start
+    before or after dy's first row, rows of dx the forward window never reached, padding beyond the filter."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from conv_cases import case
+
+    k, s, d, p, hw = geom
+    for groups, cin, cout in ((1, 5, 7), (2, 4, 6)):
+        c = case(k, p, s, d, cin, cout, False, groups, False)
+        _run_case(dlp, torch, oracle_mod, c, (2, hw, hw + 3), 31)
+        _run_case(dlp, torch, oracle_mod, c, (3, hw + 2, hw), 32, factor_dx=-0.5, factor_dw=0.0)
 
 
 LAYERS = [  # ResNet-18 / MobileNet-v2 layer shapes: cin, cout, k, s, p, groups, H, batch
