@@ -97,7 +97,9 @@ def build_layers(layer_list, batch, seed, bf16=False):
         op = dlp.Conv2DForward.create(st, True, L["activation"], L["algo"])
         assert op.algo() == L["algo"], (op.algo(), L["algo"])
         ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
-        out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch, 2 if bf16 else 4)))
+        packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda")
+        op.pack(w, packed)  # used only with --prepacked
+        out.append(dict(layer=L, op=op, x=x, w=w, b=b, y=y, ws=ws, packed=packed, flops=conv_flops(L, batch), bytes=conv_bytes(L, batch, 2 if bf16 else 4)))
     return out
 
 
@@ -292,6 +294,9 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
+    ap.add_argument("--prepacked", action="store_true",
+                    help="weights transformed once before the timed region (dlp_conv2d_fwd_pack / _enqueue_packed), as an inference "
+                         "deployment does; the default transforms them in every step, as the reference's enqueue contract implies")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -325,8 +330,12 @@ def main():
     stream = torch.cuda.current_stream()
 
     def step():
-        for e in layers:
-            e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+        if args.prepacked:
+            for e in layers:
+                e["op"].enqueue_packed(e["x"], e["w"], e["packed"], e["b"], e["y"], e["ws"], 0.0)
+        else:
+            for e in layers:
+                e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
 
     for _ in range(args.warmup):
         step()
@@ -349,7 +358,10 @@ def main():
     for s in range(args.steps):
         for i, e in enumerate(layers):
             first = dlp.timing_count()
-            e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+            if args.prepacked:
+                e["op"].enqueue_packed(e["x"], e["w"], e["packed"], e["b"], e["y"], e["ws"], 0.0)
+            else:
+                e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
             spans.append((i, first, dlp.timing_count()))
     torch.cuda.synchronize()
     dlp.timing_enable(False)
@@ -419,7 +431,8 @@ def main():
         "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32",
         "data": "synthetic",
         "config": {"workload": "%s%s, %s NCHW, batch %d" % (description, " (subset --only %s)" % args.only if args.only else "",
-                                                            "bf16" if bf16 else "fp32", args.batch),
+                                                            "bf16" if bf16 else "fp32", args.batch) +
+                               (", weights packed once before the timed region" if args.prepacked else ""),
                    "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1),
                    "mbytes_per_step": round(total_bytes / 1e6, 1)},
         "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),

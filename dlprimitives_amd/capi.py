@@ -223,6 +223,27 @@ class Conv2DForward:
         _check(lib().dlp_conv2d_fwd_enqueue(self._h, xs, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
                                             float(factor), _stream(stream)))
 
+    def packed_size(self):
+        """bytes of the buffer that pack() fills (0: nothing to transform)"""
+        lib().dlp_conv2d_fwd_packed_bytes.restype = ctypes.c_size_t
+        lib().dlp_conv2d_fwd_packed_bytes.argtypes = [ctypes.c_void_p]
+        return int(lib().dlp_conv2d_fwd_packed_bytes(self._h))
+
+    def pack(self, w, packed, stream=None):
+        """transform weights that stay constant once; packed: uint8 device tensor of packed_size() bytes"""
+        lib().dlp_conv2d_fwd_pack.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        _check(lib().dlp_conv2d_fwd_pack(self._h, _ptr(w), _ptr(packed), _stream(stream)))
+
+    def enqueue_packed(self, x, w, packed, bias, y, ws=None, factor=0.0, stream=None):
+        """enqueue() on weights that pack() transformed earlier; ws is per-call scratch only"""
+        lib().dlp_conv2d_fwd_enqueue_packed.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float,
+                                                        ctypes.c_void_p]
+        xs = (ctypes.c_int * 4)(*x.shape)
+        ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
+        _check(lib().dlp_conv2d_fwd_enqueue_packed(self._h, xs, _ptr(x), _ptr(w), _ptr(packed), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
+                                                   float(factor), _stream(stream)))
+
     def __del__(self):
         if getattr(self, "_h", None):
             lib().dlp_conv2d_fwd_destroy(self._h)

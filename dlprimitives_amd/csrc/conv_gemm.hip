@@ -2323,21 +2323,30 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     return p.wpack_bytes + split_workspace_bytes(p, a, g.groups, a.splitk);
 }
 
+namespace {
+__global__ __launch_bounds__(256) void clear_counters_kernel(int *p, int n)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n)
+        p[i] = 0;
+}
+} // namespace
+
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
-                           size_t part_bytes)
+                           size_t part_bytes, int mode)
 {
     if (p.wdirect && ((uintptr_t)w & 15) == 0)
         return DLP_OK; // conv_gemm_launch reads w in place
     int *zero = nullptr; // tile counters of the stream-K launch that follows
     int nzero = 0;
-    if (p.patch && part_ws != nullptr) {
+    if (mode != GEMM_PACK_ONLY && p.patch && part_ws != nullptr) {
         const PatchShape ps = patch_shape(g, p, (long long)g.B * g.OH * g.OW);
         if (part_bytes >= ps.ws_bytes && ps.tiles <= 0x7fffffffLL) {
             zero = (int *)part_ws;
             nzero = (int)ps.tiles;
         }
     }
-    if (!p.patch && !bf16_mfma_order(p.order) && part_ws != nullptr) { // counters of the in-place split-K reduction
+    if (mode != GEMM_PACK_ONLY && !p.patch && !bf16_mfma_order(p.order) && part_ws != nullptr) { // counters of the in-place split-K reduction
         GemmArgs a;
         a.N = g.B * g.OH * g.OW;
         a.Cout = g.Cout;
@@ -2347,6 +2356,14 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
             zero = (int *)part_ws;
             nzero = (int)((long long)a.mtiles * a.ntiles * g.groups);
         }
+    }
+    if (mode == GEMM_CLEAR_ONLY) { // the weights were packed earlier: only the counters of the coming launch
+        if (zero != nullptr) {
+            TimingScope ts("clear_counters", stream);
+            hipLaunchKernelGGL(clear_counters_kernel, dim3((unsigned)((nzero + 255) / 256)), dim3(256), 0, stream, zero, nzero);
+            DLP_HIP_TRY(hipGetLastError());
+        }
+        return DLP_OK;
     }
     const long long total = (long long)g.groups * p.mtiles * p.nkt * (bf16_mfma_order(p.order) ? BK2 : BK) * p.BM;
     if (total >= 0x7fffffffLL * 256)

@@ -491,14 +491,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 template <class T>
 int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, const Epilogue &ep,
-                 hipStream_t stream)
+                 hipStream_t stream, int mode)
 {
     float *U = (float *)ws;
-    {
+    if (mode != WINO_RUN_ONLY) {
         TimingScope ts("winograd_filter", stream);
         const int total = plan.Npad * plan.Cpad;
         hipLaunchKernelGGL(wino_filter_kernel<T>, dim3((total + 255) / 256), dim3(256), 0, stream, g.Cout, g.Cin, plan.Npad, plan.Cpad,
                            (const T *)w, U);
+    }
+    if (mode == WINO_FILTER_ONLY) {
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
     }
     WinoArgs a;
     a.U = U;
@@ -607,15 +611,15 @@ WinoPlan winograd_plan(const ConvGeom &g)
 }
 
 int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, size_t ws_bytes,
-                    const Epilogue &ep, hipStream_t stream)
+                    const Epilogue &ep, hipStream_t stream, int mode)
 {
     DLP_REQUIRE(winograd_supported(g), "geometry is not Winograd compatible");
     DLP_REQUIRE(ws != nullptr && ws_bytes >= plan.ws_bytes, "workspace smaller than workspace()");
-    if (g.B == 0)
+    if (g.B == 0 && mode != WINO_FILTER_ONLY)
         return DLP_OK;
     if (g.dtype == DLP_BFLOAT16)
-        return launch_typed<bf16_t>(g, plan, x, w, y, ws, ep, stream);
-    return launch_typed<float>(g, plan, x, w, y, ws, ep, stream);
+        return launch_typed<bf16_t>(g, plan, x, w, y, ws, ep, stream, mode);
+    return launch_typed<float>(g, plan, x, w, y, ws, ep, stream, mode);
 }
 
 } // namespace dlp

@@ -77,6 +77,7 @@ struct dlp_conv2d_fwd {
     KTabEntry *ktab; // device gather table of the GEMM stage
     WinoPlan wino;
     size_t workspace;
+    int packed_layout[6]; // of the last dlp_conv2d_fwd_pack: order, BM, K tiles, m tiles, patch, in-place
 };
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -279,6 +280,66 @@ int dlp_stream_destroy(void *stream)
     return DLP_OK;
 }
 
+// ---- HIP graphs: record what a stream is given once, replay it with one launch ----
+struct dlp_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+int dlp_graph_capture_begin(void *stream)
+{
+    DLP_REQUIRE(stream != nullptr, "capture needs a stream of its own (not the default stream)");
+    {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        DLP_REQUIRE(!g_timing_enabled, "per-kernel timing records events: switch it off before capturing");
+    }
+    // relaxed: other threads of the process (a framework's allocator) may keep calling the runtime meanwhile
+    DLP_HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed));
+    return DLP_OK;
+}
+
+int dlp_graph_capture_end(void *stream, dlp_graph **out)
+{
+    DLP_REQUIRE(stream != nullptr && out != nullptr, "null argument");
+    *out = nullptr;
+    hipGraph_t graph = nullptr;
+    DLP_HIP_TRY(hipStreamEndCapture((hipStream_t)stream, &graph));
+    if (!graph)
+        return fail(DLP_ERR_RUNTIME, "stream capture produced no graph");
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return fail(DLP_ERR_RUNTIME, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
+    }
+    dlp_graph *g = new (std::nothrow) dlp_graph();
+    if (!g) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    }
+    g->graph = graph;
+    g->exec = exec;
+    *out = g;
+    return DLP_OK;
+}
+
+int dlp_graph_launch(dlp_graph *g, void *stream)
+{
+    DLP_REQUIRE(g != nullptr, "null argument");
+    DLP_HIP_TRY(hipGraphLaunch(g->exec, (hipStream_t)stream));
+    return DLP_OK;
+}
+
+void dlp_graph_destroy(dlp_graph *g)
+{
+    if (!g)
+        return;
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    delete g;
+}
+
 int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], int out_shape[4])
 {
     return output_shape(cfg, in_shape, out_shape);
@@ -328,6 +389,8 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     op->algo = chosen;
     op->ktab = nullptr;
     op->workspace = 0;
+    for (int i = 0; i < 6; i++)
+        op->packed_layout[i] = -1;
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
@@ -399,6 +462,92 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
         if (rc != DLP_OK)
             return rc;
         return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0, w);
+    }
+    }
+}
+
+// ---- weights that stay constant between calls: transformed once into a buffer of the caller ----
+static void layout_of(const GemmPlan &p, int (&sig)[6])
+{
+    sig[0] = p.order;
+    sig[1] = p.BM;
+    sig[2] = p.nkt;
+    sig[3] = p.mtiles;
+    sig[4] = p.patch;
+    sig[5] = p.wdirect;
+}
+
+size_t dlp_conv2d_fwd_packed_bytes(const dlp_conv2d_fwd *op)
+{
+    if (!op)
+        return 0;
+    if (op->algo == ALGO_WINOGRAD)
+        return round256(op->wino.ws_bytes);
+    if (op->algo == ALGO_DEPTHWISE)
+        return 0;
+    ConvGeom g;
+    if (make_geom(op->cfg, op->cfg.shape, g) != DLP_OK)
+        return 0;
+    return round256(conv_gemm_plan(g, op->activation).wpack_bytes);
+}
+
+int dlp_conv2d_fwd_pack(dlp_conv2d_fwd *op, const void *w, void *packed, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && w != nullptr, "null argument");
+    if (op->algo == ALGO_DEPTHWISE)
+        return DLP_OK; // the kernel reads the filter as it is
+    DLP_REQUIRE(packed != nullptr, "null buffer for the packed weights");
+    ConvGeom g;
+    int rc = make_geom(op->cfg, op->cfg.shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    if (op->algo == ALGO_WINOGRAD) {
+        Epilogue ep = {nullptr, 0.0f, op->activation};
+        return winograd_launch(g, op->wino, nullptr, w, nullptr, packed, op->wino.ws_bytes, ep, (hipStream_t)stream, WINO_FILTER_ONLY);
+    }
+    const GemmPlan plan = conv_gemm_plan(g, op->activation);
+    layout_of(plan, op->packed_layout);
+    return conv_gemm_pack_weights(g, plan, w, packed, (hipStream_t)stream, nullptr, 0, GEMM_PACK_ONLY);
+}
+
+int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], const void *x, const void *w, const void *packed, const void *bias,
+                                  void *y, void *ws, size_t ws_bytes, float factor, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[0] >= 0, "negative batch");
+    DLP_REQUIRE(x_shape[1] == op->cfg.channels_in && x_shape[2] == op->cfg.shape[2] && x_shape[3] == op->cfg.shape[3],
+                "input shape differs from the shape given at create (only the batch may change)");
+    DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
+    ConvGeom g;
+    int rc = make_geom(op->cfg, x_shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    if (g.B == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && w != nullptr && y != nullptr, "null tensor pointer");
+    Epilogue ep;
+    ep.bias = (const float *)bias;
+    ep.factor = factor;
+    ep.activation = op->activation;
+    hipStream_t s = (hipStream_t)stream;
+    switch (op->algo) {
+    case ALGO_WINOGRAD:
+        DLP_REQUIRE(packed != nullptr, "null buffer of packed weights");
+        return winograd_launch(g, op->wino, x, w, y, const_cast<void *>(packed), op->wino.ws_bytes, ep, s, WINO_RUN_ONLY);
+    case ALGO_DEPTHWISE:
+        return depthwise_launch(g, x, w, y, ep, s);
+    default: {
+        const GemmPlan plan = conv_gemm_plan(g, op->activation);
+        int sig[6];
+        layout_of(plan, sig);
+        for (int i = 0; i < 6; i++)
+            DLP_REQUIRE(sig[i] == op->packed_layout[i], "the weights were packed for another tile plan (pack again for this batch)");
+        DLP_REQUIRE(packed != nullptr, "null buffer of packed weights");
+        void *part = ws_bytes > 0 ? ws : nullptr;
+        rc = conv_gemm_pack_weights(g, plan, w, const_cast<void *>(packed), s, part, ws_bytes, GEMM_CLEAR_ONLY);
+        if (rc != DLP_OK)
+            return rc;
+        return conv_gemm_launch(g, plan, op->ktab, x, packed, y, ep, s, -1, part, ws_bytes, w);
     }
     }
 }

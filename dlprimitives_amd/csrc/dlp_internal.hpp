@@ -171,8 +171,10 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation);
 // Repack [Cout][Cin/groups][KH][KW] weights into the tile order the kernel loads.
 // part_ws/part_bytes: the workspace behind the packed weights that conv_gemm_launch will be given
 // (the packing kernel clears the counters the launch keeps there).
+// mode: both steps, the packing alone (weights that stay constant are packed once), or the counters alone.
+enum { GEMM_PACK_AND_CLEAR = 0, GEMM_PACK_ONLY = 1, GEMM_CLEAR_ONLY = 2 };
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream,
-                           void *part_ws = nullptr, size_t part_bytes = 0);
+                           void *part_ws = nullptr, size_t part_bytes = 0, int mode = GEMM_PACK_AND_CLEAR);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 // part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.
 // w: the weight tensor as the caller gave it (plans with wdirect read it in place when it is 16-byte aligned).
@@ -194,8 +196,10 @@ struct WinoPlan {
 };
 bool winograd_supported(const ConvGeom &g);
 WinoPlan winograd_plan(const ConvGeom &g);
+// mode: filter transform and convolution, the transform alone (into ws), or the convolution on a ws transformed earlier
+enum { WINO_FILTER_AND_RUN = 0, WINO_FILTER_ONLY = 1, WINO_RUN_ONLY = 2 };
 int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, size_t ws_bytes,
-                    const Epilogue &ep, hipStream_t stream);
+                    const Epilogue &ep, hipStream_t stream, int mode = WINO_FILTER_AND_RUN);
 
 // ---- InnerProduct GEMM (ip_gemm.hip) ------------------------------------------
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype);

@@ -59,6 +59,14 @@ public:
     // y = factor != 0 ? factor * y + act(conv(x, w) + bias) : act(conv(x, w) + bias)
     // ws: uint8 tensor of at least workspace() bytes; asynchronous on e
     virtual void enqueue(Tensor &x, Tensor &w, Tensor *bias, Tensor &y, Tensor &ws, float factor, ExecutionContext const &e) = 0;
+    // Not in the reference: weights that stay constant between calls are transformed once into `packed`
+    // (uint8 tensor of packed_size() bytes, may be empty when that is 0) and enqueue_packed reads them
+    // from there; ws is then per-call scratch only (workspace() bytes are enough, operators that run
+    // one after another may share it).
+    virtual size_t packed_size() = 0;
+    virtual void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) = 0;
+    virtual void enqueue_packed(Tensor &x, Tensor &w, Tensor &packed, Tensor *bias, Tensor &y, Tensor &ws, float factor,
+                                ExecutionContext const &e) = 0;
     static std::unique_ptr<Conv2DForward> create(Context &ctx, Conv2DSettings const &config, bool bias,
                                                  StandardActivations activation = StandardActivations::identity,
                                                  std::string const &algo = std::string());
@@ -91,6 +99,23 @@ public:
         dlprim::details::check_status(dlp_conv2d_fwd_enqueue(op_, xs, x.device_ptr(), w.device_ptr(), bias ? bias->device_ptr() : nullptr,
                                                              y.device_ptr(), ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, factor,
                                                              e.stream()));
+    }
+
+    size_t packed_size() override { return dlp_conv2d_fwd_packed_bytes(op_); }
+    void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) override
+    {
+        dlprim::details::check_status(dlp_conv2d_fwd_pack(op_, w.device_ptr(), packed_size() ? packed.device_ptr() : nullptr, e.stream()));
+    }
+    void enqueue_packed(Tensor &x, Tensor &w, Tensor &packed, Tensor *bias, Tensor &y, Tensor &ws, float factor, ExecutionContext const &e) override
+    {
+        DLPRIM_CHECK(x.shape().size() == 4);
+        int xs[4];
+        for (int i = 0; i < 4; i++)
+            xs[i] = int(x.shape()[i]);
+        const size_t ws_bytes = workspace() ? ws.memory_size() : 0;
+        dlprim::details::check_status(dlp_conv2d_fwd_enqueue_packed(op_, xs, x.device_ptr(), w.device_ptr(), packed_size() ? packed.device_ptr() : nullptr,
+                                                                    bias ? bias->device_ptr() : nullptr, y.device_ptr(),
+                                                                    ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, factor, e.stream()));
     }
 
 private:

@@ -92,6 +92,9 @@ public:
     bool keep_intermediate_tensors() const { return keep_intermediate_; }
     // fold BatchNorm into the preceding convolution / inner product and merge activations (default on)
     void fuse(bool on) { fuse_ = on; }
+    // transform the convolution weights once, when the parameters go to the device (default on);
+    // off: every forward pass transforms them again, as the reference's operators do
+    void prepack(bool on) { prepack_ = on; }
 
     // shapes, rewrites, operators, memory; parameters are allocated (zero on the host) and wait for load_parameters
     void setup()
@@ -218,12 +221,47 @@ public:
         DLPRIM_CHECK(ready_);
         if (ctx_.is_cpu_context())
             throw NotImplementedError("Net::forward needs a device context");
-        for (auto &n : nodes_)
-            if (!n.skipped)
-                run(n, e);
+        if (graph_ && graph_stream_ == e.stream())
+            details::check_status(dlp_graph_launch(graph_.get(), e.stream()));
+        else
+            for (auto &n : nodes_)
+                if (!n.skipped)
+                    run(n, e);
         if (sync)
             e.finish();
     }
+
+    // Record one forward pass on e's stream as a HIP graph; later forward(e) calls replay it with a
+    // single launch (inputs, outputs and parameters stay where they are: refill them in place).  Not in
+    // the reference: for networks whose step is bound by launch overhead.  Parameters loaded after the
+    // capture need copy_parameters_to_device() only: the graph reads the same buffers.
+    void capture_forward(ExecutionContext const &e)
+    {
+        DLPRIM_CHECK(ready_);
+        release_graph();
+        forward(e, true); // first-use allocations happen here, not under capture
+        details::check_status(dlp_graph_capture_begin(e.stream()));
+        try {
+            for (auto &n : nodes_)
+                if (!n.skipped)
+                    run(n, e);
+        } catch (...) {
+            dlp_graph *broken = nullptr;
+            dlp_graph_capture_end(e.stream(), &broken);
+            dlp_graph_destroy(broken);
+            throw;
+        }
+        dlp_graph *g = nullptr;
+        details::check_status(dlp_graph_capture_end(e.stream(), &g));
+        graph_.reset(g, dlp_graph_destroy);
+        graph_stream_ = e.stream();
+    }
+    void release_graph()
+    {
+        graph_.reset();
+        graph_stream_ = nullptr;
+    }
+    bool has_graph() const { return bool(graph_); }
 
     // bytes of device memory behind the tensors (after planning) and operators that run (after the rewrites)
     size_t tensor_memory() const { return tensor_memory_; }
@@ -250,9 +288,11 @@ private:
         std::string algo;
         int ip_inputs = -1, ip_outputs = -1;
         Node *folded_bn = nullptr; // BatchNorm folded into this operator
+        bool is_packed = false;
         std::unique_ptr<core::Conv2DForward> conv_op;
         std::unique_ptr<core::IPForward> ip_op;
         Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
+        Tensor packed;       // the weights in the order the kernel loads them
         // BatchNorm
         float eps = 1e-5f;
         bool affine = true;
@@ -644,6 +684,13 @@ private:
             n.w_dev.to_device(e);
             n.b_dev.to_device(e);
         }
+        if (n.kind == k_conv && prepack_ && n.conv_op) {
+            const size_t bytes = n.conv_op->packed_size();
+            if (bytes > 0 && n.packed.shape().total_size() != bytes)
+                n.packed = Tensor(ctx_, Shape(bytes), uint8_data);
+            n.conv_op->pack(n.folded_bn ? n.w_dev : param(n.param_names[0]), n.packed, e);
+            n.is_packed = true;
+        }
     }
 
     void run(Node &n, ExecutionContext const &e)
@@ -654,7 +701,10 @@ private:
         case k_conv: {
             Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
-            n.conv_op->enqueue(x, w, b, y, workspace_, 0.0f, e);
+            if (n.is_packed)
+                n.conv_op->enqueue_packed(x, w, n.packed, b, y, workspace_, 0.0f, e);
+            else
+                n.conv_op->enqueue(x, w, b, y, workspace_, 0.0f, e);
             break;
         }
         case k_ip: {
@@ -693,7 +743,9 @@ private:
     std::map<std::string, Tensor> tensors_, params_;
     Tensor workspace_;
     size_t workspace_bytes_ = 0, tensor_memory_ = 0;
-    bool keep_intermediate_ = false, fuse_ = true, ready_ = false;
+    bool keep_intermediate_ = false, fuse_ = true, prepack_ = true, ready_ = false;
+    std::shared_ptr<dlp_graph> graph_;
+    void *graph_stream_ = nullptr;
 };
 
 } // namespace dlprim

@@ -84,6 +84,19 @@ int dlp_stream_create(void **stream);   /* ExecutionContext's in-order queue */
 int dlp_stream_sync(void *stream);      /* ExecutionContext::finish, context.hpp:216-220 */
 int dlp_stream_destroy(void *stream);
 
+/* ---- HIP graphs.  No counterpart in the reference (an OpenCL queue has no such thing); for callers whose
+ *      step is bound by launch overhead (small batches, many small layers).  Between begin and end every
+ *      enqueue on `stream` (a stream of its own, not the default one) is recorded instead of run; launch
+ *      replays the recording on a stream.  The recording holds the pointers it was given: tensors,
+ *      workspaces and operators must stay alive and in place.  Run one eager pass before capturing
+ *      (dlp_ip_fwd_enqueue allocates its scratch buffer on first use), keep per-kernel timing off, and
+ *      make no dlp_malloc / dlp_free / dlp_memcpy_* call on the capturing stream. -------------------- */
+typedef struct dlp_graph dlp_graph;
+int dlp_graph_capture_begin(void *stream);
+int dlp_graph_capture_end(void *stream, dlp_graph **out);
+int dlp_graph_launch(dlp_graph *graph, void *stream);
+void dlp_graph_destroy(dlp_graph *graph);
+
 /* ---- per-kernel timing: replaces ExecutionContext::enable_timing / TimingData
  *      (include/dlprim/context.hpp:23-94,180,237-243).  While enabled, every kernel
  *      launched by the calls below is bracketed by a HIP event pair on its stream and
@@ -119,6 +132,21 @@ size_t dlp_conv2d_fwd_workspace(const dlp_conv2d_fwd *op);
 int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4],
                            const void *x, const void *w, const void *bias, void *y,
                            void *ws, size_t ws_bytes, float factor, void *stream);
+
+/* Weights that stay constant between calls (inference).  No counterpart in the reference, whose enqueue
+ * takes the raw filter every time; dlp_conv2d_fwd_enqueue does the same and transforms the filter on
+ * every call.  Here the caller transforms it once: `packed` is a device buffer of
+ * dlp_conv2d_fwd_packed_bytes(op) bytes (0 for "depthwise_separable") that dlp_conv2d_fwd_pack fills
+ * (tile-ordered weights of "gemm", the transformed filter of "winograd") and that
+ * dlp_conv2d_fwd_enqueue_packed reads instead of transforming `w` again (`w` is still passed: 1x1
+ * bf16 convolutions read it in place).  `ws` then only holds the per-call scratch: workspace() bytes
+ * are always enough, and convolutions that run one after another on a stream may share it.  Pack
+ * again after the weights change. */
+size_t dlp_conv2d_fwd_packed_bytes(const dlp_conv2d_fwd *op);
+int dlp_conv2d_fwd_pack(dlp_conv2d_fwd *op, const void *w, void *packed, void *stream);
+int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], const void *x, const void *w,
+                                  const void *packed, const void *bias, void *y, void *ws, size_t ws_bytes,
+                                  float factor, void *stream);
 
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 

@@ -6,10 +6,11 @@
 //   net_forward plan <net.json> [keep] [nofuse]
 //       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
 //       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
-//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [resave=<file.dlpw>] [repeat=<n>]
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [resave=<file.dlpw>] [repeat=<n>]
 //       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
 //       network's input order), runs forward and writes the outputs (float32, in output order)
-//   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse]
+//   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse] [graph]
+//       (graph: the forward pass is recorded once as a HIP graph and replayed)
 //       random parameters and inputs, ms per forward pass on HIP device 0 (what the reference's
 //       tools/benchmark.cpp reports for its docs/nets_for_benchmark files)
 #include <dlprim/net.hpp>
@@ -21,6 +22,7 @@
 #include <iostream>
 #include <random>
 #include <sstream>
+#include <vector>
 
 namespace dp = dlprim;
 
@@ -44,7 +46,7 @@ int main(int argc, char **argv)
             std::cout << v.save() << std::endl;
             return 0;
         }
-        bool keep = false, fuse = true;
+        bool keep = false, fuse = true, graph = false, prepack = true;
         std::string resave;
         int repeat = 1, warmup = 5, iters = 20;
         const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
@@ -54,6 +56,10 @@ int main(int argc, char **argv)
                 keep = true;
             else if (a == "nofuse")
                 fuse = false;
+            else if (a == "graph")
+                graph = true;
+            else if (a == "nopack")
+                prepack = false;
             else if (a.compare(0, 7, "resave=") == 0)
                 resave = a.substr(7);
             else if (a.compare(0, 7, "repeat=") == 0)
@@ -70,6 +76,7 @@ int main(int argc, char **argv)
             dp::Net net(ctx);
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
+            net.prepack(prepack);
             net.load_from_json_file(argv[2]);
             net.setup();
             std::printf("operators %zu tensor_memory %zu\n", net.operators_run(), net.tensor_memory());
@@ -87,6 +94,7 @@ int main(int argc, char **argv)
             dp::Net net(ctx);
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
+            net.prepack(prepack);
             net.load_from_json_file(argv[2]);
             net.setup();
             std::mt19937 rng(1);
@@ -111,6 +119,8 @@ int main(int argc, char **argv)
                     v[j] = d(rng);
                 t.to_device(e);
             }
+            if (graph)
+                net.capture_forward(e);
             for (int i = 0; i < warmup; i++)
                 net.forward(e, false);
             e.finish();
@@ -130,6 +140,7 @@ int main(int argc, char **argv)
         dp::Net net(ctx);
         net.keep_intermediate_tensors(keep);
         net.fuse(fuse);
+        net.prepack(prepack);
         net.mode(dp::CalculationsMode::predict);
         net.load_from_json_file(argv[2]);
         net.setup();
@@ -146,6 +157,16 @@ int main(int argc, char **argv)
             if (!in)
                 throw dp::ValidationError("input file is too short");
             t.to_device(e);
+        }
+        if (graph) { // recorded with other input values than the ones that count: a replay must read the tensors anew
+            std::vector<float> keep_in(net.input(0).shape().total_size());
+            float *in0 = net.input(0).data<float>();
+            std::copy(in0, in0 + keep_in.size(), keep_in.begin());
+            std::fill(in0, in0 + keep_in.size(), 0.25f);
+            net.input(0).to_device(e);
+            net.capture_forward(e);
+            std::copy(keep_in.begin(), keep_in.end(), in0);
+            net.input(0).to_device(e);
         }
         for (int r = 0; r < repeat; r++) // later passes must give what the first one gave: shared chunks are rewritten
             net.forward(e, true);

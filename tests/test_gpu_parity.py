@@ -387,3 +387,55 @@ def test_inner_product_flattens_trailing_dims(gpu, oracle_mod):
     x = rng.uniform(-1, 1, (4, 8, 3, 3)).astype(np.float32)
     w = rng.standard_normal((10, 72)).astype(np.float32)
     np.testing.assert_allclose(gpu.run_ip(x, w, None), oracle_mod.ip_forward(x, w, None), **TOL)
+
+
+PACKED_CASES = [  # cin, cout, k, s, p, groups, hw, batch, algo, dtype
+    (64, 64, 3, 1, 1, 1, 28, 4, "gemm", "float32"),       # LDS-patch kernel, stream-K counters in the scratch
+    (64, 64, 3, 1, 1, 1, 28, 4, "winograd", "float32"),
+    (128, 256, 3, 2, 1, 1, 14, 8, "gemm", "float32"),     # split-K counters
+    (3, 64, 7, 2, 3, 1, 64, 2, "gemm", "float32"),
+    (48, 48, 3, 1, 1, 48, 20, 3, "", "float32"),          # depthwise: nothing to pack
+    (24, 40, 1, 1, 0, 2, 9, 2, "gemm", "float32"),
+    (64, 256, 1, 1, 0, 1, 28, 4, "gemm", "bfloat16"),     # weights read in place
+    (64, 64, 3, 1, 1, 1, 28, 4, "gemm", "bfloat16"),
+    (128, 128, 3, 2, 1, 1, 28, 4, "gemm", "bfloat16"),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", PACKED_CASES, ids=lambda c: "c%d_o%d_k%d_s%d_g%d_%s_%s" % (c[0], c[1], c[2], c[3], c[5], c[8] or "auto", c[9]))
+def test_gpu_packed_weights_give_the_same_bits(case):
+    """dlp_conv2d_fwd_pack + dlp_conv2d_fwd_enqueue_packed against dlp_conv2d_fwd_enqueue (which is checked against
+    the oracle above): same kernels on the same operands, so the outputs must be identical; the packed buffer is
+    reused by three calls, one with another batch, while the scratch is shared with a second operator."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    cin, cout, k, s, p, groups, hw, batch, algo, dtype = case
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    code = dlp.capi.FLOAT_DATA if dtype == "float32" else dlp.capi.BFLOAT16_DATA
+    torch.manual_seed(cin * 31 + cout)
+    st = dlp.Conv2DSettings(cin, cout, k, s, 1, p, groups, (batch, cin, hw, hw), dtype=code)
+    op = dlp.Conv2DForward.create(st, True, "relu", algo)
+    other = dlp.Conv2DForward.create(st, True, "relu", algo)
+    w = (torch.randn(cout, cin // groups, k, k, device="cuda:0") * 0.1).to(tdt)
+    bias = torch.randn(cout, device="cuda:0")
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+    assert op.packed_size() <= max(op.workspace(), 0) + 256
+    op.pack(w, packed)
+    for b in (batch, batch, max(batch // 2, 1)):
+        x = torch.randn(b, cin, hw, hw, device="cuda:0").to(tdt)
+        oshape = dlp.conv2d_output_shape(st, x.shape)
+        want = torch.empty(oshape, device="cuda:0", dtype=tdt)
+        other.enqueue(x, w, bias, want, ws)  # also scribbles over the shared scratch
+        got = torch.full(oshape, float("nan"), device="cuda:0", dtype=tdt)
+        op.enqueue_packed(x, w, packed, bias, got, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (b, float((got.float() - want.float()).abs().max()))
+        old = torch.randn(oshape, device="cuda:0").to(tdt)
+        got2, want2 = old.clone(), old.clone()
+        other.enqueue(x, w, bias, want2, ws, 0.5)
+        op.enqueue_packed(x, w, packed, bias, got2, ws, 0.5)
+        assert torch.equal(got2, want2)

@@ -7,7 +7,8 @@ docs/nets_for_benchmark/*.js.
 
 GPU: networks written in the reference's JSON + DLPW formats run through Net::forward and are compared
 with a float64 torch evaluation of the same operator list (BatchNorm unfused there), to 1e-4 of the
-output's largest magnitude; with and without the graph rewrites, with and without shared memory.
+output's largest magnitude; with and without the graph rewrites, with and without shared memory, and
+replayed three times from a HIP graph that was recorded with other input values.
 """
 import json
 import os
@@ -277,7 +278,8 @@ NETS = {
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("flags", [(), ("nofuse",), ("keep",), ("nofuse", "keep")], ids=["default", "nofuse", "keep", "nofuse_keep"])
+@pytest.mark.parametrize("flags", [(), ("nofuse",), ("keep",), ("nofuse", "keep"), ("graph",), ("graph", "nofuse")],
+                         ids=["default", "nofuse", "keep", "nofuse_keep", "graph", "graph_nofuse"])
 @pytest.mark.parametrize("net", list(NETS))
 def test_gpu_net_forward_matches_torch(tmp_path, net, flags):
     make, seed = NETS[net]
