@@ -223,6 +223,11 @@ class Conv2DForward:
         _check(lib().dlp_conv2d_fwd_enqueue(self._h, xs, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
                                             float(factor), _stream(stream)))
 
+    def accumulate_before_activation(self, on=True):
+        """y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)"""
+        lib().dlp_conv2d_fwd_set_accumulate_first.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        _check(lib().dlp_conv2d_fwd_set_accumulate_first(self._h, int(bool(on))))
+
     def packed_size(self):
         """bytes of the buffer that pack() fills (0: nothing to transform)"""
         lib().dlp_conv2d_fwd_packed_bytes.restype = ctypes.c_size_t

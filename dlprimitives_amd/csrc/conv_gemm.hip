@@ -87,6 +87,7 @@ struct GemmArgs {
     uint32_t hw4;     // H*W*sizeof(T): byte stride between input channels
     uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
     float factor;
+    int pre; // the old value of y is added before the activation (Epilogue::accumulate_first)
     int act;
     float clamp_lo, clamp_hi;
 };
@@ -488,7 +489,8 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
     // Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the tile's rows goes
     // through LDS (free after the last barrier) and the stores are buffer stores whose row offset
     // is scalar, instead of a bias load and 64-bit address arithmetic per value.
-    if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
+    const bool pre = sizeof(T) == 4 && a.pre != 0 && a.factor != 0.0f;
+    if ((a.factor == 0.0f || pre) && (a.M & 7) == 0 && a.y_bytes != 0) {
         float *bias_s = lds;
         if (tid < BM)
             bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
@@ -513,12 +515,14 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
 #pragma unroll
                     for (int rr = 0; rr < 4; rr++) {
                         float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        const uint32_t soff = (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * (int)sizeof(T));
+                        if (pre)
+                            v = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, voff, soff, 0)), a.factor, v);
                         if (ACT == ACT_CLAMP) {
                             if (clamp) // identity must keep NaNs: no min/max
                                 v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
                         } else
                             v = apply_act(v, a.act);
-                        const uint32_t soff = (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * (int)sizeof(T));
                         if (sizeof(T) == 4)
                             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
                         else
@@ -547,12 +551,14 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
                     float v = acc[i][j][r];
                     if (a.bias)
                         v += a.bias[g * a.M + m];
+                    if (pre)
+                        v = fmaf(to_float(yb[(size_t)m * a.OHW]), a.factor, v);
                     if (ACT == ACT_CLAMP) {
                         if (a.act != DLP_ACT_IDENTITY) // identity must keep NaNs: no min/max
                             v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
                     } else
                         v = apply_act(v, a.act);
-                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
+                    store_out(yb + (size_t)m * a.OHW, v, pre ? 0.0f : a.factor);
                 }
             }
         }
@@ -1747,14 +1753,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
         if (n >= a.N)
             break;
         float r = v[i] + bv;
+        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+        const int pix = n - b * a.OHW;
+        T *yp = (T *)a.y + ((size_t)b * a.Cout + row) * a.OHW + pix;
+        const bool pre = sizeof(T) == 4 && a.pre != 0 && a.factor != 0.0f;
+        if (pre)
+            r = fmaf(to_float(*yp), a.factor, r);
         if (ACT == ACT_CLAMP) {
             if (a.act != DLP_ACT_IDENTITY)
                 r = fminf(fmaxf(r, a.clamp_lo), a.clamp_hi);
         } else
             r = apply_act(r, a.act);
-        const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
-        const int pix = n - b * a.OHW;
-        store_out((T *)a.y + ((size_t)b * a.Cout + row) * a.OHW + pix, r, a.factor);
+        store_out(yp, r, pre ? 0.0f : a.factor);
     }
 }
 
@@ -2449,6 +2459,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     make_magic((uint32_t)a.OHW, a.ohw_magic, a.ohw_shift);
     make_magic((uint32_t)a.OW, a.ow_magic, a.ow_shift);
     a.factor = ep.factor;
+    a.pre = ep.accumulate_first;
     a.act = ep.activation;
     a.clamp_lo = -__builtin_huge_valf();
     a.clamp_hi = __builtin_huge_valf();

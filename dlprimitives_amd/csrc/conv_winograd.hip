@@ -59,6 +59,7 @@ struct WinoArgs {
     int stage_stride;        // staged variant: floats per channel of the staging buffer
     uint32_t ss_magic, ss_shift;
     float factor;
+    int pre; // the old value of y is added before the activation
     int act;
 };
 
@@ -455,15 +456,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     v[i] = o[i] + bv;
+                const int row = 2 * ty, col = 2 * tx;
+                T *yp = ybase + (((size_t)b * a.N + n) * a.H + row) * a.W + col;
+                const bool r1 = row + 1 < a.H, c1 = col + 1 < a.W; // odd H / W: the last tile is cut
+                const bool pre = a.pre != 0 && a.factor != 0.0f;
+                if (pre) {
+                    v[0] = fmaf(to_float(yp[0]), a.factor, v[0]);
+                    if (c1)
+                        v[1] = fmaf(to_float(yp[1]), a.factor, v[1]);
+                    if (r1) {
+                        v[2] = fmaf(to_float(yp[a.W]), a.factor, v[2]);
+                        if (c1)
+                            v[3] = fmaf(to_float(yp[a.W + 1]), a.factor, v[3]);
+                    }
+                }
                 if (a.act != DLP_ACT_IDENTITY) { // one uniform branch for the four values
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         v[i] = apply_act(v[i], a.act);
                 }
-                const int row = 2 * ty, col = 2 * tx;
-                T *yp = ybase + (((size_t)b * a.N + n) * a.H + row) * a.W + col;
-                const bool r1 = row + 1 < a.H, c1 = col + 1 < a.W; // odd H / W: the last tile is cut
-                if (a.factor != 0.0f) {
+                if (a.factor != 0.0f && !pre) {
                     store_out(yp, v[0], a.factor);
                     if (c1)
                         store_out(yp + 1, v[1], a.factor);
@@ -526,6 +538,7 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
     if (plan.stage_stride > 0)
         make_magic((uint32_t)plan.stage_stride, a.ss_magic, a.ss_shift);
     a.factor = ep.factor;
+    a.pre = ep.accumulate_first;
     a.act = ep.activation;
     const size_t x_img = (size_t)g.Cin * g.H * g.W, y_img = (size_t)g.Cout * g.H * g.W;
     for (int b0 = 0; b0 < g.B; b0 += plan.chunk_imgs) {

@@ -78,6 +78,7 @@ struct dlp_conv2d_fwd {
     WinoPlan wino;
     size_t workspace;
     int packed_layout[6]; // of the last dlp_conv2d_fwd_pack: order, BM, K tiles, m tiles, patch, in-place
+    int accumulate_first; // y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)
 };
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -391,6 +392,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     op->workspace = 0;
     for (int i = 0; i < 6; i++)
         op->packed_layout[i] = -1;
+    op->accumulate_first = 0;
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
@@ -446,6 +448,7 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
     ep.bias = (const float *)bias;
     ep.factor = factor;
     ep.activation = op->activation;
+    ep.accumulate_first = op->accumulate_first;
     hipStream_t s = (hipStream_t)stream;
     switch (op->algo) {
     case ALGO_WINOGRAD:
@@ -475,6 +478,15 @@ static void layout_of(const GemmPlan &p, int (&sig)[6])
     sig[3] = p.mtiles;
     sig[4] = p.patch;
     sig[5] = p.wdirect;
+}
+
+int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    if (on && (op->cfg.dtype != DLP_FLOAT || op->algo == ALGO_DEPTHWISE))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "accumulation before the activation: float_data, algorithms gemm and winograd");
+    op->accumulate_first = on ? 1 : 0;
+    return DLP_OK;
 }
 
 size_t dlp_conv2d_fwd_packed_bytes(const dlp_conv2d_fwd *op)
@@ -529,6 +541,7 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
     ep.bias = (const float *)bias;
     ep.factor = factor;
     ep.activation = op->activation;
+    ep.accumulate_first = op->accumulate_first;
     hipStream_t s = (hipStream_t)stream;
     switch (op->algo) {
     case ALGO_WINOGRAD:

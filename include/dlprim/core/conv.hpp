@@ -63,6 +63,9 @@ public:
     // (uint8 tensor of packed_size() bytes, may be empty when that is 0) and enqueue_packed reads them
     // from there; ws is then per-call scratch only (workspace() bytes are enough, operators that run
     // one after another may share it).
+    // Not in the reference: y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias), so that a
+    // residual sum whose other branch is already in y costs no pass of its own
+    virtual void accumulate_before_activation(bool on) = 0;
     virtual size_t packed_size() = 0;
     virtual void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) = 0;
     virtual void enqueue_packed(Tensor &x, Tensor &w, Tensor &packed, Tensor *bias, Tensor &y, Tensor &ws, float factor,
@@ -101,6 +104,7 @@ public:
                                                              e.stream()));
     }
 
+    void accumulate_before_activation(bool on) override { dlprim::details::check_status(dlp_conv2d_fwd_set_accumulate_first(op_, on ? 1 : 0)); }
     size_t packed_size() override { return dlp_conv2d_fwd_packed_bytes(op_); }
     void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) override
     {

@@ -288,6 +288,8 @@ private:
         std::string algo;
         int ip_inputs = -1, ip_outputs = -1;
         Node *folded_bn = nullptr; // BatchNorm folded into this operator
+        bool residual = false;     // a residual sum runs in this convolution's epilogue: inputs[1] is the other branch, the output lies over it
+        float residual_factor = 1.0f;
         bool is_packed = false;
         std::unique_ptr<core::Conv2DForward> conv_op;
         std::unique_ptr<core::IPForward> ip_op;
@@ -497,37 +499,96 @@ private:
     }
     bool is_net_output(std::string const &t) const { return std::find(output_names_.begin(), output_names_.end(), t) != output_names_.end(); }
 
+    int producer_before(size_t before, std::string const &t) const
+    {
+        for (size_t i = before; i-- > 0;) {
+            if (nodes_[i].skipped)
+                continue;
+            for (auto const &s : nodes_[i].outputs)
+                if (s == t)
+                    return int(i);
+        }
+        return -1;
+    }
+    bool is_net_input(std::string const &t) const { return std::find(input_names_.begin(), input_names_.end(), t) != input_names_.end(); }
+
+    // BatchNorm into the convolution / inner product that feeds only it
+    void try_fold_batch_norm(size_t i)
+    {
+        Node &p = nodes_[i];
+        if (!((p.kind == k_conv || p.kind == k_ip) && p.activation == StandardActivations::identity && !p.folded_bn && !p.residual))
+            return;
+        std::string const &t = p.outputs[0];
+        int u = next_user(i, t);
+        if (u >= 0 && nodes_[u].kind == k_bn && nodes_[u].inputs[0] == t && !is_net_output(t) &&
+            (nodes_[u].outputs[0] == t || readers_after(i, t) == 1)) {
+            Node &bn = nodes_[u];
+            p.folded_bn = &bn;
+            p.activation = bn.activation;
+            p.outputs[0] = bn.outputs[0];
+            bn.skipped = true;
+        }
+    }
+    // Activation into the fused slot of its producer
+    void try_merge_activation(size_t i)
+    {
+        Node &p = nodes_[i];
+        if (!((p.kind == k_conv || p.kind == k_ip || p.kind == k_eltwise || p.kind == k_bn) && p.activation == StandardActivations::identity))
+            return;
+        std::string const &t = p.outputs[0];
+        int u = next_user(i, t);
+        if (u >= 0 && nodes_[u].kind == k_act && nodes_[u].inputs[0] == t &&
+            (nodes_[u].outputs[0] == t || (!is_net_output(t) && readers_after(i, t) == 1))) {
+            Node &a = nodes_[u];
+            p.activation = a.activation;
+            p.outputs[0] = a.outputs[0];
+            a.skipped = true;
+        }
+    }
+    // A residual sum into the convolution that produces its later branch: the convolution then writes
+    // act(conv + bias + coef * other) over the other branch, which must be dead after the sum.
+    // Returns the index of that convolution, or -1.
+    int try_fuse_residual(size_t e)
+    {
+        Node &el = nodes_[e];
+        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || el.inputs[0] == el.inputs[1])
+            return -1;
+        const int p0 = producer_before(e, el.inputs[0]), p1 = producer_before(e, el.inputs[1]);
+        const int side = p0 > p1 ? 0 : 1; // the branch that is produced later
+        const int pi = side == 0 ? p0 : p1, ri = side == 0 ? p1 : p0;
+        if (pi < 0 || ri < 0)
+            return -1; // the other branch is a network input (never written over) or unknown
+        Node &p = nodes_[size_t(pi)];
+        std::string const a = el.inputs[size_t(side)], r = el.inputs[size_t(1 - side)];
+        if (p.kind != k_conv || p.conv.groups != 1 || p.activation != StandardActivations::identity || p.residual || el.coef[side] != 1.0f)
+            return -1;
+        if (is_net_output(a) || is_net_output(r) || is_net_input(r) || readers_after(size_t(pi), a) != 1 || next_user(e, r) >= 0)
+            return -1; // both branches must end in this sum
+        if (spec(a) != spec(r) || std::find(p.inputs.begin(), p.inputs.end(), r) != p.inputs.end())
+            return -1;
+        for (size_t i = size_t(pi) + 1; i < e; i++) // nothing between the convolution and the sum may still read the other branch
+            if (!nodes_[i].skipped && std::find(nodes_[i].inputs.begin(), nodes_[i].inputs.end(), r) != nodes_[i].inputs.end())
+                return -1;
+        p.residual = true;
+        p.residual_factor = el.coef[1 - side];
+        p.activation = el.activation;
+        p.outputs[0] = el.outputs[0];
+        p.inputs.push_back(r); // keeps the branch alive until the convolution has run
+        alias_of_[el.outputs[0]] = r;
+        el.skipped = true;
+        return pi;
+    }
+
     void rewrite_graph()
     {
         for (size_t i = 0; i < nodes_.size(); i++) {
-            Node &p = nodes_[i];
-            if (p.skipped)
+            if (nodes_[i].skipped)
                 continue;
-            // BatchNorm into the convolution / inner product that feeds only it
-            if ((p.kind == k_conv || p.kind == k_ip) && p.activation == StandardActivations::identity && !p.folded_bn) {
-                std::string const &t = p.outputs[0];
-                int u = next_user(i, t);
-                if (u >= 0 && nodes_[u].kind == k_bn && nodes_[u].inputs[0] == t && !is_net_output(t) &&
-                    (nodes_[u].outputs[0] == t || readers_after(i, t) == 1)) {
-                    Node &bn = nodes_[u];
-                    p.folded_bn = &bn;
-                    p.activation = bn.activation;
-                    p.outputs[0] = bn.outputs[0];
-                    bn.skipped = true;
-                }
-            }
-            // Activation into the fused slot of its producer
-            if ((p.kind == k_conv || p.kind == k_ip || p.kind == k_eltwise || p.kind == k_bn) && p.activation == StandardActivations::identity) {
-                std::string const &t = p.outputs[0];
-                int u = next_user(i, t);
-                if (u >= 0 && nodes_[u].kind == k_act && nodes_[u].inputs[0] == t &&
-                    (nodes_[u].outputs[0] == t || (!is_net_output(t) && readers_after(i, t) == 1))) {
-                    Node &a = nodes_[u];
-                    p.activation = a.activation;
-                    p.outputs[0] = a.outputs[0];
-                    a.skipped = true;
-                }
-            }
+            try_fold_batch_norm(i);
+            try_merge_activation(i);
+            const int p = try_fuse_residual(i);
+            if (p >= 0)
+                try_merge_activation(size_t(p));
         }
     }
 
@@ -544,6 +605,8 @@ private:
             case k_conv: {
                 core::Conv2DSettings cfg(n.conv, in, float_data);
                 n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
+                if (n.residual)
+                    n.conv_op->accumulate_before_activation(true);
                 workspace_bytes_ = std::max(workspace_bytes_, n.conv_op->workspace());
                 break;
             }
@@ -604,6 +667,16 @@ private:
             for (auto const &t : n.outputs) {
                 if (tensors_.count(t))
                     continue; // in place, or written before
+                auto al = alias_of_.find(t);
+                if (al != alias_of_.end()) { // written over the other branch of a residual sum: takes over its memory
+                    tensors_[t] = tensors_.at(al->second);
+                    auto h = held.find(al->second);
+                    if (h != held.end()) {
+                        held[t] = h->second;
+                        held.erase(h);
+                    }
+                    continue;
+                }
                 if (keep_intermediate_ || is_net_output(t)) {
                     own(t);
                     continue;
@@ -701,10 +774,11 @@ private:
         case k_conv: {
             Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
+            const float factor = n.residual ? n.residual_factor : 0.0f;
             if (n.is_packed)
-                n.conv_op->enqueue_packed(x, w, n.packed, b, y, workspace_, 0.0f, e);
+                n.conv_op->enqueue_packed(x, w, n.packed, b, y, workspace_, factor, e);
             else
-                n.conv_op->enqueue(x, w, b, y, workspace_, 0.0f, e);
+                n.conv_op->enqueue(x, w, b, y, workspace_, factor, e);
             break;
         }
         case k_ip: {
@@ -741,6 +815,7 @@ private:
     std::vector<std::string> input_names_, output_names_;
     std::map<std::string, Shape> specs_;
     std::map<std::string, Tensor> tensors_, params_;
+    std::map<std::string, std::string> alias_of_; // output of a fused residual sum -> the branch it is written over
     Tensor workspace_;
     size_t workspace_bytes_ = 0, tensor_memory_ = 0;
     bool keep_intermediate_ = false, fuse_ = true, prepack_ = true, ready_ = false;

@@ -148,6 +148,12 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
                                   const void *packed, const void *bias, void *y, void *ws, size_t ws_bytes,
                                   float factor, void *stream);
 
+/* Residual connections.  No counterpart in the reference, where the sum is an Elementwise operator of
+ * its own (src/ops/elementwise.cpp).  With `on`, enqueue computes y = act(conv + bias + factor * y)
+ * instead of y = factor * y + act(conv + bias): when y already holds the other branch of a residual
+ * block, factor 1 gives act(conv + bias + branch) in one pass.  float_data, "gemm" and "winograd". */
+int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
+
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
 /* ---- core::Conv2DBackwardData, include/dlprim/core/conv.hpp:60-68, src/core/conv.cpp:113-163,299-367,

@@ -439,3 +439,61 @@ def test_gpu_packed_weights_give_the_same_bits(case):
         other.enqueue(x, w, bias, want2, ws, 0.5)
         op.enqueue_packed(x, w, packed, bias, got2, ws, 0.5)
         assert torch.equal(got2, want2)
+
+
+RESIDUAL_CASES = [  # cin, cout, k, s, p, hw, batch, algo
+    (64, 64, 3, 1, 1, 28, 4, "gemm"),       # LDS-patch kernel
+    (64, 256, 1, 1, 0, 28, 4, "gemm"),      # buffer-store epilogue
+    (24, 37, 1, 1, 0, 9, 3, "gemm"),        # 37 filters: per-element epilogue
+    (256, 512, 3, 2, 1, 14, 8, "gemm"),     # split-K, reduced in place
+    (64, 64, 3, 1, 1, 28, 4, "winograd"),
+    (32, 48, 3, 1, 1, 13, 2, "winograd"),   # odd planes: cut tiles
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", RESIDUAL_CASES, ids=lambda c: "c%d_o%d_k%d_s%d_h%d_%s" % (c[0], c[1], c[2], c[3], c[5], c[7]))
+@pytest.mark.parametrize("activation,factor", [("relu", 1.0), ("tanh", 0.5), ("identity", -2.0)])
+def test_gpu_accumulate_before_activation(case, activation, factor):
+    """y = act(conv(x, w) + bias + factor * y): a residual sum in the convolution's epilogue, against torch in float64;
+    plain and packed enqueue; factor 0 must leave the usual result."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    cin, cout, k, s, p, hw, batch, algo = case
+    torch.manual_seed(cin + cout + k)
+    st = dlp.Conv2DSettings(cin, cout, k, s, 1, p, 1, (batch, cin, hw, hw))
+    op = dlp.Conv2DForward.create(st, True, activation, algo)
+    assert op.algo() == algo
+    op.accumulate_before_activation(True)
+    x = torch.randn(batch, cin, hw, hw, device="cuda:0")
+    w = torch.randn(cout, cin, k, k, device="cuda:0") * (2.0 / (cin * k * k)) ** 0.5
+    bias = torch.randn(cout, device="cuda:0")
+    conv = torch.nn.functional.conv2d(x.double().cpu(), w.double().cpu(), bias.double().cpu(), s, p)
+    old = torch.randn(conv.shape, device="cuda:0")
+    act = {"relu": torch.relu, "tanh": torch.tanh, "identity": lambda v: v}[activation]
+    want = act(conv + factor * old.double().cpu())
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    y = old.clone()
+    op.enqueue(x, w, bias, y, ws, factor)
+    err = float((y.double().cpu() - want).abs().max() / want.abs().max())
+    assert err < 1e-4, err
+    packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+    op.pack(w, packed)
+    y2 = old.clone()
+    op.enqueue_packed(x, w, packed, bias, y2, ws, factor)
+    assert torch.equal(y, y2)
+    y3 = torch.full(conv.shape, float("nan"), device="cuda:0")
+    op.enqueue(x, w, bias, y3, ws, 0.0)
+    err = float((y3.double().cpu() - act(conv)).abs().max() / act(conv).abs().max())
+    assert err < 1e-4, err
+
+
+def test_accumulate_before_activation_is_refused_where_not_built():
+    import dlprimitives_amd as dlp
+
+    dw = dlp.Conv2DForward.create(dlp.Conv2DSettings(16, 16, 3, 1, 1, 1, 16, (1, 16, 8, 8)), False, "relu", "depthwise_separable")
+    with pytest.raises(dlp.NotImplementedErrorDlprim):
+        dw.accumulate_before_activation(True)
+    dw.accumulate_before_activation(False)

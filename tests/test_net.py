@@ -111,8 +111,9 @@ def test_plan_resnet18_rewrites_and_memory(tmp_path):
     keep = parse_plan(tool("plan", p, "keep").stdout)
     n_ops = len(b.doc["operators"])
     assert plain["operators"] == n_ops == 20 + 20 + 9 + 1 + 8 + 1 + 1
-    # 20 BatchNorm folded, 9 Activation merged
-    assert fused["operators"] == 20 + 1 + 8 + 1 + 1
+    # 20 BatchNorm folded, 9 Activation merged, 8 residual sums run in the epilogue of a convolution
+    assert fused["operators"] == 20 + 1 + 1 + 1
+    assert keep["operators"] == 20 + 1 + 8 + 1 + 1  # separate tensors: the sums stay operators
     assert fused["tensors"] == {"loss": (4, 10)} == plain["tensors"]
     # every tensor in memory of its own: the sum over all tensors the fused graph produces
     names = {"data"}
@@ -169,9 +170,9 @@ def test_plan_rejects_bad_networks(tmp_path):
 @pytest.mark.parametrize(
     "name,ops_fused",
     [
-        ("resnet18-b16", 20 + 1 + 8 + 1 + 1),
-        ("resnet50-b16", 53 + 1 + 16 + 1 + 1),
-        ("mobilenet_v2-b16", 52 + 10 + 1 + 1),
+        ("resnet18-b16", 20 + 1 + 1 + 1),
+        ("resnet50-b16", 53 + 1 + 1 + 1),
+        ("mobilenet_v2-b16", 52 + 1 + 1),
         ("alexnet-b16", 5 + 4 + 3),
         ("vgg16-b16", 13 + 6 + 3),
     ],
@@ -264,8 +265,18 @@ def mixed_net():
     f = b.ip(q, "f0", 17, activation="relu")
     f = b.ip(f, "f1", 9, bias=False)
     f = b.bn(f, "f1n")  # folds into the inner product
+    # residual sums: one that moves into the epilogue of the later convolution (with a coefficient on the
+    # other branch and an activation of its own), one that cannot (the other branch is read again later)
+    ra = b.conv(q, "ra", 12, 3, 1, 1, bias=True)
+    rb = b.conv(ra, "rb", 12, 3, 1, 1, activation="relu")
+    rc = b.bn(b.conv(rb, "rc", 12, 1), "rcn")
+    rs = b.eltwise(ra, rc, "rs", "sum", coef1=0.5, activation="tanh")
+    rd = b.conv(rs, "rd", 12, 3, 1, 1, bias=True)
+    rt = b.eltwise(rd, rs, "rt", "sum")
+    ru = b.eltwise(rt, rs, "ru", "max")
     b.output("f1n")
     b.output("e3")
+    b.output("ru")
     return b
 
 
