@@ -22,6 +22,8 @@
 #pragma once
 #include <algorithm>
 #include <cmath>
+#include <cstdint>
+#include <cstring>
 #include <fstream>
 #include <map>
 #include <memory>
@@ -92,6 +94,54 @@ public:
     bool keep_intermediate_tensors() const { return keep_intermediate_; }
     // fold BatchNorm into the preceding convolution / inner product and merge activations (default on)
     void fuse(bool on) { fuse_ = on; }
+    // Storage type of the tensors between operators (inputs and outputs included) and of the convolution /
+    // inner-product weights on the device: float_data (as the reference) or bfloat16_data (16-bit elements,
+    // arithmetic in fp32, biases and BatchNorm coefficients stay fp32).  Set before setup().  Parameters on
+    // the host and in DLPW files are float either way; set_input / get_output convert.
+    void storage_type(DataType dt)
+    {
+        DLPRIM_CHECK(!ready_);
+        if (dt != float_data && dt != bfloat16_data)
+            throw NotImplementedError("Net storage types: float_data and bfloat16_data");
+        dtype_ = dt;
+    }
+    DataType storage_type() const { return dtype_; }
+    // float values into input `id` (converted to the storage type, copied to the device) / output `id` as floats
+    void set_input(unsigned id, float const *values, ExecutionContext const &e)
+    {
+        Tensor &t = input(id);
+        const size_t n = t.shape().total_size();
+        if (dtype_ == float_data)
+            std::copy(values, values + n, t.data<float>());
+        else
+            for (size_t i = 0; i < n; i++)
+                t.data<uint16_t>()[i] = to_bf16_bits(values[i]);
+        t.to_device(e);
+    }
+    void get_output(unsigned id, float *values, ExecutionContext const &e)
+    {
+        Tensor &t = output(id);
+        t.to_host(e);
+        e.finish();
+        const size_t n = t.shape().total_size();
+        if (dtype_ == float_data)
+            std::copy(t.data<float>(), t.data<float>() + n, values);
+        else
+            for (size_t i = 0; i < n; i++) {
+                const uint32_t bits = uint32_t(t.data<uint16_t>()[i]) << 16;
+                std::memcpy(values + i, &bits, 4);
+            }
+    }
+    // round to nearest even, NaN stays NaN
+    static uint16_t to_bf16_bits(float f)
+    {
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u)
+            return uint16_t((u >> 16) | 0x40);
+        return uint16_t((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+    }
+
     // transform the convolution weights once, when the parameters go to the device (default on);
     // off: every forward pass transforms them again, as the reference's operators do
     void prepack(bool on) { prepack_ = on; }
@@ -290,7 +340,7 @@ private:
         Node *folded_bn = nullptr; // BatchNorm folded into this operator
         bool residual = false;     // a residual sum runs in this convolution's epilogue: inputs[1] is the other branch, the output lies over it
         float residual_factor = 1.0f;
-        bool is_packed = false;
+        bool is_packed = false, use_w_dev = false;
         std::unique_ptr<core::Conv2DForward> conv_op;
         std::unique_ptr<core::IPForward> ip_op;
         Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
@@ -551,7 +601,7 @@ private:
     int try_fuse_residual(size_t e)
     {
         Node &el = nodes_[e];
-        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || el.inputs[0] == el.inputs[1])
+        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || dtype_ != float_data || el.inputs[0] == el.inputs[1])
             return -1;
         const int p0 = producer_before(e, el.inputs[0]), p1 = producer_before(e, el.inputs[1]);
         const int side = p0 > p1 ? 0 : 1; // the branch that is produced later
@@ -603,7 +653,7 @@ private:
             Shape const &in = spec(n.inputs[0]);
             switch (n.kind) {
             case k_conv: {
-                core::Conv2DSettings cfg(n.conv, in, float_data);
+                core::Conv2DSettings cfg(n.conv, in, dtype_);
                 n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
                 if (n.residual)
                     n.conv_op->accumulate_before_activation(true);
@@ -615,16 +665,17 @@ private:
                 cfg.inputs = n.ip_inputs;
                 cfg.outputs = n.ip_outputs;
                 cfg.optimal_batch_size = int(in[0]);
+                cfg.dtype = dtype_;
                 n.ip_op = core::IPForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation);
                 break;
             }
             case k_pool:
-                n.pool_op = n.max_mode ? core::Pooling2DForward::create_max_pooling(ctx_, n.kernel, n.pad, n.stride)
-                                       : core::Pooling2DForward::create_avg_pooling(ctx_, n.kernel, n.pad, n.stride, n.count_include_pad);
+                n.pool_op = n.max_mode ? core::Pooling2DForward::create_max_pooling(ctx_, n.kernel, n.pad, n.stride, dtype_)
+                                       : core::Pooling2DForward::create_avg_pooling(ctx_, n.kernel, n.pad, n.stride, n.count_include_pad, dtype_);
                 break;
             case k_gpool:
-                n.pool_op = n.max_mode ? core::Pooling2DForward::create_global_max_pooling(ctx_, in)
-                                       : core::Pooling2DForward::create_global_avg_pooling(ctx_, in);
+                n.pool_op = n.max_mode ? core::Pooling2DForward::create_global_max_pooling(ctx_, in, dtype_)
+                                       : core::Pooling2DForward::create_global_avg_pooling(ctx_, in, dtype_);
                 break;
             default: break;
             }
@@ -649,7 +700,7 @@ private:
         }
         tensor_memory_ = 0;
         auto own = [&](std::string const &name) {
-            tensors_[name] = Tensor(ctx_, spec(name));
+            tensors_[name] = Tensor(ctx_, spec(name), dtype_);
             tensor_memory_ += tensors_[name].memory_size();
         };
         for (auto const &name : input_names_)
@@ -681,7 +732,7 @@ private:
                     own(t);
                     continue;
                 }
-                const size_t bytes = spec(t).total_size() * sizeof(float);
+                const size_t bytes = spec(t).total_size() * size_t(size_of_data_type(dtype_));
                 int best = -1;
                 for (size_t c = 0; c < free_chunks.size(); c++)
                     if (free_chunks[c].bytes >= bytes && (best < 0 || free_chunks[c].bytes < free_chunks[size_t(best)].bytes))
@@ -695,7 +746,7 @@ private:
                     ch.bytes = bytes;
                     tensor_memory_ += bytes;
                 }
-                tensors_[t] = ch.mem.sub_tensor(0, spec(t), float_data);
+                tensors_[t] = ch.mem.sub_tensor(0, spec(t), dtype_);
                 held[t] = ch;
             }
             std::set<std::string> touched(n.inputs.begin(), n.inputs.end());
@@ -741,27 +792,41 @@ private:
             std::copy(shift.begin(), shift.end(), n.shift.data<float>());
             n.scale.to_device(e);
             n.shift.to_device(e);
-        } else if ((n.kind == k_conv || n.kind == k_ip) && n.folded_bn) {
-            std::vector<float> scale, shift;
-            bn_scale_shift(*n.folded_bn, scale, shift);
+        } else if (n.kind == k_conv || n.kind == k_ip) {
+            // the weights the kernel reads: the parameter itself, or a copy with the BatchNorm folded in
+            // and / or in the 16-bit storage type
             Tensor &w = param(n.param_names[0]);
-            const size_t cout = scale.size(), per = w.shape().total_size() / cout;
-            n.w_dev = Tensor(ctx_, w.shape());
-            n.b_dev = Tensor(ctx_, Shape(cout));
-            for (size_t c = 0; c < cout; c++) {
-                for (size_t i = 0; i < per; i++)
-                    n.w_dev.data<float>()[c * per + i] = w.data<float>()[c * per + i] * scale[c];
-                const float b = n.bias ? param(n.param_names[1]).data<float>()[c] : 0.0f;
-                n.b_dev.data<float>()[c] = shift[c] + b * scale[c];
+            const size_t total = w.shape().total_size();
+            n.use_w_dev = n.folded_bn != nullptr || dtype_ != float_data;
+            if (n.use_w_dev) {
+                std::vector<float> wf(w.data<float>(), w.data<float>() + total);
+                if (n.folded_bn) {
+                    std::vector<float> scale, shift;
+                    bn_scale_shift(*n.folded_bn, scale, shift);
+                    const size_t cout = scale.size(), per = total / cout;
+                    n.b_dev = Tensor(ctx_, Shape(cout));
+                    for (size_t c = 0; c < cout; c++) {
+                        for (size_t k = 0; k < per; k++)
+                            wf[c * per + k] *= scale[c];
+                        const float b = n.bias ? param(n.param_names[1]).data<float>()[c] : 0.0f;
+                        n.b_dev.data<float>()[c] = shift[c] + b * scale[c];
+                    }
+                    n.b_dev.to_device(e);
+                }
+                n.w_dev = Tensor(ctx_, w.shape(), dtype_);
+                if (dtype_ == float_data)
+                    std::copy(wf.begin(), wf.end(), n.w_dev.data<float>());
+                else
+                    for (size_t k = 0; k < total; k++)
+                        n.w_dev.data<uint16_t>()[k] = to_bf16_bits(wf[k]);
+                n.w_dev.to_device(e);
             }
-            n.w_dev.to_device(e);
-            n.b_dev.to_device(e);
         }
         if (n.kind == k_conv && prepack_ && n.conv_op) {
             const size_t bytes = n.conv_op->packed_size();
             if (bytes > 0 && n.packed.shape().total_size() != bytes)
                 n.packed = Tensor(ctx_, Shape(bytes), uint8_data);
-            n.conv_op->pack(n.folded_bn ? n.w_dev : param(n.param_names[0]), n.packed, e);
+            n.conv_op->pack(n.use_w_dev ? n.w_dev : param(n.param_names[0]), n.packed, e);
             n.is_packed = true;
         }
     }
@@ -772,7 +837,7 @@ private:
         Tensor &y = tensor(n.outputs[0]);
         switch (n.kind) {
         case k_conv: {
-            Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
+            Tensor &w = n.use_w_dev ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
             const float factor = n.residual ? n.residual_factor : 0.0f;
             if (n.is_packed)
@@ -782,28 +847,28 @@ private:
             break;
         }
         case k_ip: {
-            Tensor &w = n.folded_bn ? n.w_dev : param(n.param_names[0]);
+            Tensor &w = n.use_w_dev ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
             n.ip_op->enqueue(x, w, b, y, e);
             break;
         }
         case k_bn: {
             Shape const &s = x.shape();
-            details::check_status(dlp_channel_affine_fwd_enqueue(int(float_data), int(n.activation), int(s[0]), int(s[1]),
+            details::check_status(dlp_channel_affine_fwd_enqueue(int(dtype_), int(n.activation), int(s[0]), int(s[1]),
                                                                  int(s.total_size() / (s[0] * s[1])), x.device_ptr(),
                                                                  static_cast<const float *>(n.scale.device_ptr()),
                                                                  static_cast<const float *>(n.shift.device_ptr()), y.device_ptr(), e.stream()));
             break;
         }
         case k_act:
-            details::check_status(dlp_activation_fwd_enqueue(int(float_data), int(n.activation), x.shape().total_size(), x.device_ptr(), y.device_ptr(),
+            details::check_status(dlp_activation_fwd_enqueue(int(dtype_), int(n.activation), x.shape().total_size(), x.device_ptr(), y.device_ptr(),
                                                              e.stream()));
             break;
         case k_pool:
         case k_gpool: n.pool_op->enqueue(x, y, e); break;
         case k_eltwise: {
             Tensor &x1 = tensor(n.inputs[1]);
-            details::check_status(dlp_eltwise_fwd_enqueue(n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),
+            details::check_status(dlp_eltwise_fwd_enqueue_dtype(int(dtype_), n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),
                                                           x1.device_ptr(), y.device_ptr(), e.stream()));
             break;
         }
@@ -819,6 +884,7 @@ private:
     Tensor workspace_;
     size_t workspace_bytes_ = 0, tensor_memory_ = 0;
     bool keep_intermediate_ = false, fuse_ = true, prepack_ = true, ready_ = false;
+    DataType dtype_ = float_data;
     std::shared_ptr<dlp_graph> graph_;
     void *graph_stream_ = nullptr;
 };

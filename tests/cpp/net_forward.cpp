@@ -6,7 +6,8 @@
 //   net_forward plan <net.json> [keep] [nofuse]
 //       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
 //       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
-//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [resave=<file.dlpw>] [repeat=<n>]
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [resave=<file.dlpw>] [repeat=<n>]
+//       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32)
 //       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
 //       network's input order), runs forward and writes the outputs (float32, in output order)
 //   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse] [graph]
@@ -46,7 +47,7 @@ int main(int argc, char **argv)
             std::cout << v.save() << std::endl;
             return 0;
         }
-        bool keep = false, fuse = true, graph = false, prepack = true;
+        bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false;
         std::string resave;
         int repeat = 1, warmup = 5, iters = 20;
         const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
@@ -60,6 +61,8 @@ int main(int argc, char **argv)
                 graph = true;
             else if (a == "nopack")
                 prepack = false;
+            else if (a == "bf16")
+                bf16 = true;
             else if (a.compare(0, 7, "resave=") == 0)
                 resave = a.substr(7);
             else if (a.compare(0, 7, "repeat=") == 0)
@@ -77,6 +80,7 @@ int main(int argc, char **argv)
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
             net.prepack(prepack);
+            net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
             std::printf("operators %zu tensor_memory %zu\n", net.operators_run(), net.tensor_memory());
@@ -95,6 +99,7 @@ int main(int argc, char **argv)
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
             net.prepack(prepack);
+            net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
             std::mt19937 rng(1);
@@ -113,11 +118,10 @@ int main(int argc, char **argv)
             dp::ExecutionContext e = ctx.make_execution_context();
             std::uniform_real_distribution<float> d(-1.0f, 1.0f);
             for (unsigned i = 0; i < net.input_names().size(); i++) {
-                dp::Tensor &t = net.input(i);
-                float *v = t.data<float>();
-                for (size_t j = 0; j < t.shape().total_size(); j++)
-                    v[j] = d(rng);
-                t.to_device(e);
+                std::vector<float> v(net.input(i).shape().total_size());
+                for (float &f : v)
+                    f = d(rng);
+                net.set_input(i, v.data(), e);
             }
             if (graph)
                 net.capture_forward(e);
@@ -141,6 +145,7 @@ int main(int argc, char **argv)
         net.keep_intermediate_tensors(keep);
         net.fuse(fuse);
         net.prepack(prepack);
+        net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
         net.mode(dp::CalculationsMode::predict);
         net.load_from_json_file(argv[2]);
         net.setup();
@@ -151,30 +156,27 @@ int main(int argc, char **argv)
         std::ifstream in(argv[4], std::ios::binary);
         if (!in)
             throw dp::ValidationError(std::string("cannot open ") + argv[4]);
-        for (unsigned i = 0; i < net.input_names().size(); i++) {
-            dp::Tensor &t = net.input(i);
-            in.read(static_cast<char *>(t.host_data()), (std::streamsize)t.memory_size());
+        std::vector<std::vector<float>> inputs(net.input_names().size());
+        for (unsigned i = 0; i < inputs.size(); i++) {
+            inputs[i].resize(net.input(i).shape().total_size());
+            in.read(reinterpret_cast<char *>(inputs[i].data()), (std::streamsize)(inputs[i].size() * sizeof(float)));
             if (!in)
                 throw dp::ValidationError("input file is too short");
-            t.to_device(e);
+            net.set_input(i, inputs[i].data(), e);
         }
         if (graph) { // recorded with other input values than the ones that count: a replay must read the tensors anew
-            std::vector<float> keep_in(net.input(0).shape().total_size());
-            float *in0 = net.input(0).data<float>();
-            std::copy(in0, in0 + keep_in.size(), keep_in.begin());
-            std::fill(in0, in0 + keep_in.size(), 0.25f);
-            net.input(0).to_device(e);
+            std::vector<float> other(inputs[0].size(), 0.25f);
+            net.set_input(0, other.data(), e);
             net.capture_forward(e);
-            std::copy(keep_in.begin(), keep_in.end(), in0);
-            net.input(0).to_device(e);
+            net.set_input(0, inputs[0].data(), e);
         }
         for (int r = 0; r < repeat; r++) // later passes must give what the first one gave: shared chunks are rewritten
             net.forward(e, true);
         std::ofstream out(argv[5], std::ios::binary);
         for (unsigned i = 0; i < net.output_names().size(); i++) {
-            dp::Tensor &t = net.output(i);
-            t.to_host(e);
-            out.write(static_cast<char *>(t.host_data()), (std::streamsize)t.memory_size());
+            std::vector<float> v(net.output(i).shape().total_size());
+            net.get_output(i, v.data(), e);
+            out.write(reinterpret_cast<char *>(v.data()), (std::streamsize)(v.size() * sizeof(float)));
         }
         std::printf("operators %zu tensor_memory %zu\nok\n", net.operators_run(), net.tensor_memory());
         return 0;
