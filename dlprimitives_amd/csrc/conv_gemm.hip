@@ -489,8 +489,8 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
     // Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the tile's rows goes
     // through LDS (free after the last barrier) and the stores are buffer stores whose row offset
     // is scalar, instead of a bias load and 64-bit address arithmetic per value.
-    const bool pre = sizeof(T) == 4 && a.pre != 0 && a.factor != 0.0f;
-    if ((a.factor == 0.0f || pre) && (a.M & 7) == 0 && a.y_bytes != 0) {
+    const bool pre = a.pre != 0 && a.factor != 0.0f;
+    if ((a.factor == 0.0f || (pre && sizeof(T) == 4)) && (a.M & 7) == 0 && a.y_bytes != 0) {
         float *bias_s = lds;
         if (tid < BM)
             bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
@@ -983,7 +983,8 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
         if (tid < BM)
             bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
         __syncthreads();
-        const bool clamp = a.act != DLP_ACT_IDENTITY;
+        const bool pre = a.pre != 0 && a.factor != 0.0f; // the old y joins before the activation: in the second phase
+        const bool clamp = a.act != DLP_ACT_IDENTITY && !pre;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             unsigned char *col = smem + (wn * WTN + j * 32 + l32) * 2 + (wm * WTM + 4 * h) * PITCH;
@@ -998,7 +999,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         if (ACT == ACT_CLAMP) {
                             if (clamp)
                                 v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
-                        } else
+                        } else if (!pre)
                             v = apply_act(v, a.act);
                         *(uint16_t *)(col + (i * 32 + 8 * rq + rr) * PITCH) = to_bf16(v).bits;
                     }
@@ -1018,6 +1019,46 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                 const int pix = n - b * a.OHW;
                 const uint32_t voff = (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
                 const unsigned char *src = smem + row * PITCH + cp * (PXV * 2);
+                if (pre) { // y = act(staged value + factor * old y), the run read with one load of the store's width
+                    uint32_t mine[PXV / 2], old[PXV / 2];
+#pragma unroll
+                    for (int d = 0; d < PXV / 2; d++)
+                        mine[d] = ((const uint32_t *)src)[d];
+                    if constexpr (PXV == 8) {
+                        const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(yr, voff, 0, 0);
+                        old[0] = o[0], old[1] = o[1], old[2] = o[2], old[3] = o[3];
+                    } else if constexpr (PXV == 4) {
+                        const u32x2 o = __builtin_amdgcn_raw_buffer_load_b64(yr, voff, 0, 0);
+                        old[0] = o[0], old[1] = o[1];
+                    } else
+                        old[0] = __builtin_amdgcn_raw_buffer_load_b32(yr, voff, 0, 0);
+#pragma unroll
+                    for (int d = 0; d < PXV / 2; d++) {
+                        float lo = fmaf(__builtin_bit_cast(float, old[d] << 16), a.factor, __builtin_bit_cast(float, mine[d] << 16));
+                        float hi = fmaf(__builtin_bit_cast(float, old[d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[d] & 0xFFFF0000u));
+                        if (ACT == ACT_CLAMP) {
+                            if (a.act != DLP_ACT_IDENTITY) {
+                                lo = fminf(fmaxf(lo, a.clamp_lo), a.clamp_hi);
+                                hi = fminf(fmaxf(hi, a.clamp_lo), a.clamp_hi);
+                            }
+                        } else {
+                            lo = apply_act(lo, a.act);
+                            hi = apply_act(hi, a.act);
+                        }
+                        mine[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                    }
+                    if constexpr (PXV == 8) {
+                        u32x4 o;
+                        o[0] = mine[0], o[1] = mine[1], o[2] = mine[2], o[3] = mine[3];
+                        __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff, 0, 0);
+                    } else if constexpr (PXV == 4) {
+                        u32x2 o;
+                        o[0] = mine[0], o[1] = mine[1];
+                        __builtin_amdgcn_raw_buffer_store_b64(o, yr, voff, 0, 0);
+                    } else
+                        __builtin_amdgcn_raw_buffer_store_b32(mine[0], yr, voff, 0, 0);
+                    continue;
+                }
                 if constexpr (PXV == 8)
                     __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
                 else if constexpr (PXV == 4)
@@ -1087,12 +1128,15 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                     float v = acc[i][j][r];
                     if (a.bias)
                         v += a.bias[g * a.M + m];
+                    const bool pre = a.pre != 0 && a.factor != 0.0f;
+                    if (pre)
+                        v = fmaf(to_float(yb[(size_t)m * a.OHW]), a.factor, v);
                     if (ACT == ACT_CLAMP) {
                         if (a.act != DLP_ACT_IDENTITY)
                             v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
                     } else
                         v = apply_act(v, a.act);
-                    store_out(yb + (size_t)m * a.OHW, v, a.factor);
+                    store_out(yb + (size_t)m * a.OHW, v, pre ? 0.0f : a.factor);
                 }
             }
         }
@@ -1756,7 +1800,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
         const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
         const int pix = n - b * a.OHW;
         T *yp = (T *)a.y + ((size_t)b * a.Cout + row) * a.OHW + pix;
-        const bool pre = sizeof(T) == 4 && a.pre != 0 && a.factor != 0.0f;
+        const bool pre = a.pre != 0 && a.factor != 0.0f;
         if (pre)
             r = fmaf(to_float(*yp), a.factor, r);
         if (ACT == ACT_CLAMP) {
@@ -2490,7 +2534,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     a.pxv = 0;
     if (bf16_mfma_order(p.order)) {
         // wide output stores: runs of 8, 4 or 2 pixels that stay inside one image, dword aligned
-        if (ep.factor == 0.0f && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1)
+        if ((ep.factor == 0.0f || ep.accumulate_first) && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1)
             a.pxv = a.OHW % 8 == 0 ? 8 : a.OHW % 4 == 0 ? 4 : a.OHW % 2 == 0 ? 2 : 0;
         // dense loader (1x1, stride 1, no padding): runs of 8 or 4 input pixels, dword aligned
         if (p.patch_bf16 && ((uintptr_t)x & 3) == 0)

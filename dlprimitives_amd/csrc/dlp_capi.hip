@@ -483,8 +483,8 @@ static void layout_of(const GemmPlan &p, int (&sig)[6])
 int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on)
 {
     DLP_REQUIRE(op != nullptr, "null argument");
-    if (on && (op->cfg.dtype != DLP_FLOAT || op->algo == ALGO_DEPTHWISE))
-        return fail(DLP_ERR_NOT_IMPLEMENTED, "accumulation before the activation: float_data, algorithms gemm and winograd");
+    if (on && op->algo == ALGO_DEPTHWISE)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "accumulation before the activation: algorithms gemm and winograd");
     op->accumulate_first = on ? 1 : 0;
     return DLP_OK;
 }

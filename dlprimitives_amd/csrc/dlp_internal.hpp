@@ -49,7 +49,7 @@ struct ConvGeom {
 // Fused epilogue: v = act(acc + bias[c]); y = factor != 0 ? factor*y + v : v
 // (src/kernels/sgemm.cl:658-672,707-710 in the reference).
 // With accumulate_first the old value goes inside the activation: y = act(acc + bias[c] + factor*y)
-// (a residual connection whose other branch already sits in y); float_data only.
+// (a residual connection whose other branch already sits in y).
 struct Epilogue {
     const float *bias; // nullptr when the op was created without bias
     float factor;

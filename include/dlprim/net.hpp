@@ -601,7 +601,7 @@ private:
     int try_fuse_residual(size_t e)
     {
         Node &el = nodes_[e];
-        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || dtype_ != float_data || el.inputs[0] == el.inputs[1])
+        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || el.inputs[0] == el.inputs[1])
             return -1;
         const int p0 = producer_before(e, el.inputs[0]), p1 = producer_before(e, el.inputs[1]);
         const int side = p0 > p1 ? 0 : 1; // the branch that is produced later
@@ -611,6 +611,10 @@ private:
         Node &p = nodes_[size_t(pi)];
         std::string const a = el.inputs[size_t(side)], r = el.inputs[size_t(1 - side)];
         if (p.kind != k_conv || p.conv.groups != 1 || p.activation != StandardActivations::identity || p.residual || el.coef[side] != 1.0f)
+            return -1;
+        // 1x1 convolutions only: their epilogue is a large share of a short kernel and hides the extra reads;
+        // behind a 3x3 convolution (matrix-bound, epilogue exposed) the fused read cost what the sum saved
+        if (p.conv.kernel[0] != 1 || p.conv.kernel[1] != 1)
             return -1;
         if (is_net_output(a) || is_net_output(r) || is_net_input(r) || readers_after(size_t(pi), a) != 1 || next_user(e, r) >= 0)
             return -1; // both branches must end in this sum

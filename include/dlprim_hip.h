@@ -151,7 +151,7 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
 /* Residual connections.  No counterpart in the reference, where the sum is an Elementwise operator of
  * its own (src/ops/elementwise.cpp).  With `on`, enqueue computes y = act(conv + bias + factor * y)
  * instead of y = factor * y + act(conv + bias): when y already holds the other branch of a residual
- * block, factor 1 gives act(conv + bias + branch) in one pass.  float_data, "gemm" and "winograd". */
+ * block, factor 1 gives act(conv + bias + branch) in one pass.  "gemm" and "winograd". */
 int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
 
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);

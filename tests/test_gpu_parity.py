@@ -454,40 +454,44 @@ RESIDUAL_CASES = [  # cin, cout, k, s, p, hw, batch, algo
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", RESIDUAL_CASES, ids=lambda c: "c%d_o%d_k%d_s%d_h%d_%s" % (c[0], c[1], c[2], c[3], c[5], c[7]))
 @pytest.mark.parametrize("activation,factor", [("relu", 1.0), ("tanh", 0.5), ("identity", -2.0)])
-def test_gpu_accumulate_before_activation(case, activation, factor):
-    """y = act(conv(x, w) + bias + factor * y): a residual sum in the convolution's epilogue, against torch in float64;
-    plain and packed enqueue; factor 0 must leave the usual result."""
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_accumulate_before_activation(case, activation, factor, dtype):
+    """y = act(conv(x, w) + bias + factor * y): a residual sum in the convolution's epilogue, against torch in float64
+    (1e-4; bfloat16 tensors 2e-2: the sum is rounded once before and once after the old value joins, as it is when
+    the sum is an operator of its own); plain and packed enqueue; factor 0 must leave the usual result."""
     import torch
 
     import dlprimitives_amd as dlp
 
     cin, cout, k, s, p, hw, batch, algo = case
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    tol = 1e-4 if dtype == "float32" else 2e-2
     torch.manual_seed(cin + cout + k)
-    st = dlp.Conv2DSettings(cin, cout, k, s, 1, p, 1, (batch, cin, hw, hw))
+    st = dlp.Conv2DSettings(cin, cout, k, s, 1, p, 1, (batch, cin, hw, hw), dtype=dlp.capi.FLOAT_DATA if dtype == "float32" else dlp.capi.BFLOAT16_DATA)
     op = dlp.Conv2DForward.create(st, True, activation, algo)
     assert op.algo() == algo
     op.accumulate_before_activation(True)
-    x = torch.randn(batch, cin, hw, hw, device="cuda:0")
-    w = torch.randn(cout, cin, k, k, device="cuda:0") * (2.0 / (cin * k * k)) ** 0.5
+    x = torch.randn(batch, cin, hw, hw, device="cuda:0").to(tdt)
+    w = (torch.randn(cout, cin, k, k, device="cuda:0") * (2.0 / (cin * k * k)) ** 0.5).to(tdt)
     bias = torch.randn(cout, device="cuda:0")
     conv = torch.nn.functional.conv2d(x.double().cpu(), w.double().cpu(), bias.double().cpu(), s, p)
-    old = torch.randn(conv.shape, device="cuda:0")
+    old = torch.randn(conv.shape, device="cuda:0").to(tdt)
     act = {"relu": torch.relu, "tanh": torch.tanh, "identity": lambda v: v}[activation]
     want = act(conv + factor * old.double().cpu())
     ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
     y = old.clone()
     op.enqueue(x, w, bias, y, ws, factor)
     err = float((y.double().cpu() - want).abs().max() / want.abs().max())
-    assert err < 1e-4, err
+    assert err < tol, err
     packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
     op.pack(w, packed)
     y2 = old.clone()
     op.enqueue_packed(x, w, packed, bias, y2, ws, factor)
     assert torch.equal(y, y2)
-    y3 = torch.full(conv.shape, float("nan"), device="cuda:0")
+    y3 = torch.full(conv.shape, float("nan"), device="cuda:0", dtype=tdt)
     op.enqueue(x, w, bias, y3, ws, 0.0)
     err = float((y3.double().cpu() - act(conv)).abs().max() / act(conv).abs().max())
-    assert err < 1e-4, err
+    assert err < tol, err
 
 
 def test_accumulate_before_activation_is_refused_where_not_built():

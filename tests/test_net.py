@@ -111,8 +111,8 @@ def test_plan_resnet18_rewrites_and_memory(tmp_path):
     keep = parse_plan(tool("plan", p, "keep").stdout)
     n_ops = len(b.doc["operators"])
     assert plain["operators"] == n_ops == 20 + 20 + 9 + 1 + 8 + 1 + 1
-    # 20 BatchNorm folded, 9 Activation merged, 8 residual sums run in the epilogue of a convolution
-    assert fused["operators"] == 20 + 1 + 1 + 1
+    # 20 BatchNorm folded, 9 Activation merged, the 3 residual sums behind a 1x1 convolution run in its epilogue
+    assert fused["operators"] == 20 + 1 + 5 + 1 + 1
     assert keep["operators"] == 20 + 1 + 8 + 1 + 1  # separate tensors: the sums stay operators
     assert fused["tensors"] == {"loss": (4, 10)} == plain["tensors"]
     # every tensor in memory of its own: the sum over all tensors the fused graph produces
@@ -170,7 +170,7 @@ def test_plan_rejects_bad_networks(tmp_path):
 @pytest.mark.parametrize(
     "name,ops_fused",
     [
-        ("resnet18-b16", 20 + 1 + 1 + 1),
+        ("resnet18-b16", 20 + 1 + 5 + 1 + 1),
         ("resnet50-b16", 53 + 1 + 1 + 1),
         ("mobilenet_v2-b16", 52 + 1 + 1),
         ("alexnet-b16", 5 + 4 + 3),
