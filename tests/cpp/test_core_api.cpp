@@ -216,6 +216,61 @@ static void conv_backward_case(dp::Context &ctx, dp::ExecutionContext &q, int B,
     EXPECT(ex < 1e-4 && ew < 1e-4 && eb < 1e-4);
 }
 
+// Inner-product gradients as InnerProduct::backward calls them (src/ops/inner_product.cpp:186-240), against the definition in double.
+static void ip_backward_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int in, int out, float factor)
+{
+    dp::core::IPSettings cfg;
+    cfg.inputs = in;
+    cfg.outputs = out;
+    cfg.optimal_batch_size = B;
+    std::unique_ptr<dp::core::IPBackwardData> bd = dp::core::IPBackwardData::create(ctx, cfg);
+    std::unique_ptr<dp::core::IPBackwardFilter> bf = dp::core::IPBackwardFilter::create(ctx, cfg);
+    dp::Tensor X(ctx, dp::Shape(B, in)), W(ctx, dp::Shape(out, in)), dY(ctx, dp::Shape(B, out)), dX(ctx, dp::Shape(B, in)), dW(ctx, dp::Shape(out, in));
+    std::mt19937 rng(in * 3 + out);
+    fill(X, rng, -1, 1);
+    fill(W, rng, -0.3f, 0.3f);
+    fill(dY, rng, -1, 1);
+    fill(dX, rng, -1, 1);
+    fill(dW, rng, -1, 1);
+    std::vector<double> want_dx(size_t(B) * in), want_dw(size_t(out) * in);
+    for (size_t i = 0; i < want_dx.size(); i++)
+        want_dx[i] = double(factor) * dX.data<float>()[i];
+    for (size_t i = 0; i < want_dw.size(); i++)
+        want_dw[i] = double(factor) * dW.data<float>()[i];
+    for (int b = 0; b < B; b++)
+        for (int o = 0; o < out; o++) {
+            const double g = dY.data<float>()[size_t(b) * out + o];
+            for (int i = 0; i < in; i++) {
+                want_dx[size_t(b) * in + i] += g * W.data<float>()[size_t(o) * in + i];
+                want_dw[size_t(o) * in + i] += g * X.data<float>()[size_t(b) * in + i];
+            }
+        }
+    for (dp::Tensor *t : {&X, &W, &dY, &dX, &dW})
+        t->to_device(q);
+    for (int rep = 0; rep < 2; rep++) { // the second call reuses the operator's workspace
+        if (rep == 1) {
+            dX.to_device(q);
+            dW.to_device(q);
+        }
+        bf->enqueue(X, dW, dY, factor, q);
+        bd->enqueue(dX, W, dY, factor, q);
+    }
+    dX.to_host(q);
+    dW.to_host(q);
+    q.finish();
+    double sx = 1e-6, sw = 1e-6, ex = 0, ew = 0;
+    for (double v : want_dx)
+        sx = std::max(sx, std::fabs(v));
+    for (double v : want_dw)
+        sw = std::max(sw, std::fabs(v));
+    for (size_t i = 0; i < want_dx.size(); i++)
+        ex = std::max(ex, std::fabs(want_dx[i] - dX.data<float>()[i]) / sx);
+    for (size_t i = 0; i < want_dw.size(); i++)
+        ew = std::max(ew, std::fabs(want_dw[i] - dW.data<float>()[i]) / sw);
+    std::printf("ip backward b%d %d->%d factor %.2f : max err dx %.2e dw %.2e\n", B, in, out, factor, ex, ew);
+    EXPECT(ex < 1e-4 && ew < 1e-4);
+}
+
 static void ip_case(dp::Context &ctx, dp::ExecutionContext &q, int B, int in, int out)
 {
     dp::core::IPSettings cfg;
@@ -320,6 +375,9 @@ int main(int argc, char **argv)
             conv_backward_case(ctx, q, 2, 24, 24, 9, 3, 1, 1, 24, 1.0f);
             conv_backward_case(ctx, q, 2, 3, 8, 20, 7, 2, 3, 1, 0.0f);
             ip_case(ctx, q, 5, 64, 10);
+            ip_backward_case(ctx, q, 5, 64, 10, 0.0f);
+            ip_backward_case(ctx, q, 70, 33, 129, 0.5f);
+            ip_backward_case(ctx, q, 1, 512, 1000, 1.0f);
             pool_case(ctx, q);
             // sub-tensor views share memory: run on the second image of a batch-2 tensor
             dp::Tensor big(ctx, dp::Shape(2, 4, 6, 6));
