@@ -335,6 +335,76 @@ def test_gpu_net_forward_matches_torch(tmp_path, net, flags):
         np.testing.assert_array_equal(again[k].reshape(-1), params[k].reshape(-1))
 
 
+def random_net(seed):
+    """A random graph over one spatial size: convolutions (1x1 / 3x3, with and without bias / activation), BatchNorm,
+    activations in place and not, element-wise operations between any two tensors made so far, now and then a
+    pooling that starts a new size.  Tensors are read again long after they were made, which is what the memory
+    plan, the BatchNorm folding and the residual rewrite have to get right."""
+    rng = np.random.default_rng(seed)
+    c = int(rng.choice([4, 8, 12]))
+    b = netfile.NetBuilder("data", (2, c, 12, 10))
+    live = ["data"]  # tensors of the current shape
+    made = 0
+    for step in range(int(rng.integers(8, 16))):
+        kind = rng.choice(["conv", "conv", "conv", "bn", "act", "elt", "elt", "pool"])
+        src = live[-1] if rng.random() < 0.65 else str(rng.choice(live))
+        made += 1
+        name = "t%d" % made
+        if kind == "conv":
+            k = int(rng.choice([1, 1, 3]))
+            act = str(rng.choice(["", "", "relu", "tanh"]))
+            b.conv(src, name, c, k, 1, k // 2, bias=bool(rng.integers(2)), activation=act or None)
+        elif kind == "bn":
+            b.bn(src, name, affine=bool(rng.integers(4)), activation=str(rng.choice(["", "relu"])) or None)
+        elif kind == "act":
+            if rng.integers(2) and src != "data":
+                b.act(src, str(rng.choice(["relu", "sigmoid"])))  # in place
+                continue
+            b.act(src, str(rng.choice(["relu", "relu6"])), dst=name)
+        elif kind == "elt":
+            other = str(rng.choice(live))
+            if other == src:
+                continue
+            op = str(rng.choice(["sum", "sum", "sum", "prod", "max"]))
+            coefs = [(None, None), (None, 0.5), (2.0, None)][int(rng.integers(3))]
+            b.eltwise(src, other, name, op, coef1=coefs[0], coef2=coefs[1], activation=str(rng.choice(["", "relu"])) or None)
+        else:
+            if b.shapes[src][2] < 6:
+                continue
+            b.pool(src, name, str(rng.choice(["max", "avg"])), 2, 2)
+            live = []
+        live.append(name)
+    b.output(live[-1])
+    if len(live) > 2 and live[0] != "data":
+        b.output(live[0])
+    return b
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(40))
+def test_gpu_net_random_graphs(tmp_path, seed):
+    b = random_net(seed)
+    p = write_net(tmp_path, b)
+    params = b.random_parameters(seed)
+    netfile.save_dlpw(tmp_path / "w.dlpw", params)
+    rng = np.random.default_rng(seed + 500)
+    x = rng.uniform(-1, 1, b.doc["inputs"][0]["shape"]).astype(np.float32)
+    x.tofile(tmp_path / "in.bin")
+    want = torch_forward(b.doc, params, {"data": x})
+    results = {}
+    for flags in ((), ("nofuse", "keep")):
+        tool("run", p, tmp_path / "w.dlpw", tmp_path / "in.bin", tmp_path / "out.bin", "repeat=2", *flags)
+        got = np.fromfile(tmp_path / "out.bin", dtype=np.float32)
+        off = 0
+        for name, w in zip(b.doc["outputs"], want):
+            g = got[off : off + w.size].reshape(w.shape)
+            off += w.size
+            scale = max(np.abs(w).max(), 1e-3)
+            err = np.abs(g - w).max() / scale
+            assert err < 1e-4, (seed, flags, name, err, json.dumps(b.doc["operators"]))
+        results[flags] = got
+
+
 @pytest.mark.gpu
 def test_gpu_net_missing_parameter_is_an_error(tmp_path):
     b = netfile.resnet18(1, 32, 4)
