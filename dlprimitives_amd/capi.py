@@ -72,6 +72,11 @@ def lib():
         if not os.path.exists(_LIB):
             raise DlprimError(
                 "libdlprim_hip.so is not built (%s); run `make -C dlprimitives_amd/csrc` -- there is no CPU fallback" % _LIB)
+        # This binding works on torch tensors, and torch ships a HIP runtime of its own: it has to be the one
+        # the process loads first.  With the library (and the system's runtime behind it) loaded before torch,
+        # torch's own initialisation afterwards reports "No HIP GPUs are available".
+        import torch  # noqa: F401
+
         L = ctypes.CDLL(_LIB)
         L.dlp_last_error.restype = ctypes.c_char_p
         L.dlp_conv2d_fwd_algo.restype = ctypes.c_char_p

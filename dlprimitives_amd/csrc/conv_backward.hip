@@ -51,8 +51,9 @@ struct WgradArgs {
 
 // dW tile of BM filters x BN (channel, tap) columns over the chunks of one slice.
 // AVEC: OH * OW is a multiple of 4, dy rows are read 16 bytes per lane.
-// MASKED: KH * KW <= 31, the padding test of a gathered element is one bit of a per-lane tap mask.
-template <int BM, int BN, bool AVEC, bool MASKED>
+// MASKED: the padding test of a gathered element is one bit of a per-lane tap mask: 1 = KH * KW <= 31 (one word),
+// 2 = KH * KW <= 63 (two words); 0 = row and column comparisons per element.
+template <int BM, int BN, bool AVEC, int MASKED>
 __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 MFMA blocks per wavefront (wavefronts 2 x 2)
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
         const int dr = r * a.dh - a.ph, ds = s * a.dw - a.pw;
         const bool nv = n < a.Ncol;
         rowtab[tid * 4 + 0] = nv ? ((int)c * a.H + dr) * a.W + ds : 0;
-        rowtab[tid * 4 + 1] = nv ? rs : 31; // bit 31 of a tap mask is never set
+        rowtab[tid * 4 + 1] = nv ? rs : (MASKED == 2 ? 63 : 31); // the last bit of a tap mask is never set
         rowtab[tid * 4 + 2] = nv ? dr : -(1 << 28); // far outside the image for the comparing path
         rowtab[tid * 4 + 3] = ds;
     }
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
             const int ow = pix - oh * a.OW;
             const int ohs = oh * a.sh, ows = ow * a.sw;
             const int xbase = (b * a.Cin + g * a.Cin_g) * a.H * a.W + ohs * a.W + ows;
-            if (MASKED) {
+            if (MASKED == 1) {
                 uint32_t cols = 0, taps = 0;
                 for (int s = 0; s < a.KW; s++)
                     cols |= ((unsigned)(ows + s * a.dw - a.pw) < (unsigned)a.W ? 1u : 0u) << s;
@@ -123,6 +124,21 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
                 for (int i = 0; i < RB; i++) {
                     const int2 rt = *reinterpret_cast<const int2 *>(&rowtab[(brow + 8 * i) * 4]);
                     const uint32_t off = ((uint32_t)(xbase + rt.x) << 2) | (((bad >> rt.y) & 1u) << 31);
+                    rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+                }
+            } else if (MASKED == 2) {
+                uint64_t cols = 0, taps = 0;
+                for (int s = 0; s < a.KW; s++)
+                    cols |= (uint64_t)((unsigned)(ows + s * a.dw - a.pw) < (unsigned)a.W ? 1u : 0u) << s;
+                for (int r = 0; r < a.KH; r++)
+                    taps |= ((unsigned)(ohs + r * a.dh - a.ph) < (unsigned)a.H ? cols : 0ull) << (r * a.KW);
+                const uint64_t bad = pv ? ~taps : ~0ull;
+                const uint32_t bad_lo = (uint32_t)bad, bad_hi = (uint32_t)(bad >> 32);
+#pragma unroll
+                for (int i = 0; i < RB; i++) {
+                    const int2 rt = *reinterpret_cast<const int2 *>(&rowtab[(brow + 8 * i) * 4]);
+                    const uint32_t word = (rt.y & 32) ? bad_hi : bad_lo;
+                    const uint32_t off = ((uint32_t)(xbase + rt.x) << 2) | (((word >> (rt.y & 31)) & 1u) << 31);
                     rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
                 }
             } else {
@@ -832,17 +848,23 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
         TimingScope ts("wgrad", st);
         const dim3 grid((unsigned)wgs), block(256);
         const bool avec = a.OHW % 4 == 0 && ((uintptr_t)dy & 15) == 0;
-        const bool masked = a.KH * a.KW <= 31;
+        const int taps = a.KH * a.KW;
+        const int masked = taps <= 31 ? 1 : taps <= 63 ? 2 : 0;
+#define DLP_WGRAD_LAUNCH_M(BM_, BN_, AV_)                                                                      \
+    do {                                                                                                       \
+        if (masked == 1)                                                                                       \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, AV_, 1>), grid, block, 0, st, a);              \
+        else if (masked == 2)                                                                                  \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, AV_, 2>), grid, block, 0, st, a);              \
+        else                                                                                                   \
+            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, AV_, 0>), grid, block, 0, st, a);              \
+    } while (0)
 #define DLP_WGRAD_LAUNCH(BM_, BN_)                                                                             \
     do {                                                                                                       \
-        if (avec && masked)                                                                                    \
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, true, true>), grid, block, 0, st, a);          \
-        else if (avec)                                                                                         \
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, true, false>), grid, block, 0, st, a);         \
-        else if (masked)                                                                                       \
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, false, true>), grid, block, 0, st, a);         \
+        if (avec)                                                                                              \
+            DLP_WGRAD_LAUNCH_M(BM_, BN_, true);                                                                \
         else                                                                                                   \
-            hipLaunchKernelGGL((conv_wgrad_f32_kernel<BM_, BN_, false, false>), grid, block, 0, st, a);        \
+            DLP_WGRAD_LAUNCH_M(BM_, BN_, false);                                                               \
     } while (0)
         if (p.BM == 128 && p.BN == 128)
             DLP_WGRAD_LAUNCH(128, 128);
@@ -853,6 +875,7 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
         else
             DLP_WGRAD_LAUNCH(64, 64);
 #undef DLP_WGRAD_LAUNCH
+#undef DLP_WGRAD_LAUNCH_M
     }
     if (p.slices > 1) {
         TimingScope ts("wgrad_reduce", st);
