@@ -436,6 +436,8 @@ WgradPlan wgrad_plan(const dlp_conv2d_settings &c, int batch, int OH, int OW)
     }
     p.BM = cout_g > 64 ? 128 : 64;
     p.BN = ncol > 64 ? 128 : 64;
+    if (p.BN == 128 && (ncol + 63) / 64 * 64 * 5 <= (ncol + 127) / 128 * 128 * 4)
+        p.BN = 64; // the narrower tile wastes at least a fifth less of its columns on padding (conv1: 147 columns)
     p.mtiles = (cout_g + p.BM - 1) / p.BM;
     p.ntiles = (ncol + p.BN - 1) / p.BN;
     p.chunks = (int)(((long long)batch * OH * OW + KC - 1) / KC);
