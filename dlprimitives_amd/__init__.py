@@ -27,6 +27,7 @@ from .capi import (  # noqa: F401
     lib,
     library_path,
     pool2d_output_size,
+    softmax_forward,
     timing_count,
     timing_enable,
     timing_records,

@@ -448,3 +448,14 @@ def channel_affine_forward(x, scale, shift, y, activation="identity", stream=Non
                                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     _check(lib().dlp_channel_affine_fwd_enqueue(torch_dtype_code(x), _act(activation), batch, channels, plane, _ptr(x), _ptr(scale), _ptr(shift),
                                                 _ptr(y), _stream(stream)))
+
+
+def softmax_forward(x, y, log=False, stream=None):
+    """Softmax::forward over dimension 1 of a [B, C] or [B, C, S] tensor (log: log-softmax)"""
+    if x.dim() not in (2, 3):
+        raise ValidationError("softmax: 2 or 3 dimensions")
+    inner = int(x.shape[2]) if x.dim() == 3 else 1
+    lib().dlp_softmax_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                              ctypes.c_void_p]
+    _check(lib().dlp_softmax_fwd_enqueue(torch_dtype_code(x), int(bool(log)), int(x.shape[0]), int(x.shape[1]), inner, _ptr(x), _ptr(y),
+                                         _stream(stream)))

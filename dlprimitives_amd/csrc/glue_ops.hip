@@ -257,6 +257,41 @@ __global__ __launch_bounds__(256) void channel_affine_kernel(size_t packs, int C
     }
 }
 
+// Softmax over dimension 1 of x[B][C][S] (S = 1 for a matrix): one wavefront per (b, s) column;
+// max, sum of exp(x - max), then exp(x - max) / sum or, for the log variant, x - max - log(sum).
+template <class T>
+__global__ __launch_bounds__(256) void softmax_kernel(int B, int C, int S, int log_softmax, const T *__restrict__ x, T *__restrict__ y)
+{
+    const int lane = threadIdx.x & 63;
+    const long long col = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (col >= (long long)B * S)
+        return;
+    const int b = (int)(col / S), sp = (int)(col - (long long)b * S);
+    const T *xp = x + ((size_t)b * C) * S + sp;
+    T *yp = y + ((size_t)b * C) * S + sp;
+    float m = -3.402823466e+38f;
+    for (int j = lane; j < C; j += 64)
+        m = fmaxf(m, to_float(xp[(size_t)j * S]));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+        m = fmaxf(m, __shfl_xor(m, off));
+    float sum = 0.0f;
+    for (int j = lane; j < C; j += 64)
+        sum += expf(to_float(xp[(size_t)j * S]) - m);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+        sum += __shfl_xor(sum, off);
+    if (log_softmax) {
+        const float shift = -m - logf(sum);
+        for (int j = lane; j < C; j += 64)
+            store_plain(yp + (size_t)j * S, to_float(xp[(size_t)j * S]) + shift);
+    } else {
+        const float inv = 1.0f / sum;
+        for (int j = lane; j < C; j += 64)
+            store_plain(yp + (size_t)j * S, expf(to_float(xp[(size_t)j * S]) - m) * inv);
+    }
+}
+
 } // namespace dlp
 
 using namespace dlp;
@@ -468,6 +503,27 @@ int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int cha
             hipLaunchKernelGGL((channel_affine_kernel<float, 1>), dim3((unsigned)blocks), dim3(256), 0, st, packs, channels, plane_packs,
                                activation, (const float *)x, scale, shift, (float *)y);
     }
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+int dlp_softmax_fwd_enqueue(int dtype, int log_softmax, int batch, int classes, int inner, const void *x, void *y, void *stream)
+{
+    DLP_REQUIRE(dtype == DLP_FLOAT || dtype == DLP_BFLOAT16, "float_data and bfloat16_data are implemented");
+    DLP_REQUIRE(batch >= 0 && classes > 0 && inner > 0, "shape");
+    if (batch == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && y != nullptr, "null tensor pointer");
+    const long long cols = (long long)batch * inner;
+    DLP_REQUIRE((cols + 3) / 4 < (1ll << 31), "too many columns");
+    hipStream_t st = (hipStream_t)stream;
+    TimingScope ts("softmax", st);
+    if (dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(softmax_kernel<bf16_t>, dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, st, batch, classes, inner, log_softmax,
+                           (const bf16_t *)x, (bf16_t *)y);
+    else
+        hipLaunchKernelGGL(softmax_kernel<float>, dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, st, batch, classes, inner, log_softmax,
+                           (const float *)x, (float *)y);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }

@@ -173,6 +173,17 @@ class NetBuilder:
         self.shapes[dst] = (s[0], outputs)
         return dst
 
+    def flatten(self, src, dst):
+        s = self.shapes[src]
+        self._op("Flatten", "Flatten", [src], [dst], {})
+        self.shapes[dst] = (s[0], int(np.prod(s[1:])))
+        return dst
+
+    def softmax(self, src, dst, log=False):
+        self._op("Softmax", "Softmax", [src], [dst], {"log": bool(log)})
+        self.shapes[dst] = self.shapes[src]
+        return dst
+
     def output(self, name):
         self.doc["outputs"].append(name)
 

@@ -324,7 +324,7 @@ public:
     }
 
 private:
-    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip };
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten };
     struct Node {
         std::string name, type;
         std::vector<std::string> inputs, outputs, param_names;
@@ -356,6 +356,8 @@ private:
         // Elementwise
         int eltwise_op = DLP_ELTWISE_SUM;
         float coef[2] = {1.0f, 1.0f};
+        // Softmax
+        bool log_softmax = false;
     };
 
     static Shape shape_of(std::vector<int> const &d)
@@ -507,6 +509,19 @@ private:
                 n.coef[0] = o.get("coef1", 1.0f);
                 n.coef[1] = o.get("coef2", 1.0f);
                 specs_[n.outputs[0]] = spec(n.inputs[0]);
+            } else if (n.type == "Softmax") {
+                n.kind = k_softmax;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() == 2 || in.size() == 3); // as core::softmax_forward
+                n.log_softmax = o.type() == json::is_object ? o.get("log", false) : false;
+                specs_[n.outputs[0]] = in;
+            } else if (n.type == "Flatten") { // a view: [B, everything else]; no kernel, no memory
+                n.kind = k_flatten;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
+                Shape const &in = spec(n.inputs[0]);
+                specs_[n.outputs[0]] = Shape(in[0], in.size_no_batch());
+                alias_of_[n.outputs[0]] = n.inputs[0];
             } else
                 throw NotImplementedError("Operator type " + n.type + " (" + n.name + ")");
         }
@@ -702,6 +717,11 @@ private:
             for (auto const &t : nodes_[i].outputs)
                 last_use[t] = std::max(last_use.count(t) ? last_use[t] : -1, int(i));
         }
+        for (int pass = 0; pass < 2; pass++) // a view and its source live as long as either is used (two passes: views of views)
+            for (auto const &al : alias_of_) {
+                const int both = std::max(last_use.count(al.first) ? last_use[al.first] : -1, last_use.count(al.second) ? last_use[al.second] : -1);
+                last_use[al.first] = last_use[al.second] = both;
+            }
         tensor_memory_ = 0;
         auto own = [&](std::string const &name) {
             tensors_[name] = Tensor(ctx_, spec(name), dtype_);
@@ -725,6 +745,7 @@ private:
                 auto al = alias_of_.find(t);
                 if (al != alias_of_.end()) { // written over the other branch of a residual sum: takes over its memory
                     tensors_[t] = tensors_.at(al->second);
+                    tensors_[t].reshape(spec(t));
                     auto h = held.find(al->second);
                     if (h != held.end()) {
                         held[t] = h->second;
@@ -870,6 +891,13 @@ private:
             break;
         case k_pool:
         case k_gpool: n.pool_op->enqueue(x, y, e); break;
+        case k_softmax: {
+            Shape const &s = x.shape();
+            details::check_status(dlp_softmax_fwd_enqueue(int(dtype_), n.log_softmax ? 1 : 0, int(s[0]), int(s[1]), s.size() == 3 ? int(s[2]) : 1,
+                                                          x.device_ptr(), y.device_ptr(), e.stream()));
+            break;
+        }
+        case k_flatten: break; // the output is a view of the input
         case k_eltwise: {
             Tensor &x1 = tensor(n.inputs[1]);
             details::check_status(dlp_eltwise_fwd_enqueue_dtype(int(dtype_), n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),

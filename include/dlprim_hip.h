@@ -156,6 +156,11 @@ int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
 
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
+/* ---- Softmax::forward, src/ops/softmax.cpp:189-222 (core::softmax_forward, src/core/loss.cpp:13-40):
+ *      softmax (or log-softmax) over dimension 1 of x[batch][classes][inner] (inner = 1 for a matrix);
+ *      y may be x ------------------------------------------------------------------------------- */
+int dlp_softmax_fwd_enqueue(int dtype, int log_softmax, int batch, int classes, int inner, const void *x, void *y, void *stream);
+
 /* ---- core::Conv2DBackwardData, include/dlprim/core/conv.hpp:60-68, src/core/conv.cpp:113-163,299-367,
  *      512-590 (CPU contract: src/ops/conv2d.cpp:426-430,485-498):
  *      dx [B,Cin,H,W] = factor * dx + gradient of the convolution with respect to x, from

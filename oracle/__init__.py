@@ -314,6 +314,24 @@ def batch_norm_forward(x, mean, var, gamma=None, beta=None, eps=1e-5, activation
     return apply_activation(y.astype(np.float32), activation).reshape(x.shape)
 
 
+def softmax_forward(x, log=False):
+    """Softmax::forward_cpu, src/ops/softmax.cpp:189-222: over dimension 1 of [B, C] or [B, C, S]; per column the maximum,
+    sum of expf(x - max) in float32 in index order, then expf(x - max) * (1 / sum), or x - max - logf(sum) for log."""
+    x = _f32(x)
+    shape = x.shape
+    v = x.reshape(shape[0], shape[1], -1)
+    m = v.max(axis=1, keepdims=True)
+    e = np.exp((v - m).astype(np.float32)).astype(np.float32)
+    total = np.zeros((v.shape[0], 1, v.shape[2]), dtype=np.float32)
+    for j in range(v.shape[1]):
+        total[:, 0, :] += e[:, j, :]
+    if log:
+        y = (v - m) + (-np.log(total)).astype(np.float32)
+    else:
+        y = e * (np.float32(1.0) / total)
+    return y.astype(np.float32).reshape(shape)
+
+
 def bf16_round(a):
     a = _f32(a).copy()
     lib().orc_bf16_round_array(_ptr(a), ctypes.c_size_t(a.size))

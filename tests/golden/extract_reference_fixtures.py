@@ -5,6 +5,8 @@ Reads DATA files only (JSON written by the reference's PyTorch fixture generator
   tests/test_case_activation.json     -> activation_fwd.json
   tests/test_case_pooling2d.json      -> pooling2d_fwd.json
   tests/test_case_global_pooling.json -> global_pooling_fwd.json
+  tests/test_case_softmax.json        -> softmax_fwd.json       (cases of up to 1100 values)
+  tests/test_case_log_softmax.json    -> log_softmax_fwd.json   (likewise)
 keeping options, parameters, inputs and expected forward outputs (gradients are
 dropped: the path is forward only).  Run in the build container, where the
 reference tree is mounted:  python tests/golden/extract_reference_fixtures.py
@@ -17,7 +19,7 @@ REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def extract(src, dst):
+def extract(src, dst, max_values=None):
     with open(os.path.join(REF, "tests", src)) as f:
         doc = json.load(f)
     out = {"operator": doc["operator"], "source": "tests/" + src, "tests": []}
@@ -37,6 +39,7 @@ def extract(src, dst):
                     **({"in": c["in_tensors"], "out": c["out_tensors"]} if "in_tensors" in c else {"use_cpu_reference": True}),
                 }
                 for c in t["cases"]
+                if max_values is None or all(len(v) <= max_values for v in c.get("in_tensors", []))
             ],
         }
         out["tests"].append(rec)
@@ -50,3 +53,5 @@ if __name__ == "__main__":
     extract("test_case_activation.json", "activation_fwd.json")
     extract("test_case_pooling2d.json", "pooling2d_fwd.json")
     extract("test_case_global_pooling.json", "global_pooling_fwd.json")
+    extract("test_case_softmax.json", "softmax_fwd.json", 1100)
+    extract("test_case_log_softmax.json", "log_softmax_fwd.json", 1100)

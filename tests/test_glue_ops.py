@@ -286,3 +286,55 @@ def test_gpu_channel_affine_is_batch_norm_with_fixed_statistics(oracle_mod, dtyp
         np.testing.assert_allclose(y.float().cpu().numpy(), want, rtol=2 ** -7 if dtype == "bfloat16" else 1e-5, atol=2 ** -7 if dtype == "bfloat16" else 1e-5)
         dlp.channel_affine_forward(tx, _dev(alpha), _dev(shift), tx, act)
         np.testing.assert_array_equal(tx.float().cpu().numpy(), y.float().cpu().numpy())
+
+
+def _softmax_cases(log):
+    doc = json.load(open(os.path.join(GOLDEN, "log_softmax_fwd.json" if log else "softmax_fwd.json")))
+    assert doc["operator"] == "Softmax" and doc["tests"][0]["options"] == {"log": log}
+    for c in doc["tests"][0]["cases"]:
+        if "in" not in c:
+            continue  # the reference's "compare with the CPU operator on random inputs" cases hold no values
+        shape = c["in_shapes"][0]
+        yield np.asarray(c["in"][0], dtype=np.float32).reshape(shape), np.asarray(c["out"][0], dtype=np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("log", [False, True])
+def test_oracle_softmax_reference_goldens(oracle_mod, log):
+    """The golden cases of the reference's own tests (tests/test_case_softmax.json, test_case_log_softmax.json)."""
+    n = 0
+    for x, want in _softmax_cases(log):
+        np.testing.assert_allclose(oracle_mod.softmax_forward(x, log), want, rtol=2e-5, atol=1e-6)
+        n += 1
+    assert n == 46
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("log", [False, True])
+def test_gpu_softmax_reference_goldens(oracle_mod, log):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    for x, want in _softmax_cases(log):
+        y = torch.full(x.shape, float("nan"), device="cuda:0")
+        dlp.softmax_forward(_dev(x), y, log)
+        np.testing.assert_allclose(y.cpu().numpy(), want, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_softmax_inner_dimension_in_place(oracle_mod, dtype):
+    """[B, C, S] tensors (softmax over dimension 1, as the reference does for three dimensions), in place, bfloat16 storage."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(14)
+    for shape in [(3, 7, 5), (2, 100, 1), (1, 1000, 3), (5, 1, 4), (4, 65)]:
+        x = oracle_mod.bf16_round(rng.standard_normal(shape).astype(np.float32) * 3)
+        for log in (False, True):
+            t = _dev(x).to(tdt)
+            dlp.softmax_forward(t, t, log)
+            want = oracle_mod.softmax_forward(x, log)
+            np.testing.assert_allclose(t.float().cpu().numpy(), want, rtol=2 ** -7 if dtype == "bfloat16" else 2e-5, atol=2 ** -7 if dtype == "bfloat16" else 1e-6)

@@ -233,6 +233,10 @@ def torch_forward(doc, params, inputs, bf16=False):
                 y = F.avg_pool2d(x, k, s, p, ceil_mode=bool(o.get("ceil_mode", False)), count_include_pad=bool(o.get("count_include_pad", False)))
         elif kind == "GlobalPooling":
             y = x.amax((2, 3), keepdim=True) if o.get("mode", "max") == "max" else x.mean((2, 3), keepdim=True)
+        elif kind == "Flatten":
+            y = x.reshape(x.shape[0], -1)
+        elif kind == "Softmax":
+            y = torch.log_softmax(x, 1) if o.get("log", False) else torch.softmax(x, 1)
         elif kind == "Elementwise":
             a, b = x * o.get("coef1", 1.0), t[op["inputs"][1]] * o.get("coef2", 1.0)
             y = {"sum": a + b, "prod": a * b, "max": torch.maximum(a, b)}[o.get("operation", "sum")]
@@ -247,7 +251,7 @@ def mixed_net():
     separate activations (in place and not), BatchNorm that folds and BatchNorm that cannot
     (after pooling; feeding two readers; without affine), a dilated and a grouped convolution,
     avg pooling with ceil mode, all three elementwise operations with coefficients, two inputs
-    and two outputs."""
+    a Flatten view, Softmax and log-Softmax, and several outputs."""
     b = netfile.NetBuilder("data", (3, 5, 23, 19))
     b.input("side", (3, 12, 12, 10))
     t = b.conv("data", "c0", 12, 3, 2, 1, bias=True, scalar_options=True)
@@ -268,9 +272,11 @@ def mixed_net():
     g = b.global_pool(q, "g0", "max")
     h = b.global_pool(q, "g1", "avg")
     gh = b.eltwise(g, h, "e3", "sum")
-    f = b.ip(q, "f0", 17, activation="relu")
+    f = b.ip(b.flatten(q, "qf"), "f0", 17, activation="relu")  # q is read again below, after its view
     f = b.ip(f, "f1", 9, bias=False)
     f = b.bn(f, "f1n")  # folds into the inner product
+    b.softmax(f, "prob")
+    b.softmax(f, "logprob", log=True)
     # residual sums: one that moves into the epilogue of the later convolution (with a coefficient on the
     # other branch and an activation of its own), one that cannot (the other branch is read again later)
     ra = b.conv(q, "ra", 12, 3, 1, 1, bias=True)
@@ -283,6 +289,8 @@ def mixed_net():
     b.output("f1n")
     b.output("e3")
     b.output("ru")
+    b.output("prob")
+    b.output("logprob")
     return b
 
 
