@@ -295,21 +295,34 @@ __global__ __launch_bounds__(256) void depthwise_wgrad3x3_kernel(const float *__
         part[((size_t)slice * Cout + k) * 9 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
-// out[i] = factor * out[i] + sum over slices, in slice order
+// out[i] = factor * out[i] + sum over slices.  A wavefront owns 64 consecutive outputs; the four wavefronts of a
+// workgroup take every fourth slice each (slice order within a wavefront, then the four sums in wavefront order:
+// the same bits every run), so a launch with few outputs and many slices still fills the chip.
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ out, size_t n, int slices, float factor)
 {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    __shared__ float sums[3][64];
+    const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
+    for (size_t base = (size_t)blockIdx.x * 64; base < n; base += (size_t)gridDim.x * 64) {
+        const size_t i = base + lane;
         float s = 0.0f;
-        int k = 0;
-        for (; k + 4 <= slices; k += 4) {
-            const float v0 = part[(size_t)k * n + i], v1 = part[(size_t)(k + 1) * n + i], v2 = part[(size_t)(k + 2) * n + i],
-                        v3 = part[(size_t)(k + 3) * n + i];
-            s = (((s + v0) + v1) + v2) + v3;
+        if (i < n) {
+            int k = sub;
+            for (; k + 12 < slices; k += 16) {
+                const float v0 = part[(size_t)k * n + i], v1 = part[(size_t)(k + 4) * n + i], v2 = part[(size_t)(k + 8) * n + i],
+                            v3 = part[(size_t)(k + 12) * n + i];
+                s = (((s + v0) + v1) + v2) + v3;
+            }
+            for (; k < slices; k += 4)
+                s += part[(size_t)k * n + i];
         }
-        for (; k < slices; k++)
-            s += part[(size_t)k * n + i];
-        out[i] = factor != 0.0f ? fmaf(out[i], factor, s) : s;
+        if (sub > 0)
+            sums[sub - 1][lane] = s;
+        __syncthreads();
+        if (sub == 0 && i < n) {
+            s = ((s + sums[0][lane]) + sums[1][lane]) + sums[2][lane];
+            out[i] = factor != 0.0f ? fmaf(out[i], factor, s) : s;
+        }
+        __syncthreads();
     }
 }
 
@@ -407,6 +420,11 @@ __global__ __launch_bounds__(256) void bias_backward_kernel(const float *__restr
 }
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+unsigned reduce_grid_for(size_t n)
+{
+    return (unsigned)std::min<size_t>(std::max<size_t>((n + 63) / 64, 1), 256 * 64);
+}
 
 unsigned grid_for(size_t n)
 {
@@ -772,7 +790,7 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
     const size_t n_out = (size_t)c.channels_out * ncol;
     if (batch == 0) { // the gradient is zero: dw = factor * dw
         TimingScope ts("wgrad_reduce", st);
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)dw, (float *)dw, n_out, 0, factor);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(reduce_grid_for(n_out)), dim3(256), 0, st, (const float *)dw, (float *)dw, n_out, 0, factor);
         DLP_HIP_TRY(hipGetLastError());
         return DLP_OK;
     }
@@ -794,7 +812,7 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
                                c.stride[0], c.stride[1], c.pad[0], c.pad[1], c.dilate[0], c.dilate[1]);
         }
         TimingScope ts("wgrad_reduce", st);
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(reduce_grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
         DLP_HIP_TRY(hipGetLastError());
         return DLP_OK;
     }
@@ -881,7 +899,7 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
     }
     if (p.slices > 1) {
         TimingScope ts("wgrad_reduce", st);
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(reduce_grid_for(n_out)), dim3(256), 0, st, (const float *)ws, (float *)dw, n_out, p.slices, factor);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
