@@ -157,6 +157,63 @@ public:
         ready_ = true;
     }
 
+    // After the inputs were given other shapes (net.input(i).reshape(...)): every tensor takes the shape that follows.
+    // As in the reference (include/dlprim/net.hpp: "reshape all tensors in network after reshaping the input data"),
+    // tensors keep their memory, so shapes may shrink (a smaller batch, a smaller image) but not grow beyond what
+    // setup() allocated.  Convolutions whose image size changed are planned again (and their weights packed again).
+    void reshape()
+    {
+        DLPRIM_CHECK(ready_);
+        release_graph();
+        for (auto const &name : input_names_)
+            specs_[name] = tensors_.at(name).shape();
+        ExecutionContext e = ctx_.is_cpu_context() ? ExecutionContext() : ctx_.make_execution_context();
+        for (auto &n : nodes_) {
+            if (n.skipped)
+                continue;
+            Shape const in = spec(n.inputs[0]);
+            Shape out;
+            switch (n.kind) {
+            case k_conv: {
+                DLPRIM_CHECK(in.size() == 4 && int(in[1]) == n.conv.channels_in);
+                out = core::Conv2DBase::get_output_shape(n.conv, in);
+                Shape const &old = n.planned_in;
+                if (n.conv_op && (old[2] != in[2] || old[3] != in[3])) {
+                    create_conv_operator(n, in);
+                    if (workspace_bytes_ > workspace_.memory_size())
+                        workspace_ = Tensor(ctx_, Shape(workspace_bytes_), uint8_data);
+                    if (n.is_packed) {
+                        n.is_packed = false;
+                        pack_conv_weights(n, e);
+                    }
+                }
+                break;
+            }
+            case k_ip:
+                DLPRIM_CHECK(in.size_no_batch() == size_t(n.ip_inputs));
+                out = Shape(in[0], size_t(n.ip_outputs));
+                break;
+            case k_pool:
+                DLPRIM_CHECK(in.size() == 4);
+                out = Shape(in[0], in[1], size_t(core::calc_pooling_output_size(int(in[2]), n.kernel[0], n.pad[0], n.stride[0], n.ceil_mode)),
+                            size_t(core::calc_pooling_output_size(int(in[3]), n.kernel[1], n.pad[1], n.stride[1], n.ceil_mode)));
+                break;
+            case k_gpool: out = Shape(in[0], in[1], 1, 1); break;
+            case k_flatten: out = Shape(in[0], in.size_no_batch()); break;
+            case k_eltwise:
+                if (spec(n.inputs[1]) != in)
+                    throw ValidationError("Elementwise inputs of different shapes after reshape (" + n.name + ")");
+                out = in;
+                break;
+            default: out = in; break;
+            }
+            specs_[n.outputs[0]] = out;
+            tensors_.at(n.outputs[0]).reshape(out);
+        }
+        if (!ctx_.is_cpu_context())
+            e.finish();
+    }
+
     void load_parameters(std::string const &file, bool allow_missing = false)
     {
         std::ifstream f(file, std::ios::binary);
@@ -345,6 +402,7 @@ private:
         std::unique_ptr<core::IPForward> ip_op;
         Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
         Tensor packed;       // the weights in the order the kernel loads them
+        Shape planned_in;    // input shape the convolution operator was created for
         // BatchNorm
         float eps = 1e-5f;
         bool affine = true;
@@ -661,6 +719,24 @@ private:
         }
     }
 
+    void create_conv_operator(Node &n, Shape const &in)
+    {
+        core::Conv2DSettings cfg(n.conv, in, dtype_);
+        n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
+        if (n.residual)
+            n.conv_op->accumulate_before_activation(true);
+        n.planned_in = in;
+        workspace_bytes_ = std::max(workspace_bytes_, n.conv_op->workspace());
+    }
+    void pack_conv_weights(Node &n, ExecutionContext const &e)
+    {
+        const size_t bytes = n.conv_op->packed_size();
+        if (bytes > 0 && n.packed.shape().total_size() != bytes)
+            n.packed = Tensor(ctx_, Shape(bytes), uint8_data);
+        n.conv_op->pack(n.use_w_dev ? n.w_dev : param(n.param_names[0]), n.packed, e);
+        n.is_packed = true;
+    }
+
     void create_operators()
     {
         workspace_bytes_ = 0;
@@ -671,14 +747,7 @@ private:
                 continue;
             Shape const &in = spec(n.inputs[0]);
             switch (n.kind) {
-            case k_conv: {
-                core::Conv2DSettings cfg(n.conv, in, dtype_);
-                n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
-                if (n.residual)
-                    n.conv_op->accumulate_before_activation(true);
-                workspace_bytes_ = std::max(workspace_bytes_, n.conv_op->workspace());
-                break;
-            }
+            case k_conv: create_conv_operator(n, in); break;
             case k_ip: {
                 core::IPSettings cfg;
                 cfg.inputs = n.ip_inputs;
@@ -847,13 +916,8 @@ private:
                 n.w_dev.to_device(e);
             }
         }
-        if (n.kind == k_conv && prepack_ && n.conv_op) {
-            const size_t bytes = n.conv_op->packed_size();
-            if (bytes > 0 && n.packed.shape().total_size() != bytes)
-                n.packed = Tensor(ctx_, Shape(bytes), uint8_data);
-            n.conv_op->pack(n.use_w_dev ? n.w_dev : param(n.param_names[0]), n.packed, e);
-            n.is_packed = true;
-        }
+        if (n.kind == k_conv && prepack_ && n.conv_op)
+            pack_conv_weights(n, e);
     }
 
     void run(Node &n, ExecutionContext const &e)

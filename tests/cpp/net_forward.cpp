@@ -6,7 +6,8 @@
 //   net_forward plan <net.json> [keep] [nofuse]
 //       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
 //       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
-//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [resave=<file.dlpw>] [repeat=<n>]
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [batch=<n>] [resave=<file.dlpw>] [repeat=<n>]
+//       (batch=<n>: the inputs are reshaped to n images and Net::reshape() is called before the pass)
 //       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32)
 //       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
 //       network's input order), runs forward and writes the outputs (float32, in output order)
@@ -49,7 +50,7 @@ int main(int argc, char **argv)
         }
         bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false;
         std::string resave;
-        int repeat = 1, warmup = 5, iters = 20;
+        int repeat = 1, warmup = 5, iters = 20, batch = 0;
         const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
         for (int i = first_flag; i < argc; i++) {
             std::string a = argv[i];
@@ -67,6 +68,8 @@ int main(int argc, char **argv)
                 resave = a.substr(7);
             else if (a.compare(0, 7, "repeat=") == 0)
                 repeat = std::atoi(a.c_str() + 7);
+            else if (a.compare(0, 6, "batch=") == 0)
+                batch = std::atoi(a.c_str() + 6);
             else if (a.compare(0, 7, "warmup=") == 0)
                 warmup = std::atoi(a.c_str() + 7);
             else if (a.compare(0, 6, "iters=") == 0)
@@ -153,6 +156,14 @@ int main(int argc, char **argv)
         if (!resave.empty())
             net.save_parameters(resave);
         dp::ExecutionContext e = ctx.make_execution_context();
+        if (batch > 0) { // run on fewer images than the network file says: Net::reshape
+            for (unsigned i = 0; i < net.input_names().size(); i++) {
+                dp::Shape s = net.input(i).shape();
+                s[0] = size_t(batch);
+                net.input(i).reshape(s);
+            }
+            net.reshape();
+        }
         std::ifstream in(argv[4], std::ios::binary);
         if (!in)
             throw dp::ValidationError(std::string("cannot open ") + argv[4]);

@@ -414,6 +414,40 @@ def test_gpu_net_random_graphs(tmp_path, seed):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("net", ["mixed", "resnet18_b2_64"])
+@pytest.mark.parametrize("flags", [(), ("bf16",)], ids=["float", "bf16"])
+def test_gpu_net_reshape_to_a_smaller_batch(tmp_path, net, flags):
+    """The network file says batch 4 (3 for the mixed one); the pass runs on fewer images after Net::reshape()."""
+    make, seed = NETS[net]
+    b = make()
+    for i in b.doc["inputs"]:
+        i["shape"][0] += 2  # set up for a larger batch than the one that runs
+    p = write_net(tmp_path, b)
+    params = b.random_parameters(seed)
+    netfile.save_dlpw(tmp_path / "w.dlpw", params)
+    small = make()
+    rng = np.random.default_rng(seed + 7)
+    inputs = {i["name"]: rng.uniform(-1, 1, i["shape"]).astype(np.float32) for i in small.doc["inputs"]}
+    with open(tmp_path / "in.bin", "wb") as f:
+        for i in small.doc["inputs"]:
+            f.write(inputs[i["name"]].tobytes())
+    n = small.doc["inputs"][0]["shape"][0]
+    tool("run", p, tmp_path / "w.dlpw", tmp_path / "in.bin", tmp_path / "out.bin", "batch=%d" % n, "repeat=2", *flags)
+    want = torch_forward(small.doc, params, inputs)
+    emulated = torch_forward(small.doc, params, inputs, bf16=True) if "bf16" in flags else want
+    got = np.fromfile(tmp_path / "out.bin", dtype=np.float32)
+    assert got.size == sum(w.size for w in want)
+    off = 0
+    for name, w, em in zip(small.doc["outputs"], want, emulated):
+        g = got[off : off + w.size].reshape(w.shape)
+        off += w.size
+        scale = np.abs(w).max()
+        err = np.abs(g - w).max() / scale
+        noise = np.abs(em - w).max() / scale
+        assert err < (3 * noise + 1e-2 if "bf16" in flags else 1e-4), (name, err, noise)
+
+
+@pytest.mark.gpu
 def test_gpu_net_missing_parameter_is_an_error(tmp_path):
     b = netfile.resnet18(1, 32, 4)
     p = write_net(tmp_path, b)
