@@ -69,7 +69,15 @@ __global__ __launch_bounds__(256) void conv_wgrad_f32_kernel(WgradArgs a)
     const int l32 = lane & 31, h = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    int t = blockIdx.x; // tile fastest: workgroups that share a slice (the same dy / x data) are neighbours
+    // tile fastest: workgroups that share a slice read the same dy / x data.  Workgroup ids are dealt round-robin
+    // to the 8 XCDs, each with its own L2: renumber so that an XCD runs a contiguous range (whole slices).
+    int t;
+    {
+        const int nb = gridDim.x, bid = blockIdx.x;
+        const int q = nb >> 3, r = nb & 7;
+        const int xcd = bid & 7, slot = bid >> 3;
+        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+    }
     const int mt = t % a.mtiles;
     t /= a.mtiles;
     const int nt = t % a.ntiles;
