@@ -175,14 +175,31 @@ int main(int argc, char **argv)
                 throw dp::ValidationError("input file is too short");
             net.set_input(i, inputs[i].data(), e);
         }
-        if (graph) { // recorded with other input values than the ones that count: a replay must read the tensors anew
+        std::vector<std::vector<float>> eager_out;
+        if (graph) {
+            // the eager result first; then the recording, made with other input values than the ones that count
+            // (a replay must read the tensors anew); every replay below must reproduce the eager result bit for bit
+            net.forward(e, true);
+            eager_out.resize(net.output_names().size());
+            for (unsigned i = 0; i < eager_out.size(); i++) {
+                eager_out[i].resize(net.output(i).shape().total_size());
+                net.get_output(i, eager_out[i].data(), e);
+            }
             std::vector<float> other(inputs[0].size(), 0.25f);
             net.set_input(0, other.data(), e);
             net.capture_forward(e);
-            net.set_input(0, inputs[0].data(), e);
         }
-        for (int r = 0; r < repeat; r++) // later passes must give what the first one gave: shared chunks are rewritten
+        for (int r = 0; r < repeat; r++) { // later passes must give what the first one gave: shared chunks are rewritten
+            if (graph)
+                net.set_input(0, inputs[0].data(), e); // eager work between the replays
             net.forward(e, true);
+            for (unsigned i = 0; graph && i < eager_out.size(); i++) {
+                std::vector<float> v(eager_out[i].size());
+                net.get_output(i, v.data(), e);
+                if (std::memcmp(v.data(), eager_out[i].data(), v.size() * sizeof(float)) != 0)
+                    throw dp::ValidationError("graph replay " + std::to_string(r) + " differs from the eager pass in output " + std::to_string(i));
+            }
+        }
         std::ofstream out(argv[5], std::ios::binary);
         for (unsigned i = 0; i < net.output_names().size(); i++) {
             std::vector<float> v(net.output(i).shape().total_size());
