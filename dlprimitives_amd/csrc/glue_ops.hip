@@ -135,29 +135,31 @@ __global__ __launch_bounds__(256) void maxpool3x3s2p1_kernel(PoolArgs a, int nst
     }
 }
 
-// one wavefront per plane: lanes stride over the plane, then a shuffle reduction.
+// LPP lanes per plane (64: one wavefront per plane; 16: four planes per wavefront, for the 7x7 and
+// smaller planes at the end of a network): lanes stride over the plane, then a shuffle reduction.
 // The average is accumulated per lane in ascending index order and combined pairwise,
 // so it differs from the reference's single running sum only by fp32 rounding.
-template <class T>
+template <class T, int LPP>
 __global__ __launch_bounds__(256) void global_pool_kernel(const T *__restrict__ x, T *__restrict__ y, long long planes, int plane_size,
                                                           int mode)
 {
-    const int lane = threadIdx.x & 63;
-    const long long plane = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (plane >= planes)
-        return;
-    const T *src = x + plane * plane_size;
+    constexpr int PPB = 256 / LPP; // planes per workgroup
+    const int sub = threadIdx.x % LPP;
+    const long long plane = (long long)blockIdx.x * PPB + threadIdx.x / LPP;
+    const bool ok = plane < planes;
+    const T *src = x + (ok ? plane : 0) * plane_size;
     float v = mode == 0 ? -3.402823466e+38f : 0.0f;
-    for (int i = lane; i < plane_size; i += 64) {
-        const float t = to_float(src[i]);
-        v = mode == 0 ? fmaxf(v, t) : v + t;
-    }
+    if (ok)
+        for (int i = sub; i < plane_size; i += LPP) {
+            const float t = to_float(src[i]);
+            v = mode == 0 ? fmaxf(v, t) : v + t;
+        }
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const float o = __shfl_down(v, off);
+    for (int off = LPP / 2; off >= 1; off >>= 1) {
+        const float o = __shfl_down(v, off, LPP);
         v = mode == 0 ? fmaxf(v, o) : v + o;
     }
-    if (lane == 0)
+    if (ok && sub == 0)
         store_plain(y + plane, mode == 0 ? v : v * (1.0f / plane_size));
 }
 
@@ -379,12 +381,23 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         const long long plane_size = (long long)x_shape[2] * x_shape[3];
         DLP_REQUIRE(plane_size > 0 && plane_size < 0x7fffffffLL, "plane size");
         TimingScope ts("global_pooling", s);
-        if (op->dtype == DLP_BFLOAT16)
-            hipLaunchKernelGGL(global_pool_kernel<bf16_t>, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const bf16_t *)x, (bf16_t *)y,
-                               planes, (int)plane_size, op->mode);
-        else
-            hipLaunchKernelGGL(global_pool_kernel<float>, dim3((unsigned)((planes + 3) / 4)), dim3(256), 0, s, (const float *)x, (float *)y,
-                               planes, (int)plane_size, op->mode);
+        const bool small = plane_size <= 64;
+        const unsigned grid = (unsigned)((planes + (small ? 15 : 3)) / (small ? 16 : 4));
+        if (op->dtype == DLP_BFLOAT16) {
+            if (small)
+                hipLaunchKernelGGL((global_pool_kernel<bf16_t, 16>), dim3(grid), dim3(256), 0, s, (const bf16_t *)x, (bf16_t *)y, planes, (int)plane_size,
+                                   op->mode);
+            else
+                hipLaunchKernelGGL((global_pool_kernel<bf16_t, 64>), dim3(grid), dim3(256), 0, s, (const bf16_t *)x, (bf16_t *)y, planes, (int)plane_size,
+                                   op->mode);
+        } else {
+            if (small)
+                hipLaunchKernelGGL((global_pool_kernel<float, 16>), dim3(grid), dim3(256), 0, s, (const float *)x, (float *)y, planes, (int)plane_size,
+                                   op->mode);
+            else
+                hipLaunchKernelGGL((global_pool_kernel<float, 64>), dim3(grid), dim3(256), 0, s, (const float *)x, (float *)y, planes, (int)plane_size,
+                                   op->mode);
+        }
     } else {
         // the output shape fixes ceil_mode; every window must start inside the padded input (pool.hpp:17-27)
         for (int i = 0; i < 2; i++) {
