@@ -2256,6 +2256,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
 {
     GemmPlan p;
     p.wdirect = 0;
+    p.stem = conv_stem_supported(g) ? 1 : 0;
     p.dense_pxl = 0;
     p.dense_sx = 1;
     p.patch_bf16 = 0;
@@ -2391,6 +2392,8 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 {
     if (p.wdirect && ((uintptr_t)w & 15) == 0)
         return DLP_OK; // conv_gemm_launch reads w in place
+    if (p.stem)
+        return DLP_OK; // conv_stem_f32_kernel reads w in place and keeps no counters
     int *zero = nullptr; // tile counters of the stream-K launch that follows
     int nzero = 0;
     if (mode != GEMM_PACK_ONLY && p.patch && part_ws != nullptr) {
@@ -2463,6 +2466,11 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
+    if (p.stem) {
+        if (w == nullptr || n_valid >= 0)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "stem convolution: needs the weight tensor and the whole batch");
+        return conv_stem_launch(g, x, w, y, ep, stream);
+    }
 
     GemmArgs a;
     a.x = x;

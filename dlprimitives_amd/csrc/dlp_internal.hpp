@@ -157,6 +157,7 @@ struct GemmPlan {
     int M, K, nkt;      // per group: rows, reduction length, K tiles of 16
     int mtiles;         // ceil(M / BM)
     int patch;          // 1: stride-1 "same" convolution run by the LDS-patch kernel (tap-major packed weights)
+    int stem;           // 1: 3-channel 7x7 stride-2 convolution run by conv_stem_f32_kernel (reads the weight tensor in place, nothing is packed)
     int wdirect;        // bf16 matrix-instruction path, 1x1: the kernel reads the weight tensor in place, nothing is packed
     int dense_pxl;      // bf16 matrix-instruction path, 1x1 stride 1 pad 0: input pixels per load of the dense loader (8, 4; 0 = gather)
     int dense_sx;       // ... 2: the dense loader on a 1x1 stride-2 convolution (dense_pxl output pixels = 2 * dense_pxl loaded)
@@ -184,6 +185,10 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
                      void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *part_ws = nullptr,
                      size_t part_bytes = 0, const void *w = nullptr);
+
+// ---- few-channel strided stem convolution (conv_stem.hip) ----------------------
+bool conv_stem_supported(const ConvGeom &g);
+int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
 
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);

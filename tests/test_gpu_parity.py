@@ -160,6 +160,67 @@ def test_patch_kernel_integer_exact_and_small_workspace(gpu):
     assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
 
 
+# 7x7 / stride 2 convolutions of 3 channels (the ResNet stem) run a kernel of their own: a band of four output rows per
+# workgroup, input rows and filter rows in LDS, blocks of 32 pixels handed out inside the workgroup.
+# (batch, cout, H, W, pad, bias, activation)
+STEM_SHAPES = [
+    (2, 64, 224, 224, 3, True, "relu"),       # the real shape: 28 bands of 14 blocks
+    (3, 64, 37, 53, 3, True, "identity"),     # width off the 16-byte loads, last band of three rows
+    (1, 8, 9, 12, 3, False, "relu"),          # one m tile with eight filters, OH = 5
+    (2, 72, 40, 64, 3, True, "tanh"),         # second m tile holds eight filters
+    (2, 128, 30, 36, 2, True, "relu6"),       # two whole m tiles, pad 2
+    (1, 16, 21, 20, 0, True, "identity"),     # no padding
+    (2, 24, 7, 8, 3, True, "sigmoid"),        # image as small as the filter
+    (2, 32, 33, 44, (3, 1), True, "relu"),    # different row / column padding
+    (2, 16, 20, 232, (0, 4), False, "relu"),  # widest row the LDS rows hold
+    (5, 64, 64, 64, 3, True, "relu"),
+]
+
+
+@pytest.mark.parametrize("shape", STEM_SHAPES, ids=lambda s: "b%d_o%d_%dx%d_p%s_%s" % (s[0], s[1], s[2], s[3], s[4], s[6]))
+def test_stem_kernel(gpu, oracle_mod, shape):
+    b, cout, h, w_, pad, has_bias, act = shape
+    c = case(7, pad, 2, 1, 3, cout, has_bias, 1, False)
+    c["activation"] = act
+    x, w, bias = make_tensors(c, (b, h, w_), seed=b * 100 + cout + w_)
+    print("stem case", shape, flush=True)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+    again, _ = gpu.run_conv(c, x, w, bias, algo="gemm")
+    assert np.array_equal(got, again)
+    old = np.random.default_rng(5).standard_normal(want.shape).astype(np.float32)
+    got_f, _ = gpu.run_conv(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got_f, oracle_mod.apply_factor(want, old, 0.5), **TOL)
+
+
+def test_stem_kernel_integer_exact_and_unaligned_input(gpu):
+    # integer-valued tensors: every summation order gives the same fp32 result, which must EQUAL the integer result;
+    # the input starts 4 bytes off a 16-byte boundary the second time (the kernel then loads single elements)
+    import torch
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(11)
+    x = np.round(rng.standard_normal((3, 3, 50, 72)) * 3).astype(np.float32)
+    w = np.round(rng.standard_normal((40, 3, 7, 7)) * 3).astype(np.float32)
+    bias = np.round(rng.standard_normal(40) * 3).astype(np.float32)
+    want = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(bias).double(),
+                                      stride=2, padding=3).numpy()
+    st = dlp.Conv2DSettings(3, 40, 7, 2, 1, 3, 1, x.shape)
+    op = dlp.Conv2DForward.create(st, True, "identity", "gemm")
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    wd, bd = torch.from_numpy(w).cuda(), torch.from_numpy(bias).cuda()
+    for shift in (0, 1):
+        store = torch.zeros(x.size + 8, dtype=torch.float32, device="cuda:0")
+        xd = store[shift:shift + x.size].view(x.shape)
+        xd.copy_(torch.from_numpy(x))
+        assert xd.data_ptr() % 16 == 4 * shift
+        y = torch.full(want.shape, float("nan"), dtype=torch.float32, device="cuda:0")
+        op.enqueue(xd, wd, bd, y, ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy().astype(np.float64), want), shift
+
+
 def test_gemm_integer_exact(gpu):
     # integer-valued inputs: fp32 sums are exact in any order, so the MFMA result must
     # EQUAL the integer result -- catches any indexing/layout slip that a tolerance could hide
@@ -448,6 +509,7 @@ RESIDUAL_CASES = [  # cin, cout, k, s, p, hw, batch, algo
     (256, 512, 3, 2, 1, 14, 8, "gemm"),     # split-K, reduced in place
     (64, 64, 3, 1, 1, 28, 4, "winograd"),
     (32, 48, 3, 1, 1, 13, 2, "winograd"),   # odd planes: cut tiles
+    (3, 64, 7, 2, 3, 45, 2, "gemm"),        # stem kernel
 ]
 
 
