@@ -520,7 +520,7 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
                             v = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, voff, soff, 0)), a.factor, v);
                         if (ACT == ACT_CLAMP) {
                             if (clamp) // identity must keep NaNs: no min/max
-                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                                v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                         } else
                             v = apply_act(v, a.act);
                         if (sizeof(T) == 4)
@@ -555,7 +555,7 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
                         v = fmaf(to_float(yb[(size_t)m * a.OHW]), a.factor, v);
                     if (ACT == ACT_CLAMP) {
                         if (a.act != DLP_ACT_IDENTITY) // identity must keep NaNs: no min/max
-                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                            v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                     } else
                         v = apply_act(v, a.act);
                     store_out(yb + (size_t)m * a.OHW, v, pre ? 0.0f : a.factor);
@@ -998,7 +998,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         float v = acc[i][j][4 * rq + rr] + bv[rr];
                         if (ACT == ACT_CLAMP) {
                             if (clamp)
-                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                                v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                         } else if (!pre)
                             v = apply_act(v, a.act);
                         *(uint16_t *)(col + (i * 32 + 8 * rq + rr) * PITCH) = to_bf16(v).bits;
@@ -1038,8 +1038,8 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         float hi = fmaf(__builtin_bit_cast(float, old[d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[d] & 0xFFFF0000u));
                         if (ACT == ACT_CLAMP) {
                             if (a.act != DLP_ACT_IDENTITY) {
-                                lo = fminf(fmaxf(lo, a.clamp_lo), a.clamp_hi);
-                                hi = fminf(fmaxf(hi, a.clamp_lo), a.clamp_hi);
+                                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
                             }
                         } else {
                             lo = apply_act(lo, a.act);
@@ -1101,7 +1101,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         float v = acc[i][j][4 * rq + rr] + bv[rr];
                         if (ACT == ACT_CLAMP) {
                             if (clamp)
-                                v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                                v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                         } else
                             v = apply_act(v, a.act);
                         __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, (uint32_t)((i * 32 + 8 * rq + rr) * a.OHW * 2), 0);
@@ -1133,7 +1133,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         v = fmaf(to_float(yb[(size_t)m * a.OHW]), a.factor, v);
                     if (ACT == ACT_CLAMP) {
                         if (a.act != DLP_ACT_IDENTITY)
-                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                            v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                     } else
                         v = apply_act(v, a.act);
                     store_out(yb + (size_t)m * a.OHW, v, pre ? 0.0f : a.factor);
@@ -1805,7 +1805,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
             r = fmaf(to_float(*yp), a.factor, r);
         if (ACT == ACT_CLAMP) {
             if (a.act != DLP_ACT_IDENTITY)
-                r = fminf(fmaxf(r, a.clamp_lo), a.clamp_hi);
+                r = clamp_med3(r, a.clamp_lo, a.clamp_hi);
         } else
             r = apply_act(r, a.act);
         store_out(yp, r, pre ? 0.0f : a.factor);

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(kStemThreads) void conv_stem_f32_kernel(StemArgs a)
                     const uint32_t soff = (uint32_t)((mrow + (r & 3)) * a.OHW * 4);
                     float v = r < 16 ? acc0[r & 15] : acc1[r & 15];
                     if constexpr (MODE == 1)
-                        v = __builtin_amdgcn_fmed3f(v, a.clamp_lo, a.clamp_hi);
+                        v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                     if constexpr (MODE == 2) {
                         float old = 0.0f;
                         if (use_old)
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kStemThreads) void conv_stem_f32_kernel(StemArgs a)
                         if constexpr (GENERIC_ACT)
                             v = apply_act(v, a.act);
                         else if (a.act != DLP_ACT_IDENTITY) // identity must keep NaNs: no min/max
-                            v = fminf(fmaxf(v, a.clamp_lo), a.clamp_hi);
+                            v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
                         if (use_old && !pre)
                             v = fmaf(old, a.factor, v);
                     }

@@ -73,6 +73,10 @@ __device__ __forceinline__ float apply_act(float v, int act)
     }
 }
 
+// min(max(v, lo), hi) for lo <= hi as one v_med3_f32 (fminf(fmaxf()) costs three vector instructions, and every
+// vector-ALU instruction of an epilogue takes issue cycles from the matrix pipe); a NaN gives lo, as the pair does.
+__device__ __forceinline__ float clamp_med3(float v, float lo, float hi) { return __builtin_amdgcn_fmed3f(v, lo, hi); }
+
 __device__ __forceinline__ void store_out(float *p, float v, float factor)
 {
     if (factor != 0.0f)
