@@ -66,6 +66,10 @@ struct GemmArgs {
     int M, N, K, nkt;
     int mtiles, ntiles;
     int splitk, kt_per_slice; // K tiles are dealt to `splitk` slices of kt_per_slice (even) tiles
+    // conv_gemm_f32_kernel: the last tail_tiles tiles (m tile fastest, then n tile, then group) are cut into tail_splitk
+    // finer slices of tail_kt K tiles, launched as the last workgroups, so that the partial last round of workgroups
+    // becomes about one small piece per CU; main_wgs = (tiles - tail_tiles) * splitk workgroups run the other tiles
+    int tail_tiles, tail_splitk, tail_kt, main_wgs;
     float *part;              // split-K partial sums [slice][Cout][N]
     int sk_units;             // stream-K (conv_patch_f32_kernel): tiles * stages
     float *sk_part;           // two 64x64 accumulator images per workgroup
@@ -151,7 +155,7 @@ __device__ __forceinline__ void static_for_all(F &&f)
 
 template <class T, int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
-                                                 int g, int slice, int wm, int wn, int h, int l32, int tid);
+                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid);
 
 template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
@@ -186,23 +190,37 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumber
     // them so that every XCD walks one contiguous range of tiles: the m tiles of one pixel
     // tile, and neighbouring pixel tiles (which share input rows), then hit the same L2.
-    int t;
+    int t, slice, splitk = a.splitk, kt_per_slice = a.kt_per_slice;
+    uint32_t image0; // index of the tile's first accumulator image in the split-K workspace
     {
-        const int nb = gridDim.x, bid = blockIdx.x;
-        const int q = nb >> 3, r = nb & 7;
-        const int xcd = bid & 7, slot = bid >> 3;
-        t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+        const int tiles = a.mtiles * a.ntiles * a.groups, tiles_main = tiles - a.tail_tiles;
+        const int bid = blockIdx.x;
+        if (bid < a.main_wgs) {
+            const int nb = a.main_wgs;
+            const int q = nb >> 3, r = nb & 7;
+            const int xcd = bid & 7, slot = bid >> 3;
+            t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
+            slice = t / tiles_main;
+            t -= slice * tiles_main;
+            image0 = (uint32_t)(t * splitk);
+        } else { // finer slices of the last tiles
+            t = bid - a.main_wgs;
+            slice = t / a.tail_tiles;
+            t -= slice * a.tail_tiles;
+            image0 = (uint32_t)((splitk > 1 ? tiles_main * splitk : 0) + t * a.tail_splitk);
+            t += tiles_main;
+            splitk = a.tail_splitk;
+            kt_per_slice = a.tail_kt;
+        }
     }
-    // tile decode: m tile fastest, then n tile, then group, then K slice
+    // tile decode: m tile fastest, then n tile, then group
     const int mt = t % a.mtiles;
     t /= a.mtiles;
     const int nt = t % a.ntiles;
-    t /= a.ntiles;
-    const int g = t % a.groups;
-    const int slice = t / a.groups;
+    const int g = t / a.ntiles;
     const int m0 = mt * BM, n0 = nt * BN;
-    const int kt_begin = slice * a.kt_per_slice;
-    const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
+    const int kt_begin = slice * kt_per_slice;
+    const int kt_end = min(kt_begin + kt_per_slice, a.nkt);
 
     // The X resource starts one padding offset before the tensor, so that the
     // per-pixel window origin is a non-negative offset; taps that the masks let
@@ -389,7 +407,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     if (kt < kt_end)
         k_step(I0{}, I1{}, I0{}, kt);
 
-    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, wm, wn, h, l32, tid);
+    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, splitk, image0, wm, wn, h, l32, tid);
 }
 
 // What a workgroup does with its finished accumulator tile: the split-K partial store, or the
@@ -397,20 +415,20 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 // last barrier of the main loop (at least BM floats).
 template <class T, int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
-                                                 int g, int slice, int wm, int wn, int h, int l32, int tid)
+                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid)
 {
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     // ---- split-K, reduced in place: the slice's accumulators go to the workspace as a register image
     // ([r][thread], write-through); the workgroup that arrives last at the tile's counter adds up all
     // slices in slice order (deterministic), whoever it is, and goes on to the epilogue.  Nobody waits. ----
-    if (a.splitk > 1 && a.sk_cnt != nullptr) {
+    if (splitk > 1 && a.sk_cnt != nullptr) {
         static_assert(TM == 1 && TN == 1, "one MFMA block per wavefront");
         constexpr int kThrough = 17; // sc0 | sc1: past the caches in both directions
         constexpr uint32_t image_bytes = BM * BN * 4;
         const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.sk_part, 0, a.sk_part_bytes, 0x00020000);
         const int tile = (g * a.ntiles + n0 / BN) * a.mtiles + m0 / BM;
-        const uint32_t base = (uint32_t)(tile * a.splitk) * image_bytes;
+        const uint32_t base = image0 * image_bytes;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const float v = acc[0][0][r];
@@ -425,18 +443,18 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
         __syncthreads();
         const int arrived = __builtin_amdgcn_readfirstlane(*arrived_s);
         __syncthreads(); // lds is reused by the epilogue
-        if (arrived != a.splitk - 1)
+        if (arrived != splitk - 1)
             return;
 #pragma unroll
         for (int r = 0; r < 16; r++)
             acc[0][0][r] = 0.0f;
-        for (int s0 = 0; s0 < a.splitk; s0 += 4) { // four slices (64 loads) in flight at a time
+        for (int s0 = 0; s0 < splitk; s0 += 4) { // four slices (64 loads) in flight at a time
             float p[4][16];
 #pragma unroll
             for (int ds = 0; ds < 4; ds++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    p[ds][r] = (s0 + ds < a.splitk) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    p[ds][r] = (s0 + ds < splitk) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
                                                           pr, (uint32_t)tid * 4u,
                                                           base + (uint32_t)(s0 + ds) * image_bytes + (uint32_t)(r * kThreads * 4), kThrough))
                                                     : 0.0f;
@@ -446,7 +464,7 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
                 for (int r = 0; r < 16; r++)
                     acc[0][0][r] += p[ds][r];
         }
-    } else if (a.splitk > 1) { // raw partial sums in output order, reduced by splitk_reduce_kernel
+    } else if (splitk > 1) { // raw partial sums in output order, reduced by splitk_reduce_kernel
         if ((a.M & 7) == 0 && a.part_bytes != 0) { // buffer stores with scalar row offsets
             const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
 #pragma unroll
@@ -878,7 +896,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         }
     }
     if (output)
-        gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, 0, wm, wn, h, l32, tid);
+        gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, 0, 1, 0u, wm, wn, h, l32, tid);
     __syncthreads(); // LDS is reused by the next piece
     u += cb_end - cb_begin;
     }
@@ -2000,15 +2018,59 @@ size_t split_workspace_bytes(const GemmPlan &p, const GemmArgs &a, int groups, i
     return split_counter_bytes(tiles) + (size_t)tiles * s * p.BM * p.BN * sizeof(float);
 }
 
+int device_cu_count();
+
+// counters | accumulator images of a launch planned by plan_split (fp32-instruction kernels)
+size_t split_total_bytes(const GemmPlan &p, const GemmArgs &a, int groups)
+{
+    if (bf16_mfma_order(p.order))
+        return split_workspace_bytes(p, a, groups, a.splitk);
+    if (a.splitk <= 1 && a.tail_tiles == 0)
+        return 0;
+    const long long tiles = (long long)a.mtiles * a.ntiles * groups;
+    const long long images = (a.splitk > 1 ? (tiles - a.tail_tiles) * a.splitk : 0) + (long long)a.tail_tiles * a.tail_splitk;
+    return split_counter_bytes(tiles) + (size_t)images * p.BM * p.BN * sizeof(float);
+}
+
 void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t ws_bytes)
 {
     a.mtiles = p.mtiles;
     a.ntiles = (a.N + p.BN - 1) / p.BN;
-    int s = choose_splitk((long long)a.mtiles * a.ntiles * groups, a.nkt, p.order);
+    const long long tiles = (long long)a.mtiles * a.ntiles * groups;
+    int s = choose_splitk(tiles, a.nkt, p.order);
     if (s > 1 && (!have_ws || ws_bytes < split_workspace_bytes(p, a, groups, s)))
         s = 1; // no (or too small a) workspace: run unsplit
     a.kt_per_slice = ((a.nkt + s - 1) / s + 1) / 2 * 2;              // even: LDS buffer parity is static
     a.splitk = (a.nkt + a.kt_per_slice - 1) / a.kt_per_slice; // every slice starts inside the K range
+    a.tail_tiles = 0;
+    a.tail_splitk = 1;
+    a.tail_kt = a.kt_per_slice;
+    // The workgroups of one launch are all resident at once (up to eight per CU) or nearly so, and a CU is done when
+    // its workgroups are: with 6.1 workgroups per CU some CUs carry 7 and the others idle for 1/7 of the time.  The
+    // tiles of the last, partial round of workgroups are therefore cut into finer K slices, about one per CU, and
+    // launched last: every CU then carries the same number of whole workgroups plus one small piece.
+    // (measured on the ResNet-18 shapes at batch 64: 3x3 stride-2 layers, 36 to 144 K tiles, 2 to 6 % faster; 1x1 layers of
+    // 4 to 16 K tiles up to 16 % slower, as the pieces' trip through the workspace then costs more than the idle time)
+    if (!bf16_mfma_order(p.order) && have_ws && tiles * a.splitk < 0x7fffffffLL && a.nkt >= DLP_SPLITK_MIN_KT) {
+        const int cus = device_cu_count();
+        const long long wgs = tiles * a.splitk, full = wgs / cus * cus;
+        if (full > 0 && full < wgs) {
+            const long long tail = tiles - full / a.splitk;
+            const long long kt2 = ((tail * a.nkt + cus - 1) / cus + 1) / 2 * 2; // the tail's K tiles per CU, even
+            const long long s2 = (a.nkt + kt2 - 1) / kt2;
+            if (kt2 < a.kt_per_slice && s2 <= 64 && tail * s2 < 0x7fffffffLL - wgs) {
+                a.tail_tiles = (int)tail;
+                a.tail_kt = (int)kt2;
+                a.tail_splitk = (int)s2;
+                if (ws_bytes < split_total_bytes(p, a, groups)) {
+                    a.tail_tiles = 0;
+                    a.tail_splitk = 1;
+                    a.tail_kt = a.kt_per_slice;
+                }
+            }
+        }
+    }
+    a.main_wgs = (int)((tiles - a.tail_tiles) * a.splitk);
 }
 
 template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
@@ -2017,6 +2079,7 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    blocks = (long long)a.main_wgs + (long long)a.tail_tiles * a.tail_splitk;
     {
         TimingScope ts("conv_gemm", stream);
         hipLaunchKernelGGL((conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
@@ -2375,7 +2438,7 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     a.Cout = g.Cout;
     a.nkt = p.nkt;
     plan_split(p, a, g.groups, true, (size_t)-1);
-    return p.wpack_bytes + split_workspace_bytes(p, a, g.groups, a.splitk);
+    return p.wpack_bytes + split_total_bytes(p, a, g.groups);
 }
 
 namespace {
@@ -2409,7 +2472,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
         a.Cout = g.Cout;
         a.nkt = p.nkt;
         plan_split(p, a, g.groups, true, part_bytes);
-        if (a.splitk > 1) {
+        if (a.splitk > 1 || a.tail_tiles > 0) {
             zero = (int *)part_ws;
             nzero = (int)((long long)a.mtiles * a.ntiles * g.groups);
         }
@@ -2525,10 +2588,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
     a.sk_cnt = nullptr;
     a.part_bytes = 0;
-    if (a.splitk > 1 && !bf16_mfma_order(p.order)) {
+    if ((a.splitk > 1 || a.tail_tiles > 0) && !bf16_mfma_order(p.order)) {
         // reduced in place; the counters were cleared by conv_gemm_pack_weights (same workspace, a batch at least as large)
         const long long tiles = (long long)a.mtiles * a.ntiles * g.groups;
-        const size_t images = split_workspace_bytes(p, a, g.groups, a.splitk) - split_counter_bytes(tiles);
+        const size_t images = split_total_bytes(p, a, g.groups) - split_counter_bytes(tiles);
         if (images >= kOutOfRange)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K workspace of 2 GiB or more");
         a.sk_cnt = (int *)part_ws;
