@@ -126,7 +126,7 @@ def kernel_class(L, bf16=False):
         return "conv_gemm_bf16_kernel<%s, %d, 0, 2, %d>" % (tile, order, pxl)
     if (not bf16 and L["groups"] == 1 and L["cin"] == 3 and L["kernel"] == 7 and L["stride"] == 2 and L["pad"] <= 4 and m % 8 == 0
             and L["hw"] <= 232 and L.get("dilate", 1) == 1):
-        return "conv_stem_f32_kernel<3, 7, 7, 2, 8, 240, 1, 0>"  # input rows of a band and the filter in LDS, no gather
+        return "conv_stem_f32_kernel<3, 7, 7, 2, 8, 240, true, false>"  # input rows of a band and the filter in LDS, no gather
     tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
     order = 1 if (small and cin_g % 16 == 0) else 0
     if (not bf16 and order == 1 and m > 32 and L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
