@@ -268,10 +268,19 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         }
     }
 
-    // ---- weight loader: 16-byte pieces of the packed tile, in tile order ----
+    // ---- weight loader: 16-byte pieces of the packed tile, in tile order; or (a.wdirect: 1x1 convolutions, whose K tile
+    // is 16 consecutive input channels) of the weight tensor itself: lane m of wavefront q takes channels 4q..4q+3 of
+    // filter row m, and the four values go to LDS one by one ----
     const uint32_t a_tile_bytes = BK * BM * 4;
-    const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes; // SGPR
+    const bool wdirect = a.wdirect != 0; // uniform
+    const uint32_t a_step = wdirect ? (uint32_t)(BK * 4) : a_tile_bytes;                                       // SGPR
+    const uint32_t a_row_base = wdirect ? 0u : (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;         // SGPR
     const bool a_active = (A_V4 >= kThreads) || (tid < A_V4);
+    uint32_t a_voff0 = a_active ? (uint32_t)(tid * 16) : kOutOfRange;
+    if (wdirect) {
+        const int m = tid % BM, kq = tid / BM;
+        a_voff0 = (a_active && m0 + m < a.M) ? (uint32_t)(((g * a.M + m0 + m) * a.K + 4 * kq) * 4) : kOutOfRange;
+    }
 
     // Two register sets for staged tiles: tile kt+2 is being fetched from memory
     // into one set while tile kt+1 moves from the other set into LDS and tile kt
@@ -287,11 +296,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         constexpr int S = decltype(set)::value;
         constexpr int Q = decltype(slice_q)::value;
         // tiles fetched past the end of K are never multiplied: re-read the last tile
-        const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
+        const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_step;
 #pragma unroll
         for (int j = 0; j < A_LD; j++)
             if (j % (BK / 2) == Q)
-                ra[S][j] = buf_load4(wr, a_active ? (uint32_t)(tid * 16 + j * kThreads * 16) : kOutOfRange, a_soff);
+                ra[S][j] = buf_load4(wr, j == 0 ? a_voff0 : (a_active ? (uint32_t)(tid * 16 + j * kThreads * 16) : kOutOfRange), a_soff);
         if (ORDER == GEMM_ORDER_TAP) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
@@ -330,8 +339,14 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         for (int j = 0; j < A_LD; j++)
             if (j % (BK / 2) == Q) {
                 const int idx = (tid + j * kThreads) * 4; // float index inside the [BK][BM] tile
-                if (a_active)
-                    *(f32x4 *)&As[BUF][idx / BM][idx % BM] = ra[S][j];
+                if (a_active) {
+                    if (A_LD == 1 && wdirect) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            As[BUF][4 * (tid / BM) + e][tid % BM] = ra[S][j][e];
+                    } else
+                        *(f32x4 *)&As[BUF][idx / BM][idx % BM] = ra[S][j];
+                }
             }
 #pragma unroll
         for (int i = 0; i < B_LD; i++)
@@ -2337,6 +2352,9 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
     }
     p.tile = tile_choice(p.M);
+    // 1x1 convolutions in the tap-major order: a K tile is 16 consecutive input channels of the filter rows, which the
+    // kernel reads from the weight tensor in place (when it is 16-byte aligned): nothing is packed
+    p.wdirect = g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && g.KH == 1 && g.KW == 1;
     // stride-1 3x3 "same" convolutions whose 64-pixel patch fits the LDS rows (W <= 62): LDS-patch kernel
     p.patch = g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && p.tile == 0 && g.KH == 3 && g.KW == 3 && g.sh == 1 && g.sw == 1 &&
               g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 && g.H * g.W >= 32 && 64 + 2 * (g.W + 1) < kPatchPitch;
@@ -2453,8 +2471,11 @@ __global__ __launch_bounds__(256) void clear_counters_kernel(int *p, int n)
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
                            size_t part_bytes, int mode)
 {
-    if (p.wdirect && ((uintptr_t)w & 15) == 0)
-        return DLP_OK; // conv_gemm_launch reads w in place
+    if (p.wdirect && ((uintptr_t)w & 15) == 0) { // conv_gemm_launch reads w in place: only the counters are left to do
+        if (mode == GEMM_PACK_ONLY || bf16_mfma_order(p.order))
+            return DLP_OK;
+        mode = GEMM_CLEAR_ONLY;
+    }
     if (p.stem)
         return DLP_OK; // conv_stem_f32_kernel reads w in place and keeps no counters
     int *zero = nullptr; // tile counters of the stream-K launch that follows
