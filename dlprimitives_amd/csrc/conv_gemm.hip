@@ -460,6 +460,8 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
         __syncthreads(); // lds is reused by the epilogue
         if (arrived != splitk - 1)
             return;
+        if (tid == 0)
+            a.sk_cnt[tile] = 0; // left at zero for the next launch (counters that the operator owns are cleared only once)
 #pragma unroll
         for (int r = 0; r < 16; r++)
             acc[0][0][r] = 0.0f;
@@ -898,6 +900,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         const int j_first = (int)(((ut0 + 1) * G - 1) / U), j_last = (int)(((ut0 + ncb) * G - 1) / U);
         output = arrived == j_last - j_first;
         if (output) {
+            if (tid == 0)
+                a.sk_cnt[tile] = 0; // left at zero for the next launch (counters that the operator owns are cleared only once)
 #pragma unroll
             for (int r = 0; r < 16; r++)
                 acc[0][0][r] = 0.0f;
@@ -2246,7 +2250,7 @@ PatchShape patch_shape(const ConvGeom &g, const GemmPlan &p, long long N)
     return ps;
 }
 
-int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t stream, void *part_ws, size_t part_bytes)
+int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t stream, void *part_ws, size_t part_bytes, int *own_counters)
 {
     a.mtiles = p.mtiles;
     a.ntiles = (a.N + p.BN - 1) / p.BN;
@@ -2261,7 +2265,7 @@ int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t 
     int grid = ps.grid;
     // same test as in conv_gemm_pack_weights, which clears the counters
     if (part_ws != nullptr && part_bytes >= patch_shape(g, p, (long long)g.B * g.OH * g.OW).ws_bytes && part_bytes >= ps.ws_bytes) {
-        a.sk_cnt = (int *)part_ws; // zeroed by conv_gemm_pack_weights, which is handed the same workspace
+        a.sk_cnt = own_counters ? own_counters : (int *)part_ws; // zeroed by conv_gemm_pack_weights, which is handed the same workspace
         a.sk_part = (float *)((char *)part_ws + ps.cnt_bytes);
         a.sk_part_bytes = (uint32_t)(ps.ws_bytes - ps.cnt_bytes);
     } else { // no room for pieces: one whole tile per workgroup
@@ -2469,7 +2473,7 @@ __global__ __launch_bounds__(256) void clear_counters_kernel(int *p, int n)
 } // namespace
 
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream, void *part_ws,
-                           size_t part_bytes, int mode)
+                           size_t part_bytes, int mode, bool counters_owned)
 {
     if (p.wdirect && ((uintptr_t)w & 15) == 0) { // conv_gemm_launch reads w in place: only the counters are left to do
         if (mode == GEMM_PACK_ONLY || bf16_mfma_order(p.order))
@@ -2497,6 +2501,10 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
             zero = (int *)part_ws;
             nzero = (int)((long long)a.mtiles * a.ntiles * g.groups);
         }
+    }
+    if (counters_owned) { // the kernels leave the operator's own counters at zero
+        zero = nullptr;
+        nzero = 0;
     }
     if (mode == GEMM_CLEAR_ONLY) { // the weights were packed earlier: only the counters of the coming launch
         if (zero != nullptr) {
@@ -2536,8 +2544,17 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
     return DLP_OK;
 }
 
+size_t conv_gemm_counter_count(const ConvGeom &g, const GemmPlan &p)
+{
+    if (g.B <= 0 || bf16_mfma_order(p.order) || p.stem)
+        return 0;
+    const long long N = (long long)g.B * g.OH * g.OW;
+    return (size_t)((long long)p.mtiles * ((N + p.BN - 1) / p.BN) * g.groups);
+}
+
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
-                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes, const void *w)
+                     void *y, const Epilogue &ep, hipStream_t stream, int n_valid, void *part_ws, size_t part_bytes, const void *w,
+                     int *own_counters)
 {
     if (g.dtype != DLP_FLOAT && g.dtype != DLP_BFLOAT16)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "implicit-GEMM convolution: float_data and bfloat16_data are implemented");
@@ -2605,7 +2622,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         a.clamp_hi = 6.0f;
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
     if (p.patch)
-        return launch_patch(g, p, a, stream, part_ws, part_bytes);
+        return launch_patch(g, p, a, stream, part_ws, part_bytes, own_counters);
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
     a.sk_cnt = nullptr;
     a.part_bytes = 0;
@@ -2615,7 +2632,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         const size_t images = split_total_bytes(p, a, g.groups) - split_counter_bytes(tiles);
         if (images >= kOutOfRange)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K workspace of 2 GiB or more");
-        a.sk_cnt = (int *)part_ws;
+        a.sk_cnt = own_counters ? own_counters : (int *)part_ws;
         a.sk_part = (float *)((char *)part_ws + split_counter_bytes(tiles));
         a.sk_part_bytes = (uint32_t)images;
     } else if (a.splitk > 1) {

@@ -79,7 +79,27 @@ struct dlp_conv2d_fwd {
     size_t workspace;
     int packed_layout[6]; // of the last dlp_conv2d_fwd_pack: order, BM, K tiles, m tiles, patch, in-place
     int accumulate_first; // y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)
+    int *counters;        // GEMM stage: tile counters of split-K / stream-K launches, zero between launches
+    size_t counter_count;
 };
+
+// The operator's own tile counters, enough for this batch (they only ever grow; a larger batch than any before
+// allocates anew, which waits for the kernels that use the old ones).
+static int own_counters(dlp_conv2d_fwd *op, const ConvGeom &g, const GemmPlan &plan, int **out)
+{
+    const size_t need = conv_gemm_counter_count(g, plan);
+    if (need > op->counter_count) {
+        if (op->counters)
+            (void)hipFree(op->counters);
+        op->counters = nullptr;
+        op->counter_count = 0;
+        DLP_HIP_TRY(hipMalloc((void **)&op->counters, need * sizeof(int)));
+        DLP_HIP_TRY(hipMemset(op->counters, 0, need * sizeof(int)));
+        op->counter_count = need;
+    }
+    *out = op->counters;
+    return DLP_OK;
+}
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 
@@ -393,11 +413,16 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     for (int i = 0; i < 6; i++)
         op->packed_layout[i] = -1;
     op->accumulate_first = 0;
+    op->counters = nullptr;
+    op->counter_count = 0;
     if (hipGetDevice(&op->device) != hipSuccess)
         op->device = 0;
     if (chosen == ALGO_GEMM) {
         op->workspace = conv_gemm_workspace_bytes(g, activation);
         rc = upload_ktab(g, activation, &op->ktab);
+        int *unused = nullptr;
+        if (rc == DLP_OK) // counters for the batch of the hint, so that a first call inside a stream capture allocates nothing
+            rc = own_counters(op, g, conv_gemm_plan(g, activation), &unused);
     } else if (chosen == ALGO_WINOGRAD) {
         op->wino = winograd_plan(g);
         op->workspace = op->wino.ws_bytes;
@@ -461,10 +486,14 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
         DLP_REQUIRE(ws != nullptr && ws_bytes >= plan.wpack_bytes, "workspace smaller than workspace()");
         const size_t used = round256(plan.wpack_bytes);
         void *part = ws_bytes > used ? (char *)ws + used : nullptr;
-        rc = conv_gemm_pack_weights(g, plan, w, ws, s, part, part ? ws_bytes - used : 0);
+        int *counters = nullptr;
+        rc = own_counters(op, g, plan, &counters);
         if (rc != DLP_OK)
             return rc;
-        return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0, w);
+        rc = conv_gemm_pack_weights(g, plan, w, ws, s, part, part ? ws_bytes - used : 0, GEMM_PACK_AND_CLEAR, true);
+        if (rc != DLP_OK)
+            return rc;
+        return conv_gemm_launch(g, plan, op->ktab, x, ws, y, ep, s, -1, part, part ? ws_bytes - used : 0, w, counters);
     }
     }
 }
@@ -557,10 +586,11 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
             DLP_REQUIRE(sig[i] == op->packed_layout[i], "the weights were packed for another tile plan (pack again for this batch)");
         DLP_REQUIRE(packed != nullptr, "null buffer of packed weights");
         void *part = ws_bytes > 0 ? ws : nullptr;
-        rc = conv_gemm_pack_weights(g, plan, w, const_cast<void *>(packed), s, part, ws_bytes, GEMM_CLEAR_ONLY);
+        int *counters = nullptr;
+        rc = own_counters(op, g, plan, &counters);
         if (rc != DLP_OK)
             return rc;
-        return conv_gemm_launch(g, plan, op->ktab, x, packed, y, ep, s, -1, part, ws_bytes, w);
+        return conv_gemm_launch(g, plan, op->ktab, x, packed, y, ep, s, -1, part, ws_bytes, w, counters);
     }
     }
 }
@@ -571,6 +601,8 @@ void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op)
         return;
     if (op->ktab)
         (void)hipFree(op->ktab);
+    if (op->counters)
+        (void)hipFree(op->counters);
     delete op;
 }
 

@@ -181,14 +181,19 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation);
 // (the packing kernel clears the counters the launch keeps there).
 // mode: both steps, the packing alone (weights that stay constant are packed once), or the counters alone.
 enum { GEMM_PACK_AND_CLEAR = 0, GEMM_PACK_ONLY = 1, GEMM_CLEAR_ONLY = 2 };
+// counters_owned: conv_gemm_launch will be given counters of the operator's own (see there): none are cleared here.
 int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, void *wpacked, hipStream_t stream,
-                           void *part_ws = nullptr, size_t part_bytes = 0, int mode = GEMM_PACK_AND_CLEAR);
+                           void *part_ws = nullptr, size_t part_bytes = 0, int mode = GEMM_PACK_AND_CLEAR, bool counters_owned = false);
+// Tile counters a launch at this batch may use (0: none).  A caller that keeps that many zeroed ints per operator and
+// hands them to conv_gemm_launch as own_counters saves the clearing before every launch: the kernels leave them at zero.
+// Such an operator must not run on two streams at once.
+size_t conv_gemm_counter_count(const ConvGeom &g, const GemmPlan &p);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 // part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.
 // w: the weight tensor as the caller gave it (plans with wdirect read it in place when it is 16-byte aligned).
 int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_ktab, const void *x, const void *wpacked,
                      void *y, const Epilogue &ep, hipStream_t stream, int n_valid = -1, void *part_ws = nullptr,
-                     size_t part_bytes = 0, const void *w = nullptr);
+                     size_t part_bytes = 0, const void *w = nullptr, int *own_counters = nullptr);
 
 // ---- few-channel strided stem convolution (conv_stem.hip) ----------------------
 bool conv_stem_supported(const ConvGeom &g);
