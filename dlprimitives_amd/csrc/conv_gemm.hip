@@ -2476,9 +2476,12 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                            size_t part_bytes, int mode, bool counters_owned)
 {
     if (p.wdirect && ((uintptr_t)w & 15) == 0) { // conv_gemm_launch reads w in place: only the counters are left to do
-        if (mode == GEMM_PACK_ONLY || bf16_mfma_order(p.order))
+        if (bf16_mfma_order(p.order))
             return DLP_OK;
-        mode = GEMM_CLEAR_ONLY;
+        // fp32: weights packed once ahead of time are still the faster operand (one 16-byte LDS store per thread and
+        // K tile instead of four); reading in place only saves the packing launch of a call that would pack every time
+        if (mode != GEMM_PACK_ONLY)
+            mode = GEMM_CLEAR_ONLY;
     }
     if (p.stem)
         return DLP_OK; // conv_stem_f32_kernel reads w in place and keeps no counters
