@@ -128,7 +128,11 @@ size_t dlp_conv2d_fwd_workspace(const dlp_conv2d_fwd *op);
  * x [B,Cin,H,W], w [Cout,Cin/groups,KH,KW], bias [Cout] or NULL (must match the
  * `bias` flag given at create), y [B,Cout,OH,OW]; ws >= workspace() bytes;
  * y = factor != 0 ? factor*y + act(conv+bias) : act(conv+bias).
- * Asynchronous on `stream` (a hipStream_t, NULL = default stream). */
+ * Asynchronous on `stream` (a hipStream_t, NULL = default stream).  The operator keeps
+ * small device buffers of its own (tile counters that its kernels leave at zero), as the
+ * reference's operators keep their kernels and buffers: do not enqueue one operator on two
+ * streams at the same time.  A batch larger than the one in the shape given at create
+ * allocates here. */
 int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4],
                            const void *x, const void *w, const void *bias, void *y,
                            void *ws, size_t ws_bytes, float factor, void *stream);
