@@ -79,6 +79,10 @@ struct GemmArgs {
 #endif
     int *sk_cnt;              // pieces arrived, per tile (zero at launch)
     int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
+    int sk_tiles;             // tiles of the stream (sk_units / stages per tile)
+    // divisions of the per-tile decode, as magic numbers (fast_div): they are uniform, and a uniform integer division
+    // would otherwise run as some forty vector instructions in every wavefront, next to the matrix instructions
+    uint32_t ncb_magic, ncb_shift, nt_magic, nt_shift, tpw_magic, tpw_shift, pg_magic, pg_shift, mbnt_magic, mbnt_shift, mb_magic, mb_shift;
     int pxv;                  // bf16 matrix-instruction kernels: pixels per output store (0 = one element per store)
     int pp_nbr;               // conv_patch_bf16_kernel: blocks of PXP rows in the largest patch of the launch
     int wdirect;              // conv_gemm_bf16_kernel: wp is the weight tensor itself (1x1 convolution), not packed tiles
@@ -664,7 +668,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
 
     for (int u = u_begin; u < u_end;) {
-    int t = u / ncb; // tile: m tile fastest, then n tile, then group
+    int t = (int)fast_div((uint32_t)u, a.ncb_magic, a.ncb_shift); // u / ncb; tile: m tile fastest, then n tile, then group
     const int tile = t;
     const int cb_begin = u - t * ncb;
     const int cb_end = min(ncb, cb_begin + (u_end - u));
@@ -676,8 +680,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     // sk_mb m tiles of one pixel tile, then the next pixel tile: an XCD's share covers few m tiles
     // (little of the weights) and a compact range of pixels.
     {
-        const int NT = (int)(U / (uint64_t)ncb);
-        int c = (int)(((int64_t)t * 8) / NT);
+        const int NT = a.sk_tiles;
+        int c = (int)fast_div((uint32_t)t * 8u, a.nt_magic, a.nt_shift); // 8 t / NT (NT < 2^27: y is below 2 GiB)
         int lo = (int)(((int64_t)c * NT) / 8), hi = (int)(((int64_t)(c + 1) * NT) / 8);
         if (t >= hi) {
             c++;
@@ -685,18 +689,18 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
             hi = (int)(((int64_t)(c + 1) * NT) / 8);
         }
         const int L = hi - lo, i = t - lo;
-        const int q = L / a.sk_tpw, r = L - q * a.sk_tpw;
-        const int col = i / a.sk_tpw, row = i - col * a.sk_tpw;
+        const int q = (int)fast_div((uint32_t)L, a.tpw_magic, a.tpw_shift), r = L - q * a.sk_tpw;
+        const int col = (int)fast_div((uint32_t)i, a.tpw_magic, a.tpw_shift), row = i - col * a.sk_tpw;
         // rows 0..r-1 of the ragged L = q*tpw + r layout hold q+1 tiles, the others q; a column index
         // past a short row's end only happens in the last (partial) column, which holds rows < r
         t = lo + row * q + min(row, r) + col;
     }
     const int per_group = a.mtiles * a.ntiles;
-    const int g = t / per_group;
+    const int g = (int)fast_div((uint32_t)t, a.pg_magic, a.pg_shift);
     t -= g * per_group;
-    const int mblk = t / (a.sk_mb * a.ntiles);
+    const int mblk = (int)fast_div((uint32_t)t, a.mbnt_magic, a.mbnt_shift);
     t -= mblk * a.sk_mb * a.ntiles;
-    const int nt = t / a.sk_mb;
+    const int nt = (int)fast_div((uint32_t)t, a.mb_magic, a.mb_shift);
     const int mt = mblk * a.sk_mb + (t - nt * a.sk_mb);
     const int m0 = mt * BM, n0 = nt * BN;
 
@@ -2292,6 +2296,13 @@ int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t 
             }
         }
     }
+    make_magic((uint32_t)(a.nkt / 9), a.ncb_magic, a.ncb_shift);
+    a.sk_tiles = (int)ps.tiles;
+    make_magic((uint32_t)ps.tiles, a.nt_magic, a.nt_shift);
+    make_magic((uint32_t)a.sk_tpw, a.tpw_magic, a.tpw_shift);
+    make_magic((uint32_t)(a.mtiles * a.ntiles), a.pg_magic, a.pg_shift);
+    make_magic((uint32_t)(a.sk_mb * a.ntiles), a.mbnt_magic, a.mbnt_shift);
+    make_magic((uint32_t)a.sk_mb, a.mb_magic, a.mb_shift);
 #ifdef DLP_PATCH_TRACE
     a.trace = (part_ws != nullptr && part_bytes >= ps.ws_bytes + (size_t)grid * 32 + (1u << 20)) ? (long long *)((char *)part_ws + part_bytes - (1u << 20)) : nullptr;
 #endif
