@@ -107,6 +107,7 @@ def lib():
         L.dlp_ip_fwd_create.argtypes = [ctypes.POINTER(_IPSettings), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
         L.dlp_ip_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                          ctypes.c_void_p, ctypes.c_void_p]
+        L.dlp_ip_fwd_enqueue_no_alloc.argtypes = L.dlp_ip_fwd_enqueue.argtypes
         L.dlp_ip_fwd_destroy.argtypes = [ctypes.c_void_p]
         L.dlp_ip_fwd_destroy.restype = None
         _lib = L
@@ -345,6 +346,10 @@ class IPForward:
 
     def enqueue(self, x, w, bias, y, stream=None):
         _check(lib().dlp_ip_fwd_enqueue(self._h, int(x.shape[0]), _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _stream(stream)))
+
+    def enqueue_no_alloc(self, x, w, bias, y, stream=None):
+        """enqueue() with its scratch in the library's own device array: no device allocation, bounded sizes"""
+        _check(lib().dlp_ip_fwd_enqueue_no_alloc(self._h, int(x.shape[0]), _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _stream(stream)))
 
     def __del__(self):
         if getattr(self, "_h", None):

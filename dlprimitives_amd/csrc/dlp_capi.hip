@@ -175,6 +175,46 @@ static int make_geom(const dlp_conv2d_settings &c, const int x_shape[4], ConvGeo
     return DLP_OK;
 }
 
+// ---- the entry point that allocates nothing ----------------------------------------------------------------
+// The tile counters and K-slice partial sums of ip_direct_kernel live in a device array of this library instead of
+// an op-owned hipMalloc buffer.  Every device the library runs on holds its own copy of the array until the process
+// ends; host code must never hand the array's name to a kernel (on the host it is a stand-in, not a device address):
+// the address on the current device comes from hipGetSymbolAddress, once per device, and is kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[DLP_IP_NO_ALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+constexpr size_t kNoAllocCounterBytes = 64 * 1024; // front of the array: tile counters; the rest: partial sums
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];
+
+// address of `scratch` on the current device (looked up on first use, with that device current)
+int scratch_on_current_device(void **out)
+{
+    int device = -1;
+    DLP_HIP_TRY(hipGetDevice(&device));
+    DLP_REQUIRE(device >= 0 && device < kMaxDevices, "device index beyond the table of scratch addresses");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        DLP_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr)
+            return fail(DLP_ERR_RUNTIME, "hipGetSymbolAddress gave no address for the scratch array");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return DLP_OK;
+}
+
+// a fill kernel, not hipMemsetAsync: the call may be recorded into a HIP graph
+__global__ void clear_ints_kernel(int *p, int n)
+{
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i < n)
+        p[i] = 0;
+}
+} // namespace
+
 extern "C" {
 
 const char *dlp_last_error(void) { return g_last_error.c_str(); }
@@ -632,6 +672,10 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
     op->scratch = nullptr;
     op->scratch_bytes = op->scratch_cnt_bytes = 0;
     int rc = upload_ktab(g1, activation, &op->ktab);
+    if (rc == DLP_OK) { // set-up of dlp_ip_fwd_enqueue_no_alloc on this device, so that its first call may sit inside a stream capture
+        void *unused = nullptr;
+        rc = scratch_on_current_device(&unused);
+    }
     if (rc == DLP_OK && hipMalloc(&op->wpacked, op->plan.wpack_bytes) != hipSuccess)
         rc = fail(DLP_ERR_RUNTIME, "hipMalloc(packed weights) failed");
     if (rc != DLP_OK) {
@@ -683,6 +727,44 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
     if (rc != DLP_OK)
         return rc;
     return conv_gemm_launch(g, op->plan, op->ktab, x, op->wpacked, y, ep, (hipStream_t)stream, -1, nullptr, 0, w);
+}
+
+int dlp_ip_fwd_enqueue_no_alloc(dlp_ip_fwd *op, int batch, const void *x, const void *w, const void *bias, void *y, void *stream)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    DLP_REQUIRE(batch >= 0, "negative batch");
+    DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
+    if (batch == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && w != nullptr && y != nullptr, "null tensor pointer");
+    if (!ip_direct_supported(op->cfg.inputs, op->cfg.dtype, x, w))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "dlp_ip_fwd_enqueue_no_alloc: bfloat16 rows must have an even length and dword-aligned tensors");
+    IpPlan ip;
+    ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
+    // (an unsplit K uses neither counters nor partial sums)
+    if (ip.S > 1 && (ip.cnt_bytes > kNoAllocCounterBytes || ip.part_bytes > (size_t)DLP_IP_NO_ALLOC_SCRATCH_BYTES - kNoAllocCounterBytes))
+        return fail(DLP_ERR_VALIDATION, "dlp_ip_fwd_enqueue_no_alloc: this batch x outputs needs " + std::to_string(ip.cnt_bytes) + " + " +
+                                            std::to_string(ip.part_bytes) + " bytes of scratch, the library's array holds " +
+                                            std::to_string(kNoAllocCounterBytes) + " + " +
+                                            std::to_string((size_t)DLP_IP_NO_ALLOC_SCRATCH_BYTES - kNoAllocCounterBytes) +
+                                            " (use dlp_ip_fwd_enqueue)");
+    void *base = nullptr;
+    int rc = scratch_on_current_device(&base);
+    if (rc != DLP_OK)
+        return rc;
+    Epilogue ep;
+    ep.bias = (const float *)bias;
+    ep.factor = 0.0f;
+    ep.activation = op->activation;
+    int *counters = (int *)base;
+    float *partials = (float *)((char *)base + kNoAllocCounterBytes);
+    if (ip.S > 1) {
+        // the array keeps what the last call left: the counters of this launch start from zero whatever that was
+        const int n = ip.mblocks * ip.nchunks;
+        hipLaunchKernelGGL(clear_ints_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, counters, n);
+        DLP_HIP_TRY(hipGetLastError());
+    }
+    return ip_direct_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, counters, partials, (hipStream_t)stream);
 }
 
 void dlp_ip_fwd_destroy(dlp_ip_fwd *op)

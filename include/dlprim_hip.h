@@ -204,6 +204,21 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w,
                        const void *bias, void *y, void *stream);
 void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
 
+/* dlp_ip_fwd_enqueue for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same
+ * result bit for bit; the tile counters and K-slice partial sums that dlp_ip_fwd_enqueue keeps in a buffer
+ * the operator allocates (and regrows for a larger batch) live here in one array of
+ * DLP_IP_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends.
+ * The call makes no hipMalloc / hipFree and records no memset.  The array holds 64 KiB of tile counters and
+ * 4 MiB of partial sums (4 KiB per tile of 32 outputs x 32 batch rows and K slice): enough for 2048 -> 1000 at
+ * batch 128 (3.5 MiB) or 25088 -> 4096 at batch 16 (4 MiB).  A batch x outputs that needs more is a validation
+ * error that names both sizes (e.g. 1024 -> 4096 at batch 160: 5 MiB); bfloat16 rows of odd length are
+ * NotImplemented.  All calls on one device share the array: two calls that overlap on one device (different
+ * streams, or two threads) race; calls on one stream do not. */
+#define DLP_IP_NO_ALLOC_SCRATCH_BYTES (4 * 1024 * 1024 + 64 * 1024)
+int dlp_ip_fwd_enqueue_no_alloc(dlp_ip_fwd *op, int batch, const void *x, const void *w,
+                                const void *bias, void *y, void *stream);
+
 /* ===== glue operators around the convolution path (forward only) ================= */
 
 typedef struct dlp_pool2d_fwd dlp_pool2d_fwd; /* core::Pooling2DForward object */
