@@ -9,12 +9,20 @@ stream, with every tensor already resident in HBM.  Synthetic data: inputs
 uniform[-1,1], weights Kaiming-normal, bias uniform[-0.1,0.1], fixed seed.
 
 Other workloads (same JSON contract, for the remaining configurations):
+  --workload single         one 3x3 64->64 convolution at 56x56 (configuration 1 with --batch 16)
   --workload mobilenet      depthwise 3x3 stride 1/2 (HBM bound) + 1x1 pointwise, ReLU6
   --workload winograd       the two Winograd shapes, algo winograd
   --workload winograd-gemm  the same two shapes through the implicit GEMM
   --workload resnet18-full / resnet50-full   whole network forward incl. pooling, adds, GAP, IP
   --workload resnet18-backward   gradients of the 20 ResNet-18 convolutions (backward filter for all,
                             backward data for all but conv1, whose input needs none), fp32
+
+The default run (no flags) also carries a `configs` object: the other four configurations of the baseline
+(single layer at batch 16; the two Winograd shapes through "winograd" and through "gemm"; the MobileNet blocks with
+every depthwise layer scored against 8 TB/s and against a plain streaming kernel on tensors of the same size;
+the whole ResNet-50 forward in bf16 storage at batch 128), each with ms_per_step, its dominant kernel and that
+kernel's roofline fraction, plus `measured_peak` (MFMA-only loops and streaming copies run on this device) next
+to `vendor_peak`.  Kernel names come from the library's timing records (dlp_timing_get_kernel), not from this file.
 
 Prints ONE JSON line.  `value` = images/s of the whole workload; `gflops_per_s` is
 the same run expressed with the reference's flop accounting (tools/flops.cpp:660).
@@ -38,21 +46,43 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3
 BF16_MATRIX_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 BASELINE_METRIC = "conv2d fwd GFLOP/s + % of MI355X roofline; ResNet-18 b64 images/sec"
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
 
-# HBM bytes per launch of the dominant kernel of each workload at batch 64, from hardware
-# counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, one counter per run, KiB per dispatch,
-# scaled by what the same counter reads for a plain copy of known size: x2.0 / x1.0).
-# Measured offline (a benchmark run cannot collect counters on itself); keyed by (workload, kernel).
-MEASURED_TRAFFIC_BYTES = {
-    ("resnet18", "conv_patch_f32_kernel<float, 3, 3, 192, 0>"): (32886.5 * 2.0 + 46377.9) * 1024,
-    ("winograd", "wino_fused_kernel<float, ...>"): ((16817.5 + 40712.4) / 2 * 2.0 + (25377.0 + 12838.6) / 2) * 1024,
-    ("mobilenet", "depthwise3x3_kernel<float, 1>"): (27364.9 * 2.0 + 45795.7) * 1024,
-}
+
+def measured_traffic_bytes(workload, kernel):
+    """HBM bytes per launch of `kernel` in `workload` at batch 64, from the hardware-counter summary kept under
+    profiles/ (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, one counter per run, KiB per dispatch; a benchmark run
+    cannot collect counters on itself).  Each counter is scaled by what it reads for the copy kernel of known size in
+    the same file.  None when the file has no row for this kernel: a renamed or new kernel has no stale number."""
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+    except OSError:
+        return None
+    section, rows = None, {}
+    for ln in lines:
+        if ln.startswith("== "):
+            section = ln[3:].split()[0]
+            continue
+        if section and " n=" in ln and "FETCH_SIZE" in ln and "WRITE_SIZE" in ln:
+            name = ln[:ln.index(" n=")].strip()
+            t = ln.split()
+            rows.setdefault(section, []).append((name, float(t[t.index("FETCH_SIZE") + 1]), float(t[t.index("WRITE_SIZE") + 1])))
+    copy = [r for r in rows.get("copy", []) if r[0].startswith("copy_f4")]
+    if not copy or copy[0][1] <= 0 or copy[0][2] <= 0:
+        return None
+    copied_kib = 262144.0  # the calibration run copies 256 MiB per launch
+    fetch_scale, write_scale = copied_kib / copy[0][1], copied_kib / copy[0][2]
+    for (name, fetch, write) in rows.get(workload, []):
+        if kernel == name or (len(name) >= 50 and kernel.startswith(name)):  # (older summaries cut names at 50 characters)
+            return (fetch * fetch_scale + write * write_scale) * 1024
+    return None
 
 
 def workload_layers(name):
     from dlprimitives_amd.workloads import MOBILENET_DEPTHWISE, MOBILENET_POINTWISE, RESNET18_CONVS, WINOGRAD_SHAPES, conv
 
+    if name == "single":
+        return [dict(conv("3x3_64to64_at56", 3, 1, 1, 64, 64, 56), algo="gemm")], "single Conv2D 3x3 s1 p1 64->64 at 56x56, bias + ReLU, algo gemm"
     if name == "resnet18":
         return [dict(L, algo="gemm") for L in RESNET18_CONVS], "ResNet-18 conv stack forward: 20 convs, BN folded, fused ReLU, algo gemm"
     if name == "resnet50":
@@ -103,39 +133,6 @@ def build_layers(layer_list, batch, seed, bf16=False):
     return out
 
 
-def kernel_class(L, bf16=False):
-    """Name of the kernel that does the layer's arithmetic, as a profiler lists it."""
-    if L["algo"] == "depthwise_separable":
-        return "depthwise3x3_kernel<%s, %d>" % ("bf16_t" if bf16 else "float", L["stride"])
-    cin_g = L["cin"] // L["groups"]
-    m = L["cout"] // L["groups"]
-    if L["algo"] == "winograd":
-        return "wino_fused_kernel<%s, ...>" % ("bf16_t" if bf16 else "float")
-    small = L["kernel"] ** 2 <= 31
-    if bf16 and L["activation"] not in ("tanh", "sigmoid"):
-        order = 2 if (small and cin_g % 32 == 0) else 3  # one tap x 32 channels per K tile, or the per-element table
-        tile = "128, 128, 2, 2" if m > 64 else "64, 256, 1, 4"
-        hw = L["hw"] * L["hw"]
-        same3 = L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
-        if order == 2 and same3 and hw % 4 == 0 and hw >= (128 if m > 64 else 254):
-            # stride-1 3x3: input patch through LDS (the library falls back to the gather when the patch does not fit)
-            return "conv_patch_bf16_kernel<%s, %d, %d, 0>" % (tile, 320 if m > 64 else 448, 8 if hw % 8 == 0 else 4)
-        pxl = 0
-        if order == 2 and L["kernel"] == 1 and L["stride"] == 1 and L["pad"] == 0 and hw % 4 == 0:
-            pxl = 8 if hw % 8 == 0 else 4  # dense loader: 8 or 4 pixels per load
-        return "conv_gemm_bf16_kernel<%s, %d, 0, 2, %d>" % (tile, order, pxl)
-    if (not bf16 and L["groups"] == 1 and L["cin"] == 3 and L["kernel"] == 7 and L["stride"] == 2 and L["pad"] <= 4 and m % 8 == 0
-            and L["hw"] <= 232 and L.get("dilate", 1) == 1):
-        return "conv_stem_f32_kernel<3, 7, 7, 2, 8, 240, true, false>"  # input rows of a band and the filter in LDS, no gather
-    tile = "64, 64, 2, 2" if m > 32 else "32, 128, 1, 4"
-    order = 1 if (small and cin_g % 16 == 0) else 0
-    if (not bf16 and order == 1 and m > 32 and L["kernel"] == 3 and L["stride"] == 1 and L["pad"] == 1 and L.get("dilate", 1) == 1
-            and L["hw"] * L["hw"] >= 32 and 64 + 2 * (L["hw"] + 1) < 192 and L["activation"] not in ("tanh", "sigmoid")):
-        return "conv_patch_f32_kernel<float, 3, 3, 192, 0>"  # stride-1 3x3: input patch through LDS, stream-K
-    mask = 1 if small else 2
-    return "conv_gemm_f32_kernel<%s, %s, %d, %d, 0>" % ("bf16_t" if bf16 else "float", tile, order, mask)
-
-
 def matrix_peak_tflops(kernel_name):
     return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith(("conv_gemm_bf16_kernel", "conv_patch_bf16_kernel")) else FP32_MATRIX_PEAK_TFLOPS
 
@@ -171,6 +168,10 @@ def cpu_baseline(layer_list, images, seed, threads=1):
 
 
 def run_graph_workload(args):
+    return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup)
+
+
+def graph_workload(net, batch, algo, bf16, steps, warmup):
     """Whole-network forward (convolutions + pooling + residual adds + global pooling + inner
     product) through the C-ABI operators; same JSON contract, no per-kernel roofline split."""
     import torch
@@ -178,50 +179,51 @@ def run_graph_workload(args):
     import dlprimitives_amd as dlp
     from dlprimitives_amd import graphs
 
-    net = args.workload[:-len("-full")]
     ops = getattr(graphs, net)()
     params = graphs.random_parameters(ops, 2024)
-    shape = (args.batch, 3, 224, 224)
-    bf16 = args.dtype == "bf16"
-    runner = graphs.GraphRunner(ops, params, shape, algo=args.algo, dtype="bfloat16" if bf16 else "float32")
+    shape = (batch, 3, 224, 224)
+    runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32")
     x = torch.rand(shape, device="cuda:0") * 2 - 1
     runner.t["data"].copy_(x)  # converts to the storage type
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         runner.forward()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         runner.forward()
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     dlp.timing_reset()
     dlp.timing_enable(True)
     runner.forward()
     torch.cuda.synchronize()
     dlp.timing_enable(False)
-    sections = {}
-    for (section, ms) in dlp.timing_records():
+    sections, by_kernel = {}, {}
+    for (section, ms, kname) in dlp.timing_records(kernels=True):
         sections[section] = round(sections.get(section, 0.0) + ms, 4)
+        if section in ("conv_gemm", "winograd_fused"):
+            by_kernel[kname] = by_kernel.get(kname, 0.0) + ms
     dlp.timing_reset()
     flops = runner.flops()
     conv_ms = sections.get("conv_gemm", 0.0) + sections.get("winograd_fused", 0.0)
-    out = {
-        "metric": BASELINE_METRIC, "value": round(args.batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32 arithmetic on bf16-stored tensors" if bf16 else "f32", "data": "synthetic",
+    peak = BF16_MATRIX_PEAK_TFLOPS if bf16 else FP32_MATRIX_PEAK_TFLOPS
+    dominant = max(by_kernel.items(), key=lambda kv: kv[1])[0] if by_kernel else ""
+    return {
+        "metric": BASELINE_METRIC, "value": round(batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds, global avg pool, inner product), "
-                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, "bf16 storage" if bf16 else "fp32", args.batch,
-                                                                                 args.algo or "auto"),
-                   "batch": args.batch, "gflop_per_step": round(flops / 1e9, 1)},
+                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, "bf16 storage" if bf16 else "fp32", batch, algo or "auto"),
+                   "batch": batch, "gflop_per_step": round(flops / 1e9, 1)},
         "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
-        "frac_of_fp32_matrix_peak": round(flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
+        "frac_of_matrix_peak_whole_pass": round(flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
         "kernel_ms_by_section": sections,
-        "roofline": {"bound": "mfma", "kernel": "conv_gemm + wino_fused (all launches of one forward; direct-convolution flops)", "achieved": round(flops / (conv_ms * 1e-3) / 1e12, 2) if conv_ms else None,
-                     "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (conv_ms * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4) if conv_ms else None,
+        "roofline": {"bound": "mfma", "kernel": "all convolution launches of one forward (direct-convolution flops); largest share: " + dominant,
+                     "achieved": round(flops / (conv_ms * 1e-3) / 1e12, 2) if conv_ms else None,
+                     "peak": peak, "unit": "TFLOP/s", "frac": round(flops / (conv_ms * 1e-3) / 1e12 / peak, 4) if conv_ms else None,
                      "traffic": None},
         "cpu_baseline": None,
     }
-    print(json.dumps(out))
 
 
 def run_backward_workload(args):
@@ -288,116 +290,88 @@ def run_backward_workload(args):
     print(json.dumps(out))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "resnet18-full", "resnet50-full", "resnet18-backward"])
-    ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
-    ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
-    ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
-    ap.add_argument("--prepacked", action="store_true",
-                    help="weights transformed once before the timed region (dlp_conv2d_fwd_pack / _enqueue_packed), as an inference "
-                         "deployment does; the default transforms them in every step, as the reference's enqueue contract implies")
-    ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over batch with no exchange)" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
-
+def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, only="", seed=2024):
+    """Times `steps` passes over the layers of a convolution workload (back to back on one stream, tensors resident),
+    then a second pass with the library's per-kernel timing.  Returns the pieces of the JSON line."""
     import torch
 
     import dlprimitives_amd as dlp
 
-    dlp.lib()  # fails loudly when the HIP library is missing
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    torch.cuda.set_device(0)
-    if args.workload.endswith("-full"):
-        run_graph_workload(args)
-        return
-    if args.workload == "resnet18-backward":
-        run_backward_workload(args)
-        return
-    layer_list, description = workload_layers(args.workload)
-    if args.only:
-        layer_list = [L for L in layer_list if args.only in L["name"]]
+    layer_list, description = workload_layers(workload)
+    if only:
+        layer_list = [L for L in layer_list if only in L["name"]]
         if not layer_list:
             print("bench.py: --only matches no layer", file=sys.stderr)
             sys.exit(2)
-    bf16 = args.dtype == "bf16"
-    layers = build_layers(layer_list, args.batch, 2024, bf16)
-    stream = torch.cuda.current_stream()
+    layers = build_layers(layer_list, batch, seed, bf16)
+
+    def enqueue(e):
+        if prepacked:
+            e["op"].enqueue_packed(e["x"], e["w"], e["packed"], e["b"], e["y"], e["ws"], 0.0)
+        else:
+            e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
 
     def step():
-        if args.prepacked:
-            for e in layers:
-                e["op"].enqueue_packed(e["x"], e["w"], e["packed"], e["b"], e["y"], e["ws"], 0.0)
-        else:
-            for e in layers:
-                e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+        for e in layers:
+            enqueue(e)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     total_flops = sum(e["flops"] for e in layers)
     total_bytes = sum(e["bytes"] for e in layers)
 
-    # second pass: the library's own per-kernel timing (a HIP event pair around every
-    # kernel launch, on the launch stream); a layer = its main kernel + helper kernels
+    # second pass: the library's own per-kernel timing (a HIP event pair around every kernel launch, on the launch
+    # stream); a layer = its main kernel + helper kernels.  The records also say which kernel ran.
     nl = len(layers)
     dlp.timing_reset()
     dlp.timing_enable(True)
     spans = []
-    for s in range(args.steps):
+    for _ in range(steps):
         for i, e in enumerate(layers):
             first = dlp.timing_count()
-            if args.prepacked:
-                e["op"].enqueue_packed(e["x"], e["w"], e["packed"], e["b"], e["y"], e["ws"], 0.0)
-            else:
-                e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+            enqueue(e)
             spans.append((i, first, dlp.timing_count()))
     torch.cuda.synchronize()
     dlp.timing_enable(False)
-    records = dlp.timing_records()
+    records = dlp.timing_records(kernels=True)
     layer_ms = [0.0] * nl   # all kernels of the layer
     kernel_ms = [0.0] * nl  # the main kernel only
+    kernel_name = [""] * nl
     for (i, first, last) in spans:
         main = MAIN_SECTION[layers[i]["layer"]["algo"]]
-        for (section, ms) in records[first:last]:
-            layer_ms[i] += ms / args.steps
+        for (section, ms, kname) in records[first:last]:
+            layer_ms[i] += ms / steps
             if section == main:
-                kernel_ms[i] += ms / args.steps
+                kernel_ms[i] += ms / steps
+                kernel_name[i] = kname or section
     dlp.timing_reset()
 
     table = []
     classes = {}
-    for e, ms, kms in zip(layers, layer_ms, kernel_ms):
+    for e, ms, kms, kname in zip(layers, layer_ms, kernel_ms, kernel_name):
         L = e["layer"]
-        kname = kernel_class(L, bf16)
         peak = matrix_peak_tflops(kname) * 1e12
         ai = e["flops"] / e["bytes"]
         mfma_bound = ai * HBM_PEAK_GBS * 1e9 >= peak
         roof = min(peak, ai * HBM_PEAK_GBS * 1e9)
-        ach = e["flops"] / (ms * 1e-3)
-        table.append(dict(name=L["name"], ms=round(ms, 4), main_kernel_ms=round(kms, 4), tflops=round(ach / 1e12, 2), gbs=round(e["bytes"] / (ms * 1e-3) / 1e9, 1),
-                          bound="mfma" if mfma_bound else "hbm", frac_of_roofline=round(ach / roof, 4), kernel=kname))
+        # Winograd F(2x2,3x3) multiplies 16 values per 2x2 outputs instead of 36: against the matrix peak it is scored
+        # on the flops it issues (direct / 2.25), so the fraction cannot pass 100 %; tflops stays direct-equivalent
+        issued = e["flops"] / 2.25 if L["algo"] == "winograd" else e["flops"]
+        row = dict(name=L["name"], ms=round(ms, 4), main_kernel_ms=round(kms, 4), tflops=round(e["flops"] / (ms * 1e-3) / 1e12, 2),
+                   gbs=round(e["bytes"] / (ms * 1e-3) / 1e9, 1), bound="mfma" if mfma_bound else "hbm",
+                   frac_of_roofline=round((issued if mfma_bound else e["flops"]) / (ms * 1e-3) / roof, 4), kernel=kname)
+        if L["algo"] == "winograd":
+            row["tflops_issued"] = round(issued / (ms * 1e-3) / 1e12, 2)
+        table.append(row)
         c = classes.setdefault(kname, dict(ms=0.0, flops=0.0, bytes=0.0, launches=0, hbm=0))
         c["ms"] += kms
-        # Winograd F(2x2,3x3) multiplies 16 values per 2x2 outputs instead of 36: the matrix-core
-        # fraction is scored on the flops actually issued (direct / 2.25), so it cannot pass 100 %
-        c["flops"] += e["flops"] / 2.25 if L["algo"] == "winograd" else e["flops"]
+        c["flops"] += issued
         c["bytes"] += e["bytes"]
         c["launches"] += 1
         c["hbm"] += 0 if mfma_bound else 1
@@ -414,19 +388,123 @@ def main():
                         flops_per_launch=dom["flops"] / dom["launches"], bytes_per_launch=dom["bytes"] / dom["launches"],
                         achieved=round(achieved, 2), peak=peak_tf,
                         unit="TFLOP/s", frac=round(achieved / peak_tf, 4), traffic=None)
-    if args.batch == 64 and not args.only:
-        roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, dom_name))
-    if args.layers:
-        for r in table:
-            print(json.dumps(r), file=sys.stderr)
+    if batch == 64 and not only and not bf16:
+        roofline["traffic"] = measured_traffic_bytes(workload, dom_name)
+    return dict(layer_list=layer_list, description=description, ms_per_step=ms_per_step, total_flops=total_flops, total_bytes=total_bytes,
+                kernel_ms_per_step=sum(layer_ms), roofline=roofline, table=table, nl=nl)
 
-    cpu = cpu_baseline(layer_list, args.cpu_images, 2024) if args.cpu_images > 0 else None  # the fp32 reference path
+
+def compact(r, batch, extra=None):
+    """One configuration as an entry of the `configs` object of the default line."""
+    rf = r["roofline"]
+    out = {"workload": r["description"], "batch": batch, "ms_per_step": round(r["ms_per_step"], 4),
+           "images_per_s": round(batch / (r["ms_per_step"] * 1e-3), 1), "gflops_per_s": round(r["total_flops"] / (r["ms_per_step"] * 1e-3) / 1e9, 1),
+           "kernel": rf["kernel"], "bound": rf["bound"], "achieved": rf["achieved"], "unit": rf["unit"], "frac": rf["frac"]}
+    if extra:
+        out.update(extra)
+    return out
+
+
+def other_configs(steps, warmup, peaks):
+    """Configurations 1, 3, 4 and 5 of the baseline, each through the same timing as the headline (fewer steps)."""
+    import torch
+
+    from dlprimitives_amd import probe
+
+    cfgs = {}
+    r = run_conv_workload("single", 16, False, steps, warmup)
+    cfgs["config1_single_conv_b16"] = compact(r, 16)
+    for wl in ("winograd", "winograd-gemm"):
+        r = run_conv_workload(wl, 64, False, steps, warmup)
+        cfgs["config3_%s" % wl.replace("-", "_")] = compact(r, 64, {"layers": [
+            {k: row[k] for k in ("name", "ms", "main_kernel_ms", "tflops", "tflops_issued", "frac_of_roofline", "kernel") if k in row} for row in r["table"]]})
+    r = run_conv_workload("mobilenet", 64, False, steps, warmup)
+    rows = []
+    for L, row in zip(r["layer_list"], r["table"]):
+        e = {k: row[k] for k in ("name", "ms", "gbs", "tflops", "bound", "frac_of_roofline", "kernel")}
+        if L["algo"] == "depthwise_separable":
+            # bandwidth-bound: against the vendor's 8 TB/s, and against a plain streaming kernel that reads |X| and
+            # writes |Y| of this very layer, timed the same way (event pair per launch, cold tensors)
+            xb, yb = 4 * 64 * L["cin"] * L["hw"] ** 2, 4 * 64 * L["cout"] * L["ohw"] ** 2
+            gbs, us = probe.copy_at_size(xb, yb)
+            e["frac_of_hbm_peak"] = round(row["gbs"] / HBM_PEAK_GBS, 4)
+            e["copy_same_size_gbs"] = round(gbs, 1)
+            e["copy_same_size_us"] = round(us, 2)
+            e["frac_of_copy_same_size"] = round(row["gbs"] / gbs, 4)
+        rows.append(e)
+    dw = [e for e in rows if "frac_of_hbm_peak" in e]
+    pw = [e for e in rows if "frac_of_hbm_peak" not in e]
+    cfgs["config4_mobilenet_blocks_b64"] = compact(r, 64, {
+        "depthwise_min_frac_of_hbm_peak": min(e["frac_of_hbm_peak"] for e in dw), "depthwise_min_frac_of_copy_same_size": min(e["frac_of_copy_same_size"] for e in dw),
+        "pointwise_min_frac_of_roofline": min(e["frac_of_roofline"] for e in pw), "layers": rows})
+    del r
+    torch.cuda.empty_cache()
+    cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2))
+    return cfgs
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "single", "resnet18-full",
+                                                                 "resnet50-full", "resnet18-backward"])
+    ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
+    ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
+    ap.add_argument("--prepacked", action="store_true",
+                    help="weights transformed once before the timed region (dlp_conv2d_fwd_pack / _enqueue_packed), as an inference "
+                         "deployment does; the default transforms them in every step, as the reference's enqueue contract implies")
+    ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
+    ap.add_argument("--no-configs", action="store_true", help="default workload only: leave out the `configs` object (the other four configurations)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over batch with no exchange)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    dlp.lib()  # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    if args.workload.endswith("-full"):
+        print(json.dumps(run_graph_workload(args)))
+        return
+    if args.workload == "resnet18-backward":
+        run_backward_workload(args)
+        return
+    bf16 = args.dtype == "bf16"
+    r = run_conv_workload(args.workload, args.batch, bf16, args.steps, args.warmup, args.prepacked, args.only)
+    ms_per_step = r["ms_per_step"]
+    if args.layers:
+        for row in r["table"]:
+            print(json.dumps(row), file=sys.stderr)
+    headline = args.workload == "resnet18" and args.batch == 64 and not bf16 and not args.only
+
+    cpu = cpu_baseline(r["layer_list"], args.cpu_images, 2024) if args.cpu_images > 0 else None  # the fp32 reference path
     # the same arithmetic with the batch spread over the host's cores (what a reference build with a threaded BLAS
     # would approach); the box gives a GPU 16 cores whatever os.cpu_count() says
     cpu_mt = None
     if args.cpu_images > 0:
         nthreads = max(1, min(16, os.cpu_count() or 1))
-        cpu_mt = cpu_baseline(layer_list, max(args.cpu_images, 2 * nthreads), 2024, threads=nthreads)
+        cpu_mt = cpu_baseline(r["layer_list"], max(args.cpu_images, 2 * nthreads), 2024, threads=nthreads)
+
+    # what this chip reaches with no convolution around it (MFMA-only loops, streaming copies), next to the vendor peaks
+    from dlprimitives_amd import probe
+
+    peaks = probe.measured_peaks()
+    rf = r["roofline"]
+    measured = peaks["mfma_bf16_tflops" if rf["peak"] == BF16_MATRIX_PEAK_TFLOPS else "mfma_f32_tflops"] if rf["bound"] == "mfma" else peaks["copy_2048mib_gbs"]
+    rf["measured_peak"] = measured
+    rf["frac_of_measured_peak"] = round(rf["achieved"] / measured, 4)
 
     out = {
         "metric": BASELINE_METRIC,
@@ -441,19 +519,26 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32",
         "data": "synthetic",
-        "config": {"workload": "%s%s, %s NCHW, batch %d" % (description, " (subset --only %s)" % args.only if args.only else "",
+        "config": {"workload": "%s%s, %s NCHW, batch %d" % (r["description"], " (subset --only %s)" % args.only if args.only else "",
                                                             "bf16" if bf16 else "fp32", args.batch) +
                                (", weights packed once before the timed region" if args.prepacked else ""),
-                   "batch": args.batch, "layers": nl, "gflop_per_step": round(total_flops / 1e9, 1),
-                   "mbytes_per_step": round(total_bytes / 1e6, 1)},
-        "gflops_per_s": round(total_flops / (ms_per_step * 1e-3) / 1e9, 1),
-        "frac_of_fp32_matrix_peak": round(total_flops / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
-        "kernel_ms_per_step": round(sum(layer_ms), 4),
-        "roofline": roofline,
+                   "batch": args.batch, "layers": r["nl"], "gflop_per_step": round(r["total_flops"] / 1e9, 1),
+                   "mbytes_per_step": round(r["total_bytes"] / 1e6, 1)},
+        "gflops_per_s": round(r["total_flops"] / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac_of_fp32_matrix_peak": round(r["total_flops"] / (ms_per_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS, 4),
+        "kernel_ms_per_step": round(r["kernel_ms_per_step"], 4),
+        "roofline": rf,
         "cpu_baseline": cpu,
         "cpu_baseline_all_cores": cpu_mt,
-        "layers": table,
+        "vendor_peak": {"fp32_matrix_tflops": FP32_MATRIX_PEAK_TFLOPS, "bf16_matrix_tflops": BF16_MATRIX_PEAK_TFLOPS, "hbm_gbs": HBM_PEAK_GBS},
+        "measured_peak": peaks,
+        "layers": r["table"],
     }
+    if headline and not args.no_configs:
+        del r
+        torch.cuda.empty_cache()
+        out["configs"] = other_configs(max(5, args.steps // 2), max(2, args.warmup // 2), peaks)
+        out["configs"]["config2_resnet18_conv_stack_b64"] = "the headline of this line: value, ms_per_step, roofline, layers"
     print(json.dumps(out))
 
 

@@ -129,15 +129,21 @@ def timing_count():
     return n.value
 
 
-def timing_records(first=0, last=None):
-    """[(section, milliseconds)] of the kernels launched since the last reset (waits for them)."""
+def timing_records(first=0, last=None, kernels=False):
+    """[(section, milliseconds)] of the kernels launched since the last reset (waits for them);
+    with kernels=True [(section, milliseconds, kernel name as a profiler lists it)]."""
     last = timing_count() if last is None else last
     out = []
     name = ctypes.create_string_buffer(64)
+    kname = ctypes.create_string_buffer(256)
     ms = ctypes.c_float()
     for i in range(first, last):
         _check(lib().dlp_timing_get(i, name, 64, ctypes.byref(ms)))
-        out.append((name.value.decode(), ms.value))
+        if kernels:
+            _check(lib().dlp_timing_get_kernel(i, kname, 256))
+            out.append((name.value.decode(), ms.value, kname.value.decode()))
+        else:
+            out.append((name.value.decode(), ms.value))
     return out
 
 

@@ -186,22 +186,22 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         if (blocks > 0x7fffffffLL)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
         if (g.sh == 1 && !bf16)
-            hipLaunchKernelGGL((depthwise3x3_kernel<float, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+            DLP_LAUNCH_TIMED(ts, (depthwise3x3_kernel<float, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         else if (g.sh == 1)
-            hipLaunchKernelGGL((depthwise3x3_kernel<bf16_t, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+            DLP_LAUNCH_TIMED(ts, (depthwise3x3_kernel<bf16_t, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         else if (!bf16)
-            hipLaunchKernelGGL((depthwise3x3_kernel<float, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+            DLP_LAUNCH_TIMED(ts, (depthwise3x3_kernel<float, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         else
-            hipLaunchKernelGGL((depthwise3x3_kernel<bf16_t, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+            DLP_LAUNCH_TIMED(ts, (depthwise3x3_kernel<bf16_t, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
     } else {
         const long long total = (long long)a.planes * g.OH * g.OW;
         const long long blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffLL)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "depthwise convolution too large for a single launch");
         if (bf16)
-            hipLaunchKernelGGL(depthwise_direct_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
+            DLP_LAUNCH_TIMED(ts, depthwise_direct_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
         else
-            hipLaunchKernelGGL(depthwise_direct_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
+            DLP_LAUNCH_TIMED(ts, depthwise_direct_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, a, g.KH, g.sh);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;

@@ -74,9 +74,6 @@ struct GemmArgs {
     int sk_units;             // stream-K (conv_patch_f32_kernel): tiles * stages
     float *sk_part;           // two 64x64 accumulator images per workgroup
     uint32_t sk_part_bytes;
-#ifdef DLP_PATCH_TRACE
-    long long *trace;
-#endif
     int *sk_cnt;              // pieces arrived, per tile (zero at launch)
     int sk_tpw, sk_mb;        // tile order of the stream: tiles per workgroup (transposition), m tiles per pixel tile run
     int sk_tiles;             // tiles of the stream (sk_units / stages per tile)
@@ -659,10 +656,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const int ncb = a.nkt / KHW; // stages per tile
     const uint64_t U = (uint64_t)a.sk_units, G = gridDim.x;
     const int u_begin = (int)((uint64_t)j * U / G), u_end = (int)((uint64_t)(j + 1) * U / G);
-#ifdef DLP_PATCH_TRACE
-    long long tr[4] = {(long long)wall_clock64(), 0, 0, 0};
-    const long long ck0 = (long long)clock64();
-#endif
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
@@ -859,10 +852,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         for (int kk = 0; kk < BK / 2; kk++)
             read_operands(I0{}, I0{}, I0{}, I0{}, kk);
     }
-#ifdef DLP_PATCH_TRACE
-    if (u == u_begin)
-        tr[1] = (long long)wall_clock64();
-#endif
     int cb = cb_begin;
     for (; cb + 1 < cb_end; cb += 2) {
         stage(I0{}, cb);
@@ -871,10 +860,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     if (cb < cb_end)
         stage(I0{}, cb);
 
-#ifdef DLP_PATCH_TRACE
-    if (u == u_begin)
-        tr[2] = (long long)wall_clock64();
-#endif
     bool output = true;
     if (cb_begin != 0 || cb_end != ncb) {
         // A piece of a tile: its accumulators go to this workgroup's first or second slot (register
@@ -923,13 +908,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     __syncthreads(); // LDS is reused by the next piece
     u += cb_end - cb_begin;
     }
-#ifdef DLP_PATCH_TRACE
-    tr[3] = (long long)wall_clock64();
-    tr[2] = (long long)clock64() - ck0;
-    if (tid == 0 && a.trace)
-        for (int i = 0; i < 4; i++)
-            a.trace[j * 4 + i] = tr[i];
-#endif
 }
 
 // ---- bfloat16 storage on the bf16 matrix instruction ------------------------------------
@@ -2105,7 +2083,7 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     blocks = (long long)a.main_wgs + (long long)a.tail_tiles * a.tail_splitk;
     {
         TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL((conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1 && a.sk_cnt == nullptr) {
         TimingScope ts("splitk_reduce", stream);
@@ -2188,13 +2166,13 @@ int launch_patch_bf16(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStre
     TimingScope ts("conv_gemm", stream);
     const dim3 grid((unsigned)blocks), block(kThreads);
     if (p.tile == 2 && p.patch_bf16 == 8)
-        hipLaunchKernelGGL((conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 8, ACT_CLAMP>), grid, block, 0, stream, a);
     else if (p.tile == 2)
-        hipLaunchKernelGGL((conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 4, ACT_CLAMP>), grid, block, 0, stream, a);
     else if (p.patch_bf16 == 8)
-        hipLaunchKernelGGL((conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 8, ACT_CLAMP>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 4, ACT_CLAMP>), grid, block, 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -2206,7 +2184,8 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     {
         TimingScope ts("conv_gemm", stream);
-        hipLaunchKernelGGL(bf16_kernel(p.tile, p.order, pxl, p.dense_sx), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        const Bf16Kernel kernel = bf16_kernel(p.tile, p.order, pxl, p.dense_sx);
+        DLP_LAUNCH_TIMED(ts, kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
         TimingScope ts("splitk_reduce", stream);
@@ -2303,11 +2282,8 @@ int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t 
     make_magic((uint32_t)(a.mtiles * a.ntiles), a.pg_magic, a.pg_shift);
     make_magic((uint32_t)(a.sk_mb * a.ntiles), a.mbnt_magic, a.mbnt_shift);
     make_magic((uint32_t)a.sk_mb, a.mb_magic, a.mb_shift);
-#ifdef DLP_PATCH_TRACE
-    a.trace = (part_ws != nullptr && part_bytes >= ps.ws_bytes + (size_t)grid * 32 + (1u << 20)) ? (long long *)((char *)part_ws + part_bytes - (1u << 20)) : nullptr;
-#endif
     TimingScope ts("conv_gemm", stream);
-    hipLaunchKernelGGL((conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+    DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -2461,13 +2437,14 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
 
 size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
 {
-    if (g.B <= 0)
-        return 0;
+    // the batch of the shape given at create is a hint: without one (0) the workspace is sized for a single image, so that
+    // it always holds the packed weights, which every batch needs
+    const int B = std::max(g.B, 1);
     const GemmPlan p = conv_gemm_plan(g, activation);
     if (p.patch)
-        return p.wpack_bytes + patch_shape(g, p, (long long)g.B * g.OH * g.OW).ws_bytes;
+        return p.wpack_bytes + patch_shape(g, p, (long long)B * g.OH * g.OW).ws_bytes;
     GemmArgs a;
-    a.N = g.B * g.OH * g.OW;
+    a.N = B * g.OH * g.OW;
     a.Cout = g.Cout;
     a.nkt = p.nkt;
     plan_split(p, a, g.groups, true, (size_t)-1);
@@ -2487,7 +2464,8 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
                            size_t part_bytes, int mode, bool counters_owned)
 {
     if (p.wdirect && ((uintptr_t)w & 15) == 0) { // conv_gemm_launch reads w in place: only the counters are left to do
-        if (bf16_mfma_order(p.order))
+        // (a buffer packed ahead of time is filled all the same: a later call may come with a weight pointer that cannot be read in place)
+        if (bf16_mfma_order(p.order) && mode != GEMM_PACK_ONLY)
             return DLP_OK;
         // fp32: weights packed once ahead of time are still the faster operand (one 16-byte LDS store per thread and
         // K tile instead of four); reading in place only saves the packing launch of a call that would pack every time

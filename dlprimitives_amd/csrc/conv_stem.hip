@@ -403,13 +403,13 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     TimingScope ts("conv_gemm", stream);
     const bool gen = generic_activation(ep.activation);
     if (vec && !gen)
-        hipLaunchKernelGGL((conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, false>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, false>), grid, block, 0, stream, a);
     else if (vec)
-        hipLaunchKernelGGL((conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, true>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, true>), grid, block, 0, stream, a);
     else if (!gen)
-        hipLaunchKernelGGL((conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, false>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, false>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, true>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, true>), grid, block, 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }

@@ -553,9 +553,9 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
 #define DLP_WINO_LAUNCH(NL)                                                                                          \
     do {                                                                                                             \
         if (tail)                                                                                                    \
-            hipLaunchKernelGGL((wino_fused_kernel<T, true, NL>), dim3(grid), dim3(kThreads), 0, stream, a);          \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, true, NL>), dim3(grid), dim3(kThreads), 0, stream, a);        \
         else                                                                                                         \
-            hipLaunchKernelGGL((wino_fused_kernel<T, false, NL>), dim3(grid), dim3(kThreads), 0, stream, a);         \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, false, NL>), dim3(grid), dim3(kThreads), 0, stream, a);       \
     } while (0)
         if (plan.stage_loads == 8)
             DLP_WINO_LAUNCH(8);

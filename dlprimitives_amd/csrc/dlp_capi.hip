@@ -8,7 +8,9 @@
 
 #include <algorithm>
 
+#include <cstdlib>
 #include <cstring>
+#include <cxxabi.h>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -28,6 +30,8 @@ int fail(int code, const std::string &msg)
 namespace {
 struct TimingRecord {
     const char *section;
+    const void *kernel; // host-side handle of the kernel, or null
+    hipStream_t stream;
     hipEvent_t start, stop;
 };
 std::mutex g_timing_mutex;
@@ -42,6 +46,8 @@ TimingScope::TimingScope(const char *section, hipStream_t stream) : stream_(stre
         return;
     TimingRecord r;
     r.section = section;
+    r.kernel = nullptr;
+    r.stream = stream;
     if (hipEventCreate(&r.start) != hipSuccess)
         return;
     if (hipEventCreate(&r.stop) != hipSuccess) {
@@ -60,6 +66,15 @@ TimingScope::~TimingScope()
     std::lock_guard<std::mutex> lock(g_timing_mutex);
     if (index_ < (int)g_timing_records.size())
         (void)hipEventRecord(g_timing_records[index_].stop, stream_);
+}
+
+void TimingScope::kernel(const void *host_function)
+{
+    if (index_ < 0)
+        return;
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    if (index_ < (int)g_timing_records.size())
+        g_timing_records[index_].kernel = host_function;
 }
 
 } // namespace dlp
@@ -257,6 +272,45 @@ int dlp_timing_get(int index, char *section, size_t section_len, float *millisec
     DLP_HIP_TRY(hipEventElapsedTime(milliseconds, r.start, r.stop));
     std::strncpy(section, r.section, section_len - 1);
     section[section_len - 1] = 0;
+    return DLP_OK;
+}
+
+int dlp_timing_get_kernel(int index, char *kernel, size_t kernel_len)
+{
+    DLP_REQUIRE(kernel != nullptr && kernel_len > 0, "null argument");
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    DLP_REQUIRE(index >= 0 && index < (int)g_timing_records.size(), "timing record index out of range");
+    const TimingRecord &r = g_timing_records[index];
+    std::string name;
+    if (r.kernel) {
+        const char *mangled = hipKernelNameRefByPtr(r.kernel, r.stream);
+        if (mangled) {
+            int status = 0;
+            char *plain = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
+            name = (status == 0 && plain) ? plain : mangled;
+            std::free(plain);
+            // as a kernel trace prints it: no namespaces, no parameter list
+            if (!name.empty() && name.back() == ')') { // the parameter list: back to the parenthesis that matches the last one
+                int depth = 0;
+                for (size_t i = name.size(); i-- > 0;) {
+                    depth += name[i] == ')' ? 1 : name[i] == '(' ? -1 : 0;
+                    if (depth == 0) {
+                        name.erase(i);
+                        break;
+                    }
+                }
+            }
+            if (name.compare(0, 5, "void ") == 0)
+                name.erase(0, 5);
+            for (const char *ns : {"dlp::(anonymous namespace)::", "(anonymous namespace)::", "dlp::"}) {
+                const std::string n(ns);
+                for (size_t at; (at = name.find(n)) != std::string::npos;)
+                    name.erase(at, n.size());
+            }
+        }
+    }
+    std::strncpy(kernel, name.c_str(), kernel_len - 1);
+    kernel[kernel_len - 1] = 0;
     return DLP_OK;
 }
 
@@ -676,8 +730,6 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
         void *unused = nullptr;
         rc = scratch_on_current_device(&unused);
     }
-    if (rc == DLP_OK && hipMalloc(&op->wpacked, op->plan.wpack_bytes) != hipSuccess)
-        rc = fail(DLP_ERR_RUNTIME, "hipMalloc(packed weights) failed");
     if (rc != DLP_OK) {
         if (op->ktab)
             (void)hipFree(op->ktab);
@@ -723,6 +775,9 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
                                 (float *)((char *)op->scratch + op->scratch_cnt_bytes), (hipStream_t)stream);
     }
     const ConvGeom g = ip_gemm_geom(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype);
+    // the packed copy of w (about the size of w) exists only for operators that ever come here: bf16 rows of odd length
+    if (!op->wpacked)
+        DLP_HIP_TRY(hipMalloc(&op->wpacked, op->plan.wpack_bytes));
     int rc = conv_gemm_pack_weights(g, op->plan, w, op->wpacked, (hipStream_t)stream);
     if (rc != DLP_OK)
         return rc;

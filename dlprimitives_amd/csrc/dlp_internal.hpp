@@ -32,9 +32,18 @@ int fail(int code, const std::string &msg);
 struct TimingScope {
     TimingScope(const char *section, hipStream_t stream);
     ~TimingScope();
+    // which kernel the record is about: the host-side handle of the kernel launched inside this scope (what
+    // hipLaunchKernelGGL is given); dlp_timing_get_kernel turns it into the name a profiler's kernel trace shows
+    void kernel(const void *host_function);
     hipStream_t stream_;
     int index_;
 };
+// hipLaunchKernelGGL + TimingScope::kernel in one: launches `fn` and notes it in the record of `ts`
+#define DLP_LAUNCH_TIMED(ts, fn, grid, block, lds, stream, ...)          \
+    do {                                                                 \
+        (ts).kernel(reinterpret_cast<const void *>(fn));                 \
+        hipLaunchKernelGGL(fn, grid, block, lds, stream, __VA_ARGS__);   \
+    } while (0)
 
 // Geometry of one forward convolution call (whole tensor, all groups).
 struct ConvGeom {

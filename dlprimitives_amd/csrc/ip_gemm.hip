@@ -305,7 +305,7 @@ int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *
     TimingScope ts("ip_direct", stream);
     // 16-byte loads when every row of x and w starts on a 16-byte boundary, dword loads otherwise
     const bool wide = (inputs * esize) % 16 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
-    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, a); };
+    auto launch = [&](auto kernel) { DLP_LAUNCH_TIMED(ts, kernel, grid, block, 0, stream, a); };
     auto pick = [&](auto type_tag, auto nb_c) {
         using T = decltype(type_tag);
         constexpr int NBV = decltype(nb_c)::value;

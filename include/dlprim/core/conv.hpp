@@ -59,17 +59,26 @@ public:
     // y = factor != 0 ? factor * y + act(conv(x, w) + bias) : act(conv(x, w) + bias)
     // ws: uint8 tensor of at least workspace() bytes; asynchronous on e
     virtual void enqueue(Tensor &x, Tensor &w, Tensor *bias, Tensor &y, Tensor &ws, float factor, ExecutionContext const &e) = 0;
-    // Not in the reference: weights that stay constant between calls are transformed once into `packed`
+    // Not in the reference (default bodies, so that a class written against the reference's interface, which has
+    // enqueue alone, still compiles): weights that stay constant between calls are transformed once into `packed`
     // (uint8 tensor of packed_size() bytes, may be empty when that is 0) and enqueue_packed reads them
     // from there; ws is then per-call scratch only (workspace() bytes are enough, operators that run
-    // one after another may share it).
+    // one after another may share it).  The defaults keep nothing: packed_size() is 0, pack() does
+    // nothing and enqueue_packed() is enqueue().
+    virtual size_t packed_size() { return 0; }
+    virtual void pack(Tensor & /*w*/, Tensor & /*packed*/, ExecutionContext const & /*e*/) {}
+    virtual void enqueue_packed(Tensor &x, Tensor &w, Tensor & /*packed*/, Tensor *bias, Tensor &y, Tensor &ws, float factor,
+                                ExecutionContext const &e)
+    {
+        enqueue(x, w, bias, y, ws, factor, e);
+    }
     // Not in the reference: y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias), so that a
-    // residual sum whose other branch is already in y costs no pass of its own
-    virtual void accumulate_before_activation(bool on) = 0;
-    virtual size_t packed_size() = 0;
-    virtual void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) = 0;
-    virtual void enqueue_packed(Tensor &x, Tensor &w, Tensor &packed, Tensor *bias, Tensor &y, Tensor &ws, float factor,
-                                ExecutionContext const &e) = 0;
+    // residual sum whose other branch is already in y costs no pass of its own.  The default refuses.
+    virtual void accumulate_before_activation(bool on)
+    {
+        if (on)
+            throw NotImplementedError("accumulate_before_activation is not implemented by this Conv2DForward");
+    }
     static std::unique_ptr<Conv2DForward> create(Context &ctx, Conv2DSettings const &config, bool bias,
                                                  StandardActivations activation = StandardActivations::identity,
                                                  std::string const &algo = std::string());

@@ -71,7 +71,7 @@ inline StandardActivations activation_from_name(std::string const &name)
         return StandardActivations::sigmoid;
     if (name == "relu6")
         return StandardActivations::relu6;
-    throw ValidationError("Invalid cativation name:" + name);
+    throw ValidationError("unknown activation \"" + name + "\" (identity, relu, tanh, sigmoid, relu6)");
 }
 
 struct Convolution2DConfigBase {

@@ -107,6 +107,11 @@ int dlp_timing_enable(int on);
 int dlp_timing_reset(void);
 int dlp_timing_count(int *count);
 int dlp_timing_get(int index, char *section, size_t section_len, float *milliseconds);
+/* Name of the kernel a record is about, as a profiler's kernel trace lists it (template arguments included,
+ * namespaces and parameter list left out), e.g. "conv_patch_f32_kernel<float, 3, 3, 192, 0>"; empty for
+ * records of helper launches that do not note their kernel.  No counterpart in the reference, whose kernels
+ * are named by the OpenCL program that holds them. */
+int dlp_timing_get_kernel(int index, char *kernel, size_t kernel_len);
 
 /* ---- Conv2DBase::get_output_shape, src/core/conv.cpp:17-29 ------------------ */
 int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], int out_shape[4]);

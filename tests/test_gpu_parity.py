@@ -362,7 +362,8 @@ def test_depthwise_odd_shapes(gpu, oracle_mod, geom):
 
 
 # ------------------------------------------------------------ pointwise followers of the depthwise blocks
-@pytest.mark.parametrize("pw", [(144, 24, 56), (192, 64, 14), (960, 320, 7)], ids=lambda p: "%dto%d_at%d" % p)
+@pytest.mark.parametrize("pw", [(144, 24, 56), (144, 32, 28), (192, 32, 28), (192, 64, 14), (384, 64, 14), (384, 96, 14), (960, 160, 7), (960, 320, 7)],
+                         ids=lambda p: "%dto%d_at%d" % p)
 def test_pointwise_1x1(gpu, oracle_mod, pw):
     cin, cout, hw = pw
     c = case(1, 0, 1, 1, cin, cout, True, 1, False)
