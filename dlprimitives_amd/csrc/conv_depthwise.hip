@@ -25,6 +25,10 @@
 // Other odd kernel sizes use a plain direct kernel.
 #include "dlp_internal.hpp"
 
+#include <algorithm>
+#include <cstdlib>
+#include <type_traits>
+
 namespace dlp {
 namespace {
 
@@ -121,6 +125,265 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
     }
 }
 
+// ---- 3x3, whole planes through LDS ------------------------------------------------------------------
+// In NCHW the planes of a depthwise convolution are independent and lie one after another in memory, so a run of
+// P whole planes is one contiguous piece of x and produces one contiguous piece of y.  A workgroup takes such a
+// run of at most 16 KB: it copies it to LDS with 16-byte loads, all in flight at once (every byte of x is read
+// exactly once: no halo rows, whatever the plane size), computes from LDS into a second LDS buffer and writes that
+// with 16-byte stores.  The filter and bias of the run's channels travel to LDS next to the input.
+// The layer is bound by memory, but only if the arithmetic stays out of the way: 9 multiply-adds per output are a
+// seventh of the chip's vector rate at 5 TB/s, so every other instruction per output counts.  A lane therefore takes
+// a tile of R rows x kPlaneSeg columns of outputs and slides a three-row window down it: 9 (stride 1) input values
+// read from LDS per output row of 7, edge handling decided once per tile (padding is read from a block of zeros
+// behind the run by choosing the address, so the reads carry no condition), one v_med3 for ReLU / ReLU6.
+// R is chosen by the host so that the tiles of a run are about one per thread.
+// Accumulation order is the reference's: sum = bias; sum = fma(k[dr][dc], x, sum) for dr, dc ascending.
+constexpr int kPlaneSeg = 7;          // output columns of a tile (divides the 56 / 28 / 14 / 7 wide feature maps)
+constexpr int kPlaneThreads = 256;
+constexpr int kPlaneMaxPieces = 4;    // 16-byte pieces per thread: a run is at most 16 KB
+constexpr int kPlaneMaxBytes = kPlaneMaxPieces * kPlaneThreads * 16;
+constexpr int kPlaneMaxP = 64;        // planes of a run
+constexpr int kPlaneWStride = 11;     // floats per plane in the LDS filter table (9 weights, bias; odd: no bank conflicts)
+
+struct DwPlaneArgs {
+    const void *x, *w;
+    const float *bias;
+    void *y;
+    int planes, C, H, W, OH, OW;
+    int P;      // planes per run
+    int nseg;   // tiles per row of tiles
+    int R, nrt; // output rows per tile, rows of tiles per plane
+    uint32_t tpp_magic, tpp_shift, nseg_magic, nseg_shift; // divisions by (nrt * nseg) and by nseg
+    float factor;
+    int act;
+    float clamp_lo, clamp_hi;
+};
+
+// GENERIC_ACT: tanh / sigmoid; otherwise identity, ReLU or ReLU6 as one clamp (a per-output switch on the activation turns into
+// scalar branches around every output, which cost more than the arithmetic)
+template <class T, int STRIDE, bool FULL, int NLD, bool GENERIC_ACT>
+__global__ __launch_bounds__(kPlaneThreads) void depthwise3x3_plane_kernel(DwPlaneArgs a)
+{
+    constexpr int kPlanePieces = NLD;
+    constexpr int kRunBytes = NLD * kPlaneThreads * 16;
+    constexpr int EPP = 16 / (int)sizeof(T);           // elements per 16-byte piece
+    constexpr int NIN = (kPlaneSeg - 1) * STRIDE + 3;  // input columns of a tile
+    constexpr int NZ = 16;                              // zeros behind the run: what a padding row or column reads
+    static_assert(NIN <= NZ, "tile shape");
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kRunBytes + NZ * sizeof(T)]; // the run | zeros
+    __shared__ __attribute__((aligned(16))) unsigned char lds_out_raw[kRunBytes];              // the run's output
+    __shared__ float lds_w[kPlaneMaxP * kPlaneWStride];
+    T *lds = reinterpret_cast<T *>(lds_raw);
+    T *lds_out = reinterpret_cast<T *>(lds_out_raw);
+    T *zeros = reinterpret_cast<T *>(lds_raw + kRunBytes);
+    const int tid = threadIdx.x;
+    const int HW = a.H * a.W, OHW = a.OH * a.OW;
+    const int plane0 = (int)blockIdx.x * a.P;
+    const int np = min(a.P, a.planes - plane0); // planes of this run
+    const int n_in = np * HW, n_out = np * OHW;
+    const T *xg = (const T *)a.x + (size_t)plane0 * HW;
+    T *yg = (T *)a.y + (size_t)plane0 * OHW;
+
+    // ---- the run's input, filter and bias: global -> registers (every load issued before anything waits) -> LDS ----
+    uint4 piece[kPlanePieces];
+#pragma unroll
+    for (int q = 0; q < kPlanePieces; q++) {
+        const int e0 = (tid + kPlaneThreads * q) * EPP;
+        piece[q] = make_uint4(0, 0, 0, 0);
+        if (e0 + EPP <= n_in)
+            piece[q] = *reinterpret_cast<const uint4 *>(xg + e0);
+        else if (e0 < n_in) { // the last piece of the tensor may be cut short
+            T tmp[EPP];
+#pragma unroll
+            for (int e = 0; e < EPP; e++)
+                tmp[e] = (e0 + e < n_in) ? xg[e0 + e] : T();
+            piece[q] = *reinterpret_cast<const uint4 *>(tmp);
+        }
+    }
+    float wreg[3]; // 9 weights and the bias of every plane of the run: np * 10 <= 640 values
+    int w_pl[3], w_j[3];
+    {
+        const int c0 = plane0 % a.C;
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            const int i = tid + kPlaneThreads * q;
+            w_pl[q] = i / 10;
+            w_j[q] = i - w_pl[q] * 10;
+            wreg[q] = 0.0f;
+            if (w_pl[q] < np) {
+                int c = c0 + w_pl[q];
+                c = c >= a.C ? c % a.C : c;
+                wreg[q] = w_j[q] < 9 ? to_float(((const T *)a.w)[c * 9 + w_j[q]]) : (a.bias ? a.bias[c] : 0.0f);
+            }
+        }
+    }
+    if (tid < NZ)
+        zeros[tid] = T();
+#pragma unroll
+    for (int q = 0; q < kPlanePieces; q++)
+        if ((tid + kPlaneThreads * q) * EPP < n_in)
+            *reinterpret_cast<uint4 *>(lds_raw + (tid + kPlaneThreads * q) * 16) = piece[q];
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+        if (w_pl[q] < np)
+            lds_w[w_pl[q] * kPlaneWStride + w_j[q]] = wreg[q];
+    __syncthreads();
+
+    // ---- tiles of R x kPlaneSeg outputs: numbered (plane, row of tiles, tile in the row) ----
+    const int tpp = a.nrt * a.nseg;
+    const int tiles = np * tpp;
+    for (int tile = tid; tile < tiles; tile += kPlaneThreads) {
+        const int pl = (int)fast_div((uint32_t)tile, a.tpp_magic, a.tpp_shift);
+        const int rem = tile - pl * tpp;
+        const int ty = (int)fast_div((uint32_t)rem, a.nseg_magic, a.nseg_shift);
+        const int ox0 = (rem - ty * a.nseg) * kPlaneSeg;
+        const int oy0 = ty * a.R;
+        const int rows = min(a.R, a.OH - oy0);
+        const int out_n = min(kPlaneSeg, a.OW - ox0);
+        T *pout = lds_out + pl * OHW + oy0 * a.OW + ox0;
+        const float *kw = lds_w + pl * kPlaneWStride;
+        float k[9];
+#pragma unroll
+        for (int i = 0; i < 9; i++)
+            k[i] = kw[i];
+        const float bias = kw[9];
+        const T *pin = lds + pl * HW;
+        const int ix0 = ox0 * STRIDE - 1;
+        const bool left_ok = ix0 >= 0, right_ok = ix0 + NIN - 1 < a.W;
+        const bool clamp = a.act != DLP_ACT_IDENTITY;
+        float v[3][NIN]; // the window: input rows of the current output row
+        auto load_row = [&](auto slot_c, int iy) {
+            constexpr int SL = decltype(slot_c)::value;
+            const bool vy = iy >= 0 && iy < a.H;
+            if (FULL) {
+                // every tile is whole (OW is a multiple of kPlaneSeg): only the first and the last column of the window can
+                // fall outside the image; a padding row reads zeros[j], a padding column zeros[0]
+                const T *row = vy ? pin + iy * a.W + ix0 : zeros;
+                const T *first = left_ok ? row : zeros, *last = right_ok ? row + (NIN - 1) : zeros;
+                v[SL][0] = to_float(*first);
+#pragma unroll
+                for (int j = 1; j < NIN - 1; j++)
+                    v[SL][j] = to_float(row[j]);
+                v[SL][NIN - 1] = to_float(*last);
+            } else {
+                const T *row = pin + (vy ? iy : 0) * a.W;
+#pragma unroll
+                for (int j = 0; j < NIN; j++) {
+                    const int ix = ix0 + j;
+                    v[SL][j] = (vy && ix >= 0 && ix < a.W) ? to_float(row[ix]) : 0.0f;
+                }
+            }
+        };
+        auto compute_row = [&](auto s0_c, auto s1_c, auto s2_c, int r) { // output row r of the tile from window slots s0, s1, s2
+            constexpr int S0 = decltype(s0_c)::value, S1 = decltype(s1_c)::value, S2 = decltype(s2_c)::value;
+#pragma unroll
+            for (int o = 0; o < kPlaneSeg; o++) {
+                float sum = bias;
+#pragma unroll
+                for (int dc = 0; dc < 3; dc++)
+                    sum = fmaf(k[dc], v[S0][o * STRIDE + dc], sum);
+#pragma unroll
+                for (int dc = 0; dc < 3; dc++)
+                    sum = fmaf(k[3 + dc], v[S1][o * STRIDE + dc], sum);
+#pragma unroll
+                for (int dc = 0; dc < 3; dc++)
+                    sum = fmaf(k[6 + dc], v[S2][o * STRIDE + dc], sum);
+                if (GENERIC_ACT)
+                    sum = apply_act(sum, a.act);
+                else {
+                    const float clamped = clamp_med3(sum, a.clamp_lo, a.clamp_hi);
+                    sum = clamp ? clamped : sum; // identity keeps NaNs: no clamp
+                }
+                if (FULL || o < out_n)
+                    store_plain(pout + r * a.OW + o, sum);
+            }
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        const int iy0 = oy0 * STRIDE - 1;
+        if (STRIDE == 1) { // the window moves down one row per output row: one new row each, slots rotate
+            load_row(I0{}, iy0);
+            load_row(I1{}, iy0 + 1);
+            for (int r = 0; r < rows; r += 3) {
+                load_row(I2{}, iy0 + r + 2);
+                compute_row(I0{}, I1{}, I2{}, r);
+                if (r + 1 < rows) {
+                    load_row(I0{}, iy0 + r + 3);
+                    compute_row(I1{}, I2{}, I0{}, r + 1);
+                }
+                if (r + 2 < rows) {
+                    load_row(I1{}, iy0 + r + 4);
+                    compute_row(I2{}, I0{}, I1{}, r + 2);
+                }
+            }
+        } else { // two rows per output row: the last row of one window is the first of the next
+            load_row(I0{}, iy0);
+            for (int r = 0; r < rows; r += 2) {
+                load_row(I1{}, iy0 + 2 * r + 1);
+                load_row(I2{}, iy0 + 2 * r + 2);
+                compute_row(I0{}, I1{}, I2{}, r);
+                if (r + 1 < rows) {
+                    load_row(I0{}, iy0 + 2 * r + 3);
+                    load_row(I1{}, iy0 + 2 * r + 4);
+                    compute_row(I2{}, I0{}, I1{}, r + 1);
+                }
+                // an even number of rows later the first window slot holds the shared row again
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- the run's output: LDS -> global, 16 bytes per store ----
+#pragma unroll
+    for (int q = 0; q < kPlanePieces; q++) {
+        const int e0 = (tid + kPlaneThreads * q) * EPP;
+        if (e0 >= n_out)
+            continue;
+        const uint4 r = *reinterpret_cast<const uint4 *>(lds_out_raw + (tid + kPlaneThreads * q) * 16);
+        if (e0 + EPP <= n_out && a.factor == 0.0f) {
+            *reinterpret_cast<uint4 *>(yg + e0) = r;
+        } else { // y = factor * y + value (reference: depthwise_separable_conv.cl:96-101), and the cut last piece
+            T tmp[EPP];
+            *reinterpret_cast<uint4 *>(tmp) = r;
+#pragma unroll
+            for (int e = 0; e < EPP; e++)
+                if (e0 + e < n_out)
+                    store_out(yg + e0 + e, to_float(tmp[e]), a.factor);
+        }
+    }
+}
+
+// Planes per run for this geometry (0: the plane kernel does not take it): as many as fit 16 KB of input and 64 planes,
+// and such that every run starts on a 16-byte boundary in x and in y.
+static int plane_run(const ConvGeom &g)
+{
+    if (g.KH != 3 || g.KW != 3)
+        return 0;
+    const long long es = (long long)dtype_size(g.dtype);
+    const long long in_bytes = (long long)g.H * g.W * es, out_bytes = (long long)g.OH * g.OW * es;
+    if (in_bytes > kPlaneMaxBytes)
+        return 0;
+    // Measured on the MobileNet shapes at batch 64 (fp32, back-to-back launches on tensors that start cold): the plane kernel against the
+    // strip kernel 47.7 / 51.9 us (C144 at 56 x 56), 19.0 / 21.8, 13.3 / 15.7, 9.0 / 11.5 us at stride 1; 36.3 / 32.9, 13.8 / 15.3,
+    // 10.1 / 10.0, 7.6 / 7.7 us at stride 2: with large planes at stride 2 a run holds few tiles (112 for 256 threads) and the strip kernel wins.
+    // With bf16 tensors the plane kernel wins throughout (its loads and stores stay 16 bytes wide).
+    if (g.dtype == DLP_FLOAT && g.sh == 2 && in_bytes > 8192)
+        return 0;
+    const long long pmax = std::min<long long>(kPlaneMaxP, kPlaneMaxBytes / in_bytes);
+    auto gcd = [](long long x, long long y) {
+        while (y) {
+            const long long r = x % y;
+            x = y;
+            y = r;
+        }
+        return x;
+    };
+    const long long s_in = 16 / gcd(16, in_bytes), s_out = 16 / gcd(16, out_bytes);
+    const long long step = s_in / gcd(s_in, s_out) * s_out;
+    return (int)(pmax / step * step);
+}
+
 // Any odd kernel size, stride 1 or 2, pad = K/2: one output per thread.
 template <class T>
 __global__ __launch_bounds__(256) void depthwise_direct_kernel(DwArgs a, int K, int stride)
@@ -179,6 +442,64 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.factor = ep.factor;
     a.act = ep.activation;
     TimingScope ts("sep_conv", stream);
+    const int run = plane_run(g);
+    if (run > 0 && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
+        DwPlaneArgs pa;
+        pa.x = x;
+        pa.w = w;
+        pa.bias = ep.bias;
+        pa.y = y;
+        pa.planes = a.planes;
+        pa.C = g.Cin;
+        pa.H = g.H;
+        pa.W = g.W;
+        pa.OH = g.OH;
+        pa.OW = g.OW;
+        pa.P = run;
+        pa.nseg = (g.OW + kPlaneSeg - 1) / kPlaneSeg;
+        // rows per tile: about one tile per thread (up to 7 rows: the window slides, so a taller tile reads fewer input rows per output)
+        pa.R = (int)std::min<long long>(7, std::max<long long>(1, ((long long)run * pa.nseg * g.OH + kPlaneThreads - 1) / kPlaneThreads));
+        pa.nrt = (g.OH + pa.R - 1) / pa.R;
+        make_magic((uint32_t)(pa.nrt * pa.nseg), pa.tpp_magic, pa.tpp_shift);
+        make_magic((uint32_t)pa.nseg, pa.nseg_magic, pa.nseg_shift);
+        pa.factor = ep.factor;
+        pa.act = ep.activation;
+        pa.clamp_lo = 0.0f;
+        pa.clamp_hi = ep.activation == DLP_ACT_RELU6 ? 6.0f : __builtin_huge_valf();
+        const dim3 grid((unsigned)(((long long)a.planes + run - 1) / run)), block(kPlaneThreads);
+        const bool full = g.OW % kPlaneSeg == 0;
+        const bool generic = ep.activation == DLP_ACT_TANH || ep.activation == DLP_ACT_SIGMOID;
+        auto launch = [&](auto type_tag, auto stride_c) {
+            using T = decltype(type_tag);
+            constexpr int S = decltype(stride_c)::value;
+            const long long run_bytes = (long long)run * g.H * g.W * (long long)dtype_size(g.dtype);
+            auto with_nld = [&](auto nld_c) {
+                constexpr int N = decltype(nld_c)::value;
+                if (generic)
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_plane_kernel<T, S, false, N, true>), grid, block, 0, stream, pa);
+                else if (full)
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_plane_kernel<T, S, true, N, false>), grid, block, 0, stream, pa);
+                else
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_plane_kernel<T, S, false, N, false>), grid, block, 0, stream, pa);
+            };
+            if (run_bytes <= 4096)
+                with_nld(std::integral_constant<int, 1>{});
+            else if (run_bytes <= 8192)
+                with_nld(std::integral_constant<int, 2>{});
+            else
+                with_nld(std::integral_constant<int, 4>{});
+        };
+        if (!bf16 && g.sh == 1)
+            launch(float{}, std::integral_constant<int, 1>{});
+        else if (!bf16)
+            launch(float{}, std::integral_constant<int, 2>{});
+        else if (g.sh == 1)
+            launch(bf16_t{}, std::integral_constant<int, 1>{});
+        else
+            launch(bf16_t{}, std::integral_constant<int, 2>{});
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
     if (g.KH == 3) {
         const int per_wave = g.sh == 1 ? 62 : 63;
         const long long waves = (a.total_cols + per_wave - 1) / per_wave;

@@ -2202,18 +2202,7 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
 // the prologue), every one with the same number of (tile, stage) units, but no fewer than 4
 // stages per workgroup.
 constexpr int kPatchWgsPerCu = 3;
-int device_cu_count()
-{
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
+int device_cu_count() { return dlp_cu_count(); }
 struct PatchShape {
     long long tiles, units;
     int grid;

@@ -68,6 +68,19 @@ TimingScope::~TimingScope()
         (void)hipEventRecord(g_timing_records[index_].stop, stream_);
 }
 
+int dlp_cu_count()
+{
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
 void TimingScope::kernel(const void *host_function)
 {
     if (index_ < 0)

@@ -45,6 +45,9 @@ struct TimingScope {
         hipLaunchKernelGGL(fn, grid, block, lds, stream, __VA_ARGS__);   \
     } while (0)
 
+// Compute units of the current device (256 on MI355X); cached after the first call.
+int dlp_cu_count();
+
 // Geometry of one forward convolution call (whole tensor, all groups).
 struct ConvGeom {
     int B, Cin, H, W;

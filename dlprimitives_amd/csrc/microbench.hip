@@ -79,20 +79,16 @@ __global__ __launch_bounds__(256) void write_f4(float4 *__restrict__ dst, size_t
         dst[i] = v;
 }
 
-// reads n_in and writes n_out 16-byte pieces (the sizes may differ, as for a strided convolution)
-__global__ __launch_bounds__(256) void read_write_f4(const float4 *__restrict__ src, size_t n_in, float4 *__restrict__ dst, size_t n_out)
+// reads n_in and writes n_out 16-byte pieces (the sizes may differ, as for a strided convolution): one piece per thread and
+// direction, 32-bit index, no loop -- the plainest streaming kernel there is
+__global__ __launch_bounds__(256) void read_write_f4(const float4 *__restrict__ src, int n_in, float4 *__restrict__ dst, int n_out)
 {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t n = n_in > n_out ? n_in : n_out;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        float4 v = {0, 0, 0, 0};
-        if (i < n_in)
-            v = src[i];
-        if (i < n_out)
-            dst[i] = v;
-        else if (v.x == 12345.678f) // never true for the probe's data: keeps the read alive
-            dst[0] = v;
-    }
+    const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+    float4 v = {0, 0, 0, 0};
+    if (i < n_in)
+        v = src[i];
+    if (i < n_out)
+        dst[i] = v;
 }
 
 static float time_ms(hipStream_t s, hipEvent_t e0, hipEvent_t e1)
@@ -189,9 +185,10 @@ int dlp_probe_copy(int mbytes, double *gbs)
 }
 
 // What a plain streaming kernel reaches on tensors of a given size: reads in_bytes, writes out_bytes (16-byte
-// accesses, one grid-stride pass), each launch timed by its own event pair on the stream (the way the library's
-// per-kernel timing measures a convolution launch) and on its own pair of buffers out of a ring that is larger
-// than the 256 MB last-level cache, so every launch starts cold, as a layer in a network does.
+// accesses, one piece per thread and direction).  The launches run back
+// to back, each on its own pair of buffers out of a ring that is larger than the 256 MB last-level cache, so every
+// launch starts cold, as a layer in a network does; one event pair brackets all of them (an event between two
+// launches makes the first one write back its part of the L2 before it ends, which a kernel inside a network does not).
 // gbs = (in_bytes + out_bytes) / mean launch time; us = that mean time in microseconds.
 int dlp_probe_copy_sized(size_t in_bytes, size_t out_bytes, double *gbs, double *us)
 {
@@ -210,37 +207,28 @@ int dlp_probe_copy_sized(size_t in_bytes, size_t out_bytes, double *gbs, double 
         return 1;
     (void)hipMemset(ring, 1, pair * nbuf);
     const int reps = 3 * nbuf > 40 ? 3 * nbuf : 40;
-    hipEvent_t *e0 = new hipEvent_t[reps], *e1 = new hipEvent_t[reps];
-    for (int r = 0; r < reps; r++) {
-        (void)hipEventCreate(&e0[r]);
-        (void)hipEventCreate(&e1[r]);
-    }
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
     const size_t n_in = in_bytes / 16, n_out = out_bytes / 16;
     const size_t n = n_in > n_out ? n_in : n_out;
-    size_t blocks = (n + 255) / 256;
-    if (blocks > 256 * 16)
-        blocks = 256 * 16;
+    if (n >= ((size_t)1 << 31))
+        return 1;
+    const size_t blocks = (n + 255) / 256;
     for (int r = -nbuf; r < reps; r++) { // one untimed pass over the ring first
         char *base = ring + pair * (size_t)((r + nbuf) % nbuf);
-        if (r >= 0)
-            (void)hipEventRecord(e0[r], 0);
-        read_write_f4<<<(unsigned)blocks, 256>>>((const float4 *)base, n_in, (float4 *)(base + in_bytes), n_out);
-        if (r >= 0)
-            (void)hipEventRecord(e1[r], 0);
+        if (r == 0)
+            (void)hipEventRecord(e0, 0);
+        read_write_f4<<<(unsigned)blocks, 256>>>((const float4 *)base, (int)n_in, (float4 *)(base + in_bytes), (int)n_out);
     }
-    (void)hipDeviceSynchronize();
-    double total_ms = 0;
-    for (int r = 0; r < reps; r++) {
-        float ms = 0;
-        (void)hipEventElapsedTime(&ms, e0[r], e1[r]);
-        total_ms += ms;
-        (void)hipEventDestroy(e0[r]);
-        (void)hipEventDestroy(e1[r]);
-    }
-    delete[] e0;
-    delete[] e1;
+    (void)hipEventRecord(e1, 0);
+    (void)hipEventSynchronize(e1);
+    float total_ms = 0;
+    (void)hipEventElapsedTime(&total_ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     (void)hipFree(ring);
-    const double mean_ms = total_ms / reps;
+    const double mean_ms = (double)total_ms / reps;
     *us = mean_ms * 1e3;
     *gbs = (double)pair / (mean_ms * 1e-3) / 1e9;
     return hipGetLastError() == hipSuccess ? 0 : 1;

@@ -361,6 +361,39 @@ def test_depthwise_odd_shapes(gpu, oracle_mod, geom):
     np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
 
 
+@pytest.mark.parametrize("geom", [(1, 5, 7, 7, 3), (2, 5, 7, 7, 3), (1, 130, 7, 7, 1), (1, 3, 56, 56, 2), (2, 3, 56, 56, 1), (1, 7, 14, 21, 2), (1, 2, 64, 64, 1),
+                                  (1, 2, 65, 64, 1), (2, 6, 13, 13, 5)], ids=lambda g: "s%d_c%d_%dx%d_b%d" % g)
+@pytest.mark.parametrize("unaligned", [False, True])
+def test_depthwise_plane_runs(gpu, oracle_mod, geom, unaligned):
+    """3x3 depthwise planes of at most 16 KB go through LDS in runs of whole planes: run tails (fewer planes than a run, a last
+    16-byte piece cut short), 1 and 2 tasks per thread, the largest plane that fits (64 x 64) and the first that does not, the
+    factor path -- and tensors that do not start on a 16-byte boundary, which take the strip kernel."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    s, ch, h, w_, b = geom
+    c = case(3, 1, s, 1, ch, ch, True, ch, True)
+    x, w, bias = make_tensors(c, (b, h, w_), seed=ch + h)
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    st = gpu.settings_of(c, x.shape)
+    op = dlp.Conv2DForward.create(st, True, "relu", "depthwise_separable")
+    assert op.algo() == "depthwise_separable"
+    off = 1 if unaligned else 0
+    xbuf = torch.zeros(x.size + off, device="cuda:0")
+    ybuf = torch.full((want.size + off,), float("nan"), device="cuda:0")
+    xd, yd = xbuf[off:].view(x.shape), ybuf[off:].view(want.shape)
+    xd.copy_(torch.from_numpy(x))
+    op.enqueue(xd, gpu.dev(w), gpu.dev(bias), yd, None, 0.0)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(yd.cpu().numpy(), want, **TOL)
+    old = np.random.default_rng(1).standard_normal(want.shape).astype(np.float32)
+    yd.copy_(torch.from_numpy(old))
+    op.enqueue(xd, gpu.dev(w), gpu.dev(bias), yd, None, 0.5)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(yd.cpu().numpy(), oracle_mod.apply_factor(want, old, 0.5), **TOL)
+
+
 # ------------------------------------------------------------ pointwise followers of the depthwise blocks
 @pytest.mark.parametrize("pw", [(144, 24, 56), (144, 32, 28), (192, 32, 28), (192, 64, 14), (384, 64, 14), (384, 96, 14), (960, 160, 7), (960, 320, 7)],
                          ids=lambda p: "%dto%d_at%d" % p)
