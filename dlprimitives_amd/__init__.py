@@ -17,12 +17,14 @@ from .capi import (  # noqa: F401
     IPSettings,
     NotImplementedErrorDlprim,
     Pooling2DForward,
+    TransposedConv2DForward,
     ValidationError,
     activation_forward,
     bias_backward,
     build_library,
     channel_affine_forward,
     conv2d_output_shape,
+    conv2d_transposed_output_shape,
     eltwise_forward,
     lib,
     library_path,

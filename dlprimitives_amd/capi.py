@@ -317,6 +317,66 @@ class Conv2DBackwardFilter(_Conv2DBackward):
         _check(lib().dlp_conv2d_bwd_filter_enqueue(self._h, xs, _ptr(x), _ptr(dw), _ptr(dy), _ptr(ws), ws_bytes, float(factor), _stream(stream)))
 
 
+def conv2d_transposed_output_shape(settings, in_shape, output_pad=(0, 0)):
+    """Conv2DBase::get_output_shape_transposed"""
+    L = lib()
+    L.dlp_conv2d_transposed_output_shape.argtypes = [ctypes.POINTER(_Settings), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                                     ctypes.POINTER(ctypes.c_int)]
+    ish = (ctypes.c_int * 4)(*[int(v) for v in in_shape])
+    osh = (ctypes.c_int * 4)()
+    c = settings._c()
+    _check(L.dlp_conv2d_transposed_output_shape(ctypes.byref(c), ish, (ctypes.c_int * 2)(*_pair(output_pad)), osh))
+    return tuple(osh)
+
+
+class TransposedConv2DForward:
+    """TransposedConvolution2D::forward on the device: `settings` describe the transposed operator
+    (channels_in = channels of x, shape = shape of x); w is [channels_in, channels_out / groups, kh, kw]."""
+
+    def __init__(self, handle, settings, output_pad):
+        self._h = handle
+        self.settings = settings
+        self.output_pad = output_pad
+
+    @staticmethod
+    def create(settings, output_pad=(0, 0), bias=True, activation="identity", algo=""):
+        L = lib()
+        L.dlp_tconv2d_fwd_create.argtypes = [ctypes.POINTER(_Settings), ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_char_p,
+                                             ctypes.POINTER(ctypes.c_void_p)]
+        L.dlp_tconv2d_fwd_algo.restype = ctypes.c_char_p
+        L.dlp_tconv2d_fwd_algo.argtypes = [ctypes.c_void_p]
+        L.dlp_tconv2d_fwd_workspace.restype = ctypes.c_size_t
+        L.dlp_tconv2d_fwd_workspace.argtypes = [ctypes.c_void_p]
+        L.dlp_tconv2d_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                              ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.dlp_tconv2d_fwd_destroy.argtypes = [ctypes.c_void_p]
+        L.dlp_tconv2d_fwd_destroy.restype = None
+        h = ctypes.c_void_p()
+        c = settings._c()
+        _check(L.dlp_tconv2d_fwd_create(ctypes.byref(c), (ctypes.c_int * 2)(*_pair(output_pad)), int(bool(bias)), _act(activation),
+                                        (algo or "").encode(), ctypes.byref(h)))
+        return TransposedConv2DForward(h, settings, _pair(output_pad))
+
+    def algo(self):
+        return lib().dlp_tconv2d_fwd_algo(self._h).decode()
+
+    def workspace(self):
+        return int(lib().dlp_tconv2d_fwd_workspace(self._h))
+
+    def output_shape(self, in_shape):
+        return conv2d_transposed_output_shape(self.settings, in_shape, self.output_pad)
+
+    def enqueue(self, x, w, bias, y, ws=None, stream=None):
+        xs = (ctypes.c_int * 4)(*x.shape)
+        ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
+        _check(lib().dlp_tconv2d_fwd_enqueue(self._h, xs, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes, _stream(stream)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().dlp_tconv2d_fwd_destroy(self._h)
+            self._h = None
+
+
 def bias_backward(dy, db, beta=0.0, stream=None):
     """core::BiasBackwardFilter::enqueue: db[f] = beta * db[f] + sum of dy[:, f] over batch and plane"""
     batch, features = int(dy.shape[0]), int(dy.shape[1])

@@ -915,6 +915,109 @@ int dlp_conv2d_bwd_filter_enqueue(dlp_conv2d_bwd_filter *op, const int x_shape[4
 
 void dlp_conv2d_bwd_filter_destroy(dlp_conv2d_bwd_filter *op) { delete op; }
 
+// ---- TransposedConvolution2D forward (src/ops/conv2d.cpp:559-805): the gradient-of-data pass of the convolution whose
+//      input and output channels are swapped (:588-590), then bias (core::add_bias) and activation ----
+struct dlp_tconv2d_fwd {
+    dlp_conv2d_settings cfg; // of the transposed operator: shape = its input shape
+    int output_pad[2];
+    int out_shape[4];
+    bool bias;
+    int activation;
+    dlp_conv2d_bwd_data *bwd;
+};
+
+int dlp_conv2d_transposed_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], const int output_pad[2], int out_shape[4])
+{
+    DLP_REQUIRE(cfg != nullptr && in_shape != nullptr && output_pad != nullptr && out_shape != nullptr, "null argument");
+    DLP_REQUIRE(in_shape[1] == cfg->channels_in, "input channels differ from channels_in");
+    for (int i = 0; i < 2; i++) {
+        DLP_REQUIRE(cfg->kernel[i] > 0 && cfg->stride[i] > 0 && cfg->dilate[i] > 0 && cfg->pad[i] >= 0 && output_pad[i] >= 0, "kernel/stride/dilate/pad");
+        const int o = (in_shape[2 + i] - 1) * cfg->stride[i] - 2 * cfg->pad[i] + cfg->dilate[i] * (cfg->kernel[i] - 1) + output_pad[i] + 1;
+        DLP_REQUIRE(o > 0, "empty output");
+        out_shape[2 + i] = o;
+    }
+    out_shape[0] = in_shape[0];
+    out_shape[1] = cfg->channels_out;
+    return DLP_OK;
+}
+
+int dlp_tconv2d_fwd_create(const dlp_conv2d_settings *cfg, const int output_pad[2], int bias, int activation, const char *algo, dlp_tconv2d_fwd **out)
+{
+    DLP_REQUIRE(cfg != nullptr && output_pad != nullptr && out != nullptr, "null argument");
+    *out = nullptr;
+    DLP_REQUIRE(cfg->channels_in > 0 && cfg->channels_out > 0 && cfg->groups > 0, "channels/groups must be positive");
+    DLP_REQUIRE(cfg->channels_in % cfg->groups == 0 && cfg->channels_out % cfg->groups == 0, "channels not divisible by groups");
+    DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
+    if (cfg->dtype != DLP_FLOAT) // src/ops/conv2d.cpp:584
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "TransposedConvolution2D: float_data is implemented");
+    int oshape[4];
+    int rc = dlp_conv2d_transposed_output_shape(cfg, cfg->shape, output_pad, oshape);
+    if (rc != DLP_OK)
+        return rc;
+    // the convolution it is the data gradient of: channels swapped, input = this operator's output (:588-590, :693-699)
+    dlp_conv2d_settings conv = *cfg;
+    conv.channels_in = cfg->channels_out;
+    conv.channels_out = cfg->channels_in;
+    for (int i = 0; i < 4; i++)
+        conv.shape[i] = oshape[i];
+    int back[4];
+    rc = dlp_conv2d_output_shape(&conv, conv.shape, back);
+    if (rc != DLP_OK)
+        return rc;
+    // an output_pad of a whole stride or more would describe the next larger input
+    DLP_REQUIRE(back[2] == cfg->shape[2] && back[3] == cfg->shape[3], "output_pad must be smaller than the stride");
+    dlp_tconv2d_fwd *op = new (std::nothrow) dlp_tconv2d_fwd();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *cfg;
+    op->output_pad[0] = output_pad[0];
+    op->output_pad[1] = output_pad[1];
+    for (int i = 0; i < 4; i++)
+        op->out_shape[i] = oshape[i];
+    op->bias = bias != 0;
+    op->activation = activation;
+    op->bwd = nullptr;
+    rc = dlp_conv2d_bwd_data_create(&conv, algo, &op->bwd);
+    if (rc != DLP_OK) {
+        delete op;
+        return rc;
+    }
+    *out = op;
+    return DLP_OK;
+}
+
+const char *dlp_tconv2d_fwd_algo(const dlp_tconv2d_fwd *op) { return op ? dlp_conv2d_bwd_data_algo(op->bwd) : ""; }
+
+size_t dlp_tconv2d_fwd_workspace(const dlp_tconv2d_fwd *op) { return op ? dlp_conv2d_bwd_data_workspace(op->bwd) : 0; }
+
+int dlp_tconv2d_fwd_enqueue(dlp_tconv2d_fwd *op, const int x_shape[4], const void *x, const void *w, const void *bias, void *y, void *ws,
+                            size_t ws_bytes, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[0] >= 0, "negative batch");
+    DLP_REQUIRE(x_shape[1] == op->cfg.channels_in && x_shape[2] == op->cfg.shape[2] && x_shape[3] == op->cfg.shape[3],
+                "input shape differs from the shape given at create (only the batch may change)");
+    DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
+    if (x_shape[0] == 0)
+        return DLP_OK;
+    const int y_shape[4] = {x_shape[0], op->out_shape[1], op->out_shape[2], op->out_shape[3]};
+    int rc = dlp_conv2d_bwd_data_enqueue(op->bwd, y_shape, y, w, x, ws, ws_bytes, 0.0f, stream); // :782
+    if (rc != DLP_OK)
+        return rc;
+    if (op->bias || op->activation != DLP_ACT_IDENTITY) // :783-790; one pass for both
+        rc = channel_affine_launch(DLP_FLOAT, op->activation, y_shape[0], y_shape[1], y_shape[2] * y_shape[3], y, nullptr, (const float *)bias, y,
+                                   (hipStream_t)stream);
+    return rc;
+}
+
+void dlp_tconv2d_fwd_destroy(dlp_tconv2d_fwd *op)
+{
+    if (!op)
+        return;
+    dlp_conv2d_bwd_data_destroy(op->bwd);
+    delete op;
+}
+
 int dlp_bias_bwd_enqueue(int dtype, int batch, int features, int plane, const void *dy, float *db, float beta, void *stream)
 {
     if (dtype != DLP_FLOAT)

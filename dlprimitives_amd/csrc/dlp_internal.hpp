@@ -230,6 +230,10 @@ enum { WINO_FILTER_AND_RUN = 0, WINO_FILTER_ONLY = 1, WINO_RUN_ONLY = 2 };
 int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, size_t ws_bytes,
                     const Epilogue &ep, hipStream_t stream, int mode = WINO_FILTER_AND_RUN);
 
+// ---- per-channel affine + activation (glue_ops.hip): y = act(x * scale[c] + shift[c]); null scale = 1, null shift = 0
+int channel_affine_launch(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale, const float *shift,
+                          void *y, hipStream_t stream);
+
 // ---- InnerProduct GEMM (ip_gemm.hip) ------------------------------------------
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype);
 // Launch shape of the direct kernel (operands loaded from memory straight into matrix-instruction registers)

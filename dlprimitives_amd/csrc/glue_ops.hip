@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256) void channel_affine_kernel(size_t packs, int C
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < packs; k += stride) {
         const int c = (int)((k / (size_t)plane_packs) % (size_t)C);
-        const float sc = scale[c], sh = shift[c];
+        const float sc = scale ? scale[c] : 1.0f, sh = shift ? shift[c] : 0.0f; // (x * 1 + sh rounds once, like x + sh)
         const Pack px = ((const Pack *)x)[k];
         Pack py;
 #pragma unroll
@@ -485,12 +485,22 @@ int dlp_activation_fwd_enqueue(int dtype, int activation, size_t n, const void *
 int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale,
                                    const float *shift, void *y, void *stream)
 {
+    DLP_REQUIRE(batch <= 0 || (scale != nullptr && shift != nullptr), "null tensor pointer");
+    return dlp::channel_affine_launch(dtype, activation, batch, channels, plane, x, scale, shift, y, (hipStream_t)stream);
+}
+
+} // extern "C"
+
+// y = act(x * scale[c] + shift[c]); a null scale is 1, a null shift 0 (bias and activation behind an operator that has no epilogue of its own)
+int dlp::channel_affine_launch(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale,
+                               const float *shift, void *y, hipStream_t stream)
+{
     DLP_REQUIRE(dtype == DLP_FLOAT || dtype == DLP_BFLOAT16, "float_data and bfloat16_data are implemented");
     DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
     DLP_REQUIRE(batch >= 0 && channels > 0 && plane > 0, "shape");
     if (batch == 0)
         return DLP_OK;
-    DLP_REQUIRE(x != nullptr && y != nullptr && scale != nullptr && shift != nullptr, "null tensor pointer");
+    DLP_REQUIRE(x != nullptr && y != nullptr, "null tensor pointer");
     const size_t n = (size_t)batch * channels * plane;
     hipStream_t st = (hipStream_t)stream;
     const int vec = 16 / (dtype == DLP_BFLOAT16 ? 2 : 4);
@@ -519,6 +529,8 @@ int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int cha
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
+
+extern "C" {
 
 int dlp_softmax_fwd_enqueue(int dtype, int log_softmax, int batch, int classes, int inner, const void *x, void *y, void *stream)
 {

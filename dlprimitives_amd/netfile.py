@@ -100,6 +100,25 @@ class NetBuilder:
         self.shapes[dst] = (n, cout, ho, wo)
         return dst
 
+    def tconv(self, src, dst, cout, k, stride=1, pad=0, output_pad=0, groups=1, bias=False, activation=None, dilate=1, prefix=None):
+        """TransposedConvolution2D: weights [channels_in, channels_out / groups, kh, kw] (src/ops/conv2d.cpp:629-634)"""
+        n, cin, h, w = self.shapes[src]
+        k2, s2, p2, d2, o2 = _pair(k), _pair(stride), _pair(pad), _pair(dilate), _pair(output_pad)
+        opts = {"bias": bias, "groups": groups, "channels_out": cout, "channels_in": cin, "kernel": k2, "stride": s2, "dilate": d2, "pad": p2,
+                "output_pad": o2}
+        if activation:
+            opts["activation"] = activation
+        prefix = prefix or dst
+        params = [prefix + ".weight"] + ([prefix + ".bias"] if bias else [])
+        self._op("ConvTranspose", "TransposedConvolution2D", [src], [dst], opts, params)
+        self.param_shapes[params[0]] = (cin, cout // groups, k2[0], k2[1])
+        if bias:
+            self.param_shapes[params[1]] = (cout,)
+        ho = (h - 1) * s2[0] - 2 * p2[0] + d2[0] * (k2[0] - 1) + o2[0] + 1
+        wo = (w - 1) * s2[1] - 2 * p2[1] + d2[1] * (k2[1] - 1) + o2[1] + 1
+        self.shapes[dst] = (n, cout, ho, wo)
+        return dst
+
     def bn(self, src, dst, eps=1e-5, affine=True, activation=None, prefix=None):
         c = self.shapes[src][1]
         prefix = prefix or dst

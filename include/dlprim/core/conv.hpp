@@ -51,6 +51,14 @@ public:
         dlprim::details::check_status(dlp_conv2d_output_shape(&s, s.shape, out));
         return Shape(size_t(out[0]), out[1], out[2], out[3]);
     }
+    // output shape of the transposed convolution (src/core/conv.cpp:31-43 in the reference)
+    static Shape get_output_shape_transposed(Convolution2DConfigBase const &config, Shape const &in, int output_pad[2])
+    {
+        dlp_conv2d_settings s = details::to_c(config, in, float_data);
+        int out[4];
+        dlprim::details::check_status(dlp_conv2d_transposed_output_shape(&s, s.shape, output_pad, out));
+        return Shape(size_t(out[0]), out[1], out[2], out[3]);
+    }
 };
 
 class Conv2DForward : public Conv2DBase {
@@ -150,6 +158,40 @@ public:
     virtual ~Conv2DBackwardFilter() {}
     virtual void enqueue(Tensor &x, Tensor &dw, Tensor &dy, Tensor &ws, float factor, ExecutionContext const &e) = 0;
     static std::unique_ptr<Conv2DBackwardFilter> create(Context &ctx, Conv2DSettings const &config, std::string const &algo = std::string());
+};
+
+// The device half of the reference's TransposedConvolution2D operator (include/dlprim/ops/conv2d.hpp:96-171,
+// TransposedConvolution2D::forward, src/ops/conv2d.cpp:741-805): y = act(transposed convolution of x with
+// w [channels_in, channels_out / groups, kh, kw] + bias).  `config` describes the transposed operator (shape = shape of x).
+class TransposedConv2DForward : public Conv2DBase {
+public:
+    TransposedConv2DForward(Context &ctx, Conv2DSettings const &config, int const output_pad[2], bool bias,
+                            StandardActivations activation = StandardActivations::identity, std::string const &algo = std::string())
+    {
+        if (!ctx.is_hip_context())
+            throw ValidationError("core::TransposedConv2DForward needs a device context");
+        ctx.select();
+        dlp_conv2d_settings s = details::to_c(config, config.shape, config.dtype);
+        dlprim::details::check_status(dlp_tconv2d_fwd_create(&s, output_pad, bias ? 1 : 0, int(activation), algo.c_str(), &op_));
+    }
+    ~TransposedConv2DForward() { dlp_tconv2d_fwd_destroy(op_); }
+    TransposedConv2DForward(TransposedConv2DForward const &) = delete;
+    void operator=(TransposedConv2DForward const &) = delete;
+    char const *algo() const override { return dlp_tconv2d_fwd_algo(op_); }
+    size_t workspace() override { return dlp_tconv2d_fwd_workspace(op_); }
+    void enqueue(Tensor &x, Tensor &w, Tensor *bias, Tensor &y, Tensor &ws, ExecutionContext const &e)
+    {
+        DLPRIM_CHECK(x.shape().size() == 4);
+        int xs[4];
+        for (int i = 0; i < 4; i++)
+            xs[i] = int(x.shape()[i]);
+        const size_t ws_bytes = workspace() ? ws.memory_size() : 0;
+        dlprim::details::check_status(dlp_tconv2d_fwd_enqueue(op_, xs, x.device_ptr(), w.device_ptr(), bias ? bias->device_ptr() : nullptr, y.device_ptr(),
+                                                              ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, e.stream()));
+    }
+
+private:
+    dlp_tconv2d_fwd *op_ = nullptr;
 };
 
 namespace details {

@@ -8,8 +8,8 @@
 // liveness (src/net.cpp:585-654: intermediate tensors share chunks unless keep_intermediate_tensors),
 // and runs the operators in order on one ExecutionContext with one shared workspace
 // (src/net.cpp:836-851).  Operator types: Convolution2D, BatchNorm, Activation, Pooling2D,
-// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- with the option
-// names of the reference's *Config::from_json functions.
+// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- plus Softmax, Flatten and
+// TransposedConvolution2D, with the option names of the reference's *Config::from_json functions.
 //
 // In predict mode two graph rewrites are applied at setup (fuse(true), the default):
 //  * a BatchNorm that is the only consumer of a Convolution2D / InnerProduct output is folded into its
@@ -186,6 +186,17 @@ public:
                         n.is_packed = false;
                         pack_conv_weights(n, e);
                     }
+                }
+                break;
+            }
+            case k_tconv: {
+                DLPRIM_CHECK(in.size() == 4 && int(in[1]) == n.conv.channels_in);
+                out = core::Conv2DBase::get_output_shape_transposed(n.conv, in, n.output_pad);
+                Shape const &old = n.planned_in;
+                if (n.tconv_op && (old[2] != in[2] || old[3] != in[3] || in[0] > old[0])) {
+                    create_tconv_operator(n, in);
+                    if (workspace_bytes_ > workspace_.memory_size())
+                        workspace_ = Tensor(ctx_, Shape(workspace_bytes_), uint8_data);
                 }
                 break;
             }
@@ -381,7 +392,7 @@ public:
     }
 
 private:
-    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten };
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv };
     struct Node {
         std::string name, type;
         std::vector<std::string> inputs, outputs, param_names;
@@ -399,6 +410,8 @@ private:
         float residual_factor = 1.0f;
         bool is_packed = false, use_w_dev = false;
         std::unique_ptr<core::Conv2DForward> conv_op;
+        std::unique_ptr<core::TransposedConv2DForward> tconv_op; // TransposedConvolution2D
+        int output_pad[2] = {0, 0};
         std::unique_ptr<core::IPForward> ip_op;
         Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
         Tensor packed;       // the weights in the order the kernel loads them
@@ -496,6 +509,31 @@ private:
                 DLPRIM_CHECK(n.conv.channels_in == int(in[1]));
                 specs_[n.outputs[0]] = core::Conv2DBase::get_output_shape(n.conv, in);
                 make_param(n, 0, Shape(size_t(n.conv.channels_out), n.conv.channels_in / n.conv.groups, n.conv.kernel[0], n.conv.kernel[1]));
+                if (n.bias)
+                    make_param(n, 1, Shape(size_t(n.conv.channels_out)));
+            } else if (n.type == "TransposedConvolution2D") { // src/ops/conv2d.cpp:559-660: weights [channels_in, channels_out / groups, kh, kw]
+                n.kind = k_tconv;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                Shape const &in = spec(n.inputs[0]);
+                DLPRIM_CHECK(in.size() == 4);
+                if (dtype_ != float_data)
+                    throw NotImplementedError("TransposedConvolution2D in a 16-bit storage type (" + n.name + ")");
+                n.conv.channels_in = o.get("channels_in", int(in[1]));
+                n.conv.channels_out = o.get<int>("channels_out");
+                pair_option(o, "kernel", n.conv.kernel, true);
+                pair_option(o, "stride", n.conv.stride);
+                pair_option(o, "dilate", n.conv.dilate);
+                pair_option(o, "pad", n.conv.pad);
+                pair_option(o, "output_pad", n.output_pad);
+                n.conv.groups = o.get("groups", 1);
+                n.bias = o.get("bias", true);
+                n.algo = o.get("bwd_data_algo", "auto"); // the forward pass is the data-gradient operator (:693-699)
+                if (n.algo == "auto")
+                    n.algo = "";
+                DLPRIM_CHECK(n.conv.channels_in == int(in[1]));
+                DLPRIM_CHECK(n.conv.channels_in % n.conv.groups == 0 && n.conv.channels_out % n.conv.groups == 0);
+                specs_[n.outputs[0]] = core::Conv2DBase::get_output_shape_transposed(n.conv, in, n.output_pad);
+                make_param(n, 0, Shape(size_t(n.conv.channels_in), n.conv.channels_out / n.conv.groups, n.conv.kernel[0], n.conv.kernel[1]));
                 if (n.bias)
                     make_param(n, 1, Shape(size_t(n.conv.channels_out)));
             } else if (n.type == "InnerProduct") {
@@ -656,7 +694,7 @@ private:
     void try_merge_activation(size_t i)
     {
         Node &p = nodes_[i];
-        if (!((p.kind == k_conv || p.kind == k_ip || p.kind == k_eltwise || p.kind == k_bn) && p.activation == StandardActivations::identity))
+        if (!((p.kind == k_conv || p.kind == k_ip || p.kind == k_eltwise || p.kind == k_bn || p.kind == k_tconv) && p.activation == StandardActivations::identity))
             return;
         std::string const &t = p.outputs[0];
         int u = next_user(i, t);
@@ -728,6 +766,13 @@ private:
         n.planned_in = in;
         workspace_bytes_ = std::max(workspace_bytes_, n.conv_op->workspace());
     }
+    void create_tconv_operator(Node &n, Shape const &in)
+    {
+        core::Conv2DSettings cfg(n.conv, in, dtype_);
+        n.tconv_op.reset(new core::TransposedConv2DForward(ctx_, cfg, n.output_pad, n.bias, n.activation, n.algo));
+        n.planned_in = in;
+        workspace_bytes_ = std::max(workspace_bytes_, n.tconv_op->workspace());
+    }
     void pack_conv_weights(Node &n, ExecutionContext const &e)
     {
         const size_t bytes = n.conv_op->packed_size();
@@ -748,6 +793,7 @@ private:
             Shape const &in = spec(n.inputs[0]);
             switch (n.kind) {
             case k_conv: create_conv_operator(n, in); break;
+            case k_tconv: create_tconv_operator(n, in); break;
             case k_ip: {
                 core::IPSettings cfg;
                 cfg.inputs = n.ip_inputs;
@@ -941,6 +987,9 @@ private:
             n.ip_op->enqueue(x, w, b, y, e);
             break;
         }
+        case k_tconv:
+            n.tconv_op->enqueue(x, param(n.param_names[0]), n.bias ? &param(n.param_names[1]) : nullptr, y, workspace_, e);
+            break;
         case k_bn: {
             Shape const &s = x.shape();
             details::check_status(dlp_channel_affine_fwd_enqueue(int(dtype_), int(n.activation), int(s[0]), int(s[1]),

@@ -185,6 +185,23 @@ int dlp_conv2d_bwd_data_enqueue(dlp_conv2d_bwd_data *op, const int x_shape[4], v
                                 const void *dy, void *ws, size_t ws_bytes, float factor, void *stream);
 void dlp_conv2d_bwd_data_destroy(dlp_conv2d_bwd_data *op);
 
+/* ---- TransposedConvolution2D::forward on a device, src/ops/conv2d.cpp:559-805 (operator declared in
+ *      include/dlprim/ops/conv2d.hpp:96-171): y [B,Cout,OH,OW] = act(transposed convolution of x [B,Cin,H,W] with
+ *      w [Cin,Cout/groups,KH,KW] + bias [Cout]).  As in the reference it is the data-gradient pass of the convolution with
+ *      the channels swapped (:588-590,:693-699,:782), followed by bias and activation.  `cfg` describes the transposed
+ *      operator itself (channels_in = channels of x, shape = shape of x, batch a hint); float_data only (:584).
+ *      dlp_conv2d_transposed_output_shape is Conv2DBase::get_output_shape_transposed, src/core/conv.cpp:31-43:
+ *      o = (i - 1) * stride - 2 * pad + dilate * (kernel - 1) + output_pad + 1. ------------------------------------ */
+typedef struct dlp_tconv2d_fwd dlp_tconv2d_fwd;
+int dlp_conv2d_transposed_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4], const int output_pad[2], int out_shape[4]);
+int dlp_tconv2d_fwd_create(const dlp_conv2d_settings *cfg, const int output_pad[2], int bias, int activation, const char *algo,
+                           dlp_tconv2d_fwd **out);
+const char *dlp_tconv2d_fwd_algo(const dlp_tconv2d_fwd *op);
+size_t dlp_tconv2d_fwd_workspace(const dlp_tconv2d_fwd *op);
+int dlp_tconv2d_fwd_enqueue(dlp_tconv2d_fwd *op, const int x_shape[4], const void *x, const void *w, const void *bias, void *y,
+                            void *ws, size_t ws_bytes, void *stream);
+void dlp_tconv2d_fwd_destroy(dlp_tconv2d_fwd *op);
+
 /* ---- core::Conv2DBackwardFilter, include/dlprim/core/conv.hpp:70-78, src/core/conv.cpp:165-220,
  *      369-434,592-669 (CPU contract: src/ops/conv2d.cpp:431-435,475-484):
  *      dw [Cout,Cin/groups,KH,KW] = factor * dw + gradient with respect to the filter, from

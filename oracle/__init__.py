@@ -139,6 +139,32 @@ def conv2d_backward_data(dy, w, cfg, in_shape, dx_old=None, factor=0.0):
     return dx
 
 
+def tconv2d_output_shape(cfg, in_shape, output_pad=(0, 0)):
+    """Conv2DBase::get_output_shape_transposed restated"""
+    ish = (ctypes.c_int * 4)(*in_shape)
+    op = (ctypes.c_int * 2)(*output_pad)
+    osh = (ctypes.c_int * 4)()
+    if lib().orc_tconv2d_output_shape(ctypes.byref(cfg), ish, op, osh) < 0:
+        raise ValueError("invalid transposed convolution configuration")
+    return tuple(osh)
+
+
+def tconv2d_forward(x, w, bias, cfg, output_pad=(0, 0), activation="identity"):
+    """TransposedConvolution2D::forward (CPU path) restated; cfg describes the transposed operator
+    (channels_in = x.shape[1]); w is [channels_in, channels_out / groups, kh, kw]."""
+    x, w = _f32(x), _f32(w)
+    osh = tconv2d_output_shape(cfg, x.shape, output_pad)
+    y = np.empty(osh, dtype=np.float32)
+    conv = make_cfg(cfg.channels_out, cfg.channels_in, tuple(cfg.kernel), tuple(cfg.stride), tuple(cfg.dilate), tuple(cfg.pad), cfg.groups)
+    ws = np.empty(max(1, lib().orc_conv2d_workspace(ctypes.byref(conv), (ctypes.c_int * 4)(*osh)) // 4), dtype=np.float32)
+    b = _f32(bias) if bias is not None else None
+    rc = lib().orc_tconv2d_forward(ctypes.byref(cfg), (ctypes.c_int * 4)(*x.shape), (ctypes.c_int * 2)(*output_pad), _ptr(x), _ptr(w),
+                                   _ptr(b) if b is not None else None, _ptr(y), _ptr(ws), ACTIVATIONS[activation])
+    if rc < 0:
+        raise ValueError("invalid transposed convolution configuration")
+    return y
+
+
 def conv2d_backward_filter(dy, x, cfg, dw_old=None, factor=0.0):
     """Convolution2D::backward_filter_cpu restated: returns factor * dw_old + gradient with respect to w."""
     dy, x = _f32(dy), _f32(x)

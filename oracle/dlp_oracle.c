@@ -345,6 +345,49 @@ int orc_conv2d_backward_data(const orc_conv2d_cfg *cfg, const int in_shape[4],
     return 0;
 }
 
+/* Conv2DBase::get_output_shape_transposed, src/core/conv.cpp:31-43 */
+int orc_tconv2d_output_shape(const orc_conv2d_cfg *cfg, const int in_shape[4], const int output_pad[2], int out_shape[4])
+{
+    if (in_shape[1] != cfg->channels_in)
+        return -1;
+    for (int i = 0; i < 2; i++) {
+        const int o = (in_shape[2 + i] - 1) * cfg->stride[i] - 2 * cfg->pad[i] + cfg->dilate[i] * (cfg->kernel[i] - 1) + output_pad[i] + 1;
+        if (o <= 0)
+            return -1;
+        out_shape[2 + i] = o;
+    }
+    out_shape[0] = in_shape[0];
+    out_shape[1] = cfg->channels_out;
+    return 0;
+}
+
+/* TransposedConvolution2D::forward, CPU branch, src/ops/conv2d.cpp:760-778 and :798-801: the output is filled with the bias
+ * (or zeros), the data-gradient pass of the convolution with swapped channels (:588-590) adds into it, the activation
+ * runs over the whole tensor last.  cfg describes the transposed operator; w is [channels_in][channels_out / groups][kh][kw];
+ * ws: orc_conv2d_workspace() bytes of the swapped convolution on the output shape. */
+int orc_tconv2d_forward(const orc_conv2d_cfg *cfg, const int in_shape[4], const int output_pad[2], const float *x, const float *w,
+                        const float *bias, float *y, void *ws, int activation)
+{
+    int out[4];
+    if (orc_tconv2d_output_shape(cfg, in_shape, output_pad, out) != 0)
+        return -1;
+    orc_conv2d_cfg conv = *cfg;
+    conv.channels_in = cfg->channels_out;
+    conv.channels_out = cfg->channels_in;
+    const size_t plane = (size_t)out[2] * out[3];
+    float *p = y;
+    for (int b = 0; b < out[0]; b++)
+        for (int c = 0; c < out[1]; c++) {
+            const float v = bias ? bias[c] : 0.0f;
+            for (size_t k = 0; k < plane; k++)
+                *p++ = v;
+        }
+    if (orc_conv2d_backward_data(&conv, out, x, w, y, ws, 1.0f) != 0)
+        return -1;
+    orc_apply_activation(y, (size_t)out[0] * out[1] * plane, activation);
+    return 0;
+}
+
 /* src/ops/conv2d.cpp:431-435 and the backward_filter branch :475-484 */
 int orc_conv2d_backward_filter(const orc_conv2d_cfg *cfg, const int in_shape[4],
                                const float *dy, const float *x, float *dw, void *ws, float factor)

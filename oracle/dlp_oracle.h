@@ -86,6 +86,11 @@ void orc_col2im(const orc_conv2d_cfg *cfg, int cin_g, int H, int W, int OH, int 
  * ws: scratch of at least orc_conv2d_workspace() bytes.  Returns 0, or -1 on invalid configuration. */
 int orc_conv2d_backward_data(const orc_conv2d_cfg *cfg, const int in_shape[4],
                              const float *dy, const float *w, float *dx, void *ws, float factor);
+/* TransposedConvolution2D (src/ops/conv2d.cpp:559-805): output shape (src/core/conv.cpp:31-43) and the CPU forward pass;
+ * cfg describes the transposed operator, w is [channels_in][channels_out / groups][kh][kw] */
+int orc_tconv2d_output_shape(const orc_conv2d_cfg *cfg, const int in_shape[4], const int output_pad[2], int out_shape[4]);
+int orc_tconv2d_forward(const orc_conv2d_cfg *cfg, const int in_shape[4], const int output_pad[2], const float *x, const float *w,
+                        const float *bias, float *y, void *ws, int activation);
 int orc_conv2d_backward_filter(const orc_conv2d_cfg *cfg, const int in_shape[4],
                                const float *dy, const float *x, float *dw, void *ws, float factor);
 
