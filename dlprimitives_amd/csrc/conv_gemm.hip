@@ -158,9 +158,13 @@ template <class T, int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
                                                  int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid);
 
-template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
+// NSET: register sets of tiles in flight = how many K tiles ahead of the matrix instructions the loads are issued.  Two is
+// enough when eight workgroups share a CU and cover each other's waits; launches with few workgroups per CU (small layers,
+// short K) run four, so that one workgroup alone has four K tiles on their way.
+template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT, int NSET = 2>
 __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 {
+    static_assert(NSET == 2 || NSET == 4, "register sets");
     static_assert(BK == 16, "the slice helpers assume 8 MFMA steps per K tile");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
@@ -287,9 +291,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     // into one set while tile kt+1 moves from the other set into LDS and tile kt
     // (already in LDS) feeds the matrix cores.  A global load therefore has a whole
     // K step to land before anything waits on it.
-    f32x4 ra[2][A_LD];
-    float rb[2][B_LD];
-    uint32_t vsel[2] = {kOutOfRange, kOutOfRange}; // GEMM_ORDER_TAP: this tile's (masked) pixel offset
+    f32x4 ra[NSET][A_LD];
+    float rb[NSET][B_LD];
+    uint32_t vsel[NSET]; // GEMM_ORDER_TAP: this tile's (masked) pixel offset
+#pragma unroll
+    for (int i = 0; i < NSET; i++)
+        vsel[i] = kOutOfRange;
 
     // one slice of the loads of tile kt into register set S: called once per MFMA
     // group so that vector-memory issue is spread under the MFMAs
@@ -302,9 +309,11 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         for (int j = 0; j < A_LD; j++)
             if (j % (BK / 2) == Q)
                 ra[S][j] = buf_load4(wr, j == 0 ? a_voff0 : (a_active ? (uint32_t)(tid * 16 + j * kThreads * 16) : kOutOfRange), a_soff);
+        // (tiles fetched past the end of K are never multiplied; their table entries are the spare ones behind the last tile)
+        const int ktt = min(kt, a.nkt + 1);
         if (ORDER == GEMM_ORDER_TAP) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
-            ConstInt *e = ktab + kt * 4;
+            ConstInt *e = ktab + ktt * 4;
             const uint32_t xoff = (uint32_t)e[0], tap = (uint32_t)e[1];
             if (Q == 0) {
                 // bit `tap` of the pixel's tap mask, spread over a word, picks the offset (two VALU operations)
@@ -317,7 +326,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                     rb[S][i] = buf_load<T>(xr, vsel[S], xoff + (uint32_t)(ks * B_LD + i) * a.hw4);
         } else {
             // table entry of a k: {x byte offset of (c,ky,kx), tap bit or ky|kx<<8}
-            ConstInt *e = ktab + (kt * BK + ks * B_LD) * 2;
+            ConstInt *e = ktab + (ktt * BK + ks * B_LD) * 2;
 #pragma unroll
             for (int i = 0; i < B_LD; i++) {
                 if (i % (BK / 2) != Q)
@@ -393,7 +402,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
                 read_operands(buf_c, kk + 1, cur ^ 1);
             static_for_slice(kk, [&](auto q) {
                 store_slice(set_next, NextBuf{}, q);
-                load_slice(set_load, kt + 2, q);
+                load_slice(set_load, kt + NSET, q);
             });
             if (ORDER != GEMM_ORDER_CHANNEL || kk < kk_valid) {
 #pragma unroll
@@ -409,19 +418,40 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
-    // prologue: first tile -> set 0 -> LDS[0]; second tile -> set 1
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    // prologue: the first NSET tiles -> sets 0 .. NSET - 1; set 0 -> LDS[0]
     static_for_all([&](auto q) { load_slice(I0{}, kt_begin, q); });
     static_for_all([&](auto q) { load_slice(I1{}, kt_begin + 1, q); });
+    if (NSET == 4) {
+        static_for_all([&](auto q) { load_slice(I2{}, kt_begin + 2, q); });
+        static_for_all([&](auto q) { load_slice(I3{}, kt_begin + 3, q); });
+    }
     static_for_all([&](auto q) { store_slice(I0{}, I0{}, q); });
     __syncthreads();
-    // tiles fetched past kt_end are never multiplied: the table has two spare entries
+    // step on tile kt (in LDS[kt & 1]): set (kt + 1) % NSET goes to the other LDS buffer, tile kt + NSET is fetched into set kt % NSET
     int kt = kt_begin;
-    for (; kt + 1 < kt_end; kt += 2) {
-        k_step(I0{}, I1{}, I0{}, kt);
-        k_step(I1{}, I0{}, I1{}, kt + 1);
+    if (NSET == 2) {
+        for (; kt + 1 < kt_end; kt += 2) {
+            k_step(I0{}, I1{}, I0{}, kt);
+            k_step(I1{}, I0{}, I1{}, kt + 1);
+        }
+        if (kt < kt_end)
+            k_step(I0{}, I1{}, I0{}, kt);
+    } else {
+        for (; kt + 3 < kt_end; kt += 4) {
+            k_step(I0{}, I1{}, I0{}, kt);
+            k_step(I1{}, I2{}, I1{}, kt + 1);
+            k_step(I0{}, I3{}, I2{}, kt + 2);
+            k_step(I1{}, I0{}, I3{}, kt + 3);
+        }
+        if (kt < kt_end)
+            k_step(I0{}, I1{}, I0{}, kt);
+        if (kt + 1 < kt_end)
+            k_step(I1{}, I2{}, I1{}, kt + 1);
+        if (kt + 2 < kt_end)
+            k_step(I0{}, I3{}, I2{}, kt + 2);
     }
-    if (kt < kt_end)
-        k_step(I0{}, I1{}, I0{}, kt);
 
     gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, splitk, image0, wm, wn, h, l32, tid);
 }
@@ -2075,7 +2105,7 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
 }
 
 template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
-int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
+int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream, int nset = 2)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
@@ -2083,7 +2113,13 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream)
     blocks = (long long)a.main_wgs + (long long)a.tail_tiles * a.tail_splitk;
     {
         TimingScope ts("conv_gemm", stream);
-        DLP_LAUNCH_TIMED(ts, (conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        if constexpr (ORDER == GEMM_ORDER_TAP && ACT == ACT_CLAMP && std::is_same<T, float>::value) {
+            if (nset == 4)
+                DLP_LAUNCH_TIMED(ts, (conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT, 4>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+            else
+                DLP_LAUNCH_TIMED(ts, (conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+        } else
+            DLP_LAUNCH_TIMED(ts, (conv_gemm_f32_kernel<T, BM, BN, WM, WN, ORDER, MASK, ACT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1 && a.sk_cnt == nullptr) {
         TimingScope ts("splitk_reduce", stream);
@@ -2282,8 +2318,14 @@ int launch_tile(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, int act, hipS
 {
     if (act == ACT_GENERIC)
         return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_GENERIC>(g, a, stream);
-    if (p.order == GEMM_ORDER_TAP)
-        return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_TAP, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
+    if (p.order == GEMM_ORDER_TAP) {
+        // At most about one workgroup per CU: nothing else covers a workgroup's waits, so it keeps four K tiles in flight
+        // instead of two (measured alone on cold tensors, batch 64: 1x1 192->64 at 14x14 10.5 -> 9.3 us, 384->64 16.0 -> 13.4,
+        // 960->160 at 7x7 21.6 -> 20.3; launches with more workgroups per CU lose 3 to 10 % with four).
+        const long long wgs = (long long)a.main_wgs + (long long)a.tail_tiles * a.tail_splitk;
+        const int nset = (wgs * 5 <= (long long)device_cu_count() * 6 && a.kt_per_slice >= 8) ? 4 : 2;
+        return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_TAP, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream, nset);
+    }
     if (p.mask == GEMM_MASK_TAPS)
         return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_TAPS, ACT_CLAMP>(g, a, stream);
     return launch_inst<T, BM, BN, WM, WN, GEMM_ORDER_CHANNEL, GEMM_MASK_ROWCOL, ACT_CLAMP>(g, a, stream);
@@ -2319,6 +2361,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
     p.dense_sx = 1;
     p.patch_bf16 = 0;
     p.pp_nbr = 0;
+    p.pointwise = conv_pointwise_supported(g, activation) ? 1 : 0;
     const int cin_g = g.Cin / g.groups;
     p.M = g.Cout / g.groups;
     p.K = cin_g * g.KH * g.KW;
@@ -2553,6 +2596,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
             return fail(DLP_ERR_NOT_IMPLEMENTED, "stem convolution: needs the weight tensor and the whole batch");
         return conv_stem_launch(g, x, w, y, ep, stream);
     }
+    // few output channels, 1x1: X streams from memory straight into the matrix instructions (needs the filter as it lies in memory)
+    if (p.pointwise && w != nullptr && n_valid < 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) == 0 && ep.activation != DLP_ACT_TANH &&
+        ep.activation != DLP_ACT_SIGMOID)
+        return conv_pointwise_launch(g, x, w, y, ep, stream);
 
     GemmArgs a;
     a.x = x;

@@ -698,7 +698,7 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
         if (rc != DLP_OK)
             return rc;
         // fp32 1x1 convolutions could read w in place, but the packed tiles are there and load faster: no w, no in-place reading
-        const void *w_arg = (plan.wdirect && plan.order < GEMM_ORDER_TAP_BF16) ? nullptr : w;
+        const void *w_arg = (plan.wdirect && plan.order < GEMM_ORDER_TAP_BF16 && !plan.pointwise) ? nullptr : w;
         return conv_gemm_launch(g, plan, op->ktab, x, packed, y, ep, s, -1, part, ws_bytes, w_arg, counters);
     }
     }

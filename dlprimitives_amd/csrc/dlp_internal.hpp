@@ -177,6 +177,7 @@ struct GemmPlan {
     int wdirect;        // bf16 matrix-instruction path, 1x1: the kernel reads the weight tensor in place, nothing is packed
     int dense_pxl;      // bf16 matrix-instruction path, 1x1 stride 1 pad 0: input pixels per load of the dense loader (8, 4; 0 = gather)
     int dense_sx;       // ... 2: the dense loader on a 1x1 stride-2 convolution (dense_pxl output pixels = 2 * dense_pxl loaded)
+    int pointwise;      // 1x1 stride-1 convolution with few output channels, fp32: conv_pointwise_f32_kernel (reads x and w in place)
     int patch_bf16;     // bf16 matrix-instruction path, stride-1 3x3 "same": pixels per load of the LDS-patch kernel (8, 4; 0 = gather)
     int pp_nbr;         // ... and the blocks of that many patch rows in its largest patch
     size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded
@@ -210,6 +211,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
 // ---- few-channel strided stem convolution (conv_stem.hip) ----------------------
 bool conv_stem_supported(const ConvGeom &g);
 int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
+
+// ---- pointwise convolutions with few output channels (conv_pointwise.hip) --------
+bool conv_pointwise_supported(const ConvGeom &g, int activation);
+int conv_pointwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
 
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);

@@ -484,6 +484,65 @@ def test_inner_product_flattens_trailing_dims(gpu, oracle_mod):
     np.testing.assert_allclose(gpu.run_ip(x, w, None), oracle_mod.ip_forward(x, w, None), **TOL)
 
 
+# (cin, cout, H, W, batch): shapes that conv_pointwise_f32_kernel takes (at most 32 output channels, H * W % 4 == 0, Cin % 16 == 0,
+# at least 1024 tiles of 128 pixels)
+POINTWISE_STREAM_SHAPES = [
+    (16, 24, 56, 56, 42),    # 131 712 pixels: 1029 tiles; rows 24..31 of the block are padding
+    (144, 32, 56, 56, 42),   # K = 2 chunks + 16
+    (80, 5, 60, 60, 37),     # one chunk + 16, a last pixel tile that is cut short (133 200 pixels)
+]
+
+
+@pytest.mark.parametrize("shape", POINTWISE_STREAM_SHAPES, ids=lambda s: "%dto%d_%dx%d_b%d" % s)
+def test_pointwise_streaming_kernel(gpu, oracle_mod, shape):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    cin, cout, h, w_, b = shape
+    for act, with_bias in (("relu6", True), ("identity", False)):
+        c = case(1, 0, 1, 1, cin, cout, with_bias, 1, False)
+        c["activation"] = act
+        x, w, bias = make_tensors(c, (b, h, w_), seed=cin + cout)
+        w *= 3
+        want = oracle_conv(oracle_mod, c, x, w, bias)
+        st = gpu.settings_of(c, x.shape)
+        op = dlp.Conv2DForward.create(st, with_bias, act, "gemm")
+        xd, wd, bd = gpu.dev(x), gpu.dev(w), gpu.dev(bias)
+        ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+        y = torch.full(want.shape, float("nan"), device="cuda:0")
+        dlp.timing_reset()
+        dlp.timing_enable(True)
+        op.enqueue(xd, wd, bd, y, ws, 0.0)
+        torch.cuda.synchronize()
+        dlp.timing_enable(False)
+        kernels = [k for (_, _, k) in dlp.timing_records(kernels=True)]
+        dlp.timing_reset()
+        assert any(k.startswith("conv_pointwise_f32_kernel") for k in kernels), kernels
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+        # y = factor * y + act(...)
+        old = np.random.default_rng(1).standard_normal(want.shape).astype(np.float32)
+        y = gpu.dev(old)
+        op.enqueue(xd, wd, bd, y, ws, 0.5)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(y.cpu().numpy(), oracle_mod.apply_factor(want, old, 0.5), **TOL)
+        # y = act(conv + bias + factor * y): the residual form
+        op.accumulate_before_activation(True)
+        y = gpu.dev(old)
+        op.enqueue(xd, wd, bd, y, ws, 1.0)
+        torch.cuda.synchronize()
+        lin = oracle_conv(oracle_mod, dict(c, activation="identity"), x, w, bias) + old
+        np.testing.assert_allclose(y.cpu().numpy(), np.clip(lin, 0, 6) if act == "relu6" else lin, **TOL)
+        # weights packed ahead of time: same kernel, same result
+        op.accumulate_before_activation(False)
+        packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+        op.pack(wd, packed)
+        y = torch.full(want.shape, float("nan"), device="cuda:0")
+        op.enqueue_packed(xd, wd, packed, bd, y, ws, 0.0)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(y.cpu().numpy(), want, **TOL)
+
+
 PACKED_CASES = [  # cin, cout, k, s, p, groups, hw, batch, algo, dtype
     (64, 64, 3, 1, 1, 1, 28, 4, "gemm", "float32"),       # LDS-patch kernel, stream-K counters in the scratch
     (64, 64, 3, 1, 1, 1, 28, 4, "winograd", "float32"),
