@@ -290,9 +290,11 @@ def run_backward_workload(args):
     print(json.dumps(out))
 
 
-def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, only="", seed=2024):
+def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, only="", seed=2024, warm_seconds=0.0):
     """Times `steps` passes over the layers of a convolution workload (back to back on one stream, tensors resident),
-    then a second pass with the library's per-kernel timing.  Returns the pieces of the JSON line."""
+    then a second pass with the library's per-kernel timing.  Returns the pieces of the JSON line.
+    warm_seconds: keep running untimed passes after the `warmup` ones until this much time has gone by (the sub-millisecond
+    configurations otherwise start their timed passes before the device has left its idle clocks)."""
     import torch
 
     import dlprimitives_amd as dlp
@@ -318,6 +320,11 @@ def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, onl
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < warm_seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
@@ -394,7 +401,7 @@ def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, onl
                 kernel_ms_per_step=sum(layer_ms), roofline=roofline, table=table, nl=nl)
 
 
-def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7):
+def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_seconds=0.2):
     """One layer alone: launches back to back, each on its own x / y pair out of a ring larger than the 256 MB last-level
     cache (every launch starts cold, as inside a network), ONE event pair around all of them.  An event between two
     launches makes the first write its part of the L2 back before it ends, which inflates short kernels by microseconds;
@@ -421,6 +428,11 @@ def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7):
     ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
     reps = 3 * ring
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < warm_seconds:  # untimed launches until the device runs at its working clocks
+        for j in range(ring):
+            op.enqueue(xs[j], w, b, ys[j], ws, 0.0)
+        torch.cuda.synchronize()
     for r in range(-ring, reps):
         if r == 0:
             e0.record()
@@ -449,13 +461,16 @@ def other_configs(steps, warmup, peaks):
     from dlprimitives_amd import probe
 
     cfgs = {}
-    r = run_conv_workload("single", 16, False, steps, warmup)
-    cfgs["config1_single_conv_b16"] = compact(r, 16)
+    # a pass of these two configurations lasts 40-250 us: 200 timed passes after 0.3 s of untimed ones, so that the
+    # wall clock around them measures the kernels and not the wake-up of the device or the one synchronization
+    small = dict(steps=max(steps, 200), warmup=warmup, warm_seconds=0.3)
+    r = run_conv_workload("single", 16, False, **small)
+    cfgs["config1_single_conv_b16"] = compact(r, 16, {"steps": small["steps"], "warm_seconds": 0.3})
     for wl in ("winograd", "winograd-gemm"):
-        r = run_conv_workload(wl, 64, False, steps, warmup)
+        r = run_conv_workload(wl, 64, False, **small)
         cfgs["config3_%s" % wl.replace("-", "_")] = compact(r, 64, {"layers": [
             {k: row[k] for k in ("name", "ms", "main_kernel_ms", "tflops", "tflops_issued", "frac_of_roofline", "kernel") if k in row} for row in r["table"]]})
-    r = run_conv_workload("mobilenet", 64, False, steps, warmup)
+    r = run_conv_workload("mobilenet", 64, False, max(steps, 100), warmup, warm_seconds=0.3)
     rows = []
     for L, row in zip(r["layer_list"], r["table"]):
         e = {k: row[k] for k in ("name", "kernel")}

@@ -502,8 +502,15 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     ConvAlgo chosen = ALGO_GEMM;
     // bf16 tensors whose GEMM runs on the bf16 matrix instruction are faster there than through
     // Winograd (whose transforms force fp32 matrix instructions): automatic choice keeps gemm
-    const bool bf16_mfma = conv_gemm_plan(g, activation).order >= GEMM_ORDER_TAP_BF16;
-    if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && cfg->channels_in >= 8 && cfg->channels_out >= 8))
+    const GemmPlan gplan = conv_gemm_plan(g, activation);
+    const bool bf16_mfma = gplan.order >= GEMM_ORDER_TAP_BF16;
+    // Where the reference rule would pick Winograd (src/core/conv.cpp:714-718), the automatic choice here keeps "gemm" for the layers
+    // the LDS-patch kernel serves with fewer than 128 input channels.  Whole layers at batch 64, weights transformed in the call,
+    // cold tensors, gemm / winograd: 64->64 at 56x56 126 / 130 us, 128->128 at 28x28 120 / 114 us, 256->256 at 14x14 120 / 107 us,
+    // 512->512 at 7x7 122 / 105 us: Winograd's transforms cost a fixed amount per pixel and channel, the multiplications they save
+    // grow with the channel count.
+    const bool gemm_faster = gplan.patch && cfg->channels_in / cfg->groups < 128;
+    if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && !gemm_faster && cfg->channels_in >= 8 && cfg->channels_out >= 8))
         chosen = ALGO_WINOGRAD;
     else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))
         chosen = ALGO_DEPTHWISE;

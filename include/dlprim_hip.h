@@ -119,7 +119,12 @@ int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4
 /* ---- core::Conv2DForward::create, include/dlprim/core/conv.hpp:49-53,
  *      src/core/conv.cpp:704-729.  algo: NULL, "", "auto", "gemm", "winograd",
  *      "depthwise_separable"; a requested but incompatible algorithm falls back
- *      to "gemm" exactly as the reference does (:725-727). -------------------- */
+ *      to "gemm" exactly as the reference does (:725-727).  The automatic
+ *      choice ("" / "auto") differs from the reference's rule (:714-718) in one
+ *      place: a Winograd-compatible fp32 convolution with fewer than 128 input
+ *      channels that the LDS-patch GEMM kernel serves (image at most 62 wide,
+ *      Cin a multiple of 16, more than 32 filters) stays "gemm", which is the
+ *      faster of the two there on gfx950; algo() reports what was chosen. ------ */
 int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activation,
                           const char *algo, dlp_conv2d_fwd **out);
 
