@@ -1203,11 +1203,15 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
 // B tiles are dealt to the wavefronts in turn (LW wavefronts per tile).
 // SX = 2: the same for 1x1 stride-2 convolutions whose output width is a multiple of PXL: a lane
 // loads 2 * PXL consecutive input pixels of an even input row and keeps the even ones.
-template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL, int SX = 1>
+// XT = 1: a.x is the channels-last copy of the input ([image][pixel][channel], made by stage_channels_last_kernel; a.H, a.W,
+// a.sh, a.sw describe that copy): a pixel's 32 channels of a K tile are 64 consecutive bytes, four 16-byte pieces that go to
+// LDS as they come, exactly like the weight tile.  Any kernel extent, stride, padding and image size.
+template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL, int SX = 1, int XT = 0>
 __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
 {
     static_assert(PXL == 0 || ((PXL == 2 || PXL == 4 || PXL == 8) && PXL * SX >= 4 && PXL * SX <= 8 && ORDER == GEMM_ORDER_TAP_BF16),
                   "dense loader variants: loads of 8 or 16 bytes");
+    static_assert(XT == 0 || (PXL == 0 && ORDER == GEMM_ORDER_TAP_BF16), "the channels-last loader is a tap-major gather");
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -1288,6 +1292,38 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
             } else {
                 my = ry;
                 mx = rx;
+            }
+        }
+    }
+
+    // channels-last loader: B_PC 16-byte pieces per thread and K tile; piece = (pixel (tid / 4) + 64 j, channels 8 (tid % 4) ..)
+    constexpr int B_PC = BN * 4 / kThreads;
+    uint32_t xbase[B_PC], xmask[B_PC];
+    if constexpr (XT) {
+#pragma unroll
+        for (int j = 0; j < B_PC; j++) {
+            const int n = n0 + (tid >> 2) + j * (kThreads / 4);
+            xbase[j] = kOutOfRange;
+            xmask[j] = 0;
+            if (n < a.N) {
+                const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
+                const int pix = n - b * a.OHW;
+                const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
+                const int ox = pix - oy * a.OW;
+                const int iy0 = oy * a.sh - a.ph;
+                const int ix0 = ox * a.sw - a.pw;
+                xbase[j] = (uint32_t)((((b * a.H + oy * a.sh) * a.W + ox * a.sw) * a.Cin + g * a.Cin_g) * 2 + (tid & 3) * 16);
+                uint32_t rx = 0;
+                for (int kx = 0; kx < a.KW; kx++) {
+                    const int xx = ix0 + kx * a.dw;
+                    if (xx >= 0 && xx < a.W)
+                        rx |= 1u << kx;
+                }
+                for (int ky = 0; ky < a.KH; ky++) {
+                    const int yy = iy0 + ky * a.dh;
+                    if (yy >= 0 && yy < a.H)
+                        xmask[j] |= rx << (ky * a.KW);
+                }
             }
         }
     }
@@ -1389,6 +1425,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     u32x4 ra[NSET][A_LD];
     uint32_t rb[NSET][B_LD]; // one bf16 each, zero extended
     uint32_t vsel[NSET];
+    u32x4 rbx[NSET][B_PC];   // channels-last loader: the pieces as they come
 
     auto load_half = [&](auto set, int kt, auto half_c) {
         constexpr int S = decltype(set)::value;
@@ -1402,6 +1439,16 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         if constexpr (PXL > 0) {
             if (Q == 1 && my_tile(kt))
                 load_b(set, kt);
+        } else if constexpr (XT) {
+            // table entry of a K tile: {byte offset of (tap, channel block) in the channels-last copy, tap bit, -, -}
+            ConstInt *e = ktab + kt * 4;
+            const uint32_t xoff = (uint32_t)e[0], tap = (uint32_t)e[1];
+            constexpr int PH = B_PC / 2 ? B_PC / 2 : 1;
+#pragma unroll
+            for (int j = Q * PH; j < (Q + 1) * PH && j < B_PC; j++) {
+                const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)xmask[j], tap, 1u);
+                rbx[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, opaque((xbase[j] & m) | (kOutOfRange & ~m)), xoff, 0));
+            }
         } else if (ORDER == GEMM_ORDER_TAP_BF16) {
             // table entry of a K tile: {x byte offset of (channel block, tap), tap bit, -, -}
             ConstInt *e = ktab + kt * 4;
@@ -1441,6 +1488,13 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         if constexpr (PXL > 0) {
             if (Q == 0 && my_tile(kt))
                 store_b(set, buf_c);
+            return;
+        }
+        if constexpr (XT) {
+            constexpr int PH = B_PC / 2 ? B_PC / 2 : 1;
+#pragma unroll
+            for (int j = Q * PH; j < (Q + 1) * PH && j < B_PC; j++)
+                *(u32x4 *)&Bs[BUF][(tid >> 2) + j * (kThreads / 4)][(tid & 3) * 8] = rbx[S][j];
             return;
         }
 #pragma unroll
@@ -1811,6 +1865,74 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
 }
 
+// Channels-last copy of a bf16 input for conv_gemm_bf16_kernel<..., XT = 1>: xt[b][py][px][c] = x[b][c][py * sy][px * sx]
+// (sy, sx > 1 only for a 1x1 convolution, whose stride then lives in the copy).  One workgroup transposes 64 channels of an
+// image through LDS and writes 16-byte pieces (8 channels of a pixel; 8 lanes = the 128 bytes of a pixel's 64 channels).
+//  MODE 0: 64 pixels per workgroup, read one element at a time (any size and alignment, strided copies);
+//  MODE 1: the whole image (at most 256 pixels): 64 channels x P pixels are one contiguous run, read in 16-byte pieces;
+//  MODE 2: 64 pixels per workgroup, P a multiple of 8: 16-byte pieces of 8 pixels.
+// MODE 1 and 2 need x 16-byte aligned; all modes need xt 16-byte aligned and C a multiple of 8.
+struct StageArgs {
+    const uint16_t *x;
+    uint16_t *xt;
+    int C, H, W, PH, PW, sy, sx; // the copy is PH x PW pixels
+    uint32_t pw_magic, pw_shift;
+};
+constexpr int kStageFlatPixels = 256;
+template <int MODE>
+__global__ __launch_bounds__(256) void stage_channels_last_kernel(StageArgs a)
+{
+    constexpr int PITCH = 66; // 16-bit elements per LDS row (MODE 0, 2): 33 dwords, so that the 8 x 8 reads of a piece spread over the banks
+    __shared__ __attribute__((aligned(16))) uint16_t tile[MODE == 1 ? 64 * kStageFlatPixels : 64 * PITCH];
+    const int P = a.PH * a.PW;
+    const int p0 = MODE == 1 ? 0 : (int)blockIdx.x * 64, c0 = (int)blockIdx.y * 64, b = (int)blockIdx.z;
+    const int tid = (int)threadIdx.x;
+    const int pitch = MODE == 1 ? P : PITCH;
+    const int nch = min(64, a.C - c0);
+    if constexpr (MODE == 0) {
+        const int lane = tid & 63, row = tid >> 6;
+        const int p = p0 + lane;
+        int src = p;
+        if (a.sy != 1 || a.sx != 1) {
+            const int py = (int)fast_div((uint32_t)p, a.pw_magic, a.pw_shift);
+            src = py * a.sy * a.W + (p - py * a.PW) * a.sx;
+        }
+        const uint16_t *xp = a.x + ((size_t)b * a.C + c0) * ((size_t)a.H * a.W) + src;
+#pragma unroll 4
+        for (int c = row; c < 64; c += 4)
+            if (p < P && c < nch)
+                tile[c * PITCH + lane] = xp[(size_t)c * ((size_t)a.H * a.W)];
+    } else if constexpr (MODE == 1) {
+        const u32x4 *xp = reinterpret_cast<const u32x4 *>(a.x + ((size_t)b * a.C + c0) * (size_t)P);
+        const int pieces = nch * P / 8; // nch is a multiple of 8
+        for (int q = tid; q < pieces; q += 256)
+            reinterpret_cast<u32x4 *>(tile)[q] = xp[q];
+    } else {
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int q = tid + 256 * r, c = q >> 3, pg = q & 7;
+            if (c < nch && p0 + 8 * pg < P) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(a.x + ((size_t)b * a.C + c0 + c) * (size_t)P + p0 + 8 * pg);
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    *reinterpret_cast<uint32_t *>(&tile[c * PITCH + 8 * pg + 2 * d]) = v[d];
+            }
+        }
+    }
+    __syncthreads();
+    const int npx = MODE == 1 ? P : min(64, P - p0);
+    for (int q = tid; q < npx * 8; q += 256) {
+        const int oct = q & 7, p = q >> 3;
+        if (oct * 8 < nch) {
+            u32x4 v;
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                v[d] = (uint32_t)tile[(oct * 8 + 2 * d) * pitch + p] | ((uint32_t)tile[(oct * 8 + 2 * d + 1) * pitch + p] << 16);
+            *reinterpret_cast<u32x4 *>(a.xt + ((size_t)b * P + p0 + p) * a.C + c0 + oct * 8) = v;
+        }
+    }
+}
+
 // Sums the split-K slices in slice order (deterministic) and applies the epilogue.
 // One grid row (blockIdx.y) per output channel, four consecutive pixels per thread:
 // 16-byte loads of the partial sums, no 64-bit index arithmetic.
@@ -2133,25 +2255,23 @@ int launch_inst(const ConvGeom &g, GemmArgs &a, hipStream_t stream, int nset = 2
 
 typedef void (*Bf16Kernel)(GemmArgs);
 template <int BM, int BN, int WM, int WN>
-Bf16Kernel bf16_kernel_of_tile(int order, int pxl, int sx)
+Bf16Kernel bf16_kernel_of_tile(int order, int pxl, int sx, bool xt)
 {
     if (order == GEMM_ORDER_TAP_BF16 && sx == 2 && pxl == 4)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 4, 2>;
-    if constexpr (BN == 128) {
-        if (order == GEMM_ORDER_TAP_BF16 && sx == 2 && pxl == 2)
-            return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 2, 2>;
-    }
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 8)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 8>;
     if (order == GEMM_ORDER_TAP_BF16 && pxl == 4)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_DENSE_NSET, 4>;
+    if (order == GEMM_ORDER_TAP_BF16 && xt)
+        return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET, 0, 1, 1>;
     if (order == GEMM_ORDER_TAP_BF16)
         return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_TAP_BF16, ACT_CLAMP, DLP_BF16_NSET, 0>;
     return conv_gemm_bf16_kernel<BM, BN, WM, WN, GEMM_ORDER_CHANNEL_BF16, ACT_CLAMP, 2, 0>;
 }
-Bf16Kernel bf16_kernel(int tile, int order, int pxl, int sx)
+Bf16Kernel bf16_kernel(int tile, int order, int pxl, int sx, bool xt)
 {
-    return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl, sx) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl, sx);
+    return tile == 2 ? bf16_kernel_of_tile<128, 128, 2, 2>(order, pxl, sx, xt) : bf16_kernel_of_tile<64, 256, 1, 4>(order, pxl, sx, xt);
 }
 
 // Largest number of patch rows any pixel tile of conv_patch_bf16_kernel needs (same arithmetic as the kernel).
@@ -2213,14 +2333,61 @@ int launch_patch_bf16(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStre
     return DLP_OK;
 }
 
-int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a, hipStream_t stream)
+// The channels-last copy that the XT kernels read: geometry, and size in bytes (256-byte rounded).
+struct XtGeom {
+    int H, W, sy, sx; // pixels of the copy; strides of the copy (1x1 convolutions without padding fold theirs into it)
+};
+XtGeom xt_geom(const ConvGeom &g)
+{
+    if (g.KH == 1 && g.KW == 1 && g.ph == 0 && g.pw == 0)
+        return {g.OH, g.OW, g.sh, g.sw};
+    return {g.H, g.W, 1, 1};
+}
+size_t xt_bytes(const ConvGeom &g, int batch)
+{
+    const XtGeom t = xt_geom(g);
+    return ((size_t)batch * t.H * t.W * g.Cin * sizeof(bf16_t) + 255) / 256 * 256;
+}
+
+int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a, hipStream_t stream, void *xt)
 {
     long long blocks = (long long)a.mtiles * a.ntiles * g.groups * a.splitk;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
+    if (xt != nullptr) {
+        const XtGeom t = xt_geom(g);
+        StageArgs sa;
+        sa.x = (const uint16_t *)a.x;
+        sa.xt = (uint16_t *)xt;
+        sa.C = g.Cin; sa.H = g.H; sa.W = g.W; sa.PH = t.H; sa.PW = t.W; sa.sy = t.sy; sa.sx = t.sx;
+        make_magic((uint32_t)t.W, sa.pw_magic, sa.pw_shift);
+        if (g.B > 65535 || (g.Cin + 63) / 64 > 65535)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last staging: more than 65535 images or channel blocks");
+        {
+            TimingScope ts("stage_input", stream);
+            const int P = t.H * t.W;
+            const bool whole = t.sy == 1 && t.sx == 1 && ((uintptr_t)a.x & 15) == 0;
+            const dim3 grid64((unsigned)((P + 63) / 64), (unsigned)((g.Cin + 63) / 64), (unsigned)g.B);
+            if (whole && P <= kStageFlatPixels)
+                DLP_LAUNCH_TIMED(ts, stage_channels_last_kernel<1>, dim3(1, grid64.y, grid64.z), dim3(256), 0, stream, sa);
+            else if (whole && P % 8 == 0)
+                DLP_LAUNCH_TIMED(ts, stage_channels_last_kernel<2>, grid64, dim3(256), 0, stream, sa);
+            else
+                DLP_LAUNCH_TIMED(ts, stage_channels_last_kernel<0>, grid64, dim3(256), 0, stream, sa);
+        }
+        // the convolution the matrix kernel now sees: the copy as input, strides that the copy has taken over set to 1
+        a.x = xt;
+        a.x_bytes = (uint32_t)((size_t)g.B * t.H * t.W * g.Cin * sizeof(bf16_t));
+        a.H = t.H;
+        a.W = t.W;
+        a.sh = g.sh / t.sy;
+        a.sw = g.sw / t.sx;
+        a.x_shift = (uint32_t)(((size_t)g.ph * t.W + g.pw) * g.Cin * sizeof(bf16_t));
+        a.ktab += (p.nkt + 2) * BK2; // the second table of conv_gemm_fill_ktab
+    }
     {
         TimingScope ts("conv_gemm", stream);
-        const Bf16Kernel kernel = bf16_kernel(p.tile, p.order, pxl, p.dense_sx);
+        const Bf16Kernel kernel = bf16_kernel(p.tile, p.order, pxl, p.dense_sx, xt != nullptr);
         DLP_LAUNCH_TIMED(ts, kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
     }
     if (a.splitk > 1) {
@@ -2361,6 +2528,7 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
     p.dense_sx = 1;
     p.patch_bf16 = 0;
     p.pp_nbr = 0;
+    p.xt = 0;
     p.pointwise = conv_pointwise_supported(g, activation) ? 1 : 0;
     const int cin_g = g.Cin / g.groups;
     p.M = g.Cout / g.groups;
@@ -2392,7 +2560,9 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
             p.dense_pxl = (g.H * g.W) % 8 == 0 ? 8 : 4;
         // 1x1 stride 2 on even-sized images: runs of 4 (2) output pixels of a row = 8 (4) consecutive input pixels
         if (tap_major && g.KH == 1 && g.KW == 1 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.W % 2 == 0 && g.H % 2 == 0) {
-            const int pxl = g.OW % 4 == 0 ? 4 : (g.OW % 2 == 0 && p.tile == 2) ? 2 : 0;
+            // (runs of 2 output pixels exist as a kernel variant, but the channels-last staging below is faster there:
+            // 80 against 88 us on 512->1024 at 28x28, batch 128)
+            const int pxl = g.OW % 4 == 0 ? 4 : 0;
             if (pxl) {
                 p.dense_pxl = pxl;
                 p.dense_sx = 2;
@@ -2409,6 +2579,9 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
                 p.pp_nbr = nbr;
             }
         }
+        // everything else in the tap-major order (strided and dilated kernels, odd image sizes): channels-last staging
+        p.xt = tap_major && p.dense_pxl == 0 && p.patch_bf16 == 0 && g.Cin <= 65535 * 64 &&
+               (size_t)g.H * g.W * g.Cin * sizeof(bf16_t) < kOutOfRange / 2;
     }
     p.BM = 64;
     p.BN = 64;
@@ -2453,6 +2626,19 @@ void conv_gemm_fill_ktab(const ConvGeom &g, int activation, KTabEntry *tab_entri
                 }
         for (; (size_t)(4 * t + 1) < words; t++)
             tab[4 * t + 1] = 31; // bit 31 of a tap mask is never set (at most 31 taps use this order)
+        if (p.xt) {
+            // second table, (nkt + 2) * 32 words in (the first uses 4 * (nkt + 2) of them): the same K tiles as byte offsets into
+            // the channels-last copy of the input
+            const XtGeom xg = xt_geom(g);
+            int32_t *tab2 = tab + (p.nkt + 2) * BK2;
+            t = 0;
+            for (int cb = 0; cb < cin_g / cblock; cb++)
+                for (int ky = 0; ky < g.KH; ky++)
+                    for (int kx = 0; kx < g.KW; kx++, t++) {
+                        tab2[4 * t + 0] = ((ky * g.dh * xg.W + kx * g.dw) * g.Cin + cb * cblock) * esize;
+                        tab2[4 * t + 1] = ky * g.KW + kx;
+                    }
+        }
         return;
     }
     size_t k = 0;
@@ -2480,7 +2666,7 @@ size_t conv_gemm_workspace_bytes(const ConvGeom &g, int activation)
     a.Cout = g.Cout;
     a.nkt = p.nkt;
     plan_split(p, a, g.groups, true, (size_t)-1);
-    return p.wpack_bytes + split_total_bytes(p, a, g.groups);
+    return p.wpack_bytes + split_total_bytes(p, a, g.groups) + (p.xt ? xt_bytes(g, B) : 0);
 }
 
 namespace {
@@ -2651,6 +2837,15 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     const int act = generic_act(ep.activation) ? ACT_GENERIC : ACT_CLAMP;
     if (p.patch)
         return launch_patch(g, p, a, stream, part_ws, part_bytes, own_counters);
+    // workspace behind the packed weights, bf16 kernels: channels-last copy of the input | split-K partial sums
+    void *xt = nullptr;
+    if (p.xt && part_ws != nullptr && part_bytes >= xt_bytes(g, g.B) && ((uintptr_t)part_ws & 15) == 0 && n_valid < 0 &&
+        xt_bytes(g, g.B) + ((size_t)g.ph * g.W + g.pw) * g.Cin * esize < kOutOfRange) {
+        xt = part_ws;
+        part_ws = (char *)part_ws + xt_bytes(g, g.B);
+        part_bytes -= xt_bytes(g, g.B);
+        a.part = (float *)part_ws;
+    }
     plan_split(p, a, g.groups, part_ws != nullptr, part_bytes);
     a.sk_cnt = nullptr;
     a.part_bytes = 0;
@@ -2677,7 +2872,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         if (p.patch_bf16 && ((uintptr_t)x & 3) == 0)
             return launch_patch_bf16(g, p, a, stream);
         const int pxl = ((uintptr_t)x & 3) == 0 ? p.dense_pxl : 0;
-        return launch_bf16_mfma(g, p, pxl, a, stream);
+        return launch_bf16_mfma(g, p, pxl, a, stream, xt);
     }
     return with_tile(p.tile, [&](auto bm, auto bn, auto wm, auto wn) {
         if (g.dtype == DLP_BFLOAT16)

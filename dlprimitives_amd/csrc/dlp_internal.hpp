@@ -180,6 +180,9 @@ struct GemmPlan {
     int pointwise;      // 1x1 stride-1 convolution with few output channels, fp32: conv_pointwise_f32_kernel (reads x and w in place)
     int patch_bf16;     // bf16 matrix-instruction path, stride-1 3x3 "same": pixels per load of the LDS-patch kernel (8, 4; 0 = gather)
     int pp_nbr;         // ... and the blocks of that many patch rows in its largest patch
+    int xt;             // bf16 matrix-instruction path, neither dense nor patch: the input is first copied channels-last into the workspace
+                        // ([image][pixel][channel], a 1x1 convolution's stride folded into the copy), so that a K tile of a pixel
+                        // is 64 consecutive bytes and loads as 16-byte pieces instead of 32 two-byte gathers
     size_t wpack_bytes; // packed weights [group][m tile][K tile][16][BM] floats, 256-byte rounded
 };
 GemmPlan conv_gemm_plan(const ConvGeom &g, int activation);

@@ -69,9 +69,14 @@ CASES = [
     (case(3, 1, 1, 1, 64, 256, True, 2, True), (2, 12, 12)),     # two groups of 32 channels: a single stage
     (case(3, 1, 1, 1, 32, 128, True, 1, True), (5, 8, 8)),       # images smaller than a tile: three segments
     (case(3, 1, 1, 1, 64, 64, True, 1, True), (1, 4, 60)),       # wide, flat image
-    # per-pixel loader (strided or size-changing)
+    # channels-last staging (strided or size-changing kernels, odd image sizes): the input is copied [image][pixel][channel] first
     (case(3, 0, 1, 1, 32, 64, True, 1, True), (2, 12, 12)),
-    (case(3, 1, 2, 1, 256, 256, True, 1, True), (2, 28, 28)),
+    (case(3, 1, 2, 1, 256, 256, True, 1, True), (2, 28, 28)),    # 784 pixels: 64-pixel transposition tiles, 16-byte reads, last tile partial
+    (case(3, 1, 2, 1, 96, 64, True, 1, True), (2, 17, 19)),      # 323 pixels, odd: element-wise reads; 96 channels: half a channel block
+    (case(3, 1, 1, 1, 96, 160, False, 1, True), (3, 7, 7)),      # whole-image transposition (49 pixels), 96 channels
+    (case(1, 0, 2, 1, 64, 128, True, 1, True), (3, 15, 15)),     # 1x1 stride 2 on an odd image: the copy takes the stride over
+    (case(1, 0, (2, 1), 1, 64, 64, True, 1, True), (2, 9, 10)),  # ... in one direction only
+    (case(3, (2, 0), (1, 2), (2, 1), 64, 96, True, 2, True), (2, 11, 14)),  # groups, dilation, uneven padding and stride together
 ]
 
 
