@@ -12,6 +12,7 @@ from .capi import (  # noqa: F401
     Conv2DBackwardFilter,
     Conv2DForward,
     Conv2DSettings,
+    DepthwisePointwiseForward,
     DlprimError,
     IPForward,
     IPSettings,

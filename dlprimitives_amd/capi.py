@@ -267,6 +267,53 @@ class Conv2DForward:
             self._h = None
 
 
+class DepthwisePointwiseForward:
+    """Depthwise 3x3 + pointwise 1x1 convolution in one launch (dlp_dwpw_fwd_*): no counterpart in the reference,
+    which runs them as two Convolution2D operators with the depthwise result written to memory in between."""
+
+    def __init__(self, handle, settings, channels_out):
+        self._h = handle
+        self.settings = settings
+        self.channels_out = channels_out
+
+    @staticmethod
+    def supported(settings, dw_activation, channels_out, pw_activation):
+        L = lib()
+        L.dlp_dwpw_fwd_supported.argtypes = [ctypes.POINTER(_Settings), ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        c = settings._c()
+        return bool(L.dlp_dwpw_fwd_supported(ctypes.byref(c), _act(dw_activation), int(channels_out), _act(pw_activation)))
+
+    @staticmethod
+    def create(settings, dw_bias, dw_activation, channels_out, pw_bias, pw_activation="identity"):
+        """settings: the depthwise layer (groups = channels, kernel 3, pad 1, stride 1 or 2, shape of x)"""
+        L = lib()
+        L.dlp_dwpw_fwd_create.argtypes = [ctypes.POINTER(_Settings), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.POINTER(ctypes.c_void_p)]
+        L.dlp_dwpw_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+        L.dlp_dwpw_fwd_set_accumulate_first.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        L.dlp_dwpw_fwd_destroy.argtypes = [ctypes.c_void_p]
+        L.dlp_dwpw_fwd_destroy.restype = None
+        h = ctypes.c_void_p()
+        c = settings._c()
+        _check(L.dlp_dwpw_fwd_create(ctypes.byref(c), int(bool(dw_bias)), _act(dw_activation), int(channels_out), int(bool(pw_bias)),
+                                     _act(pw_activation), ctypes.byref(h)))
+        return DepthwisePointwiseForward(h, settings, int(channels_out))
+
+    def accumulate_before_activation(self, on=True):
+        _check(lib().dlp_dwpw_fwd_set_accumulate_first(self._h, int(bool(on))))
+
+    def enqueue(self, x, dw_w, dw_bias, pw_w, pw_bias, y, factor=0.0, stream=None):
+        xs = (ctypes.c_int * 4)(*x.shape)
+        _check(lib().dlp_dwpw_fwd_enqueue(self._h, xs, _ptr(x), _ptr(dw_w), _ptr(dw_bias), _ptr(pw_w), _ptr(pw_bias), _ptr(y), float(factor),
+                                          _stream(stream)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().dlp_dwpw_fwd_destroy(self._h)
+            self._h = None
+
+
 class _Conv2DBackward:
     _kind = None
 

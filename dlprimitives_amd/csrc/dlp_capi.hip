@@ -722,6 +722,90 @@ void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op)
     delete op;
 }
 
+// ---- depthwise 3x3 + pointwise 1x1 in one launch (conv_dwpw.hip) ----
+struct dlp_dwpw_fwd {
+    dlp_conv2d_settings cfg; // the depthwise layer
+    int channels_out;        // filters of the pointwise layer
+    bool dw_bias, pw_bias;
+    int dw_activation, pw_activation;
+    int accumulate_first;
+};
+
+int dlp_dwpw_fwd_supported(const dlp_conv2d_settings *dw_cfg, int dw_activation, int channels_out, int pw_activation)
+{
+    if (!dw_cfg || !valid_activation(dw_activation) || !valid_activation(pw_activation) || channels_out <= 0)
+        return 0;
+    if (dw_cfg->channels_in <= 0 || dw_cfg->groups <= 0 || dw_cfg->channels_in % dw_cfg->groups != 0 || dw_cfg->channels_out % dw_cfg->groups != 0)
+        return 0;
+    ConvGeom g;
+    if (make_geom(*dw_cfg, dw_cfg->shape, g) != DLP_OK)
+        return 0;
+    return conv_dwpw_supported(g, channels_out, dw_activation, pw_activation) ? 1 : 0;
+}
+
+int dlp_dwpw_fwd_create(const dlp_conv2d_settings *dw_cfg, int dw_bias, int dw_activation, int channels_out, int pw_bias, int pw_activation,
+                        dlp_dwpw_fwd **out)
+{
+    DLP_REQUIRE(dw_cfg != nullptr && out != nullptr, "null argument");
+    *out = nullptr;
+    DLP_REQUIRE(dw_cfg->channels_in > 0 && dw_cfg->channels_out > 0 && dw_cfg->groups > 0 && channels_out > 0, "channels/groups must be positive");
+    DLP_REQUIRE(dw_cfg->channels_in % dw_cfg->groups == 0 && dw_cfg->channels_out % dw_cfg->groups == 0, "channels not divisible by groups");
+    DLP_REQUIRE(valid_activation(dw_activation) && valid_activation(pw_activation), "unknown activation");
+    ConvGeom g;
+    int rc = make_geom(*dw_cfg, dw_cfg->shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    if (!conv_dwpw_supported(g, channels_out, dw_activation, pw_activation))
+        return fail(DLP_ERR_NOT_IMPLEMENTED,
+                    "fused depthwise + pointwise: float_data, depthwise 3x3 with padding 1 and stride 1 or 2 on images up to 56 wide (width a multiple of 4, "
+                    "or of 2 up to 16), channels a multiple of 8, at most 128 filters, identity / relu / relu6; run the two operators separately otherwise");
+    dlp_dwpw_fwd *op = new (std::nothrow) dlp_dwpw_fwd();
+    if (!op)
+        return fail(DLP_ERR_RUNTIME, "out of host memory");
+    op->cfg = *dw_cfg;
+    op->channels_out = channels_out;
+    op->dw_bias = dw_bias != 0;
+    op->pw_bias = pw_bias != 0;
+    op->dw_activation = dw_activation;
+    op->pw_activation = pw_activation;
+    op->accumulate_first = 0;
+    *out = op;
+    return DLP_OK;
+}
+
+int dlp_dwpw_fwd_set_accumulate_first(dlp_dwpw_fwd *op, int on)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    op->accumulate_first = on ? 1 : 0;
+    return DLP_OK;
+}
+
+int dlp_dwpw_fwd_enqueue(dlp_dwpw_fwd *op, const int x_shape[4], const void *x, const void *dw_w, const void *dw_bias, const void *pw_w,
+                         const void *pw_bias, void *y, float factor, void *stream)
+{
+    DLP_REQUIRE(op != nullptr && x_shape != nullptr, "null argument");
+    DLP_REQUIRE(x_shape[0] >= 0, "negative batch");
+    DLP_REQUIRE(x_shape[1] == op->cfg.channels_in && x_shape[2] == op->cfg.shape[2] && x_shape[3] == op->cfg.shape[3],
+                "input shape differs from the shape given at create (only the batch may change)");
+    DLP_REQUIRE((dw_bias != nullptr) == op->dw_bias && (pw_bias != nullptr) == op->pw_bias,
+                "bias pointers must be given exactly when the op was created with that bias");
+    ConvGeom g;
+    int rc = make_geom(op->cfg, x_shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    if (g.B == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && dw_w != nullptr && pw_w != nullptr && y != nullptr, "null tensor pointer");
+    Epilogue ep;
+    ep.bias = (const float *)pw_bias;
+    ep.factor = factor;
+    ep.activation = op->pw_activation;
+    ep.accumulate_first = op->accumulate_first;
+    return conv_dwpw_launch(g, op->channels_out, x, dw_w, (const float *)dw_bias, op->dw_activation, pw_w, y, ep, (hipStream_t)stream);
+}
+
+void dlp_dwpw_fwd_destroy(dlp_dwpw_fwd *op) { delete op; }
+
 int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_ip_fwd **out)
 {
     DLP_REQUIRE(cfg != nullptr && out != nullptr, "null argument");

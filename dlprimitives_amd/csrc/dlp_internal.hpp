@@ -219,6 +219,12 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
 bool conv_pointwise_supported(const ConvGeom &g, int activation);
 int conv_pointwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
 
+// ---- depthwise 3x3 + pointwise 1x1 in one launch (conv_dwpw.hip) ----------------
+// g: the depthwise layer; M: filters of the pointwise layer; act1 / ep.activation: the two activations; bd: depthwise bias or null
+bool conv_dwpw_supported(const ConvGeom &g, int M, int act1, int act2);
+int conv_dwpw_launch(const ConvGeom &g, int M, const void *x, const void *wd, const float *bd, int act1, const void *wp, void *y, const Epilogue &ep,
+                     hipStream_t stream);
+
 // ---- depthwise (conv_depthwise.hip) ------------------------------------------
 bool depthwise_supported(const ConvGeom &g);
 int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);

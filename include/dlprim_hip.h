@@ -170,6 +170,26 @@ int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
 
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
+/* ---- Depthwise 3x3 convolution followed by a pointwise (1x1) convolution in one launch.  No counterpart in the
+ *      reference, where these are two Convolution2D operators ("depthwise_separable", then the 1x1 path of "gemm") with a
+ *      tensor as large as x written and read back between them; here that tensor never reaches memory:
+ *        t = dw_act(depthwise3x3(x, dw_w) + dw_bias),  y = pw_act(pw_w * t + pw_bias),  y = factor != 0 ? factor * y + that : that
+ *      t is bit for bit what the depthwise operator alone would write; the pointwise sum is accumulated in fp32 like "gemm".
+ *      `dw_cfg` describes the depthwise layer (groups = channels_in = channels_out, kernel 3, pad 1, stride 1 or 2, shape =
+ *      shape of x); x [B,C,H,W], dw_w [C,1,3,3], dw_bias [C], pw_w [channels_out,C,1,1], pw_bias [channels_out],
+ *      y [B,channels_out,OH,OW].  float_data, W <= 56 (a multiple of 4, or of 2 up to 16), C a multiple of 8,
+ *      channels_out <= 128, activations identity / relu / relu6: create returns DLP_ERR_NOT_IMPLEMENTED otherwise
+ *      (dlp_dwpw_fwd_supported tells beforehand) and the caller keeps the two operators.  No workspace. ------------------ */
+typedef struct dlp_dwpw_fwd dlp_dwpw_fwd;
+int dlp_dwpw_fwd_supported(const dlp_conv2d_settings *dw_cfg, int dw_activation, int channels_out, int pw_activation);
+int dlp_dwpw_fwd_create(const dlp_conv2d_settings *dw_cfg, int dw_bias, int dw_activation, int channels_out, int pw_bias,
+                        int pw_activation, dlp_dwpw_fwd **out);
+/* y = pw_act(conv + pw_bias + factor * y), as dlp_conv2d_fwd_set_accumulate_first */
+int dlp_dwpw_fwd_set_accumulate_first(dlp_dwpw_fwd *op, int on);
+int dlp_dwpw_fwd_enqueue(dlp_dwpw_fwd *op, const int x_shape[4], const void *x, const void *dw_w, const void *dw_bias,
+                         const void *pw_w, const void *pw_bias, void *y, float factor, void *stream);
+void dlp_dwpw_fwd_destroy(dlp_dwpw_fwd *op);
+
 /* ---- Softmax::forward, src/ops/softmax.cpp:189-222 (core::softmax_forward, src/core/loss.cpp:13-40):
  *      softmax (or log-softmax) over dimension 1 of x[batch][classes][inner] (inner = 1 for a matrix);
  *      y may be x ------------------------------------------------------------------------------- */
