@@ -443,6 +443,100 @@ def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_s
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
+def mobilenet_pairs(layer_list):
+    """(index of a depthwise layer, index of the pointwise layer that can follow it): same channels, the depthwise
+    layer's output size; every layer in at most one pair."""
+    pairs, used = [], set()
+    for i, d in enumerate(layer_list):
+        if d["algo"] != "depthwise_separable":
+            continue
+        for j, p in enumerate(layer_list):
+            if j not in used and p["kernel"] == 1 and p["groups"] == 1 and p["cin"] == d["cout"] and p["hw"] == d["ohw"]:
+                pairs.append((i, j))
+                used.add(j)
+                break
+    return pairs
+
+
+def fused_pair_op(D, P, batch):
+    """The depthwise layer D and the pointwise layer P as ONE operator (dlp_dwpw_fwd_*), or None where the library keeps them apart."""
+    import dlprimitives_amd as dlp
+
+    st = dlp.Conv2DSettings(D["cin"], D["cout"], 3, D["stride"], 1, 1, D["groups"], (batch, D["cin"], D["hw"], D["hw"]))
+    if D["kernel"] != 3 or D["pad"] != 1 or not dlp.DepthwisePointwiseForward.supported(st, D["activation"], P["cout"], P["activation"]):
+        return None
+    return dlp.DepthwisePointwiseForward.create(st, True, D["activation"], P["cout"], True, P["activation"])
+
+
+def isolated_fused_us(D, P, batch, ring_bytes=768 << 20, seed=7, warm_seconds=0.2):
+    """isolated_layer_us for the fused depthwise + pointwise operator: x of the depthwise layer in, y of the pointwise layer out."""
+    import torch
+
+    op = fused_pair_op(D, P, batch)
+    xshape = (batch, D["cin"], D["hw"], D["hw"])
+    yshape = (batch, P["cout"], P["ohw"], P["ohw"])
+    pair = 4 * (batch * D["cin"] * D["hw"] ** 2 + batch * P["cout"] * P["ohw"] ** 2)
+    ring = max(3, min(48, ring_bytes // pair + 1))
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    xs = [torch.rand(xshape, device="cuda", generator=g) * 2 - 1 for _ in range(ring)]
+    ys = [torch.empty(yshape, device="cuda") for _ in range(ring)]
+    wd = torch.randn((D["cout"], 1, 3, 3), device="cuda", generator=g) * (2.0 / 9) ** 0.5
+    bd = torch.rand(D["cout"], device="cuda", generator=g) * 0.2 - 0.1
+    wp = torch.randn((P["cout"], P["cin"], 1, 1), device="cuda", generator=g) * (2.0 / P["cin"]) ** 0.5
+    bp = torch.rand(P["cout"], device="cuda", generator=g) * 0.2 - 0.1
+    reps = 3 * ring
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < warm_seconds:
+        for j in range(ring):
+            op.enqueue(xs[j], wd, bd, wp, bp, ys[j])
+        torch.cuda.synchronize()
+    for r in range(-ring, reps):
+        if r == 0:
+            e0.record()
+        op.enqueue(xs[r % ring], wd, bd, wp, bp, ys[r % ring])
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def mobilenet_fused_pass_ms(batch, steps, warmup, warm_seconds=0.3, seed=2024):
+    """The mobilenet workload with every pair the library fuses run as one operator (the pointwise layer reads what the
+    depthwise stage left on the chip); the other layers as in run_conv_workload.  Wall clock per pass."""
+    import torch
+
+    layer_list, _ = workload_layers("mobilenet")
+    layers = build_layers(layer_list, batch, seed)
+    fused, skip = {}, set()
+    for (i, j) in mobilenet_pairs(layer_list):
+        op = fused_pair_op(layer_list[i], layer_list[j], batch)
+        if op is not None:
+            fused[i] = (op, j)
+            skip.add(j)
+
+    def step():
+        for i, e in enumerate(layers):
+            if i in fused:
+                op, j = fused[i]
+                op.enqueue(e["x"], e["w"], e["b"], layers[j]["w"], layers[j]["b"], layers[j]["y"])
+            elif i not in skip:
+                e["op"].enqueue(e["x"], e["w"], e["b"], e["y"], e["ws"], 0.0)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < warm_seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3, len(fused)
+
+
 def compact(r, batch, extra=None):
     """One configuration as an entry of the `configs` object of the default line."""
     rf = r["roofline"]
@@ -500,9 +594,29 @@ def other_configs(steps, warmup, peaks):
         rows.append(e)
     dw = [e for e in rows if "frac_of_hbm_peak" in e]
     pw = [e for e in rows if "frac_of_hbm_peak" not in e]
+    # depthwise + pointwise pairs as one launch (the tensor between them never reaches memory): algorithmic bytes are
+    # |x of the depthwise layer| + |y of the pointwise layer| + both filters; scored like the depthwise layers
+    pairs = []
+    LL = r["layer_list"]
+    for (i, j) in mobilenet_pairs(LL):
+        D, P = LL[i], LL[j]
+        e = {"name": "%s+%s" % (D["name"], P["name"]), "separate_us": round(rows[i]["us"] + rows[j]["us"], 2)}
+        if fused_pair_op(D, P, 64) is None:
+            e["fused"] = False  # the library keeps this pair as two operators (faster there)
+        else:
+            us = isolated_fused_us(D, P, 64)
+            xb, yb = 4 * 64 * D["cin"] * D["hw"] ** 2, 4 * 64 * P["cout"] * P["ohw"] ** 2
+            wb = 4 * (D["cout"] * 9 + P["cout"] * P["cin"])
+            gbs, cus = probe.copy_at_size(xb, yb)
+            e.update({"fused": True, "kernel": "conv_dwpw_f32_kernel", "us": round(us, 2), "speedup": round(e["separate_us"] / us, 3), "bound": "hbm",
+                      "gbs": round((xb + yb + wb) / us / 1e3, 1), "frac_of_hbm_peak": round((xb + yb + wb) / us / 1e3 / HBM_PEAK_GBS, 4),
+                      "copy_same_size_us": round(cus, 2), "frac_of_copy_same_size": round(cus / us, 4)})
+        pairs.append(e)
+    fused_ms, nfused = mobilenet_fused_pass_ms(64, max(steps, 100), warmup)
     cfgs["config4_mobilenet_blocks_b64"] = compact(r, 64, {
         "depthwise_min_frac_of_hbm_peak": min(e["frac_of_hbm_peak"] for e in dw), "depthwise_min_frac_of_copy_same_size": min(e["frac_of_copy_same_size"] for e in dw),
-        "pointwise_min_frac_of_roofline": min(e["frac_of_roofline"] for e in pw), "layers": rows})
+        "pointwise_min_frac_of_roofline": min(e["frac_of_roofline"] for e in pw), "layers": rows,
+        "ms_per_step_with_fused_pairs": round(fused_ms, 4), "fused_pairs_in_step": nfused, "fused_pairs": pairs})
     del r
     torch.cuda.empty_cache()
     cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2))

@@ -194,6 +194,45 @@ private:
     dlp_tconv2d_fwd *op_ = nullptr;
 };
 
+// A depthwise 3x3 convolution and the pointwise (1x1) convolution behind it as one operator: the tensor between them never
+// reaches memory.  No counterpart in the reference, which runs two Conv2DForward operators; `config` describes the depthwise
+// layer (groups = channels_in = channels_out, kernel 3, pad 1, stride 1 or 2, shape = shape of x).  supported() tells whether
+// the device code takes the pair (and is faster than the two operators there); the constructor throws NotImplementedError otherwise.
+class DepthwisePointwiseForward {
+public:
+    static bool supported(Conv2DSettings const &config, StandardActivations dw_activation, int channels_out, StandardActivations pw_activation)
+    {
+        dlp_conv2d_settings s = details::to_c(config, config.shape, config.dtype);
+        return dlp_dwpw_fwd_supported(&s, int(dw_activation), channels_out, int(pw_activation)) != 0;
+    }
+    DepthwisePointwiseForward(Context &ctx, Conv2DSettings const &config, bool dw_bias, StandardActivations dw_activation, int channels_out,
+                              bool pw_bias, StandardActivations pw_activation)
+    {
+        if (!ctx.is_hip_context())
+            throw ValidationError("core::DepthwisePointwiseForward needs a device context");
+        ctx.select();
+        dlp_conv2d_settings s = details::to_c(config, config.shape, config.dtype);
+        dlprim::details::check_status(dlp_dwpw_fwd_create(&s, dw_bias ? 1 : 0, int(dw_activation), channels_out, pw_bias ? 1 : 0, int(pw_activation), &op_));
+    }
+    ~DepthwisePointwiseForward() { dlp_dwpw_fwd_destroy(op_); }
+    DepthwisePointwiseForward(DepthwisePointwiseForward const &) = delete;
+    void operator=(DepthwisePointwiseForward const &) = delete;
+    // y = pw_act(conv + pw_bias + factor * y) instead of factor * y + pw_act(conv + pw_bias)
+    void accumulate_before_activation(bool on) { dlprim::details::check_status(dlp_dwpw_fwd_set_accumulate_first(op_, on ? 1 : 0)); }
+    void enqueue(Tensor &x, Tensor &dw_w, Tensor *dw_bias, Tensor &pw_w, Tensor *pw_bias, Tensor &y, float factor, ExecutionContext const &e)
+    {
+        DLPRIM_CHECK(x.shape().size() == 4);
+        int xs[4];
+        for (int i = 0; i < 4; i++)
+            xs[i] = int(x.shape()[i]);
+        dlprim::details::check_status(dlp_dwpw_fwd_enqueue(op_, xs, x.device_ptr(), dw_w.device_ptr(), dw_bias ? dw_bias->device_ptr() : nullptr,
+                                                           pw_w.device_ptr(), pw_bias ? pw_bias->device_ptr() : nullptr, y.device_ptr(), factor, e.stream()));
+    }
+
+private:
+    dlp_dwpw_fwd *op_ = nullptr;
+};
+
 namespace details {
 inline void shape4(Shape const &s, int (&out)[4])
 {

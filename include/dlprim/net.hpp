@@ -17,7 +17,10 @@
 //    (closed form of src/ops/batch_normalization.cpp:210-232);
 //  * an Activation that is the next user of the output of an operator with a fused activation slot
 //    (Convolution2D, InnerProduct, Elementwise, BatchNorm) whose activation is identity moves into that
-//    slot (the reference's ONNX importer does the same merge, src/importers/onnx.cpp:531-580).
+//    slot (the reference's ONNX importer does the same merge, src/importers/onnx.cpp:531-580);
+//  * a residual sum moves into the epilogue of the 1x1 convolution that produces its later branch;
+//  * a depthwise 3x3 convolution and the 1x1 convolution that is its only reader run as one kernel where the library serves
+//    the pair (core::DepthwisePointwiseForward: float tensors, images 20 to 56 wide), so the tensor between them is never written.
 // Training, gradients and the other operator types are not part of this library.
 #pragma once
 #include <algorithm>
@@ -176,6 +179,12 @@ public:
             switch (n.kind) {
             case k_conv: {
                 DLPRIM_CHECK(in.size() == 4 && int(in[1]) == n.conv.channels_in);
+                if (n.dw_node >= 0) { // `in` is the input of the depthwise convolution that this node runs as well
+                    out = core::Conv2DBase::get_output_shape(n.conv, core::Conv2DBase::get_output_shape(nodes_[size_t(n.dw_node)].conv, in));
+                    if (n.dwpw_op && (n.planned_in[2] != in[2] || n.planned_in[3] != in[3]))
+                        create_conv_operator(n, in); // NotImplementedError if the pair is not served at the new size: set up again, or fuse(false)
+                    break;
+                }
                 out = core::Conv2DBase::get_output_shape(n.conv, in);
                 Shape const &old = n.planned_in;
                 if (n.conv_op && (old[2] != in[2] || old[3] != in[3])) {
@@ -411,6 +420,8 @@ private:
         bool is_packed = false, use_w_dev = false;
         std::unique_ptr<core::Conv2DForward> conv_op;
         std::unique_ptr<core::TransposedConv2DForward> tconv_op; // TransposedConvolution2D
+        int dw_node = -1; // a 1x1 convolution that also runs the depthwise convolution in front of it: index of that (skipped) node
+        std::unique_ptr<core::DepthwisePointwiseForward> dwpw_op;
         int output_pad[2] = {0, 0};
         std::unique_ptr<core::IPForward> ip_op;
         Tensor w_dev, b_dev; // what the kernel reads when a BatchNorm is folded in
@@ -744,6 +755,37 @@ private:
         return pi;
     }
 
+    // A depthwise 3x3 convolution into the 1x1 convolution that is its only reader (the pair a MobileNet block ends in), where
+    // the device code runs the pair as one kernel: the 1x1 node then reads the depthwise node's input and runs both.
+    void try_fuse_depthwise_pointwise(size_t i)
+    {
+        Node &d = nodes_[i];
+        if (d.kind != k_conv || d.residual || d.dw_node >= 0 || dtype_ != float_data || keep_intermediate_ || ctx_.is_cpu_context())
+            return;
+        if (d.conv.groups != d.conv.channels_in || d.conv.channels_out != d.conv.channels_in || d.conv.kernel[0] != 3 || d.conv.kernel[1] != 3)
+            return;
+        if (!d.algo.empty() && d.algo != "depthwise_separable")
+            return; // the network file asks for another algorithm
+        std::string const t = d.outputs[0];
+        const int u = next_user(i, t);
+        if (u < 0 || is_net_output(t) || readers_after(i, t) != 1)
+            return;
+        Node &p = nodes_[size_t(u)];
+        if (p.kind != k_conv || p.dw_node >= 0 || p.inputs[0] != t || p.conv.groups != 1 || p.conv.kernel[0] != 1 || p.conv.kernel[1] != 1 ||
+            p.conv.stride[0] != 1 || p.conv.stride[1] != 1 || p.conv.pad[0] != 0 || p.conv.pad[1] != 0 || (!p.algo.empty() && p.algo != "gemm"))
+            return;
+        std::string const &x = d.inputs[0];
+        for (size_t k = i + 1; k <= size_t(u); k++) // the depthwise input must still hold its value when the 1x1 node runs
+            if (!nodes_[k].skipped && std::find(nodes_[k].outputs.begin(), nodes_[k].outputs.end(), x) != nodes_[k].outputs.end())
+                return;
+        core::Conv2DSettings cfg(d.conv, spec(x), dtype_);
+        if (!core::DepthwisePointwiseForward::supported(cfg, d.activation, p.conv.channels_out, p.activation))
+            return;
+        p.dw_node = int(i);
+        p.inputs[0] = x;
+        d.skipped = true;
+    }
+
     void rewrite_graph()
     {
         for (size_t i = 0; i < nodes_.size(); i++) {
@@ -755,10 +797,23 @@ private:
             if (p >= 0)
                 try_merge_activation(size_t(p));
         }
+        for (size_t i = 0; i < nodes_.size(); i++) // after the loop above: both nodes have their final activation and bias
+            if (!nodes_[i].skipped)
+                try_fuse_depthwise_pointwise(i);
     }
 
     void create_conv_operator(Node &n, Shape const &in)
     {
+        if (n.dw_node >= 0) { // in: the input of the depthwise convolution
+            Node &d = nodes_[size_t(n.dw_node)];
+            core::Conv2DSettings dcfg(d.conv, in, dtype_);
+            n.dwpw_op.reset(new core::DepthwisePointwiseForward(ctx_, dcfg, d.bias || d.folded_bn, d.activation, n.conv.channels_out, n.bias || n.folded_bn,
+                                                                n.activation));
+            if (n.residual)
+                n.dwpw_op->accumulate_before_activation(true);
+            n.planned_in = in;
+            return;
+        }
         core::Conv2DSettings cfg(n.conv, in, dtype_);
         n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
         if (n.residual)
@@ -964,6 +1019,8 @@ private:
         }
         if (n.kind == k_conv && prepack_ && n.conv_op)
             pack_conv_weights(n, e);
+        if (n.kind == k_conv && n.dw_node >= 0) // the depthwise convolution that this node runs as well
+            prepare_derived_parameters(nodes_[size_t(n.dw_node)], e);
     }
 
     void run(Node &n, ExecutionContext const &e)
@@ -975,6 +1032,13 @@ private:
             Tensor &w = n.use_w_dev ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
             const float factor = n.residual ? n.residual_factor : 0.0f;
+            if (n.dw_node >= 0) {
+                Node &d = nodes_[size_t(n.dw_node)];
+                Tensor &dw = d.use_w_dev ? d.w_dev : param(d.param_names[0]);
+                Tensor *db = d.folded_bn ? &d.b_dev : d.bias ? &param(d.param_names[1]) : nullptr;
+                n.dwpw_op->enqueue(x, dw, db, w, b, y, factor, e);
+                break;
+            }
             if (n.is_packed)
                 n.conv_op->enqueue_packed(x, w, n.packed, b, y, workspace_, factor, e);
             else

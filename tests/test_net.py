@@ -368,6 +368,33 @@ def test_gpu_net_forward_matches_torch(tmp_path, net, flags):
         np.testing.assert_array_equal(again[k].reshape(-1), params[k].reshape(-1))
 
 
+@pytest.mark.gpu
+def test_gpu_mobilenet_224_fuses_depthwise_pointwise_pairs(tmp_path):
+    """MobileNet-v2 at 224 x 224: the five depthwise -> 1x1 pairs on 56 x 56 and 28 x 28 images run as one kernel each
+    (two at 64 x 64, on the 32 x 32 images).  Same logits as the float64 evaluation of the unfused operator list; the operator
+    count tells that the pairs were taken."""
+    for size, pairs in ((224, 5), (64, 2)):
+        b = netfile.mobilenet_v2(2, size, 10)
+        p = write_net(tmp_path, b)
+        params = b.random_parameters(11)
+        netfile.save_dlpw(tmp_path / "w.dlpw", params)
+        rng = np.random.default_rng(size)
+        x = rng.uniform(-1, 1, b.doc["inputs"][0]["shape"]).astype(np.float32)
+        x.tofile(tmp_path / "in.bin")
+        ops = {}
+        for flags in ((), ("keep",)):
+            r = tool("run", p, tmp_path / "w.dlpw", tmp_path / "in.bin", tmp_path / "out.bin", "repeat=2", *flags)
+            assert "ok" in r.stdout
+            ops[flags] = int(r.stdout.split("operators")[1].split()[0])
+            want = torch_forward(b.doc, params, {"data": x})[0]
+            got = np.fromfile(tmp_path / "out.bin", dtype=np.float32).reshape(want.shape)
+            err = np.abs(got - want).max() / np.abs(want).max()
+            print("mobilenet", size, flags, "operators", ops[flags], "max err / max |y| = %.3g" % err)
+            assert err < 1e-4
+        # "keep" gives every tensor memory of its own: no residual sum in an epilogue (10 of them), no fused pair
+        assert ops[("keep",)] - ops[()] == 10 + pairs
+
+
 def random_net(seed):
     """A random graph over one spatial size: convolutions (1x1 / 3x3, with and without bias / activation), BatchNorm,
     activations in place and not, element-wise operations between any two tensors made so far, now and then a
