@@ -11,6 +11,7 @@ uniform[-1,1], weights Kaiming-normal, bias uniform[-0.1,0.1], fixed seed.
 Other workloads (same JSON contract, for the remaining configurations):
   --workload single         one 3x3 64->64 convolution at 56x56 (configuration 1 with --batch 16)
   --workload mobilenet      depthwise 3x3 stride 1/2 (HBM bound) + 1x1 pointwise, ReLU6
+  --workload mobilenet-fused  the same layers with the depthwise -> pointwise pairs the library fuses run as one launch each
   --workload winograd       the two Winograd shapes, algo winograd
   --workload winograd-gemm  the same two shapes through the implicit GEMM
   --workload resnet18-full / resnet50-full   whole network forward incl. pooling, adds, GAP, IP
@@ -629,8 +630,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "winograd", "winograd-gemm", "single", "resnet18-full",
-                                                                 "resnet50-full", "resnet18-backward"])
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "resnet50", "mobilenet", "mobilenet-fused", "winograd", "winograd-gemm", "single",
+                                                                 "resnet18-full", "resnet50-full", "resnet18-backward"])
     ap.add_argument("--algo", default="gemm", help="conv algorithm of the -full workloads ('' = auto)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="storage type of the tensors (accumulation and epilogue are fp32 either way)")
     ap.add_argument("--cpu-images", type=int, default=8, help="images of the CPU baseline sample (0 = skip)")
@@ -660,6 +661,14 @@ def main():
         return
     if args.workload == "resnet18-backward":
         run_backward_workload(args)
+        return
+    if args.workload == "mobilenet-fused":
+        # the mobilenet workload with the depthwise -> pointwise pairs that the library fuses run as one launch each
+        ms, nfused = mobilenet_fused_pass_ms(args.batch, args.steps, args.warmup)
+        print(json.dumps({"metric": BASELINE_METRIC, "value": round(args.batch / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+                          "data": "synthetic", "config": {"workload": "MobileNet-v2 style blocks, batch %d, %d depthwise + pointwise pairs as one launch each" %
+                                                          (args.batch, nfused), "batch": args.batch}}))
         return
     bf16 = args.dtype == "bf16"
     r = run_conv_workload(args.workload, args.batch, bf16, args.steps, args.warmup, args.prepacked, args.only)

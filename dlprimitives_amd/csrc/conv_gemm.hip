@@ -1386,7 +1386,7 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     auto my_tile = [&](int kt) { return LW == 4 || (kt & (4 / LW - 1)) == my_turn; };
     auto load_b = [&](auto set, int kt) {
         constexpr int S = (decltype(set)::value * LW / 4) % NSETB;
-        const uint32_t soff = (uint32_t)(min(kt, a.nkt - 1) * BK2) * a.hw4;
+        const uint32_t soff = (uint32_t)(kt * BK2) * a.hw4;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             if constexpr (DW == 4) {
@@ -1430,8 +1430,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
     auto load_half = [&](auto set, int kt, auto half_c) {
         constexpr int S = decltype(set)::value;
         constexpr int Q = decltype(half_c)::value;
+        // tiles past the end of this workgroup's K range are never multiplied: no loads for them (with two or four K tiles in
+        // all, as in the 1x1 layers of 64 or 128 channels, they would be more than half of all loads); a uniform branch
+        if (kt >= kt_end)
+            return;
         if (Q == 0) {
-            const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
+            const uint32_t a_soff = a_row_base + (uint32_t)kt * a_tile_bytes;
 #pragma unroll
             for (int j = 0; j < A_LD; j++)
                 ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, a_voff[j], a_soff, 0));
@@ -1478,6 +1482,8 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
         constexpr int S = decltype(set)::value;
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int Q = decltype(half_c)::value;
+        if (kt >= kt_end) // nothing was loaded for it (load_half)
+            return;
         if (Q == 0) {
 #pragma unroll
             for (int j = 0; j < A_LD; j++) {
