@@ -169,10 +169,10 @@ def cpu_baseline(layer_list, images, seed, threads=1):
 
 
 def run_graph_workload(args):
-    return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup)
+    return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup, args.fuse_residual)
 
 
-def graph_workload(net, batch, algo, bf16, steps, warmup):
+def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False):
     """Whole-network forward (convolutions + pooling + residual adds + global pooling + inner
     product) through the C-ABI operators; same JSON contract, no per-kernel roofline split."""
     import torch
@@ -183,7 +183,7 @@ def graph_workload(net, batch, algo, bf16, steps, warmup):
     ops = getattr(graphs, net)()
     params = graphs.random_parameters(ops, 2024)
     shape = (batch, 3, 224, 224)
-    runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32")
+    runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32", fuse_residual=fuse_residual)
     x = torch.rand(shape, device="cuda:0") * 2 - 1
     runner.t["data"].copy_(x)  # converts to the storage type
     for _ in range(warmup):
@@ -213,8 +213,9 @@ def graph_workload(net, batch, algo, bf16, steps, warmup):
         "metric": BASELINE_METRIC, "value": round(batch / (ms_per_step * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
         "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32", "data": "synthetic",
-        "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds, global avg pool, inner product), "
-                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, "bf16 storage" if bf16 else "fp32", batch, algo or "auto"),
+        "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds%s, global avg pool, inner product), "
+                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, " in the epilogue of the 1x1 convolution in front of them" if fuse_residual else "",
+                                                                             "bf16 storage" if bf16 else "fp32", batch, algo or "auto"),
                    "batch": batch, "gflop_per_step": round(flops / 1e9, 1)},
         "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_matrix_peak_whole_pass": round(flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
@@ -620,7 +621,9 @@ def other_configs(steps, warmup, peaks):
         "ms_per_step_with_fused_pairs": round(fused_ms, 4), "fused_pairs_in_step": nfused, "fused_pairs": pairs})
     del r
     torch.cuda.empty_cache()
-    cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2))
+    # the residual sums run in the epilogue of the 1x1 convolution that produces their later branch, as dlprim::Net does
+    # with the same network (--workload resnet50-full --fuse-residual; without the flag the sums are operators of their own)
+    cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True)
     return cfgs
 
 
@@ -639,6 +642,8 @@ def main():
     ap.add_argument("--prepacked", action="store_true",
                     help="weights transformed once before the timed region (dlp_conv2d_fwd_pack / _enqueue_packed), as an inference "
                          "deployment does; the default transforms them in every step, as the reference's enqueue contract implies")
+    ap.add_argument("--fuse-residual", action="store_true",
+                    help="-full workloads: residual sums behind a 1x1 convolution run in that convolution's epilogue (dlp_conv2d_fwd_set_accumulate_first)")
     ap.add_argument("--only", default="", help="profiling aid: keep only layers whose name contains this text")
     ap.add_argument("--no-configs", action="store_true", help="default workload only: leave out the `configs` object (the other four configurations)")
     args = ap.parse_args()

@@ -114,18 +114,31 @@ def infer_shapes(ops, in_shape):
 class GraphRunner:
     """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
 
-    def __init__(self, ops, params, in_shape, algo="", dtype="float32"):
-        """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32)."""
+    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False):
+        """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32).
+        fuse_residual: a residual sum whose later branch is a 1x1 convolution runs in that convolution's epilogue
+        (dlp_conv2d_fwd_set_accumulate_first: y = act(conv + bias + y) written over the other branch), which is what
+        dlprim::Net does with the same graphs; 3x3 convolutions keep their sum as an operator."""
         import torch
 
         import dlprimitives_amd as dlp
         from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA
 
+        ops = [dict(o) for o in ops]
+        alias = {}
+        if fuse_residual:
+            ops = self._fuse_residual_sums(ops, alias)
         self.ops = ops
         self.shapes = infer_shapes(ops, in_shape)
         tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
         code = BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA
-        self.t = {n: torch.empty(s, dtype=tdt, device="cuda:0") for n, s in self.shapes.items()}
+        self.t = {n: torch.empty(s, dtype=tdt, device="cuda:0") for n, s in self.shapes.items() if n not in alias}
+        for n in self.shapes:  # the output of a fused sum lies over the branch it was added to (chains of blocks: follow the aliases)
+            if n in alias:
+                m = alias[n]
+                while m in alias:
+                    m = alias[m]
+                self.t[n] = self.t[m]
         self.p = {n: (torch.from_numpy(w).cuda().to(tdt), torch.from_numpy(b).cuda()) for n, (w, b) in params.items()}
         self.k = []
         ws_bytes = 1
@@ -133,6 +146,8 @@ class GraphRunner:
             if o["op"] == "conv":
                 st = dlp.Conv2DSettings(o["cin"], o["cout"], o["k"], o["s"], 1, o["p"], 1, self.shapes[o["src"]], dtype=code)
                 op = dlp.Conv2DForward.create(st, True, o["act"], algo)
+                if o.get("residual"):
+                    op.accumulate_before_activation(True)
                 ws_bytes = max(ws_bytes, op.workspace())
             elif o["op"] == "maxpool":
                 op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"], dtype=code)
@@ -146,6 +161,29 @@ class GraphRunner:
         # one workspace shared by all operators, as the reference's Net does
         self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda:0")
 
+    @staticmethod
+    def _fuse_residual_sums(ops, alias):
+        """add(c, skip) with c = a 1x1 convolution without activation that only the sum reads: the convolution takes the
+        sum's activation, reads skip as its old output and writes the sum's tensor, which shares skip's memory; the
+        convolution that makes skip (the downsample) moves in front of it.  skip must not be read after the sum."""
+        out = []
+        for i, o in enumerate(ops):
+            if o["op"] != "add":
+                out.append(o)
+                continue
+            c, skip = o["src"]
+            ci = next((k for k, q in enumerate(out) if q["dst"] == c), None)
+            later = any((skip == q["src"] or (isinstance(q["src"], list) and skip in q["src"])) for q in ops[i + 1:])
+            readers_c = sum(1 for q in ops if c == q["src"] or (isinstance(q["src"], list) and c in q["src"]))
+            if ci is None or out[ci]["op"] != "conv" or out[ci]["k"] != 1 or out[ci]["act"] != "identity" or later or readers_c != 1 or skip == "data":
+                out.append(o)
+                continue
+            conv = out.pop(ci)  # appended again below: behind everything made so far, the other branch included
+            conv.update(act=o["act"], residual=True, pname=conv["dst"], dst=o["dst"])
+            alias[o["dst"]] = skip
+            out.append(conv)
+        return out
+
     def forward(self, x=None):
         import dlprimitives_amd as dlp
 
@@ -153,8 +191,8 @@ class GraphRunner:
             self.t["data"].copy_(x)
         for o, op in zip(self.ops, self.k):
             if o["op"] == "conv":
-                w, b = self.p[o["dst"]]
-                op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]], self.ws, 0.0)
+                w, b = self.p[o.get("pname", o["dst"])]
+                op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]], self.ws, 1.0 if o.get("residual") else 0.0)
             elif o["op"] in ("maxpool", "gap"):
                 op.enqueue(self.t[o["src"]], self.t[o["dst"]])
             elif o["op"] == "add":

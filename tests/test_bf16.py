@@ -203,10 +203,11 @@ def test_resnet50_bf16_logits_vs_fp32_reference(oracle_mod):
     ops = graphs.resnet50()
     params = graphs.random_parameters(ops, seed=11)
     x = np.random.default_rng(3).standard_normal((4, 3, 224, 224)).astype(np.float32)
-    runner = graphs.GraphRunner(ops, params, x.shape, algo="", dtype="bfloat16")
-    got = runner.forward(torch.from_numpy(x).cuda().to(torch.bfloat16)).float().cpu().numpy()
     want = run_graph_on_oracle(oracle_mod, ops, params, x)
-    rel = np.abs(got - want).max() / np.abs(want).max()
-    print("resnet50 bf16 vs fp32 reference: max relative error of the logits %.4f" % rel)
-    assert rel <= 1e-2
-    assert (got.argmax(1) == want.argmax(1)).all()
+    for fuse_residual in (False, True):  # residual sums as operators of their own, and in the epilogues of the 1x1 convolutions
+        runner = graphs.GraphRunner(ops, params, x.shape, algo="", dtype="bfloat16", fuse_residual=fuse_residual)
+        got = runner.forward(torch.from_numpy(x).cuda().to(torch.bfloat16)).float().cpu().numpy()
+        rel = np.abs(got - want).max() / np.abs(want).max()
+        print("resnet50 bf16 vs fp32 reference (sums fused: %s): max relative error of the logits %.4f" % (fuse_residual, rel))
+        assert rel <= 1e-2
+        assert (got.argmax(1) == want.argmax(1)).all()
