@@ -1207,7 +1207,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
 // a.sh, a.sw describe that copy): a pixel's 32 channels of a K tile are 64 consecutive bytes, four 16-byte pieces that go to
 // LDS as they come, exactly like the weight tile.  Any kernel extent, stride, padding and image size.
 template <int BM, int BN, int WM, int WN, int ORDER, int ACT, int NSET, int PXL, int SX = 1, int XT = 0>
-__global__ __launch_bounds__(kThreads) void conv_gemm_bf16_kernel(GemmArgs a)
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM == 128 || PXL == 8 || (PXL == 4 && SX == 1) || XT == 1) ? 3 : 2))) void conv_gemm_bf16_kernel(GemmArgs a)
 {
     static_assert(PXL == 0 || ((PXL == 2 || PXL == 4 || PXL == 8) && PXL * SX >= 4 && PXL * SX <= 8 && ORDER == GEMM_ORDER_TAP_BF16),
                   "dense loader variants: loads of 8 or 16 bytes");
