@@ -169,10 +169,10 @@ def cpu_baseline(layer_list, images, seed, threads=1):
 
 
 def run_graph_workload(args):
-    return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup, args.fuse_residual)
+    return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup, args.fuse_residual, args.prepacked)
 
 
-def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False):
+def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, prepack=False):
     """Whole-network forward (convolutions + pooling + residual adds + global pooling + inner
     product) through the C-ABI operators; same JSON contract, no per-kernel roofline split."""
     import torch
@@ -183,7 +183,7 @@ def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False):
     ops = getattr(graphs, net)()
     params = graphs.random_parameters(ops, 2024)
     shape = (batch, 3, 224, 224)
-    runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32", fuse_residual=fuse_residual)
+    runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32", fuse_residual=fuse_residual, prepack=prepack)
     x = torch.rand(shape, device="cuda:0") * 2 - 1
     runner.t["data"].copy_(x)  # converts to the storage type
     for _ in range(warmup):
@@ -214,8 +214,9 @@ def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False):
         "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 storage, fp32 accumulate" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": "%s full forward (conv + BN folded + ReLU, max pool, residual adds%s, global avg pool, inner product), "
-                               "%s NCHW, batch %d, 224x224, conv algo '%s'" % (net, " in the epilogue of the 1x1 convolution in front of them" if fuse_residual else "",
-                                                                             "bf16 storage" if bf16 else "fp32", batch, algo or "auto"),
+                               "%s NCHW, batch %d, 224x224, conv algo '%s'%s" % (net, " in the epilogue of the 1x1 convolution in front of them" if fuse_residual else "",
+                                                                               "bf16 storage" if bf16 else "fp32", batch, algo or "auto",
+                                                                               ", filters transformed once before the timed region" if prepack else ""),
                    "batch": batch, "gflop_per_step": round(flops / 1e9, 1)},
         "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_matrix_peak_whole_pass": round(flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
@@ -593,6 +594,10 @@ def other_configs(steps, warmup, peaks):
             roof = min(FP32_MATRIX_PEAK_TFLOPS * 1e12, ai * HBM_PEAK_GBS * 1e9)
             e["bound"] = "mfma" if ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12 else "hbm"
             e["frac_of_roofline"] = round(flops / (us * 1e-6) / roof, 4)
+            # what a launch of this size costs at the least on this chip: a plain streaming kernel over the same |X| and |Y|
+            gbs, cus = probe.copy_at_size(xb, yb)
+            e["roofline_us"] = round(flops / roof * 1e6, 2)
+            e["copy_same_size_us"] = round(cus, 2)
         rows.append(e)
     dw = [e for e in rows if "frac_of_hbm_peak" in e]
     pw = [e for e in rows if "frac_of_hbm_peak" not in e]
@@ -621,9 +626,10 @@ def other_configs(steps, warmup, peaks):
         "ms_per_step_with_fused_pairs": round(fused_ms, 4), "fused_pairs_in_step": nfused, "fused_pairs": pairs})
     del r
     torch.cuda.empty_cache()
-    # the residual sums run in the epilogue of the 1x1 convolution that produces their later branch, as dlprim::Net does
-    # with the same network (--workload resnet50-full --fuse-residual; without the flag the sums are operators of their own)
-    cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True)
+    # an inference deployment, as dlprim::Net runs the same network: the residual sums run in the epilogue of the 1x1 convolution
+    # that produces their later branch and the filters are transformed once (--workload resnet50-full --fuse-residual
+    # --prepacked; without the flags the sums are operators of their own and every enqueue transforms its filter)
+    cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True, prepack=True)
     return cfgs
 
 

@@ -114,11 +114,14 @@ def infer_shapes(ops, in_shape):
 class GraphRunner:
     """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
 
-    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False):
+    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False, prepack=False):
         """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32).
         fuse_residual: a residual sum whose later branch is a 1x1 convolution runs in that convolution's epilogue
         (dlp_conv2d_fwd_set_accumulate_first: y = act(conv + bias + y) written over the other branch), which is what
-        dlprim::Net does with the same graphs; 3x3 convolutions keep their sum as an operator."""
+        dlprim::Net does with the same graphs; 3x3 convolutions keep their sum as an operator.
+        prepack: the filters are transformed once here (dlp_conv2d_fwd_pack) and forward() calls enqueue_packed, as a
+        network with constant weights does (dlprim::Net::copy_parameters_to_device); otherwise every enqueue transforms
+        its filter again, which is the contract of the reference's enqueue."""
         import torch
 
         import dlprimitives_amd as dlp
@@ -141,6 +144,7 @@ class GraphRunner:
                 self.t[n] = self.t[m]
         self.p = {n: (torch.from_numpy(w).cuda().to(tdt), torch.from_numpy(b).cuda()) for n, (w, b) in params.items()}
         self.k = []
+        self.packed = {}
         ws_bytes = 1
         for o in ops:
             if o["op"] == "conv":
@@ -149,6 +153,10 @@ class GraphRunner:
                 if o.get("residual"):
                     op.accumulate_before_activation(True)
                 ws_bytes = max(ws_bytes, op.workspace())
+                if prepack:
+                    buf = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+                    op.pack(self.p[o.get("pname", o["dst"])][0], buf)
+                    self.packed[len(self.k)] = buf
             elif o["op"] == "maxpool":
                 op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"], dtype=code)
             elif o["op"] == "gap":
@@ -189,10 +197,14 @@ class GraphRunner:
 
         if x is not None:
             self.t["data"].copy_(x)
-        for o, op in zip(self.ops, self.k):
+        for i, (o, op) in enumerate(zip(self.ops, self.k)):
             if o["op"] == "conv":
                 w, b = self.p[o.get("pname", o["dst"])]
-                op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]], self.ws, 1.0 if o.get("residual") else 0.0)
+                factor = 1.0 if o.get("residual") else 0.0
+                if i in self.packed:
+                    op.enqueue_packed(self.t[o["src"]], w, self.packed[i], b, self.t[o["dst"]], self.ws, factor)
+                else:
+                    op.enqueue(self.t[o["src"]], w, b, self.t[o["dst"]], self.ws, factor)
             elif o["op"] in ("maxpool", "gap"):
                 op.enqueue(self.t[o["src"]], self.t[o["dst"]])
             elif o["op"] == "add":

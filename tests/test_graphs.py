@@ -43,7 +43,7 @@ def test_full_forward_matches_oracle(oracle_mod, net, fuse_residual):
     ops = getattr(graphs, net)()
     params = graphs.random_parameters(ops, seed=7)
     x = np.random.default_rng(1).uniform(-1, 1, (2, 3, 224, 224)).astype(np.float32)
-    runner = graphs.GraphRunner(ops, params, x.shape, fuse_residual=fuse_residual)
+    runner = graphs.GraphRunner(ops, params, x.shape, fuse_residual=fuse_residual, prepack=fuse_residual)  # (filters transformed once, or in every call)
     # ResNet-50's 16 sums all follow a 1x1 convolution; ResNet-18's follow 3x3 convolutions and stay operators
     assert len(runner.ops) == len(ops) - (16 if fuse_residual and net == "resnet50" else 0)
     got = runner.forward(torch.from_numpy(x).cuda())
