@@ -1060,54 +1060,70 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
         auto store_runs = [&](auto pxv_c) {
             constexpr int PXV = decltype(pxv_c)::value;
             constexpr int RUNS = BN / PXV; // per row
-#pragma unroll 4
-            for (int q = tid; q < BM * RUNS; q += kThreads) {
+            static_assert((BM * RUNS) % (4 * kThreads) == 0, "runs are dealt to the threads in batches of four");
+            auto run_offset = [&](int q) { // byte offset in y of run q of the staged tile (out of range: nothing is stored)
                 const int row = q / RUNS, cp = q % RUNS;
                 const int n = n0 + cp * PXV, m = m0 + row;
                 const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
                 const int pix = n - b * a.OHW;
-                const uint32_t voff = (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
-                const unsigned char *src = smem + row * PITCH + cp * (PXV * 2);
-                if (pre) { // y = act(staged value + factor * old y), the run read with one load of the store's width
-                    uint32_t mine[PXV / 2], old[PXV / 2];
+                return (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
+            };
+            if (pre) {
+                // y = act(staged value + factor * old y): the old runs of four runs are requested together (loads of the stores'
+                // width), so that a thread waits for memory twice per tile and not eight times
+                for (int q0 = tid; q0 < BM * RUNS; q0 += 4 * kThreads) {
+                    uint32_t voff[4], old[4][PXV / 2];
 #pragma unroll
-                    for (int d = 0; d < PXV / 2; d++)
-                        mine[d] = ((const uint32_t *)src)[d];
-                    if constexpr (PXV == 8) {
-                        const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(yr, voff, 0, 0);
-                        old[0] = o[0], old[1] = o[1], old[2] = o[2], old[3] = o[3];
-                    } else if constexpr (PXV == 4) {
-                        const u32x2 o = __builtin_amdgcn_raw_buffer_load_b64(yr, voff, 0, 0);
-                        old[0] = o[0], old[1] = o[1];
-                    } else
-                        old[0] = __builtin_amdgcn_raw_buffer_load_b32(yr, voff, 0, 0);
-#pragma unroll
-                    for (int d = 0; d < PXV / 2; d++) {
-                        float lo = fmaf(__builtin_bit_cast(float, old[d] << 16), a.factor, __builtin_bit_cast(float, mine[d] << 16));
-                        float hi = fmaf(__builtin_bit_cast(float, old[d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[d] & 0xFFFF0000u));
-                        if (ACT == ACT_CLAMP) {
-                            if (a.act != DLP_ACT_IDENTITY) {
-                                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
-                                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
-                            }
-                        } else {
-                            lo = apply_act(lo, a.act);
-                            hi = apply_act(hi, a.act);
-                        }
-                        mine[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                    for (int u = 0; u < 4; u++) {
+                        voff[u] = run_offset(q0 + u * kThreads);
+                        if constexpr (PXV == 8) {
+                            const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(yr, voff[u], 0, 0);
+                            old[u][0] = o[0], old[u][1] = o[1], old[u][2] = o[2], old[u][3] = o[3];
+                        } else if constexpr (PXV == 4) {
+                            const u32x2 o = __builtin_amdgcn_raw_buffer_load_b64(yr, voff[u], 0, 0);
+                            old[u][0] = o[0], old[u][1] = o[1];
+                        } else
+                            old[u][0] = __builtin_amdgcn_raw_buffer_load_b32(yr, voff[u], 0, 0);
                     }
-                    if constexpr (PXV == 8) {
-                        u32x4 o;
-                        o[0] = mine[0], o[1] = mine[1], o[2] = mine[2], o[3] = mine[3];
-                        __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff, 0, 0);
-                    } else if constexpr (PXV == 4) {
-                        u32x2 o;
-                        o[0] = mine[0], o[1] = mine[1];
-                        __builtin_amdgcn_raw_buffer_store_b64(o, yr, voff, 0, 0);
-                    } else
-                        __builtin_amdgcn_raw_buffer_store_b32(mine[0], yr, voff, 0, 0);
-                    continue;
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const int q = q0 + u * kThreads;
+                        const unsigned char *src = smem + (q / RUNS) * PITCH + (q % RUNS) * (PXV * 2);
+                        uint32_t mine[PXV / 2];
+#pragma unroll
+                        for (int d = 0; d < PXV / 2; d++) {
+                            mine[d] = ((const uint32_t *)src)[d];
+                            float lo = fmaf(__builtin_bit_cast(float, old[u][d] << 16), a.factor, __builtin_bit_cast(float, mine[d] << 16));
+                            float hi = fmaf(__builtin_bit_cast(float, old[u][d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[d] & 0xFFFF0000u));
+                            if (ACT == ACT_CLAMP) {
+                                if (a.act != DLP_ACT_IDENTITY) {
+                                    lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                                    hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
+                                }
+                            } else {
+                                lo = apply_act(lo, a.act);
+                                hi = apply_act(hi, a.act);
+                            }
+                            mine[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                        }
+                        if constexpr (PXV == 8) {
+                            u32x4 o;
+                            o[0] = mine[0], o[1] = mine[1], o[2] = mine[2], o[3] = mine[3];
+                            __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff[u], 0, 0);
+                        } else if constexpr (PXV == 4) {
+                            u32x2 o;
+                            o[0] = mine[0], o[1] = mine[1];
+                            __builtin_amdgcn_raw_buffer_store_b64(o, yr, voff[u], 0, 0);
+                        } else
+                            __builtin_amdgcn_raw_buffer_store_b32(mine[0], yr, voff[u], 0, 0);
+                    }
                 }
+                return;
+            }
+#pragma unroll 4
+            for (int q = tid; q < BM * RUNS; q += kThreads) {
+                const uint32_t voff = run_offset(q);
+                const unsigned char *src = smem + (q / RUNS) * PITCH + (q % RUNS) * (PXV * 2);
                 if constexpr (PXV == 8)
                     __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
                 else if constexpr (PXV == 4)
