@@ -91,6 +91,9 @@ struct GemmArgs {
     uint32_t x_shift; // bytes by which the X resource base is moved back (padding offset)
     uint32_t hw4;     // H*W*sizeof(T): byte stride between input channels
     uint32_t ohw_magic, ohw_shift, ow_magic, ow_shift;
+    // divisions of the tile decode: by mtiles, ntiles, groups, by the tiles of the main part and of the tail of a split launch
+    // (an integer division by a run-time value costs some forty vector instructions, per wavefront, before the first load)
+    uint32_t mt_magic, mt_shift, ntl_magic, ntl_shift, gr_magic, gr_shift, tm_magic, tm_shift, tt_magic, tt_shift;
     float factor;
     int pre; // the old value of y is added before the activation (Epilogue::accumulate_first)
     int act;
@@ -205,12 +208,12 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             const int q = nb >> 3, r = nb & 7;
             const int xcd = bid & 7, slot = bid >> 3;
             t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
-            slice = t / tiles_main;
+            slice = (int)fast_div((uint32_t)t, a.tm_magic, a.tm_shift); // t / tiles_main
             t -= slice * tiles_main;
             image0 = (uint32_t)(t * splitk);
         } else { // finer slices of the last tiles
             t = bid - a.main_wgs;
-            slice = t / a.tail_tiles;
+            slice = (int)fast_div((uint32_t)t, a.tt_magic, a.tt_shift); // t / tail_tiles
             t -= slice * a.tail_tiles;
             image0 = (uint32_t)((splitk > 1 ? tiles_main * splitk : 0) + t * a.tail_splitk);
             t += tiles_main;
@@ -219,10 +222,10 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
         }
     }
     // tile decode: m tile fastest, then n tile, then group
-    const int mt = t % a.mtiles;
-    t /= a.mtiles;
-    const int nt = t % a.ntiles;
-    const int g = t / a.ntiles;
+    const int tm = (int)fast_div((uint32_t)t, a.mt_magic, a.mt_shift);
+    const int mt = t - tm * a.mtiles;
+    const int g = (int)fast_div((uint32_t)tm, a.ntl_magic, a.ntl_shift);
+    const int nt = tm - g * a.ntiles;
     const int m0 = mt * BM, n0 = nt * BN;
     const int kt_begin = slice * kt_per_slice;
     const int kt_end = min(kt_begin + kt_per_slice, a.nkt);
@@ -1061,13 +1064,20 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
             constexpr int PXV = decltype(pxv_c)::value;
             constexpr int RUNS = BN / PXV; // per row
             static_assert((BM * RUNS) % (4 * kThreads) == 0, "runs are dealt to the threads in batches of four");
-            auto run_offset = [&](int q) { // byte offset in y of run q of the staged tile (out of range: nothing is stored)
-                const int row = q / RUNS, cp = q % RUNS;
-                const int n = n0 + cp * PXV, m = m0 + row;
-                const int b = (int)fast_div((uint32_t)n, a.ohw_magic, a.ohw_shift);
-                const int pix = n - b * a.OHW;
-                return (n < a.N && m < a.M) ? (uint32_t)(((b * a.Cout + g * a.M + m) * a.OHW + pix) * 2) : kOutOfRange;
+            static_assert(kThreads % RUNS == 0, "a thread keeps its column of runs: q += kThreads only moves the row");
+            // run q = row * RUNS + cp of the staged tile; the image and pixel of a thread's runs are found once
+            const int cp = tid % RUNS, row_t = tid / RUNS;
+            const int n_run = n0 + cp * PXV;
+            const int b_run = (int)fast_div((uint32_t)n_run, a.ohw_magic, a.ohw_shift);
+            const uint32_t col_off = (uint32_t)(((b_run * a.Cout + g * a.M + m0) * a.OHW + (n_run - b_run * a.OHW)) * 2);
+            const uint32_t row_pitch = (uint32_t)a.OHW * 2u;
+            const int rows_ok = n_run < a.N ? a.M - m0 : 0;
+            const unsigned char *src_t = smem + row_t * PITCH + cp * (PXV * 2);
+            auto run_offset = [&](int q) { // byte offset in y of run q (q = tid + a multiple of kThreads; out of range: nothing is stored)
+                const int row = row_t + (q - tid) / RUNS;
+                return row < rows_ok ? col_off + (uint32_t)row * row_pitch : kOutOfRange;
             };
+            auto run_source = [&](int q) { return src_t + ((q - tid) / RUNS) * PITCH; };
             if (pre) {
                 // y = act(staged value + factor * old y): the old runs of four runs are requested together (loads of the stores'
                 // width), so that a thread waits for memory twice per tile and not eight times
@@ -1088,7 +1098,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
                         const int q = q0 + u * kThreads;
-                        const unsigned char *src = smem + (q / RUNS) * PITCH + (q % RUNS) * (PXV * 2);
+                        const unsigned char *src = run_source(q);
                         uint32_t mine[PXV / 2];
 #pragma unroll
                         for (int d = 0; d < PXV / 2; d++) {
@@ -1123,7 +1133,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
 #pragma unroll 4
             for (int q = tid; q < BM * RUNS; q += kThreads) {
                 const uint32_t voff = run_offset(q);
-                const unsigned char *src = smem + (q / RUNS) * PITCH + (q % RUNS) * (PXV * 2);
+                const unsigned char *src = run_source(q);
                 if constexpr (PXV == 8)
                     __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
                 else if constexpr (PXV == 4)
@@ -1260,12 +1270,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM ==
         const int xcd = bid & 7, slot = bid >> 3;
         t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
     }
-    const int mt = t % a.mtiles;
-    t /= a.mtiles;
-    const int nt = t % a.ntiles;
-    t /= a.ntiles;
-    const int g = t % a.groups;
-    const int slice = t / a.groups;
+    const int tm = (int)fast_div((uint32_t)t, a.mt_magic, a.mt_shift);
+    const int mt = t - tm * a.mtiles;
+    const int tn = (int)fast_div((uint32_t)tm, a.ntl_magic, a.ntl_shift);
+    const int nt = tm - tn * a.ntiles;
+    const int slice = (int)fast_div((uint32_t)tn, a.gr_magic, a.gr_shift);
+    const int g = tn - slice * a.groups;
     const int m0 = mt * BM, n0 = nt * BN;
     const int kt_begin = slice * a.kt_per_slice;
     const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
@@ -1669,10 +1679,10 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         const int xcd = bid & 7, slot = bid >> 3;
         t = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
     }
-    const int mt = t % a.mtiles;
-    t /= a.mtiles;
-    const int nt = t % a.ntiles;
-    const int g = t / a.ntiles;
+    const int tm = (int)fast_div((uint32_t)t, a.mt_magic, a.mt_shift);
+    const int mt = t - tm * a.mtiles;
+    const int g = (int)fast_div((uint32_t)tm, a.ntl_magic, a.ntl_shift);
+    const int nt = tm - g * a.ntiles;
     const int m0 = mt * BM, n0 = nt * BN;
     const int ncb = a.nkt / KHW; // stages
 
@@ -2207,6 +2217,17 @@ size_t split_total_bytes(const GemmPlan &p, const GemmArgs &a, int groups)
     return split_counter_bytes(tiles) + (size_t)images * p.BM * p.BN * sizeof(float);
 }
 
+// Multipliers for the kernels' decode of a workgroup number into (row tile, pixel tile, group, K slice).
+void set_tile_magics(GemmArgs &a, int groups)
+{
+    const long long tiles_main = (long long)a.mtiles * a.ntiles * groups - a.tail_tiles;
+    make_magic((uint32_t)std::max(a.mtiles, 1), a.mt_magic, a.mt_shift);
+    make_magic((uint32_t)std::max(a.ntiles, 1), a.ntl_magic, a.ntl_shift);
+    make_magic((uint32_t)std::max(groups, 1), a.gr_magic, a.gr_shift);
+    make_magic((uint32_t)std::max<long long>(tiles_main, 1), a.tm_magic, a.tm_shift);
+    make_magic((uint32_t)std::max(a.tail_tiles, 1), a.tt_magic, a.tt_shift);
+}
+
 void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t ws_bytes)
 {
     a.mtiles = p.mtiles;
@@ -2246,6 +2267,7 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
         }
     }
     a.main_wgs = (int)((tiles - a.tail_tiles) * a.splitk);
+    set_tile_magics(a, groups);
 }
 
 template <class T, int BM, int BN, int WM, int WN, int ORDER, int MASK, int ACT>
@@ -2338,6 +2360,8 @@ int launch_patch_bf16(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStre
     a.part = nullptr;
     a.part_bytes = 0;
     a.pp_nbr = p.pp_nbr;
+    a.tail_tiles = 0;
+    set_tile_magics(a, g.groups);
     const long long blocks = (long long)a.mtiles * a.ntiles * g.groups;
     if (blocks > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");

@@ -757,8 +757,9 @@ int dlp_dwpw_fwd_create(const dlp_conv2d_settings *dw_cfg, int dw_bias, int dw_a
         return rc;
     if (!conv_dwpw_supported(g, channels_out, dw_activation, pw_activation))
         return fail(DLP_ERR_NOT_IMPLEMENTED,
-                    "fused depthwise + pointwise: float_data, depthwise 3x3 with padding 1 and stride 1 or 2 on images up to 56 wide (width a multiple of 4, "
-                    "or of 2 up to 16), channels a multiple of 8, at most 128 filters, identity / relu / relu6; run the two operators separately otherwise");
+                    "fused depthwise + pointwise: float_data, depthwise 3x3 with padding 1 and stride 1 or 2 on images of at least 512 pixels and at most "
+                    "56 wide (output width a multiple of 4, or of 2 at stride 2 up to 28 wide), channels a multiple of 8, at most 128 filters, "
+                    "identity / relu / relu6; run the two operators separately otherwise");
     dlp_dwpw_fwd *op = new (std::nothrow) dlp_dwpw_fwd();
     if (!op)
         return fail(DLP_ERR_RUNTIME, "out of host memory");

@@ -177,9 +177,11 @@ void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
  *      t is bit for bit what the depthwise operator alone would write; the pointwise sum is accumulated in fp32 like "gemm".
  *      `dw_cfg` describes the depthwise layer (groups = channels_in = channels_out, kernel 3, pad 1, stride 1 or 2, shape =
  *      shape of x); x [B,C,H,W], dw_w [C,1,3,3], dw_bias [C], pw_w [channels_out,C,1,1], pw_bias [channels_out],
- *      y [B,channels_out,OH,OW].  float_data, W <= 56 (a multiple of 4, or of 2 up to 16), C a multiple of 8,
- *      channels_out <= 128, activations identity / relu / relu6: create returns DLP_ERR_NOT_IMPLEMENTED otherwise
- *      (dlp_dwpw_fwd_supported tells beforehand) and the caller keeps the two operators.  No workspace. ------------------ */
+ *      y [B,channels_out,OH,OW].  Served: float_data, images of at least 512 pixels and at most 56 wide whose output width is a
+ *      multiple of 4 (of 2 at stride 2 up to 28 wide), C a multiple of 8, channels_out <= 128, activations identity / relu /
+ *      relu6 -- the shapes where one launch beats the two operators (smaller images stay faster as two launches): create
+ *      returns DLP_ERR_NOT_IMPLEMENTED otherwise (dlp_dwpw_fwd_supported tells beforehand) and the caller keeps the two
+ *      operators.  No workspace. --------------------------------------------------------------------------------------- */
 typedef struct dlp_dwpw_fwd dlp_dwpw_fwd;
 int dlp_dwpw_fwd_supported(const dlp_conv2d_settings *dw_cfg, int dw_activation, int channels_out, int pw_activation);
 int dlp_dwpw_fwd_create(const dlp_conv2d_settings *dw_cfg, int dw_bias, int dw_activation, int channels_out, int pw_bias,
