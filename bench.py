@@ -135,7 +135,7 @@ def build_layers(layer_list, batch, seed, bf16=False):
 
 
 def matrix_peak_tflops(kernel_name):
-    return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith(("conv_gemm_bf16_kernel", "conv_patch_bf16_kernel")) else FP32_MATRIX_PEAK_TFLOPS
+    return BF16_MATRIX_PEAK_TFLOPS if kernel_name.startswith(("conv_gemm_bf16_kernel", "conv_patch_bf16_kernel", "conv_stem_bf16_kernel")) else FP32_MATRIX_PEAK_TFLOPS
 
 
 MAIN_SECTION = {"gemm": "conv_gemm", "winograd": "winograd_fused", "depthwise_separable": "sep_conv"}

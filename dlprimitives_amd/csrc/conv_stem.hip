@@ -1,5 +1,5 @@
 // Strided convolutions with very few input channels (the 7x7 / stride 2 / 3-channel stem of the
-// ResNet family): conv_stem_f32_kernel.
+// ResNet family): conv_stem_f32_kernel and, for bfloat16 tensors, conv_stem_bf16_kernel (described at the kernel).
 //
 // With 3 input channels the reduction index of the implicit GEMM runs over filter taps, so the
 // gathering kernel of conv_gemm.hip spends vector-ALU work on every gathered element and a K loop
@@ -40,14 +40,16 @@ constexpr int kStemPadL = 4;                    // zero columns left of an input
 constexpr uint32_t kStemOutOfRange = 0x80000000u; // >= num_records of every buffer we accept
 
 struct StemArgs {
-    const float *x, *w, *bias;
-    float *y;
+    const void *x, *w; // float or bfloat16, as the kernel says
+    const float *bias;
+    void *y;
     int B, H, W, Cout, OH, OW, OHW;
     int ph, pw;
     int total_rows, rows_per_wg; // output rows of the launch, numbered (m tile, image, row); rows per workgroup
     uint32_t x_img_bytes, y_img_bytes, w_bytes;
     uint32_t ow_magic, ow_shift;
     uint32_t padw, padw_magic, padw_shift; // PITCH - W zero columns per LDS row
+    int e0;                                // bf16 kernel: LDS column of the first of a lane's eight k for output column 0
     float factor;
     int pre, act;
     float clamp_lo, clamp_hi;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(kStemThreads) void conv_stem_f32_kernel(StemArgs a)
     }
     auto load_band = [&](int n, int iy0, unit_t (&xv)[NROWIT * NCH]) {
         const __amdgpu_buffer_rsrc_t xr =
-            __builtin_amdgcn_make_buffer_rsrc((void *)(a.x + (size_t)n * CIN * a.H * a.W), 0, a.x_img_bytes, 0x00020000);
+            __builtin_amdgcn_make_buffer_rsrc((void *)((const float *)a.x + (size_t)n * CIN * a.H * a.W), 0, a.x_img_bytes, 0x00020000);
 #pragma unroll
         for (int i = 0; i < NROWIT; i++) {
             const int q = wave + (kStemThreads / 64) * i;
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(kStemThreads) void conv_stem_f32_kernel(StemArgs a)
         // ---- blocks of 32 pixels of the band ----
         const int npix = rb * a.OW, nblk = (npix + 31) >> 5;
         const __amdgpu_buffer_rsrc_t yr =
-            __builtin_amdgcn_make_buffer_rsrc((void *)(a.y + (size_t)n * a.Cout * a.OHW), 0, a.y_img_bytes, 0x00020000);
+            __builtin_amdgcn_make_buffer_rsrc((void *)((float *)a.y + (size_t)n * a.Cout * a.OHW), 0, a.y_img_bytes, 0x00020000);
         // blocks are dealt round-robin: with wavefront w on SIMD w % 4 every SIMD gets the same number (+-1)
         for (int blk = wave; blk < nblk; blk += kStemThreads / 64) {
             const int p = blk * 32 + l32;
@@ -329,6 +331,266 @@ __global__ __launch_bounds__(kStemThreads) void conv_stem_f32_kernel(StemArgs a)
     }
 }
 
+// ---- bfloat16 tensors ----------------------------------------------------------------------------------------------
+// The same walk (one workgroup per CU, bands of R output rows, the next band's input rows in flight while this one is
+// computed) around v_mfma_f32_32x32x16_bf16, whose lanes hold EIGHT consecutive k each: one filter row of seven taps
+// and a leading zero.  The reduction therefore runs over the CIN * KH filter rows, two per instruction (one per half of
+// the wavefront), and an operand is 16 contiguous bytes on both sides:
+//   * pixels are the M side: lane (pixel p, half h) reads the eight input values left of and under filter row
+//     2j + h from the band in LDS, starting one element left of the window so that the address is a multiple of four
+//     bytes (even column: the kernel takes odd paddings only); the spare first element meets a zero weight;
+//   * filters are the N side: the tile's filters lie in LDS as [filter][filter row][8] with the zero in front.
+// With 21 filter rows that is 11 matrix instructions per 32 pixels x 32 filters -- some 15 us of matrix time for
+// ResNet-50's stem at batch 128 -- so the kernel is bound by its stores: the accumulators (lane = filter, register =
+// pixel, four consecutive pixels per register quad) are rounded, staged through LDS as [filter][pixel] and leave as
+// 16-byte stores, four lanes per 64-byte run of a filter's row.  Accumulation with an old y, and images whose rows are
+// not multiples of eight pixels, take 2-byte accesses straight from the accumulators.
+// As in the fp32 kernel, input values that are not finite may spread to the neighbouring output column through the
+// spare element (0 * inf).
+typedef __bf16 stem_bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t stem_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t stem_u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kStemPadL16 = 8;     // zero columns left of an input row (keeps the 16-byte LDS stores aligned)
+constexpr int kStemStagePitch = 80; // bytes per filter of a wavefront's staged 32 x 32 output block (64 + 16: 16-byte rows)
+
+template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, int NT>
+constexpr int stem_bf16_lds_bytes()
+{
+    constexpr int ROWS = STRIDE * (R - 1) + KH, QP = (CIN * KH + 1) / 2 * 2;
+    return CIN * ROWS * PITCH * 2 + 64 * (QP * 8 + 8) * 2 + 64 * 4 + (NT / 64) * 32 * kStemStagePitch;
+}
+
+template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, bool VEC, int NT>
+__global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
+{
+    static_assert(KW <= 7, "a filter row and its leading zero are the eight k of a lane");
+    constexpr int K = CIN * KH * KW;
+    constexpr int Q = CIN * KH, QP = (Q + 1) / 2 * 2, NJ = QP / 2; // filter rows, two per matrix instruction
+    constexpr int ROWS = STRIDE * (R - 1) + KH;                   // input rows of a full band
+    constexpr int QROWS = CIN * ROWS;
+    constexpr int WPITCH = QP * 8 + 8;                            // elements per filter in LDS (16-byte rows, off the powers of two)
+    constexpr int D1 = PITCH;                                     // filter row -> the next of the same channel
+    constexpr int D2 = (ROWS - KH + 1) * PITCH;                   // last filter row of a channel -> first of the next
+    constexpr int XU = VEC ? 8 : 1;                               // elements per load
+    constexpr int NROWIT = (QROWS + NT / 64 - 1) / (NT / 64);
+    constexpr int NCH = ((PITCH - 2 * kStemPadL16) / XU + 63) / 64;
+    constexpr int NWLOAD = (64 * K + NT - 1) / NT;
+    constexpr int YP = kStemStagePitch;
+    static_assert(PITCH % 8 == 0 && (QROWS * PITCH * 2) % 16 == 0 && (WPITCH * 2) % 16 == 0, "16-byte LDS rows");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char stem_lds[];
+    uint16_t *Ps = (uint16_t *)stem_lds;     // [QROWS][PITCH] input rows of the band
+    uint16_t *Ws = Ps + QROWS * PITCH;       // [64][WPITCH] filters of the tile
+    float *Bs = (float *)(Ws + 64 * WPITCH); // [64] bias
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    unsigned char *Ys = (unsigned char *)(Bs + 64) + wave * (32 * YP); // this wavefront's staged block
+    typedef typename std::conditional<VEC, stem_u32x4, uint16_t>::type unit_t;
+
+    const int first = (int)blockIdx.x * a.rows_per_wg, last = min(first + a.rows_per_wg, a.total_rows);
+    if (first >= last)
+        return;
+    const int boh = a.B * a.OH;
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+    // written once: the zero columns left and right of every input row, and the filter tile's zeros (leading element
+    // of every filter row, the spare filter row)
+    for (uint32_t idx = (uint32_t)tid; idx < (uint32_t)QROWS * a.padw; idx += NT) {
+        const uint32_t q = fast_div(idx, a.padw_magic, a.padw_shift), j = idx - q * a.padw;
+        Ps[q * PITCH + (j < (uint32_t)kStemPadL16 ? j : (uint32_t)a.W + j)] = 0;
+    }
+    for (int i = tid; i < 64 * WPITCH / 2; i += NT)
+        ((uint32_t *)Ws)[i] = 0u;
+
+    uint32_t lane_off[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        const int col = (lane + 64 * j) * XU;
+        lane_off[j] = col < a.W ? (uint32_t)col * 2u : kStemOutOfRange;
+    }
+    auto load_band = [&](int n, int iy0, unit_t (&xv)[NROWIT * NCH]) {
+        const __amdgpu_buffer_rsrc_t xr =
+            __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)a.x + (size_t)n * CIN * a.H * a.W), 0, a.x_img_bytes, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < NROWIT; i++) {
+            const int q = wave + (NT / 64) * i;
+            const int c = q / ROWS, pr = q - c * ROWS, iy = iy0 + pr;
+            const bool ok = q < QROWS && (unsigned)iy < (unsigned)a.H; // uniform
+            const uint32_t soff = ok ? (uint32_t)((c * a.H + iy) * a.W * 2) : 0u;
+#pragma unroll
+            for (int j = 0; j < NCH; j++) {
+                const uint32_t voff = ok ? lane_off[j] : kStemOutOfRange;
+                if constexpr (VEC)
+                    xv[i * NCH + j] = __builtin_amdgcn_raw_buffer_load_b128(xr, voff, soff, 0);
+                else
+                    xv[i * NCH + j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(xr, voff, soff, 0);
+            }
+        }
+    };
+    auto store_band = [&](const unit_t (&xv)[NROWIT * NCH]) {
+#pragma unroll
+        for (int i = 0; i < NROWIT; i++) {
+            const int q = wave + (NT / 64) * i;
+            if (q >= QROWS)
+                continue;
+#pragma unroll
+            for (int j = 0; j < NCH; j++) {
+                const int col = (lane + 64 * j) * XU;
+                if (col < a.W) {
+                    if constexpr (VEC)
+                        *(stem_u32x4 *)&Ps[q * PITCH + kStemPadL16 + col] = xv[i * NCH + j];
+                    else
+                        Ps[q * PITCH + kStemPadL16 + col] = xv[i * NCH + j];
+                }
+            }
+        }
+    };
+    auto decode = [&](int row, int &mt, int &n, int &oy, int &rb) {
+        mt = row / boh;
+        const int rem = row - mt * boh;
+        n = rem / a.OH;
+        oy = rem - n * a.OH;
+        rb = min(min(R, a.OH - oy), last - row);
+    };
+
+    int cur = first, mt, n, oy, rb, loaded_mt = -1;
+    decode(cur, mt, n, oy, rb);
+    unit_t xv[NROWIT * NCH];
+    load_band(n, STRIDE * oy - a.ph, xv);
+    const uint16_t *Wb = Ws + l32 * WPITCH + h * 8;
+    const bool use_old = a.factor != 0.0f, pre = a.pre != 0;
+    const bool generic = a.act == DLP_ACT_TANH || a.act == DLP_ACT_SIGMOID;
+    // 16-byte stores: rows of whole 8-pixel runs, every run 16-byte aligned
+    const bool wide = !use_old && a.OW % 8 == 0 && ((uintptr_t)a.y & 15) == 0;
+    auto activate = [&](float v) {
+        if (generic)
+            return apply_act(v, a.act);
+        return a.act != DLP_ACT_IDENTITY ? clamp_med3(v, a.clamp_lo, a.clamp_hi) : v; // identity must keep NaNs: no min/max
+    };
+
+    for (;;) {
+        const int m0 = mt * 64;
+        const bool new_tile = mt != loaded_mt; // uniform
+        __syncthreads(); // every wavefront has finished the previous band: LDS may be overwritten
+        store_band(xv);
+        if (new_tile) {
+            // filter m of the tile: K contiguous elements [c][r][s] -> LDS [c * KH + r][1 + s]; filters past Cout read as zero
+#pragma unroll
+            for (int i = 0; i < NWLOAD; i++) {
+                const int f = tid + i * NT;
+                const uint32_t voff = f < 64 * K ? ((uint32_t)m0 * K + (uint32_t)f) * 2u : kStemOutOfRange;
+                const uint16_t v = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(wr, voff, 0, 0);
+                if (f < 64 * K) {
+                    const int m = f / K, k = f - m * K, q = k / KW, s_ = k - q * KW;
+                    Ws[m * WPITCH + q * 8 + 1 + s_] = v;
+                }
+            }
+            if (tid < 64)
+                Bs[tid] = (a.bias != nullptr && m0 + tid < a.Cout) ? a.bias[m0 + tid] : 0.0f;
+        }
+        __syncthreads();
+        loaded_mt = mt;
+        const int next = cur + rb;
+        int nmt = mt, nn = n, noy = oy, nrb = 0;
+        if (next < last) {
+            decode(next, nmt, nn, noy, nrb);
+            load_band(nn, STRIDE * noy - a.ph, xv);
+        }
+
+        // ---- blocks of 32 pixels of the band ----
+        const int npix = rb * a.OW, nblk = (npix + 31) >> 5;
+        const __amdgpu_buffer_rsrc_t yr =
+            __builtin_amdgcn_make_buffer_rsrc((void *)((uint16_t *)a.y + (size_t)n * a.Cout * a.OHW), 0, a.y_img_bytes, 0x00020000);
+        for (int blk = wave; blk < nblk; blk += NT / 64) {
+            const int p = blk * 32 + l32;
+            const uint32_t pc = p < npix ? (uint32_t)p : 0u;
+            const int ro = (int)fast_div(pc, a.ow_magic, a.ow_shift), co = (int)pc - ro * a.OW;
+            const int lb = STRIDE * (ro * PITCH + co) + a.e0; // even
+            const uint32_t *P0 = (const uint32_t *)(Ps + lb), *P1 = (const uint32_t *)(Ps + lb + h * D1), *P2 = (const uint32_t *)(Ps + lb + h * D2);
+
+            stem_f32x16 acc[2];
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++) {
+                const float b = Bs[cb * 32 + l32];
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[cb][r] = b;
+            }
+            stem_for<NJ>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                constexpr int q0 = 2 * j, q1 = 2 * j + 1;
+                constexpr int o0 = ((q0 / KH) * ROWS + q0 % KH) * PITCH, o1 = ((q1 / KH) * ROWS + q1 % KH) * PITCH;
+                constexpr int d = q1 < Q ? o1 - o0 : 0; // the spare filter row has zero weights: the other half's values do
+                static_assert(d == 0 || d == D1 || d == D2, "filter row distance");
+                static_assert(o0 % 2 == 0, "dword aligned");
+                const uint32_t *pp = (d == D1 ? P1 : d == D2 ? P2 : P0) + o0 / 2;
+                stem_u32x4 px;
+                px[0] = pp[0], px[1] = pp[1], px[2] = pp[2], px[3] = pp[3];
+                const stem_bf16x8 xa = __builtin_bit_cast(stem_bf16x8, px);
+                const stem_bf16x8 w0 = *(const stem_bf16x8 *)(Wb + j * 16), w1 = *(const stem_bf16x8 *)(Wb + 32 * WPITCH + j * 16);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w0, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w1, acc[1], 0, 0, 0);
+            });
+
+            // accumulator register r of filter block cb: filter m0 + 32 * cb + l32, pixel blk * 32 + 8 * (r / 4) + 4 * h + r % 4
+            if (wide) {
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); // the block's previous reads are done
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        stem_u32x2 o;
+#pragma unroll
+                        for (int e = 0; e < 2; e++) {
+                            const float lo = activate(acc[cb][4 * rq + 2 * e]), hi = activate(acc[cb][4 * rq + 2 * e + 1]);
+                            o[e] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                        }
+                        *(stem_u32x2 *)(Ys + l32 * YP + (8 * rq + 4 * h) * 2) = o;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const int fl = t * 16 + (lane >> 2), seg = lane & 3; // filter of the block, run of eight pixels
+                        const stem_u32x4 o = *(const stem_u32x4 *)(Ys + fl * YP + seg * 16);
+                        const int m = m0 + cb * 32 + fl, p0 = blk * 32 + seg * 8;
+                        const uint32_t voff = (m < a.Cout && p0 < npix) ? (uint32_t)((m * a.OHW + oy * a.OW + p0) * 2) : kStemOutOfRange;
+                        __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff, 0, 0);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++) {
+                    const int m = m0 + cb * 32 + l32;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int pp = blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                        const uint32_t voff = (m < a.Cout && pp < npix) ? (uint32_t)((m * a.OHW + oy * a.OW + pp) * 2) : kStemOutOfRange;
+                        float v = acc[cb][r], old = 0.0f;
+                        if (use_old)
+                            old = __builtin_bit_cast(float, (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(yr, voff, 0, 0) << 16);
+                        if (use_old && pre)
+                            v = fmaf(old, a.factor, v);
+                        v = activate(v);
+                        if (use_old && !pre)
+                            v = fmaf(old, a.factor, v);
+                        __builtin_amdgcn_raw_buffer_store_b16((short)to_bf16(v).bits, yr, voff, 0, 0);
+                    }
+                }
+            }
+        }
+        if (next >= last)
+            break;
+        cur = next;
+        mt = nmt;
+        n = nn;
+        oy = noy;
+        rb = nrb;
+    }
+}
+
 constexpr int kStemR = 8, kStemPitch = 240;
 
 bool generic_activation(int act) { return act == DLP_ACT_TANH || act == DLP_ACT_SIGMOID; }
@@ -350,15 +612,24 @@ int stem_cu_count()
 
 bool conv_stem_supported(const ConvGeom &g)
 {
-    if (g.dtype != DLP_FLOAT || g.groups != 1 || g.Cin != 3 || g.KH != 7 || g.KW != 7 || g.sh != 2 || g.sw != 2 || g.dh != 1 || g.dw != 1)
+    if ((g.dtype != DLP_FLOAT && g.dtype != DLP_BFLOAT16) || g.groups != 1 || g.Cin != 3 || g.KH != 7 || g.KW != 7 || g.sh != 2 || g.sw != 2 || g.dh != 1 ||
+        g.dw != 1)
         return false;
-    if (g.pw < 0 || g.pw > kStemPadL || g.ph < 0 || g.Cout % 8 != 0 || g.OH <= 0 || g.OW <= 0)
+    if (g.pw < 0 || g.ph < 0 || g.OH <= 0 || g.OW <= 0)
+        return false;
+    const long long esize = g.dtype == DLP_FLOAT ? 4 : 2;
+    if ((long long)g.Cin * g.H * g.W * esize >= 0x7fffffffLL || (long long)g.Cout * g.OH * g.OW * esize >= 0x7fffffffLL || (long long)g.Cout * 147 * esize >= 0x7fffffffLL)
+        return false;
+    if (g.dtype == DLP_BFLOAT16) {
+        // a lane's eight k start one element left of the window, on an even LDS column: odd paddings only;
+        // rightmost column read: the eighth element of the last output column
+        const int e0 = kStemPadL16 - g.pw - 1;
+        return e0 >= 0 && e0 % 2 == 0 && 2 * (g.OW - 1) + e0 + 7 < kStemPitch && g.W + 2 * kStemPadL16 <= kStemPitch;
+    }
+    if (g.pw > kStemPadL || g.Cout % 8 != 0)
         return false;
     // rightmost LDS column a lane may read: last tap of the last output column, plus the spare k
-    if (2 * (g.OW - 1) - g.pw + 6 + kStemPadL + 1 >= kStemPitch || g.W + 2 * kStemPadL > kStemPitch)
-        return false;
-    return (long long)g.Cin * g.H * g.W * 4 < 0x7fffffffLL && (long long)g.Cout * g.OH * g.OW * 4 < 0x7fffffffLL &&
-           (long long)g.Cout * 147 * 4 < 0x7fffffffLL;
+    return 2 * (g.OW - 1) - g.pw + 6 + kStemPadL + 1 < kStemPitch && g.W + 2 * kStemPadL <= kStemPitch;
 }
 
 int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream)
@@ -368,10 +639,12 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     if (g.B == 0)
         return DLP_OK;
     StemArgs a;
-    a.x = (const float *)x;
-    a.w = (const float *)w;
+    const bool bf16 = g.dtype == DLP_BFLOAT16;
+    const size_t esize = bf16 ? 2 : 4;
+    a.x = x;
+    a.w = w;
     a.bias = ep.bias;
-    a.y = (float *)y;
+    a.y = y;
     a.B = g.B; a.H = g.H; a.W = g.W; a.Cout = g.Cout; a.OH = g.OH; a.OW = g.OW; a.OHW = g.OH * g.OW;
     a.ph = g.ph; a.pw = g.pw;
     const int mtiles = (g.Cout + 63) / 64;
@@ -382,13 +655,14 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     const int wgs = (int)std::min<long long>(stem_cu_count(), (total + 1) / 2);
     a.total_rows = (int)total;
     a.rows_per_wg = (int)((total + wgs - 1) / wgs);
-    a.x_img_bytes = (uint32_t)((size_t)g.Cin * g.H * g.W * 4);
-    a.y_img_bytes = (uint32_t)((size_t)g.Cout * g.OH * g.OW * 4);
-    a.w_bytes = (uint32_t)((size_t)g.Cout * 147 * 4);
-    // 16-byte loads: every input row and the filter rows of every m tile then start 16-byte aligned
-    const bool vec = g.W % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
+    a.x_img_bytes = (uint32_t)((size_t)g.Cin * g.H * g.W * esize);
+    a.y_img_bytes = (uint32_t)((size_t)g.Cout * g.OH * g.OW * esize);
+    a.w_bytes = (uint32_t)((size_t)g.Cout * 147 * esize);
+    // 16-byte loads: every input row and (fp32) the filter rows of every m tile then start 16-byte aligned
+    const bool vec = bf16 ? g.W % 8 == 0 && ((uintptr_t)x & 15) == 0 : g.W % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
     make_magic((uint32_t)g.OW, a.ow_magic, a.ow_shift);
     a.padw = (uint32_t)(kStemPitch - g.W);
+    a.e0 = kStemPadL16 - g.pw - 1;
     make_magic(a.padw, a.padw_magic, a.padw_shift);
     a.factor = ep.factor;
     a.pre = ep.accumulate_first;
@@ -401,6 +675,19 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         a.clamp_hi = 6.0f;
     const dim3 grid((unsigned)((a.total_rows + a.rows_per_wg - 1) / a.rows_per_wg)), block(kStemThreads);
     TimingScope ts("conv_gemm", stream);
+    if (bf16) {
+        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemR, kStemPitch, kStemThreads>();
+        auto kernel = vec ? conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, kStemThreads> : conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, kStemThreads>;
+        // more than 64 KB of LDS has to be asked for (bands of 16 rows, or two workgroups of 8 wavefronts per CU, were no faster)
+        static bool asked[2] = {false, false};
+        if (!asked[vec]) {
+            DLP_HIP_TRY(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            asked[vec] = true;
+        }
+        DLP_LAUNCH_TIMED(ts, kernel, grid, block, lds, stream, a);
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
     const bool gen = generic_activation(ep.activation);
     if (vec && !gen)
         DLP_LAUNCH_TIMED(ts, (conv_stem_f32_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, false>), grid, block, 0, stream, a);

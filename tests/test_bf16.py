@@ -139,6 +139,40 @@ def test_bf16_depthwise_vs_fp32_reference(oracle_mod, ch, hw, stride, k):
     assert np.abs(got - want).max() <= 1e-2 * max(np.abs(want).max(), 1.0)
 
 
+# the 3-channel 7x7 stride-2 stem kernel: (case, (batch, H, W)); integer-valued tensors must come out exactly
+STEM_CASES = [
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (3, 224, 224)),    # the ResNet stem: 16-byte loads and stores
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (2, 100, 92)),     # rows off the 16-byte units: 2-byte loads and stores
+    (case(7, 3, 2, 1, 3, 24, False, 1, False), (2, 45, 96)),    # fewer filters than a block, odd height, no bias
+    (case(7, 1, 2, 1, 3, 96, True, 1, True), (2, 70, 88)),      # padding 1, two filter tiles (the second half empty)
+    (case(7, (2, 5), 2, 1, 3, 40, True, 1, False), (5, 33, 64)),  # uneven padding; bands that end with the image
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (1, 7, 8)),        # a single band of four pixels per row
+]
+
+
+@pytest.mark.parametrize("c,bhw", STEM_CASES, ids=case_id)
+def test_bf16_stem(oracle_mod, c, bhw):
+    print("stem", c["pad"], c["cout"], bhw, flush=True)
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    x, w, bias = make_tensors(c, bhw, seed=41)
+    x, w = oracle_mod.bf16_round(x), oracle_mod.bf16_round(w)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm")
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8)
+    np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-4 * np.abs(want).max())
+    rng = np.random.default_rng(3)
+    xi = rng.integers(-2, 3, x.shape).astype(np.float32)
+    wi = rng.integers(-1, 2, w.shape).astype(np.float32)
+    bi = rng.integers(-3, 4, c["cout"]).astype(np.float32) if c["bias"] else None
+    want = oracle_mod.conv2d_forward(xi, wi, bi, cfg, c["activation"], threads=8)
+    assert np.abs(want).max() <= 256  # exactly representable in bf16
+    assert np.array_equal(run_conv_bf16(c, xi, wi, bi, algo="gemm"), want)
+    # accumulation with the old y (2-byte path), after the activation
+    old = rng.standard_normal(want.shape).astype(np.float32)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    want = oracle_mod.apply_factor(oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8), oracle_mod.bf16_round(old), 0.5)
+    np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-3)
+
+
 def test_bf16_factor_contract(oracle_mod):
     c = case(3, 1, 1, 1, 16, 24, True, 1, True)
     x, w, bias = make_tensors(c, (2, 11, 9), seed=5)
