@@ -679,10 +679,13 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemR, kStemPitch, kStemThreads>();
         auto kernel = vec ? conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, kStemThreads> : conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, kStemThreads>;
         // more than 64 KB of LDS has to be asked for (bands of 16 rows, or two workgroups of 8 wavefronts per CU, were no faster)
-        static bool asked[2] = {false, false};
-        if (!asked[vec]) {
+        static bool asked[2][64] = {}; // per kernel and device
+        int dev = 0;
+        DLP_HIP_TRY(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 64 || !asked[vec][dev]) {
             DLP_HIP_TRY(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-            asked[vec] = true;
+            if (dev >= 0 && dev < 64)
+                asked[vec][dev] = true;
         }
         DLP_LAUNCH_TIMED(ts, kernel, grid, block, lds, stream, a);
         DLP_HIP_TRY(hipGetLastError());
