@@ -135,6 +135,90 @@ __global__ __launch_bounds__(256) void maxpool3x3s2p1_kernel(PoolArgs a, int nst
     }
 }
 
+// The same pooling for rows of whole groups of eight input columns (W % 8 == 0, OW == W / 2, 16-byte aligned tensors): a lane owns
+// FOUR output columns, loads their eight input columns of a row with one 16-byte load (two for float) and stores four results at
+// once -- a quarter of the memory instructions per byte, which is what bounds the kernel above on 2-byte elements (the texture
+// path takes four lanes per clock whatever the width of the access).
+template <class T>
+__global__ __launch_bounds__(256) void maxpool3x3s2p1_wide_kernel(PoolArgs a, int nstrips, long long total_groups, int groups_per_row)
+{
+    constexpr int NIN = 2 * kMaxStrip + 1;
+    constexpr float kLowest = -3.402823466e+38f;
+    typedef uint32_t pool_u32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t pool_u32x2 __attribute__((ext_vector_type(2)));
+    typedef float pool_f32x4 __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x & 63;
+    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long f = wave * 63 + lane - 1; // flat (plane, strip, group of four output columns) index
+    const bool in_range = f >= 0 && f < total_groups;
+    const long long ps = in_range ? f / groups_per_row : 0;
+    const int gx = in_range ? (int)(f - ps * groups_per_row) : 0;
+    const long long plane = ps / nstrips;
+    const int strip = (int)(ps - plane * nstrips);
+    const int oy0 = strip * kMaxStrip;
+    const T *xp = (const T *)a.x + plane * a.H * a.W + 8 * gx;
+    const bool has_left = gx > 0;
+
+    float m[NIN][4]; // maxima over the three window columns of the four outputs, per input row
+    const int iy0 = 2 * oy0 - 1;
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+        const int yy = iy0 + r;
+        const bool vy = in_range && yy >= 0 && yy < a.H;
+        const T *p = xp + (size_t)(vy ? yy : 0) * a.W;
+        float c[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            c[e] = kLowest;
+        if (vy) {
+            if constexpr (sizeof(T) == 4) {
+                const pool_f32x4 v0 = *(const pool_f32x4 *)p, v1 = *(const pool_f32x4 *)(p + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    c[e] = v0[e];
+                    c[4 + e] = v1[e];
+                }
+            } else {
+                const pool_u32x4 v = *(const pool_u32x4 *)p;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    c[2 * e] = __builtin_bit_cast(float, v[e] << 16);
+                    c[2 * e + 1] = __builtin_bit_cast(float, v[e] & 0xffff0000u);
+                }
+            }
+        }
+        const float l = __shfl_up(c[7], 1); // the left lane's last column = 8 * gx - 1
+        m[r][0] = fmaxf(fmaxf(has_left ? l : kLowest, c[0]), c[1]);
+        m[r][1] = fmaxf(fmaxf(c[1], c[2]), c[3]);
+        m[r][2] = fmaxf(fmaxf(c[3], c[4]), c[5]);
+        m[r][3] = fmaxf(fmaxf(c[5], c[6]), c[7]);
+    }
+    if (!in_range || lane == 0)
+        return;
+    T *yp = (T *)a.y + plane * a.OH * a.OW + 4 * gx;
+#pragma unroll
+    for (int j = 0; j < kMaxStrip; j++) {
+        const int oy = oy0 + j;
+        if (oy >= a.OH)
+            continue;
+        float o[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            o[q] = fmaxf(fmaxf(m[2 * j][q], m[2 * j + 1][q]), m[2 * j + 2][q]);
+        if constexpr (sizeof(T) == 4) {
+            pool_f32x4 v;
+            v[0] = o[0], v[1] = o[1], v[2] = o[2], v[3] = o[3];
+            *(pool_f32x4 *)(yp + (size_t)oy * a.OW) = v;
+        } else {
+            // the values are bf16 already (maxima of stored values): the upper halves are the results
+            pool_u32x2 v;
+            v[0] = (__builtin_bit_cast(uint32_t, o[0]) >> 16) | (__builtin_bit_cast(uint32_t, o[1]) & 0xffff0000u);
+            v[1] = (__builtin_bit_cast(uint32_t, o[2]) >> 16) | (__builtin_bit_cast(uint32_t, o[3]) & 0xffff0000u);
+            *(pool_u32x2 *)(yp + (size_t)oy * a.OW) = v;
+        }
+    }
+}
+
 // LPP lanes per plane (64: one wavefront per plane; 16: four planes per wavefront, for the 7x7 and
 // smaller planes at the end of a network): lanes stride over the plane, then a shuffle reduction.
 // The average is accumulated per lane in ascending index order and combined pairwise,
@@ -425,6 +509,18 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         TimingScope ts("pooling", s);
         if (a.mode == 0 && a.kh == 3 && a.kw == 3 && a.sh == 2 && a.sw == 2 && a.ph == 1 && a.pw == 1) {
             const int nstrips = (a.OH + kMaxStrip - 1) / kMaxStrip;
+            if (a.W % 8 == 0 && a.OW * 2 == a.W && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
+                const int groups_per_row = a.OW / 4;
+                const long long total_groups = planes * nstrips * groups_per_row;
+                const long long wblocks = ((total_groups + 62) / 63 + 3) / 4;
+                DLP_REQUIRE(wblocks < 0x7fffffffLL, "tensor too large");
+                if (op->dtype == DLP_BFLOAT16)
+                    hipLaunchKernelGGL(maxpool3x3s2p1_wide_kernel<bf16_t>, dim3((unsigned)wblocks), dim3(256), 0, s, a, nstrips, total_groups, groups_per_row);
+                else
+                    hipLaunchKernelGGL(maxpool3x3s2p1_wide_kernel<float>, dim3((unsigned)wblocks), dim3(256), 0, s, a, nstrips, total_groups, groups_per_row);
+                DLP_HIP_TRY(hipGetLastError());
+                return DLP_OK;
+            }
             const long long total_cols = planes * nstrips * a.OW;
             const long long blocks = ((total_cols + 62) / 63 + 3) / 4;
             const size_t esize = dtype_size(op->dtype);

@@ -136,7 +136,8 @@ def test_gpu_pooling_large_shapes_vs_oracle(oracle_mod):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gpu_maxpool_3x3_stride2_pad1_shapes(oracle_mod, dtype):
     """The strip kernel behind max pooling 3x3 / stride 2 / pad 1: odd and even sizes, planes smaller than a
-    strip, rows shorter than a wavefront, ceil-mode output sizes; a maximum of stored values is exact."""
+    strip, rows shorter than a wavefront, ceil-mode output sizes, and rows of whole groups of eight columns (four outputs per lane);
+    a maximum of stored values is exact."""
     import torch
 
     import dlprimitives_amd as dlp
@@ -145,7 +146,7 @@ def test_gpu_maxpool_3x3_stride2_pad1_shapes(oracle_mod, dtype):
     rng = np.random.default_rng(3)
     tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     for (b, c, h, w, ceil_mode) in [(2, 3, 112, 112, 0), (1, 5, 7, 7, 0), (3, 2, 13, 9, 1), (2, 4, 30, 31, 0), (1, 1, 2, 2, 0), (2, 7, 15, 64, 1),
-                                    (1, 2, 57, 130, 0)]:
+                                    (1, 2, 57, 130, 0), (2, 3, 56, 48, 0), (1, 2, 9, 8, 0), (3, 1, 113, 16, 0), (1, 65, 5, 24, 0)]:
         x = rng.standard_normal((b, c, h, w)).astype(np.float32)
         if dtype == "bfloat16":
             x = oracle_mod.bf16_round(x)
