@@ -303,3 +303,45 @@ def mobilenet_v2(batch, size=224, classes=1000, activation="relu6"):
     b.ip(t, "loss", classes, prefix="classifier")
     b.output("loss")
     return b
+
+
+def alexnet(batch, size=224, classes=1000, hidden=4096):
+    """The operator list of docs/nets_for_benchmark/alexnet-b16.js at another batch / image size / width of the hidden layers:
+    convolutions 11x11/4, 5x5 and 3x3 with bias and ReLU in their epilogues, max pooling 3x3/2 without padding, the 1x1
+    average pooling that the exporter leaves where torchvision's adaptive pooling is the identity, and three inner products,
+    the first of which takes the 4-D tensor as it is."""
+    b = NetBuilder("data", (batch, 3, size, size))
+    x = b.conv("data", "c1", 64, 11, 4, 2, bias=True, activation="relu")
+    x = b.pool(x, "p1", "max", 3, 2, 0)
+    x = b.conv(x, "c2", 192, 5, 1, 2, bias=True, activation="relu")
+    x = b.pool(x, "p2", "max", 3, 2, 0)
+    x = b.conv(x, "c3", 384, 3, 1, 1, bias=True, activation="relu")
+    x = b.conv(x, "c4", 256, 3, 1, 1, bias=True, activation="relu")
+    x = b.conv(x, "c5", 256, 3, 1, 1, bias=True, activation="relu")
+    x = b.pool(x, "p5", "max", 3, 2, 0)
+    x = b.pool(x, "p6", "avg", 1, 1, 0)
+    x = b.ip(x, "f6", hidden, activation="relu")
+    x = b.ip(x, "f7", hidden, activation="relu")
+    b.ip(x, "loss", classes)
+    b.output("loss")
+    return b
+
+
+def vgg16(batch, size=224, classes=1000, hidden=4096):
+    """The operator list of docs/nets_for_benchmark/vgg16-b16.js at another batch / image size / width of the hidden layers:
+    thirteen 3x3 convolutions with bias and ReLU, five max poolings 2x2/2, the identity average pooling and three inner products."""
+    b = NetBuilder("data", (batch, 3, size, size))
+    x = "data"
+    n = 0
+    for block, (cout, convs) in enumerate(((64, 2), (128, 2), (256, 3), (512, 3), (512, 3))):
+        for _ in range(convs):
+            n += 1
+            x = b.conv(x, "c%d" % n, cout, 3, 1, 1, bias=True, activation="relu")
+        x = b.pool(x, "p%d" % (block + 1), "max", 2, 2, 0)
+    x = b.pool(x, "p6", "avg", 1, 1, 0)
+    x = b.ip(x, "f6", hidden, activation="relu")
+    x = b.ip(x, "f7", hidden, activation="relu")
+    b.ip(x, "loss", classes)
+    b.output("loss")
+    return b
+

@@ -128,7 +128,7 @@ def test_plan_resnet18_rewrites_and_memory(tmp_path):
 
 
 @pytest.mark.skipif(not os.path.isdir(REF_NETS), reason="reference tree not present")
-@pytest.mark.parametrize("name", ["resnet18", "resnet50", "mobilenet_v2"])
+@pytest.mark.parametrize("name", ["resnet18", "resnet50", "mobilenet_v2", "alexnet", "vgg16"])
 def test_builders_write_the_reference_operator_lists(name):
     """Same operator types, in the same order, with the same options, as the reference's file."""
     ref = json.load(open(os.path.join(REF_NETS, name + "-b16.js")))
@@ -322,6 +322,8 @@ NETS = {
     "resnet18_b2_64": (lambda: netfile.resnet18(2, 64, 10), 6),
     "resnet50_b2_64": (lambda: netfile.resnet50(2, 64, 10), 8),
     "mobilenet_v2_b3_64": (lambda: netfile.mobilenet_v2(3, 64, 10), 7),
+    "alexnet_b2_224": (lambda: netfile.alexnet(2, 224, 10, hidden=192), 3),
+    "vgg16_b2_64": (lambda: netfile.vgg16(2, 64, 10, hidden=160), 4),
 }
 
 
