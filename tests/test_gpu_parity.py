@@ -110,6 +110,12 @@ PATCH_SHAPES = [
     (3, 64, 128, 2, 9, 11),    # groups, odd width
     (2, 48, 80, 1, 6, 62),     # widest supported row; 3 stages (odd), Cout off the tile size
     (2, 48, 80, 1, 6, 63),     # one pixel wider: the gathering kernel
+    (2, 32, 64, 1, 20, 112),   # wide rows (the gathering kernel from here on): tiles inside a row and across two rows
+    (1, 16, 48, 1, 5, 224),    # a tile is a piece of one row
+    (2, 16, 64, 1, 3, 70),     # three rows: every tile touches the top or the bottom of the plane
+    (5, 32, 64, 1, 1, 64),     # one row per image
+    (3, 16, 40, 1, 2, 97),     # odd width, tiles crossing images, N tail
+    (2, 64, 96, 2, 9, 65),     # groups
     (4, 32, 64, 1, 5, 6),      # plane below 32 pixels: the gathering kernel
     (1, 16, 40, 1, 40, 40),    # one stage per tile
 ]
