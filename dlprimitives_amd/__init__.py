@@ -27,6 +27,7 @@ from .capi import (  # noqa: F401
     conv2d_output_shape,
     conv2d_transposed_output_shape,
     eltwise_forward,
+    slice_copy,
     lib,
     library_path,
     pool2d_output_size,

@@ -550,6 +550,28 @@ def eltwise_forward(a, b, c, operation="sum", coef1=1.0, coef2=1.0, activation="
                                                a.numel(), _ptr(a), _ptr(b), _ptr(c), _stream(stream)))
 
 
+def slice_copy(dst, dst_offset, src, src_offset, length, dim=1, stream=None):
+    """The copy of Concat::forward / Slice::forward: dst[..., dst_offset:dst_offset+length, ...] = src[..., src_offset:src_offset+length, ...]
+    along axis `dim` of two contiguous tensors that agree in every other dimension."""
+    if dst.dim() != src.dim() or dst.dtype != src.dtype or not (dst.is_contiguous() and src.is_contiguous()):
+        raise ValidationError("slice_copy: contiguous tensors of the same rank and type are needed")
+    for j in range(dst.dim()):
+        if j != dim and dst.shape[j] != src.shape[j]:
+            raise ValidationError("slice_copy: the tensors differ outside the axis")
+    if dst_offset < 0 or src_offset < 0 or dst_offset + length > dst.shape[dim] or src_offset + length > src.shape[dim]:
+        raise ValidationError("slice_copy: range outside the axis")
+    es = dst.element_size()
+    outer = 1
+    for j in range(dim):
+        outer *= int(dst.shape[j])
+    inner = es
+    for j in range(dim + 1, dst.dim()):
+        inner *= int(dst.shape[j])
+    lib().dlp_copy2d_enqueue.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
+    _check(lib().dlp_copy2d_enqueue(dst.data_ptr() + dst_offset * inner, int(dst.shape[dim]) * inner, src.data_ptr() + src_offset * inner,
+                                    int(src.shape[dim]) * inner, length * inner, outer, _stream(stream)))
+
+
 def activation_forward(x, y, activation, stream=None):
     """Activation::forward: y = act(x); y may be x"""
     lib().dlp_activation_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]

@@ -420,6 +420,18 @@ static int pool_create(const int kernel[2], const int pad[2], const int stride[2
     return DLP_OK;
 }
 
+// rows x width units of U from a pitched source to a pitched destination (pitches in units); consecutive threads take consecutive
+// units of a row
+template <class U>
+__global__ __launch_bounds__(256) void copy2d_kernel(U *__restrict__ dst, size_t dst_pitch, const U *__restrict__ src, size_t src_pitch, size_t width, size_t rows)
+{
+    const size_t total = width * rows;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t r = i / width, c = i - r * width;
+        dst[r * dst_pitch + c] = src[r * src_pitch + c];
+    }
+}
+
 extern "C" {
 
 int dlp_pool2d_output_size(int in_size, int kernel, int pad, int stride, int ceil_mode, int *out_size)
@@ -542,6 +554,33 @@ void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op) { delete op; }
 
 static int eltwise_launch(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b,
                           void *c, void *stream);
+
+int dlp_copy2d_enqueue(void *dst, size_t dst_pitch, const void *src, size_t src_pitch, size_t width_bytes, size_t rows, void *stream)
+{
+    if (width_bytes == 0 || rows == 0)
+        return DLP_OK;
+    DLP_REQUIRE(dst != nullptr && src != nullptr, "null tensor pointer");
+    DLP_REQUIRE(dst_pitch >= width_bytes && src_pitch >= width_bytes, "a row is longer than its pitch");
+    hipStream_t st = (hipStream_t)stream;
+    // the widest unit that every address of the copy is a multiple of
+    const uintptr_t all = (uintptr_t)dst | (uintptr_t)src | dst_pitch | src_pitch | width_bytes;
+    const size_t unit = (all & 15) == 0 ? 16 : (all & 3) == 0 ? 4 : (all & 1) == 0 ? 2 : 1;
+    const size_t total = width_bytes / unit * rows;
+    const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65536);
+    TimingScope ts("copy", st);
+    typedef uint32_t copy_u32x4 __attribute__((ext_vector_type(4)));
+    if (unit == 16)
+        hipLaunchKernelGGL(copy2d_kernel<copy_u32x4>, dim3(blocks), dim3(256), 0, st, (copy_u32x4 *)dst, dst_pitch / 16, (const copy_u32x4 *)src, src_pitch / 16,
+                           width_bytes / 16, rows);
+    else if (unit == 4)
+        hipLaunchKernelGGL(copy2d_kernel<uint32_t>, dim3(blocks), dim3(256), 0, st, (uint32_t *)dst, dst_pitch / 4, (const uint32_t *)src, src_pitch / 4, width_bytes / 4, rows);
+    else if (unit == 2)
+        hipLaunchKernelGGL(copy2d_kernel<uint16_t>, dim3(blocks), dim3(256), 0, st, (uint16_t *)dst, dst_pitch / 2, (const uint16_t *)src, src_pitch / 2, width_bytes / 2, rows);
+    else
+        hipLaunchKernelGGL(copy2d_kernel<uint8_t>, dim3(blocks), dim3(256), 0, st, (uint8_t *)dst, dst_pitch, (const uint8_t *)src, src_pitch, width_bytes, rows);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
 
 int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activation, size_t n, const void *a, const void *b, void *c,
                             void *stream)

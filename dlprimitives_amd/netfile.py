@@ -198,6 +198,39 @@ class NetBuilder:
         self.shapes[dst] = (s[0], int(np.prod(s[1:])))
         return dst
 
+    def concat(self, srcs, dst, dim=1):
+        shapes = [self.shapes[s] for s in srcs]
+        self._op("Concat", "Concat", list(srcs), [dst], {"dim": dim})
+        out = list(shapes[0])
+        out[dim] = sum(sh[dim] for sh in shapes)
+        self.shapes[dst] = tuple(out)
+        return dst
+
+    def slice(self, src, dst, begin=0, end=-1, dim=1):
+        s = list(self.shapes[src])
+        self._op("Slice", "Slice", [src], [dst], {"dim": dim, "begin": begin, "end": end})
+        s[dim] = (s[dim] if end == -1 else end) - begin
+        self.shapes[dst] = tuple(s)
+        return dst
+
+    def reshape(self, src, dst, dims):
+        s = self.shapes[src]
+        self._op("Reshape", "Reshape", [src], [dst], {"dims": list(dims)})
+        out = [s[i] if d == 0 else d for i, d in enumerate(dims)]
+        if -1 in out:
+            known = int(np.prod([d for d in out if d != -1]))
+            out[out.index(-1)] = int(np.prod(s)) // known
+        self.shapes[dst] = tuple(out)
+        return dst
+
+    def squeeze(self, src, dst, dims=None):
+        s = self.shapes[src]
+        opts = {"dims": list(dims)} if dims is not None else {"all": True}
+        self._op("Squeeze", "Squeeze", [src], [dst], opts)
+        axes = [d % len(s) for d in dims] if dims is not None else [i for i, d in enumerate(s) if d == 1]
+        self.shapes[dst] = tuple(d for i, d in enumerate(s) if i not in axes) or (1,)
+        return dst
+
     def softmax(self, src, dst, log=False):
         self._op("Softmax", "Softmax", [src], [dst], {"log": bool(log)})
         self.shapes[dst] = self.shapes[src]

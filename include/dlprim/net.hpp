@@ -8,7 +8,7 @@
 // liveness (src/net.cpp:585-654: intermediate tensors share chunks unless keep_intermediate_tensors),
 // and runs the operators in order on one ExecutionContext with one shared workspace
 // (src/net.cpp:836-851).  Operator types: Convolution2D, BatchNorm, Activation, Pooling2D,
-// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- plus Softmax, Flatten and
+// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- plus Softmax, Flatten, Concat, Slice, Reshape, Squeeze and
 // TransposedConvolution2D, with the option names of the reference's *Config::from_json functions.
 //
 // In predict mode two graph rewrites are applied at setup (fuse(true), the default):
@@ -220,6 +220,9 @@ public:
                 break;
             case k_gpool: out = Shape(in[0], in[1], 1, 1); break;
             case k_flatten: out = Shape(in[0], in.size_no_batch()); break;
+            case k_concat: out = concat_shape(n); break;
+            case k_slice: out = slice_shape(n, in); break;
+            case k_view: out = view_shape(n, in); break;
             case k_eltwise:
                 if (spec(n.inputs[1]) != in)
                     throw ValidationError("Elementwise inputs of different shapes after reshape (" + n.name + ")");
@@ -401,7 +404,7 @@ public:
     }
 
 private:
-    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv };
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv, k_concat, k_slice, k_view };
     struct Node {
         std::string name, type;
         std::vector<std::string> inputs, outputs, param_names;
@@ -440,7 +443,104 @@ private:
         float coef[2] = {1.0f, 1.0f};
         // Softmax
         bool log_softmax = false;
+        // Concat / Slice: the axis, and the range of a Slice (end -1: to the end of the axis)
+        int dim = 1, slice_begin = 0, slice_end = -1;
+        // Reshape (view_dims as given: 0 keeps the input's dimension, -1 is deduced) / Squeeze (view_dims: the axes; empty: all of extent 1)
+        bool squeeze = false;
+        std::vector<int> view_dims;
     };
+
+    static std::vector<int> int_list(json::value const &o, char const *key)
+    {
+        std::vector<int> r;
+        json::value const &v = o.find(key);
+        if (v.is_undefined())
+            return r;
+        if (v.type() == json::is_array) {
+            for (size_t i = 0; i < v.size(); i++)
+                r.push_back((int)v[i].number());
+        } else
+            r.push_back((int)v.number());
+        return r;
+    }
+    // Concat: all inputs agree but for the axis (src/ops/concat.cpp:44-64)
+    Shape concat_shape(Node const &n) const
+    {
+        Shape r = spec(n.inputs[0]);
+        DLPRIM_CHECK(n.dim >= 0 && n.dim < r.size());
+        size_t total = 0;
+        for (auto const &name : n.inputs) {
+            Shape const &in = spec(name);
+            DLPRIM_CHECK(in.size() == r.size());
+            for (int j = 0; j < r.size(); j++)
+                if (j != n.dim && in[j] != r[j])
+                    throw ValidationError("Concat inputs differ outside the axis (" + n.name + ")");
+            total += in[n.dim];
+        }
+        r[n.dim] = total;
+        return r;
+    }
+    // Slice (src/ops/concat.cpp:231-249)
+    static Shape slice_shape(Node const &n, Shape const &in)
+    {
+        DLPRIM_CHECK(n.dim >= 0 && n.dim < in.size());
+        const int end = n.slice_end == -1 ? int(in[n.dim]) : n.slice_end;
+        DLPRIM_CHECK(n.slice_begin >= 0 && n.slice_begin < end && end <= int(in[n.dim]));
+        Shape r = in;
+        r[n.dim] = size_t(end - n.slice_begin);
+        return r;
+    }
+    // Reshape / Squeeze (Shape::reshape and Shape::squeeze, src/shape.cpp:29-103)
+    static Shape view_shape(Node const &n, Shape const &in)
+    {
+        std::vector<size_t> d;
+        if (n.squeeze) {
+            std::vector<int> axes = n.view_dims;
+            if (axes.empty())
+                for (int i = 0; i < in.size(); i++)
+                    if (in[i] == 1)
+                        axes.push_back(i);
+            for (auto &a : axes) {
+                if (a < 0)
+                    a += in.size();
+                DLPRIM_CHECK(a >= 0 && a < in.size() && in[a] == 1);
+            }
+            for (int i = 0; i < in.size(); i++)
+                if (std::find(axes.begin(), axes.end(), i) == axes.end())
+                    d.push_back(in[i]);
+            if (d.empty())
+                d.push_back(1);
+        } else {
+            int deduced = -1;
+            size_t given = 1;
+            for (size_t i = 0; i < n.view_dims.size(); i++) {
+                const int v = n.view_dims[i];
+                if (v == -1) {
+                    if (deduced != -1)
+                        throw ValidationError("At most one index may be -1 in reshape");
+                    deduced = int(i);
+                    d.push_back(1);
+                } else if (v == 0) {
+                    if (int(i) >= in.size())
+                        throw ValidationError("0 reshape for index too large");
+                    d.push_back(in[int(i)]);
+                } else {
+                    DLPRIM_CHECK(v > 0);
+                    d.push_back(size_t(v));
+                }
+                given *= d.back();
+            }
+            if (deduced != -1) {
+                if (given == 0 || in.total_size() % given != 0)
+                    throw ValidationError("Can't computed deduced shape, original shape isn't multiple of provided");
+                d[size_t(deduced)] = in.total_size() / given;
+            }
+        }
+        Shape r = Shape::from_range(d.begin(), d.end());
+        if (r.total_size() != in.total_size())
+            throw ValidationError("Reshape changes the number of elements (" + n.name + ")");
+        return r;
+    }
 
     static Shape shape_of(std::vector<int> const &d)
     {
@@ -623,6 +723,33 @@ private:
                 DLPRIM_CHECK(in.size() == 2 || in.size() == 3); // as core::softmax_forward
                 n.log_softmax = o.type() == json::is_object ? o.get("log", false) : false;
                 specs_[n.outputs[0]] = in;
+            } else if (n.type == "Concat") {
+                n.kind = k_concat;
+                DLPRIM_CHECK(!n.inputs.empty() && n.outputs.size() == 1);
+                for (auto const &name : n.inputs)
+                    if (name == n.outputs[0])
+                        throw ValidationError("Concat in place (" + n.name + ")");
+                n.dim = o.type() == json::is_object ? o.get("dim", 1) : 1;
+                specs_[n.outputs[0]] = concat_shape(n);
+            } else if (n.type == "Slice") {
+                n.kind = k_slice;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
+                n.dim = o.get("dim", 1);
+                n.slice_begin = o.get("begin", 0);
+                n.slice_end = o.get("end", -1);
+                specs_[n.outputs[0]] = slice_shape(n, spec(n.inputs[0]));
+            } else if (n.type == "Reshape" || n.type == "Squeeze") { // views: no kernel, no memory
+                n.kind = k_view;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
+                n.squeeze = n.type == "Squeeze";
+                n.view_dims = o.type() == json::is_object ? int_list(o, "dims") : std::vector<int>();
+                if (n.squeeze) {
+                    if (o.type() == json::is_object && o.get("all", n.view_dims.empty()) && !n.view_dims.empty())
+                        throw ValidationError("Can't use both squeeze all and squeeze by dims");
+                } else if (n.view_dims.empty())
+                    throw ValidationError("Empty reshape dims");
+                specs_[n.outputs[0]] = view_shape(n, spec(n.inputs[0]));
+                alias_of_[n.outputs[0]] = n.inputs[0];
             } else if (n.type == "Flatten") { // a view: [B, everything else]; no kernel, no memory
                 n.kind = k_flatten;
                 DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
@@ -1074,7 +1201,37 @@ private:
                                                           x.device_ptr(), y.device_ptr(), e.stream()));
             break;
         }
-        case k_flatten: break; // the output is a view of the input
+        case k_flatten:
+        case k_view: break; // the output is a view of the input
+        case k_concat: { // every input goes to its range of the axis: [outer][axis][inner]
+            Shape const &ys = y.shape();
+            size_t outer = 1, inner = size_t(size_of_data_type(dtype_));
+            for (int j = 0; j < n.dim; j++)
+                outer *= ys[j];
+            for (int j = n.dim + 1; j < ys.size(); j++)
+                inner *= ys[j];
+            size_t offset = 0;
+            for (auto const &name : n.inputs) {
+                Tensor &xi = tensor(name);
+                const size_t slice = xi.shape()[n.dim];
+                details::check_status(dlp_copy2d_enqueue(static_cast<char *>(y.device_ptr()) + offset * inner, ys[n.dim] * inner, xi.device_ptr(), slice * inner,
+                                                         slice * inner, outer, e.stream()));
+                offset += slice;
+            }
+            break;
+        }
+        case k_slice: {
+            Shape const &xs = x.shape();
+            size_t outer = 1, inner = size_t(size_of_data_type(dtype_));
+            for (int j = 0; j < n.dim; j++)
+                outer *= xs[j];
+            for (int j = n.dim + 1; j < xs.size(); j++)
+                inner *= xs[j];
+            const size_t slice = y.shape()[n.dim];
+            details::check_status(dlp_copy2d_enqueue(y.device_ptr(), slice * inner, static_cast<const char *>(x.device_ptr()) + size_t(n.slice_begin) * inner,
+                                                     xs[n.dim] * inner, slice * inner, outer, e.stream()));
+            break;
+        }
         case k_eltwise: {
             Tensor &x1 = tensor(n.inputs[1]);
             details::check_status(dlp_eltwise_fwd_enqueue_dtype(int(dtype_), n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),

@@ -23,6 +23,17 @@ public:
         for (int i = 0; i < n_; i++)
             dims_[i] = v[i];
     }
+    // the dimensions [begin, end) (include/dlprim/shape.hpp:47-58 of the reference)
+    template <typename It>
+    static Shape from_range(It begin, It end)
+    {
+        Shape s;
+        for (It p = begin; p != end; ++p) {
+            DLPRIM_CHECK(s.n_ < max_tensor_dim);
+            s.dims_[s.n_++] = size_t(*p);
+        }
+        return s;
+    }
     int size() const { return n_; }
     size_t &operator[](int i) { return dims_[index(i)]; }
     size_t operator[](int i) const { return dims_[index(i)]; }

@@ -289,6 +289,12 @@ int dlp_pool2d_fwd_create_global_avg(int dtype, dlp_pool2d_fwd **out);
 int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y_shape[4], const void *x, void *y, void *stream);
 void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op);
 
+/* The copy behind Concat::forward and Slice::forward (core::SliceCopy::tensor_slice_copy with target_scale 0,
+ * include/dlprim/core/common.hpp:63-82; src/ops/concat.cpp:66-84,150-171): `rows` runs of `width_bytes` bytes, the r-th from
+ * src + r * src_pitch to dst + r * dst_pitch (pitches in bytes).  For a tensor split over axis `dim` into [outer][dim][inner]:
+ * rows = outer, width = slice * inner elements, pitch = the tensor's dim * inner elements, offsets folded into the pointers. */
+int dlp_copy2d_enqueue(void *dst, size_t dst_pitch, const void *src, size_t src_pitch, size_t width_bytes, size_t rows, void *stream);
+
 /* Elementwise::forward for two tensors of equal shape, src/ops/elementwise.cpp:517-559:
  * operation 0 sum: c = act(coef1*a + coef2*b); 1 prod: act(a*b*coef1*coef2); 2 max: act(max(coef1*a, coef2*b)) */
 #define DLP_ELTWISE_SUM 0

@@ -339,3 +339,33 @@ def test_gpu_softmax_inner_dimension_in_place(oracle_mod, dtype):
             dlp.softmax_forward(t, t, log)
             want = oracle_mod.softmax_forward(x, log)
             np.testing.assert_allclose(t.float().cpu().numpy(), want, rtol=2 ** -7 if dtype == "bfloat16" else 2e-5, atol=2 ** -7 if dtype == "bfloat16" else 1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "uint8"])
+def test_gpu_slice_copy(dtype):
+    """The copy behind Concat and Slice (core::SliceCopy::tensor_slice_copy with scale 0): ranges along every axis, rows that allow
+    16-, 4-, 2- and 1-byte units; what lies outside the range of the target stays as it was."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(4)
+
+    def rnd(shape):
+        t = torch.randint(0, 200, shape, generator=g)
+        return t.to(tdt).cuda()
+
+    for shape_s, shape_d, dim, so, do, ln in [((3, 8, 5, 4), (3, 20, 5, 4), 1, 0, 12, 8), ((3, 8, 5, 4), (3, 20, 5, 4), 1, 3, 1, 5), ((2, 3, 7), (2, 3, 11), 2, 2, 4, 5),
+                                              ((4, 6), (9, 6), 0, 1, 5, 3), ((2, 5, 3, 3), (2, 5, 3, 3), 1, 0, 0, 5), ((5, 1, 1), (5, 3, 1), 1, 0, 2, 1),
+                                              ((2, 16, 8, 8), (2, 48, 8, 8), 1, 0, 16, 16)]:
+        src, dst = rnd(shape_s), rnd(shape_d)
+        want = dst.clone()
+        want.narrow(dim, do, ln).copy_(src.narrow(dim, so, ln))
+        dlp.slice_copy(dst, do, src, so, ln, dim)
+        torch.cuda.synchronize()
+        assert torch.equal(dst, want), (shape_s, shape_d, dim, so, do, ln)
+    with pytest.raises(dlp.ValidationError):
+        dlp.slice_copy(rnd((2, 4)), 3, rnd((2, 4)), 0, 2, 1)
+

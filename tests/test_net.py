@@ -240,6 +240,15 @@ def torch_forward(doc, params, inputs, bf16=False):
             y = x.reshape(x.shape[0], -1)
         elif kind == "Softmax":
             y = torch.log_softmax(x, 1) if o.get("log", False) else torch.softmax(x, 1)
+        elif kind == "Concat":
+            y = torch.cat([t[n] for n in op["inputs"]], o.get("dim", 1))
+        elif kind == "Slice":
+            d, b0, e0 = o.get("dim", 1), o.get("begin", 0), o.get("end", -1)
+            y = x.narrow(d, b0, (x.shape[d] if e0 == -1 else e0) - b0)
+        elif kind == "Reshape":
+            y = x.reshape([x.shape[i] if d == 0 else d for i, d in enumerate(o["dims"])])
+        elif kind == "Squeeze":
+            y = x.squeeze() if "dims" not in o else x.reshape([d for i, d in enumerate(x.shape) if i not in [a % x.dim() for a in o["dims"]]])
         elif kind == "Elementwise":
             a, b = x * o.get("coef1", 1.0), t[op["inputs"][1]] * o.get("coef2", 1.0)
             y = {"sum": a + b, "prod": a * b, "max": torch.maximum(a, b)}[o.get("operation", "sum")]
@@ -316,8 +325,39 @@ def upsampling_net():
     return b
 
 
+def branching_net():
+    """Concat over channels (three inputs, one of them read by two operators), over the batch axis and over the last axis, Slice in the
+    middle and at the end of an axis, Reshape with 0 / -1, Squeeze by axes and of everything, a BatchNorm that folds into a convolution
+    whose output feeds a Concat, and an inner product behind a Reshape."""
+    b = netfile.NetBuilder("data", (2, 6, 14, 10))
+    a = b.conv("data", "a", 8, 3, 1, 1, bias=True, activation="relu")
+    c = b.conv("data", "c", 5, 1, 1, 0, bias=False)
+    c = b.bn(c, "cn", activation="relu")                      # folds; its output goes to the Concat
+    d = b.pool("data", "d", "max", 3, 1, 1)
+    cat = b.concat([a, c, d], "cat")                          # 8 + 5 + 6 = 19 channels
+    e = b.conv(cat, "e", 12, 3, 2, 1, bias=True, activation="relu")   # [2, 12, 7, 5]
+    lo = b.slice(e, "lo", 0, 4)                               # channels 0..3
+    hi = b.slice(e, "hi", 7, -1)                              # channels 7..11
+    mid = b.slice(cat, "mid", 3, 10, dim=2)                   # rows 3..9 of the 19-channel tensor
+    w = b.concat([lo, hi], "w")                               # 9 channels
+    w2 = b.concat([w, w], "w2", dim=3)                        # last axis: [2, 9, 7, 10]
+    both = b.concat([w2, w2], "both", dim=0)                  # batch axis: [4, 9, 7, 10]
+    r = b.reshape(both, "r", [0, -1])                         # [4, 630]
+    f = b.ip(r, "f", 11, activation="tanh")
+    g = b.global_pool(mid, "g", "avg")                        # [2, 19, 1, 1]
+    q = b.squeeze(g, "q", [2, -1])                            # [2, 19]
+    q3 = b.reshape(q, "q3", [1, 2, 19])
+    q4 = b.squeeze(q3, "q4")                                  # [2, 19]
+    b.softmax(q4, "sm")
+    b.output("f")
+    b.output("sm")
+    b.output("mid")
+    return b
+
+
 NETS = {
     "mixed": (mixed_net, 5),
+    "branching": (branching_net, 11),
     "upsampling": (upsampling_net, 9),
     "resnet18_b2_64": (lambda: netfile.resnet18(2, 64, 10), 6),
     "resnet50_b2_64": (lambda: netfile.resnet50(2, 64, 10), 8),
