@@ -543,7 +543,17 @@ def torch_dtype_code(t):
 
 
 def eltwise_forward(a, b, c, operation="sum", coef1=1.0, coef2=1.0, activation="identity", stream=None):
-    """Elementwise::forward for equal shapes: c = act(op(coef1*a, coef2*b))"""
+    """Elementwise::forward: c = act(op(coef1*a, coef2*b)); shapes that differ broadcast by numpy's rule (c has the broadcast shape)"""
+    if tuple(a.shape) != tuple(b.shape):
+        rank = max(a.dim(), b.dim())
+        sa = [1] * (rank - a.dim()) + [int(d) for d in a.shape]
+        sb = [1] * (rank - b.dim()) + [int(d) for d in b.shape]
+        arr = ctypes.c_int * rank
+        lib().dlp_eltwise_bcast_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_int,
+                                                        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        _check(lib().dlp_eltwise_bcast_fwd_enqueue(torch_dtype_code(a), ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation), rank,
+                                                   arr(*sa), arr(*sb), _ptr(a), _ptr(b), _ptr(c), _stream(stream)))
+        return
     lib().dlp_eltwise_fwd_enqueue_dtype.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_size_t,
                                                     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     _check(lib().dlp_eltwise_fwd_enqueue_dtype(torch_dtype_code(a), ELTWISE_OPS[operation], float(coef1), float(coef2), _act(activation),

@@ -295,6 +295,32 @@ __global__ __launch_bounds__(256) void eltwise_scalar_kernel(size_t n, int op, f
         store_plain(c + i, eltwise_one(to_float(a[i]), to_float(b[i]), op, c1, c2, act));
 }
 
+// Broadcasting operands: the output index is taken apart into at most four (collapsed) dimensions, whose strides in a and b are
+// 0 where that operand has extent 1.  The innermost dimension runs along consecutive threads.
+struct BcastArgs {
+    unsigned dims[4];          // output extents, dims[3] innermost; unused leading ones are 1
+    long long sa[4], sb[4];    // element strides of a and b
+};
+template <class T>
+__global__ __launch_bounds__(256) void eltwise_bcast_kernel(size_t n, BcastArgs g, int op, float c1, float c2, int act, const T *__restrict__ a,
+                                                            const T *__restrict__ b, T *__restrict__ c)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        size_t r = i;
+        long long oa = 0, ob = 0;
+#pragma unroll
+        for (int d = 3; d >= 0; d--) {
+            const size_t q = r / g.dims[d], k = r - q * g.dims[d];
+            oa += (long long)k * g.sa[d];
+            ob += (long long)k * g.sb[d];
+            r = q;
+        }
+        store_plain(c + i, eltwise_one(to_float(a[oa]), to_float(b[ob]), op, c1, c2, act));
+    }
+}
+
 } // namespace
 
 // y = act(x): 16 bytes per thread and step over the aligned body, the tail one by one.
@@ -724,3 +750,67 @@ static int eltwise_launch(int dtype, int operation, float coef1, float coef2, in
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
+
+int dlp_eltwise_bcast_fwd_enqueue(int dtype, int operation, float coef1, float coef2, int activation, int rank, const int *a_shape, const int *b_shape,
+                                  const void *a, const void *b, void *c, void *stream)
+{
+    if (dtype != DLP_FLOAT && dtype != DLP_BFLOAT16)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "elementwise: float_data and bfloat16_data are implemented");
+    DLP_REQUIRE(operation >= 0 && operation <= 2, "unknown elementwise operation");
+    DLP_REQUIRE(activation >= DLP_ACT_IDENTITY && activation <= DLP_ACT_RELU6, "unknown activation");
+    DLP_REQUIRE(rank >= 1 && rank <= 8 && a_shape != nullptr && b_shape != nullptr, "rank 1 to 8 and both shapes are needed");
+    // extents of the result; runs of dimensions in which both operands either follow the result or stay put collapse into one
+    unsigned dims[8];
+    long long sa[8], sb[8];
+    int nd = 0;
+    size_t total = 1;
+    long long stride_a = 1, stride_b = 1; // element strides of the operands, built from the innermost dimension outwards
+    int kind_prev = -1;
+    for (int j = rank - 1; j >= 0; j--) {
+        const int da = a_shape[j], db = b_shape[j];
+        DLP_REQUIRE(da >= 0 && db >= 0 && (da == db || da == 1 || db == 1), "the shapes do not broadcast");
+        const int dc = da == 1 ? db : da;
+        total *= (size_t)dc;
+        if (dc == 1)
+            continue; // both operands have extent 1: no index, no stride
+        const int kind = (da == dc ? 1 : 0) | (db == dc ? 2 : 0); // who moves along this dimension
+        if (kind == kind_prev) { // same pattern as the dimension inside it: one longer dimension (strides stay the inner one's)
+            dims[nd - 1] *= (unsigned)dc;
+        } else {
+            DLP_REQUIRE(nd < 8, "too many dimensions");
+            dims[nd] = (unsigned)dc;
+            sa[nd] = da == dc ? stride_a : 0;
+            sb[nd] = db == dc ? stride_b : 0;
+            nd++;
+            kind_prev = kind;
+        }
+        stride_a *= da;
+        stride_b *= db;
+    }
+    if (total == 0)
+        return DLP_OK;
+    DLP_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "null tensor pointer");
+    if (nd <= 1 && (nd == 0 || (sa[0] == 1 && sb[0] == 1)))
+        return eltwise_launch(dtype, operation, coef1, coef2, activation, total, a, b, c, stream);
+    if (nd > 4)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "elementwise: more than four runs of broadcast / plain dimensions");
+    BcastArgs g;
+    for (int d = 0; d < 4; d++) { // dims[] was filled innermost first; the kernel wants the innermost last
+        const int src = 3 - d;
+        g.dims[d] = src < nd ? dims[src] : 1u;
+        g.sa[d] = src < nd ? sa[src] : 0;
+        g.sb[d] = src < nd ? sb[src] : 0;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 256 * 32);
+    TimingScope ts("eltwise", st);
+    if (dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(eltwise_bcast_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, total, g, operation, coef1, coef2, activation, (const bf16_t *)a,
+                           (const bf16_t *)b, (bf16_t *)c);
+    else
+        hipLaunchKernelGGL(eltwise_bcast_kernel<float>, dim3(blocks), dim3(256), 0, st, total, g, operation, coef1, coef2, activation, (const float *)a,
+                           (const float *)b, (float *)c);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+

@@ -174,7 +174,7 @@ class NetBuilder:
         if activation:
             opts["activation"] = activation
         self._op("Add", "Elementwise", [a, b], [dst], opts)
-        self.shapes[dst] = self.shapes[a]
+        self.shapes[dst] = tuple(np.broadcast_shapes(self.shapes[a], self.shapes[b]))
         return dst
 
     def ip(self, src, dst, outputs, bias=True, activation=None, prefix=None):

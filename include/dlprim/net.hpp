@@ -224,9 +224,13 @@ public:
             case k_slice: out = slice_shape(n, in); break;
             case k_view: out = view_shape(n, in); break;
             case k_eltwise:
-                if (spec(n.inputs[1]) != in)
-                    throw ValidationError("Elementwise inputs of different shapes after reshape (" + n.name + ")");
-                out = in;
+                if (n.broadcast)
+                    out = broadcast_shape(in, spec(n.inputs[1]), n.name);
+                else {
+                    if (spec(n.inputs[1]) != in)
+                        throw ValidationError("Elementwise inputs of different shapes after reshape (" + n.name + ")");
+                    out = in;
+                }
                 break;
             default: out = in; break;
             }
@@ -441,6 +445,7 @@ private:
         // Elementwise
         int eltwise_op = DLP_ELTWISE_SUM;
         float coef[2] = {1.0f, 1.0f};
+        bool broadcast = false; // the inputs differ in shape
         // Softmax
         bool log_softmax = false;
         // Concat / Slice: the axis, and the range of a Slice (end -1: to the end of the axis)
@@ -450,6 +455,19 @@ private:
         std::vector<int> view_dims;
     };
 
+    // numpy's rule, as Elementwise::setup applies it (src/ops/elementwise.cpp:223): shapes aligned at their last dimension, extents equal or 1
+    static Shape broadcast_shape(Shape const &a, Shape const &b, std::string const &who)
+    {
+        const int rank = std::max(a.size(), b.size());
+        std::vector<size_t> d(size_t(rank), 1);
+        for (int j = 0; j < rank; j++) {
+            const size_t da = j < a.size() ? a[a.size() - 1 - j] : 1, db = j < b.size() ? b[b.size() - 1 - j] : 1;
+            if (da != db && da != 1 && db != 1)
+                throw ValidationError("Elementwise inputs do not broadcast (" + who + ")");
+            d[size_t(rank - 1 - j)] = da == 1 ? db : da;
+        }
+        return Shape::from_range(d.begin(), d.end());
+    }
     static std::vector<int> int_list(json::value const &o, char const *key)
     {
         std::vector<int> r;
@@ -702,8 +720,7 @@ private:
             } else if (n.type == "Elementwise") {
                 n.kind = k_eltwise;
                 DLPRIM_CHECK(n.inputs.size() == 2 && n.outputs.size() == 1);
-                if (spec(n.inputs[0]) != spec(n.inputs[1]))
-                    throw NotImplementedError("Elementwise with broadcasting (" + n.name + ")");
+                n.broadcast = spec(n.inputs[0]) != spec(n.inputs[1]);
                 std::string op = o.get("operation", "sum");
                 if (op == "sum")
                     n.eltwise_op = DLP_ELTWISE_SUM;
@@ -715,7 +732,7 @@ private:
                     throw ValidationError("Unsupported Elementwise operation " + op);
                 n.coef[0] = o.get("coef1", 1.0f);
                 n.coef[1] = o.get("coef2", 1.0f);
-                specs_[n.outputs[0]] = spec(n.inputs[0]);
+                specs_[n.outputs[0]] = n.broadcast ? broadcast_shape(spec(n.inputs[0]), spec(n.inputs[1]), n.name) : spec(n.inputs[0]);
             } else if (n.type == "Softmax") {
                 n.kind = k_softmax;
                 DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
@@ -850,7 +867,7 @@ private:
     int try_fuse_residual(size_t e)
     {
         Node &el = nodes_[e];
-        if (el.kind != k_eltwise || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || el.inputs[0] == el.inputs[1])
+        if (el.kind != k_eltwise || el.broadcast || el.eltwise_op != DLP_ELTWISE_SUM || keep_intermediate_ || el.inputs[0] == el.inputs[1])
             return -1;
         const int p0 = producer_before(e, el.inputs[0]), p1 = producer_before(e, el.inputs[1]);
         const int side = p0 > p1 ? 0 : 1; // the branch that is produced later
@@ -1234,6 +1251,18 @@ private:
         }
         case k_eltwise: {
             Tensor &x1 = tensor(n.inputs[1]);
+            if (n.broadcast) {
+                const int rank = y.shape().size();
+                int sa[max_tensor_dim], sb[max_tensor_dim];
+                for (int j = 0; j < rank; j++) {
+                    const int ja = j - (rank - x.shape().size()), jb = j - (rank - x1.shape().size());
+                    sa[j] = ja >= 0 ? int(x.shape()[ja]) : 1;
+                    sb[j] = jb >= 0 ? int(x1.shape()[jb]) : 1;
+                }
+                details::check_status(dlp_eltwise_bcast_fwd_enqueue(int(dtype_), n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), rank, sa, sb, x.device_ptr(),
+                                                                    x1.device_ptr(), y.device_ptr(), e.stream()));
+                break;
+            }
             details::check_status(dlp_eltwise_fwd_enqueue_dtype(int(dtype_), n.eltwise_op, n.coef[0], n.coef[1], int(n.activation), x.shape().total_size(), x.device_ptr(),
                                                           x1.device_ptr(), y.device_ptr(), e.stream()));
             break;

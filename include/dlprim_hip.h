@@ -305,6 +305,12 @@ int dlp_eltwise_fwd_enqueue(int operation, float coef1, float coef2, int activat
 /* same for tensors stored as `dtype` (DLP_FLOAT or DLP_BFLOAT16; arithmetic in fp32) */
 int dlp_eltwise_fwd_enqueue_dtype(int dtype, int operation, float coef1, float coef2, int activation, size_t n, const void *a,
                                   const void *b, void *c, void *stream);
+/* same with broadcasting (Elementwise::setup / forward, src/ops/elementwise.cpp:223,517-559; Shape broadcast rules of
+ * src/shape.cpp:105-160): a_shape and b_shape have `rank` (1 to 8) extents each, padded with leading ones by the caller; in every
+ * dimension the two extents are equal or one of them is 1; c has the larger extent of each dimension.  Runs of dimensions along which
+ * the same operands move are treated as one; more than four such runs are NotImplemented. */
+int dlp_eltwise_bcast_fwd_enqueue(int dtype, int operation, float coef1, float coef2, int activation, int rank, const int *a_shape,
+                                  const int *b_shape, const void *a, const void *b, void *c, void *stream);
 
 /* Activation::forward, src/ops/activation.cpp (cpu::apply_activation, include/dlprim/cpu/cpu_ops.hpp:17-53):
  * y = act(x) over n elements stored as `dtype`; x == y (in place) is allowed. */

@@ -369,3 +369,38 @@ def test_gpu_slice_copy(dtype):
     with pytest.raises(dlp.ValidationError):
         dlp.slice_copy(rnd((2, 4)), 3, rnd((2, 4)), 0, 2, 1)
 
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_eltwise_broadcast(dtype):
+    """Elementwise with inputs that broadcast (numpy's rule, src/ops/elementwise.cpp:223) against torch: per-channel and per-plane
+    operands, ranks that differ, both operands broadcasting, scalars; sum / prod / max with coefficients and an activation."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    tdt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(9)
+    shapes = [((3, 8, 5, 7), (3, 8, 1, 1)), ((3, 8, 5, 7), (1, 8, 1, 1)), ((8, 1, 1), (3, 8, 5, 7)), ((3, 1, 5, 1), (1, 8, 1, 7)), ((4, 6), (6,)),
+              ((2, 3, 4, 5), (1,)), ((2, 3, 4, 5), (4, 1)), ((5, 1), (1, 9)), ((2, 1, 3, 4), (2, 5, 3, 4)), ((2, 1, 3, 1), (1, 5, 3, 6))]
+    for k, (sa, sb) in enumerate(shapes):
+        a = torch.randn(sa, generator=g).to(tdt).cuda()
+        b = torch.randn(sb, generator=g).to(tdt).cuda()
+        op = ("sum", "prod", "max")[k % 3]
+        act = ("identity", "relu", "tanh")[(k // 3) % 3]
+        c1, c2 = 0.5 + 0.25 * k, -1.25 + 0.5 * k
+        out_shape = torch.broadcast_shapes(sa, sb)
+        c = torch.full(out_shape, float("nan"), dtype=tdt, device="cuda:0")
+        dlp.eltwise_forward(a, b, c, op, c1, c2, act)
+        torch.cuda.synchronize()
+        af, bf = a.float() * c1, b.float() * c2
+        want = {"sum": af + bf, "prod": af * bf, "max": torch.maximum(af, bf)}[op]
+        want = {"identity": lambda v: v, "relu": torch.relu, "tanh": torch.tanh}[act](want)
+        tol = dict(rtol=1e-5, atol=1e-6) if dtype == "float32" else dict(rtol=2 ** -7, atol=2 ** -7)
+        assert torch.allclose(c.float(), want.to(tdt).float() if dtype == "bfloat16" else want, **tol), (sa, sb, op, act)
+    a = torch.zeros((2, 3), device="cuda:0")
+    with pytest.raises(dlp.ValidationError):
+        dlp.eltwise_forward(a, torch.zeros((2, 4), device="cuda:0"), torch.zeros((2, 4), device="cuda:0"))
+    with pytest.raises(dlp.NotImplementedErrorDlprim):  # five runs of dimensions that alternate between the operands
+        dlp.eltwise_forward(torch.zeros((2, 1, 2, 1, 2), device="cuda:0"), torch.zeros((1, 2, 1, 2, 1), device="cuda:0"), torch.zeros((2, 2, 2, 2, 2), device="cuda:0"))
+

@@ -328,7 +328,7 @@ def upsampling_net():
 def branching_net():
     """Concat over channels (three inputs, one of them read by two operators), over the batch axis and over the last axis, Slice in the
     middle and at the end of an axis, Reshape with 0 / -1, Squeeze by axes and of everything, a BatchNorm that folds into a convolution
-    whose output feeds a Concat, and an inner product behind a Reshape."""
+    whose output feeds a Concat, an inner product behind a Reshape, and Elementwise operators whose inputs broadcast."""
     b = netfile.NetBuilder("data", (2, 6, 14, 10))
     a = b.conv("data", "a", 8, 3, 1, 1, bias=True, activation="relu")
     c = b.conv("data", "c", 5, 1, 1, 0, bias=False)
@@ -336,8 +336,13 @@ def branching_net():
     d = b.pool("data", "d", "max", 3, 1, 1)
     cat = b.concat([a, c, d], "cat")                          # 8 + 5 + 6 = 19 channels
     e = b.conv(cat, "e", 12, 3, 2, 1, bias=True, activation="relu")   # [2, 12, 7, 5]
-    lo = b.slice(e, "lo", 0, 4)                               # channels 0..3
-    hi = b.slice(e, "hi", 7, -1)                              # channels 7..11
+    gate = b.global_pool(e, "gate", "avg")                    # [2, 12, 1, 1]
+    gate = b.act(gate, "sigmoid", dst="gates")
+    se = b.eltwise(e, gate, "se", "prod")                     # broadcast over the plane (squeeze-and-excitation)
+    b.input("side", (12, 1, 5))                               # rank 3 against rank 4, extent 1 in the middle: four runs of dimensions
+    se = b.eltwise("side", se, "se2", "sum", coef1=0.5, activation="relu")
+    lo = b.slice(se, "lo", 0, 4)                              # channels 0..3
+    hi = b.slice(se, "hi", 7, -1)                             # channels 7..11
     mid = b.slice(cat, "mid", 3, 10, dim=2)                   # rows 3..9 of the 19-channel tensor
     w = b.concat([lo, hi], "w")                               # 9 channels
     w2 = b.concat([w, w], "w2", dim=3)                        # last axis: [2, 9, 7, 10]
