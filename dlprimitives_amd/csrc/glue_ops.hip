@@ -346,6 +346,38 @@ __global__ __launch_bounds__(256) void activation_kernel(size_t n, int act, cons
         store_plain(y + k, apply_act(to_float(x[k]), act));
 }
 
+// The parameterised pointwise operators (src/ops/pointwise.cpp:90-95,120-126,154-158): 0 Threshold y = x > p0 ? 1 : 0,
+// 1 Abs y = |x|, 2 Hardtanh y = max(p0, min(p1, x)).
+__device__ __forceinline__ float pointwise_one(float v, int op, float p0, float p1)
+{
+    switch (op) {
+    case 0: return v > p0 ? 1.0f : 0.0f;
+    case 1: return fabsf(v);
+    default: return fmaxf(p0, fminf(p1, v));
+    }
+}
+template <class T>
+__global__ __launch_bounds__(256) void pointwise_kernel(size_t n, int op, float p0, float p1, const T *__restrict__ x, T *__restrict__ y, int vec_ok)
+{
+    constexpr int VEC = 16 / (int)sizeof(T);
+    struct alignas(16) Pack {
+        T v[VEC];
+    };
+    const size_t n16 = vec_ok ? n / VEC : 0;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = i; k < n16; k += stride) {
+        const Pack px = ((const Pack *)x)[k];
+        Pack py;
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            store_plain(&py.v[e], pointwise_one(to_float(px.v[e]), op, p0, p1));
+        ((Pack *)y)[k] = py;
+    }
+    for (size_t k = n16 * VEC + i; k < n; k += stride)
+        store_plain(y + k, pointwise_one(to_float(x[k]), op, p0, p1));
+}
+
 // y[b][c][i] = act(x[b][c][i] * scale[c] + shift[c]): batch normalisation with fixed statistics.
 // VEC elements per thread and step; with VEC > 1 the host guarantees plane % VEC == 0 (a pack never
 // straddles two channels) and 16-byte aligned tensors.
@@ -639,6 +671,28 @@ int dlp_activation_fwd_enqueue(int dtype, int activation, size_t n, const void *
         hipLaunchKernelGGL(activation_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, n, activation, (const bf16_t *)x, (bf16_t *)y, vec_ok);
     else
         hipLaunchKernelGGL(activation_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, n, activation, (const float *)x, (float *)y, vec_ok);
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+int dlp_pointwise_fwd_enqueue(int dtype, int operation, float p0, float p1, size_t n, const void *x, void *y, void *stream)
+{
+    DLP_REQUIRE(dtype == DLP_FLOAT || dtype == DLP_BFLOAT16, "float_data and bfloat16_data are implemented");
+    DLP_REQUIRE(operation >= DLP_POINTWISE_THRESHOLD && operation <= DLP_POINTWISE_HARDTANH, "unknown pointwise operation");
+    if (n == 0)
+        return DLP_OK;
+    DLP_REQUIRE(x != nullptr && y != nullptr, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int vec_ok = (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
+    const size_t per_block = 256 * (16 / dtype_size(dtype));
+    size_t blocks = (n + per_block - 1) / per_block;
+    if (blocks > 65536)
+        blocks = 65536;
+    TimingScope ts("activation", st);
+    if (dtype == DLP_BFLOAT16)
+        hipLaunchKernelGGL(pointwise_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, n, operation, p0, p1, (const bf16_t *)x, (bf16_t *)y, vec_ok);
+    else
+        hipLaunchKernelGGL(pointwise_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, n, operation, p0, p1, (const float *)x, (float *)y, vec_ok);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }

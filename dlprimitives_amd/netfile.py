@@ -198,6 +198,12 @@ class NetBuilder:
         self.shapes[dst] = (s[0], int(np.prod(s[1:])))
         return dst
 
+    def pointwise(self, src, dst, kind, **options):
+        """Threshold (threshold=), Abs, Hardtanh (min_val=, max_val=)"""
+        self._op(kind, kind, [src], [dst], dict(options))
+        self.shapes[dst] = self.shapes[src]
+        return dst
+
     def concat(self, srcs, dst, dim=1):
         shapes = [self.shapes[s] for s in srcs]
         self._op("Concat", "Concat", list(srcs), [dst], {"dim": dim})

@@ -8,7 +8,7 @@
 // liveness (src/net.cpp:585-654: intermediate tensors share chunks unless keep_intermediate_tensors),
 // and runs the operators in order on one ExecutionContext with one shared workspace
 // (src/net.cpp:836-851).  Operator types: Convolution2D, BatchNorm, Activation, Pooling2D,
-// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- plus Softmax, Flatten, Concat, Slice, Reshape, Squeeze and
+// GlobalPooling, Elementwise, InnerProduct -- what docs/nets_for_benchmark/*.js use -- plus Softmax, Flatten, Concat, Slice, Reshape, Squeeze, Threshold, Abs, Hardtanh and
 // TransposedConvolution2D, with the option names of the reference's *Config::from_json functions.
 //
 // In predict mode two graph rewrites are applied at setup (fuse(true), the default):
@@ -408,7 +408,7 @@ public:
     }
 
 private:
-    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv, k_concat, k_slice, k_view };
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv, k_concat, k_slice, k_view, k_pointwise };
     struct Node {
         std::string name, type;
         std::vector<std::string> inputs, outputs, param_names;
@@ -453,6 +453,9 @@ private:
         // Reshape (view_dims as given: 0 keeps the input's dimension, -1 is deduced) / Squeeze (view_dims: the axes; empty: all of extent 1)
         bool squeeze = false;
         std::vector<int> view_dims;
+        // Threshold / Abs / Hardtanh
+        int pointwise_op = 0;
+        float pointwise_p[2] = {0.0f, 0.0f};
     };
 
     // numpy's rule, as Elementwise::setup applies it (src/ops/elementwise.cpp:223): shapes aligned at their last dimension, extents equal or 1
@@ -740,6 +743,21 @@ private:
                 DLPRIM_CHECK(in.size() == 2 || in.size() == 3); // as core::softmax_forward
                 n.log_softmax = o.type() == json::is_object ? o.get("log", false) : false;
                 specs_[n.outputs[0]] = in;
+            } else if (n.type == "Threshold" || n.type == "Abs" || n.type == "Hardtanh") {
+                n.kind = k_pointwise;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1);
+                const bool has = o.type() == json::is_object;
+                if (n.type == "Threshold") {
+                    n.pointwise_op = DLP_POINTWISE_THRESHOLD;
+                    n.pointwise_p[0] = has ? o.get("threshold", 0.0f) : 0.0f;
+                } else if (n.type == "Abs")
+                    n.pointwise_op = DLP_POINTWISE_ABS;
+                else {
+                    n.pointwise_op = DLP_POINTWISE_HARDTANH;
+                    n.pointwise_p[0] = has ? o.get("min_val", -1.0f) : -1.0f;
+                    n.pointwise_p[1] = has ? o.get("max_val", 1.0f) : 1.0f;
+                }
+                specs_[n.outputs[0]] = spec(n.inputs[0]);
             } else if (n.type == "Concat") {
                 n.kind = k_concat;
                 DLPRIM_CHECK(!n.inputs.empty() && n.outputs.size() == 1);
@@ -1218,6 +1236,10 @@ private:
                                                           x.device_ptr(), y.device_ptr(), e.stream()));
             break;
         }
+        case k_pointwise:
+            details::check_status(dlp_pointwise_fwd_enqueue(int(dtype_), n.pointwise_op, n.pointwise_p[0], n.pointwise_p[1], x.shape().total_size(), x.device_ptr(),
+                                                            y.device_ptr(), e.stream()));
+            break;
         case k_flatten:
         case k_view: break; // the output is a view of the input
         case k_concat: { // every input goes to its range of the axis: [outer][axis][inner]

@@ -315,6 +315,12 @@ int dlp_eltwise_bcast_fwd_enqueue(int dtype, int operation, float coef1, float c
 /* Activation::forward, src/ops/activation.cpp (cpu::apply_activation, include/dlprim/cpu/cpu_ops.hpp:17-53):
  * y = act(x) over n elements stored as `dtype`; x == y (in place) is allowed. */
 int dlp_activation_fwd_enqueue(int dtype, int activation, size_t n, const void *x, void *y, void *stream);
+/* Threshold / Abs / Hardtanh::forward (src/ops/pointwise.cpp:84-95,113-126,154-158; defaults threshold 0, min_val -1, max_val 1 in
+ * include/dlprim/ops/pointwise.hpp:50,71-72): y = x > p0 ? 1 : 0 | y = |x| | y = max(p0, min(p1, x)); y may be x */
+#define DLP_POINTWISE_THRESHOLD 0
+#define DLP_POINTWISE_ABS 1
+#define DLP_POINTWISE_HARDTANH 2
+int dlp_pointwise_fwd_enqueue(int dtype, int operation, float p0, float p1, size_t n, const void *x, void *y, void *stream);
 
 /* BatchNorm::forward with fixed statistics (predict mode / use_global_stats), src/ops/batch_normalization.cpp:161-232:
  * y[b][c][i] = act(x[b][c][i] * scale[c] + shift[c]) with scale = gamma / sqrt(var + eps), shift = beta - mean * scale

@@ -240,6 +240,12 @@ def torch_forward(doc, params, inputs, bf16=False):
             y = x.reshape(x.shape[0], -1)
         elif kind == "Softmax":
             y = torch.log_softmax(x, 1) if o.get("log", False) else torch.softmax(x, 1)
+        elif kind == "Threshold":
+            y = (x > o.get("threshold", 0.0)).to(x.dtype)
+        elif kind == "Abs":
+            y = x.abs()
+        elif kind == "Hardtanh":
+            y = torch.clamp(x, o.get("min_val", -1.0), o.get("max_val", 1.0))
         elif kind == "Concat":
             y = torch.cat([t[n] for n in op["inputs"]], o.get("dim", 1))
         elif kind == "Slice":
@@ -328,12 +334,15 @@ def upsampling_net():
 def branching_net():
     """Concat over channels (three inputs, one of them read by two operators), over the batch axis and over the last axis, Slice in the
     middle and at the end of an axis, Reshape with 0 / -1, Squeeze by axes and of everything, a BatchNorm that folds into a convolution
-    whose output feeds a Concat, an inner product behind a Reshape, and Elementwise operators whose inputs broadcast."""
+    whose output feeds a Concat, an inner product behind a Reshape, Elementwise operators whose inputs broadcast, Hardtanh, Abs (in place) and Threshold."""
     b = netfile.NetBuilder("data", (2, 6, 14, 10))
     a = b.conv("data", "a", 8, 3, 1, 1, bias=True, activation="relu")
     c = b.conv("data", "c", 5, 1, 1, 0, bias=False)
     c = b.bn(c, "cn", activation="relu")                      # folds; its output goes to the Concat
     d = b.pool("data", "d", "max", 3, 1, 1)
+    d = b.pointwise(d, "dh", "Hardtanh", min_val=-0.25, max_val=0.5)
+    d = b.pointwise(d, "dh", "Abs")                           # in place
+    c = b.pointwise(c, "ch", "Hardtanh")                      # default range
     cat = b.concat([a, c, d], "cat")                          # 8 + 5 + 6 = 19 channels
     e = b.conv(cat, "e", 12, 3, 2, 1, bias=True, activation="relu")   # [2, 12, 7, 5]
     gate = b.global_pool(e, "gate", "avg")                    # [2, 12, 1, 1]
@@ -354,6 +363,8 @@ def branching_net():
     q3 = b.reshape(q, "q3", [1, 2, 19])
     q4 = b.squeeze(q3, "q4")                                  # [2, 19]
     b.softmax(q4, "sm")
+    b.pointwise(q, "big", "Threshold", threshold=0.05)        # 0 / 1
+    b.output("big")
     b.output("f")
     b.output("sm")
     b.output("mid")
