@@ -27,9 +27,15 @@ from .capi import (  # noqa: F401
     conv2d_output_shape,
     conv2d_transposed_output_shape,
     eltwise_forward,
+    interpolate2d_forward,
+    mse_loss_forward,
+    nll_loss_forward,
+    reduction_forward,
     slice_copy,
+    softmax_loss_forward,
     lib,
     library_path,
+    pointwise_forward,
     pool2d_output_size,
     softmax_forward,
     timing_count,

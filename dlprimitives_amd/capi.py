@@ -609,3 +609,120 @@ def softmax_forward(x, y, log=False, stream=None):
                                               ctypes.c_void_p]
     _check(lib().dlp_softmax_fwd_enqueue(torch_dtype_code(x), int(bool(log)), int(x.shape[0]), int(x.shape[1]), inner, _ptr(x), _ptr(y),
                                          _stream(stream)))
+
+
+INTERPOLATE_METHODS = {"nearest": 0, "nearest-exact": 1, "bilinear": 2}
+REDUCE_METHODS = {"sum": 0, "sumsq": 1, "abssum": 2, "mean": 3}
+LOSS_REDUCE = {"none": 0, "sum": 1, "mean": 2}
+INT32_DATA = 19
+
+
+def interpolate2d_forward(x, y, method="nearest", scale_y=-1.0, scale_x=-1.0, align_corners=False, stream=None):
+    """core::interpolate2d: x [B, C, H, W] -> y [B, C, OH, OW]; without scales the steps follow from the two sizes"""
+    if x.dim() != 4 or y.dim() != 4 or tuple(x.shape[:2]) != tuple(y.shape[:2]):
+        raise ValidationError("interpolate2d: two 4-d tensors with the same batch and channels")
+    lib().dlp_interpolate2d_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_double] + [ctypes.c_int] * 5 + [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    if method not in INTERPOLATE_METHODS:
+        raise ValidationError("Unsupported interpolation method " + str(method))
+    _check(lib().dlp_interpolate2d_fwd_enqueue(torch_dtype_code(x), INTERPOLATE_METHODS[method], int(bool(align_corners)), float(scale_y), float(scale_x),
+                                               int(x.shape[0] * x.shape[1]), int(x.shape[2]), int(x.shape[3]), int(y.shape[2]), int(y.shape[3]),
+                                               _ptr(x), _ptr(y), _stream(stream)))
+
+
+def _label_code(labels):
+    import torch
+
+    if labels.dtype == torch.float32:
+        return FLOAT_DATA
+    if labels.dtype == torch.int32:
+        return INT32_DATA
+    raise NotImplementedErrorDlprim("labels must be either int or float")
+
+
+def _workspace(nbytes, like):
+    import torch
+
+    return torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=like.device)
+
+
+def reduction_forward(x, y, method="sum", dims=None, start_axis=0, output_scale=1.0, stream=None):
+    """Reduction::forward: y = sum / sumsq / abssum / mean of x over `dims` (or over every axis from `start_axis` on); y holds the kept
+    elements in order, with or without the reduced axes as extents of 1"""
+    rank = x.dim()
+    if dims is None:
+        if start_axis < 0:
+            start_axis += rank
+        if not 0 <= start_axis < rank:
+            raise ValidationError("reduction: start_axis outside the tensor")
+        dims = range(start_axis, rank)
+    mask = [0] * rank
+    for d in dims:
+        if d < 0:
+            d += rank
+        if not 0 <= d < rank:
+            raise ValidationError("reduction: axis outside the tensor")
+        mask[d] = 1
+    arr = ctypes.c_int * rank
+    shape = arr(*[int(d) for d in x.shape])
+    red = arr(*mask)
+    code = torch_dtype_code(x)
+    need = ctypes.c_size_t(0)
+    L = lib()
+    L.dlp_reduce_fwd_workspace.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]
+    _check(L.dlp_reduce_fwd_workspace(code, REDUCE_METHODS[method], rank, shape, red, ctypes.byref(need)))
+    ws = _workspace(need.value, x)
+    L.dlp_reduce_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    _check(L.dlp_reduce_fwd_enqueue(code, REDUCE_METHODS[method], float(output_scale), rank, shape, red, _ptr(x), _ptr(y), _ptr(ws), ws.numel(),
+                                    _stream(stream)))
+    return need.value
+
+
+def mse_loss_forward(a, b, y, reduce="mean", stream=None):
+    """MSELoss::forward: y = (a - b)^2 elementwise, or the sum / mean of that in y[0]"""
+    if tuple(a.shape) != tuple(b.shape):
+        raise ValidationError("MSE loss: the inputs differ in shape")
+    code = torch_dtype_code(a)
+    need = ctypes.c_size_t(0)
+    L = lib()
+    L.dlp_mse_loss_fwd_workspace.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]
+    _check(L.dlp_mse_loss_fwd_workspace(code, LOSS_REDUCE[reduce], a.numel(), ctypes.byref(need)))
+    ws = _workspace(need.value, a)
+    L.dlp_mse_loss_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_size_t, ctypes.c_void_p]
+    _check(L.dlp_mse_loss_fwd_enqueue(code, LOSS_REDUCE[reduce], a.numel(), _ptr(a), _ptr(b), _ptr(y), _ptr(ws), ws.numel(), _stream(stream)))
+
+
+def nll_loss_forward(x, labels, y, reduce="mean", stream=None):
+    """NLLLoss::forward: x [B, C] (log-probabilities), labels [B] float32 or int32; y [B] for reduce 'none', else y [1]"""
+    if x.dim() != 2 or labels.numel() != x.shape[0]:
+        raise ValidationError("NLL loss: x [batch, classes] and one label per row")
+    lib().dlp_nll_loss_fwd_enqueue.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p] * 4
+    _check(lib().dlp_nll_loss_fwd_enqueue(torch_dtype_code(x), _label_code(labels), LOSS_REDUCE[reduce], int(x.shape[0]), int(x.shape[1]), _ptr(x),
+                                          _ptr(labels), _ptr(y), _stream(stream)))
+
+
+def softmax_loss_forward(x, labels, y, stream=None):
+    """SoftmaxWithLoss::forward: y[0] = mean cross entropy of the rows of x [B, C] against labels [B] (float32 or int32)"""
+    if x.dim() != 2 or labels.numel() != x.shape[0]:
+        raise ValidationError("softmax loss: x [batch, classes] and one label per row")
+    need = ctypes.c_size_t(0)
+    L = lib()
+    L.dlp_softmax_loss_fwd_workspace.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_size_t)]
+    _check(L.dlp_softmax_loss_fwd_workspace(int(x.shape[0]), ctypes.byref(need)))
+    ws = _workspace(need.value, x)
+    L.dlp_softmax_loss_fwd_enqueue.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 4 + [ctypes.c_size_t, ctypes.c_void_p]
+    _check(L.dlp_softmax_loss_fwd_enqueue(torch_dtype_code(x), _label_code(labels), int(x.shape[0]), int(x.shape[1]), _ptr(x), _ptr(labels), _ptr(y),
+                                          _ptr(ws), ws.numel(), _stream(stream)))
+
+
+POINTWISE_OPS = {"threshold": 0, "abs": 1, "hardtanh": 2}
+
+
+def pointwise_forward(x, y, operation, p0=0.0, p1=0.0, stream=None):
+    """Threshold / Abs / Hardtanh::forward: y = x > p0 | |x| | clamp(x, p0, p1); y may be x"""
+    lib().dlp_pointwise_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_size_t, ctypes.c_void_p,
+                                                ctypes.c_void_p, ctypes.c_void_p]
+    _check(lib().dlp_pointwise_fwd_enqueue(torch_dtype_code(x), POINTWISE_OPS[operation], float(p0), float(p1), x.numel(), _ptr(x), _ptr(y),
+                                           _stream(stream)))

@@ -74,8 +74,12 @@ class NetBuilder:
         self.doc["operators"].append(op)
         return name
 
-    def input(self, name, shape):
-        self.doc["inputs"].append({"name": name, "shape": list(shape)})
+    def input(self, name, shape, dtype=None):
+        """another input; dtype "int" for the labels of a loss (default: float)"""
+        spec = {"name": name, "shape": list(shape)}
+        if dtype is not None:
+            spec["dtype"] = dtype
+        self.doc["inputs"].append(spec)
         self.shapes[name] = tuple(shape)
         return name
 
@@ -242,6 +246,61 @@ class NetBuilder:
         self.shapes[dst] = self.shapes[src]
         return dst
 
+    def interpolation(self, src, dst, method="nearest", out_hw=None, scale=None, align_corners=False):
+        """Interpolation to a size (out_hw) or by factors (scale = (scale_y, scale_x)): nearest, nearest-exact or bilinear"""
+        n, c, h, w = self.shapes[src]
+        opts = {"method": method, "align_corners": bool(align_corners)}
+        if out_hw is not None:
+            opts.update(out_h=int(out_hw[0]), out_w=int(out_hw[1]))
+            hw = (int(out_hw[0]), int(out_hw[1]))
+        else:
+            opts.update(scale_y=scale[0], scale_x=scale[1])
+            hw = (int(h * scale[0]), int(w * scale[1]))
+        self._op("Interpolation", "Interpolation", [src], [dst], opts)
+        self.shapes[dst] = (n, c) + hw
+        return dst
+
+    def reduction(self, src, dst, method="sum", dims=None, start_axis=None, keep_dim=True, output_scale=None):
+        """Reduction over `dims`, or over every axis from `start_axis` (default 0) on"""
+        s = self.shapes[src]
+        opts = {"method": method, "keep_dim": bool(keep_dim)}
+        if dims is not None:
+            opts["dims"] = list(dims)
+            axes = {d % len(s) for d in dims}
+        else:
+            if start_axis is not None:
+                opts["start_axis"] = start_axis
+            axes = set(range((start_axis or 0) % len(s), len(s)))
+        if output_scale is not None:
+            opts["output_scale"] = output_scale
+        self._op("Reduction", "Reduction", [src], [dst], opts)
+        out = [1 if i in axes else d for i, d in enumerate(s) if keep_dim or i not in axes]
+        self.shapes[dst] = tuple(out) or (1,)
+        return dst
+
+    def parameter(self, dst, shape, pname=None):
+        """Parameter: a tensor whose values are a parameter of the network"""
+        pname = pname or dst + ".value"
+        self._op("Parameter", "Parameter", [], [dst], {"shape": list(shape), "dtype": "float"}, [pname])
+        self.param_shapes[pname] = tuple(shape)
+        self.shapes[dst] = tuple(shape)
+        return dst
+
+    def mse_loss(self, a, b, dst, reduce="mean"):
+        self._op("MSELoss", "MSELoss", [a, b], [dst], {"reduce": reduce})
+        self.shapes[dst] = self.shapes[a] if reduce == "none" else (1,)
+        return dst
+
+    def nll_loss(self, src, labels, dst, reduce="mean"):
+        self._op("NLLLoss", "NLLLoss", [src, labels], [dst], {"reduce": reduce})
+        self.shapes[dst] = (self.shapes[src][0],) if reduce == "none" else (1,)
+        return dst
+
+    def softmax_loss(self, src, labels, dst):
+        self._op("SoftmaxWithLoss", "SoftmaxWithLoss", [src, labels], [dst], {})
+        self.shapes[dst] = (1,)
+        return dst
+
     def output(self, name):
         self.doc["outputs"].append(name)
 
@@ -257,6 +316,8 @@ class NetBuilder:
                 t = rng.uniform(-0.3, 0.3, shape)
             elif len(shape) == 1 and name.endswith(".weight"):
                 t = rng.uniform(0.5, 1.5, shape)
+            elif name.endswith(".value"):  # a Parameter operator's tensor
+                t = rng.uniform(-1.0, 1.0, shape)
             elif len(shape) == 1:
                 t = rng.uniform(-0.2, 0.2, shape)
             else:

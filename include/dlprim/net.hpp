@@ -60,17 +60,20 @@ public:
     {
         for (auto const &in : v["inputs"].array()) {
             std::string dt = in.get("dtype", "float");
-            if (dt != "float")
+            DataType input_type = float_data; // float: stored as the network's storage type
+            if (dt == "int" || dt == "int32")
+                input_type = int32_data; // class labels of a loss
+            else if (dt != "float" && dt != "float32")
                 throw NotImplementedError("input dtype " + dt);
             std::vector<int> dims = in.get<std::vector<int>>("shape");
-            add_input_tensor(in.get<std::string>("name"), shape_of(dims));
+            add_input_tensor(in.get("name", "data"), shape_of(dims), input_type);
         }
         for (auto const &op : v["operators"].array()) {
             Node n;
             n.name = op.get<std::string>("name");
             n.type = op.get<std::string>("type");
-            n.inputs = op.get<std::vector<std::string>>("inputs");
-            n.outputs = op.get<std::vector<std::string>>("outputs");
+            n.inputs = op.get("inputs", std::vector<std::string>());
+            n.outputs = op.get("outputs", std::vector<std::string>());
             if (!op.find("params").is_undefined())
                 n.param_names = op.get<std::vector<std::string>>("params");
             n.options = op.find("options");
@@ -79,10 +82,15 @@ public:
         for (auto const &out : v["outputs"].array())
             mark_output_tensor(out.type() == json::is_string ? out.str() : out.get<std::string>("name"));
     }
-    void add_input_tensor(std::string const &name, Shape const &s)
+    // float_data: an input in the network's storage type; int32_data: labels of a loss operator
+    void add_input_tensor(std::string const &name, Shape const &s, DataType dt = float_data)
     {
+        if (dt != float_data && dt != int32_data)
+            throw NotImplementedError("input tensors are float or int32");
         input_names_.push_back(name);
         specs_[name] = s;
+        if (dt == int32_data)
+            int_inputs_.insert(name);
     }
     void mark_output_tensor(std::string const &name) { output_names_.push_back(name); }
 
@@ -114,7 +122,10 @@ public:
     {
         Tensor &t = input(id);
         const size_t n = t.shape().total_size();
-        if (dtype_ == float_data)
+        if (t.dtype() == int32_data)
+            for (size_t i = 0; i < n; i++)
+                t.data<int32_t>()[i] = int32_t(values[i]);
+        else if (dtype_ == float_data)
             std::copy(values, values + n, t.data<float>());
         else
             for (size_t i = 0; i < n; i++)
@@ -174,9 +185,24 @@ public:
         for (auto &n : nodes_) {
             if (n.skipped)
                 continue;
-            Shape const in = spec(n.inputs[0]);
+            Shape const in = n.inputs.empty() ? spec(n.outputs[0]) : spec(n.inputs[0]);
             Shape out;
             switch (n.kind) {
+            case k_interp: out = interpolation_shape(n, in); break;
+            case k_reduce: out = reduction_shape(n, in); break;
+            case k_mse_loss:
+                if (spec(n.inputs[1]) != in)
+                    throw ValidationError("MSELoss inputs of different shapes after reshape (" + n.name + ")");
+                out = n.loss_reduce == DLP_LOSS_REDUCE_NONE ? in : Shape(size_t(1));
+                break;
+            case k_nll_loss:
+                check_labels(n);
+                out = Shape(n.loss_reduce == DLP_LOSS_REDUCE_NONE ? in[0] : size_t(1));
+                break;
+            case k_softmax_loss:
+                check_labels(n);
+                out = Shape(size_t(1));
+                break;
             case k_conv: {
                 DLPRIM_CHECK(in.size() == 4 && int(in[1]) == n.conv.channels_in);
                 if (n.dw_node >= 0) { // `in` is the input of the depthwise convolution that this node runs as well
@@ -236,6 +262,11 @@ public:
             }
             specs_[n.outputs[0]] = out;
             tensors_.at(n.outputs[0]).reshape(out);
+            if (!ctx_.is_cpu_context()) {
+                workspace_bytes_ = std::max(workspace_bytes_, node_workspace(n));
+                if (workspace_bytes_ > workspace_.memory_size())
+                    workspace_ = Tensor(ctx_, Shape(workspace_bytes_), uint8_data);
+            }
         }
         if (!ctx_.is_cpu_context())
             e.finish();
@@ -408,7 +439,7 @@ public:
     }
 
 private:
-    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv, k_concat, k_slice, k_view, k_pointwise };
+    enum Kind { k_conv, k_bn, k_act, k_pool, k_gpool, k_eltwise, k_ip, k_softmax, k_flatten, k_tconv, k_concat, k_slice, k_view, k_pointwise, k_interp, k_reduce, k_param, k_mse_loss, k_nll_loss, k_softmax_loss };
     struct Node {
         std::string name, type;
         std::vector<std::string> inputs, outputs, param_names;
@@ -456,6 +487,17 @@ private:
         // Threshold / Abs / Hardtanh
         int pointwise_op = 0;
         float pointwise_p[2] = {0.0f, 0.0f};
+        // Interpolation: the method, the size (<= 0: from the scale) and the scale (<= 0: from the size)
+        int interp_method = DLP_INTERPOLATE_NEAREST, out_hw[2] = {-1, -1};
+        double scale_yx[2] = {-1.0, -1.0};
+        bool align_corners = false;
+        // Reduction: the method, the axes as given (negative: from the end) or the first reduced axis, and whether reduced axes stay as 1
+        int reduce_method = DLP_REDUCE_SUM, start_axis = 0;
+        float output_scale = 1.0f;
+        bool keep_dim = true, has_dims = false;
+        std::vector<int> reduce_dims;
+        // MSELoss / NLLLoss: none, sum, mean
+        int loss_reduce = DLP_LOSS_REDUCE_MEAN;
     };
 
     // numpy's rule, as Elementwise::setup applies it (src/ops/elementwise.cpp:223): shapes aligned at their last dimension, extents equal or 1
@@ -561,6 +603,88 @@ private:
         if (r.total_size() != in.total_size())
             throw ValidationError("Reshape changes the number of elements (" + n.name + ")");
         return r;
+    }
+
+    // Interpolation::calc_size (src/ops/interpolation.cpp:53-69)
+    static Shape interpolation_shape(Node const &n, Shape const &in)
+    {
+        DLPRIM_CHECK(in.size() == 4);
+        Shape r = in;
+        if (n.out_hw[0] > 0) {
+            r[2] = size_t(n.out_hw[0]);
+            r[3] = size_t(n.out_hw[1]);
+        } else {
+            r[2] = size_t(int(in[2] * n.scale_yx[0]));
+            r[3] = size_t(int(in[3] * n.scale_yx[1]));
+        }
+        DLPRIM_CHECK(r[2] > 0 && r[3] > 0);
+        return r;
+    }
+    // Reduction::setup / calc_shapes (src/ops/reduction.cpp:49-69,133-151): which axes go, and the shape that is left
+    static std::vector<int> reduced_axes(Node const &n, Shape const &in)
+    {
+        std::vector<int> mask(size_t(in.size()), 0);
+        if (!n.has_dims) {
+            int first = n.start_axis < 0 ? n.start_axis + in.size() : n.start_axis;
+            DLPRIM_CHECK(first >= 0 && first < in.size());
+            for (int a = first; a < in.size(); a++)
+                mask[size_t(a)] = 1;
+        } else
+            for (int a : n.reduce_dims) {
+                if (a < 0)
+                    a += in.size();
+                DLPRIM_CHECK(a >= 0 && a < in.size());
+                mask[size_t(a)] = 1;
+            }
+        return mask;
+    }
+    static Shape reduction_shape(Node const &n, Shape const &in)
+    {
+        std::vector<int> mask = reduced_axes(n, in);
+        std::vector<size_t> d;
+        for (int a = 0; a < in.size(); a++) {
+            if (!mask[size_t(a)])
+                d.push_back(in[a]);
+            else if (n.keep_dim)
+                d.push_back(1);
+        }
+        if (d.empty())
+            d.push_back(1);
+        return Shape::from_range(d.begin(), d.end());
+    }
+    static int loss_reduce_option(json::value const &o)
+    {
+        std::string r = o.type() == json::is_object ? o.get("reduce", "mean") : "mean";
+        if (r == "none")
+            return DLP_LOSS_REDUCE_NONE;
+        if (r == "sum")
+            return DLP_LOSS_REDUCE_SUM;
+        if (r != "mean")
+            throw ValidationError("Unknown loss reduction " + r);
+        return DLP_LOSS_REDUCE_MEAN;
+    }
+    // device memory an operator needs beside its tensors, at the current shapes
+    size_t node_workspace(Node const &n) const
+    {
+        size_t bytes = 0;
+        if (n.kind == k_reduce) {
+            Shape const &in = spec(n.inputs[0]);
+            std::vector<int> mask = reduced_axes(n, in), dims(size_t(in.size()));
+            for (int a = 0; a < in.size(); a++)
+                dims[size_t(a)] = int(in[a]);
+            details::check_status(dlp_reduce_fwd_workspace(int(dtype_), n.reduce_method, in.size(), dims.data(), mask.data(), &bytes));
+        } else if (n.kind == k_mse_loss)
+            details::check_status(dlp_mse_loss_fwd_workspace(int(dtype_), n.loss_reduce, spec(n.inputs[0]).total_size(), &bytes));
+        else if (n.kind == k_softmax_loss)
+            details::check_status(dlp_softmax_loss_fwd_workspace(int(spec(n.inputs[0])[0]), &bytes));
+        return bytes;
+    }
+    void check_labels(Node const &n) const
+    {
+        Shape const &x = spec(n.inputs[0]), &lbl = spec(n.inputs[1]);
+        DLPRIM_CHECK(x.size() == 2 && lbl.total_size() == x[0] && lbl[0] == x[0]);
+        if (dtype_ != float_data && !int_inputs_.count(n.inputs[1]))
+            throw NotImplementedError("labels stored as bfloat16 (" + n.name + "): give the label input the dtype int");
     }
 
     static Shape shape_of(std::vector<int> const &d)
@@ -785,6 +909,82 @@ private:
                     throw ValidationError("Empty reshape dims");
                 specs_[n.outputs[0]] = view_shape(n, spec(n.inputs[0]));
                 alias_of_[n.outputs[0]] = n.inputs[0];
+            } else if (n.type == "Interpolation") { // InterpolationConfig::from_json and the constructor's checks, src/ops/interpolation.cpp:18-46
+                n.kind = k_interp;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
+                n.out_hw[0] = o.get("out_h", -1);
+                n.out_hw[1] = o.get("out_w", -1);
+                n.scale_yx[0] = o.get("scale_y", -1.0);
+                n.scale_yx[1] = o.get("scale_x", -1.0);
+                n.align_corners = o.get("align_corners", false);
+                std::string method = o.get<std::string>("method");
+                if (method == "nearest")
+                    n.interp_method = DLP_INTERPOLATE_NEAREST;
+                else if (method == "nearest-exact")
+                    n.interp_method = DLP_INTERPOLATE_NEAREST_EXACT;
+                else if (method == "bilinear")
+                    n.interp_method = DLP_INTERPOLATE_BILINEAR;
+                else
+                    throw ValidationError("Unsupported interpolation method " + method);
+                DLPRIM_CHECK((n.scale_yx[0] <= 0) == (n.scale_yx[1] <= 0));
+                DLPRIM_CHECK((n.out_hw[0] <= 0) == (n.out_hw[1] <= 0));
+                DLPRIM_CHECK((n.scale_yx[1] <= 0) != (n.out_hw[1] <= 0));
+                DLPRIM_CHECK(n.interp_method == DLP_INTERPOLATE_BILINEAR || !n.align_corners);
+                specs_[n.outputs[0]] = interpolation_shape(n, spec(n.inputs[0]));
+            } else if (n.type == "Reduction") { // ReductionConfig::from_json, src/ops/reduction.cpp:15-35
+                n.kind = k_reduce;
+                DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
+                const bool has = o.type() == json::is_object;
+                std::string method = has ? o.get("method", "sum") : "sum";
+                if (method == "sum")
+                    n.reduce_method = DLP_REDUCE_SUM;
+                else if (method == "sumsq")
+                    n.reduce_method = DLP_REDUCE_SUMSQ;
+                else if (method == "abssum")
+                    n.reduce_method = DLP_REDUCE_ABSSUM;
+                else if (method == "mean")
+                    n.reduce_method = DLP_REDUCE_MEAN;
+                else
+                    throw ValidationError("Unknown reduction method " + method);
+                n.output_scale = has ? o.get("output_scale", 1.0f) : 1.0f;
+                n.keep_dim = has ? o.get("keep_dim", true) : true;
+                n.has_dims = has && !o.find("dims").is_undefined();
+                if (n.has_dims) {
+                    if (!o.find("start_axis").is_undefined())
+                        throw ValidationError("Can't use both dims and start_axis in Reduction");
+                    n.reduce_dims = int_list(o, "dims");
+                    if (n.reduce_dims.empty())
+                        throw ValidationError("Using dims in Reduction requires providing at least 1 dimension");
+                } else
+                    n.start_axis = has ? o.get("start_axis", 0) : 0;
+                specs_[n.outputs[0]] = reduction_shape(n, spec(n.inputs[0]));
+            } else if (n.type == "Parameter") { // the output is the parameter itself (ParameterConfig::from_json, src/ops/parameter.cpp:13-21)
+                n.kind = k_param;
+                DLPRIM_CHECK(n.inputs.empty() && n.outputs.size() == 1);
+                std::string dt = o.get("dtype", "float");
+                if (dt != "float" && dt != "float32")
+                    throw NotImplementedError("Parameter of dtype " + dt + " (" + n.name + ")");
+                Shape s = shape_of(o.get<std::vector<int>>("shape"));
+                specs_[n.outputs[0]] = s;
+                make_param(n, 0, s);
+            } else if (n.type == "MSELoss") { // src/ops/mse_loss.cpp:29-42
+                n.kind = k_mse_loss;
+                DLPRIM_CHECK(n.inputs.size() == 2 && n.outputs.size() == 1);
+                DLPRIM_CHECK(spec(n.inputs[0]) == spec(n.inputs[1]));
+                DLPRIM_CHECK(!int_inputs_.count(n.inputs[0]) && !int_inputs_.count(n.inputs[1]));
+                n.loss_reduce = loss_reduce_option(o);
+                specs_[n.outputs[0]] = n.loss_reduce == DLP_LOSS_REDUCE_NONE ? spec(n.inputs[0]) : Shape(size_t(1));
+            } else if (n.type == "NLLLoss") { // src/ops/nll_loss.cpp:29-45
+                n.kind = k_nll_loss;
+                DLPRIM_CHECK(n.inputs.size() == 2 && n.outputs.size() == 1);
+                check_labels(n);
+                n.loss_reduce = loss_reduce_option(o);
+                specs_[n.outputs[0]] = Shape(n.loss_reduce == DLP_LOSS_REDUCE_NONE ? spec(n.inputs[0])[0] : size_t(1));
+            } else if (n.type == "SoftmaxWithLoss") { // src/ops/softmax.cpp:71-89
+                n.kind = k_softmax_loss;
+                DLPRIM_CHECK(n.inputs.size() == 2 && n.outputs.size() == 1);
+                check_labels(n);
+                specs_[n.outputs[0]] = Shape(size_t(1));
             } else if (n.type == "Flatten") { // a view: [B, everything else]; no kernel, no memory
                 n.kind = k_flatten;
                 DLPRIM_CHECK(n.inputs.size() == 1 && n.outputs.size() == 1 && n.inputs[0] != n.outputs[0]);
@@ -1007,7 +1207,8 @@ private:
         for (auto &n : nodes_) {
             if (n.skipped)
                 continue;
-            Shape const &in = spec(n.inputs[0]);
+            Shape const &in = n.inputs.empty() ? spec(n.outputs[0]) : spec(n.inputs[0]);
+            workspace_bytes_ = std::max(workspace_bytes_, node_workspace(n));
             switch (n.kind) {
             case k_conv: create_conv_operator(n, in); break;
             case k_tconv: create_tconv_operator(n, in); break;
@@ -1056,7 +1257,7 @@ private:
             }
         tensor_memory_ = 0;
         auto own = [&](std::string const &name) {
-            tensors_[name] = Tensor(ctx_, spec(name), dtype_);
+            tensors_[name] = Tensor(ctx_, spec(name), int_inputs_.count(name) ? int32_data : dtype_);
             tensor_memory_ += tensors_[name].memory_size();
         };
         for (auto const &name : input_names_)
@@ -1179,6 +1380,13 @@ private:
                 n.w_dev.to_device(e);
             }
         }
+        if (n.kind == k_param && dtype_ != float_data) { // the values in the storage type
+            Tensor &w = param(n.param_names[0]);
+            n.w_dev = Tensor(ctx_, w.shape(), dtype_);
+            for (size_t k = 0; k < w.shape().total_size(); k++)
+                n.w_dev.data<uint16_t>()[k] = to_bf16_bits(w.data<float>()[k]);
+            n.w_dev.to_device(e);
+        }
         if (n.kind == k_conv && prepack_ && n.conv_op)
             pack_conv_weights(n, e);
         if (n.kind == k_conv && n.dw_node >= 0) // the depthwise convolution that this node runs as well
@@ -1187,9 +1395,48 @@ private:
 
     void run(Node &n, ExecutionContext const &e)
     {
-        Tensor &x = tensor(n.inputs[0]);
         Tensor &y = tensor(n.outputs[0]);
+        Tensor &x = n.inputs.empty() ? y : tensor(n.inputs[0]);
+        void *ws = workspace_bytes_ > 0 ? workspace_.device_ptr() : nullptr;
+        const size_t ws_bytes = workspace_bytes_ > 0 ? workspace_.memory_size() : 0;
         switch (n.kind) {
+        case k_interp: {
+            Shape const &xs = x.shape(), &ys = y.shape();
+            details::check_status(dlp_interpolate2d_fwd_enqueue(int(dtype_), n.interp_method, n.align_corners ? 1 : 0, n.scale_yx[0], n.scale_yx[1],
+                                                                int(xs[0] * xs[1]), int(xs[2]), int(xs[3]), int(ys[2]), int(ys[3]), x.device_ptr(),
+                                                                y.device_ptr(), e.stream()));
+            break;
+        }
+        case k_reduce: {
+            Shape const &xs = x.shape();
+            std::vector<int> mask = reduced_axes(n, xs), dims(size_t(xs.size()));
+            for (int a = 0; a < xs.size(); a++)
+                dims[size_t(a)] = int(xs[a]);
+            details::check_status(dlp_reduce_fwd_enqueue(int(dtype_), n.reduce_method, n.output_scale, xs.size(), dims.data(), mask.data(), x.device_ptr(),
+                                                         y.device_ptr(), ws, ws_bytes, e.stream()));
+            break;
+        }
+        case k_param: { // Parameter::forward copies the parameter into the output (src/ops/parameter.cpp:23-45)
+            Tensor &w = dtype_ == float_data ? param(n.param_names[0]) : n.w_dev;
+            details::check_status(dlp_copy2d_enqueue(y.device_ptr(), w.memory_size(), w.device_ptr(), w.memory_size(), w.memory_size(), 1, e.stream()));
+            break;
+        }
+        case k_mse_loss:
+            details::check_status(dlp_mse_loss_fwd_enqueue(int(dtype_), n.loss_reduce, x.shape().total_size(), x.device_ptr(),
+                                                           tensor(n.inputs[1]).device_ptr(), y.device_ptr(), ws, ws_bytes, e.stream()));
+            break;
+        case k_nll_loss: {
+            Tensor &lbl = tensor(n.inputs[1]);
+            details::check_status(dlp_nll_loss_fwd_enqueue(int(dtype_), int(lbl.dtype()), n.loss_reduce, int(x.shape()[0]), int(x.shape()[1]), x.device_ptr(),
+                                                           lbl.device_ptr(), y.device_ptr(), e.stream()));
+            break;
+        }
+        case k_softmax_loss: {
+            Tensor &lbl = tensor(n.inputs[1]);
+            details::check_status(dlp_softmax_loss_fwd_enqueue(int(dtype_), int(lbl.dtype()), int(x.shape()[0]), int(x.shape()[1]), x.device_ptr(),
+                                                               lbl.device_ptr(), y.device_ptr(), ws, ws_bytes, e.stream()));
+            break;
+        }
         case k_conv: {
             Tensor &w = n.use_w_dev ? n.w_dev : param(n.param_names[0]);
             Tensor *b = n.folded_bn ? &n.b_dev : n.bias ? &param(n.param_names[1]) : nullptr;
@@ -1297,6 +1544,7 @@ private:
     std::vector<std::string> input_names_, output_names_;
     std::map<std::string, Shape> specs_;
     std::map<std::string, Tensor> tensors_, params_;
+    std::set<std::string> int_inputs_; // inputs stored as int32 (labels), whatever the storage type of the others
     std::map<std::string, std::string> alias_of_; // output of a fused residual sum -> the branch it is written over
     Tensor workspace_;
     size_t workspace_bytes_ = 0, tensor_memory_ = 0;

@@ -30,6 +30,7 @@ extern "C" {
 #define DLP_FLOAT 3
 #define DLP_HALF 2
 #define DLP_BFLOAT16 10
+#define DLP_INT32 19 /* int32_data: class labels of the losses */
 
 /* dlprim::StandardActivations, include/dlprim/definitions.hpp:278-284 */
 #define DLP_ACT_IDENTITY 0
@@ -327,6 +328,53 @@ int dlp_pointwise_fwd_enqueue(int dtype, int operation, float p0, float p1, size
  * computed by the caller (fp32 device arrays of `channels` values); plane = H * W; x == y is allowed. */
 int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int channels, int plane, const void *x, const float *scale,
                                    const float *shift, void *y, void *stream);
+
+/* core::interpolate2d, include/dlprim/core/interpolate.hpp:17 (src/core/interpolate.cpp:10-78, kernels of
+ * src/kernels/interpolate_2d.cl): x [planes, src_h, src_w] -> y [planes, tgt_h, tgt_w], planes = batch * channels.
+ * method as dlprim::InterpolateType (include/dlprim/definitions.hpp:325-329).  scale_y / scale_x <= 0: the steps follow from the
+ * sizes; otherwise tgt = int(src * scale) is checked.  nearest: source index min(int((p + offset) * step), src - 1) with offset 0,
+ * or 0.5 for nearest-exact; bilinear: source position max(step * (p + 0.5) - 0.5, 0), or p * (src - 1) / (tgt - 1) with
+ * align_corners, and the two neighbours weighted by the fraction. */
+#define DLP_INTERPOLATE_NEAREST 0
+#define DLP_INTERPOLATE_NEAREST_EXACT 1
+#define DLP_INTERPOLATE_BILINEAR 2
+int dlp_interpolate2d_fwd_enqueue(int dtype, int method, int align_corners, double scale_y, double scale_x, int planes, int src_h,
+                                  int src_w, int tgt_h, int tgt_w, const void *x, void *y, void *stream);
+
+/* Reduction::forward, src/ops/reduction.cpp:96-111,300-361 (ReductionConfig::Method, include/dlprim/ops/reduction.hpp:16-21):
+ * y = coefficient * sum over the dimensions with reduce[j] != 0 of x | x^2 | |x|; coefficient = output_scale, for mean
+ * output_scale * (elements of y) / (elements of x).  shape and reduce have `rank` (1 to 8) entries; y holds the kept dimensions in
+ * order (its shape with or without the reduced ones as extent 1 is the caller's).  Neighbouring dimensions that are all kept or all
+ * reduced count as one group; more than three groups of either kind are NotImplemented (any tensor of rank <= 6 fits).  Sums are fp32;
+ * the pieces of a long reduction are added in a fixed order, so results repeat bit for bit.  The workspace (device memory, size from
+ * dlp_reduce_fwd_workspace, possibly 0) holds the pieces. */
+#define DLP_REDUCE_SUM 0
+#define DLP_REDUCE_SUMSQ 1
+#define DLP_REDUCE_ABSSUM 2
+#define DLP_REDUCE_MEAN 3
+int dlp_reduce_fwd_workspace(int dtype, int method, int rank, const int *shape, const int *reduce, size_t *bytes);
+int dlp_reduce_fwd_enqueue(int dtype, int method, float output_scale, int rank, const int *shape, const int *reduce, const void *x,
+                           void *y, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The forward pass of the losses.  reduce as MSELossConfig / NLLLossConfig::Reduce (none, sum, mean). */
+#define DLP_LOSS_REDUCE_NONE 0
+#define DLP_LOSS_REDUCE_SUM 1
+#define DLP_LOSS_REDUCE_MEAN 2
+/* MSELoss::forward, src/ops/mse_loss.cpp:70-111: y[i] = (a[i] - b[i])^2 over n elements, or their sum / mean in y[0] */
+int dlp_mse_loss_fwd_workspace(int dtype, int reduce, size_t n, size_t *bytes);
+int dlp_mse_loss_fwd_enqueue(int dtype, int reduce, size_t n, const void *a, const void *b, void *y, void *workspace,
+                             size_t workspace_bytes, void *stream);
+/* core::nll_loss_forward, include/dlprim/core/loss.hpp:26 (NLLLoss::forward, src/ops/nll_loss.cpp:59-110; kernel
+ * src/kernels/nll_loss_fwd.cl): x [batch, classes], labels [batch] stored as label_dtype (DLP_FLOAT or DLP_INT32);
+ * y[b] = -x[b][label[b]], 0 for a label outside [0, classes), or the sum / mean over the batch in y[0] */
+int dlp_nll_loss_fwd_enqueue(int dtype, int label_dtype, int reduce, int batch, int classes, const void *x, const void *labels,
+                             void *y, void *stream);
+/* SoftmaxWithLoss::forward, src/ops/softmax.cpp:134-155,224-244 (kernel src/kernels/softmax_with_loss.cl with CALC_LOSS 1):
+ * y[0] = mean over the rows of -(x[b][label] - max_b - log(sum_c exp(x[b][c] - max_b))); a row whose label lies outside
+ * [0, classes) adds 0, as in the reference's kernel.  The workspace holds one float per row. */
+int dlp_softmax_loss_fwd_workspace(int batch, size_t *bytes);
+int dlp_softmax_loss_fwd_enqueue(int dtype, int label_dtype, int batch, int classes, const void *x, const void *labels, void *y,
+                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* ===== data types ==================================================================
  * DLP_FLOAT: everything fp32, as in the reference (its conv/GEMM reject other types,

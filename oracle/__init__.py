@@ -358,6 +358,138 @@ def softmax_forward(x, log=False):
     return y.astype(np.float32).reshape(shape)
 
 
+def interpolate_output_size(in_hw, out_hw=(-1, -1), scale=(-1.0, -1.0)):
+    """Interpolation::calc_size, src/ops/interpolation.cpp:53-69: the given size, or int(in * scale) per axis"""
+    if out_hw[0] > 0:
+        return int(out_hw[0]), int(out_hw[1])
+    return int(in_hw[0] * scale[0]), int(in_hw[1] * scale[1])
+
+
+def _interp_step(scale, src, tgt, align_corners):
+    """Interpolation::calc_bin_scale, src/ops/interpolation.cpp:121-131 (float results)"""
+    if align_corners:
+        return np.float32(0) if tgt <= 1 else np.float32(float(src - 1) / (tgt - 1))
+    if scale > 0:
+        return np.float32(1.0 / scale)
+    return np.float32(float(src) / tgt)
+
+
+def interpolate2d_forward(x, out_hw, method="nearest", scale=(-1.0, -1.0), align_corners=False):
+    """Interpolation::forward on the CPU, src/ops/interpolation.cpp: nearest / nearest-exact as forward_cpu (:271-305: source index
+    min(int((p + offset) * step), size - 1), offset 0 or 0.5, step float(1 / scale) or float(in) / out), bilinear as
+    bilinear_fwd_bwd_cpu with HandleFWD (:86-96,133-195: position max(step * (p + 0.5) - 0.5, 0) or step * p with align_corners,
+    neighbours p0 and p0 + 1 (clamped), weights from the fraction), all in float32."""
+    x = _f32(x)
+    B, C, H, W = x.shape
+    OH, OW = out_hw
+    f = np.float32
+    if method in ("nearest", "nearest-exact"):
+        vs = f(1.0 / scale[0]) if scale[0] > 0 else f(H) / f(OH)
+        hs = f(1.0 / scale[1]) if scale[1] > 0 else f(W) / f(OW)
+        offset = f(0.0 if method == "nearest" else 0.5)
+        rows = np.minimum(((np.arange(OH, dtype=np.float32) + offset) * vs).astype(np.int32), H - 1)
+        cols = np.minimum(((np.arange(OW, dtype=np.float32) + offset) * hs).astype(np.int32), W - 1)
+        return np.ascontiguousarray(x[:, :, rows][:, :, :, cols])
+    assert method == "bilinear"
+
+    def axis(step, size, n):
+        p = np.arange(n, dtype=np.float32)
+        pos = step * p if align_corners else np.maximum(step * (p + f(0.5)) - f(0.5), f(0))
+        pos = pos.astype(np.float32)
+        p0 = pos.astype(np.int32)
+        p1 = p0 + (p0 < size - 1)
+        w1 = (pos - p0.astype(np.float32)).astype(np.float32)
+        return p0, p1, (f(1) - w1).astype(np.float32), w1
+
+    r0, r1, wr0, wr1 = axis(_interp_step(scale[0], H, OH, align_corners), H, OH)
+    c0, c1, wc0, wc1 = axis(_interp_step(scale[1], W, OW, align_corners), W, OW)
+    top = wc0 * x[:, :, r0][:, :, :, c0] + wc1 * x[:, :, r0][:, :, :, c1]
+    bottom = wc0 * x[:, :, r1][:, :, :, c0] + wc1 * x[:, :, r1][:, :, :, c1]
+    y = wr0[:, None] * top.astype(np.float32) + wr1[:, None] * bottom.astype(np.float32)
+    return y.astype(np.float32)
+
+
+def reduction_dims(rank, dims=None, start_axis=0):
+    """Reduction::setup, src/ops/reduction.cpp:49-69: the axes that are reduced"""
+    if dims is None:
+        if start_axis < 0:
+            start_axis += rank
+        assert 0 <= start_axis < rank
+        return list(range(start_axis, rank))
+    return sorted({d + rank if d < 0 else d for d in dims})
+
+
+def reduction_forward(x, method="sum", dims=None, start_axis=0, output_scale=1.0, keep_dim=True):
+    """Reduction::forward_cpu, src/ops/reduction.cpp:296-330: float32 sums of x, x*x or |x| in memory order into the kept positions,
+    then one multiplication by output_scale (mean: output_scale * outputs / elements, get_coeff :323-329); the output shape keeps
+    the reduced axes as 1 or drops them (calc_shapes :133-151)."""
+    x = _f32(x)
+    axes = reduction_dims(x.ndim, dims, start_axis)
+    term = {"sum": x, "mean": x, "sumsq": x * x, "abssum": np.abs(x)}[method]
+    # sequential float32 accumulation in memory order: move the reduced axes behind the kept ones, keeping their order
+    kept = [a for a in range(x.ndim) if a not in axes]
+    t = np.transpose(term, kept + axes).reshape(int(np.prod([x.shape[a] for a in kept], dtype=np.int64)), -1)
+    acc = np.zeros(t.shape[0], dtype=np.float32)
+    for j in range(t.shape[1]):
+        acc += t[:, j]
+    coeff = np.float32(output_scale)
+    if method == "mean":
+        coeff = np.float32(np.float32(output_scale) * np.float32(acc.size) / np.float32(x.size))
+    if coeff != np.float32(1.0):
+        acc = acc * coeff
+    shape = [1 if a in axes else x.shape[a] for a in range(x.ndim)] if keep_dim else [x.shape[a] for a in kept]
+    return acc.astype(np.float32).reshape(shape if shape else [1])
+
+
+def mse_loss_forward(a, b, reduce="mean"):
+    """MSELoss::forward_cpu, src/ops/mse_loss.cpp:70-92: (a - b)^2 per element, or their float32 sum in index order (mean: * 1 / size)"""
+    a, b = _f32(a), _f32(b)
+    d = (a - b).astype(np.float32)
+    sq = (d * d).astype(np.float32)
+    if reduce == "none":
+        return sq
+    total = np.float32(0)
+    for v in sq.reshape(-1):
+        total = np.float32(total + v)
+    if reduce == "mean":
+        total = np.float32(total * np.float32(1.0 / a.size))
+    return np.array([total], dtype=np.float32)
+
+
+def nll_loss_forward(x, labels, reduce="mean"):
+    """NLLLoss::forwad_cpu, src/ops/nll_loss.cpp:59-86: -x[b][label[b]] per row (0 for a label outside the classes), or the float32 sum
+    over the rows (mean: * 1 / batch)"""
+    x = _f32(x)
+    idx = np.asarray(labels).astype(np.int64).reshape(-1)
+    ok = (idx >= 0) & (idx < x.shape[1])
+    rows = np.where(ok, -x[np.arange(x.shape[0]), np.clip(idx, 0, x.shape[1] - 1)], np.float32(0)).astype(np.float32)
+    if reduce == "none":
+        return rows
+    total = np.float32(0)
+    for v in rows:
+        total = np.float32(total + v)
+    if reduce == "mean":
+        total = np.float32(total * np.float32(1.0 / x.shape[0]))
+    return np.array([total], dtype=np.float32)
+
+
+def softmax_loss_forward(x, labels):
+    """SoftmaxWithLoss::forward_cpu_loss, src/ops/softmax.cpp:134-155: per row the maximum, the float32 sum of expf(x - max) in index
+    order, loss -= x[label] - max - logf(sum); the total divided by the batch.  (The CPU code checks label < classes; the kernel,
+    src/kernels/softmax_with_loss.cl, adds 0 for such a row -- the behaviour kept here.)"""
+    x = _f32(x)
+    idx = np.asarray(labels).astype(np.int64).reshape(-1)
+    total = np.float32(0)
+    for b in range(x.shape[0]):
+        m = x[b].max()
+        s = np.float32(0)
+        for v in np.exp((x[b] - m).astype(np.float32)).astype(np.float32):
+            s = np.float32(s + v)
+        if 0 <= idx[b] < x.shape[1]:
+            total = np.float32(total - np.float32(np.float32(x[b, idx[b]] - m) - np.log(s).astype(np.float32)))
+    return np.array([np.float32(total / np.float32(x.shape[0]))], dtype=np.float32)
+
+
 def bf16_round(a):
     a = _f32(a).copy()
     lib().orc_bf16_round_array(_ptr(a), ctypes.c_size_t(a.size))

@@ -7,6 +7,12 @@ Reads DATA files only (JSON written by the reference's PyTorch fixture generator
   tests/test_case_global_pooling.json -> global_pooling_fwd.json
   tests/test_case_softmax.json        -> softmax_fwd.json       (cases of up to 1100 values)
   tests/test_case_log_softmax.json    -> log_softmax_fwd.json   (likewise)
+  tests/test_case_interpolation.json  -> interpolation_fwd.json (cases of up to 200 values)
+  tests/test_case_reduction.json      -> reduction_fwd.json     (cases of up to 800 values)
+  tests/test_case_mse_loss.json, test_case_nll_loss.json, test_case_softmax_loss.json
+                                      -> mse_loss_fwd.json, nll_loss_fwd.json, softmax_loss_fwd.json (up to 2000, 400, 1000 values)
+  tests/test_case_abs.json, test_case_hardtanh.json, test_case_threshold.json, test_case_concat.json, test_case_slice.json
+                                      -> abs_fwd.json, hardtanh_fwd.json, threshold_fwd.json, concat_fwd.json, slice_fwd.json
 keeping options, parameters, inputs and expected forward outputs (gradients are
 dropped: the path is forward only).  Run in the build container, where the
 reference tree is mounted:  python tests/golden/extract_reference_fixtures.py
@@ -55,3 +61,10 @@ if __name__ == "__main__":
     extract("test_case_global_pooling.json", "global_pooling_fwd.json")
     extract("test_case_softmax.json", "softmax_fwd.json", 1100)
     extract("test_case_log_softmax.json", "log_softmax_fwd.json", 1100)
+    extract("test_case_interpolation.json", "interpolation_fwd.json", 200)
+    extract("test_case_reduction.json", "reduction_fwd.json", 800)
+    extract("test_case_mse_loss.json", "mse_loss_fwd.json", 2000)
+    extract("test_case_nll_loss.json", "nll_loss_fwd.json", 400)
+    extract("test_case_softmax_loss.json", "softmax_loss_fwd.json", 1000)
+    for name in ("abs", "hardtanh", "threshold", "concat", "slice"):
+        extract("test_case_%s.json" % name, name + "_fwd.json", 2000)
