@@ -5,9 +5,13 @@
 //
 //   test_core_api host   : everything that needs no GPU (shapes, exceptions)
 //   test_core_api <dev>  : the device checks on HIP device <dev> (default 0)
+#include <dlprim/core/activation.hpp>
 #include <dlprim/core/bias.hpp>
+#include <dlprim/core/common.hpp>
 #include <dlprim/core/conv.hpp>
+#include <dlprim/core/interpolate.hpp>
 #include <dlprim/core/ip.hpp>
+#include <dlprim/core/loss.hpp>
 #include <dlprim/core/pool.hpp>
 
 #include <algorithm>
@@ -355,6 +359,87 @@ static void pool_case(dp::Context &ctx, dp::ExecutionContext &q)
     EXPECT(thrown);
 }
 
+// the free functions of core/activation.hpp, loss.hpp, interpolate.hpp and SliceCopy of common.hpp against plain loops
+static void tensor_function_case(dp::Context &ctx, dp::ExecutionContext &q)
+{
+    std::mt19937 rng(11);
+    const int B = 6, C = 9;
+    dp::Tensor X(ctx, dp::Shape(B, C)), A(ctx, dp::Shape(B, C)), L(ctx, dp::Shape(B, C)), lbl(ctx, dp::Shape(B), dp::int32_data);
+    dp::Tensor rows(ctx, dp::Shape(B)), mean(ctx, dp::Shape(1));
+    fill(X, rng, -2, 2);
+    for (int b = 0; b < B; b++)
+        lbl.data<int>()[b] = (b * 5 + 1) % C;
+    X.to_device(q);
+    lbl.to_device(q);
+    dp::core::activation_forward(X, A, dp::StandardActivations::tanh, q);
+    dp::core::softmax_forward(X, L, true, q);
+    dp::core::nll_loss_forward(L, lbl, rows, false, 1.0f, q);
+    dp::core::nll_loss_forward(L, lbl, mean, true, 1.0f / B, q);
+    A.to_host(q);
+    L.to_host(q);
+    rows.to_host(q);
+    mean.to_host(q);
+    q.finish();
+    double worst = 0, total = 0;
+    for (int b = 0; b < B; b++) {
+        double sum = 0;
+        for (int c = 0; c < C; c++) {
+            sum += std::exp(double(X.data<float>()[b * C + c]));
+            worst = std::fmax(worst, std::fabs(std::tanh(double(X.data<float>()[b * C + c])) - A.data<float>()[b * C + c]));
+        }
+        const double want = std::log(sum) - X.data<float>()[b * C + lbl.data<int>()[b]];
+        worst = std::fmax(worst, std::fabs(want - rows.data<float>()[b]));
+        total += want;
+    }
+    worst = std::fmax(worst, std::fabs(total / B - mean.data<float>()[0]));
+    std::printf("activation, log-softmax, nll loss : max err %.2e\n", worst);
+    EXPECT(worst < 1e-5);
+
+    // interpolate2d: nearest by 2 repeats every pixel; bilinear with align_corners keeps the corners
+    dp::Tensor img(ctx, dp::Shape(2, 3, 4, 5)), up(ctx, dp::Shape(2, 3, 8, 10)), lin(ctx, dp::Shape(2, 3, 7, 9));
+    fill(img, rng, -1, 1);
+    img.to_device(q);
+    dp::core::interpolate2d(img, up, 2.0, 2.0, dp::InterpolateType::nearest, false, q);
+    dp::core::interpolate2d(img, lin, -1, -1, dp::InterpolateType::bilinear, true, q);
+    up.to_host(q);
+    lin.to_host(q);
+    q.finish();
+    bool same = true;
+    for (int p = 0; p < 6; p++) {
+        for (int r = 0; r < 8; r++)
+            for (int c = 0; c < 10; c++)
+                same = same && up.data<float>()[(p * 8 + r) * 10 + c] == img.data<float>()[(p * 4 + r / 2) * 5 + c / 2];
+        same = same && std::fabs(lin.data<float>()[p * 63] - img.data<float>()[p * 20]) < 1e-6 &&
+               std::fabs(lin.data<float>()[p * 63 + 62] - img.data<float>()[p * 20 + 19]) < 1e-6;
+    }
+    EXPECT(same);
+    bool thrown = false;
+    try {
+        dp::core::interpolate2d(img, lin, 2.0, 2.0, dp::InterpolateType::nearest, false, q); // 7 x 9 is not int(4 * 2) x int(5 * 2)
+    } catch (dp::ValidationError const &) {
+        thrown = true;
+    }
+    EXPECT(thrown);
+
+    // SliceCopy: channels 1..2 of img into channels 3..4 of a wider tensor
+    dp::Tensor wide(ctx, dp::Shape(2, 6, 4, 5));
+    std::fill(wide.data<float>(), wide.data<float>() + wide.shape().total_size(), -7.0f);
+    wide.to_device(q);
+    dp::core::SliceCopy copy(ctx);
+    copy.tensor_slice_copy(1, 2, wide, 3, img, 1, 0.0f, q);
+    wide.to_host(q);
+    q.finish();
+    same = true;
+    for (int b = 0; b < 2; b++)
+        for (int c = 0; c < 6; c++)
+            for (int i = 0; i < 20; i++) {
+                const float want = (c == 3 || c == 4) ? img.data<float>()[(b * 3 + c - 2) * 20 + i] : -7.0f;
+                same = same && wide.data<float>()[(b * 6 + c) * 20 + i] == want;
+            }
+    EXPECT(same);
+    std::printf("interpolate2d, SliceCopy : %s\n", same ? "ok" : "mismatch");
+}
+
 int main(int argc, char **argv)
 {
     std::string dev = argc > 1 ? argv[1] : "0";
@@ -379,6 +464,7 @@ int main(int argc, char **argv)
             ip_backward_case(ctx, q, 70, 33, 129, 0.5f);
             ip_backward_case(ctx, q, 1, 512, 1000, 1.0f);
             pool_case(ctx, q);
+            tensor_function_case(ctx, q);
             // sub-tensor views share memory: run on the second image of a batch-2 tensor
             dp::Tensor big(ctx, dp::Shape(2, 4, 6, 6));
             dp::Tensor second = big.sub_tensor(4 * 6 * 6, dp::Shape(1, 4, 6, 6));
