@@ -556,18 +556,22 @@ def test_gpu_mobilenet_224_fuses_depthwise_pointwise_pairs(tmp_path):
         assert ops[("keep",)] - ops[()] == 10 + pairs
 
 
-def random_net(seed):
+def random_net(seed, extended=False):
     """A random graph over one spatial size: convolutions (1x1 / 3x3, with and without bias / activation), BatchNorm,
     activations in place and not, element-wise operations between any two tensors made so far, now and then a
     pooling that starts a new size.  Tensors are read again long after they were made, which is what the memory
-    plan, the BatchNorm folding and the residual rewrite have to get right."""
+    plan, the BatchNorm folding and the residual rewrite have to get right.  extended: also Interpolation (a new size), a channel mean
+    that is broadcast back, Concat followed by a Slice, Hardtanh."""
     rng = np.random.default_rng(seed)
     c = int(rng.choice([4, 8, 12]))
     b = netfile.NetBuilder("data", (2, c, 12, 10))
     live = ["data"]  # tensors of the current shape
     made = 0
     for step in range(int(rng.integers(8, 16))):
-        kind = rng.choice(["conv", "conv", "conv", "bn", "act", "elt", "elt", "pool"])
+        kinds = ["conv", "conv", "conv", "bn", "act", "elt", "elt", "pool"]
+        if extended:
+            kinds += ["interp", "gate", "catslice", "clamp"]
+        kind = rng.choice(kinds)
         src = live[-1] if rng.random() < 0.65 else str(rng.choice(live))
         made += 1
         name = "t%d" % made
@@ -589,6 +593,26 @@ def random_net(seed):
             op = str(rng.choice(["sum", "sum", "sum", "prod", "max"]))
             coefs = [(None, None), (None, 0.5), (2.0, None)][int(rng.integers(3))]
             b.eltwise(src, other, name, op, coef1=coefs[0], coef2=coefs[1], activation=str(rng.choice(["", "relu"])) or None)
+        elif kind == "interp":
+            h, w = b.shapes[src][2:]
+            if h > 20:
+                continue
+            method = str(rng.choice(["nearest", "nearest-exact", "bilinear"]))
+            if rng.integers(2):
+                b.interpolation(src, name, method, scale=(1.5, 2))
+            else:
+                b.interpolation(src, name, method, out_hw=(h + 3, max(w - 2, 2)), align_corners=bool(method == "bilinear" and rng.integers(2)))
+            live = []
+        elif kind == "gate":  # the mean over the channels, broadcast back over them
+            m = b.reduction(src, name + "m", str(rng.choice(["mean", "abssum"])), dims=[1], output_scale=0.5)
+            b.eltwise(src, m, name, str(rng.choice(["sum", "prod"])))
+        elif kind == "catslice":
+            other = str(rng.choice(live))
+            cat = b.concat([src, other], name + "c")
+            first = int(rng.integers(0, c + 1))
+            b.slice(cat, name, first, first + c)
+        elif kind == "clamp":
+            b.pointwise(src, name, "Hardtanh", min_val=-0.5, max_val=0.75)
         else:
             if b.shapes[src][2] < 6:
                 continue
@@ -602,9 +626,9 @@ def random_net(seed):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", list(range(40)) + list(range(100, 130)))
 def test_gpu_net_random_graphs(tmp_path, seed):
-    b = random_net(seed)
+    b = random_net(seed, extended=seed >= 100)
     p = write_net(tmp_path, b)
     params = b.random_parameters(seed)
     netfile.save_dlpw(tmp_path / "w.dlpw", params)
