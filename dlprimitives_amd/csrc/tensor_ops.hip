@@ -187,7 +187,7 @@ template <class T>
 __device__ __forceinline__ void reduce_emit(const ReduceArgs &a, uint32_t o, uint32_t piece, float sum, T *y, float *partial)
 {
     if (a.splits > 1)
-        partial[(size_t)o * a.splits + piece] = sum;
+        partial[(size_t)piece * a.outputs + o] = sum; // piece-major: neighbouring outputs next to each other
     else
         store_plain(y + o, sum * a.coeff);
 }
@@ -283,21 +283,45 @@ __global__ __launch_bounds__(256) void reduce_outer_kernel(ReduceArgs a, const T
     }
 }
 
-// adds up the pieces of every output in a fixed order: one wave per output, a lane takes every 64th piece
-template <class T>
+// adds up the pieces of every output (partial[piece][output]) in a fixed order: LANES lanes per output, a lane takes every
+// LANES-th piece, four loads in flight.  LANES 1: a thread per output, for a handful of pieces of many outputs (neighbouring
+// threads read neighbouring values); 64: a wave per output; 256: the block, for hundreds of pieces of a few outputs.
+template <class T, int LANES>
 __global__ __launch_bounds__(256) void reduce_finish_kernel(uint32_t outputs, uint32_t splits, float coeff, const float *__restrict__ partial,
                                                              T *__restrict__ y)
 {
-    const uint32_t o = blockIdx.x * 4 + threadIdx.x / 64;
-    const uint32_t lane = threadIdx.x % 64;
-    if (o >= outputs)
-        return;
+    __shared__ float sums[4];
+    const uint32_t o = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
+    const uint32_t lane = threadIdx.x % LANES;
+    const bool live = o < outputs; // LANES > 1: the same for all lanes of a wave, and of the block when LANES is 256
     float sum = 0.0f;
-    for (uint32_t s = lane; s < splits; s += 64)
-        sum += partial[(size_t)o * splits + s];
+    if (live) {
+        const float *p = partial + o;
+        const size_t step = (size_t)outputs * LANES;
+        uint32_t s = lane;
+        for (; s + 3 * LANES < splits; s += 4 * LANES) {
+            const float *q = p + (size_t)s * outputs;
+            sum += (q[0] + q[step]) + (q[2 * step] + q[3 * step]);
+        }
+        for (; s < splits; s += LANES)
+            sum += p[(size_t)s * outputs];
+    }
+    if (LANES == 1) {
+        if (live)
+            store_plain(y + o, sum * coeff);
+        return;
+    }
     sum = wave_sum(sum);
-    if (lane == 0)
-        store_plain(y + o, sum * coeff);
+    if (LANES == 64) {
+        if (live && lane == 0)
+            store_plain(y + o, sum * coeff);
+    } else {
+        if (threadIdx.x % 64 == 0)
+            sums[threadIdx.x / 64] = sum;
+        __syncthreads();
+        if (live && threadIdx.x == 0)
+            store_plain(y + o, (sums[0] + sums[1] + sums[2] + sums[3]) * coeff);
+    }
 }
 
 // ---- losses -----------------------------------------------------------------------------------------------------
@@ -580,7 +604,12 @@ static int launch_reduce(const ReduceCall &c, const void *x, const void *x2, voi
     }
     DLP_HIP_TRY(hipGetLastError());
     if (a.splits > 1) {
-        hipLaunchKernelGGL(reduce_finish_kernel<T>, dim3((a.outputs + 3) / 4), dim3(256), 0, st, a.outputs, a.splits, a.coeff, partial, yp);
+        if (a.splits >= 256)
+            hipLaunchKernelGGL((reduce_finish_kernel<T, 256>), dim3(a.outputs), dim3(256), 0, st, a.outputs, a.splits, a.coeff, partial, yp);
+        else if (a.splits > 8)
+            hipLaunchKernelGGL((reduce_finish_kernel<T, 64>), dim3((a.outputs + 3) / 4), dim3(256), 0, st, a.outputs, a.splits, a.coeff, partial, yp);
+        else
+            hipLaunchKernelGGL((reduce_finish_kernel<T, 1>), dim3((a.outputs + 255) / 256), dim3(256), 0, st, a.outputs, a.splits, a.coeff, partial, yp);
         DLP_HIP_TRY(hipGetLastError());
     }
     return DLP_OK;
