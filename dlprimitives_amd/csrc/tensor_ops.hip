@@ -537,6 +537,11 @@ static int prepare_reduce(int dtype, int method, float coeff, int rank, const in
     }
     total = outputs * R;
     DLP_REQUIRE(outputs < (1ull << 31) && R < (1ull << 31), "reduction: fewer than 2^31 outputs and reduced elements per output");
+    c.a.R = (uint32_t)R;
+    c.a.outputs = (uint32_t)outputs;
+    c.workspace = 0;
+    if (total == 0) // an extent of 0: nothing to plan (and no divisors to prepare)
+        return DLP_OK;
     int st = plan_reduce(rank, shape, reduce, c.a, c.inner_reduced);
     if (st != DLP_OK)
         return st;
@@ -739,9 +744,9 @@ int dlp_reduce_fwd_enqueue(int dtype, int method, float output_scale, int rank, 
     int st = prepare_reduce(dtype, method, 1.0f, rank, shape, reduce, c, total);
     if (st != DLP_OK)
         return st;
-    DLP_REQUIRE(total > 0 || c.a.outputs == 0, "reduction over no elements");
     if (c.a.outputs == 0)
         return DLP_OK;
+    DLP_REQUIRE(total > 0, "reduction over no elements");
     st = reduce_coeff(method, output_scale, c, c.a.coeff);
     if (st != DLP_OK)
         return st;

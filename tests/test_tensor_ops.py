@@ -151,6 +151,14 @@ def test_reduce_workspace_query_and_validation():
     assert b"three" in L.dlp_last_error()
     # extents of 1 and neighbours of one kind do not count as groups
     assert query([2, 1, 3, 4, 1, 5, 6, 7], [0, 1, 0, 1, 1, 1, 0, 0])[0] == 0
+    # an extent of 0: no workspace; no outputs is a call that does nothing, outputs over no elements an error (before any pointer is read)
+    assert query([4, 0, 3], [0, 1, 0]) == (0, 0) and query([0, 5], [0, 1]) == (0, 0)
+    L.dlp_reduce_fwd_enqueue.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    arr2 = ctypes.c_int * 2
+    assert L.dlp_reduce_fwd_enqueue(3, 0, 1.0, 2, arr2(0, 5), arr2(0, 1), None, None, None, 0, None) == 0
+    assert L.dlp_reduce_fwd_enqueue(3, 0, 1.0, 2, arr2(5, 0), arr2(0, 1), None, None, None, 0, None) == 1
+    assert b"no elements" in L.dlp_last_error()
 
 
 # ------------------------------------------------------------------ GPU
