@@ -5,6 +5,11 @@ dlprimitives CPU operators in ``dlp_oracle.c``) and, when it has been built, of
 ``oracle/_ref/libdlprim_ref.so`` (the reference's own internal BLAS and
 activation helpers compiled from the reference sources).
 
+Interpolation, Reduction and the losses (``interpolate2d_forward``, ``reduction_forward``, ``mse_loss_forward``,
+``nll_loss_forward``, ``softmax_loss_forward``) are numpy restatements of the reference's CPU operators; each is
+pinned by the reference's golden cases (``tests/golden/*_fwd.json``) and by the matching torch routine in
+``tests/test_tensor_ops.py``.
+
 Only tests, the smoke check and the CPU-baseline leg of the benchmark may import
 this package, and only as the checker.  The shipped library never does.
 """
