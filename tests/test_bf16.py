@@ -173,6 +173,56 @@ def test_bf16_stem(oracle_mod, c, bhw):
     np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-3)
 
 
+DENSE_1X1_CASES = [
+    # 1x1 convolutions of 64 / 128 channels over thousands of pixels (the short-K layers of a ResNet-50 bottleneck): the dense loader
+    # with two or four K tiles per workgroup, plain, bit-exact on integers, and with both ways of adding the old y
+    (case(1, 0, 1, 1, 64, 256, True, 1, True), (2, 56, 56)),     # two m tiles of 128
+    (case(1, 0, 1, 1, 128, 512, True, 1, True), (6, 28, 28)),    # four m tiles, the last pixel tile partial, tiles crossing images
+    (case(1, 0, 1, 1, 64, 64, False, 1, False), (3, 40, 40)),    # 64 filters, no bias, no activation
+    (case(1, 0, 1, 1, 128, 192, True, 1, True), (5, 32, 32)),    # 192 filters: a partial m tile
+    (case(1, 0, 1, 1, 64, 128, True, 1, True), (1, 64, 72)),     # one image, not square
+]
+
+
+@pytest.mark.parametrize("c,bhw", DENSE_1X1_CASES, ids=case_id)
+def test_bf16_dense_1x1_with_old_y(oracle_mod, c, bhw):
+    print("dense 1x1", c["cin"], c["cout"], bhw, flush=True)
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    x, w, bias = make_tensors(c, bhw, seed=51)
+    x, w = oracle_mod.bf16_round(x), oracle_mod.bf16_round(w)
+    want = oracle_mod.conv2d_forward(x, w, bias, cfg, c["activation"], threads=8)
+    np.testing.assert_allclose(run_conv_bf16(c, x, w, bias, algo="gemm"), want, rtol=2 ** -8, atol=1e-4 * np.abs(want).max())
+    # integer-valued tensors: every product and sum is exact, the result must equal the reference bit for bit
+    rng = np.random.default_rng(4)
+    xi = rng.integers(-2, 3, x.shape).astype(np.float32)
+    wi = rng.integers(-1, 2, w.shape).astype(np.float32)
+    bi = rng.integers(-3, 4, c["cout"]).astype(np.float32) if c["bias"] else None
+    wanti = oracle_mod.conv2d_forward(xi, wi, bi, cfg, c["activation"], threads=8)
+    assert np.abs(wanti).max() <= 256  # exactly representable in bf16
+    assert np.array_equal(run_conv_bf16(c, xi, wi, bi, algo="gemm"), wanti)
+    # y = factor * y_old + act(conv), and the residual form y = act(conv + factor * y_old)
+    old = rng.standard_normal(want.shape).astype(np.float32)
+    got = run_conv_bf16(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got, oracle_mod.apply_factor(want, oracle_mod.bf16_round(old), 0.5), rtol=2 ** -8, atol=1e-3)
+    st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
+    op = dlp.Conv2DForward.create(st, bias is not None, c["activation"], "gemm")
+    op.accumulate_before_activation(True)
+    y = _bf(old)
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    op.enqueue(_bf(x), _bf(w), torch.from_numpy(bias).cuda() if bias is not None else None, y, ws, 0.5)
+    torch.cuda.synchronize()
+    conv = oracle_mod.conv2d_forward(x, w, bias, cfg, "identity", threads=8)
+    pre = conv + 0.5 * oracle_mod.bf16_round(old)
+    # the convolution's value is rounded to bf16 once before the old y joins it: an error relative to the convolution, not to the sum
+    np.testing.assert_allclose(y.float().cpu().numpy(), oracle_mod.apply_activation(pre.astype(np.float32), c["activation"]), rtol=2 ** -8,
+                               atol=2 ** -8 * np.abs(conv).max())
+
+
 def test_bf16_factor_contract(oracle_mod):
     c = case(3, 1, 1, 1, 16, 24, True, 1, True)
     x, w, bias = make_tensors(c, (2, 11, 9), seed=5)
