@@ -325,6 +325,43 @@ def test_gpu_reduction_shapes_vs_float64(oracle_mod, method, dtype):
 
 
 @pytest.mark.gpu
+def test_gpu_reduction_random_shapes_and_masks():
+    """120 random tensors of rank 1 to 6 (extents 1 to 9, now and then one long axis) with random sets of reduced axes: every way the
+    axes can group into kept / reduced runs, every kernel variant behind them"""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(77)
+    methods = ["sum", "sumsq", "abssum", "mean"]
+    seen_not_implemented = 0
+    for it in range(120):
+        rank = int(rng.integers(1, 7))
+        shape = [int(rng.integers(1, 10)) for _ in range(rank)]
+        if rng.random() < 0.5:
+            shape[int(rng.integers(0, rank))] = int(rng.choice([64, 200, 1000, 4096, 20000]))
+        mask = [bool(rng.integers(0, 2)) for _ in range(rank)]
+        if not any(mask):
+            mask[int(rng.integers(0, rank))] = True
+        dims = [i for i, m in enumerate(mask) if m]
+        method = methods[it % 4]
+        x = rng.standard_normal(shape).astype(np.float32)
+        x64 = x.astype(np.float64)
+        term = {"sum": x64, "mean": x64, "sumsq": x64 * x64, "abssum": np.abs(x64)}[method]
+        want = term.mean(axis=tuple(dims), keepdims=True) if method == "mean" else term.sum(axis=tuple(dims), keepdims=True)
+        bound = np.abs(term).sum(axis=tuple(dims), keepdims=True) / (np.prod([shape[d] for d in dims]) if method == "mean" else 1)
+        y = _nan(want.shape)
+        try:
+            dlp.reduction_forward(_dev(x), y, method, dims=dims)
+        except dlp.NotImplementedErrorDlprim:
+            seen_not_implemented += 1  # more than three separate groups of one kind: rank 7 and up only
+            continue
+        got = _host(y)
+        assert np.all(np.abs(got - want) <= 2e-6 * bound + 1e-30), (shape, dims, method)
+    assert seen_not_implemented == 0
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gpu_tensor_ops_on_unaligned_addresses(oracle_mod, dtype):
     """tensors that start one element past a 16-byte address: the kernels fall back to element-wise accesses"""
