@@ -264,6 +264,38 @@ def test_gpu_interpolation_shapes_vs_oracle(oracle_mod, method, align, dtype):
 
 
 @pytest.mark.gpu
+def test_gpu_interpolation_random_sizes(oracle_mod):
+    """80 random input / output sizes (1 to 40 and a few wide ones), planes, methods and explicit factors against the oracle"""
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(88)
+    methods = [("nearest", False), ("nearest-exact", False), ("bilinear", False), ("bilinear", True)]
+    for it in range(80):
+        method, align = methods[it % 4]
+        H, W = int(rng.integers(1, 41)), int(rng.integers(1, 41))
+        if it % 9 == 0:
+            W = int(rng.integers(250, 700))
+        planes = (int(rng.integers(1, 4)), int(rng.integers(1, 6)))
+        x = rng.standard_normal(planes + (H, W)).astype(np.float32)
+        if it % 3 == 0:  # explicit factors: the size is int(in * factor)
+            scale = (float(rng.choice([0.5, 0.75, 1.0, 1.5, 2.0, 3.4])), float(rng.choice([0.5, 0.7, 1.0, 2.0, 3.3])))
+            hw = oracle_mod.interpolate_output_size((H, W), scale=scale)
+            if hw[0] < 1 or hw[1] < 1:
+                continue
+        else:
+            scale = (-1.0, -1.0)
+            hw = (int(rng.integers(1, 50)), int(rng.integers(1, 50)))
+        want = oracle_mod.interpolate2d_forward(x, hw, method=method, scale=scale, align_corners=align)
+        y = _nan(planes + hw)
+        dlp.interpolate2d_forward(_dev(x), y, method, scale[0], scale[1], align)
+        got = _host(y)
+        if method == "bilinear":
+            np.testing.assert_allclose(got, want, err_msg=str((it, method, align, x.shape, hw, scale)), **TOL)
+        else:
+            assert np.array_equal(got, want), (it, method, x.shape, hw, scale)
+
+
+@pytest.mark.gpu
 def test_gpu_reduction_reference_goldens():
     import dlprimitives_amd as dlp
 
