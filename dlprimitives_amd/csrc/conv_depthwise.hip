@@ -5,21 +5,19 @@
 // which covers stride 1 only, and adds stride 2 (the reference falls back to a
 // grouped GEMM with M = 1 there, src/core/conv.cpp:725-727).
 //
-// The op is HBM-bound (about 2 flop per byte), so no matrix cores: the kernel is
-// organised around reading every input element once (plus a two-row halo per strip)
-// and writing every output exactly once, in wide contiguous runs, with enough
-// loads in flight per CU to cover the HBM latency.
-//
-// 3x3 kernel, lanes own output columns.  The (plane, row strip, column) triples of
-// the whole tensor are laid on one flat axis; a wavefront covers 64 consecutive
-// ones.  A lane produces a strip of 7 output rows of its column: it first issues
-// the loads of ALL input rows the strip needs (9 at stride 1, 15 at stride 2), so a
-// wavefront has 9-30 independent loads in flight, then computes.  Each lane loads
-// only the input columns it owns; the columns to its left/right come from the
-// neighbouring lanes through wavefront shuffles.  Lanes at the edge of the
-// wavefront are halo lanes: they load and feed their neighbours but store
-// nothing, and adjacent wavefronts overlap by the halo, so there is no
-// divergent patch-up load.  Accumulation order is the reference's:
+// The op is HBM-bound (about 2 flop per byte), so no matrix cores: every kernel here reads
+// each input element from memory once and writes each output once.  What decides the speed
+// is how early the loads of a launch are on their way and how the requests of one wavefront
+// look to the memory system, not the arithmetic (replacing the 9 multiply-adds by one changes
+// no timing).  Three 3x3 kernels, chosen per shape by depthwise_launch:
+//   * depthwise3x3_reg_kernel   fp32, planes of 28 x 28 and larger: a lane owns IV input columns x 7 output rows, loads
+//                               its 9 (15 at stride 2) input rows straight into registers, all requested before the first
+//                               is used, and gets the column left and right of its own from the neighbouring lanes
+//                               (DPP wavefront shifts): no LDS, no barrier, 32 independent wavefronts per CU.
+//   * depthwise3x3_plane_kernel small planes (and bf16): runs of whole planes through LDS, contiguous 16-byte loads and
+//                               streaming 16-byte stores.
+//   * depthwise3x3_kernel       everything else (unaligned tensors, odd widths at stride 2, planes wider than the others take).
+// Accumulation order is the reference's everywhere:
 // sum = bias; sum = fma(k[dr][dc], x, sum) for dr, dc ascending.
 //
 // Other odd kernel sizes use a plain direct kernel.
@@ -123,6 +121,194 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DwArgs a)
         if (is_out && oy < a.OH)
             store_out(yp + (size_t)oy * a.OW, apply_act(sum, a.act), a.factor);
     }
+}
+
+// ---- 3x3, strips in registers --------------------------------------------------------------------
+// A lane owns IV neighbouring input columns (IV / STRIDE output columns) of a strip of kRegRows output rows of one plane; the
+// ncg = W / IV lanes of a strip sit side by side in a wavefront, which holds spw = 64 / ncg strips (strips are numbered plane by
+// plane, top to bottom, so a wavefront and a workgroup cover one contiguous piece of x and of y).  Every input row of the strip
+// is requested before the first is used (buffer loads: rows above and below the plane and idle lanes are sent out of range and
+// arrive as zeros, so nothing branches), the filter arrives as three 12-byte loads.  The column to the left of a lane's own is the
+// last column of the lane before it, the column to the right (stride 1) the first of the lane after it: one DPP wavefront
+// shift each, replaced by zero at the ends of a row.  HBM traffic is |x| + |y| (the rows two strips share come out of the
+// caches).  Stores are write-back unless a wavefront's share of an output row is a whole run of 128 bytes or more (NT).
+constexpr int kRegRows = 7;
+constexpr uint32_t kDwOutOfRange = 0x80000000u; // >= num_records of every buffer the kernel is given
+
+struct DwRegArgs {
+    const float *x, *w;
+    const float *bias;
+    float *y;
+    uint32_t x_bytes, y_bytes;
+    int C, H, W, OH, OW;
+    int ncg, nrb, spw, nstrips; // lanes per strip, strips per plane, strips per wavefront, strips in all
+    uint32_t ncg_magic, ncg_shift, nrb_magic, nrb_shift, c_magic, c_shift;
+    float factor;
+    int act;
+    float clamp_lo, clamp_hi;
+};
+
+typedef float dw_f32x4 __attribute__((ext_vector_type(4)));
+typedef float dw_f32x3 __attribute__((ext_vector_type(3)));
+typedef float dw_f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int dw_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int dw_u32x2 __attribute__((ext_vector_type(2)));
+
+template <int N>
+__device__ __forceinline__ void dw_load(float *d, __amdgpu_buffer_rsrc_t r, uint32_t v, uint32_t s)
+{
+    if constexpr (N == 4) {
+        const dw_f32x4 t = __builtin_bit_cast(dw_f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, v, s, 0));
+        d[0] = t.x, d[1] = t.y, d[2] = t.z, d[3] = t.w;
+    } else if constexpr (N == 2) {
+        const dw_f32x2 t = __builtin_bit_cast(dw_f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, v, s, 0));
+        d[0] = t.x, d[1] = t.y;
+    } else
+        d[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, v, s, 0));
+}
+template <int N, int AUX>
+__device__ __forceinline__ void dw_store(const float *d, __amdgpu_buffer_rsrc_t r, uint32_t v, uint32_t s)
+{
+    if constexpr (N == 4) {
+        const dw_f32x4 t = {d[0], d[1], d[2], d[3]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(dw_u32x4, t), r, v, s, AUX);
+    } else if constexpr (N == 2) {
+        const dw_f32x2 t = {d[0], d[1]};
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(dw_u32x2, t), r, v, s, AUX);
+    } else
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, d[0]), r, v, s, AUX);
+}
+// lane i receives the value of lane i - 1 / i + 1 (lane 0 / 63: zero)
+__device__ __forceinline__ float dw_from_prev_lane(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dw_from_next_lane(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+
+// ACT: 0 identity, 1 one clamp (ReLU / ReLU6), 2 tanh / sigmoid.  OLDY: y = factor * y + value.  NT: streaming stores.
+template <int STRIDE, int IV, int ACT, bool OLDY, bool NT>
+__global__ __launch_bounds__(256) void depthwise3x3_reg_kernel(DwRegArgs a)
+{
+    constexpr int R = kRegRows;
+    constexpr int OV = IV / STRIDE;
+    constexpr int NIN = (R - 1) * STRIDE + 3;
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int sl = (int)fast_div((uint32_t)lane, a.ncg_magic, a.ncg_shift);
+    const int cg = lane - sl * a.ncg;
+    const int strip = wave * a.spw + sl;
+    const bool active = sl < a.spw && strip < a.nstrips;
+    const int plane = (int)fast_div((uint32_t)strip, a.nrb_magic, a.nrb_shift);
+    const int rb = strip - plane * a.nrb;
+    const int c = plane - (int)fast_div((uint32_t)plane, a.c_magic, a.c_shift) * a.C;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void *)a.y, 0, a.y_bytes, 0x00020000);
+    // row pitches as scalars: the offset of row r is then an SGPR operand of its load, not vector arithmetic
+    const uint32_t w4 = (uint32_t)__builtin_amdgcn_readfirstlane(a.W * 4), ow4 = (uint32_t)__builtin_amdgcn_readfirstlane(a.OW * 4);
+
+    // input rows iy0 - 1 .. iy0 + NIN - 2; row r of the strip exists when 1 <= r <= rows_in (r = 0: when the strip is not the plane's first)
+    const int iy0 = rb * (R * STRIDE);
+    const uint32_t xbase = active ? (uint32_t)((plane * a.H + iy0) * a.W + cg * IV) * 4u : kDwOutOfRange;
+    const int rows_in = a.H - iy0;
+    float v[NIN][IV];
+    dw_load<IV>(v[0], xr, rb > 0 ? xbase - w4 : kDwOutOfRange, 0);
+#pragma unroll
+    for (int r = 1; r < NIN; r++)
+        dw_load<IV>(v[r], xr, (r <= rows_in) ? xbase : kDwOutOfRange, (uint32_t)(r - 1) * w4);
+    float k[9];
+    {
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, (uint32_t)a.C * 36u, 0x00020000);
+        const uint32_t wv = active ? (uint32_t)c * 36u : kDwOutOfRange;
+#pragma unroll
+        for (int dr = 0; dr < 3; dr++) {
+            const dw_f32x3 t = __builtin_bit_cast(dw_f32x3, __builtin_amdgcn_raw_buffer_load_b96(wr, wv, dr * 12, 0));
+            k[3 * dr] = t.x, k[3 * dr + 1] = t.y, k[3 * dr + 2] = t.z;
+        }
+    }
+    // no bias: a buffer of no records, every load of it gives 0
+    const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc((void *)a.bias, 0, a.bias ? (uint32_t)a.C * 4u : 0u, 0x00020000);
+    const float bias = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, active ? (uint32_t)c * 4u : kDwOutOfRange, 0, 0));
+
+    const bool has_left = cg > 0;
+    const bool has_right = cg + 1 < a.ncg;
+    const int oy0 = rb * R;
+    const int rows_out = a.OH - oy0;
+    const uint32_t ybase = active ? (uint32_t)((plane * a.OH + oy0) * a.OW + cg * OV) * 4u : kDwOutOfRange;
+    float old[OLDY ? R : 1][OV];
+    if (OLDY) {
+#pragma unroll
+        for (int j = 0; j < R; j++)
+            dw_load<OV>(old[OLDY ? j : 0], yr, (j < rows_out) ? ybase : kDwOutOfRange, (uint32_t)j * ow4);
+    }
+    float left[3], right[3]; // the columns beside the lane's own, of the three rows of the window
+    auto edge = [&](int r) {
+        const float l = dw_from_prev_lane(v[r][IV - 1]);
+        left[r % 3] = has_left ? l : 0.0f;
+        if (STRIDE == 1) {
+            const float rr = dw_from_next_lane(v[r][0]);
+            right[r % 3] = has_right ? rr : 0.0f;
+        }
+    };
+    // input column j = -1 .. IV of row r
+    auto col = [&](int r, int j) -> float { return j < 0 ? left[r % 3] : (j >= IV ? right[r % 3] : v[r][j]); };
+    edge(0);
+    if (STRIDE == 1)
+        edge(1);
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        if (STRIDE == 1)
+            edge(j + 2);
+        else {
+            edge(2 * j + 1);
+            edge(2 * j + 2);
+        }
+        float out[OV];
+#pragma unroll
+        for (int o = 0; o < OV; o++) {
+            float sum = bias;
+#pragma unroll
+            for (int dr = 0; dr < 3; dr++)
+#pragma unroll
+                for (int dc = 0; dc < 3; dc++)
+                    sum = fmaf(k[3 * dr + dc], col(j * STRIDE + dr, o * STRIDE + dc - 1), sum);
+            if (ACT == 1)
+                sum = clamp_med3(sum, a.clamp_lo, a.clamp_hi);
+            else if (ACT == 2)
+                sum = apply_act(sum, a.act);
+            if (OLDY)
+                sum = fmaf(old[OLDY ? j : 0][o], a.factor, sum);
+            out[o] = sum;
+        }
+        dw_store<OV, NT ? 2 : 0>(out, yr, (j < rows_out) ? ybase : kDwOutOfRange, (uint32_t)j * ow4);
+    }
+}
+
+// Input columns per lane of the register kernel for this geometry, 0: not taken.
+static int reg_columns(const ConvGeom &g, const void *x, const void *y)
+{
+    if (g.KH != 3 || g.KW != 3 || g.dtype != DLP_FLOAT)
+        return 0;
+    const long long xb = (long long)g.B * g.Cin * g.H * g.W * 4, yb = (long long)g.B * g.Cin * g.OH * g.OW * 4;
+    if (xb >= 0x7fffffffLL || yb >= 0x7fffffffLL || (long long)g.B * g.Cin * ((g.OH + kRegRows - 1) / kRegRows) >= 0x7fffffffLL / 64)
+        return 0;
+    const uintptr_t ax = (uintptr_t)x, ay = (uintptr_t)y;
+    if (g.sh == 1) {
+        if (g.W <= 64 && ((ax | ay) & 3) == 0)
+            return 1;
+        if (g.W % 2 == 0 && g.W <= 128 && ((ax | ay) & 7) == 0)
+            return 2;
+        if (g.W % 4 == 0 && g.W <= 256 && ((ax | ay) & 15) == 0)
+            return 4;
+        return 0;
+    }
+    if (g.W % 2 == 0 && g.W <= 128 && (ax & 7) == 0 && (ay & 3) == 0)
+        return 2;
+    if (g.W % 4 == 0 && g.W <= 256 && (ax & 15) == 0 && (ay & 7) == 0)
+        return 4;
+    return 0;
 }
 
 // ---- 3x3, whole planes through LDS ------------------------------------------------------------------
@@ -342,7 +528,8 @@ __global__ __launch_bounds__(kPlaneThreads) void depthwise3x3_plane_kernel(DwPla
             continue;
         const uint4 r = *reinterpret_cast<const uint4 *>(lds_out_raw + (tid + kPlaneThreads * q) * 16);
         if (e0 + EPP <= n_out && a.factor == 0.0f) {
-            *reinterpret_cast<uint4 *>(yg + e0) = r;
+            // streaming store: the run leaves in whole cache lines and is not read again by this launch
+            __builtin_nontemporal_store(dw_u32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<dw_u32x4 *>(yg + e0));
         } else { // y = factor * y + value (reference: depthwise_separable_conv.cl:96-101), and the cut last piece
             T tmp[EPP];
             *reinterpret_cast<uint4 *>(tmp) = r;
@@ -356,7 +543,7 @@ __global__ __launch_bounds__(kPlaneThreads) void depthwise3x3_plane_kernel(DwPla
 
 // Planes per run for this geometry (0: the plane kernel does not take it): as many as fit 16 KB of input and 64 planes,
 // and such that every run starts on a 16-byte boundary in x and in y.
-static int plane_run(const ConvGeom &g)
+static int plane_run(const ConvGeom &g, bool always = false)
 {
     if (g.KH != 3 || g.KW != 3)
         return 0;
@@ -368,7 +555,7 @@ static int plane_run(const ConvGeom &g)
     // strip kernel 47.7 / 51.9 us (C144 at 56 x 56), 19.0 / 21.8, 13.3 / 15.7, 9.0 / 11.5 us at stride 1; 36.3 / 32.9, 13.8 / 15.3,
     // 10.1 / 10.0, 7.6 / 7.7 us at stride 2: with large planes at stride 2 a run holds few tiles (112 for 256 threads) and the strip kernel wins.
     // With bf16 tensors the plane kernel wins throughout (its loads and stores stay 16 bytes wide).
-    if (g.dtype == DLP_FLOAT && g.sh == 2 && in_bytes > 8192)
+    if (g.dtype == DLP_FLOAT && g.sh == 2 && in_bytes > 8192 && !always)
         return 0;
     const long long pmax = std::min<long long>(kPlaneMaxP, kPlaneMaxBytes / in_bytes);
     auto gcd = [](long long x, long long y) {
@@ -442,7 +629,79 @@ int depthwise_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.factor = ep.factor;
     a.act = ep.activation;
     TimingScope ts("sep_conv", stream);
-    const int run = plane_run(g);
+    // DLP_DEPTHWISE_KERNEL = reg | plane | strip pins the 3x3 kernel where it applies (measurements); unset: by shape
+    static const char *pin = getenv("DLP_DEPTHWISE_KERNEL");
+    const bool pin_reg = pin && pin[0] == 'r', pin_plane = pin && pin[0] == 'p', pin_strip = pin && pin[0] == 's';
+    // Measured at batch 64 on cold tensors, register kernel / plane kernel (stride 1; stride 2): 56 x 56 40.0 / 48.2 us (26.3 / 32.8 with
+    // the strip kernel), 28 x 28 16.5 / 17.8 (10.9 / 13.1), 14 x 14 12.0 / 11.5 (8.1 / 9.1), 7 x 7 10.7 / 6.9: planes of 14 x 14 and
+    // smaller at stride 1 and 7 x 7 at stride 2 are too short a run per lane for direct loads and go through LDS.
+    const int iv = (pin_plane || pin_strip) ? 0 : reg_columns(g, x, y);
+    const bool small_plane = g.sh == 1 ? g.H * g.W < 400 : g.H * g.W < 100;
+    if (iv > 0 && (pin_reg || !small_plane)) {
+        DwRegArgs ra;
+        ra.x = (const float *)x;
+        ra.w = (const float *)w;
+        ra.bias = ep.bias;
+        ra.y = (float *)y;
+        ra.x_bytes = (uint32_t)((size_t)a.planes * g.H * g.W * 4);
+        ra.y_bytes = (uint32_t)((size_t)a.planes * g.OH * g.OW * 4);
+        ra.C = g.Cin;
+        ra.H = g.H;
+        ra.W = g.W;
+        ra.OH = g.OH;
+        ra.OW = g.OW;
+        ra.ncg = g.W / iv;
+        ra.nrb = (g.OH + kRegRows - 1) / kRegRows;
+        ra.spw = 64 / ra.ncg;
+        ra.nstrips = a.planes * ra.nrb;
+        make_magic((uint32_t)ra.ncg, ra.ncg_magic, ra.ncg_shift);
+        make_magic((uint32_t)ra.nrb, ra.nrb_magic, ra.nrb_shift);
+        make_magic((uint32_t)ra.C, ra.c_magic, ra.c_shift);
+        ra.factor = ep.factor;
+        ra.act = ep.activation;
+        ra.clamp_lo = 0.0f;
+        ra.clamp_hi = ep.activation == DLP_ACT_RELU6 ? 6.0f : __builtin_huge_valf();
+        const int waves = (ra.nstrips + ra.spw - 1) / ra.spw;
+        const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+        const int act = (ep.activation == DLP_ACT_TANH || ep.activation == DLP_ACT_SIGMOID) ? 2 : (ep.activation == DLP_ACT_IDENTITY ? 0 : 1);
+        const bool oldy = ep.factor != 0.0f;
+        // streaming stores pay when a wavefront's piece of an output row is whole cache lines (one column per lane, rows of 48 floats up)
+        const bool nt = !oldy && iv == 1 && g.sh == 1 && g.OW >= 48;
+        auto launch = [&](auto stride_c, auto iv_c) {
+            constexpr int S = decltype(stride_c)::value, IV = decltype(iv_c)::value;
+            if (oldy) {
+                if (act == 0)
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 0, true, false>), grid, block, 0, stream, ra);
+                else if (act == 1)
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 1, true, false>), grid, block, 0, stream, ra);
+                else
+                    DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 2, true, false>), grid, block, 0, stream, ra);
+            } else if (act == 2)
+                DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 2, false, false>), grid, block, 0, stream, ra);
+            else if (act == 0)
+                DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 0, false, false>), grid, block, 0, stream, ra);
+            else if (nt && S == 1 && IV == 1)
+                DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 1, false, (S == 1 && IV == 1)>), grid, block, 0, stream, ra);
+            else
+                DLP_LAUNCH_TIMED(ts, (depthwise3x3_reg_kernel<S, IV, 1, false, false>), grid, block, 0, stream, ra);
+        };
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I4 = std::integral_constant<int, 4>;
+        if (g.sh == 1 && iv == 1)
+            launch(I1{}, I1{});
+        else if (g.sh == 1 && iv == 2)
+            launch(I1{}, I2{});
+        else if (g.sh == 1)
+            launch(I1{}, I4{});
+        else if (iv == 2)
+            launch(I2{}, I2{});
+        else
+            launch(I2{}, I4{});
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
+    const int run = pin_strip ? 0 : plane_run(g, pin_plane);
     if (run > 0 && (((uintptr_t)x | (uintptr_t)y) & 15) == 0) {
         DwPlaneArgs pa;
         pa.x = x;

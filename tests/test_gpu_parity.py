@@ -404,6 +404,38 @@ def test_depthwise_plane_runs(gpu, oracle_mod, geom, unaligned):
     np.testing.assert_allclose(yd.cpu().numpy(), oracle_mod.apply_factor(want, old, 0.5), **TOL)
 
 
+@pytest.mark.parametrize("geom", [(1, 3, 28, 28, 2), (1, 5, 30, 33, 3), (1, 2, 20, 64, 2), (1, 3, 9, 100, 2), (1, 2, 23, 128, 1), (1, 2, 11, 200, 2),
+                                  (1, 2, 8, 256, 2), (2, 3, 28, 28, 2), (2, 5, 15, 22, 3), (2, 2, 33, 128, 2), (2, 2, 17, 132, 2), (2, 2, 9, 256, 2),
+                                  (2, 7, 14, 14, 5), (1, 70, 7, 64, 1)], ids=lambda g: "s%d_c%d_%dx%d_b%d" % g)
+@pytest.mark.parametrize("act", ["relu6", "identity", "tanh"])
+def test_depthwise_register_strips(gpu, oracle_mod, geom, act):
+    """fp32 3x3 depthwise planes of 400 elements and more (100 at stride 2) are computed in strips of 7 output rows held in
+    registers, one, two or four input columns per lane depending on the width: every width class at both strides, heights that
+    end a strip early, strips per wavefront that do not fill it, a last wavefront with idle strips, no bias, the factor path,
+    and integer-valued tensors, which must come out exact."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    s, ch, h, w_, b = geom
+    c = case(3, 1, s, 1, ch, ch, act != "identity", ch, False)
+    c["activation"] = act
+    x, w, bias = make_tensors(c, (b, h, w_), seed=ch * 1000 + h * w_)
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="depthwise_separable", expect_algo="depthwise_separable")
+    np.testing.assert_allclose(got, want, **TOL)
+    old = np.random.default_rng(2).standard_normal(want.shape).astype(np.float32)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="depthwise_separable", factor=-0.75, y_init=old)
+    np.testing.assert_allclose(got, oracle_mod.apply_factor(want, old, -0.75), **TOL)
+    if act != "tanh":
+        rng = np.random.default_rng(7)
+        xi = rng.integers(-4, 5, size=x.shape).astype(np.float32)
+        wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+        bi = None if bias is None else rng.integers(-5, 6, size=bias.shape).astype(np.float32)
+        got, _ = gpu.run_conv(c, xi, wi, bi, algo="depthwise_separable")
+        assert np.array_equal(got, oracle_conv(oracle_mod, c, xi, wi, bi))
+
+
 # ------------------------------------------------------------ pointwise followers of the depthwise blocks
 @pytest.mark.parametrize("pw", [(144, 24, 56), (144, 32, 28), (192, 32, 28), (192, 64, 14), (384, 64, 14), (384, 96, 14), (960, 160, 7), (960, 320, 7)],
                          ids=lambda p: "%dto%d_at%d" % p)
