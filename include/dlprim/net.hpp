@@ -1082,6 +1082,18 @@ private:
     // A residual sum into the convolution that produces its later branch: the convolution then writes
     // act(conv + bias + coef * other) over the other branch, which must be dead after the sum.
     // Returns the index of that convolution, or -1.
+    // the tensor whose memory `name` shares in the end (views of views, sums written over a branch that is itself a view)
+    std::string alias_root(std::string name) const
+    {
+        for (size_t hops = 0; hops <= alias_of_.size(); hops++) {
+            auto it = alias_of_.find(name);
+            if (it == alias_of_.end())
+                break;
+            name = it->second;
+        }
+        return name;
+    }
+
     int try_fuse_residual(size_t e)
     {
         Node &el = nodes_[e];
@@ -1137,6 +1149,10 @@ private:
             p.conv.stride[0] != 1 || p.conv.stride[1] != 1 || p.conv.pad[0] != 0 || p.conv.pad[1] != 0 || (!p.algo.empty() && p.algo != "gemm"))
             return;
         std::string const &x = d.inputs[0];
+        // a 1x1 node that already carries a residual sum writes over the skip branch: when that branch is the depthwise input
+        // (x -> depthwise -> 1x1 -> + x), the fused kernel would store output rows over input rows that other workgroups still read
+        if (p.residual && (alias_root(p.outputs[0]) == alias_root(x) || std::find(p.inputs.begin() + 1, p.inputs.end(), x) != p.inputs.end()))
+            return;
         for (size_t k = i + 1; k <= size_t(u); k++) // the depthwise input must still hold its value when the 1x1 node runs
             if (!nodes_[k].skipped && std::find(nodes_[k].outputs.begin(), nodes_[k].outputs.end(), x) != nodes_[k].outputs.end())
                 return;
@@ -1250,11 +1266,22 @@ private:
             for (auto const &t : nodes_[i].outputs)
                 last_use[t] = std::max(last_use.count(t) ? last_use[t] : -1, int(i));
         }
-        for (int pass = 0; pass < 2; pass++) // a view and its source live as long as either is used (two passes: views of views)
+        // a network output that shares memory with an intermediate tensor (a view of it, a sum written over it) keeps that memory
+        // for good: no later operator may be given the chunk
+        for (auto const &name : output_names_)
+            if (alias_of_.count(name))
+                last_use[name] = int(nodes_.size());
+        // a view and its source live as long as either is used, along chains of any length
+        for (bool changed = true; changed;) {
+            changed = false;
             for (auto const &al : alias_of_) {
-                const int both = std::max(last_use.count(al.first) ? last_use[al.first] : -1, last_use.count(al.second) ? last_use[al.second] : -1);
-                last_use[al.first] = last_use[al.second] = both;
+                const int a = last_use.count(al.first) ? last_use[al.first] : -1, b = last_use.count(al.second) ? last_use[al.second] : -1;
+                if (a != b) {
+                    last_use[al.first] = last_use[al.second] = std::max(a, b);
+                    changed = true;
+                }
             }
+        }
         tensor_memory_ = 0;
         auto own = [&](std::string const &name) {
             tensors_[name] = Tensor(ctx_, spec(name), int_inputs_.count(name) ? int32_data : dtype_);

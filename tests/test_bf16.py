@@ -295,3 +295,30 @@ def test_resnet50_bf16_logits_vs_fp32_reference(oracle_mod):
         print("resnet50 bf16 vs fp32 reference (sums fused: %s): max relative error of the logits %.4f" % (fuse_residual, rel))
         assert rel <= 1e-2
         assert (got.argmax(1) == want.argmax(1)).all()
+
+
+def test_resnet50_bf16_benchmarked_deployment_logits(oracle_mod):
+    """The form of configuration 5 that bench.py times: batch 128, bf16 storage, algo "gemm", residual sums in the epilogues of
+    the 1x1 convolutions, filters packed once (enqueue_packed).  Images are independent, so 4 of the 128 logit rows are compared
+    with the fp32 reference path run on those 4 images: 1e-2 relative to the largest logit, same arg-max."""
+    import torch
+
+    from dlprimitives_amd import graphs
+    from graph_oracle import run_graph_on_oracle
+
+    ops = graphs.resnet50()
+    params = graphs.random_parameters(ops, seed=11)
+    x = np.random.default_rng(5).standard_normal((128, 3, 224, 224)).astype(np.float32)
+    pick = [0, 41, 86, 127]
+    want = run_graph_on_oracle(oracle_mod, ops, params, np.ascontiguousarray(x[pick]))
+    runner = graphs.GraphRunner(ops, params, x.shape, algo="gemm", dtype="bfloat16", fuse_residual=True, prepack=True)
+    xd = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    first = runner.forward(xd).float().cpu().numpy()
+    again = runner.forward(xd).float().cpu().numpy()  # a second pass over the packed filters and the operators' own counters
+    assert first.shape == (128, want.shape[1])
+    assert np.array_equal(first, again)
+    got = first[pick]
+    rel = np.abs(got - want).max() / np.abs(want).max()
+    print("resnet50 bf16 b128, sums fused, filters packed once: max relative error of 4 logit rows %.4f" % rel)
+    assert rel <= 1e-2
+    assert (got.argmax(1) == want.argmax(1)).all()

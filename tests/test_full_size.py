@@ -76,6 +76,15 @@ def _run_twice(L, x, w, b, algo, batch, bf16=False):
         op.enqueue(xd, wd, bd, y, ws, 0.0)
         torch.cuda.synchronize()
         outs.append(y.float().cpu().numpy())
+    # the same through the entry points a caller with constant filters uses (pack once, enqueue_packed): what the benchmark's
+    # packed configurations and dlprim::Net run; must give the same bits as enqueue
+    packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+    op.pack(wd, packed)
+    for _ in range(2):
+        y = torch.full((batch, L["cout"], L["ohw"], L["ohw"]), float("nan"), dtype=tdt, device="cuda:0")
+        op.enqueue_packed(xd, wd, packed, bd, y, ws, 0.0)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.float().cpu().numpy(), outs[0]), "enqueue_packed differs from enqueue"
     return outs
 
 
@@ -134,3 +143,38 @@ def test_resnet50_layers_batch128_bf16(gpu, name):
     # at the end is applied to the reference as well; identity layers would exceed 256 (the largest range in which
     # bf16 holds every integer) only in the rounding, which both sides do alike
     _check(_r50(name), "gemm", 128, seed=len(name), bf16=True, wmax=1)
+
+
+@pytest.mark.parametrize("name", ["l1_0_1x1_64to256_at56", "l3_1_1x1_256to1024_at14"])
+@pytest.mark.parametrize("bf16", [False, True], ids=["fp32", "bf16"])
+def test_resnet50_residual_epilogue_batch128(gpu, name, bf16):
+    """accumulate_first on two 1x1 layers that end ResNet-50 blocks, at the benchmark's batch: y = relu(conv + bias + y_old) with
+    the skip branch already in y, through enqueue_packed, twice; integer tensors, exact."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA
+
+    L = dict(_r50(name))
+    L["activation"] = "identity"
+    batch = 128
+    x, w, b = _int_tensors(L, batch, seed=len(name) + 7, wmax=1)
+    skip = np.random.default_rng(9).integers(-4, 5, (batch, L["cout"], L["ohw"], L["ohw"])).astype(np.float32)
+    conv_out = _torch_reference(L, x, w, b)
+    want = np.maximum(conv_out + skip, 0.0)
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    if bf16:
+        want = torch.from_numpy(want).to(torch.bfloat16).float().numpy()
+    st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], x.shape, dtype=BFLOAT16_DATA if bf16 else FLOAT_DATA)
+    op = dlp.Conv2DForward.create(st, True, "relu", "gemm")
+    op.accumulate_before_activation(True)
+    xd, wd, bd = torch.from_numpy(x).cuda().to(tdt), torch.from_numpy(w).cuda().to(tdt), torch.from_numpy(b).cuda()
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+    op.pack(wd, packed)
+    for _ in range(2):
+        y = torch.from_numpy(skip).cuda().to(tdt)
+        op.enqueue_packed(xd, wd, packed, bd, y, ws, 1.0)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+        assert np.array_equal(got, want), "max |diff| %g" % np.abs(got - want).max()

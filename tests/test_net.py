@@ -423,6 +423,44 @@ def branching_net():
     return b
 
 
+def depthwise_block_with_skip_net():
+    """x -> depthwise 3x3 (stride 1) -> 1x1 with as many filters as channels -> + x, where x is made by an operator (so the sum may
+    be written over it): the 1x1 node takes the sum into its epilogue, and must then not also take the depthwise layer, whose
+    input it would be overwriting.  A second block whose skip branch is another tensor may fuse both ways."""
+    b = netfile.NetBuilder("data", (2, 16, 28, 28))
+    x = b.conv("data", "x", 32, 1, 1, 0, bias=True, activation="relu")
+    d = b.conv(x, "d", 32, 3, 1, 1, groups=32, bias=True, activation="relu6")
+    p = b.conv(d, "p", 32, 1, 1, 0, bias=True)
+    s = b.eltwise(p, x, "s", "sum", activation="relu")
+    side = b.conv(s, "side", 32, 3, 1, 1, bias=False, activation="relu")
+    d2 = b.conv(s, "d2", 32, 3, 1, 1, groups=32, bias=False, activation="relu")
+    p2 = b.conv(d2, "p2", 32, 1, 1, 0, bias=True)
+    s2 = b.eltwise(side, p2, "s2", "sum")
+    e = b.conv(s2, "e", 8, 3, 2, 1, bias=True, activation="tanh")
+    b.output(e)
+    return b
+
+
+def view_outputs_net():
+    """Network outputs that are views of intermediate tensors (a Reshape, a Flatten of a Squeeze-free chain of three views) with
+    further operators behind them: the memory under the views must not be handed to those operators."""
+    b = netfile.NetBuilder("data", (2, 6, 12, 12))
+    t = b.conv("data", "t", 8, 3, 1, 1, bias=True, activation="relu")
+    r = b.reshape(t, "r", [0, -1])                            # output 1: a view of t
+    u = b.conv(t, "u", 8, 3, 1, 1, bias=True, activation="relu")
+    v1 = b.reshape(u, "v1", [2, 8, 144])
+    v2 = b.reshape(v1, "v2", [2, 8, 12, 12])
+    v3 = b.flatten(v2, "v3")                                  # output 2: a view of a view of a view of u
+    c1 = b.conv(u, "c1", 8, 3, 1, 1, bias=False, activation="relu")
+    c2 = b.conv(c1, "c2", 8, 3, 1, 1, bias=False, activation="relu")
+    c3 = b.conv(c2, "c3", 8, 3, 1, 1, bias=False, activation="relu")
+    c4 = b.conv(c3, "c4", 8, 1, 1, 0, bias=True)
+    b.output(r)
+    b.output(v3)
+    b.output(c4)
+    return b
+
+
 def heads_net(float_labels=True):
     """A Parameter added to the input (broadcast over the batch), Interpolation of all three kinds (by factors, to a size, shrinking,
     with align_corners), Reduction of every method (over the channels, over two separate axes, from an axis on, over everything; axes
@@ -476,6 +514,8 @@ NETS = {
     "heads": (heads_net, 12),
     "heads_int_labels": (lambda: heads_net(False), 13),
     "upsampling": (upsampling_net, 9),
+    "depthwise_block_with_skip": (depthwise_block_with_skip_net, 14),
+    "view_outputs": (view_outputs_net, 15),
     "resnet18_b2_64": (lambda: netfile.resnet18(2, 64, 10), 6),
     "resnet50_b2_64": (lambda: netfile.resnet50(2, 64, 10), 8),
     "mobilenet_v2_b3_64": (lambda: netfile.mobilenet_v2(3, 64, 10), 7),
