@@ -68,7 +68,7 @@ def measured_traffic_bytes(workload, kernel):
             name = ln[:ln.index(" n=")].strip()
             t = ln.split()
             rows.setdefault(section, []).append((name, float(t[t.index("FETCH_SIZE") + 1]), float(t[t.index("WRITE_SIZE") + 1])))
-    copy = [r for r in rows.get("copy", []) if r[0].startswith("copy_f4")]
+    copy = [r for r in rows.get("copy", []) if r[0].startswith(("copy_f4", "stream_kernel<1, 256, false>"))]
     if not copy or copy[0][1] <= 0 or copy[0][2] <= 0:
         return None
     copied_kib = 262144.0  # the calibration run copies 256 MiB per launch
@@ -141,9 +141,11 @@ def matrix_peak_tflops(kernel_name):
 MAIN_SECTION = {"gemm": "conv_gemm", "winograd": "winograd_fused", "depthwise_separable": "sep_conv"}
 
 
-def cpu_baseline(layer_list, images, seed, threads=1):
+def cpu_baseline(layer_list, images, seed, threads=1, runs=3):
     """Oracle (port of the reference CPU path), `images` images through all layers; threads = 1 is the reference's
-    own single-threaded loop over the batch, more threads distribute the (independent) images over OpenMP threads."""
+    own single-threaded loop over the batch, more threads distribute the (independent) images over OpenMP threads.
+    One untimed pass, then the mean of `runs` timed passes (std::chrono around forward in the reference's own flops tool,
+    tools/flops.cpp:594-671; docs/benchmarks/methodology.md:3-6 warms up before it times)."""
     import numpy as np
 
     import oracle
@@ -158,13 +160,15 @@ def cpu_baseline(layer_list, images, seed, threads=1):
         w = (rng.standard_normal((L["cout"], cin_g, L["kernel"], L["kernel"])) * np.sqrt(2.0 / (cin_g * L["kernel"] ** 2))).astype(np.float32)
         b = rng.uniform(-0.1, 0.1, L["cout"]).astype(np.float32)
         cfg = oracle.make_cfg(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"])
-        t0 = time.perf_counter()
-        oracle.conv2d_forward(x, w, b, cfg, L["activation"], threads=threads)
-        total += time.perf_counter() - t0
+        for run in range(-1, runs):
+            t0 = time.perf_counter()
+            oracle.conv2d_forward(x, w, b, cfg, L["activation"], threads=threads)
+            if run >= 0:
+                total += (time.perf_counter() - t0) / runs
         flops += conv_flops(L, images)
     return dict(value=round(images / total, 3), unit="images/s", cores=threads, kind="port",
-                sample="%d images through all %d layers of the workload, %s, %.1f s" % (
-                    images, len(layer_list), "single thread" if threads == 1 else "%d OpenMP threads over the batch" % threads, total),
+                sample="%d images through all %d layers of the workload, %s, 1 untimed + %d timed passes of %.2f s" % (
+                    images, len(layer_list), "single thread" if threads == 1 else "%d OpenMP threads over the batch" % threads, runs, total),
                 gflops_per_s=round(flops / total / 1e9, 2))
 
 
@@ -226,6 +230,7 @@ def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, p
                      "peak": peak, "unit": "TFLOP/s", "frac": round(flops / (conv_ms * 1e-3) / 1e12 / peak, 4) if conv_ms else None,
                      "traffic": None},
         "cpu_baseline": None,
+        "dominant_kernel": dominant,
     }
 
 
@@ -404,11 +409,13 @@ def run_conv_workload(workload, batch, bf16, steps, warmup, prepacked=False, onl
                 kernel_ms_per_step=sum(layer_ms), roofline=roofline, table=table, nl=nl)
 
 
-def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_seconds=0.2):
+def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_seconds=0.2, cached=False):
     """One layer alone: launches back to back, each on its own x / y pair out of a ring larger than the 256 MB last-level
     cache (every launch starts cold, as inside a network), ONE event pair around all of them.  An event between two
     launches makes the first write its part of the L2 back before it ends, which inflates short kernels by microseconds;
-    this is how the plain streaming kernel of the probe (copy_at_size) is timed as well."""
+    this is how the streaming kernels of the probe (copy_at_size) are timed as well.
+    cached=True: a ring of two pairs only, so x and y of every launch still sit in the last-level cache from the launch
+    before last -- the state a small layer finds its input in when the preceding layer has just written it."""
     import torch
 
     import dlprimitives_amd as dlp
@@ -420,7 +427,7 @@ def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_s
     xshape = (batch, L["cin"], L["hw"], L["hw"])
     yshape = (batch, L["cout"], L["ohw"], L["ohw"])
     pair = es * (batch * L["cin"] * L["hw"] ** 2 + batch * L["cout"] * L["ohw"] ** 2)
-    ring = max(3, min(48, ring_bytes // pair + 1))
+    ring = 2 if cached else max(3, min(48, ring_bytes // pair + 1))
     g = torch.Generator(device="cuda").manual_seed(seed)
     xs = [(torch.rand(xshape, device="cuda", generator=g) * 2 - 1).to(tdt) for _ in range(ring)]
     ys = [torch.empty(yshape, dtype=tdt, device="cuda") for _ in range(ring)]
@@ -429,13 +436,38 @@ def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_s
     st = dlp.Conv2DSettings(L["cin"], L["cout"], L["kernel"], L["stride"], 1, L["pad"], L["groups"], xshape, dtype=BFLOAT16_DATA if bf16 else FLOAT_DATA)
     op = dlp.Conv2DForward.create(st, True, L["activation"], L["algo"])
     ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda")
-    reps = 3 * ring
+    reps = 60 if cached else 3 * ring
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t_warm = time.perf_counter()
     while time.perf_counter() - t_warm < warm_seconds:  # untimed launches until the device runs at its working clocks
         for j in range(ring):
             op.enqueue(xs[j], w, b, ys[j], ws, 0.0)
         torch.cuda.synchronize()
+    # One pass over the ring is recorded as a HIP graph and replayed: a launch of a few microseconds is shorter than the
+    # host's path through the Python binding, and the layer would otherwise be timed at the host's launch rate.
+    graph = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for j in range(ring):
+                    op.enqueue(xs[j], w, b, ys[j], ws, 0.0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+    except Exception:  # a layer whose enqueue cannot be captured is timed eagerly
+        graph = None
+        torch.cuda.synchronize()
+    if graph is not None:
+        passes = max(3, reps // ring)
+        graph.replay()
+        e0.record()
+        for _ in range(passes):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (passes * ring)
     for r in range(-ring, reps):
         if r == 0:
             e0.record()
@@ -551,7 +583,7 @@ def compact(r, batch, extra=None):
     return out
 
 
-def other_configs(steps, warmup, peaks):
+def other_configs(steps, warmup, peaks, with_cpu=True):
     """Configurations 1, 3, 4 and 5 of the baseline, each through the same timing as the headline (fewer steps)."""
     import torch
 
@@ -563,6 +595,8 @@ def other_configs(steps, warmup, peaks):
     small = dict(steps=max(steps, 200), warmup=warmup, warm_seconds=0.3)
     r = run_conv_workload("single", 16, False, **small)
     cfgs["config1_single_conv_b16"] = compact(r, 16, {"steps": small["steps"], "warm_seconds": 0.3})
+    if with_cpu:  # the whole layer at its own batch, one thread: the reference's CPU path as it is built
+        cfgs["config1_single_conv_b16"]["cpu_baseline"] = cpu_baseline(r["layer_list"], 16, 2024)
     # the headline's stack again as a caller with constant filters runs it (dlp_conv2d_fwd_pack once, _enqueue_packed per step):
     # what the packing launches inside the headline's timed step cost
     r = run_conv_workload("resnet18", 64, False, steps, warmup, prepacked=True, warm_seconds=0.3)
@@ -571,6 +605,8 @@ def other_configs(steps, warmup, peaks):
         r = run_conv_workload(wl, 64, False, **small)
         cfgs["config3_%s" % wl.replace("-", "_")] = compact(r, 64, {"layers": [
             {k: row[k] for k in ("name", "ms", "main_kernel_ms", "tflops", "tflops_issued", "frac_of_roofline", "kernel") if k in row} for row in r["table"]]})
+        if with_cpu and wl == "winograd":  # both shapes, 16 of the 64 images each (images are independent), one thread
+            cfgs["config3_winograd"]["cpu_baseline"] = cpu_baseline(r["layer_list"], 16, 2024)
     r = run_conv_workload("mobilenet", 64, False, max(steps, 100), warmup, warm_seconds=0.3)
     rows = []
     for L, row in zip(r["layer_list"], r["table"]):
@@ -587,21 +623,25 @@ def other_configs(steps, warmup, peaks):
         if L["algo"] == "depthwise_separable":
             # bandwidth-bound: against the vendor's 8 TB/s, and against a plain streaming kernel that reads |X| and
             # writes |Y| of this very layer, timed the same way
-            gbs, cus = probe.copy_at_size(xb, yb)
+            forms, best = probe.stream_forms(xb, yb)
+            cus = forms[best]
             e["bound"] = "hbm"
             e["frac_of_hbm_peak"] = round(e["gbs"] / HBM_PEAK_GBS, 4)
-            e["copy_same_size_us"] = round(cus, 2)
-            e["copy_same_size_gbs"] = round(gbs, 1)
-            e["frac_of_copy_same_size"] = round(cus / us, 4)
+            e["tuned_copy_us"] = round(cus, 2)
+            e["tuned_copy_gbs"] = round((xb + yb) / cus / 1e3, 1)
+            e["tuned_copy_form"] = best
+            e["frac_of_tuned_copy"] = round(cus / us, 4)
+            if xb + yb < 100e6:  # small tensors: also with x and y still in the last-level cache, as behind a producer
+                e["us_tensors_in_last_level_cache"] = round(isolated_layer_us(L, 64, cached=True), 2)
         else:
             ai = flops / (xb + yb + wb)
             roof = min(FP32_MATRIX_PEAK_TFLOPS * 1e12, ai * HBM_PEAK_GBS * 1e9)
             e["bound"] = "mfma" if ai * HBM_PEAK_GBS * 1e9 >= FP32_MATRIX_PEAK_TFLOPS * 1e12 else "hbm"
             e["frac_of_roofline"] = round(flops / (us * 1e-6) / roof, 4)
-            # what a launch of this size costs at the least on this chip: a plain streaming kernel over the same |X| and |Y|
+            # what a launch of this size costs at the least on this chip: the tuned streaming kernel over the same |X| and |Y|
             gbs, cus = probe.copy_at_size(xb, yb)
             e["roofline_us"] = round(flops / roof * 1e6, 2)
-            e["copy_same_size_us"] = round(cus, 2)
+            e["tuned_copy_us"] = round(cus, 2)
         rows.append(e)
     dw = [e for e in rows if "frac_of_hbm_peak" in e]
     pw = [e for e in rows if "frac_of_hbm_peak" not in e]
@@ -621,19 +661,30 @@ def other_configs(steps, warmup, peaks):
             gbs, cus = probe.copy_at_size(xb, yb)
             e.update({"fused": True, "kernel": "conv_dwpw_f32_kernel", "us": round(us, 2), "speedup": round(e["separate_us"] / us, 3), "bound": "hbm",
                       "gbs": round((xb + yb + wb) / us / 1e3, 1), "frac_of_hbm_peak": round((xb + yb + wb) / us / 1e3 / HBM_PEAK_GBS, 4),
-                      "copy_same_size_us": round(cus, 2), "frac_of_copy_same_size": round(cus / us, 4)})
+                      "tuned_copy_us": round(cus, 2), "frac_of_tuned_copy": round(cus / us, 4)})
         pairs.append(e)
     fused_ms, nfused = mobilenet_fused_pass_ms(64, max(steps, 100), warmup)
     cfgs["config4_mobilenet_blocks_b64"] = compact(r, 64, {
-        "depthwise_min_frac_of_hbm_peak": min(e["frac_of_hbm_peak"] for e in dw), "depthwise_min_frac_of_copy_same_size": min(e["frac_of_copy_same_size"] for e in dw),
+        "depthwise_min_frac_of_hbm_peak": min(e["frac_of_hbm_peak"] for e in dw), "depthwise_min_frac_of_tuned_copy": min(e["frac_of_tuned_copy"] for e in dw),
         "pointwise_min_frac_of_roofline": min(e["frac_of_roofline"] for e in pw), "layers": rows,
         "ms_per_step_with_fused_pairs": round(fused_ms, 4), "fused_pairs_in_step": nfused, "fused_pairs": pairs})
+    if with_cpu:  # all 16 layers, 16 of the 64 images, one thread
+        cfgs["config4_mobilenet_blocks_b64"]["cpu_baseline"] = cpu_baseline(r["layer_list"], 16, 2024)
     del r
     torch.cuda.empty_cache()
     # an inference deployment, as dlprim::Net runs the same network: the residual sums run in the epilogue of the 1x1 convolution
     # that produces their later branch and the filters are transformed once (--workload resnet50-full --fuse-residual
     # --prepacked; without the flags the sums are operators of their own and every enqueue transforms its filter)
     cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True, prepack=True)
+    if with_cpu:
+        # the fp32 reference path on the 53 convolutions of the network (99 % of its arithmetic), 16 of the 128 images
+        # spread over the host cores the box gives a GPU
+        from dlprimitives_amd.workloads import RESNET50_CONVS
+
+        nthreads = max(1, min(16, os.cpu_count() or 1))
+        cfgs["config5_resnet50_full_bf16_b128"]["cpu_baseline"] = cpu_baseline(RESNET50_CONVS, nthreads, 2024, threads=nthreads, runs=3)
+    # HBM bytes per launch of the kernel with the largest share of the pass (from the tracked counter summary)
+    cfgs["config5_resnet50_full_bf16_b128"]["roofline"]["traffic"] = measured_traffic_bytes("resnet50-bf16", cfgs["config5_resnet50_full_bf16_b128"].get("dominant_kernel", ""))
     return cfgs
 
 
@@ -742,7 +793,7 @@ def main():
     if headline and not args.no_configs:
         del r
         torch.cuda.empty_cache()
-        out["configs"] = other_configs(max(5, args.steps // 2), max(2, args.warmup // 2), peaks)
+        out["configs"] = other_configs(max(5, args.steps // 2), max(2, args.warmup // 2), peaks, with_cpu=args.cpu_images > 0)
         out["configs"]["config2_resnet18_conv_stack_b64"] = "the headline of this line: value, ms_per_step, roofline, layers"
     print(json.dumps(out))
 

@@ -1,7 +1,10 @@
-"""Device peak probes: fp32 MFMA throughput (no memory traffic) and streaming-copy
-bandwidth, from libdlp_microbench.so.  They put the roofline fractions of the
-convolution kernels in context (nominal peaks: 157.3 TFLOP/s fp32 matrix, 8 TB/s HBM)
-and give the hardware-counter runs a copy kernel of known size to be scaled by.
+"""Device peak probes: fp32 / bf16 MFMA throughput (no memory traffic) and streaming bandwidth, from libdlp_microbench.so.
+They put the roofline fractions of the convolution kernels in context (nominal peaks: 157.3 TFLOP/s fp32 matrix, 2.5 PFLOP/s
+bf16 matrix, 8 TB/s HBM) and give the hardware-counter runs a copy kernel of known size to be scaled by.
+
+The streaming probe times several forms of a copy / read / write kernel (one 16-byte piece per thread, several pieces with
+non-temporal accesses, 1024-thread workgroups, the untuned grid-stride loop, hipMemcpyAsync) on tensors of a given size, every
+launch cold (a ring of buffers larger than the last-level cache), and reports the fastest kernel form: the "tuned copy".
 
     python -m dlprimitives_amd.probe [--copy-mb 256] [--no-mfma]
 """
@@ -12,11 +15,35 @@ import os
 
 
 def _lib():
-    return ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "libdlp_microbench.so"))
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "libdlp_microbench.so"))
+    lib.dlp_probe_stream_forms.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
+    lib.dlp_probe_stream_form_name.restype = ctypes.c_char_p
+    return lib
+
+
+def stream_forms(in_bytes, out_bytes):
+    """{form name: microseconds per launch} of every streaming form that reads in_bytes and writes out_bytes, and the name of the
+    fastest kernel form"""
+    lib = _lib()
+    n = lib.dlp_probe_stream_form_count()
+    us = (ctypes.c_double * n)()
+    best = ctypes.c_int(-1)
+    if lib.dlp_probe_stream_forms(int(in_bytes), int(out_bytes), us, ctypes.byref(best)) != 0:
+        raise RuntimeError("streaming probe failed")
+    names = [lib.dlp_probe_stream_form_name(i).decode() for i in range(n)]
+    return {names[i]: us[i] for i in range(n) if us[i] > 0}, names[best.value]
+
+
+def copy_at_size(in_bytes, out_bytes):
+    """(GB/s, microseconds per launch) of the tuned copy: the fastest streaming kernel form that reads in_bytes and writes
+    out_bytes, launches back to back on cold tensors"""
+    forms, best = stream_forms(in_bytes, out_bytes)
+    us = forms[best]
+    return (in_bytes + out_bytes) / us / 1e3, us
 
 
 def measured_peaks(big_mb=2048):
-    """MFMA-only loops and streaming copies on this device: what the chip reaches with no convolution around it."""
+    """MFMA-only loops and streaming kernels on this device: what the chip reaches with no convolution around it."""
     lib = _lib()
     v = ctypes.c_double()
     out = {}
@@ -27,31 +54,24 @@ def measured_peaks(big_mb=2048):
                 raise RuntimeError(name + " probe failed")
             best = max(best, v.value)
         out[name] = round(best, 1)
-    if lib.dlp_probe_copy(256, ctypes.byref(v)) != 0:
-        raise RuntimeError("copy probe failed")
-    out["copy_256mib_gbs"] = round(v.value, 1)
-    if big_mb and lib.dlp_probe_copy(big_mb, ctypes.byref(v)) == 0:
-        out["copy_%dmib_gbs" % big_mb] = round(v.value, 1)
+    for mb in (256, big_mb):
+        if not mb:
+            continue
+        b = mb << 20
+        gbs, _ = copy_at_size(b, b)
+        out["copy_%dmib_gbs" % mb] = round(gbs, 1)
+    b = (big_mb or 256) << 20
+    out["read_%dmib_gbs" % (b >> 20)] = round(copy_at_size(b, 0)[0], 1)
+    out["write_%dmib_gbs" % (b >> 20)] = round(copy_at_size(0, b)[0], 1)
     return out
-
-
-def copy_at_size(in_bytes, out_bytes):
-    """(GB/s, microseconds per launch) of a plain streaming kernel that reads in_bytes and writes out_bytes, every launch
-    timed by its own event pair and starting cold (a ring of buffers larger than the last-level cache)."""
-    lib = _lib()
-    lib.dlp_probe_copy_sized.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
-    gbs, us = ctypes.c_double(), ctypes.c_double()
-    if lib.dlp_probe_copy_sized(int(in_bytes), int(out_bytes), ctypes.byref(gbs), ctypes.byref(us)) != 0:
-        raise RuntimeError("sized copy probe failed")
-    return gbs.value, us.value
 
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--copy-mb", type=int, default=256, help="MiB per direction of the copy kernel")
+    ap.add_argument("--copy-mb", type=int, default=256, help="MiB per direction of the copy kernels")
     ap.add_argument("--no-mfma", action="store_true")
     args = ap.parse_args()
-    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "libdlp_microbench.so"))
+    lib = _lib()
     out = {}
     v = ctypes.c_double()
     if not args.no_mfma:
@@ -63,19 +83,18 @@ def main():
             if lib.dlp_probe_mfma_bf16(waves, ctypes.byref(v)) != 0:
                 raise SystemExit("bf16 MFMA probe failed")
             out["mfma_bf16_tflops_%dwave_per_simd" % waves] = round(v.value, 1)
-    if lib.dlp_probe_copy(args.copy_mb, ctypes.byref(v)) != 0:
-        raise SystemExit("copy probe failed")
-    out["copy_gbs_read_plus_write"] = round(v.value, 1)
-    out["copy_bytes_per_launch_each_direction"] = args.copy_mb << 20
+    b = args.copy_mb << 20
+
+    def table(i, o):
+        forms, best = stream_forms(i, o)
+        return {"gbs": {k: round((i + o) / us / 1e3, 1) for k, us in forms.items()}, "best": best}
+
+    out["copy_%dmib" % args.copy_mb] = table(b, b)
     if not args.no_mfma:
-        # tensors far above the 256 MB last-level cache: what HBM itself sustains
-        big = 2048
-        if lib.dlp_probe_copy(big, ctypes.byref(v)) == 0:
-            out["copy_gbs_%dmb" % big] = round(v.value, 1)
-        if lib.dlp_probe_stream(big, 0, ctypes.byref(v)) == 0:
-            out["read_gbs_%dmb" % big] = round(v.value, 1)
-        if lib.dlp_probe_stream(big, 1, ctypes.byref(v)) == 0:
-            out["write_gbs_%dmb" % big] = round(v.value, 1)
+        big = 2048 << 20  # tensors far above the 256 MB last-level cache: what HBM itself sustains
+        out["copy_2048mib"] = table(big, big)
+        out["read_2048mib"] = table(big, 0)
+        out["write_2048mib"] = table(0, big)
     print(json.dumps(out))
 
 

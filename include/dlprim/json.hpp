@@ -257,11 +257,16 @@ private:
             case 't': s += '\t'; break;
             case 'u': {
                 unsigned cp = parse_hex4(t, pos);
-                if (cp >= 0xD800 && cp < 0xDC00 && pos + 1 < t.size() && t[pos] == '\\' && t[pos + 1] == 'u') {
+                if (cp >= 0xD800 && cp < 0xDC00) { // a high surrogate must be followed by a low one (the reference's utf16 decoder, src/json.cpp:215-229)
+                    if (!(pos + 1 < t.size() && t[pos] == '\\' && t[pos + 1] == 'u'))
+                        fail(t, pos, "unpaired surrogate");
                     pos += 2;
                     unsigned lo = parse_hex4(t, pos);
+                    if (lo < 0xDC00 || lo > 0xDFFF)
+                        fail(t, pos, "unpaired surrogate");
                     cp = 0x10000 + ((cp - 0xD800) << 10) + (lo - 0xDC00);
-                }
+                } else if (cp >= 0xDC00 && cp <= 0xDFFF)
+                    fail(t, pos, "unpaired surrogate");
                 append_utf8(s, cp);
                 break;
             }
