@@ -962,6 +962,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 // Register sets of tiles in flight (2 or 4).  Measured: 4 sets (two more K steps of load latency
 // hidden, 148 instead of 102 VGPRs) are not faster -- the kernel is bound by the vector-memory
 // access rate, not by latency -- so 2 sets and three workgroups per CU it is.
+#ifndef DLP_BF16_STORE_AUX
+#define DLP_BF16_STORE_AUX 2 // 2 = non-temporal: whole-line output runs that this launch does not read again stream past the L2 (64->256 at 56x56, batch 128: 74 -> 54 us)
+#endif
 #ifndef DLP_BF16_NSET
 #define DLP_BF16_NSET 2
 #endif
@@ -1119,7 +1122,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                         if constexpr (PXV == 8) {
                             u32x4 o;
                             o[0] = mine[0], o[1] = mine[1], o[2] = mine[2], o[3] = mine[3];
-                            __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff[u], 0, 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(o, yr, voff[u], 0, DLP_BF16_STORE_AUX);
                         } else if constexpr (PXV == 4) {
                             u32x2 o;
                             o[0] = mine[0], o[1] = mine[1];
@@ -1135,7 +1138,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
                 const uint32_t voff = run_offset(q);
                 const unsigned char *src = run_source(q);
                 if constexpr (PXV == 8)
-                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)src, yr, voff, 0, DLP_BF16_STORE_AUX);
                 else if constexpr (PXV == 4)
                     __builtin_amdgcn_raw_buffer_store_b64(*(const u32x2 *)src, yr, voff, 0, 0);
                 else

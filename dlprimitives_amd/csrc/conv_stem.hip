@@ -595,19 +595,6 @@ constexpr int kStemR = 8, kStemPitch = 240;
 
 bool generic_activation(int act) { return act == DLP_ACT_TANH || act == DLP_ACT_SIGMOID; }
 
-int stem_cu_count()
-{
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
-
 } // namespace
 
 bool conv_stem_supported(const ConvGeom &g)
@@ -652,7 +639,7 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     if (total > 0x7fffffffLL - 65536)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     // one workgroup per CU walks a contiguous range of output rows in bands of up to R rows
-    const int wgs = (int)std::min<long long>(stem_cu_count(), (total + 1) / 2);
+    const int wgs = (int)std::min<long long>(dlp_cu_count(), (total + 1) / 2);
     a.total_rows = (int)total;
     a.rows_per_wg = (int)((total + wgs - 1) / wgs);
     a.x_img_bytes = (uint32_t)((size_t)g.Cin * g.H * g.W * esize);

@@ -6,6 +6,8 @@
 // fallback: every compute entry launches a device kernel or fails.
 #include "dlp_internal.hpp"
 
+#include <atomic>
+
 #include <algorithm>
 
 #include <cstdlib>
@@ -70,15 +72,19 @@ TimingScope::~TimingScope()
 
 int dlp_cu_count()
 {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
+    // per device: every GPU of a process may be a different part
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cus[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus[dev].store(n, std::memory_order_relaxed);
     }
-    return cus;
+    return n;
 }
 
 void TimingScope::kernel(const void *host_function)

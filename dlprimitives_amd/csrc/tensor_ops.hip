@@ -88,6 +88,8 @@ __global__ __launch_bounds__(256) void interpolate_nearest_kernel(InterpArgs a, 
 // Bilinear: a lane owns one output column of a strip of kInterpStripRows output rows of one plane.  The column's two source columns
 // and weights are fixed; going down the strip the lane keeps the horizontally blended values of the two source rows and loads a
 // source row only when the strip moves onto it (going up by 2, five source rows serve eight output rows: 10 loads instead of 32).
+// Order of the arithmetic: horizontal blend of each source row, then the vertical blend of the two results -- the reference's kernel
+// adds four taps each weighted by a product (src/kernels/interpolate_2d.cl:111-140), so results agree to rounding, not bit for bit.
 constexpr int kInterpStripRows = 8;
 template <class T>
 __global__ __launch_bounds__(256) void interpolate_bilinear_kernel(InterpArgs a, const T *__restrict__ x, T *__restrict__ y)

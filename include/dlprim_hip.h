@@ -263,8 +263,11 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
  * 4 MiB of partial sums (4 KiB per tile of 32 outputs x 32 batch rows and K slice): enough for 2048 -> 1000 at
  * batch 128 (3.5 MiB) or 25088 -> 4096 at batch 16 (4 MiB).  A batch x outputs that needs more is a validation
  * error that names both sizes (e.g. 1024 -> 4096 at batch 160: 5 MiB); bfloat16 rows of odd length are
- * NotImplemented.  All calls on one device share the array: two calls that overlap on one device (different
- * streams, or two threads) race; calls on one stream do not. */
+ * NotImplemented.
+ * RULE: at most one call in flight per device.  All calls on one device share the array, whatever the operator: two
+ * calls that overlap on one device (different streams, two threads, two recorded graphs replayed side by side) race on
+ * the counters and partial sums, and nothing detects it; calls on one stream, or replays of graphs on one stream, are
+ * ordered by the stream and do not. */
 #define DLP_IP_NO_ALLOC_SCRATCH_BYTES (4 * 1024 * 1024 + 64 * 1024)
 int dlp_ip_fwd_enqueue_no_alloc(dlp_ip_fwd *op, int batch, const void *x, const void *w,
                                 const void *bias, void *y, void *stream);
@@ -334,7 +337,9 @@ int dlp_channel_affine_fwd_enqueue(int dtype, int activation, int batch, int cha
  * method as dlprim::InterpolateType (include/dlprim/definitions.hpp:325-329).  scale_y / scale_x <= 0: the steps follow from the
  * sizes; otherwise tgt = int(src * scale) is checked.  nearest: source index min(int((p + offset) * step), src - 1) with offset 0,
  * or 0.5 for nearest-exact; bilinear: source position max(step * (p + 0.5) - 0.5, 0), or p * (src - 1) / (tgt - 1) with
- * align_corners, and the two neighbours weighted by the fraction. */
+ * align_corners, and the two neighbours weighted by the fraction.  Bilinear blends along the row first and then between the two
+ * rows, where the reference's kernel sums four weighted taps (src/kernels/interpolate_2d.cl:111-140): same value to within a few
+ * ulp, not the same bits; nearest picks the reference's pixel exactly. */
 #define DLP_INTERPOLATE_NEAREST 0
 #define DLP_INTERPOLATE_NEAREST_EXACT 1
 #define DLP_INTERPOLATE_BILINEAR 2

@@ -383,7 +383,9 @@ def interpolate2d_forward(x, out_hw, method="nearest", scale=(-1.0, -1.0), align
     """Interpolation::forward on the CPU, src/ops/interpolation.cpp: nearest / nearest-exact as forward_cpu (:271-305: source index
     min(int((p + offset) * step), size - 1), offset 0 or 0.5, step float(1 / scale) or float(in) / out), bilinear as
     bilinear_fwd_bwd_cpu with HandleFWD (:86-96,133-195: position max(step * (p + 0.5) - 0.5, 0) or step * p with align_corners,
-    neighbours p0 and p0 + 1 (clamped), weights from the fraction), all in float32."""
+    neighbours p0 and p0 + 1 (clamped), weights from the fraction), all in float32.  The HIP bilinear kernel blends along the row
+    and then between rows, this restatement follows the reference's four weighted taps: tests compare the two to a tolerance
+    (nearest is compared bit for bit)."""
     x = _f32(x)
     B, C, H, W = x.shape
     OH, OW = out_hw

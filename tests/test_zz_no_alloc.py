@@ -105,3 +105,38 @@ def test_sizes_beyond_the_array_are_rejected(gpu):
         op.enqueue_no_alloc(x, w, None, y)
     op.enqueue(x, w, None, y)  # the allocating entry point takes it
     torch.cuda.synchronize()
+
+
+def test_recorded_into_a_hip_graph_and_replayed(gpu):
+    """What the entry point is for: the call is recorded into a HIP graph (it allocates nothing and records no memset: its
+    counters are cleared by a kernel) and the graph is replayed, with eager work and synchronizations between the replays and on
+    inputs that change between them; every replay must equal dlp_ip_fwd_enqueue on the same inputs bit for bit."""
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    rng = np.random.default_rng(21)
+    batch, inputs, outputs = 64, 2048, 1000
+    op = dlp.IPForward.create(dlp.IPSettings(inputs, outputs, batch), True, "relu")
+    x, w, b = _tensors(rng, batch, inputs, outputs)
+    xd, wd, bd = gpu.dev(x), gpu.dev(w), gpu.dev(b)
+    got = torch.full((batch, outputs), float("nan"), device="cuda:0")
+    op.enqueue_no_alloc(xd, wd, bd, got)  # one eager call first (module load, the array's address)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            op.enqueue_no_alloc(xd, wd, bd, got)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        xn = rng.uniform(-1, 1, x.shape).astype(np.float32)
+        xd.copy_(torch.from_numpy(xn))  # the graph holds the pointer, not the values
+        got.fill_(float("nan"))
+        want = torch.full_like(got, float("nan"))
+        op.enqueue(xd, wd, bd, want)  # eager work of the program's own between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), want.cpu().numpy()), "replay %d" % replay
