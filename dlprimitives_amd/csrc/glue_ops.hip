@@ -259,6 +259,15 @@ __device__ __forceinline__ float eltwise_one(float x0, float x1, int op, float c
     return apply_act(r, act);
 }
 
+// Measured inside whole networks (ResNet-50 at batch 64, fp32: the 16 sums 0.75 -> 0.65 ms): one 16-byte pack per thread in a grid
+// as large as the tensor (a capped grid walks the tensor with a power-of-two stride, which keeps a workgroup on the same memory
+// channels) and non-temporal accesses on both sides (bit 0: loads, bit 1: stores).
+#ifndef ELT_NT
+#define ELT_NT 3
+#endif
+#ifndef ELT_ONESHOT
+#define ELT_ONESHOT 1
+#endif
 // 16 bytes per thread and step (4 floats or 8 bf16) over the 16-byte aligned body [0, n16 * VEC);
 // the last n - n16 * VEC elements are done one by one by the first threads.
 template <class T>
@@ -272,13 +281,24 @@ __global__ __launch_bounds__(256) void eltwise_kernel(size_t n, int op, float c1
     const size_t n16 = n / VEC;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
+    typedef unsigned int elt_u32x4 __attribute__((ext_vector_type(4)));
     for (size_t k = i; k < n16; k += stride) {
-        const Pack pa = ((const Pack *)a)[k], pb = ((const Pack *)b)[k];
+        Pack pa, pb;
+        if (ELT_NT & 1) {
+            *(elt_u32x4 *)&pa = __builtin_nontemporal_load((const elt_u32x4 *)a + k);
+            *(elt_u32x4 *)&pb = __builtin_nontemporal_load((const elt_u32x4 *)b + k);
+        } else {
+            pa = ((const Pack *)a)[k];
+            pb = ((const Pack *)b)[k];
+        }
         Pack pc;
 #pragma unroll
         for (int e = 0; e < VEC; e++)
             store_plain(&pc.v[e], eltwise_one(to_float(pa.v[e]), to_float(pb.v[e]), op, c1, c2, act));
-        ((Pack *)c)[k] = pc;
+        if (ELT_NT & 2)
+            __builtin_nontemporal_store(*(const elt_u32x4 *)&pc, (elt_u32x4 *)c + k);
+        else
+            ((Pack *)c)[k] = pc;
     }
     for (size_t k = n16 * VEC + i; k < n; k += stride)
         store_plain(c + k, eltwise_one(to_float(a[k]), to_float(b[k]), op, c1, c2, act));
@@ -785,6 +805,10 @@ static int eltwise_launch(int dtype, int operation, float coef1, float coef2, in
         blocks = 256 * 32;
     TimingScope ts("eltwise", (hipStream_t)stream);
     const bool aligned = (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) == 0;
+    if (ELT_ONESHOT && aligned) {
+        const size_t packs = n / (dtype == DLP_FLOAT ? 4 : 8);
+        blocks = std::min<size_t>(std::max<size_t>(1, (packs + 255) / 256), (size_t)1 << 22);
+    }
     hipStream_t st = (hipStream_t)stream;
     if (dtype == DLP_BFLOAT16) {
         if (aligned)
