@@ -37,6 +37,7 @@
 #include "dlp_internal.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 
 namespace dlp {
@@ -655,7 +656,14 @@ __device__ __forceinline__ void static_for_n(F &&f)
     static_for_seq<N>(f, std::make_integer_sequence<int, N>{});
 }
 
-template <class T, int KH, int KW, int PITCH, int ACT>
+// STRIDE 2 (3x3, pad 1): the pixels under the taps of 64 consecutive output pixels are still one run of consecutive input pixels
+// per image -- from the first output pixel's top-left tap to the last one's bottom-right tap -- only four times as long per
+// output (up to 9 input rows of 56 for 64 outputs on 28 columns: rows of 512); a lane's taps sit at 2 * (its pixel) in that run.
+// Two such patch buffers would be 64 KB and leave two workgroups per CU, which costs more than the patch saves (measured: no
+// faster than the gathering kernel), so the strided instantiation keeps ONE patch buffer (40 KB with the A tiles, three workgroups
+// per CU): the next stage's patch waits in registers and is stored in the stage's last K tile, after the barrier behind which
+// nobody reads the buffer any more, followed by a second barrier before the next stage's first operands are read.
+template <class T, int KH, int KW, int PITCH, int ACT, int STRIDE = 1>
 __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
 {
     constexpr int BM = 64, BN = 64, WM = 2, WN = 2, KHW = KH * KW;
@@ -665,9 +673,11 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     constexpr int MAXSEG = 3;       // images a tile may touch (H*W >= 32)
     constexpr int ZERO_ROW = PITCH - 1; // never loaded: reads 0 in every channel
     static_assert(PITCH % 64 == 0 && BK == 16, "patch shape");
+    constexpr bool SINGLE = STRIDE != 1; // one patch buffer
+    constexpr int NPB = SINGLE ? 1 : 2;
 
     __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
-    __shared__ float Ps[2][BK][PITCH];
+    __shared__ float Ps[NPB][BK][PITCH];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -731,7 +741,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const int m0 = mt * BM, n0 = nt * BN;
 
     // ---- the tile's patch: one segment of consecutive plane pixels per image (wavefront-uniform) ----
-    const int HW = a.OHW;
+    const int HW = a.OHW;                            // pixels of an output plane
+    const int HWI = STRIDE == 1 ? HW : a.H * a.W;    // ... of an input plane
     const int halo = a.ph * a.W + a.pw;
     const int n_last = min(n0 + BN, a.N) - 1;
     const int b0 = (int)fast_div((uint32_t)n0, a.ohw_magic, a.ohw_shift);
@@ -744,8 +755,16 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
             const int first = max(n0, base), last = min(n_last, base + HW - 1);
             int as = 0, len = 0;
             if (first <= last) {
-                as = max(0, first - base - halo);
-                len = min(HW, last - base + 1 + halo) - as;
+                if (STRIDE == 1) {
+                    as = max(0, first - base - halo);
+                    len = min(HW, last - base + 1 + halo) - as;
+                } else { // from the top-left tap of the first output pixel to the bottom-right tap of the last one
+                    const int pf = first - base, pl = last - base;
+                    const int oyf = (int)fast_div((uint32_t)pf, a.ow_magic, a.ow_shift), oyl = (int)fast_div((uint32_t)pl, a.ow_magic, a.ow_shift);
+                    const int oxf = pf - oyf * a.OW, oxl = pl - oyl * a.OW;
+                    as = max(0, (oyf * STRIDE - a.ph) * a.W + oxf * STRIDE - a.pw);
+                    len = min(HWI, (oyl * STRIDE - a.ph + KH - 1) * a.W + oxl * STRIDE - a.pw + KW) - as;
+                }
             }
             seg_row[s] = row;
             seg_a[s] = as;
@@ -763,7 +782,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         for (int s = 0; s < MAXSEG; s++) {
             const int d = rho - seg_row[s];
             if (d >= 0 && d < seg_len[s])
-                v = (uint32_t)((((b0 + s) * a.Cin + g * a.Cin_g) * HW + seg_a[s] + d) * (int)sizeof(T));
+                v = (uint32_t)((((b0 + s) * a.Cin + g * a.Cin_g) * HWI + seg_a[s] + d) * (int)sizeof(T));
         }
         pvoff[q] = v;
     }
@@ -777,12 +796,12 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         const int oy = (int)fast_div((uint32_t)pix, a.ow_magic, a.ow_shift);
         const int ox = pix - oy * a.OW;
         const int s = b - b0;
-        const int row = pix + (s == 0 ? seg_row[0] - seg_a[0] : s == 1 ? seg_row[1] - seg_a[1] : seg_row[2] - seg_a[2]);
+        const int row = (STRIDE == 1 ? pix : (oy * a.W + ox) * STRIDE) + (s == 0 ? seg_row[0] - seg_a[0] : s == 1 ? seg_row[1] - seg_a[1] : seg_row[2] - seg_a[2]);
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
 #pragma unroll
             for (int kx = 0; kx < KW; kx++) {
-                const int yy = oy + ky - a.ph, xx = ox + kx - a.pw;
+                const int yy = oy * STRIDE + ky - a.ph, xx = ox * STRIDE + kx - a.pw;
                 const bool ok = vn && yy >= 0 && yy < a.H && xx >= 0 && xx < a.W;
                 const int r = ok ? row + (ky - a.ph) * a.W + (kx - a.pw) : ZERO_ROW;
                 baddr[ky * KW + kx] = (uint32_t)((h * PITCH + r) * 4);
@@ -810,12 +829,12 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     auto load_patch = [&](int j, uint32_t stage_soff) { // j = channel-in-wavefront * QS + row slot
         preg[j] = buf_load<T>(xr, pvoff[j % QS], stage_soff + (uint32_t)(j / QS) * a.hw4);
     };
-    auto store_patch = [&](auto buf_c, int j) { Ps[decltype(buf_c)::value][wave * CPW + j / QS][lane + 64 * (j % QS)] = preg[j]; };
+    auto store_patch = [&](auto buf_c, int j) { Ps[SINGLE ? 0 : decltype(buf_c)::value][wave * CPW + j / QS][lane + 64 * (j % QS)] = preg[j]; };
     // operands kk of the K tile (A buffer ABUF, patch buffer PB, tap TAP) into operand set OS
     auto read_operands = [&](auto os_c, auto abuf_c, auto pb_c, auto tap_c, int kk) {
         constexpr int OS = decltype(os_c)::value;
         fa[OS][kk] = As[decltype(abuf_c)::value][2 * kk + h][wm * 32 + l32];
-        fb[OS][kk] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(&Ps[decltype(pb_c)::value][0][0]) +
+        fb[OS][kk] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(&Ps[SINGLE ? 0 : decltype(pb_c)::value][0][0]) +
                                                       baddr[decltype(tap_c)::value] + 2 * kk * PITCH * 4);
     };
 
@@ -849,13 +868,25 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
                 for (int j = 0; j < NPL; j++) {
                     if (TAU == 0 && j % (BK / 2) == kk)
                         load_patch(j, next_soff);
-                    if (TAU == KHW - 1 && j / 4 == kk) // before the barrier
+                    if (!SINGLE && TAU == KHW - 1 && j / ((NPL + 3) / 4) == kk) // before the barrier
+                        store_patch(OtherP{}, j);
+                    // one buffer: behind the barrier of the stage's last K tile nobody reads it any more (that tile's operands were
+                    // read during the tile before)
+                    if (SINGLE && TAU == KHW - 1 && (kk == 4 || kk == 5) && j / (NPL / 2) == kk - 4)
                         store_patch(OtherP{}, j);
                 }
                 acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[BUF][kk], fb[BUF][kk], acc[0][0], 0, 0, 0);
                 if (kk == 3)
                     __syncthreads();
-                if (kk >= 4) {
+                if (SINGLE && TAU == KHW - 1) {
+                    if (kk == 5)
+                        __syncthreads(); // the next stage's patch is in place
+                    if (kk >= 6) {
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            read_operands(NextOps{}, NextBuf{}, NextPatch{}, NextTap{}, 4 * (kk - 6) + q);
+                    }
+                } else if (kk >= 4) {
                     read_operands(NextOps{}, NextBuf{}, NextPatch{}, NextTap{}, 2 * (kk - 4));
                     read_operands(NextOps{}, NextBuf{}, NextPatch{}, NextTap{}, 2 * (kk - 4) + 1);
                 }
@@ -868,7 +899,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     {
-        static_assert(NPL <= 12, "patch stores of the last tile fit before its barrier");
+        static_assert(NPL <= 32, "patch loads and stores are dealt over the steps of a K tile");
         const uint32_t soff0 = (uint32_t)(cb_begin * BK + wave * CPW) * a.hw4;
 #pragma unroll
         for (int j = 0; j < NPL; j++)
@@ -2454,6 +2485,34 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
 // the prologue), every one with the same number of (tile, stage) units, but no fewer than 4
 // stages per workgroup.
 constexpr int kPatchWgsPerCu = 3;
+constexpr int kPatchWgsPerCuStrided = 3;
+constexpr int kPatchPitchStrided = 512;
+// Longest patch (input pixels of all the images a tile touches) of a 64-pixel tile of a stride-2 3x3 pad-1 convolution: the
+// kernel's own segment arithmetic, run over every position a tile can have inside a plane.
+static int strided_patch_rows(const ConvGeom &g)
+{
+    const int ohw = g.OH * g.OW, hwi = g.H * g.W;
+    if (ohw > (1 << 16))
+        return 1 << 30;
+    int worst = 0;
+    for (int nt = 0; nt < ohw; nt++) { // n0 = 64 nt takes every residue modulo the plane that a tile start can have
+        const long long n0 = 64ll * nt, n_last = n0 + 63;
+        const long long b0 = n0 / ohw;
+        int total = 0;
+        for (int s = 0; s < 3; s++) {
+            const long long base = (b0 + s) * ohw;
+            const long long first = std::max(n0, base), last = std::min(n_last, base + ohw - 1);
+            if (first > last)
+                continue;
+            const int pf = (int)(first - base), pl = (int)(last - base);
+            const int oyf = pf / g.OW, oxf = pf % g.OW, oyl = pl / g.OW, oxl = pl % g.OW;
+            const int as = std::max(0, (oyf * 2 - 1) * g.W + oxf * 2 - 1);
+            total += std::min(hwi, (oyl * 2 - 1 + 2) * g.W + oxl * 2 - 1 + 3) - as;
+        }
+        worst = std::max(worst, total);
+    }
+    return worst;
+}
 int device_cu_count() { return dlp_cu_count(); }
 struct PatchShape {
     long long tiles, units;
@@ -2466,7 +2525,7 @@ PatchShape patch_shape(const ConvGeom &g, const GemmPlan &p, long long N)
     ps.tiles = (long long)p.mtiles * ((N + 63) / 64) * g.groups;
     ps.units = ps.tiles * (p.nkt / (g.KH * g.KW));
     long long grid = ps.units / 4;
-    const long long slots = (long long)device_cu_count() * kPatchWgsPerCu;
+    const long long slots = (long long)device_cu_count() * (g.sh == 1 ? kPatchWgsPerCu : kPatchWgsPerCuStrided);
     grid = grid < 1 ? 1 : grid > slots ? slots : grid;
     ps.grid = (int)grid;
     ps.cnt_bytes = (size_t)((ps.tiles * sizeof(int) + 255) / 256 * 256);
@@ -2524,7 +2583,18 @@ int launch_patch(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStream_t 
     make_magic((uint32_t)(a.sk_mb * a.ntiles), a.mbnt_magic, a.mbnt_shift);
     make_magic((uint32_t)a.sk_mb, a.mb_magic, a.mb_shift);
     TimingScope ts("conv_gemm", stream);
-    DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+    if (g.sh == 2) { // the shortest rows that hold the longest patch: fewer (empty) loads and LDS stores per stage
+        const int rows = strided_patch_rows(g);
+        if (rows < 320)
+            DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, 320, ACT_CLAMP, 2>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+        else if (rows < 384)
+            DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, 384, ACT_CLAMP, 2>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+        else if (rows < 448)
+            DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, 448, ACT_CLAMP, 2>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+        else
+            DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, kPatchPitchStrided, ACT_CLAMP, 2>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
+    } else
+        DLP_LAUNCH_TIMED(ts, (conv_patch_f32_kernel<float, 3, 3, kPatchPitch, ACT_CLAMP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
@@ -2598,6 +2668,14 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
     // stride-1 3x3 "same" convolutions whose 64-pixel patch fits the LDS rows (W <= 62): LDS-patch kernel
     p.patch = g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && p.tile == 0 && g.KH == 3 && g.KW == 3 && g.sh == 1 && g.sw == 1 &&
               g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 && g.H * g.W >= 32 && 64 + 2 * (g.W + 1) < kPatchPitch;
+    // ... and stride-2 ones (3x3, pad 1) whose longest patch fits rows of 512, from 128 input channels on.  Measured alone on cold
+    // tensors at batch 64, patch / gathering kernel with the packing launch: 128->256 at 28x28 77 / 89-94 us, 256->512 at 14x14 76 / 81-83,
+    // 64->128 at 56x56 92-96 / 88-91: with four stages per tile the set-up of the long patch is not paid back.
+    // (DLP_NO_STRIDED_PATCH in the environment keeps every strided layer on the gathering kernel, for measurements.)
+    static const bool no_strided_patch = getenv("DLP_NO_STRIDED_PATCH") != nullptr;
+    if (!no_strided_patch && g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && p.tile == 0 && g.KH == 3 && g.KW == 3 && g.sh == 2 && g.sw == 2 &&
+        g.dh == 1 && g.dw == 1 && g.ph == 1 && g.pw == 1 && g.OH * g.OW >= 32 && cin_g >= 128 && strided_patch_rows(g) < kPatchPitchStrided)
+        p.patch = 1;
     if (g.dtype == DLP_BFLOAT16 && !generic_act(activation)) { // bf16 matrix instruction
         const bool tap_major = small_kernel && cin_g % BK2 == 0;
         p.order = tap_major ? GEMM_ORDER_TAP_BF16 : GEMM_ORDER_CHANNEL_BF16;

@@ -139,6 +139,45 @@ def test_patch_kernel_stream_k(gpu, oracle_mod, shape):
     np.testing.assert_allclose(got_f, oracle_mod.apply_factor(want, old, 0.5), **TOL)
 
 
+# 3x3 stride-2 pad-1 convolutions with Cin/groups % 16 == 0 and Cout/groups > 32 run the same kernel on patch rows of 512:
+# (batch, cin, cout, groups, H, W)
+STRIDED_PATCH_SHAPES = [
+    (3, 128, 128, 1, 56, 56),  # patch rows of 448: tiles inside an image ...
+    (5, 128, 256, 1, 28, 28),  # ... rows of 384
+    (9, 256, 512, 1, 14, 14),  # ... rows of 320, tiles across two and three images
+    (3, 256, 128, 2, 9, 11),   # odd sizes (the last column and row have no right / lower neighbour), groups
+    (2, 128, 64, 1, 17, 33),   # odd sizes, tiles crossing rows at every offset
+    (2, 144, 80, 1, 12, 112),  # wide rows (512), 9 stages, Cout off the tile size
+    (1, 128, 40, 1, 64, 64),
+    (3, 64, 128, 1, 56, 56),   # fewer than 128 input channels: the gathering kernel
+    (4, 128, 64, 1, 8, 8),     # output plane below 32 pixels: the gathering kernel
+    (2, 128, 64, 1, 6, 300),   # patch longer than the rows: the gathering kernel
+]
+
+
+@pytest.mark.parametrize("shape", STRIDED_PATCH_SHAPES, ids=lambda s: "b%d_%dto%d_g%d_%dx%d" % s)
+def test_strided_patch_kernel(gpu, oracle_mod, shape):
+    b, cin, cout, groups, h, w_ = shape
+    c = case(3, 1, 2, 1, cin, cout, True, groups, True)
+    x, w, bias = make_tensors(c, (b, h, w_), seed=b * 1000 + cin + h)
+    print("strided patch case", shape, flush=True)
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+    again, _ = gpu.run_conv(c, x, w, bias, algo="gemm")
+    assert np.array_equal(got, again)
+    old = np.random.default_rng(5).standard_normal(want.shape).astype(np.float32)
+    got_f, _ = gpu.run_conv(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got_f, oracle_mod.apply_factor(want, old, 0.5), **TOL)
+    # integer-valued tensors: exact whatever the order of the sum
+    rng = np.random.default_rng(13)
+    xi = rng.integers(-3, 4, size=x.shape).astype(np.float32)
+    wi = rng.integers(-2, 3, size=w.shape).astype(np.float32)
+    bi = rng.integers(-5, 6, size=bias.shape).astype(np.float32)
+    got_i, _ = gpu.run_conv(c, xi, wi, bi, algo="gemm")
+    assert np.array_equal(got_i, oracle_conv(oracle_mod, c, xi, wi, bi))
+
+
 def test_patch_kernel_integer_exact_and_small_workspace(gpu):
     # integer-valued tensors: every summation order gives the same fp32 result, so pieces that
     # were mis-addressed, dropped or added twice cannot hide behind a tolerance.  The same op is
