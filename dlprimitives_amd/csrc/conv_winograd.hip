@@ -31,6 +31,7 @@
 //     stores the 2x2 outputs; consecutive lanes hold consecutive tiles of a row.
 #include "dlp_internal.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace dlp {
@@ -130,9 +131,13 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v)
 // NLOAD > 0 : the input rows that the 32 tiles of the workgroup touch are first copied to LDS
 //             with coalesced loads (NLOAD elements per thread and chunk, each input element
 //             once) and the patches are gathered from there; used when those rows fit.
-template <class T, bool TAIL, int NLOAD>
+// NOB: blocks of 32 output channels per workgroup.  The input transform of a (channel, tile) is the same work whatever the number of
+// output channels it is multiplied into, and it shares issue cycles with the matrix pipe: with two blocks every transformed value
+// feeds twice the matrix instructions (8 per wavefront and element pair instead of 4), at 128 accumulator registers per lane.
+template <class T, bool TAIL, int NLOAD, int NOB = 1>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void wino_fused_kernel(WinoArgs a)
 {
+    constexpr int NTW = NT * NOB; // output channels per workgroup
     // main loop: V[buffer][e][c in chunk][tile]; epilogue: M[e][n in pass][tile]
     __shared__ float lds[2 * 16 * KC * TT];
     static_assert(2 * 16 * KC * TT == 16 * (NT / 2) * TT, "the epilogue reuses the V buffers");
@@ -155,7 +160,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const int xcd = bid & 7, slot = bid >> 3;
         id = (xcd < r) ? xcd * (q + 1) + slot : r * (q + 1) + (xcd - r) * q + slot;
     }
-    const int n0 = (id % a.nblocks) * NT;
+    const int n0 = (id % a.nblocks) * NTW;
     const int t0 = (id / a.nblocks) * TT;
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
@@ -331,29 +336,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     // ---- A operand: U[e][chunk][k half][n][k pair]: one 16-byte load per lane = the operands
     //      of the four k pairs of a chunk; lane = (k half h, channel l32), e = 4*wave + ei ----
     const uint32_t u_voff = (uint32_t)(h * a.Npad + l32) * 16u;
-    f32x4 A[2][4];
+    f32x4 A[2][4][NOB];
     auto load_u = [&](auto set, int chunk) {
         constexpr int S = decltype(set)::value;
         const int ch = min(chunk, last);
 #pragma unroll
         for (int ei = 0; ei < 4; ei++) {
             const uint32_t soff = (uint32_t)((((4 * wave + ei) * a.nchunks + ch) * 2) * a.Npad + n0) * 16u;
-            A[S][ei] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ur, u_voff, soff, 0));
+#pragma unroll
+            for (int ob = 0; ob < NOB; ob++)
+                A[S][ei][ob] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ur, u_voff, soff + (uint32_t)(ob * NT * 16), 0));
         }
     };
 
-    f32x16 acc[4];
+    f32x16 acc[4][NOB];
 #pragma unroll
     for (int ei = 0; ei < 4; ei++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[ei][r] = 0.0f;
+        for (int ob = 0; ob < NOB; ob++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[ei][ob][r] = 0.0f;
 
     // bias of the four output channels this thread finishes in the epilogue (fetched now, so
     // that the epilogue does not wait on memory)
-    float bias_v[4];
+    float bias_v[4 * NOB];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < 4 * NOB; i++) {
         const int n = n0 + (i >> 1) * (NT / 2) + (tid >> 5) + 8 * (i & 1);
         bias_v[i] = (a.bias && n < a.N) ? a.bias[n] : 0.0f;
     }
@@ -385,7 +394,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int j = 0; j < KC / 2; j++)
 #pragma unroll
             for (int ei = 0; ei < 4; ei++)
-                acc[ei] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[BUF][ei][j], Bv[ei][j], acc[ei], 0, 0, 0);
+#pragma unroll
+                for (int ob = 0; ob < NOB; ob++)
+                    acc[ei][ob] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[BUF][ei][ob][j], Bv[ei][j], acc[ei][ob], 0, 0, 0);
         __syncthreads();
     };
 
@@ -421,13 +432,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     // accumulator register r of a 32x32 block holds row (channel) 8*(r/4) + 4*h + r%4, column (tile) l32
     T *const ybase = (T *)a.y;
 #pragma unroll
-    for (int pass = 0; pass < 2; pass++) {
+    for (int pass = 0; pass < 2 * NOB; pass++) { // 16 output channels per pass
 #pragma unroll
         for (int ei = 0; ei < 4; ei++)
 #pragma unroll
             for (int r8 = 0; r8 < 8; r8++) {
                 const int nl = 8 * (r8 >> 2) + 4 * h + (r8 & 3); // channel inside the pass, 0..15
-                lds[((4 * wave + ei) * (NT / 2) + nl) * TT + l32] = acc[ei][8 * pass + r8];
+                lds[((4 * wave + ei) * (NT / 2) + nl) * TT + l32] = acc[ei][pass >> 1][8 * (pass & 1) + r8];
             }
         __syncthreads();
 #pragma unroll
@@ -496,7 +507,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 }
             }
         }
-        if (pass == 0)
+        if (pass + 1 < 2 * NOB)
             __syncthreads();
     }
 }
@@ -528,7 +539,10 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
     a.Cpad = plan.Cpad;
     a.Npad = plan.Npad;
     a.nchunks = plan.Cpad / KC;
-    a.nblocks = plan.Npad / NT;
+    // two blocks of 32 output channels per workgroup where the channel count allows (DLP_WINO_NOB=1 in the environment: one, for measurements)
+    static const bool one_block = getenv("DLP_WINO_NOB") != nullptr && atoi(getenv("DLP_WINO_NOB")) == 1;
+    const int nob = (plan.Npad % (2 * NT) == 0 && !one_block) ? 2 : 1;
+    a.nblocks = plan.Npad / (NT * nob);
     make_magic((uint32_t)a.tpi, a.tpi_magic, a.tpi_shift);
     make_magic((uint32_t)a.tw, a.tw_magic, a.tw_shift);
     a.u_bytes = (uint32_t)(16u * (size_t)plan.Cpad * plan.Npad * sizeof(float));
@@ -552,10 +566,14 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
         const bool tail = (g.Cin % KC) != 0;
 #define DLP_WINO_LAUNCH(NL)                                                                                          \
     do {                                                                                                             \
-        if (tail)                                                                                                    \
-            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, true, NL>), dim3(grid), dim3(kThreads), 0, stream, a);        \
+        if (tail && nob == 2)                                                                                        \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, true, NL, 2>), dim3(grid), dim3(kThreads), 0, stream, a);     \
+        else if (tail)                                                                                               \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, true, NL, 1>), dim3(grid), dim3(kThreads), 0, stream, a);     \
+        else if (nob == 2)                                                                                           \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, false, NL, 2>), dim3(grid), dim3(kThreads), 0, stream, a);    \
         else                                                                                                         \
-            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, false, NL>), dim3(grid), dim3(kThreads), 0, stream, a);       \
+            DLP_LAUNCH_TIMED(ts, (wino_fused_kernel<T, false, NL, 1>), dim3(grid), dim3(kThreads), 0, stream, a);    \
     } while (0)
         if (plan.stage_loads == 8)
             DLP_WINO_LAUNCH(8);
