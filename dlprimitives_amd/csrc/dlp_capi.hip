@@ -511,11 +511,12 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     const GemmPlan gplan = conv_gemm_plan(g, activation);
     const bool bf16_mfma = gplan.order >= GEMM_ORDER_TAP_BF16;
     // Where the reference rule would pick Winograd (src/core/conv.cpp:714-718), the automatic choice here keeps "gemm" for the layers
-    // the LDS-patch kernel serves with fewer than 128 input channels.  Whole layers at batch 64, weights transformed in the call,
-    // cold tensors, gemm / winograd: 64->64 at 56x56 126 / 130 us, 128->128 at 28x28 120 / 114 us, 256->256 at 14x14 120 / 107 us,
-    // 512->512 at 7x7 122 / 105 us: Winograd's transforms cost a fixed amount per pixel and channel, the multiplications they save
-    // grow with the channel count.
-    const bool gemm_faster = gplan.patch && cfg->channels_in / cfg->groups < 128;
+    // the LDS-patch kernel serves with fewer than 128 input channels, unless the Winograd kernel can give a workgroup 64 output
+    // channels (a multiple of 64 filters, at least 64 input channels).  Whole layers at batch 64, weights transformed in the call, cold
+    // tensors, gemm / winograd: 64->64 at 56x56 150 / 125 us, 128->128 at 28x28 129 / 108, 256->256 at 14x14 123 / 97, 512->512 at 7x7
+    // 124 / 113; with 32 output channels per workgroup (filter counts off 64) Winograd took 130 us on 64->64 at 56x56 and lost there.
+    const int cin_g = cfg->channels_in / cfg->groups;
+    const bool gemm_faster = gplan.patch && cin_g < 128 && !(cfg->channels_out % 64 == 0 && cin_g >= 64);
     if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && !gemm_faster && cfg->channels_in >= 8 && cfg->channels_out >= 8))
         chosen = ALGO_WINOGRAD;
     else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))

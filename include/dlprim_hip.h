@@ -125,7 +125,9 @@ int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4
  *      place: a Winograd-compatible fp32 convolution with fewer than 128 input
  *      channels that the LDS-patch GEMM kernel serves (image at most 62 wide,
  *      Cin a multiple of 16, more than 32 filters) stays "gemm", which is the
- *      faster of the two there on gfx950; algo() reports what was chosen. ------ */
+ *      faster of the two there on gfx950 -- except with at least 64 input channels
+ *      and a multiple of 64 filters, where Winograd wins again; algo() reports
+ *      what was chosen. ------ */
 int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activation,
                           const char *algo, dlp_conv2d_fwd **out);
 

@@ -338,9 +338,11 @@ def test_algorithm_selection_rules(gpu):
     c33 = case(3, 1, 1, 1, 16, 16, False, 1, False)
     assert algo(c33, 8, "") == "winograd" and algo(c33, 8, "auto") == "winograd" and algo(c33, 8, "gemm") == "gemm"
     assert algo(case(3, 1, 1, 1, 4, 16, False, 1, False), 8, "") == "gemm"  # < 8 channels: not recommended
-    big = case(3, 1, 1, 1, 64, 64, False, 1, False)  # LDS-patch kernel, fewer than 128 input channels: the automatic choice keeps the GEMM
+    big = case(3, 1, 1, 1, 48, 96, False, 1, False)  # LDS-patch kernel, fewer than 128 input channels: the automatic choice keeps the GEMM
     assert algo(big, 28, "") == "gemm" and algo(big, 28, "auto") == "gemm" and algo(big, 28, "winograd") == "winograd"
     assert algo(big, 112, "") == "winograd"  # too wide for the patch rows: Winograd against the gathering GEMM
+    assert algo(case(3, 1, 1, 1, 64, 96, False, 1, False), 28, "") == "gemm"      # filters off 64: 32 output channels per workgroup
+    assert algo(case(3, 1, 1, 1, 64, 64, False, 1, False), 28, "") == "winograd"  # 64 channels in, a multiple of 64 out: Winograd again
     assert algo(case(3, 1, 1, 1, 128, 128, False, 1, False), 28, "") == "winograd"
     assert algo(case(3, 1, 1, 1, 4, 16, False, 1, False), 8, "winograd") == "winograd"
     assert algo(case(3, 1, 2, 1, 16, 16, False, 1, False), 8, "winograd") == "gemm"  # incompatible -> silent gemm
