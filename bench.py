@@ -446,28 +446,29 @@ def isolated_layer_us(L, batch, bf16=False, ring_bytes=768 << 20, seed=7, warm_s
     # One pass over the ring is recorded as a HIP graph and replayed: a launch of a few microseconds is shorter than the
     # host's path through the Python binding, and the layer would otherwise be timed at the host's launch rate.
     graph = None
+    per_graph = max(ring, 24)  # launches per replay: a replay has a start-up cost of its own, which two launches would not amortise
     try:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
-                for j in range(ring):
-                    op.enqueue(xs[j], w, b, ys[j], ws, 0.0)
+                for j in range(per_graph):
+                    op.enqueue(xs[j % ring], w, b, ys[j % ring], ws, 0.0)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
     except Exception:  # a layer whose enqueue cannot be captured is timed eagerly
         graph = None
         torch.cuda.synchronize()
     if graph is not None:
-        passes = max(3, reps // ring)
+        passes = max(3, reps // per_graph)
         graph.replay()
         e0.record()
         for _ in range(passes):
             graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / (passes * ring)
+        return e0.elapsed_time(e1) * 1e3 / (passes * per_graph)
     for r in range(-ring, reps):
         if r == 0:
             e0.record()
