@@ -539,9 +539,7 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
     a.Cpad = plan.Cpad;
     a.Npad = plan.Npad;
     a.nchunks = plan.Cpad / KC;
-    // two blocks of 32 output channels per workgroup where the channel count allows (DLP_WINO_NOB=1 in the environment: one, for measurements)
-    static const bool one_block = getenv("DLP_WINO_NOB") != nullptr && atoi(getenv("DLP_WINO_NOB")) == 1;
-    const int nob = (plan.Npad % (2 * NT) == 0 && !one_block) ? 2 : 1;
+    const int nob = winograd_blocks_per_workgroup(g, plan);
     a.nblocks = plan.Npad / (NT * nob);
     make_magic((uint32_t)a.tpi, a.tpi_magic, a.tpi_shift);
     make_magic((uint32_t)a.tw, a.tw_magic, a.tw_shift);
@@ -588,6 +586,27 @@ int launch_typed(const ConvGeom &g, const WinoPlan &plan, const void *x, const v
 }
 
 } // namespace
+
+// Blocks of 32 output channels per workgroup: two halve the input transforms per flop but also the number of workgroups, so
+// only where that still leaves one and a half workgroups per compute unit (measured on the ResNet-18 shapes at batch 16 / 32 / 64:
+// 392 workgroups of two blocks beat 784 of one by 11-13 %, 196-256 of two lose 6-40 % to twice as many of one).
+// DLP_WINO_NOB=1 / 2 in the environment pins the choice, for measurements.
+int winograd_blocks_per_workgroup(const ConvGeom &g, const WinoPlan &plan)
+{
+    if (plan.Npad % (2 * NT) != 0)
+        return 1;
+    static const int pin = getenv("DLP_WINO_NOB") != nullptr ? atoi(getenv("DLP_WINO_NOB")) : 0;
+    if (pin == 1 || pin == 2)
+        return pin;
+    return winograd_workgroups(g, plan, 2) * 2 >= 3ll * dlp_cu_count() ? 2 : 1;
+}
+
+// Workgroups of the fused kernel for a batch that fits one launch, with nob blocks of 32 output channels each
+long long winograd_workgroups(const ConvGeom &g, const WinoPlan &plan, int nob)
+{
+    const long long tiles = (long long)g.B * ((g.H + 1) / 2) * ((g.W + 1) / 2);
+    return (tiles + TT - 1) / TT * (plan.Npad / (NT * nob));
+}
 
 bool winograd_supported(const ConvGeom &g)
 {

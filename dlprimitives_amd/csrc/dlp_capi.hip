@@ -510,13 +510,19 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     // Winograd (whose transforms force fp32 matrix instructions): automatic choice keeps gemm
     const GemmPlan gplan = conv_gemm_plan(g, activation);
     const bool bf16_mfma = gplan.order >= GEMM_ORDER_TAP_BF16;
-    // Where the reference rule would pick Winograd (src/core/conv.cpp:714-718), the automatic choice here keeps "gemm" for the layers
-    // the LDS-patch kernel serves with fewer than 128 input channels, unless the Winograd kernel can give a workgroup 64 output
-    // channels (a multiple of 64 filters, at least 64 input channels).  Whole layers at batch 64, weights transformed in the call, cold
-    // tensors, gemm / winograd: 64->64 at 56x56 150 / 125 us, 128->128 at 28x28 129 / 108, 256->256 at 14x14 123 / 97, 512->512 at 7x7
-    // 124 / 113; with 32 output channels per workgroup (filter counts off 64) Winograd took 130 us on 64->64 at 56x56 and lost there.
+    // Where the reference rule would pick Winograd (src/core/conv.cpp:714-718), the automatic choice here keeps "gemm" for layers that
+    // the LDS-patch kernel serves and that (a) have fewer than 64 input channels, or fewer than 128 with a filter count off 64 (the
+    // Winograd kernel then gives a workgroup 32 output channels: 130 against 126 us on 64->64 at 56x56, batch 64), or (b) leave the
+    // Winograd kernel fewer than one and a half workgroups per compute unit at the batch of the settings.  Whole layers, weights
+    // transformed in the call, cold tensors, gemm / winograd, at batch 64: 64->64 at 56x56 150 / 125 us, 128->128 at 28x28 129 / 108,
+    // 256->256 at 14x14 123 / 97, 512->512 at 7x7 124 / 105; at batch 16: 49 / 40, 45 / 39, 47 / 46 (200 workgroups), 48 / 77 (128).
     const int cin_g = cfg->channels_in / cfg->groups;
-    const bool gemm_faster = gplan.patch && cin_g < 128 && !(cfg->channels_out % 64 == 0 && cin_g >= 64);
+    bool gemm_faster = false;
+    if (gplan.patch && win) {
+        const WinoPlan wp = winograd_plan(g);
+        const long long wgs = winograd_workgroups(g, wp, winograd_blocks_per_workgroup(g, wp));
+        gemm_faster = cin_g < 64 || (cin_g < 128 && cfg->channels_out % 64 != 0) || wgs * 2 < 3ll * dlp_cu_count();
+    }
     if ((al == "winograd" && win) || (auto_algo && win && !bf16_mfma && !gemm_faster && cfg->channels_in >= 8 && cfg->channels_out >= 8))
         chosen = ALGO_WINOGRAD;
     else if ((al == "depthwise_separable" && dsc) || (auto_algo && dsc))

@@ -239,6 +239,10 @@ struct WinoPlan {
 };
 bool winograd_supported(const ConvGeom &g);
 WinoPlan winograd_plan(const ConvGeom &g);
+// Workgroups of the fused kernel for the batch of g (when it fits one launch) with nob blocks of 32 output channels per workgroup,
+// and the nob a launch takes (two where that leaves enough workgroups for the chip)
+long long winograd_workgroups(const ConvGeom &g, const WinoPlan &plan, int nob);
+int winograd_blocks_per_workgroup(const ConvGeom &g, const WinoPlan &plan);
 // mode: filter transform and convolution, the transform alone (into ws), or the convolution on a ws transformed earlier
 enum { WINO_FILTER_AND_RUN = 0, WINO_FILTER_ONLY = 1, WINO_RUN_ONLY = 2 };
 int winograd_launch(const ConvGeom &g, const WinoPlan &plan, const void *x, const void *w, void *y, void *ws, size_t ws_bytes,

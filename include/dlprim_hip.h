@@ -122,12 +122,13 @@ int dlp_conv2d_output_shape(const dlp_conv2d_settings *cfg, const int in_shape[4
  *      "depthwise_separable"; a requested but incompatible algorithm falls back
  *      to "gemm" exactly as the reference does (:725-727).  The automatic
  *      choice ("" / "auto") differs from the reference's rule (:714-718) in one
- *      place: a Winograd-compatible fp32 convolution with fewer than 128 input
- *      channels that the LDS-patch GEMM kernel serves (image at most 62 wide,
- *      Cin a multiple of 16, more than 32 filters) stays "gemm", which is the
- *      faster of the two there on gfx950 -- except with at least 64 input channels
- *      and a multiple of 64 filters, where Winograd wins again; algo() reports
- *      what was chosen. ------ */
+ *      place: a Winograd-compatible fp32 convolution that the LDS-patch GEMM
+ *      kernel serves (image at most 62 wide, Cin a multiple of 16, more than 32
+ *      filters) stays "gemm" where that is the faster of the two on gfx950:
+ *      with fewer than 64 input channels, with fewer than 128 and a filter count
+ *      that is no multiple of 64, and when the batch of the settings leaves the
+ *      Winograd kernel fewer than one and a half workgroups per compute unit;
+ *      algo() reports what was chosen. ------ */
 int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activation,
                           const char *algo, dlp_conv2d_fwd **out);
 

@@ -331,8 +331,8 @@ def test_empty_batch_and_shape_errors(gpu):
 def test_algorithm_selection_rules(gpu):
     import dlprimitives_amd as dlp
 
-    def algo(c, hw, name):
-        st = gpu.settings_of(c, (2, c["cin"], hw, hw))
+    def algo(c, hw, name, batch=2):
+        st = gpu.settings_of(c, (batch, c["cin"], hw, hw))
         return dlp.Conv2DForward.create(st, False, "identity", name).algo()
 
     c33 = case(3, 1, 1, 1, 16, 16, False, 1, False)
@@ -341,9 +341,14 @@ def test_algorithm_selection_rules(gpu):
     big = case(3, 1, 1, 1, 48, 96, False, 1, False)  # LDS-patch kernel, fewer than 128 input channels: the automatic choice keeps the GEMM
     assert algo(big, 28, "") == "gemm" and algo(big, 28, "auto") == "gemm" and algo(big, 28, "winograd") == "winograd"
     assert algo(big, 112, "") == "winograd"  # too wide for the patch rows: Winograd against the gathering GEMM
-    assert algo(case(3, 1, 1, 1, 64, 96, False, 1, False), 28, "") == "gemm"      # filters off 64: 32 output channels per workgroup
-    assert algo(case(3, 1, 1, 1, 64, 64, False, 1, False), 28, "") == "winograd"  # 64 channels in, a multiple of 64 out: Winograd again
-    assert algo(case(3, 1, 1, 1, 128, 128, False, 1, False), 28, "") == "winograd"
+    assert algo(case(3, 1, 1, 1, 64, 96, False, 1, False), 28, "", 64) == "gemm"      # filters off 64: 32 output channels per workgroup
+    assert algo(case(3, 1, 1, 1, 64, 64, False, 1, False), 28, "", 64) == "winograd"  # 64 channels in, a multiple of 64 out: Winograd again
+    assert algo(case(3, 1, 1, 1, 128, 128, False, 1, False), 28, "", 64) == "winograd"
+    # ... as long as the batch of the settings leaves the Winograd kernel one and a half workgroups per compute unit
+    assert algo(case(3, 1, 1, 1, 128, 128, False, 1, False), 28, "", 2) == "gemm"
+    assert algo(case(3, 1, 1, 1, 512, 512, False, 1, False), 7, "", 32) == "gemm"
+    assert algo(case(3, 1, 1, 1, 512, 512, False, 1, False), 7, "", 64) == "winograd"
+    assert algo(case(3, 1, 1, 1, 128, 128, False, 1, False), 28, "winograd", 2) == "winograd"  # asked for by name: always
     assert algo(case(3, 1, 1, 1, 4, 16, False, 1, False), 8, "winograd") == "winograd"
     assert algo(case(3, 1, 2, 1, 16, 16, False, 1, False), 8, "winograd") == "gemm"  # incompatible -> silent gemm
     dw = case(3, 1, 1, 1, 16, 16, False, 16, False)
@@ -373,6 +378,30 @@ def test_winograd_three_way(gpu, oracle_mod, shape):
     np.testing.assert_allclose(got, wino_cpu, **TOL)
     np.testing.assert_allclose(got, direct, **TOL)
     np.testing.assert_allclose(got, gemm, **TOL)
+
+
+# Enough workgroups for the chip and a multiple of 64 filters: a workgroup takes two blocks of 32 output channels
+@pytest.mark.parametrize("shape", [(8, 8, 512, 28, 28),    # rows staged in LDS
+                                   (8, 12, 512, 28, 28),   # masked channel tail
+                                   (4, 8, 512, 56, 56),    # patches gathered from global memory
+                                   (33, 16, 1024, 14, 14)],  # tiles of a workgroup span images
+                         ids=lambda s: "b%d_c%d_n%d_%dx%d" % s)
+def test_winograd_two_blocks_per_workgroup(gpu, oracle_mod, shape):
+    import dlprimitives_amd as dlp
+
+    B, C, N, H, W = shape
+    c = case(3, 1, 1, 1, C, N, True, 1, True)
+    x, w, bias = make_tensors(c, (B, H, W), seed=C + H)
+    dlp.timing_enable(True)
+    dlp.timing_reset()
+    got, _ = gpu.run_conv(c, x, w, bias, algo="winograd", expect_algo="winograd")
+    kernels = [k for (_, _, k) in dlp.timing_records(kernels=True) if k.startswith("wino_fused_kernel")]
+    dlp.timing_enable(False)
+    assert kernels and all(k.endswith(", 2>") for k in kernels), kernels
+    np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
+    old = np.random.default_rng(5).standard_normal(got.shape).astype(np.float32)
+    got_f, _ = gpu.run_conv(c, x, w, bias, algo="winograd", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got_f, oracle_mod.apply_factor(got, old, 0.5), rtol=1e-5, atol=1e-5)
 
 
 def test_winograd_batch_larger_than_hint_is_chunked(gpu, oracle_mod):
