@@ -2662,6 +2662,10 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
         p.mask = small_kernel ? GEMM_MASK_TAPS : GEMM_MASK_ROWCOL;
     }
     p.tile = tile_choice(p.M);
+    // 1x1 convolutions whose last tile of 64 filters would be at most half full take tiles of 32 filters (x 128 pixels): no matrix
+    // instruction is spent on rows that do not exist (batch 64, cold: 384->96 at 14x14 21.5 -> 18.6 us, 960->160 at 7x7 21.9 -> 19.1)
+    if (g.KH == 1 && g.KW == 1 && p.M > 32 && (p.M % 64) != 0 && (p.M % 64) <= 32)
+        p.tile = 1;
     // 1x1 convolutions in the tap-major order: a K tile is 16 consecutive input channels of the filter rows, which the
     // kernel reads from the weight tensor in place (when it is 16-byte aligned): nothing is packed
     p.wdirect = g.dtype == DLP_FLOAT && p.order == GEMM_ORDER_TAP && g.KH == 1 && g.KW == 1;

@@ -518,6 +518,51 @@ def test_pointwise_1x1(gpu, oracle_mod, pw):
     np.testing.assert_allclose(got, oracle_conv(oracle_mod, c, x, w, bias), **TOL)
 
 
+# 1x1 convolutions whose last tile of 64 filters would be at most half full run on tiles of 32 filters x 128 pixels
+# (cin, cout, H, W, batch, stride, activation)
+NARROW_TILE_SHAPES = [(384, 96, 14, 14, 3, 1, "relu6"), (960, 160, 7, 7, 2, 1, "relu"), (48, 96, 9, 11, 3, 1, "identity"), (32, 65, 5, 7, 2, 1, "relu"),
+                      (128, 96, 28, 28, 2, 2, "relu"), (20, 70, 6, 6, 2, 1, "tanh")]
+
+
+@pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "%dto%d_%dx%d_b%d_s%d_%s" % s)
+def test_pointwise_tiles_of_32_filters(gpu, oracle_mod, shape):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    cin, cout, h, w_, b, stride, act = shape
+    c = case(1, 0, stride, 1, cin, cout, True, 1, False)
+    c["activation"] = act
+    x, w, bias = make_tensors(c, (b, h, w_), seed=cin + cout)
+    dlp.timing_enable(True)
+    dlp.timing_reset()
+    got, _ = gpu.run_conv(c, x, w, bias, algo="gemm", expect_algo="gemm")
+    kernels = [k for (_, _, k) in dlp.timing_records(kernels=True) if k.startswith("conv_gemm_f32_kernel")]
+    dlp.timing_enable(False)
+    assert kernels and all(k.startswith("conv_gemm_f32_kernel<float, 32, 128") for k in kernels), kernels
+    want = oracle_conv(oracle_mod, c, x, w, bias)
+    np.testing.assert_allclose(got, want, **TOL)
+    old = np.random.default_rng(5).standard_normal(want.shape).astype(np.float32)
+    got_f, _ = gpu.run_conv(c, x, w, bias, algo="gemm", factor=0.5, y_init=old)
+    np.testing.assert_allclose(got_f, oracle_mod.apply_factor(want, old, 0.5), **TOL)
+    # packed once + enqueue_packed gives the same bits as enqueue
+    op = dlp.Conv2DForward.create(gpu.settings_of(c, x.shape), True, act, "gemm")
+    packed = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
+    ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    op.pack(gpu.dev(w), packed)
+    y2 = torch.full(want.shape, float("nan"), dtype=torch.float32, device="cuda:0")
+    op.enqueue_packed(gpu.dev(x), gpu.dev(w), packed, gpu.dev(bias), y2, ws, 0.0)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(y2.cpu().numpy(), got, rtol=1e-6, atol=1e-6)
+    if act != "tanh":  # integer-valued tensors: exact whatever the order of the sum
+        rng = np.random.default_rng(13)
+        xi = rng.integers(-3, 4, size=x.shape).astype(np.float32)
+        wi = rng.integers(-2, 3, size=w.shape).astype(np.float32)
+        bi = rng.integers(-5, 6, size=(cout,)).astype(np.float32)
+        got_i, _ = gpu.run_conv(c, xi, wi, bi, algo="gemm")
+        assert np.array_equal(got_i, oracle_conv(oracle_mod, c, xi, wi, bi))
+
+
 # ------------------------------------------------------------ InnerProduct
 def test_inner_product_reference_goldens(gpu):
     doc = json.load(open(os.path.join(GOLDEN, "inner_product_fwd.json")))
