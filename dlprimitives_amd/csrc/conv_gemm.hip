@@ -2286,7 +2286,10 @@ void plan_split(const GemmPlan &p, GemmArgs &a, int groups, bool have_ws, size_t
         const long long wgs = tiles * a.splitk, full = wgs / cus * cus;
         if (full > 0 && full < wgs) {
             const long long tail = tiles - full / a.splitk;
-            const long long kt2 = ((tail * a.nkt + cus - 1) / cus + 1) / 2 * 2; // the tail's K tiles per CU, even
+            // the tail's K tiles per CU, even; no finer than sixteen slices per tile: the workgroup that arrives last reads the others'
+            // pieces back four at a time, and a tail of two tiles of a small launch is not worth a 64-way reduction
+            // (1x1 2048->512 at 7x7, batch 16: 46 -> 26 us)
+            const long long kt2 = std::max<long long>(((tail * a.nkt + cus - 1) / cus + 1) / 2 * 2, ((a.nkt + 15) / 16 + 1) / 2 * 2);
             const long long s2 = (a.nkt + kt2 - 1) / kt2;
             if (kt2 < a.kt_per_slice && s2 <= 64 && tail * s2 < 0x7fffffffLL - wgs) {
                 a.tail_tiles = (int)tail;
