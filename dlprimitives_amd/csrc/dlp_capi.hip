@@ -854,6 +854,7 @@ int dlp_ip_fwd_create(const dlp_ip_settings *cfg, int bias, int activation, dlp_
         delete op;
         return rc;
     }
+    ip_stream_prepare(cfg->dtype);
     *out = op;
     return DLP_OK;
 }
@@ -872,7 +873,10 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
     ep.activation = op->activation;
     if (ip_direct_supported(op->cfg.inputs, op->cfg.dtype, x, w)) {
         IpPlan ip;
-        const size_t need = ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
+        // large weight matrices stream through LDS (ip_stream_kernel); the scratch layout is the same for both kernels
+        const bool streamed = ip_stream_supported(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w);
+        const size_t need = streamed ? ip_stream_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip)
+                                     : ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
         (void)need;
         // op-owned scratch = [counters | partial sums]; both regions only ever grow, and the counter region keeps
         // its place so that no partial sum is ever written where a later, larger batch expects zeroed counters
@@ -889,6 +893,9 @@ int dlp_ip_fwd_enqueue(dlp_ip_fwd *op, int batch, const void *x, const void *w, 
             op->scratch_bytes = cnt_bytes + part_bytes;
             op->scratch_cnt_bytes = cnt_bytes;
         }
+        if (streamed)
+            return ip_stream_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, (int *)op->scratch,
+                                    (float *)((char *)op->scratch + op->scratch_cnt_bytes), (hipStream_t)stream);
         return ip_direct_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, (int *)op->scratch,
                                 (float *)((char *)op->scratch + op->scratch_cnt_bytes), (hipStream_t)stream);
     }
@@ -913,7 +920,11 @@ int dlp_ip_fwd_enqueue_no_alloc(dlp_ip_fwd *op, int batch, const void *x, const 
     if (!ip_direct_supported(op->cfg.inputs, op->cfg.dtype, x, w))
         return fail(DLP_ERR_NOT_IMPLEMENTED, "dlp_ip_fwd_enqueue_no_alloc: bfloat16 rows must have an even length and dword-aligned tensors");
     IpPlan ip;
-    ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
+    const bool streamed = ip_stream_supported(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w); // the kernel dlp_ip_fwd_enqueue takes
+    if (streamed)
+        ip_stream_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
+    else
+        ip_direct_scratch_bytes(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, &ip);
     // (an unsplit K uses neither counters nor partial sums)
     if (ip.S > 1 && (ip.cnt_bytes > kNoAllocCounterBytes || ip.part_bytes > (size_t)DLP_IP_NO_ALLOC_SCRATCH_BYTES - kNoAllocCounterBytes))
         return fail(DLP_ERR_VALIDATION, "dlp_ip_fwd_enqueue_no_alloc: this batch x outputs needs " + std::to_string(ip.cnt_bytes) + " + " +
@@ -937,6 +948,8 @@ int dlp_ip_fwd_enqueue_no_alloc(dlp_ip_fwd *op, int batch, const void *x, const 
         hipLaunchKernelGGL(clear_ints_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, counters, n);
         DLP_HIP_TRY(hipGetLastError());
     }
+    if (streamed)
+        return ip_stream_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, counters, partials, (hipStream_t)stream);
     return ip_direct_launch(batch, op->cfg.inputs, op->cfg.outputs, op->cfg.dtype, x, w, y, ep, counters, partials, (hipStream_t)stream);
 }
 

@@ -266,5 +266,11 @@ bool ip_direct_supported(int inputs, int dtype, const void *x, const void *w);
 // counters: cnt_bytes of zeros (they are left zero); partials: part_bytes
 int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
                      float *partials, hipStream_t stream);
+// Large weight matrices at small batch: w streamed through LDS in 1 KB runs per row (same scratch layout and contract)
+bool ip_stream_supported(int batch, int inputs, int outputs, int dtype, const void *x, const void *w);
+void ip_stream_prepare(int dtype); // one-time set-up of the kernel on the current device (called when an operator is created)
+size_t ip_stream_scratch_bytes(int batch, int inputs, int outputs, int dtype, IpPlan *plan);
+int ip_stream_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
+                     float *partials, hipStream_t stream);
 
 } // namespace dlp

@@ -4,6 +4,9 @@
 // (src/core/ip.cpp:15-50, src/gemm.cpp:240-345):
 //   y[B x Out] = act(x[B x In] * w[Out x In]^T + bias[Out])
 //
+// Two kernels: ip_stream_kernel (further down; rows on 16-byte boundaries: the weights go through LDS in runs of 1 KB per row)
+// and ip_direct_kernel (every other alignment), which share the operand layout and the way K slices are reduced.
+//
 // Both operands are stored with the reduction index innermost, which is exactly what a matrix
 // instruction wants in a lane: ip_direct_kernel loads them straight from memory into operand
 // registers -- no LDS, no repacking of the weights, no barriers.
@@ -26,6 +29,8 @@
 #include "dlp_internal.hpp"
 
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 namespace dlp {
@@ -71,6 +76,90 @@ __device__ __forceinline__ ip_u32x4 load_piece(__amdgpu_buffer_rsrc_t r, uint32_
         return v;
     }
     return __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, row_off, soff, 0));
+}
+
+// What the wavefront that owns a tile's K slice does with its accumulators: with several slices, the partial sums go to the
+// scratch buffer (write-through) and the wavefront that arrives last at the tile's counter adds all slices in slice order; then
+// bias, activation and the store of y.
+template <class T, int NB>
+__device__ __forceinline__ void ip_finish(const IpArgs &a, ip_f32x16 (&acc)[NB], int tile, int slice, int m0, int n0, int lane, int l32, int h)
+{
+    if (a.S > 1) {
+        constexpr int kThrough = 17; // sc0 | sc1: past the caches in both directions
+        constexpr uint32_t image_bytes = NB * 16 * 64 * 4;
+        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
+        const uint32_t base = (uint32_t)(tile * a.S) * image_bytes;
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float v = acc[j][r];
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, (uint32_t)lane * 4u,
+                                                      base + (uint32_t)slice * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough);
+            }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the partial sums have been written through
+        int arrived = 0;
+        if (lane == 0)
+            arrived = atomicAdd(a.cnt + tile, 1);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != a.S - 1)
+            return;
+        if (lane == 0)
+            atomicExch(a.cnt + tile, 0); // ready for the next launch on the stream
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[j][r] = 0.0f;
+            // four slices (64 loads) in flight at a time: these loads come from memory, not from a cache
+            for (int s0 = 0; s0 < a.S; s0 += 4) {
+                float p[4][16];
+#pragma unroll
+                for (int ds = 0; ds < 4; ds++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        p[ds][r] = (s0 + ds < a.S) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                         pr, (uint32_t)lane * 4u,
+                                                         base + (uint32_t)(s0 + ds) * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough))
+                                                   : 0.0f;
+#pragma unroll
+                for (int ds = 0; ds < 4; ds++) // slice order
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        acc[j][r] += p[ds][r];
+            }
+        }
+    }
+
+    // epilogue: accumulator register r of a block holds output m0 + 8*(r/4) + 4*h + r%4 of batch row n0 + 32*j + l32
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const int n = n0 + j * 32 + l32;
+        if (n >= a.B)
+            continue;
+        T *yrow = (T *)a.y + (size_t)n * a.Out;
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            const int mq = m0 + 8 * rq + 4 * h; // four consecutive outputs
+            float v[4];
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                v[rr] = acc[j][4 * rq + rr];
+                if (a.bias && mq + rr < a.Out)
+                    v[rr] += a.bias[mq + rr];
+                v[rr] = apply_act(v[rr], a.act);
+            }
+            if (sizeof(T) == 4 && (a.Out & 3) == 0 && ((uintptr_t)a.y & 15) == 0) {
+                if (mq < a.Out)
+                    *(ip_f32x4 *)((float *)yrow + mq) = ip_f32x4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++)
+                    if (mq + rr < a.Out)
+                        store_plain(yrow + mq + rr, v[rr]);
+            }
+        }
+    }
 }
 
 template <class T, int NB, bool WIDE>
@@ -153,82 +242,112 @@ __global__ __launch_bounds__(256) void ip_direct_kernel(IpArgs a)
         }
     }
 
-    if (a.S > 1) {
-        constexpr int kThrough = 17; // sc0 | sc1: past the caches in both directions
-        constexpr uint32_t image_bytes = NB * 16 * 64 * 4;
-        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc(a.part, 0, a.part_bytes, 0x00020000);
-        const uint32_t base = (uint32_t)(tile * a.S) * image_bytes;
+    ip_finish<T, NB>(a, acc, tile, slice, m0, n0, lane, l32, h);
+}
+
+// ---- large weight matrices at small batch: w streamed through LDS in runs of 1 KB per row ----
+// The direct kernel above reads 32 bytes of each of 32 rows per load instruction: with rows tens of kilobytes apart that is
+// 32768 concurrent streams of 128 bytes for the memory system, and a 411 MB matrix arrives at 2.7 TB/s.  Here a workgroup owns
+// 32 outputs x 32 batch rows over one K slice and walks it in chunks of 1 KB per row: every wavefront load is 1 KB of ONE row
+// (what a copy kernel issues), the chunk of the next step travels into registers while this one is multiplied, the tiles go
+// to LDS as they lie in memory ([row][1 KB + 16]: the 16-byte operand reads of 16 lanes cover 256 consecutive bytes, no bank
+// conflicts), and the four wavefronts each take a quarter of the chunk's k with the same operand layout as the direct kernel
+// (a lane's 16 bytes: four k of four fp32 matrix instructions, or the eight k of one bf16 instruction).  The wavefronts'
+// accumulators are added in wavefront order through LDS; wavefront 0 then finishes the slice like the direct kernel does.
+constexpr int kIpRowBytes = 1024;            // bytes of a row per chunk
+constexpr int kIpLdsRow = kIpRowBytes + 16;  // LDS bytes per row
+constexpr int kIpLdsBytes = 2 * 32 * kIpLdsRow; // the tiles of w and of x: 65 KB, two workgroups per compute unit
+
+template <class T>
+__global__ __launch_bounds__(256) void ip_stream_kernel(IpArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char ip_lds[]; // kIpLdsBytes, asked for at launch
+    unsigned char *Ws = ip_lds, *Xs = ip_lds + 32 * kIpLdsRow;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int wg = (int)blockIdx.x;
+    const int nc = wg % a.nchunks;
+    const int slice = (wg / a.nchunks) % a.S;
+    const int mb = wg / (a.nchunks * a.S);
+    const int tile = mb * a.nchunks + nc;
+    const int m0 = mb * 32, n0 = nc * 32;
+
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+    const uint32_t row_bytes = (uint32_t)a.In * (uint32_t)sizeof(T); // a multiple of 16
+    // piece i of this thread: row wave + 4 i of the tile, bytes [16 lane, 16 lane + 16) of the chunk.  Rows of w past the end are
+    // clamped to the last one (valid memory; their results are never stored), batch rows past the end read as zeros.
+    uint32_t w_off[8], x_off[8];
 #pragma unroll
-        for (int j = 0; j < NB; j++)
+    for (int i = 0; i < 8; i++) {
+        const int r = wave + 4 * i;
+        w_off[i] = (uint32_t)min(m0 + r, a.Out - 1) * row_bytes + (uint32_t)lane * 16u;
+        x_off[i] = n0 + r < a.B ? (uint32_t)(n0 + r) * row_bytes + (uint32_t)lane * 16u : kIpOutOfRange;
+    }
+    ip_u32x4 rw[8], rx[8];
+    auto load_chunk = [&](int c) {
+        const uint32_t soff = (uint32_t)c * (uint32_t)kIpRowBytes;
+        const bool inside = soff + (uint32_t)lane * 16u < row_bytes; // the last chunk of a row may be short: what follows is the next row
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float v = acc[j][r];
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), pr, (uint32_t)lane * 4u,
-                                                      base + (uint32_t)slice * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough);
-            }
-        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the partial sums have been written through
-        int arrived = 0;
-        if (lane == 0)
-            arrived = atomicAdd(a.cnt + tile, 1);
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        if (arrived != a.S - 1)
-            return;
-        if (lane == 0)
-            atomicExch(a.cnt + tile, 0); // ready for the next launch on the stream
+        for (int i = 0; i < 8; i++) {
+            rw[i] = __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, inside ? w_off[i] : kIpOutOfRange, soff, 0));
+            rx[i] = __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, inside ? x_off[i] : kIpOutOfRange, soff, 0));
+        }
+    };
+
+    ip_f32x16 acc[1];
 #pragma unroll
-        for (int j = 0; j < NB; j++) {
+    for (int r = 0; r < 16; r++)
+        acc[0][r] = 0.0f;
+
+    const int c_begin = slice * a.gps, c_end = min(c_begin + a.gps, a.ngroups); // chunks of this slice
+    if (c_begin < c_end)
+        load_chunk(c_begin);
+    for (int c = c_begin; c < c_end; c++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-                acc[j][r] = 0.0f;
-            // four slices (64 loads) in flight at a time: these loads come from memory, not from a cache
-            for (int s0 = 0; s0 < a.S; s0 += 4) {
-                float p[4][16];
+        for (int i = 0; i < 8; i++) {
+            *(ip_u32x4 *)(Ws + (wave + 4 * i) * kIpLdsRow + lane * 16) = rw[i];
+            *(ip_u32x4 *)(Xs + (wave + 4 * i) * kIpLdsRow + lane * 16) = rx[i];
+        }
+        __syncthreads();
+        if (c + 1 < c_end)
+            load_chunk(c + 1);
+        // this wavefront's quarter of the chunk: eight steps of 32 bytes per row
 #pragma unroll
-                for (int ds = 0; ds < 4; ds++)
+        for (int g = 0; g < 8; g++) {
+            const int off = l32 * kIpLdsRow + wave * 256 + g * 32 + h * 16;
+            const ip_u32x4 fa = *(const ip_u32x4 *)(Ws + off);
+            const ip_u32x4 fb = *(const ip_u32x4 *)(Xs + off);
+            if constexpr (sizeof(T) == 4) {
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        p[ds][r] = (s0 + ds < a.S) ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                         pr, (uint32_t)lane * 4u,
-                                                         base + (uint32_t)(s0 + ds) * image_bytes + (uint32_t)((j * 16 + r) * 256), kThrough))
-                                                   : 0.0f;
-#pragma unroll
-                for (int ds = 0; ds < 4; ds++) // slice order
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        acc[j][r] += p[ds][r];
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t ae = fa[e], be = fb[e]; // copies: bit_cast applied to a vector element reads element 0
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, ae), __builtin_bit_cast(float, be), acc[0], 0, 0, 0);
+                }
+            } else {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ip_bf16x8, fa), __builtin_bit_cast(ip_bf16x8, fb), acc[0], 0, 0, 0);
             }
         }
+        __syncthreads(); // the tiles are overwritten by the next chunk
     }
 
-    // epilogue: accumulator register r of a block holds output m0 + 8*(r/4) + 4*h + r%4 of batch row n0 + 32*j + l32
+    // the four quarters, added in wavefront order by wavefront 0 (register images [wavefront][r][lane] in LDS)
+    float *red = reinterpret_cast<float *>(Ws);
+    if (wave != 0) {
 #pragma unroll
-    for (int j = 0; j < NB; j++) {
-        const int n = n0 + j * 32 + l32;
-        if (n >= a.B)
-            continue;
-        T *yrow = (T *)a.y + (size_t)n * a.Out;
-#pragma unroll
-        for (int rq = 0; rq < 4; rq++) {
-            const int mq = m0 + 8 * rq + 4 * h; // four consecutive outputs
-            float v[4];
-#pragma unroll
-            for (int rr = 0; rr < 4; rr++) {
-                v[rr] = acc[j][4 * rq + rr];
-                if (a.bias && mq + rr < a.Out)
-                    v[rr] += a.bias[mq + rr];
-                v[rr] = apply_act(v[rr], a.act);
-            }
-            if (sizeof(T) == 4 && (a.Out & 3) == 0 && ((uintptr_t)a.y & 15) == 0) {
-                if (mq < a.Out)
-                    *(ip_f32x4 *)((float *)yrow + mq) = ip_f32x4{v[0], v[1], v[2], v[3]};
-            } else {
-#pragma unroll
-                for (int rr = 0; rr < 4; rr++)
-                    if (mq + rr < a.Out)
-                        store_plain(yrow + mq + rr, v[rr]);
-            }
-        }
+        for (int r = 0; r < 16; r++)
+            red[((wave - 1) * 16 + r) * 64 + lane] = acc[0][r];
     }
+    __syncthreads();
+    if (wave != 0)
+        return;
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            acc[0][r] += red[(q * 16 + r) * 64 + lane];
+    ip_finish<T, 1>(a, acc, tile, slice, m0, n0, lane, l32, h);
 }
 
 } // namespace
@@ -326,6 +445,114 @@ int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *
         pick_nb(bf16_t{});
     else
         pick_nb(float{});
+    DLP_HIP_TRY(hipGetLastError());
+    return DLP_OK;
+}
+
+// The streaming kernel: wherever the rows of w and of x start on 16-byte boundaries.  Measured against the direct kernel on cold
+// weights, fp32 (bf16): 25088 -> 4096 at batch 16 162 -> 98 us = 4.2 TB/s (83 -> 48), 9216 -> 4096 68 -> 46 (39 -> 24),
+// 4096 -> 1000 32 -> 15 (27 -> 11), 2048 -> 1000 at batch 128 26 -> 16 (22 -> 11), 1280 -> 1000 at batch 16 26 -> 12 (18 -> 8),
+// 25088 -> 4096 at batch 128 563 -> 318 (263 -> 135).
+bool ip_stream_supported(int batch, int inputs, int outputs, int dtype, const void *x, const void *w)
+{
+    static const char *pin = getenv("DLP_IP_KERNEL"); // "direct" / "stream": one kernel wherever it can run, for measurements
+    if (pin && pin[0] == 'd')
+        return false;
+    if (dtype != DLP_FLOAT && dtype != DLP_BFLOAT16)
+        return false;
+    const size_t esize = dtype_size(dtype);
+    if (batch < 1 || ((size_t)inputs * esize) % 16 != 0 || (((uintptr_t)x | (uintptr_t)w) & 15) != 0)
+        return false;
+    (void)outputs;
+    return true;
+}
+
+size_t ip_stream_scratch_bytes(int batch, int inputs, int outputs, int dtype, IpPlan *plan)
+{
+    IpPlan p;
+    const int kc = kIpRowBytes / (int)dtype_size(dtype); // k per chunk
+    p.nb = 1;
+    p.mblocks = (outputs + 31) / 32;
+    p.nchunks = (batch + 31) / 32;
+    p.ngroups = (inputs + kc - 1) / kc; // chunks of a row
+    // K slices: about two workgroups per compute unit, slices of at least two chunks, at most 16 slices
+    const long long tiles = (long long)p.mblocks * p.nchunks;
+    long long s = (2ll * dlp_cu_count() + tiles - 1) / tiles;
+    s = std::min<long long>(s, p.ngroups / 2);
+    s = std::max<long long>(1, std::min<long long>(s, 16));
+    p.gps = (int)((p.ngroups + s - 1) / s);
+    p.S = (p.ngroups + p.gps - 1) / p.gps;
+    p.cnt_bytes = (size_t)((tiles * sizeof(int) + 255) / 256 * 256);
+    p.part_bytes = p.S > 1 ? (size_t)tiles * p.S * 16 * 64 * sizeof(float) : 0;
+    if (plan)
+        *plan = p;
+    return p.cnt_bytes + p.part_bytes;
+}
+
+// More than 64 KB of LDS has to be asked for, once per kernel and device.  Done when an operator is created (best effort: there
+// may be no device yet) so that a first enqueue inside a stream capture has nothing left to set up; the launch checks again.
+static std::atomic<bool> g_ip_lds_asked[2][64];
+static int ip_stream_ask_lds(bool bf16)
+{
+    int dev = 0;
+    DLP_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !g_ip_lds_asked[bf16][dev].load()) {
+        DLP_HIP_TRY(hipFuncSetAttribute(bf16 ? (const void *)ip_stream_kernel<bf16_t> : (const void *)ip_stream_kernel<float>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kIpLdsBytes));
+        if (dev >= 0 && dev < 64)
+            g_ip_lds_asked[bf16][dev].store(true);
+    }
+    return DLP_OK;
+}
+void ip_stream_prepare(int dtype)
+{
+    if (dtype == DLP_FLOAT || dtype == DLP_BFLOAT16) {
+        (void)ip_stream_ask_lds(dtype == DLP_BFLOAT16);
+        (void)hipGetLastError(); // no device, no harm: the launch asks again
+    }
+}
+
+int ip_stream_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
+                     float *partials, hipStream_t stream)
+{
+    IpPlan p;
+    ip_stream_scratch_bytes(batch, inputs, outputs, dtype, &p);
+    const size_t esize = dtype_size(dtype);
+    const size_t x_bytes = (size_t)batch * inputs * esize, w_bytes = (size_t)outputs * inputs * esize;
+    if (x_bytes >= kIpOutOfRange || w_bytes >= kIpOutOfRange || p.part_bytes >= kIpOutOfRange)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
+    IpArgs a;
+    a.x = x;
+    a.w = w;
+    a.bias = ep.bias;
+    a.y = y;
+    a.cnt = counters;
+    a.part = partials;
+    a.B = batch;
+    a.In = inputs;
+    a.Out = outputs;
+    a.S = p.S;
+    a.ngroups = p.ngroups;
+    a.gps = p.gps;
+    a.mblocks = p.mblocks;
+    a.nchunks = p.nchunks;
+    a.act = ep.activation;
+    a.x_bytes = (uint32_t)x_bytes;
+    a.w_bytes = (uint32_t)w_bytes;
+    a.part_bytes = (uint32_t)p.part_bytes;
+    const long long wgs = (long long)p.mblocks * p.nchunks * p.S;
+    if (wgs > 0x7fffffffLL)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "inner product too large for a single launch");
+    const dim3 grid((unsigned)wgs), block(256);
+    TimingScope ts("ip_direct", stream);
+    const bool bf16 = dtype == DLP_BFLOAT16;
+    const int rc = ip_stream_ask_lds(bf16);
+    if (rc != DLP_OK)
+        return rc;
+    if (bf16)
+        DLP_LAUNCH_TIMED(ts, ip_stream_kernel<bf16_t>, grid, block, kIpLdsBytes, stream, a);
+    else
+        DLP_LAUNCH_TIMED(ts, ip_stream_kernel<float>, grid, block, kIpLdsBytes, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }

@@ -263,10 +263,11 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
  * the operator allocates (and regrows for a larger batch) live here in one array of
  * DLP_IP_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends.
  * The call makes no hipMalloc / hipFree and records no memset.  The array holds 64 KiB of tile counters and
- * 4 MiB of partial sums (4 KiB per tile of 32 outputs x 32 batch rows and K slice): enough for 2048 -> 1000 at
- * batch 128 (3.5 MiB) or 25088 -> 4096 at batch 16 (4 MiB).  A batch x outputs that needs more is a validation
- * error that names both sizes (e.g. 1024 -> 4096 at batch 160: 5 MiB); bfloat16 rows of odd length are
- * NotImplemented.
+ * 4 MiB of partial sums (4 KiB per tile of 32 outputs x 32 batch rows and K slice).  With rows on 16-byte
+ * boundaries (the kernel that streams w through LDS) K is only cut while there are fewer than two workgroups
+ * per compute unit, which keeps the partial sums under 4 MiB on an MI355X whatever the shape; other
+ * alignments cut K more freely, and a batch x outputs that then needs more is a validation error that
+ * names both sizes (e.g. 1026 -> 4096 at batch 160: 5 MiB).  bfloat16 rows of odd length are NotImplemented.
  * RULE: at most one call in flight per device.  All calls on one device share the array, whatever the operator: two
  * calls that overlap on one device (different streams, two threads, two recorded graphs replayed side by side) race on
  * the counters and partial sums, and nothing detects it; calls on one stream, or replays of graphs on one stream, are

@@ -276,6 +276,39 @@ def test_bf16_glue_and_inner_product(oracle_mod):
         np.testing.assert_allclose(yi.float().cpu().numpy(), oracle_mod.ip_forward(xi, wi, bi, "relu"), rtol=2 ** -8, atol=1e-3)
 
 
+def test_bf16_inner_product_streamed_weights(oracle_mod):
+    """bf16 weight matrices of 16 MB and more go through ip_stream_kernel: 512 k per chunk, a short last chunk, outputs and batch
+    off the block sizes; integer-valued operands must come out exact."""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    rng = np.random.default_rng(14)
+    for (B, I, O, act) in ((16, 8192, 1024, "relu"), (37, 8200, 1030, "identity")):
+        xi = oracle_mod.bf16_round(rng.uniform(-1, 1, (B, I)).astype(np.float32))
+        wi = oracle_mod.bf16_round((rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32))
+        bi = rng.uniform(-0.1, 0.1, O).astype(np.float32)
+        ip = dlp.IPForward.create(dlp.IPSettings(I, O, B, dtype=BFLOAT16_DATA), True, act)
+        yi = torch.full((B, O), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        dlp.timing_enable(True)
+        dlp.timing_reset()
+        ip.enqueue(_bf(xi), _bf(wi), torch.from_numpy(bi).cuda(), yi)
+        torch.cuda.synchronize()
+        kernels = [k for (_, _, k) in dlp.timing_records(kernels=True)]
+        dlp.timing_enable(False)
+        assert kernels and kernels[-1].startswith("ip_stream_kernel"), kernels
+        np.testing.assert_allclose(yi.float().cpu().numpy(), oracle_mod.ip_forward(xi, wi, bi, act), rtol=2 ** -8, atol=1e-3)
+        xq = rng.integers(-2, 3, (B, I)).astype(np.float32)
+        wq = rng.integers(-1, 2, (O, I)).astype(np.float32)
+        want = (xq.astype(np.int64) @ wq.astype(np.int64).T).astype(np.float32)
+        ip2 = dlp.IPForward.create(dlp.IPSettings(I, O, B, dtype=BFLOAT16_DATA), False, "identity")
+        yq = torch.full((B, O), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        ip2.enqueue(_bf(xq), _bf(wq), None, yq)
+        torch.cuda.synchronize()
+        assert np.array_equal(yq.float().cpu().numpy(), oracle_mod.bf16_round(want))  # the sum is exact in fp32, rounded once
+
+
 def test_resnet50_bf16_logits_vs_fp32_reference(oracle_mod):
     """Configuration 5 at a batch the CPU oracle finishes in seconds: ResNet-50 forward with bf16
     storage against the fp32 reference path on the same fp32 weights and inputs, 1e-2 relative."""

@@ -622,6 +622,65 @@ def test_inner_product_same_op_many_calls(gpu, oracle_mod):
         first[B] = (x, got)
 
 
+# Weight matrices whose rows start on 16-byte boundaries are streamed through LDS in runs of 1 KB per row (ip_stream_kernel).
+# (batch, inputs, outputs, activation, bias)
+IP_STREAM_SHAPES = [(16, 4096, 1024, "relu", True),      # whole chunks of 256 k, one batch chunk
+                    (1, 24, 5, "identity", True),        # one short chunk, one row, five outputs
+                    (3, 260, 40, "relu", True),          # a chunk and four k
+                    (5, 4100, 1030, "identity", True),   # a last chunk of 4 k, outputs off the block of 32
+                    (33, 4096, 1056, "relu", False),     # two batch chunks
+                    (130, 8200, 520, "tanh", True)]      # five batch chunks, a short last chunk
+
+
+@pytest.mark.parametrize("shape", IP_STREAM_SHAPES, ids=lambda s: "b%d_%dto%d_%s_%s" % s)
+def test_inner_product_streamed_weights(gpu, oracle_mod, shape):
+    import torch
+
+    import dlprimitives_amd as dlp
+
+    B, I, O, act, with_bias = shape
+    rng = np.random.default_rng(B + I)
+    x = rng.uniform(-1, 1, (B, I)).astype(np.float32)
+    w = (rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, O).astype(np.float32) if with_bias else None
+    dlp.timing_enable(True)
+    dlp.timing_reset()
+    got = gpu.run_ip(x, w, b, act)
+    kernels = [k for (_, _, k) in dlp.timing_records(kernels=True)]
+    dlp.timing_enable(False)
+    assert kernels and kernels[-1].startswith("ip_stream_kernel"), kernels
+    np.testing.assert_allclose(got, oracle_mod.ip_forward(x, w, b, act), **TOL)
+    # one operator, this batch and a smaller one, twice each: counters return to zero, a batch repeats bit for bit (the number
+    # of K slices, and with it the order of the sum, depends on the batch)
+    op = dlp.IPForward.create(dlp.IPSettings(I, O, B), with_bias, act)
+    wd, bd = gpu.dev(w), gpu.dev(b)
+    seen = {}
+    for rows in (B, max(1, B // 3), B, max(1, B // 3)):
+        yd = torch.full((rows, O), float("nan"), dtype=torch.float32, device="cuda:0")
+        op.enqueue(gpu.dev(x[:rows]), wd, bd, yd)
+        op.enqueue(gpu.dev(x[:rows]), wd, bd, yd)
+        torch.cuda.synchronize()
+        out = yd.cpu().numpy()
+        np.testing.assert_allclose(out, got[:rows], **TOL)
+        if rows in seen:
+            assert np.array_equal(out, seen[rows])
+        seen[rows] = out
+    assert np.array_equal(seen[B], got)
+    # integer-valued operands: exact whatever the order of the sum
+    xi = rng.integers(-3, 4, (B, I)).astype(np.float32)
+    wi = rng.integers(-3, 4, (O, I)).astype(np.float32)
+    if act != "tanh":
+        want = xi.astype(np.int64) @ wi.astype(np.int64).T
+        if with_bias:
+            bi = rng.integers(-5, 6, O).astype(np.float32)
+            want = want + bi.astype(np.int64)
+        else:
+            bi = None
+        if act == "relu":
+            want = np.maximum(want, 0)
+        assert np.array_equal(gpu.run_ip(xi, wi, bi, act), want.astype(np.float32))
+
+
 def test_inner_product_integer_exact(gpu):
     # integer-valued operands: every partial sum is exact in fp32, so the split over K slices and the
     # pairing of k inside a matrix instruction must reproduce the integer result exactly
