@@ -256,12 +256,14 @@ __global__ __launch_bounds__(256) void ip_direct_kernel(IpArgs a)
 // accumulators are added in wavefront order through LDS; wavefront 0 then finishes the slice like the direct kernel does.
 constexpr int kIpRowBytes = 1024;            // bytes of a row per chunk
 constexpr int kIpLdsRow = kIpRowBytes + 16;  // LDS bytes per row
-constexpr int kIpLdsBytes = 2 * 32 * kIpLdsRow; // the tiles of w and of x: 65 KB, two workgroups per compute unit
+// LDS of an instance: the tile of w and XR (+ 1 row of zeros when XR < 32) rows of x.  32 rows of x: 65 KB, two workgroups per
+// compute unit; 16 rows (batches of at most 16): 50 KB, three.
+constexpr int ip_stream_lds_bytes(int xr) { return (32 + xr + (xr < 32 ? 1 : 0)) * kIpLdsRow; }
 
-template <class T>
+template <class T, int XR>
 __global__ __launch_bounds__(256) void ip_stream_kernel(IpArgs a)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char ip_lds[]; // kIpLdsBytes, asked for at launch
+    extern __shared__ __attribute__((aligned(16))) unsigned char ip_lds[]; // ip_stream_lds_bytes(XR), asked for at launch
     unsigned char *Ws = ip_lds, *Xs = ip_lds + 32 * kIpLdsRow;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -285,16 +287,24 @@ __global__ __launch_bounds__(256) void ip_stream_kernel(IpArgs a)
         w_off[i] = (uint32_t)min(m0 + r, a.Out - 1) * row_bytes + (uint32_t)lane * 16u;
         x_off[i] = n0 + r < a.B ? (uint32_t)(n0 + r) * row_bytes + (uint32_t)lane * 16u : kIpOutOfRange;
     }
-    ip_u32x4 rw[8], rx[8];
+    constexpr int XP = XR / 4; // pieces of x per thread
+    ip_u32x4 rw[8], rx[XP];
     auto load_chunk = [&](int c) {
         const uint32_t soff = (uint32_t)c * (uint32_t)kIpRowBytes;
         const bool inside = soff + (uint32_t)lane * 16u < row_bytes; // the last chunk of a row may be short: what follows is the next row
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             rw[i] = __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, inside ? w_off[i] : kIpOutOfRange, soff, 0));
-            rx[i] = __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, inside ? x_off[i] : kIpOutOfRange, soff, 0));
+            if (i < XP)
+                rx[i] = __builtin_bit_cast(ip_u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, inside ? x_off[i] : kIpOutOfRange, soff, 0));
         }
     };
+    // batch rows past XR do not exist: their lanes read a row of zeros
+    const int x_row = l32 < XR ? l32 : XR;
+    if (XR < 32) {
+        for (int i = tid; i < kIpLdsRow / 16; i += 256)
+            *(ip_u32x4 *)(Xs + XR * kIpLdsRow + i * 16) = ip_u32x4{0u, 0u, 0u, 0u};
+    }
 
     ip_f32x16 acc[1];
 #pragma unroll
@@ -308,7 +318,8 @@ __global__ __launch_bounds__(256) void ip_stream_kernel(IpArgs a)
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             *(ip_u32x4 *)(Ws + (wave + 4 * i) * kIpLdsRow + lane * 16) = rw[i];
-            *(ip_u32x4 *)(Xs + (wave + 4 * i) * kIpLdsRow + lane * 16) = rx[i];
+            if (i < XP)
+                *(ip_u32x4 *)(Xs + (wave + 4 * i) * kIpLdsRow + lane * 16) = rx[i];
         }
         __syncthreads();
         if (c + 1 < c_end)
@@ -316,9 +327,9 @@ __global__ __launch_bounds__(256) void ip_stream_kernel(IpArgs a)
         // this wavefront's quarter of the chunk: eight steps of 32 bytes per row
 #pragma unroll
         for (int g = 0; g < 8; g++) {
-            const int off = l32 * kIpLdsRow + wave * 256 + g * 32 + h * 16;
-            const ip_u32x4 fa = *(const ip_u32x4 *)(Ws + off);
-            const ip_u32x4 fb = *(const ip_u32x4 *)(Xs + off);
+            const int koff = wave * 256 + g * 32 + h * 16;
+            const ip_u32x4 fa = *(const ip_u32x4 *)(Ws + l32 * kIpLdsRow + koff);
+            const ip_u32x4 fb = *(const ip_u32x4 *)(Xs + x_row * kIpLdsRow + koff);
             if constexpr (sizeof(T) == 4) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -450,7 +461,7 @@ int ip_direct_launch(int batch, int inputs, int outputs, int dtype, const void *
 }
 
 // The streaming kernel: wherever the rows of w and of x start on 16-byte boundaries.  Measured against the direct kernel on cold
-// weights, fp32 (bf16): 25088 -> 4096 at batch 16 162 -> 98 us = 4.2 TB/s (83 -> 48), 9216 -> 4096 68 -> 46 (39 -> 24),
+// weights, fp32 (bf16): 25088 -> 4096 at batch 16 162 -> 93 us = 4.4 TB/s (83 -> 49), 9216 -> 4096 68 -> 43 (39 -> 23),
 // 4096 -> 1000 32 -> 15 (27 -> 11), 2048 -> 1000 at batch 128 26 -> 16 (22 -> 11), 1280 -> 1000 at batch 16 26 -> 12 (18 -> 8),
 // 25088 -> 4096 at batch 128 563 -> 318 (263 -> 135).
 bool ip_stream_supported(int batch, int inputs, int outputs, int dtype, const void *x, const void *w)
@@ -475,9 +486,12 @@ size_t ip_stream_scratch_bytes(int batch, int inputs, int outputs, int dtype, Ip
     p.mblocks = (outputs + 31) / 32;
     p.nchunks = (batch + 31) / 32;
     p.ngroups = (inputs + kc - 1) / kc; // chunks of a row
-    // K slices: about two workgroups per compute unit, slices of at least two chunks, at most 16 slices
+    // K slices: as many workgroups as fit the compute units at once (three each with the 16-row tile of x, else two), slices of at
+    // least two chunks, at most 16 slices, and never more than 1024 tiles x slices once K is cut (4 MiB of partial sums, what the
+    // entry point that allocates nothing holds)
     const long long tiles = (long long)p.mblocks * p.nchunks;
-    long long s = (2ll * dlp_cu_count() + tiles - 1) / tiles;
+    long long s = ((batch <= 16 ? 3ll : 2ll) * dlp_cu_count() + tiles - 1) / tiles;
+    s = std::min<long long>(s, std::max<long long>(1, 1024 / tiles));
     s = std::min<long long>(s, p.ngroups / 2);
     s = std::max<long long>(1, std::min<long long>(s, 16));
     p.gps = (int)((p.ngroups + s - 1) / s);
@@ -489,27 +503,42 @@ size_t ip_stream_scratch_bytes(int batch, int inputs, int outputs, int dtype, Ip
     return p.cnt_bytes + p.part_bytes;
 }
 
-// More than 64 KB of LDS has to be asked for, once per kernel and device.  Done when an operator is created (best effort: there
-// may be no device yet) so that a first enqueue inside a stream capture has nothing left to set up; the launch checks again.
-static std::atomic<bool> g_ip_lds_asked[2][64];
-static int ip_stream_ask_lds(bool bf16)
+// An instance that needs more than 64 KB of LDS has to ask for it, once per device.  Done when an operator is created (best
+// effort: there may be no device yet) so that a first enqueue inside a stream capture has nothing left to set up; the launch
+// checks again.
+template <class T, int XR>
+static int ip_stream_instance(const IpArgs *a, dim3 grid, hipStream_t stream, TimingScope *ts)
 {
-    int dev = 0;
-    DLP_HIP_TRY(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64 || !g_ip_lds_asked[bf16][dev].load()) {
-        DLP_HIP_TRY(hipFuncSetAttribute(bf16 ? (const void *)ip_stream_kernel<bf16_t> : (const void *)ip_stream_kernel<float>,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kIpLdsBytes));
-        if (dev >= 0 && dev < 64)
-            g_ip_lds_asked[bf16][dev].store(true);
+    constexpr int lds = ip_stream_lds_bytes(XR);
+    if (lds > 65536) {
+        static std::atomic<bool> asked[64];
+        int dev = 0;
+        DLP_HIP_TRY(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 64 || !asked[dev].load()) {
+            DLP_HIP_TRY(hipFuncSetAttribute((const void *)ip_stream_kernel<T, XR>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            if (dev >= 0 && dev < 64)
+                asked[dev].store(true);
+        }
     }
+    if (a == nullptr) // set-up only
+        return DLP_OK;
+    DLP_LAUNCH_TIMED((*ts), (ip_stream_kernel<T, XR>), grid, dim3(256), lds, stream, *a);
+    DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
+}
+template <class T>
+static int ip_stream_dispatch(bool small_batch, const IpArgs *a, dim3 grid, hipStream_t stream, TimingScope *ts)
+{
+    return small_batch ? ip_stream_instance<T, 16>(a, grid, stream, ts) : ip_stream_instance<T, 32>(a, grid, stream, ts);
 }
 void ip_stream_prepare(int dtype)
 {
-    if (dtype == DLP_FLOAT || dtype == DLP_BFLOAT16) {
-        (void)ip_stream_ask_lds(dtype == DLP_BFLOAT16);
-        (void)hipGetLastError(); // no device, no harm: the launch asks again
-    }
+    if (dtype != DLP_FLOAT && dtype != DLP_BFLOAT16)
+        return;
+    for (int small = 0; small < 2; small++)
+        (void)(dtype == DLP_BFLOAT16 ? ip_stream_dispatch<bf16_t>(small != 0, nullptr, dim3(1), nullptr, nullptr)
+                                     : ip_stream_dispatch<float>(small != 0, nullptr, dim3(1), nullptr, nullptr));
+    (void)hipGetLastError(); // no device, no harm: the launch asks again
 }
 
 int ip_stream_launch(int batch, int inputs, int outputs, int dtype, const void *x, const void *w, void *y, const Epilogue &ep, int *counters,
@@ -543,18 +572,11 @@ int ip_stream_launch(int batch, int inputs, int outputs, int dtype, const void *
     const long long wgs = (long long)p.mblocks * p.nchunks * p.S;
     if (wgs > 0x7fffffffLL)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "inner product too large for a single launch");
-    const dim3 grid((unsigned)wgs), block(256);
+    const dim3 grid((unsigned)wgs);
     TimingScope ts("ip_direct", stream);
-    const bool bf16 = dtype == DLP_BFLOAT16;
-    const int rc = ip_stream_ask_lds(bf16);
-    if (rc != DLP_OK)
-        return rc;
-    if (bf16)
-        DLP_LAUNCH_TIMED(ts, ip_stream_kernel<bf16_t>, grid, block, kIpLdsBytes, stream, a);
-    else
-        DLP_LAUNCH_TIMED(ts, ip_stream_kernel<float>, grid, block, kIpLdsBytes, stream, a);
-    DLP_HIP_TRY(hipGetLastError());
-    return DLP_OK;
+    // batches of at most 16 rows keep 16 rows of x in LDS: three workgroups per compute unit instead of two
+    return dtype == DLP_BFLOAT16 ? ip_stream_dispatch<bf16_t>(batch <= 16, &a, grid, stream, &ts)
+                                 : ip_stream_dispatch<float>(batch <= 16, &a, grid, stream, &ts);
 }
 
 ConvGeom ip_gemm_geom(int batch, int inputs, int outputs, int dtype)

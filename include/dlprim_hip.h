@@ -264,8 +264,8 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op);
  * DLP_IP_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends.
  * The call makes no hipMalloc / hipFree and records no memset.  The array holds 64 KiB of tile counters and
  * 4 MiB of partial sums (4 KiB per tile of 32 outputs x 32 batch rows and K slice).  With rows on 16-byte
- * boundaries (the kernel that streams w through LDS) K is only cut while there are fewer than two workgroups
- * per compute unit, which keeps the partial sums under 4 MiB on an MI355X whatever the shape; other
+ * boundaries (the kernel that streams w through LDS) K is only cut while tiles x slices stay within 1024,
+ * which keeps the partial sums within 4 MiB whatever the shape; other
  * alignments cut K more freely, and a batch x outputs that then needs more is a validation error that
  * names both sizes (e.g. 1026 -> 4096 at batch 160: 5 MiB).  bfloat16 rows of odd length are NotImplemented.
  * RULE: at most one call in flight per device.  All calls on one device share the array, whatever the operator: two

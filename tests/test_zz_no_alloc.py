@@ -56,7 +56,7 @@ def test_two_calls_in_a_row_second_smaller(gpu, oracle_mod):
         np.testing.assert_allclose(got, oracle_mod.ip_forward(x, w, b, "relu"), rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("bio", [(1, 512, 1000), (16, 25088, 96), (33, 4100, 31), (3, 1030, 70), (2, 1, 1)], ids=lambda v: "b%d_%dto%d" % v)
+@pytest.mark.parametrize("bio", [(1, 512, 1000), (16, 25088, 96), (33, 4100, 31), (3, 1030, 70), (2, 1, 1), (16, 1024, 20000), (16, 2048, 16000)], ids=lambda v: "b%d_%dto%d" % v)
 def test_shapes_equal_the_allocating_entry_point(gpu, bio):
     import dlprimitives_amd as dlp
 
@@ -97,7 +97,7 @@ def test_sizes_beyond_the_array_are_rejected(gpu):
 
     # rows that do not start on 16-byte boundaries take the direct kernel, whose plan cuts K whatever the number of tiles:
     # 128 blocks of outputs x 5 chunks of batch rows = 640 tiles of 4 KiB x 2 K slices: 5 MiB of partial sums
-    # (the streaming kernel splits K only below two workgroups per compute unit: its partial sums stay under 4 MiB on this chip)
+    # (the streaming kernel keeps tiles x K slices within 1024, so its partial sums stay within 4 MiB: 16 x 1024 -> 20000 above)
     inputs, outputs, batch = 1026, 4096, 160
     op = dlp.IPForward.create(dlp.IPSettings(inputs, outputs, batch), False, "identity")
     x = torch.zeros((batch, inputs), device="cuda:0")
