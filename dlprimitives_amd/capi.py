@@ -230,7 +230,7 @@ class Conv2DForward:
 
     def enqueue(self, x, w, bias, y, ws=None, factor=0.0, stream=None):
         """x, w, bias, y, ws: torch device tensors (ws: uint8 of >= workspace() bytes)."""
-        xs = (ctypes.c_int * 4)(*x.shape)
+        xs = self._x_shape(x)
         ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
         _check(lib().dlp_conv2d_fwd_enqueue(self._h, xs, _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
                                             float(factor), _stream(stream)))
@@ -239,6 +239,20 @@ class Conv2DForward:
         """y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)"""
         lib().dlp_conv2d_fwd_set_accumulate_first.argtypes = [ctypes.c_void_p, ctypes.c_int]
         _check(lib().dlp_conv2d_fwd_set_accumulate_first(self._h, int(bool(on))))
+
+    def channels_last(self, x=False, y=False):
+        """dlp_conv2d_fwd_set_channels_last: the operator reads x / writes y as [image][row][column][channel] (bfloat16 gemm
+        only; NotImplementedError otherwise).  Call before workspace().  A channels-last x is passed to enqueue as a tensor
+        of shape [B, H, W, C]."""
+        lib().dlp_conv2d_fwd_set_channels_last.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+        _check(lib().dlp_conv2d_fwd_set_channels_last(self._h, int(bool(x)), int(bool(y))))
+        self._x_channels_last = bool(x)
+
+    def _x_shape(self, x):
+        """the [B, C, H, W] that the C interface takes, whatever the layout of x"""
+        if getattr(self, "_x_channels_last", False):
+            return (ctypes.c_int * 4)(int(x.shape[0]), self.settings.channels_in, self.settings.shape[2], self.settings.shape[3])
+        return (ctypes.c_int * 4)(*x.shape)
 
     def packed_size(self):
         """bytes of the buffer that pack() fills (0: nothing to transform)"""
@@ -256,7 +270,7 @@ class Conv2DForward:
         lib().dlp_conv2d_fwd_enqueue_packed.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float,
                                                         ctypes.c_void_p]
-        xs = (ctypes.c_int * 4)(*x.shape)
+        xs = self._x_shape(x)
         ws_bytes = ws.numel() * ws.element_size() if ws is not None else 0
         _check(lib().dlp_conv2d_fwd_enqueue_packed(self._h, xs, _ptr(x), _ptr(w), _ptr(packed), _ptr(bias), _ptr(y), _ptr(ws), ws_bytes,
                                                    float(factor), _stream(stream)))
@@ -513,8 +527,17 @@ class Pooling2DForward:
     def workspace(self):
         return 0
 
+    def channels_last(self, on=True):
+        """dlp_pool2d_fwd_set_channels_last (global pooling only): x is passed to enqueue as a tensor of shape [B, H, W, C]"""
+        lib().dlp_pool2d_fwd_set_channels_last.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        _check(lib().dlp_pool2d_fwd_set_channels_last(self._h, int(bool(on))))
+        self._channels_last = bool(on)
+
     def enqueue(self, x, y, stream=None):
-        xs = (ctypes.c_int * 4)(*x.shape)
+        if getattr(self, "_channels_last", False):
+            xs = (ctypes.c_int * 4)(int(x.shape[0]), int(x.shape[3]), int(x.shape[1]), int(x.shape[2]))
+        else:
+            xs = (ctypes.c_int * 4)(*x.shape)
         ys = (ctypes.c_int * 4)(*y.shape)
         lib().dlp_pool2d_fwd_enqueue.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.c_void_p,
                                                  ctypes.c_void_p, ctypes.c_void_p]

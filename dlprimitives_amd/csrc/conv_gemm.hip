@@ -84,6 +84,7 @@ struct GemmArgs {
     int pxv;                  // bf16 matrix-instruction kernels: pixels per output store (0 = one element per store)
     int pp_nbr;               // conv_patch_bf16_kernel: blocks of PXP rows in the largest patch of the launch
     int wdirect;              // conv_gemm_bf16_kernel: wp is the weight tensor itself (1x1 convolution), not packed tiles
+    int y_cl;                 // bf16 matrix-instruction kernels: y is [image][pixel][channel]
     int Cin, Cin_g, H, W, Cout, OW, OHW, groups;
     int sh, sw, ph, pw, dh, dw, KH, KW;
     uint32_t x_bytes, wp_bytes;
@@ -1053,6 +1054,100 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
         return;
     }
 
+    // ---- channels-last output, y[(image, pixel)][channel] (the host checks: no factor or accumulate_first, M a multiple of 8,
+    // y 16-byte aligned and below 2 GiB).  The tile goes to LDS as bf16 [n][m]: a lane's four consecutive accumulator rows are four
+    // consecutive channels of its pixel, one 8-byte LDS store (pixels 16 bytes more than BM channels apart: the lanes of a
+    // store hit different banks), and leaves in 16-byte pieces of 8 channels, BM / 8 consecutive lanes on the contiguous
+    // bytes of a pixel. ----
+    if (a.y_cl) {
+        constexpr int PITCH = BM * 2 + 16;
+        float *bias_s = (float *)(smem + BN * PITCH);
+        if (tid < BM)
+            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
+        __syncthreads();
+        const bool pre = a.pre != 0 && a.factor != 0.0f; // the old y joins before the activation: in the second phase
+        const bool clamp = a.act != DLP_ACT_IDENTITY && !pre;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            unsigned char *rowp = smem + (wn * WTN + j * 32 + l32) * PITCH + (wm * WTM + 4 * h) * 2;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const f32x4 bv = *(const f32x4 *)&bias_s[wm * WTM + i * 32 + 8 * rq + 4 * h];
+                    uint32_t bits[4];
+#pragma unroll
+                    for (int rr = 0; rr < 4; rr++) {
+                        float v = acc[i][j][4 * rq + rr] + bv[rr];
+                        if (ACT == ACT_CLAMP) {
+                            if (clamp)
+                                v = clamp_med3(v, a.clamp_lo, a.clamp_hi);
+                        } else if (!pre)
+                            v = apply_act(v, a.act);
+                        bits[rr] = to_bf16(v).bits;
+                    }
+                    u32x2 o;
+                    o[0] = bits[0] | (bits[1] << 16);
+                    o[1] = bits[2] | (bits[3] << 16);
+                    *(u32x2 *)(rowp + (i * 32 + 8 * rq) * 2) = o;
+                }
+            }
+        }
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        constexpr int PPR = BM / 8; // pieces of a pixel's row
+        static_assert((BN * PPR) % kThreads == 0 && kThreads % PPR == 0, "pieces are dealt to the threads evenly");
+        // every pixel's run is whole 128-byte lines, and the tensor is too large for the next layer to find it in the last-level cache:
+        // streaming stores
+        const bool streaming = (a.Cout & 63) == 0 && (BM & 63) == 0 && a.y_bytes >= (96u << 20);
+        const int piece = tid % PPR, pix_t = tid / PPR;
+        const int m = m0 + piece * 8;
+        const uint32_t col_off = (uint32_t)(g * a.M + m) * 2u;
+        const unsigned char *src_t = smem + pix_t * PITCH + piece * 16;
+        constexpr int STEP = kThreads / PPR;           // pixels between a thread's pieces
+        constexpr int PER_THREAD = BN * PPR / kThreads; // pieces per thread
+        static_assert(PER_THREAD % 4 == 0, "pieces are handled four at a time");
+#pragma unroll 1
+        for (int q0 = 0; q0 < PER_THREAD; q0 += 4) {
+            uint32_t voff[4];
+            u32x4 old[4], mine[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) { // the old values of four pieces are requested together: two waits for memory per tile, not eight
+                const int n = n0 + pix_t + (q0 + u) * STEP;
+                voff[u] = (n < a.N && m < a.M) ? (uint32_t)n * (uint32_t)a.Cout * 2u + col_off : kOutOfRange;
+                if (pre)
+                    old[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(yr, voff[u], 0, 0));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                mine[u] = *(const u32x4 *)(src_t + (q0 + u) * STEP * PITCH);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (pre) {
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        float lo = fmaf(__builtin_bit_cast(float, old[u][d] << 16), a.factor, __builtin_bit_cast(float, mine[u][d] << 16));
+                        float hi = fmaf(__builtin_bit_cast(float, old[u][d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[u][d] & 0xFFFF0000u));
+                        if (ACT == ACT_CLAMP) {
+                            if (a.act != DLP_ACT_IDENTITY) {
+                                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
+                            }
+                        } else {
+                            lo = apply_act(lo, a.act);
+                            hi = apply_act(hi, a.act);
+                        }
+                        mine[u][d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                    }
+                }
+                if (streaming)
+                    __builtin_amdgcn_raw_buffer_store_b128(mine[u], yr, voff[u], 0, DLP_BF16_STORE_AUX);
+                else
+                    __builtin_amdgcn_raw_buffer_store_b128(mine[u], yr, voff[u], 0, 0);
+            }
+        }
+        return;
+    }
     // ---- epilogue.  Fast path (no factor, M a multiple of 8, y below 2 GiB): the bias of the
     // tile's rows goes through LDS (free after the last barrier), the result is rounded by the
     // hardware conversion and stored with buffer stores whose row offset is scalar: a handful of
@@ -1659,6 +1754,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM ==
     }
 
     static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
+    static_assert(BN * (BM * 2 + 16) + BM * 4 <= (int)sizeof(smem), "and so does the channels-last one");
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, slice, wm, wn, h, l32, tid);
 }
 
@@ -1928,6 +2024,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     __syncthreads(); // the operand reads issued after the last barrier are done before LDS is reused
 
     static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
+    static_assert(BN * (BM * 2 + 16) + BM * 4 <= (int)sizeof(smem), "and so does the channels-last one");
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
 }
 
@@ -2047,6 +2144,52 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
             r = apply_act(r, a.act);
         store_out(yp, r, pre ? 0.0f : a.factor);
     }
+}
+
+// The same for a channels-last bf16 y: a thread sums eight consecutive channels of one pixel (consecutive threads on consecutive
+// pixels: the partial sums are read in whole lines) and writes them as one 16-byte piece.  Cout a multiple of 8.
+template <int ACT>
+__global__ __launch_bounds__(256) void splitk_reduce_cl_kernel(GemmArgs a)
+{
+    const int c0 = blockIdx.y * 8;
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= a.N)
+        return;
+    const size_t total = (size_t)a.Cout * a.N;
+    const float *pp = a.part + (size_t)c0 * a.N + n;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        v[i] = a.bias ? a.bias[c0 + i] : 0.0f;
+    for (int s = 0; s < a.splitk; s++)
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            v[i] += pp[(size_t)s * total + (size_t)i * a.N];
+    u32x4 *yp = (u32x4 *)((uint16_t *)a.y + (size_t)n * a.Cout + c0);
+    const bool pre = a.pre != 0 && a.factor != 0.0f;
+    u32x4 old = {0u, 0u, 0u, 0u};
+    if (pre)
+        old = *yp;
+    u32x4 out;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        float lo = v[2 * d], hi = v[2 * d + 1];
+        if (pre) {
+            lo = fmaf(__builtin_bit_cast(float, old[d] << 16), a.factor, lo);
+            hi = fmaf(__builtin_bit_cast(float, old[d] & 0xFFFF0000u), a.factor, hi);
+        }
+        if (ACT == ACT_CLAMP) {
+            if (a.act != DLP_ACT_IDENTITY) {
+                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
+            }
+        } else {
+            lo = apply_act(lo, a.act);
+            hi = apply_act(hi, a.act);
+        }
+        out[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+    }
+    *yp = out;
 }
 
 // Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
@@ -2422,12 +2565,16 @@ struct XtGeom {
 };
 XtGeom xt_geom(const ConvGeom &g)
 {
+    if (g.x_channels_last) // the input itself, as it lies
+        return {g.H, g.W, 1, 1};
     if (g.KH == 1 && g.KW == 1 && g.ph == 0 && g.pw == 0)
         return {g.OH, g.OW, g.sh, g.sw};
     return {g.H, g.W, 1, 1};
 }
 size_t xt_bytes(const ConvGeom &g, int batch)
 {
+    if (g.x_channels_last) // no copy
+        return 0;
     const XtGeom t = xt_geom(g);
     return ((size_t)batch * t.H * t.W * g.Cin * sizeof(bf16_t) + 255) / 256 * 256;
 }
@@ -2439,6 +2586,7 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     if (xt != nullptr) {
         const XtGeom t = xt_geom(g);
+        if (!g.x_channels_last) {
         StageArgs sa;
         sa.x = (const uint16_t *)a.x;
         sa.xt = (uint16_t *)xt;
@@ -2457,6 +2605,7 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
                 DLP_LAUNCH_TIMED(ts, stage_channels_last_kernel<2>, grid64, dim3(256), 0, stream, sa);
             else
                 DLP_LAUNCH_TIMED(ts, stage_channels_last_kernel<0>, grid64, dim3(256), 0, stream, sa);
+        }
         }
         // the convolution the matrix kernel now sees: the copy as input, strides that the copy has taken over set to 1
         a.x = xt;
@@ -2477,7 +2626,10 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         TimingScope ts("splitk_reduce", stream);
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
-        hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
+        if (a.y_cl)
+            hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP>), dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.Cout / 8)), dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
     }
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
@@ -2713,6 +2865,11 @@ GemmPlan conv_gemm_plan(const ConvGeom &g, int activation)
                 p.pp_nbr = nbr;
             }
         }
+        if (g.x_channels_last) { // (conv_gemm_layouts_supported has checked tap_major) the channels-last loader, on x as it lies
+            p.dense_pxl = 0;
+            p.dense_sx = 1;
+            p.patch_bf16 = 0;
+        }
         // everything else in the tap-major order (strided and dilated kernels, odd image sizes): channels-last staging
         p.xt = tap_major && p.dense_pxl == 0 && p.patch_bf16 == 0 && g.Cin <= 65535 * 64 &&
                (size_t)g.H * g.W * g.Cin * sizeof(bf16_t) < kOutOfRange / 2;
@@ -2888,6 +3045,22 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
     return DLP_OK;
 }
 
+// Channels-last x and / or y: served by the bf16 matrix-instruction kernels only (x: the channels-last loader, i.e. input
+// channels per group in multiples of 32 and a kernel extent the tap masks hold; y: output channels per group in eights).
+bool conv_gemm_layouts_supported(const ConvGeom &g, int activation)
+{
+    if (!g.x_channels_last && !g.y_channels_last)
+        return true;
+    const GemmPlan p = conv_gemm_plan(g, activation);
+    if (!bf16_mfma_order(p.order) || p.stem || p.pointwise || p.patch)
+        return false;
+    if (g.x_channels_last && !p.xt)
+        return false;
+    if (g.y_channels_last && (p.M & 7) != 0)
+        return false;
+    return true;
+}
+
 size_t conv_gemm_counter_count(const ConvGeom &g, const GemmPlan &p)
 {
     if (g.B <= 0 || bf16_mfma_order(p.order) || p.stem)
@@ -2911,6 +3084,9 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
+    if (!conv_gemm_layouts_supported(g, ep.activation))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: served by the bf16 matrix-instruction kernels only (input channels per group in "
+                                             "multiples of 32 for x, output channels per group in eights for y)");
     if (p.stem) {
         if (w == nullptr || n_valid >= 0)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "stem convolution: needs the weight tensor and the whole batch");
@@ -2973,7 +3149,11 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         return launch_patch(g, p, a, stream, part_ws, part_bytes, own_counters);
     // workspace behind the packed weights, bf16 kernels: channels-last copy of the input | split-K partial sums
     void *xt = nullptr;
-    if (p.xt && part_ws != nullptr && part_bytes >= xt_bytes(g, g.B) && ((uintptr_t)part_ws & 15) == 0 && n_valid < 0 &&
+    if (g.x_channels_last) {
+        if (!p.xt || n_valid >= 0 || ((uintptr_t)x & 15) != 0 || x_elems * esize + ((size_t)g.ph * g.W + g.pw) * g.Cin * esize >= kOutOfRange)
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last input: needs the bf16 matrix-instruction kernel, a 16-byte aligned x below 2 GiB and the whole batch");
+        xt = const_cast<void *>(x);
+    } else if (p.xt && part_ws != nullptr && part_bytes >= xt_bytes(g, g.B) && ((uintptr_t)part_ws & 15) == 0 && n_valid < 0 &&
         xt_bytes(g, g.B) + ((size_t)g.ph * g.W + g.pw) * g.Cin * esize < kOutOfRange) {
         xt = part_ws;
         part_ws = (char *)part_ws + xt_bytes(g, g.B);
@@ -2998,9 +3178,16 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     }
 
     a.pxv = 0;
+    a.y_cl = 0;
+    if (g.y_channels_last) {
+        if (!bf16_mfma_order(p.order) || (p.M & 7) != 0 || a.y_bytes == 0 || ((uintptr_t)y & 15) != 0 || !(ep.factor == 0.0f || ep.accumulate_first))
+            return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last output: needs the bf16 matrix-instruction kernel, output channels per group in eights, a 16-byte "
+                                                 "aligned y below 2 GiB, and factor 0 or accumulate_before_activation");
+        a.y_cl = 1;
+    }
     if (bf16_mfma_order(p.order)) {
         // wide output stores: runs of 8, 4 or 2 pixels that stay inside one image, dword aligned
-        if ((ep.factor == 0.0f || ep.accumulate_first) && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1)
+        if ((ep.factor == 0.0f || ep.accumulate_first) && a.y_bytes != 0 && ((uintptr_t)y & 3) == 0 && a.splitk == 1 && !a.y_cl)
             a.pxv = a.OHW % 8 == 0 ? 8 : a.OHW % 4 == 0 ? 4 : a.OHW % 2 == 0 ? 2 : 0;
         // dense loader (1x1, stride 1, no padding): runs of 8 or 4 input pixels, dword aligned
         if (p.patch_bf16 && ((uintptr_t)x & 3) == 0)

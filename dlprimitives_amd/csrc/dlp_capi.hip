@@ -113,6 +113,7 @@ struct dlp_conv2d_fwd {
     size_t workspace;
     int packed_layout[6]; // of the last dlp_conv2d_fwd_pack: order, BM, K tiles, m tiles, patch, in-place
     int accumulate_first; // y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)
+    int x_channels_last, y_channels_last; // tensor layouts of the gemm algorithm on bf16 tensors (dlp_conv2d_fwd_set_channels_last)
     int *counters;        // GEMM stage: tile counters of split-K / stream-K launches, zero between launches
     size_t counter_count;
 };
@@ -136,6 +137,16 @@ static int own_counters(dlp_conv2d_fwd *op, const ConvGeom &g, const GemmPlan &p
 }
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+static int make_geom(const dlp_conv2d_settings &c, const int x_shape[4], ConvGeom &g);
+// geometry of an operator's convolution on an input of this shape, with the operator's tensor layouts
+static int op_geom(const dlp_conv2d_fwd *op, const int x_shape[4], ConvGeom &g)
+{
+    const int rc = make_geom(op->cfg, x_shape, g);
+    g.x_channels_last = op->x_channels_last;
+    g.y_channels_last = op->y_channels_last;
+    return rc;
+}
 
 struct dlp_ip_fwd {
     dlp_ip_settings cfg;
@@ -540,6 +551,8 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     for (int i = 0; i < 6; i++)
         op->packed_layout[i] = -1;
     op->accumulate_first = 0;
+    op->x_channels_last = 0;
+    op->y_channels_last = 0;
     op->counters = nullptr;
     op->counter_count = 0;
     if (hipGetDevice(&op->device) != hipSuccess)
@@ -590,7 +603,7 @@ int dlp_conv2d_fwd_enqueue(dlp_conv2d_fwd *op, const int x_shape[4], const void 
     // bias pointer present iff created with bias (src/gemm.cpp:526-533)
     DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
     ConvGeom g;
-    int rc = make_geom(op->cfg, x_shape, g);
+    int rc = op_geom(op, x_shape, g);
     if (rc != DLP_OK)
         return rc;
     if (g.B == 0)
@@ -645,6 +658,38 @@ int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on)
     return DLP_OK;
 }
 
+int dlp_conv2d_fwd_set_channels_last(dlp_conv2d_fwd *op, int x_channels_last, int y_channels_last)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    x_channels_last = x_channels_last ? 1 : 0;
+    y_channels_last = y_channels_last ? 1 : 0;
+    if (x_channels_last == op->x_channels_last && y_channels_last == op->y_channels_last)
+        return DLP_OK;
+    if ((x_channels_last || y_channels_last) && op->algo != ALGO_GEMM)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: algorithm gemm on bfloat16_data only");
+    ConvGeom g;
+    int rc = make_geom(op->cfg, op->cfg.shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    g.x_channels_last = x_channels_last;
+    g.y_channels_last = y_channels_last;
+    if (!conv_gemm_layouts_supported(g, op->activation))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: served by the bf16 matrix-instruction kernels only (bfloat16_data, relu-like or no "
+                                             "activation, input channels per group in multiples of 32 for x, output channels per group in eights for y)");
+    // the gather table and the workspace depend on the layout of x: build them anew
+    KTabEntry *ktab = nullptr;
+    rc = upload_ktab(g, op->activation, &ktab);
+    if (rc != DLP_OK)
+        return rc;
+    if (op->ktab)
+        (void)hipFree(op->ktab); // synchronises with the launches that still read the old table
+    op->ktab = ktab;
+    op->x_channels_last = x_channels_last;
+    op->y_channels_last = y_channels_last;
+    op->workspace = conv_gemm_workspace_bytes(g, op->activation);
+    return DLP_OK;
+}
+
 size_t dlp_conv2d_fwd_packed_bytes(const dlp_conv2d_fwd *op)
 {
     if (!op)
@@ -654,7 +699,7 @@ size_t dlp_conv2d_fwd_packed_bytes(const dlp_conv2d_fwd *op)
     if (op->algo == ALGO_DEPTHWISE)
         return 0;
     ConvGeom g;
-    if (make_geom(op->cfg, op->cfg.shape, g) != DLP_OK)
+    if (op_geom(op, op->cfg.shape, g) != DLP_OK)
         return 0;
     return round256(conv_gemm_plan(g, op->activation).wpack_bytes);
 }
@@ -666,7 +711,7 @@ int dlp_conv2d_fwd_pack(dlp_conv2d_fwd *op, const void *w, void *packed, void *s
         return DLP_OK; // the kernel reads the filter as it is
     DLP_REQUIRE(packed != nullptr, "null buffer for the packed weights");
     ConvGeom g;
-    int rc = make_geom(op->cfg, op->cfg.shape, g);
+    int rc = op_geom(op, op->cfg.shape, g);
     if (rc != DLP_OK)
         return rc;
     if (op->algo == ALGO_WINOGRAD) {
@@ -687,7 +732,7 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
                 "input shape differs from the shape given at create (only the batch may change)");
     DLP_REQUIRE((bias != nullptr) == op->bias, "bias pointer must be given exactly when the op was created with bias");
     ConvGeom g;
-    int rc = make_geom(op->cfg, x_shape, g);
+    int rc = op_geom(op, x_shape, g);
     if (rc != DLP_OK)
         return rc;
     if (g.B == 0)
@@ -967,3 +1012,4 @@ void dlp_ip_fwd_destroy(dlp_ip_fwd *op)
 }
 
 } // extern "C"
+

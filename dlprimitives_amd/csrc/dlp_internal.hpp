@@ -56,6 +56,9 @@ struct ConvGeom {
     int sh, sw, ph, pw, dh, dw;
     int groups;
     int dtype; // DLP_FLOAT / DLP_BFLOAT16 / DLP_HALF
+    // tensor layouts of the implicit-GEMM convolution on the bf16 matrix instruction: x and / or y as [image][pixel][channel]
+    // instead of [image][channel][pixel] (the reference knows the latter only: src/core/conv.cpp works on NCHW throughout)
+    int x_channels_last = 0, y_channels_last = 0;
 };
 
 // Fused epilogue: v = act(acc + bias[c]); y = factor != 0 ? factor*y + v : v
@@ -203,6 +206,7 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 // Tile counters a launch at this batch may use (0: none).  A caller that keeps that many zeroed ints per operator and
 // hands them to conv_gemm_launch as own_counters saves the clearing before every launch: the kernels leave them at zero.
 // Such an operator must not run on two streams at once.
+bool conv_gemm_layouts_supported(const ConvGeom &g, int activation);
 size_t conv_gemm_counter_count(const ConvGeom &g, const GemmPlan &p);
 // n_valid >= 0 limits the GEMM N dimension (output pixels computed) below B*OH*OW.
 // part_ws/part_bytes: optional split-K workspace; without it the launch runs unsplit.

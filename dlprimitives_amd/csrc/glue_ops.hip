@@ -247,6 +247,26 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const T *__restrict__ 
         store_plain(y + plane, mode == 0 ? v : v * (1.0f / plane_size));
 }
 
+// Global pooling of a channels-last x ([image][pixel][channel]): one thread per (image, channel), consecutive threads on
+// consecutive channels (every load of a wavefront is one run of a pixel's channels), a single running sum in pixel order as
+// in the reference (src/kernels/global_pooling.cl accumulates the same way per plane).
+template <class T>
+__global__ __launch_bounds__(256) void global_pool_cl_kernel(const T *__restrict__ x, T *__restrict__ y, int batch, int channels, int plane_size,
+                                                             int mode)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long long)batch * channels)
+        return;
+    const int b = (int)(i / channels), c = (int)(i - (long long)b * channels);
+    const T *src = x + (size_t)b * plane_size * channels + c;
+    float v = mode == 0 ? -3.402823466e+38f : 0.0f;
+    for (int p = 0; p < plane_size; p++) {
+        const float t = to_float(src[(size_t)p * channels]);
+        v = mode == 0 ? fmaxf(v, t) : v + t;
+    }
+    store_plain(y + i, mode == 0 ? v : v * (1.0f / plane_size));
+}
+
 __device__ __forceinline__ float eltwise_one(float x0, float x1, int op, float c1, float c2, int act)
 {
     float r;
@@ -466,6 +486,7 @@ struct dlp_pool2d_fwd {
     int count_include_pad;
     int global;
     int dtype;
+    int channels_last; // global pooling: x is [image][pixel][channel]
 };
 
 static int pool_create(const int kernel[2], const int pad[2], const int stride[2], int mode, int cip, int global, int dtype,
@@ -541,6 +562,15 @@ int dlp_pool2d_fwd_create_global_max(int dtype, dlp_pool2d_fwd **out) { return p
 
 int dlp_pool2d_fwd_create_global_avg(int dtype, dlp_pool2d_fwd **out) { return pool_create(nullptr, nullptr, nullptr, 1, 0, 1, dtype, out); }
 
+int dlp_pool2d_fwd_set_channels_last(dlp_pool2d_fwd *op, int on)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    if (on && !op->global)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last input: global pooling only");
+    op->channels_last = on ? 1 : 0;
+    return DLP_OK;
+}
+
 int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y_shape[4], const void *x, void *y, void *stream)
 {
     DLP_REQUIRE(op != nullptr && x_shape != nullptr && y_shape != nullptr, "null argument");
@@ -555,6 +585,17 @@ int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y
         const long long plane_size = (long long)x_shape[2] * x_shape[3];
         DLP_REQUIRE(plane_size > 0 && plane_size < 0x7fffffffLL, "plane size");
         TimingScope ts("global_pooling", s);
+        if (op->channels_last) {
+            const unsigned cl_grid = (unsigned)((planes + 255) / 256);
+            if (op->dtype == DLP_BFLOAT16)
+                hipLaunchKernelGGL((global_pool_cl_kernel<bf16_t>), dim3(cl_grid), dim3(256), 0, s, (const bf16_t *)x, (bf16_t *)y, x_shape[0], x_shape[1],
+                                   (int)plane_size, op->mode);
+            else
+                hipLaunchKernelGGL((global_pool_cl_kernel<float>), dim3(cl_grid), dim3(256), 0, s, (const float *)x, (float *)y, x_shape[0], x_shape[1],
+                                   (int)plane_size, op->mode);
+            DLP_HIP_TRY(hipGetLastError());
+            return DLP_OK;
+        }
         const bool small = plane_size <= 64;
         const unsigned grid = (unsigned)((planes + (small ? 15 : 3)) / (small ? 16 : 4));
         if (op->dtype == DLP_BFLOAT16) {

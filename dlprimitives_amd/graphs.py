@@ -114,14 +114,17 @@ def infer_shapes(ops, in_shape):
 class GraphRunner:
     """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
 
-    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False, prepack=False):
+    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False, prepack=False, channels_last=False):
         """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32).
         fuse_residual: a residual sum whose later branch is a 1x1 convolution runs in that convolution's epilogue
         (dlp_conv2d_fwd_set_accumulate_first: y = act(conv + bias + y) written over the other branch), which is what
         dlprim::Net does with the same graphs; 3x3 convolutions keep their sum as an operator.
         prepack: the filters are transformed once here (dlp_conv2d_fwd_pack) and forward() calls enqueue_packed, as a
         network with constant weights does (dlprim::Net::copy_parameters_to_device); otherwise every enqueue transforms
-        its filter again, which is the contract of the reference's enqueue."""
+        its filter again, which is the contract of the reference's enqueue.
+        channels_last (bfloat16, algorithm gemm): tensors between convolutions are kept as [image][row][column][channel]
+        wherever every operator that touches them can take that layout and one of the readers is faster on it
+        (dlp_conv2d_fwd_set_channels_last; see _plan_layouts).  Input, logits and parameters keep their layout."""
         import torch
 
         import dlprimitives_amd as dlp
@@ -135,7 +138,9 @@ class GraphRunner:
         self.shapes = infer_shapes(ops, in_shape)
         tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
         code = BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA
-        self.t = {n: torch.empty(s, dtype=tdt, device="cuda:0") for n, s in self.shapes.items() if n not in alias}
+        self.cl = self._plan_layouts(ops, alias, self.shapes) if (channels_last and dtype == "bfloat16" and algo in ("", "auto", "gemm")) else set()
+        stored = lambda n, s: (s[0], s[2], s[3], s[1]) if n in self.cl else s
+        self.t = {n: torch.empty(stored(n, s), dtype=tdt, device="cuda:0") for n, s in self.shapes.items() if n not in alias}
         for n in self.shapes:  # the output of a fused sum lies over the branch it was added to (chains of blocks: follow the aliases)
             if n in alias:
                 m = alias[n]
@@ -152,6 +157,8 @@ class GraphRunner:
                 op = dlp.Conv2DForward.create(st, True, o["act"], algo)
                 if o.get("residual"):
                     op.accumulate_before_activation(True)
+                if o["src"] in self.cl or o["dst"] in self.cl:
+                    op.channels_last(o["src"] in self.cl, o["dst"] in self.cl)
                 ws_bytes = max(ws_bytes, op.workspace())
                 if prepack:
                     buf = torch.empty(max(op.packed_size(), 1), dtype=torch.uint8, device="cuda:0")
@@ -161,6 +168,8 @@ class GraphRunner:
                 op = dlp.Pooling2DForward.create_max_pooling(o["k"], o["p"], o["s"], dtype=code)
             elif o["op"] == "gap":
                 op = dlp.Pooling2DForward.create_global_avg_pooling(dtype=code)
+                if o["src"] in self.cl:
+                    op.channels_last(True)
             elif o["op"] == "ip":
                 op = dlp.IPForward.create(dlp.IPSettings(o["inputs"], o["outputs"], in_shape[0], dtype=code), True, "identity")
             else:
@@ -168,6 +177,43 @@ class GraphRunner:
             self.k.append(op)
         # one workspace shared by all operators, as the reference's Net does
         self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda:0")
+
+    @staticmethod
+    def _plan_layouts(ops, alias, shapes):
+        """Names of the tensors kept channels-last.  Tensors that share memory (the output of a fused residual sum lies over the
+        branch it was added to) share a layout.  A group becomes channels-last when every operator that writes it is a
+        convolution that can (channels in multiples of 32 in, of 8 out: the bf16 matrix-instruction kernel with K tiles of one
+        filter tap), every reader is such a convolution or the global pooling, and at least one reader gains: measured inside
+        ResNet-50 at batch 128, the channels-last loader beats the others on 1x1 layers of more than 64 input channels, on
+        everything with a stride and on 7 x 7 images, and loses to the LDS-patch kernel on 3x3 stride-1 layers of larger images
+        (14 x 14: 43 against 48 us) and to the dense loader on 1x1 layers of 64 channels (52 against 55 us)."""
+        def root(n):
+            while n in alias:
+                n = alias[n]
+            return n
+
+        def conv_ok(o):
+            return o["op"] == "conv" and o["cin"] % 32 == 0 and o["cout"] % 8 == 0
+
+        def gains(o):
+            if o["op"] != "conv":
+                return False
+            _, _, h, w = shapes[o["src"]]
+            if o["k"] == 3 and o["s"] == 1:
+                return h * w < 14 * 14
+            return not (o["k"] == 1 and o["s"] == 1 and o["cin"] <= 64)
+
+        writers, readers = {}, {}
+        for o in ops:
+            for n in (o["src"] if isinstance(o["src"], list) else [o["src"]]):
+                readers.setdefault(root(n), []).append(o)
+            writers.setdefault(root(o["dst"]), []).append(o)
+        chosen = set()
+        for g, ws in writers.items():
+            rs = readers.get(g, [])
+            if all(conv_ok(o) for o in ws) and rs and all(conv_ok(o) or o["op"] == "gap" for o in rs) and any(gains(o) for o in rs):
+                chosen.add(g)
+        return {n for n in shapes if root(n) in chosen}
 
     @staticmethod
     def _fuse_residual_sums(ops, alias):

@@ -172,6 +172,18 @@ int dlp_conv2d_fwd_enqueue_packed(dlp_conv2d_fwd *op, const int x_shape[4], cons
  * block, factor 1 gives act(conv + bias + branch) in one pass.  "gemm" and "winograd". */
 int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
 
+/* Tensor layouts.  No counterpart in the reference, whose tensors are [image][channel][row][column] throughout
+ * (src/core/conv.cpp).  With x_channels_last (y_channels_last) the operator reads x (writes y, and reads the old y
+ * of a factor) as [image][row][column][channel]; weights and bias keep their layout.  For chains of bfloat16
+ * convolutions: on the bf16 matrix instruction a channels-last input is loaded the way the weights are (16-byte
+ * pieces of one pixel's channels) instead of being transposed on the way in, and a channels-last output leaves in
+ * runs of a whole tile of channels per pixel.  Served: algorithm "gemm", bfloat16_data, activations identity / relu /
+ * relu6; x: input channels per group a multiple of 32 and x 16-byte aligned; y: output channels per group a multiple
+ * of 8, y 16-byte aligned, factor 0 or accumulate_first.  Anything else: DLP_ERR_NOT_IMPLEMENTED, here or (alignment,
+ * factor) from enqueue, and the operator stays as it was.  Call before workspace(): the workspace size depends on the
+ * layout of x (no channels-last copy of the input is staged). */
+int dlp_conv2d_fwd_set_channels_last(dlp_conv2d_fwd *op, int x_channels_last, int y_channels_last);
+
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
 /* ---- Depthwise 3x3 convolution followed by a pointwise (1x1) convolution in one launch.  No counterpart in the
@@ -295,6 +307,9 @@ int dlp_pool2d_fwd_create_global_avg(int dtype, dlp_pool2d_fwd **out);
  * x [B,C,H,W] -> y [B,C,OH,OW]; the output shape (from dlp_pool2d_output_size, with or
  * without ceil_mode) is the caller's, as in the reference; global variants need [B,C,1,1]. */
 int dlp_pool2d_fwd_enqueue(dlp_pool2d_fwd *op, const int x_shape[4], const int y_shape[4], const void *x, void *y, void *stream);
+/* Global pooling of a channels-last x ([image][row][column][channel], as dlp_conv2d_fwd_set_channels_last writes it); x_shape stays
+ * [B, C, H, W] and y is [B, C, 1, 1] either way.  No counterpart in the reference.  Other pooling: DLP_ERR_NOT_IMPLEMENTED. */
+int dlp_pool2d_fwd_set_channels_last(dlp_pool2d_fwd *op, int on);
 void dlp_pool2d_fwd_destroy(dlp_pool2d_fwd *op);
 
 /* The copy behind Concat::forward and Slice::forward (core::SliceCopy::tensor_slice_copy with target_scale 0,

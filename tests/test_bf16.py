@@ -223,6 +223,131 @@ def test_bf16_dense_1x1_with_old_y(oracle_mod, c, bhw):
                                atol=2 ** -8 * np.abs(conv).max())
 
 
+# Channels-last tensors (dlp_conv2d_fwd_set_channels_last): x and / or y as [image][row][column][channel].  Every loader that
+# can feed a channels-last output (dense 1x1, LDS patch, staged copy) and the channels-last loader on every kind of geometry.
+CHANNELS_LAST_CASES = [
+    (case(1, 0, 1, 1, 1024, 256, True, 1, True), (3, 14, 14)),    # long K, tiles crossing images, pixel tail
+    (case(1, 0, 1, 1, 64, 256, True, 1, True), (2, 56, 56)),      # two K tiles, many pixel tiles
+    (case(1, 0, 1, 1, 256, 64, False, 1, False), (3, 14, 14)),    # 64 x 256 tiles
+    (case(1, 0, 1, 1, 64, 80, True, 1, True), (3, 8, 8)),         # output channels off the tile size
+    (case(1, 0, 1, 1, 128, 96, True, 2, False), (3, 6, 6)),       # two groups
+    (case(1, 0, 1, 1, 2048, 512, True, 1, True), (3, 7, 7)),      # split over K slices: the channels-last reduction
+    (case(1, 0, 2, 1, 256, 512, True, 1, False), (2, 28, 28)),    # 1x1 stride 2 read in place
+    (case(1, 0, 2, 1, 64, 128, True, 1, True), (3, 15, 15)),      # ... on an odd image
+    (case(3, 1, 2, 1, 128, 128, True, 1, True), (2, 28, 28)),     # 3x3 stride 2
+    (case(3, 1, 1, 1, 128, 128, True, 1, True), (3, 28, 28)),     # 3x3 stride 1: LDS-patch kernel unless x is channels-last
+    (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),       # 7x7 planes, split-K
+    (case(3, (2, 0), (1, 2), (2, 1), 64, 96, True, 2, True), (2, 11, 14)),  # groups, dilation, uneven padding and stride together
+    (case(5, 2, 1, 1, 32, 48, True, 1, False), (2, 9, 9)),        # 25 taps
+]
+
+
+@pytest.mark.parametrize("layouts", [(True, False), (False, True), (True, True)], ids=["x", "y", "xy"])
+@pytest.mark.parametrize("c,bhw", CHANNELS_LAST_CASES, ids=case_id)
+def test_bf16_channels_last(oracle_mod, c, bhw, layouts):
+    print("channels-last", layouts, c["cin"], c["cout"], c["kernel"], c["stride"], bhw, flush=True)
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    x_cl, y_cl = layouts
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    x, w, bias = make_tensors(c, bhw, seed=77)
+    x, w = oracle_mod.bf16_round(x), oracle_mod.bf16_round(w)
+    conv = oracle_mod.conv2d_forward(x, w, bias, cfg, "identity", threads=8)
+    want = oracle_mod.apply_activation(conv, c["activation"])
+    st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
+    bd = torch.from_numpy(bias).cuda() if bias is not None else None
+    xd = _bf(x.transpose(0, 2, 3, 1)) if x_cl else _bf(x)
+
+    def run(op, old=None, factor=0.0):
+        ws = torch.empty(max(op.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+        if old is None:
+            y = torch.full(want.shape, float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        else:
+            y = _bf(old)
+        if y_cl:
+            y = y.permute(0, 2, 3, 1).contiguous()
+        op.enqueue(xd, _bf(w), bd, y, ws, factor)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+        return got.transpose(0, 3, 1, 2) if y_cl else got
+
+    op = dlp.Conv2DForward.create(st, bias is not None, c["activation"], "gemm")
+    op.channels_last(x_cl, y_cl)
+    got = run(op)
+    assert not np.isnan(got).any()
+    np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-4 * np.abs(want).max())
+    # the residual form y = act(conv + factor * y_old), the old y in the layout of the new one
+    op.accumulate_before_activation(True)
+    old = np.random.default_rng(5).standard_normal(want.shape).astype(np.float32)
+    got = run(op, old, 0.5)
+    pre = conv + 0.5 * oracle_mod.bf16_round(old)
+    np.testing.assert_allclose(got, oracle_mod.apply_activation(pre.astype(np.float32), c["activation"]), rtol=2 ** -8,
+                               atol=2 ** -8 * np.abs(conv).max())
+    # integer-valued tensors: every product and sum is exact, the result must equal the reference bit for bit
+    rng = np.random.default_rng(4)
+    xi = rng.integers(-2, 3, x.shape).astype(np.float32)
+    wi = rng.integers(-1, 2, w.shape).astype(np.float32)
+    wanti = oracle_mod.conv2d_forward(xi, wi, bias * 0 if bias is not None else None, cfg, c["activation"], threads=8)
+    if np.abs(wanti).max() <= 256:  # exactly representable in bf16
+        op.accumulate_before_activation(False)
+        xd = _bf(xi.transpose(0, 2, 3, 1)) if x_cl else _bf(xi)
+        w = wi
+        bd = torch.zeros_like(bd) if bd is not None else None
+        assert np.array_equal(run(op), wanti)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_global_pooling_channels_last(dtype):
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA, NotImplementedErrorDlprim
+
+    tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    code = BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA
+    rng = np.random.default_rng(2)
+    for shape in [(3, 2048, 7, 7), (2, 72, 5, 9), (1, 8, 1, 1)]:
+        x = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).cuda().to(tdt)
+        for make in (dlp.Pooling2DForward.create_global_avg_pooling, dlp.Pooling2DForward.create_global_max_pooling):
+            want = torch.empty((shape[0], shape[1], 1, 1), dtype=tdt, device="cuda:0")
+            make(dtype=code).enqueue(x, want)
+            op = make(dtype=code)
+            op.channels_last(True)
+            got = torch.full_like(want, float("nan"))
+            op.enqueue(x.permute(0, 2, 3, 1).contiguous(), got)
+            torch.cuda.synchronize()
+            # the same fp32 sums in another order, rounded to the storage type once
+            np.testing.assert_allclose(got.float().cpu().numpy(), want.float().cpu().numpy(), rtol=2 ** -7 if dtype == "bfloat16" else 1e-5, atol=1e-6)
+    with pytest.raises(NotImplementedErrorDlprim):
+        dlp.Pooling2DForward.create_max_pooling(3, 1, 2, dtype=code).channels_last(True)
+
+
+def test_bf16_channels_last_is_refused_where_not_served(oracle_mod):
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA, NotImplementedErrorDlprim
+
+    def op_of(cin, cout, k, dtype, act="relu", algo="gemm", groups=1, hw=14):
+        st = dlp.Conv2DSettings(cin, cout, k, 1, 1, k // 2, groups, (2, cin, hw, hw), dtype=dtype)
+        return dlp.Conv2DForward.create(st, True, act, algo)
+
+    with pytest.raises(NotImplementedErrorDlprim):
+        op_of(64, 64, 1, FLOAT_DATA).channels_last(True, True)       # float tensors
+    with pytest.raises(NotImplementedErrorDlprim):
+        op_of(48, 64, 1, BFLOAT16_DATA).channels_last(True, False)   # input channels off 32
+    with pytest.raises(NotImplementedErrorDlprim):
+        op_of(64, 36, 1, BFLOAT16_DATA).channels_last(False, True)   # output channels off 8
+    with pytest.raises(NotImplementedErrorDlprim):
+        op_of(64, 64, 1, BFLOAT16_DATA, act="tanh").channels_last(True, True)
+    with pytest.raises(NotImplementedErrorDlprim):
+        op_of(64, 64, 3, BFLOAT16_DATA, algo="winograd").channels_last(True, True)
+    op = op_of(48, 64, 1, BFLOAT16_DATA)
+    op.channels_last(False, True)  # the output alone is served
+    op.channels_last(False, False)
+
+
 def test_bf16_factor_contract(oracle_mod):
     c = case(3, 1, 1, 1, 16, 24, True, 1, True)
     x, w, bias = make_tensors(c, (2, 11, 9), seed=5)
@@ -355,3 +480,16 @@ def test_resnet50_bf16_benchmarked_deployment_logits(oracle_mod):
     print("resnet50 bf16 b128, sums fused, filters packed once: max relative error of 4 logit rows %.4f" % rel)
     assert rel <= 1e-2
     assert (got.argmax(1) == want.argmax(1)).all()
+    # the same deployment with the tensors between convolutions kept channels-last wherever the planner finds it pays
+    del runner
+    runner = graphs.GraphRunner(ops, params, x.shape, algo="gemm", dtype="bfloat16", fuse_residual=True, prepack=True, channels_last=True)
+    assert len(runner.cl) >= 25, sorted(runner.cl)  # about half of the tensors between the 53 convolutions
+    assert "data" not in runner.cl and "stem" not in runner.cl and "logits" not in runner.cl
+    cl_first = runner.forward(xd).float().cpu().numpy()
+    cl_again = runner.forward(xd).float().cpu().numpy()
+    assert np.array_equal(cl_first, cl_again)
+    rel_cl = np.abs(cl_first[pick] - want).max() / np.abs(want).max()
+    print("... channels-last (%d tensors): max relative error %.4f; against the run above %.4f" %
+          (len(runner.cl), rel_cl, np.abs(cl_first - first).max() / np.abs(want).max()))
+    assert rel_cl <= 1e-2
+    assert (cl_first[pick].argmax(1) == want.argmax(1)).all()
