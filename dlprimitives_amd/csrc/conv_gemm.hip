@@ -1772,28 +1772,28 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM ==
 // (lane's patch row + (ky-1)*W + (kx-1)); taps that fall into the padding read a row that is always zero.  Compared with gathering every tap from memory with
 // 16-bit loads this is 9 * 8 times fewer trips through the texture path, which is what bounds that
 // kernel.  Runs start on multiples of PXP pixels of their plane (H*W % PXP == 0), so every load is
-// dword aligned.  Weights: the packed tap-major tiles of conv_gemm_bf16_kernel (K tile = stage * 9 + tap).
+// dword aligned.  Weights: the packed tap-major tiles of conv_gemm_bf16_kernel (K tile = stage * 9 + tap), read from memory
+// straight into the matrix instruction's registers (a wavefront owns 32 filters and all the pixels of the tile: WM x WN = 4 x 1
+// on the 128 x 128 tile, 2 x 2 on 64 x 256), so that the patch is the only thing ever stored to LDS and a stage needs one barrier.
 template <int BM, int BN, int WM, int WN, int PITCH, int PXP, int ACT>
 __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
 {
     constexpr int KHW = 9;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int A_V4 = BM * BK2 * 2 / 16; // 16-byte pieces of a packed A tile
-    static_assert(A_V4 % kThreads == 0, "A loader shape");
-    constexpr int A_LD = A_V4 / kThreads;
-    constexpr int A_TILE_BYTES = BM * LDK * 2;
+    static_assert(TM == 1 && WM * WN == 4, "a wavefront owns 32 filters: its share of a weight tile is one operand per half K tile");
     constexpr int P_BUF_BYTES = 4 * PITCH * 16;
     constexpr int MAXSEG = 3;           // images a tile may touch (H*W >= BN / 2 + 1 is checked by the host)
     constexpr int DW = PXP / 2;         // dwords per load
     constexpr int ZERO_ROW = PITCH - 1; // its aligned group of 8 rows is never loaded
     static_assert(PITCH % 8 == 0 && (PXP == 4 || PXP == 8), "patch shape");
-    constexpr int NA = DLP_PATCH_BF16_NA; // register sets of A tiles
-    static_assert((2 * KHW) % NA == 0, "the A register sets rotate with a period that divides a pair of stages");
+    constexpr int NA = DLP_PATCH_BF16_NA; // register sets of weight operands: tile kt + NA is requested when tile kt has been multiplied
+    static_assert((2 * KHW) % NA == 0, "the register sets rotate with a period that divides a pair of stages");
+    constexpr int OUT_BYTES = (BM * (BN * 2 + 16) > BN * (BM * 2 + 16) ? BM * (BN * 2 + 16) : BN * (BM * 2 + 16)) + BM * 4; // the staged output tile
+    constexpr int SMEM_BYTES = 2 * P_BUF_BYTES > OUT_BYTES ? 2 * P_BUF_BYTES : OUT_BYTES;
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * A_TILE_BYTES + 2 * P_BUF_BYTES];
-    auto As = reinterpret_cast<uint16_t(*)[BM][LDK]>(smem);
-    unsigned char *const ps_bytes = smem + 2 * A_TILE_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+    unsigned char *const ps_bytes = smem;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1886,9 +1886,15 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         *(u32x4 *)(ps_bytes + (tid >> 2) * P_BUF_BYTES + ((tid & 3) * PITCH + ZERO_ROW) * 16) = z;
     }
 
+    // The weights never touch LDS: a wavefront's operand of a half K tile -- filter wm * 32 + l32, sixteen bytes of its row of the
+    // packed tile [BM][32] -- comes from memory (the last-level caches: every workgroup reads the same tiles) straight into
+    // the register the matrix instruction reads.  LDS stores run at a quarter of the rate of LDS loads on this chip (measured:
+    // 67 against 200 bytes per clock and compute unit), and a weight tile written per K tile was as much LDS time as all
+    // the operand reads of that K tile together.
     const uint32_t a_tile_bytes = BM * BK2 * 2;
     const uint32_t a_row_base = (uint32_t)((g * a.mtiles + mt) * a.nkt) * a_tile_bytes;
-    u32x4 ra[NA][A_LD]; // packed A tiles in flight: tile kt + 1 + NA is requested while tile kt is multiplied
+    const uint32_t a_voff = (uint32_t)((wm * 32 + l32) * (BK2 * 2) + h * 16);
+    bf16x8 fa[NA][2]; // weight operands in flight: [register set][half of the K tile]
     uint32_t rbw[8][DW];
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -1903,17 +1909,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         constexpr int S = decltype(set)::value;
         const uint32_t a_soff = a_row_base + (uint32_t)min(kt, a.nkt - 1) * a_tile_bytes;
 #pragma unroll
-        for (int j = 0; j < A_LD; j++)
-            ra[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr, (uint32_t)(tid + j * kThreads) * 16u, a_soff, 0));
-    };
-    auto store_a = [&](auto set, auto buf_c) {
-        constexpr int S = decltype(set)::value;
-        constexpr int BUF = decltype(buf_c)::value;
-#pragma unroll
-        for (int j = 0; j < A_LD; j++) {
-            const int idx = tid + j * kThreads;
-            *(u32x4 *)&As[BUF][idx >> 2][(idx & 3) * 8] = ra[S][j];
-        }
+        for (int s = 0; s < 2; s++)
+            fa[S][s] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(wr, a_voff + (uint32_t)s * 32u, a_soff, 0));
     };
     auto load_patch = [&](int cb) {
         if (!loader)
@@ -1948,59 +1945,46 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         }
     };
 
-    // operands of a K tile (A buffer ABUF, patch buffer PB, tap TAP) into operand set OS
-    bf16x8 fa[2][2][TM], fb[2][2][TN];
-    auto read_operands = [&](auto os_c, auto abuf_c, auto pb_c, auto tap_c) {
-        constexpr int OS = decltype(os_c)::value;
+    // B operands of half a K tile (patch buffer PB, tap TAP, half S)
+    bf16x8 fb[2][TN];
+    auto read_operands = [&](auto pb_c, auto tap_c, auto s_c) {
+        constexpr int S = decltype(s_c)::value;
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                fa[OS][s][i] = *(const bf16x8 *)&As[decltype(abuf_c)::value][wm * WTM + i * 32 + l32][s * 16 + h * 8];
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                fb[OS][s][j] = *(const bf16x8 *)(ps_bytes + decltype(pb_c)::value * P_BUF_BYTES + baddr[j][decltype(tap_c)::value] + s * (2 * PITCH * 16));
-        }
+        for (int j = 0; j < TN; j++)
+            fb[S][j] = *(const bf16x8 *)(ps_bytes + decltype(pb_c)::value * P_BUF_BYTES + baddr[j][decltype(tap_c)::value] + S * (2 * PITCH * 16));
     };
 
-    // One stage: nine K tiles (taps) on patch buffer P.  The patch of the next stage is requested during
-    // the first tap and goes to the other buffer during the last one; the A tiles run through two
-    // register sets and two LDS buffers (tile kt+1 stored, tile kt+3 requested while tile kt is
-    // multiplied).  One barrier per K tile, in its middle: before it, the next tile's A (and patch) go
-    // to the LDS buffers nobody reads any more; after it, the next tile's operands are read while the
-    // second half of this tile's matrix instructions runs, so a wavefront that is alone on its SIMD
-    // does not wait for LDS at the start of a tile.
+    // One stage: nine K tiles (taps) on patch buffer P.  The operands of each half of a K tile are read from LDS while the
+    // matrix instructions of the half before run; the weight operands of tile kt + NA are requested as soon as those of tile kt
+    // have been used.  The patch of the next stage is requested during the first tap and goes to the other buffer during the
+    // last one: the only LDS stores of a stage, and the only barrier (between them and the first reads of the next stage).
     auto stage = [&](auto par, int cb) {
         constexpr int P = decltype(par)::value;
         using OtherP = std::integral_constant<int, P ^ 1>;
         const bool has_next = cb + 1 < ncb;
         static_for_n<KHW>([&](auto tau_c) {
             constexpr int TAU = decltype(tau_c)::value;
-            constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2
-            constexpr int BUF = IDX & 1;       // A buffer and operand set of this tile
-            using NextBuf = std::integral_constant<int, BUF ^ 1>;
-            using Set = std::integral_constant<int, (IDX + 1) % NA>;
+            constexpr int IDX = P * KHW + TAU; // K tile counter modulo 2 * KHW
+            using Set = std::integral_constant<int, IDX % NA>;
             using NextTap = std::integral_constant<int, (TAU + 1) % KHW>;
             using NextPatch = std::integral_constant<int, (TAU + 1 < KHW) ? P : (P ^ 1)>;
             const int kt = cb * KHW + TAU;
-            store_a(Set{}, NextBuf{});
             if (TAU == KHW - 1 && has_next)
                 store_patch(OtherP{});
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[BUF][0][i], fb[BUF][0][j], acc[i][j], 0, 0, 0);
-            __syncthreads();
-            read_operands(NextBuf{}, NextBuf{}, NextPatch{}, NextTap{});
-            load_a(Set{}, kt + 1 + NA);
+            for (int j = 0; j < TN; j++)
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[Set::value][0], fb[0][j], acc[0][j], 0, 0, 0);
+            if (TAU == KHW - 1)
+                __syncthreads();
+            read_operands(NextPatch{}, NextTap{}, std::integral_constant<int, 0>{});
             if (TAU == 0 && has_next)
                 load_patch(cb + 1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[BUF][1][i], fb[BUF][1][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; j++)
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[Set::value][1], fb[1][j], acc[0][j], 0, 0, 0);
+            read_operands(NextPatch{}, NextTap{}, std::integral_constant<int, 1>{});
+            load_a(Set{}, kt + NA);
             __builtin_amdgcn_sched_barrier(0); // keep this order: the scheduler would sink the operand reads to their uses
         });
     };
@@ -2010,10 +1994,9 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     load_patch(0);
     static_for_n<NA>([&](auto set) { load_a(set, decltype(set)::value); });
     store_patch(I0{});
-    store_a(I0{}, I0{});
-    load_a(I0{}, NA);
     __syncthreads();
-    read_operands(I0{}, I0{}, I0{}, I0{});
+    read_operands(I0{}, I0{}, I0{});
+    read_operands(I0{}, I0{}, I1{});
     int cb = 0;
     for (; cb + 1 < ncb; cb += 2) {
         stage(I0{}, cb);
@@ -2023,8 +2006,6 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         stage(I0{}, cb);
     __syncthreads(); // the operand reads issued after the last barrier are done before LDS is reused
 
-    static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
-    static_assert(BN * (BM * 2 + 16) + BM * 4 <= (int)sizeof(smem), "and so does the channels-last one");
     bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
 }
 
@@ -2548,13 +2529,13 @@ int launch_patch_bf16(const ConvGeom &g, const GemmPlan &p, GemmArgs &a, hipStre
     TimingScope ts("conv_gemm", stream);
     const dim3 grid((unsigned)blocks), block(kThreads);
     if (p.tile == 2 && p.patch_bf16 == 8)
-        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 4, 1, kPatchPitchBf16_128, 8, ACT_CLAMP>), grid, block, 0, stream, a);
     else if (p.tile == 2)
-        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 2, 2, kPatchPitchBf16_128, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<128, 128, 4, 1, kPatchPitchBf16_128, 4, ACT_CLAMP>), grid, block, 0, stream, a);
     else if (p.patch_bf16 == 8)
-        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 8, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 2, 2, kPatchPitchBf16_256, 8, ACT_CLAMP>), grid, block, 0, stream, a);
     else
-        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 1, 4, kPatchPitchBf16_256, 4, ACT_CLAMP>), grid, block, 0, stream, a);
+        DLP_LAUNCH_TIMED(ts, (conv_patch_bf16_kernel<64, 256, 2, 2, kPatchPitchBf16_256, 4, ACT_CLAMP>), grid, block, 0, stream, a);
     DLP_HIP_TRY(hipGetLastError());
     return DLP_OK;
 }
