@@ -87,6 +87,13 @@ public:
         if (on)
             throw NotImplementedError("accumulate_before_activation is not implemented by this Conv2DForward");
     }
+    // Not in the reference (its tensors are NCHW throughout): x is read / y is written as [image][row][column][channel]
+    // (dlp_conv2d_fwd_set_channels_last; shapes stay [B, C, H, W]).  The default refuses.
+    virtual void channels_last(bool x, bool y)
+    {
+        if (x || y)
+            throw NotImplementedError("channels_last is not implemented by this Conv2DForward");
+    }
     static std::unique_ptr<Conv2DForward> create(Context &ctx, Conv2DSettings const &config, bool bias,
                                                  StandardActivations activation = StandardActivations::identity,
                                                  std::string const &algo = std::string());
@@ -122,6 +129,7 @@ public:
     }
 
     void accumulate_before_activation(bool on) override { dlprim::details::check_status(dlp_conv2d_fwd_set_accumulate_first(op_, on ? 1 : 0)); }
+    void channels_last(bool x, bool y) override { dlprim::details::check_status(dlp_conv2d_fwd_set_channels_last(op_, x ? 1 : 0, y ? 1 : 0)); }
     size_t packed_size() override { return dlp_conv2d_fwd_packed_bytes(op_); }
     void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) override
     {

@@ -25,6 +25,12 @@ public:
     // X [B,C,H,W] -> Y [B,C,OH,OW]; OH/OW as calc_pooling_output_size gives them (either rounding);
     // the global variants need Y [B,C,1,1]
     virtual void enqueue(Tensor &X, Tensor &Y, ExecutionContext const &e) = 0;
+    // Not in the reference: X is [image][row][column][channel] (global pooling only; shapes stay [B, C, H, W]).  The default refuses.
+    virtual void channels_last(bool on)
+    {
+        if (on)
+            throw NotImplementedError("channels_last is not implemented by this Pooling2DForward");
+    }
 
     static std::unique_ptr<Pooling2DForward> create_max_pooling(Context &ctx, int kernel[2], int pad[2], int stride[2],
                                                                 DataType dt = float_data);
@@ -49,6 +55,7 @@ public:
     void operator=(Pooling2DForwardHip const &) = delete;
 
     size_t workspace() override { return 0; }
+    void channels_last(bool on) override { dlprim::details::check_status(dlp_pool2d_fwd_set_channels_last(op_, on ? 1 : 0)); }
     void enqueue(Tensor &X, Tensor &Y, ExecutionContext const &e) override
     {
         DLPRIM_CHECK(X.shape().size() == 4 && Y.shape().size() == 4);

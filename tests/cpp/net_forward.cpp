@@ -6,9 +6,9 @@
 //   net_forward plan <net.json> [keep] [nofuse]
 //       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
 //       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
-//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [batch=<n>] [resave=<file.dlpw>] [repeat=<n>]
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [nchw] [batch=<n>] [resave=<file.dlpw>] [repeat=<n>]
 //       (batch=<n>: the inputs are reshaped to n images and Net::reshape() is called before the pass)
-//       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32)
+//       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32; nchw: no channels-last tensors between bf16 convolutions)
 //       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
 //       network's input order), runs forward and writes the outputs (float32, in output order)
 //   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse] [graph]
@@ -48,7 +48,7 @@ int main(int argc, char **argv)
             std::cout << v.save() << std::endl;
             return 0;
         }
-        bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false;
+        bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false, nchw = false;
         std::string resave;
         int repeat = 1, warmup = 5, iters = 20, batch = 0;
         const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
@@ -64,6 +64,8 @@ int main(int argc, char **argv)
                 prepack = false;
             else if (a == "bf16")
                 bf16 = true;
+            else if (a == "nchw")
+                nchw = true;
             else if (a.compare(0, 7, "resave=") == 0)
                 resave = a.substr(7);
             else if (a.compare(0, 7, "repeat=") == 0)
@@ -83,6 +85,7 @@ int main(int argc, char **argv)
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
             net.prepack(prepack);
+            net.channels_last(!nchw);
             net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
@@ -102,6 +105,7 @@ int main(int argc, char **argv)
             net.keep_intermediate_tensors(keep);
             net.fuse(fuse);
             net.prepack(prepack);
+            net.channels_last(!nchw);
             net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
@@ -148,6 +152,7 @@ int main(int argc, char **argv)
         net.keep_intermediate_tensors(keep);
         net.fuse(fuse);
         net.prepack(prepack);
+            net.channels_last(!nchw);
         net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
         net.mode(dp::CalculationsMode::predict);
         net.load_from_json_file(argv[2]);
