@@ -3028,11 +3028,17 @@ int conv_gemm_pack_weights(const ConvGeom &g, const GemmPlan &p, const void *w, 
 
 // Channels-last x and / or y: served by the bf16 matrix-instruction kernels only (x: the channels-last loader, i.e. input
 // channels per group in multiples of 32 and a kernel extent the tap masks hold; y: output channels per group in eights).
+static bool layouts_supported(const ConvGeom &g, const GemmPlan &p);
 bool conv_gemm_layouts_supported(const ConvGeom &g, int activation)
 {
     if (!g.x_channels_last && !g.y_channels_last)
         return true;
-    const GemmPlan p = conv_gemm_plan(g, activation);
+    return layouts_supported(g, conv_gemm_plan(g, activation));
+}
+static bool layouts_supported(const ConvGeom &g, const GemmPlan &p)
+{
+    if (!g.x_channels_last && !g.y_channels_last)
+        return true;
     if (!bf16_mfma_order(p.order) || p.stem || p.pointwise || p.patch)
         return false;
     if (g.x_channels_last && !p.xt)
@@ -3065,7 +3071,7 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
         return fail(DLP_ERR_NOT_IMPLEMENTED, "tensors of 2 GiB or more are not supported by the 32-bit buffer addressing");
     if (g.B == 0)
         return DLP_OK;
-    if (!conv_gemm_layouts_supported(g, ep.activation))
+    if (!layouts_supported(g, p))
         return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: served by the bf16 matrix-instruction kernels only (input channels per group in "
                                              "multiples of 32 for x, output channels per group in eights for y)");
     if (p.stem) {

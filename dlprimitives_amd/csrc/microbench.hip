@@ -2,6 +2,7 @@
 // an MFMA-only loop (no memory traffic) and a streaming copy.  Not part of the
 // operator ABI; built as a separate library, libdlp_microbench.so.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <cstdio>
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -152,6 +153,167 @@ static float time_ms(hipStream_t s, hipEvent_t e0, hipEvent_t e1)
     return ms;
 }
 
+
+// ---- one K step of a 128 x 128 x 32 bf16 tile in a four-wavefront workgroup, piece by piece --------------------------------
+// What LDS and the matrix pipe sustain together: 8 v_mfma_f32_32x32x16_bf16 per wavefront (2 x 2 blocks of 32 x 32, two halves of
+// the K tile), their operands as 8 ds_read_b128 per lane (32 KB per workgroup), the next tile as 4 ds_write_b128 per lane (16 KB),
+// one barrier.  Tiles lie in LDS as rows of 64 bytes whose 16-byte pieces are XOR-swizzled with the row number: reads (one row
+// per lane) and stores (four lanes per row) are free of bank conflicts.
+// PARTS: 1 LDS reads, 2 LDS stores, 4 barrier, 8 matrix instructions, 16 the tiles come from memory (an L2-resident buffer,
+// requested three steps ahead), 32 with 16: the weight tile goes from memory straight into the operand registers (4 x 1 wavefronts
+// of 32 x 128) and only the pixel tile passes through LDS.
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+template <int PARTS>
+__global__ __launch_bounds__(256) void tile_step_kernel(int iters, float *out, const unsigned char *src, unsigned src_mask)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char step_lds[];
+    constexpr int TILE = 128 * 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    for (int i = tid; i < 4 * TILE / 4; i += 256)
+        ((unsigned *)step_lds)[i] = 0x3f803f80u;
+    __syncthreads();
+    auto at = [&](int tile, int buf, int row, int piece) { return step_lds + (buf * 2 + tile) * TILE + row * 64 + ((piece ^ ((row >> 2) & 3)) * 16); };
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)src, 0, src_mask + 1, 0x00020000);
+    const unsigned pos = (blockIdx.x * 2654435761u) & src_mask & ~16383u; // this workgroup's stream of 16 KB tile pairs
+    probe_f32x16 acc[4];
+    for (int j = 0; j < 4; j++)
+        for (int q = 0; q < 16; q++)
+            acc[j][q] = 0.f;
+    u32x4 regs[3][4];
+    const u32x4 fill = {1u, 2u, 3u, 4u};
+    for (int q = 0; q < 3; q++)
+        for (int j = 0; j < 4; j++)
+            regs[q][j] = fill;
+    probe_bf16x8 fa[2][2], fb[2][2], fw[3][2], fp[2][4];
+    auto request = [&](auto set, int t) {
+        constexpr int S = decltype(set)::value;
+        const unsigned soff = (pos + (unsigned)t * 16384u) & src_mask;
+        if (PARTS & 32) { // weight operands of this wavefront's 32 rows + its two pieces of the pixel tile
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++)
+                fw[S][s2] = __builtin_bit_cast(probe_bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, (unsigned)((wave * 32 + l32) * 64 + h * 16), soff + s2 * 32, 0));
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                regs[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (unsigned)(tid * 16 + j * 4096), soff + 8192, 0));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                regs[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (unsigned)(tid * 16 + j * 4096), soff, 0));
+        }
+    };
+    auto step = [&](auto set, int it) {
+        constexpr int S = decltype(set)::value;
+        const int buf = it & 1;
+        if (PARTS & 1) {
+            if (PARTS & 32) {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        fp[s2][j] = *(const probe_bf16x8 *)at(1, buf, j * 32 + l32, s2 * 2 + h);
+            } else {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        fa[s2][i] = *(const probe_bf16x8 *)at(0, buf, wm * 64 + i * 32 + l32, s2 * 2 + h);
+                        fb[s2][i] = *(const probe_bf16x8 *)at(1, buf, wn * 64 + i * 32 + l32, s2 * 2 + h);
+                    }
+            }
+        }
+        if (PARTS & 8) {
+            if (PARTS & 32) {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[S][s2], fp[s2][j], acc[j], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int j = 0; j < 2; j++)
+                            acc[i * 2 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s2][i], fb[s2][j], acc[i * 2 + j], 0, 0, 0);
+            }
+        } else {
+            asm volatile("" ::"v"(fa[0][0]), "v"(fa[0][1]), "v"(fa[1][0]), "v"(fa[1][1]), "v"(fb[0][0]), "v"(fb[0][1]), "v"(fb[1][0]), "v"(fb[1][1]));
+        }
+        if (PARTS & 2) { // the tile of the next step, from the registers that were requested three steps ago
+            constexpr int N = (PARTS & 32) ? 2 : 4;
+#pragma unroll
+            for (int j = 0; j < N; j++) {
+                const int idx = tid + j * 256, tile = (PARTS & 32) ? 1 : idx >> 9, row = (idx >> 2) & 127;
+                *(u32x4 *)at(tile, buf ^ 1, row, idx & 3) = regs[(S + 1) % 3][j];
+            }
+        }
+        if (PARTS & 16)
+            request(std::integral_constant<int, (S + 1) % 3>{}, it + 4);
+        if (PARTS & 4)
+            __syncthreads();
+        else
+            asm volatile("" ::: "memory");
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    if (PARTS & 16) {
+        request(I0{}, 0);
+        request(I1{}, 1);
+        request(I2{}, 2);
+    }
+    for (int it = 0; it < iters; it += 3) {
+        step(I0{}, it);
+        step(I1{}, it + 1);
+        step(I2{}, it + 2);
+    }
+    float sum = 0.f;
+    for (int j = 0; j < 4; j++)
+        for (int q = 0; q < 16; q++)
+            sum += acc[j][q];
+    if (sum == 123.456f)
+        out[tid] = sum;
+}
+
+template <int PARTS>
+static int run_tile_step(int wgs_per_cu, double *ns_per_step)
+{
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess)
+        return 1;
+    const int cus = prop.multiProcessorCount, iters = 6000;
+    // LDS per workgroup fixes how many share a compute unit
+    const int lds = wgs_per_cu <= 1 ? 150 * 1024 : wgs_per_cu == 2 ? 75 * 1024 : 50 * 1024;
+    float *out = nullptr;
+    unsigned char *src = nullptr;
+    const unsigned src_bytes = 2u << 20;
+    if (hipMalloc(&out, 4096) != hipSuccess || hipMalloc(&src, src_bytes) != hipSuccess)
+        return 1;
+    (void)hipMemset(src, 0x3f, src_bytes);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    int rc = hipFuncSetAttribute((const void *)tile_step_kernel<PARTS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess;
+    if (!rc) {
+        tile_step_kernel<PARTS><<<cus * wgs_per_cu, 256, lds>>>(300, out, src, src_bytes - 1);
+        (void)hipEventRecord(e0);
+        tile_step_kernel<PARTS><<<cus * wgs_per_cu, 256, lds>>>(iters, out, src, src_bytes - 1);
+        (void)hipEventRecord(e1);
+        rc = hipDeviceSynchronize() != hipSuccess;
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        *ns_per_step = ms * 1e6 / iters;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    (void)hipFree(src);
+    return rc;
+}
+
 extern "C" {
 
 // fp32 MFMA throughput in TFLOP/s with `waves_per_simd` wavefronts resident per SIMD.
@@ -272,4 +434,31 @@ int dlp_probe_stream_forms(size_t in_bytes, size_t out_bytes, double *us, int *b
 
 const char *dlp_probe_stream_form_name(int form) { return form >= 0 && form < N_FORMS ? kFormNames[form] : ""; }
 int dlp_probe_stream_form_count(void) { return N_FORMS; }
+
+// Time per K step of a 128 x 128 x 32 bf16 tile (2 * 128 * 128 * 32 flop) in a four-wavefront workgroup, `wgs_per_cu` (1..3) of them
+// per compute unit, for one of the forms of tile_step_kernel (see dlp_probe_tile_step_name).  Returns 0 on success.
+static const char *kStepNames[] = {"matrix instructions only",
+                                   "matrix instructions + operand reads from LDS",
+                                   "... + barrier",
+                                   "... + next tile stored to LDS",
+                                   "LDS stores + barrier alone (16 KB per step)",
+                                   "LDS reads + barrier alone (32 KB per step)",
+                                   "whole step, both tiles from memory (L2) through registers and LDS",
+                                   "whole step, weights from memory straight into registers, pixels through LDS"};
+int dlp_probe_tile_step(int form, int wgs_per_cu, double *ns_per_step)
+{
+    switch (form) {
+    case 0: return run_tile_step<8>(wgs_per_cu, ns_per_step);
+    case 1: return run_tile_step<9>(wgs_per_cu, ns_per_step);
+    case 2: return run_tile_step<13>(wgs_per_cu, ns_per_step);
+    case 3: return run_tile_step<15>(wgs_per_cu, ns_per_step);
+    case 4: return run_tile_step<6>(wgs_per_cu, ns_per_step);
+    case 5: return run_tile_step<5>(wgs_per_cu, ns_per_step);
+    case 6: return run_tile_step<31>(wgs_per_cu, ns_per_step);
+    case 7: return run_tile_step<63>(wgs_per_cu, ns_per_step);
+    default: return 1;
+    }
+}
+const char *dlp_probe_tile_step_name(int form) { return form >= 0 && form < 8 ? kStepNames[form] : ""; }
+int dlp_probe_tile_step_count(void) { return 8; }
 }

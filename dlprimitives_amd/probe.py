@@ -7,6 +7,7 @@ non-temporal accesses, 1024-thread workgroups, the untuned grid-stride loop, hip
 launch cold (a ring of buffers larger than the last-level cache), and reports the fastest kernel form: the "tuned copy".
 
     python -m dlprimitives_amd.probe [--copy-mb 256] [--no-mfma]
+    python -m dlprimitives_amd.probe --tile-step
 """
 import argparse
 import ctypes
@@ -42,6 +43,31 @@ def copy_at_size(in_bytes, out_bytes):
     return (in_bytes + out_bytes) / us / 1e3, us
 
 
+def tile_steps():
+    """What LDS and the matrix pipe sustain together on one K step of a 128 x 128 x 32 bf16 tile in a four-wavefront workgroup, piece by
+    piece (tile_step_kernel of csrc/microbench.hip): {form: {workgroups per CU: {"ns_per_step", "clocks_at_2.4GHz", "tflops"}}}, and the LDS
+    rates that follow from the reads-only and stores-only forms."""
+    lib = _lib()
+    lib.dlp_probe_tile_step_name.restype = ctypes.c_char_p
+    v = ctypes.c_double()
+    out = {}
+    for f in range(lib.dlp_probe_tile_step_count()):
+        name = lib.dlp_probe_tile_step_name(f).decode()
+        out[name] = {}
+        for w in (1, 2, 3):
+            if lib.dlp_probe_tile_step(f, w, ctypes.byref(v)) != 0:
+                raise RuntimeError("tile step probe failed")
+            ns = v.value
+            row = {"ns_per_step": round(ns, 1), "clocks_at_2.4GHz": round(ns * 2.4)}
+            if "alone" not in name:
+                row["tflops"] = round(2.0 * 128 * 128 * 32 * 256 * w / (ns * 1e-9) / 1e12)
+            out[name]["%d per CU" % w] = row
+    rd = out["LDS reads + barrier alone (32 KB per step)"]["3 per CU"]["clocks_at_2.4GHz"] / 3.0
+    wr = out["LDS stores + barrier alone (16 KB per step)"]["3 per CU"]["clocks_at_2.4GHz"] / 3.0
+    out["lds_bytes_per_clock_and_cu"] = {"ds_read_b128": round(32768 / rd), "ds_write_b128": round(16384 / wr)}
+    return out
+
+
 def measured_peaks(big_mb=2048):
     """MFMA-only loops and streaming kernels on this device: what the chip reaches with no convolution around it."""
     lib = _lib()
@@ -70,7 +96,11 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--copy-mb", type=int, default=256, help="MiB per direction of the copy kernels")
     ap.add_argument("--no-mfma", action="store_true")
+    ap.add_argument("--tile-step", action="store_true", help="only the K-step probe of a bf16 tile (LDS reads, LDS stores, matrix instructions together)")
     args = ap.parse_args()
+    if args.tile_step:
+        print(json.dumps(tile_steps(), indent=1))
+        return
     lib = _lib()
     out = {}
     v = ctypes.c_double()
