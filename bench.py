@@ -174,10 +174,10 @@ def cpu_baseline(layer_list, images, seed, threads=1, runs=3):
 
 def run_graph_workload(args):
     return graph_workload(args.workload[:-len("-full")], args.batch, args.algo, args.dtype == "bf16", args.steps, args.warmup, args.fuse_residual, args.prepacked,
-                          args.channels_last)
+                          args.channels_last, args.fuse_stem_pool)
 
 
-def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, prepack=False, channels_last=False):
+def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, prepack=False, channels_last=False, fuse_stem_pool=False):
     """Whole-network forward (convolutions + pooling + residual adds + global pooling + inner
     product) through the C-ABI operators; same JSON contract, no per-kernel roofline split."""
     import torch
@@ -189,7 +189,8 @@ def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, p
     params = graphs.random_parameters(ops, 2024)
     shape = (batch, 3, 224, 224)
     runner = graphs.GraphRunner(ops, params, shape, algo=algo, dtype="bfloat16" if bf16 else "float32", fuse_residual=fuse_residual, prepack=prepack,
-                                channels_last=channels_last)
+                                channels_last=channels_last, fuse_stem_pool=fuse_stem_pool)
+    pooled_inside = sum(1 for o in runner.ops if o.get("pool"))
     x = torch.rand(shape, device="cuda:0") * 2 - 1
     runner.t["data"].copy_(x)  # converts to the storage type
     for _ in range(warmup):
@@ -223,7 +224,8 @@ def graph_workload(net, batch, algo, bf16, steps, warmup, fuse_residual=False, p
                                "%s NCHW, batch %d, 224x224, conv algo '%s'%s" % (net, " in the epilogue of the 1x1 convolution in front of them" if fuse_residual else "",
                                                                                "bf16 storage" if bf16 else "fp32", batch, algo or "auto",
                                                                                ", filters transformed once before the timed region" if prepack else "") +
-                               ("; %d of the tensors between operators kept channels-last (input, logits and parameters as given)" % len(runner.cl) if runner.cl else ""),
+                               ("; %d of the tensors between operators kept channels-last (input, logits and parameters as given)" % len(runner.cl) if runner.cl else "") +
+                               ("; the stem's max pooling runs inside the stem's convolution kernel (its time counts as convolution time)" if pooled_inside else ""),
                    "batch": batch, "gflop_per_step": round(flops / 1e9, 1)},
         "gflops_per_s": round(flops / (ms_per_step * 1e-3) / 1e9, 1),
         "frac_of_matrix_peak_whole_pass": round(flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
@@ -684,7 +686,7 @@ def other_configs(steps, warmup, peaks, with_cpu=True):
     nchw = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True, prepack=True)
     torch.cuda.empty_cache()
     cfgs["config5_resnet50_full_bf16_b128"] = graph_workload("resnet50", 128, "gemm", True, max(3, steps // 2), max(2, warmup // 2), fuse_residual=True, prepack=True,
-                                                             channels_last=True)
+                                                             channels_last=True, fuse_stem_pool=True)
     cfgs["config5_resnet50_full_bf16_b128"]["nchw_between_layers"] = {"ms_per_step": nchw["ms_per_step"], "images_per_s": nchw["value"],
                                                                        "roofline_frac": nchw["roofline"]["frac"]}
     if with_cpu:
@@ -714,6 +716,8 @@ def main():
     ap.add_argument("--layers", action="store_true", help="also print the per-layer table to stderr")
     ap.add_argument("--channels-last", action="store_true",
                     help="*-full workloads in bf16: tensors between convolutions are kept channels-last where the planner finds it faster")
+    ap.add_argument("--fuse-stem-pool", action="store_true",
+                    help="*-full workloads in bf16: the 3x3 stride-2 max pooling behind the 7x7 stem runs inside the stem's kernel (dlp_conv2d_fwd_fuse_max_pool)")
     ap.add_argument("--prepacked", action="store_true",
                     help="weights transformed once before the timed region (dlp_conv2d_fwd_pack / _enqueue_packed), as an inference "
                          "deployment does; the default transforms them in every step, as the reference's enqueue contract implies")

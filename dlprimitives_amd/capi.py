@@ -248,6 +248,12 @@ class Conv2DForward:
         _check(lib().dlp_conv2d_fwd_set_channels_last(self._h, int(bool(x)), int(bool(y))))
         self._x_channels_last = bool(x)
 
+    def fuse_max_pool(self, kernel=3, stride=2, pad=1, ceil_mode=False):
+        """dlp_conv2d_fwd_fuse_max_pool: enqueue writes max_pool(act(conv + bias)), a tensor of the pooled shape, and never the
+        convolution's own output (the bfloat16 stem of a ResNet and its 3x3 stride-2 pad-1 pooling; NotImplementedError otherwise)"""
+        lib().dlp_conv2d_fwd_fuse_max_pool.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        _check(lib().dlp_conv2d_fwd_fuse_max_pool(self._h, int(kernel), int(stride), int(pad), int(bool(ceil_mode))))
+
     def _x_shape(self, x):
         """the [B, C, H, W] that the C interface takes, whatever the layout of x"""
         if getattr(self, "_x_channels_last", False):

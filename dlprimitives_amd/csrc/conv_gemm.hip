@@ -3077,8 +3077,10 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
     if (p.stem) {
         if (w == nullptr || n_valid >= 0)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "stem convolution: needs the weight tensor and the whole batch");
-        return conv_stem_launch(g, x, w, y, ep, stream);
+        return conv_stem_launch(g, x, w, y, ep, stream, g.pool_ph, g.pool_pw);
     }
+    if (g.pool_ph > 0)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "max pooling inside the convolution: the bf16 stem kernel only");
     // few output channels, 1x1: X streams from memory straight into the matrix instructions (needs the filter as it lies in memory)
     if (p.pointwise && w != nullptr && n_valid < 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) == 0 && ep.activation != DLP_ACT_TANH &&
         ep.activation != DLP_ACT_SIGMOID)

@@ -53,6 +53,7 @@ struct StemArgs {
     float factor;
     int pre, act;
     float clamp_lo, clamp_hi;
+    int PH, PW, upi; // max pooling inside the bf16 kernel: pooled size, units (pairs of pooled rows) per image
 };
 
 template <class F, int... I>
@@ -354,16 +355,24 @@ typedef uint32_t stem_u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kStemPadL16 = 8;     // zero columns left of an input row (keeps the 16-byte LDS stores aligned)
 constexpr int kStemStagePitch = 80; // bytes per filter of a wavefront's staged 32 x 32 output block (64 + 16: 16-byte rows)
 
-template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, int NT>
+template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, int NT, bool POOL = false>
 constexpr int stem_bf16_lds_bytes()
 {
     constexpr int ROWS = STRIDE * (R - 1) + KH, QP = (CIN * KH + 1) / 2 * 2;
-    return CIN * ROWS * PITCH * 2 + 64 * (QP * 8 + 8) * 2 + 64 * 4 + (NT / 64) * 32 * kStemStagePitch;
+    return CIN * ROWS * PITCH * 2 + 64 * (QP * 8 + 8) * 2 + 64 * 4 + (POOL ? 64 * R * (PITCH / 2) * 2 : (NT / 64) * 32 * kStemStagePitch);
 }
 
-template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, bool VEC, int NT>
+// POOL: the 3x3 stride-2 pad-1 max pooling that follows the stem of every ResNet runs inside the kernel.  The workgroup walks units
+// of two pooled rows instead of bands: pooled rows 2u and 2u + 1 look at convolution rows 4u - 1 .. 4u + 3.  Results go to LDS as bf16
+// [filter][row % 5][column] -- eight columns of -inf to the left stand for column -1 -- so row 4u - 1 is still there from the unit
+// before and a unit computes four rows; only the first unit of a workgroup's range, when it is not the top of an image, computes
+// all five (R = 5).  The pooled rows leave as 16-byte stores: a quarter of the convolution's bytes, and the pooling operator's pass
+// over them (as long again as the convolution) is gone.  Values equal those of the two operators run one after the other bit for bit.
+template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, bool VEC, int NT, bool POOL = false>
 __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
 {
+    static_assert(!POOL || (VEC && R == 5), "the pooled form: five rows at most and 16-byte input loads");
+    constexpr int OBP = PITCH / 2; // POOL: elements per row of the results in LDS
     static_assert(KW <= 7, "a filter row and its leading zero are the eight k of a lane");
     constexpr int K = CIN * KH * KW;
     constexpr int Q = CIN * KH, QP = (Q + 1) / 2 * 2, NJ = QP / 2; // filter rows, two per matrix instruction
@@ -385,7 +394,8 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
     float *Bs = (float *)(Ws + 64 * WPITCH); // [64] bias
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    unsigned char *Ys = (unsigned char *)(Bs + 64) + wave * (32 * YP); // this wavefront's staged block
+    unsigned char *Ys = (unsigned char *)(Bs + 64) + (POOL ? 0 : wave * (32 * YP)); // this wavefront's staged block
+    uint16_t *Ob = (uint16_t *)(Bs + 64);                                            // POOL: [64][5][OBP] results, row r in slot r % 5
     typedef typename std::conditional<VEC, stem_u32x4, uint16_t>::type unit_t;
 
     const int first = (int)blockIdx.x * a.rows_per_wg, last = min(first + a.rows_per_wg, a.total_rows);
@@ -402,6 +412,9 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
     }
     for (int i = tid; i < 64 * WPITCH / 2; i += NT)
         ((uint32_t *)Ws)[i] = 0u;
+    if constexpr (POOL)
+        for (int i = tid; i < 64 * R * 8; i += NT) // left of column 0: never the maximum
+            Ob[(i >> 3) * OBP + (i & 7)] = 0xFF80u;
 
     uint32_t lane_off[NCH];
 #pragma unroll
@@ -446,12 +459,23 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
             }
         }
     };
+    int unit_u = 0; // POOL: the pair of pooled rows in hand
     auto decode = [&](int row, int &mt, int &n, int &oy, int &rb) {
-        mt = row / boh;
-        const int rem = row - mt * boh;
-        n = rem / a.OH;
-        oy = rem - n * a.OH;
-        rb = min(min(R, a.OH - oy), last - row);
+        if constexpr (POOL) { // `row` numbers units: (m tile, image, pair of pooled rows)
+            const int per_tile = a.B * a.upi;
+            mt = row / per_tile;
+            const int rem = row - mt * per_tile;
+            n = rem / a.upi;
+            const int u = rem - n * a.upi;
+            oy = (u > 0 && row == first) ? 4 * u - 1 : 4 * u; // row 4u - 1 is in LDS unless the range starts here
+            rb = max(min(4 * u + 4, a.OH) - oy, 0);
+        } else {
+            mt = row / boh;
+            const int rem = row - mt * boh;
+            n = rem / a.OH;
+            oy = rem - n * a.OH;
+            rb = min(min(R, a.OH - oy), last - row);
+        }
     };
 
     int cur = first, mt, n, oy, rb, loaded_mt = -1;
@@ -491,7 +515,9 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
         }
         __syncthreads();
         loaded_mt = mt;
-        const int next = cur + rb;
+        const int next = POOL ? cur + 1 : cur + rb;
+        if constexpr (POOL)
+            unit_u = (cur - mt * a.B * a.upi) % a.upi;
         int nmt = mt, nn = n, noy = oy, nrb = 0;
         if (next < last) {
             decode(next, nmt, nn, noy, nrb);
@@ -534,7 +560,27 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
             });
 
             // accumulator register r of filter block cb: filter m0 + 32 * cb + l32, pixel blk * 32 + 8 * (r / 4) + 4 * h + r % 4
-            if (wide) {
+            if constexpr (POOL) {
+                // a register quad is four consecutive pixels of one row (rows are multiples of eight pixels): one 8-byte LDS store
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int p4 = blk * 32 + 8 * rq + 4 * h;
+                    const uint32_t p4c = p4 < npix ? (uint32_t)p4 : 0u;
+                    const int r4 = (int)fast_div(p4c, a.ow_magic, a.ow_shift), c4 = (int)p4c - r4 * a.OW;
+                    const int slot = (oy + r4) % 5;
+#pragma unroll
+                    for (int cb = 0; cb < 2; cb++) {
+                        stem_u32x2 o;
+#pragma unroll
+                        for (int e = 0; e < 2; e++) {
+                            const float lo = activate(acc[cb][4 * rq + 2 * e]), hi = activate(acc[cb][4 * rq + 2 * e + 1]);
+                            o[e] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                        }
+                        if (p4 < npix)
+                            *(stem_u32x2 *)(Ob + ((cb * 32 + l32) * 5 + slot) * OBP + 8 + c4) = o;
+                    }
+                }
+            } else if (wide) {
 #pragma unroll
                 for (int cb = 0; cb < 2; cb++) {
                     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); // the block's previous reads are done
@@ -581,6 +627,48 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
                 }
             }
         }
+        if constexpr (POOL) {
+            // ---- the unit's pooled rows: a thread takes eight pooled columns of a (filter, row): 17 columns of up to three rows ----
+            __syncthreads();
+            constexpr float kLowest = -3.402823466e+38f;
+            const int pw8 = a.PW >> 3, prs = min(2, a.PH - 2 * unit_u), per_m = prs * pw8;
+            const __amdgpu_buffer_rsrc_t pyr =
+                __builtin_amdgcn_make_buffer_rsrc((void *)((uint16_t *)a.y + (size_t)n * a.Cout * a.PH * a.PW), 0, a.y_img_bytes, 0x00020000);
+            for (int t = tid; t < 64 * per_m; t += NT) {
+                const int m = t / per_m, r2 = t - m * per_m, pr = r2 / pw8, k = r2 - pr * pw8;
+                const int prow = 2 * unit_u + pr;
+                float rowmax[3][8];
+#pragma unroll
+                for (int dr = 0; dr < 3; dr++) {
+                    const int row = 2 * prow - 1 + dr;
+                    const bool ok = row >= 0 && row < a.OH;
+                    const uint16_t *src = Ob + (m * 5 + (ok ? row % 5 : 0)) * OBP + 8 + 16 * k;
+                    float e[17];
+                    e[0] = __builtin_bit_cast(float, (uint32_t)src[-1] << 16);
+                    const stem_u32x4 v0 = *(const stem_u32x4 *)src, v1 = *(const stem_u32x4 *)(src + 8);
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        e[1 + 2 * q] = __builtin_bit_cast(float, v0[q] << 16);
+                        e[2 + 2 * q] = __builtin_bit_cast(float, v0[q] & 0xffff0000u);
+                        e[9 + 2 * q] = __builtin_bit_cast(float, v1[q] << 16);
+                        e[10 + 2 * q] = __builtin_bit_cast(float, v1[q] & 0xffff0000u);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; j++)
+                        rowmax[dr][j] = ok ? fmaxf(fmaxf(e[2 * j], e[2 * j + 1]), e[2 * j + 2]) : kLowest;
+                }
+                float best[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    best[j] = fmaxf(fmaxf(rowmax[0][j], rowmax[1][j]), rowmax[2][j]);
+                stem_u32x4 o;
+#pragma unroll
+                for (int q = 0; q < 4; q++) // maxima of stored values are bf16 already: the upper halves are the results
+                    o[q] = (__builtin_bit_cast(uint32_t, best[2 * q]) >> 16) | (__builtin_bit_cast(uint32_t, best[2 * q + 1]) & 0xffff0000u);
+                const uint32_t voff = (m0 + m < a.Cout) ? (uint32_t)((((m0 + m) * a.PH + prow) * a.PW + 8 * k) * 2) : kStemOutOfRange;
+                __builtin_amdgcn_raw_buffer_store_b128(o, pyr, voff, 0, 0);
+            }
+        }
         if (next >= last)
             break;
         cur = next;
@@ -591,7 +679,7 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
     }
 }
 
-constexpr int kStemR = 8, kStemPitch = 240;
+constexpr int kStemR = 8, kStemPitch = 240, kStemPoolR = 5;
 
 bool generic_activation(int act) { return act == DLP_ACT_TANH || act == DLP_ACT_SIGMOID; }
 
@@ -619,10 +707,21 @@ bool conv_stem_supported(const ConvGeom &g)
     return 2 * (g.OW - 1) - g.pw + 6 + kStemPadL + 1 < kStemPitch && g.W + 2 * kStemPadL <= kStemPitch;
 }
 
-int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream)
+bool conv_stem_pool_supported(const ConvGeom &g, int PH, int PW)
+{
+    // whole runs of eight pixels in convolution and pooled rows; the last pooling window ends inside the row (the columns
+    // right of it are not initialised in LDS) and starts inside the image
+    return g.dtype == DLP_BFLOAT16 && conv_stem_supported(g) && g.W % 8 == 0 && g.OW % 8 == 0 && PW % 8 == 0 && PW >= 8 && 2 * PW == g.OW &&
+           PH >= 1 && 2 * (PH - 1) - 1 < g.OH && 8 + g.OW <= kStemPitch / 2 && (long long)g.Cout * PH * PW * 2 < 0x7fffffffLL;
+}
+
+int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream, int PH, int PW)
 {
     if (!conv_stem_supported(g))
         return fail(DLP_ERR_NOT_IMPLEMENTED, "conv_stem: unsupported geometry");
+    const bool pool = PH > 0;
+    if (pool && (!conv_stem_pool_supported(g, PH, PW) || ep.factor != 0.0f || ((uintptr_t)x & 15) != 0 || ((uintptr_t)y & 15) != 0))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "conv_stem: the max pooling cannot run inside the kernel for this geometry, alignment or scale of the old y");
     if (g.B == 0)
         return DLP_OK;
     StemArgs a;
@@ -635,7 +734,8 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.B = g.B; a.H = g.H; a.W = g.W; a.Cout = g.Cout; a.OH = g.OH; a.OW = g.OW; a.OHW = g.OH * g.OW;
     a.ph = g.ph; a.pw = g.pw;
     const int mtiles = (g.Cout + 63) / 64;
-    const long long total = (long long)mtiles * g.B * g.OH;
+    a.PH = PH; a.PW = PW; a.upi = (PH + 1) / 2;
+    const long long total = (long long)mtiles * g.B * (pool ? a.upi : g.OH); // rows, or pairs of pooled rows
     if (total > 0x7fffffffLL - 65536)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "convolution too large for a single launch");
     // one workgroup per CU walks a contiguous range of output rows in bands of up to R rows
@@ -643,7 +743,7 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     a.total_rows = (int)total;
     a.rows_per_wg = (int)((total + wgs - 1) / wgs);
     a.x_img_bytes = (uint32_t)((size_t)g.Cin * g.H * g.W * esize);
-    a.y_img_bytes = (uint32_t)((size_t)g.Cout * g.OH * g.OW * esize);
+    a.y_img_bytes = pool ? (uint32_t)((size_t)g.Cout * PH * PW * esize) : (uint32_t)((size_t)g.Cout * g.OH * g.OW * esize);
     a.w_bytes = (uint32_t)((size_t)g.Cout * 147 * esize);
     // 16-byte loads: every input row and (fp32) the filter rows of every m tile then start 16-byte aligned
     const bool vec = bf16 ? g.W % 8 == 0 && ((uintptr_t)x & 15) == 0 : g.W % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
@@ -662,6 +762,21 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         a.clamp_hi = 6.0f;
     const dim3 grid((unsigned)((a.total_rows + a.rows_per_wg - 1) / a.rows_per_wg)), block(kStemThreads);
     TimingScope ts("conv_gemm", stream);
+    if (pool) {
+        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemPoolR, kStemPitch, kStemThreads, true>();
+        auto kernel = conv_stem_bf16_kernel<3, 7, 7, 2, kStemPoolR, kStemPitch, true, kStemThreads, true>;
+        static bool asked[64] = {}; // per device
+        int dev = 0;
+        DLP_HIP_TRY(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 64 || !asked[dev]) {
+            DLP_HIP_TRY(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            if (dev >= 0 && dev < 64)
+                asked[dev] = true;
+        }
+        DLP_LAUNCH_TIMED(ts, kernel, grid, block, lds, stream, a);
+        DLP_HIP_TRY(hipGetLastError());
+        return DLP_OK;
+    }
     if (bf16) {
         constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemR, kStemPitch, kStemThreads>();
         auto kernel = vec ? conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, kStemThreads> : conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, kStemThreads>;

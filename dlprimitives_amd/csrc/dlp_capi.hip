@@ -114,6 +114,7 @@ struct dlp_conv2d_fwd {
     int packed_layout[6]; // of the last dlp_conv2d_fwd_pack: order, BM, K tiles, m tiles, patch, in-place
     int accumulate_first; // y = act(conv + bias + factor * y) instead of factor * y + act(conv + bias)
     int x_channels_last, y_channels_last; // tensor layouts of the gemm algorithm on bf16 tensors (dlp_conv2d_fwd_set_channels_last)
+    int max_pool;                         // a 3x3 stride-2 pad-1 max pooling runs behind the convolution (dlp_conv2d_fwd_fuse_max_pool)
     int *counters;        // GEMM stage: tile counters of split-K / stream-K launches, zero between launches
     size_t counter_count;
 };
@@ -145,6 +146,10 @@ static int op_geom(const dlp_conv2d_fwd *op, const int x_shape[4], ConvGeom &g)
     const int rc = make_geom(op->cfg, x_shape, g);
     g.x_channels_last = op->x_channels_last;
     g.y_channels_last = op->y_channels_last;
+    if (op->max_pool) { // sizes as Pooling2D with ceil_mode false computes them
+        g.pool_ph = (g.OH + 2 - 3) / 2 + 1;
+        g.pool_pw = (g.OW + 2 - 3) / 2 + 1;
+    }
     return rc;
 }
 
@@ -553,6 +558,7 @@ int dlp_conv2d_fwd_create(const dlp_conv2d_settings *cfg, int bias, int activati
     op->accumulate_first = 0;
     op->x_channels_last = 0;
     op->y_channels_last = 0;
+    op->max_pool = 0;
     op->counters = nullptr;
     op->counter_count = 0;
     if (hipGetDevice(&op->device) != hipSuccess)
@@ -665,6 +671,8 @@ int dlp_conv2d_fwd_set_channels_last(dlp_conv2d_fwd *op, int x_channels_last, in
     y_channels_last = y_channels_last ? 1 : 0;
     if (x_channels_last == op->x_channels_last && y_channels_last == op->y_channels_last)
         return DLP_OK;
+    if ((x_channels_last || y_channels_last) && op->max_pool)
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: not with a max pooling inside the convolution");
     if ((x_channels_last || y_channels_last) && op->algo != ALGO_GEMM)
         return fail(DLP_ERR_NOT_IMPLEMENTED, "channels-last tensors: algorithm gemm on bfloat16_data only");
     ConvGeom g;
@@ -687,6 +695,23 @@ int dlp_conv2d_fwd_set_channels_last(dlp_conv2d_fwd *op, int x_channels_last, in
     op->x_channels_last = x_channels_last;
     op->y_channels_last = y_channels_last;
     op->workspace = conv_gemm_workspace_bytes(g, op->activation);
+    return DLP_OK;
+}
+
+int dlp_conv2d_fwd_fuse_max_pool(dlp_conv2d_fwd *op, int kernel, int stride, int pad, int ceil_mode)
+{
+    DLP_REQUIRE(op != nullptr, "null argument");
+    ConvGeom g;
+    const int rc = make_geom(op->cfg, op->cfg.shape, g);
+    if (rc != DLP_OK)
+        return rc;
+    const int ph = (g.OH + 2 - 3) / 2 + 1, pw = (g.OW + 2 - 3) / 2 + 1;
+    if (kernel != 3 || stride != 2 || pad != 1 || ceil_mode || op->algo != ALGO_GEMM || op->x_channels_last || op->y_channels_last ||
+        op->activation == DLP_ACT_TANH || op->activation == DLP_ACT_SIGMOID || !conv_stem_pool_supported(g, ph, pw))
+        return fail(DLP_ERR_NOT_IMPLEMENTED, "max pooling inside the convolution: 3x3 stride 2 pad 1 (floor mode) behind the bfloat16 7x7 stride-2 "
+                                             "convolution of 3 channels, rows of the image, of y and of the pooled y in multiples of 8 (y up to 112 wide), "
+                                             "relu-like or no activation");
+    op->max_pool = 1;
     return DLP_OK;
 }
 

@@ -59,6 +59,7 @@ struct ConvGeom {
     // tensor layouts of the implicit-GEMM convolution on the bf16 matrix instruction: x and / or y as [image][pixel][channel]
     // instead of [image][channel][pixel] (the reference knows the latter only: src/core/conv.cpp works on NCHW throughout)
     int x_channels_last = 0, y_channels_last = 0;
+    int pool_ph = 0, pool_pw = 0; // > 0: the stem kernel runs a 3x3 stride-2 pad-1 max pooling behind the convolution, y is [B, Cout, pool_ph, pool_pw]
 };
 
 // Fused epilogue: v = act(acc + bias[c]); y = factor != 0 ? factor*y + v : v
@@ -217,7 +218,9 @@ int conv_gemm_launch(const ConvGeom &g, const GemmPlan &p, const KTabEntry *dev_
 
 // ---- few-channel strided stem convolution (conv_stem.hip) ----------------------
 bool conv_stem_supported(const ConvGeom &g);
-int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream);
+// PH > 0: a 3x3 stride-2 pad-1 max pooling runs inside the kernel and y is the pooled [B, Cout, PH, PW] tensor (bfloat16 only)
+bool conv_stem_pool_supported(const ConvGeom &g, int PH, int PW);
+int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream, int PH = 0, int PW = 0);
 
 // ---- pointwise convolutions with few output channels (conv_pointwise.hip) --------
 bool conv_pointwise_supported(const ConvGeom &g, int activation);

@@ -97,7 +97,11 @@ def infer_shapes(ops, in_shape):
     for o in ops:
         if o["op"] == "conv":
             b, _, h, w = shapes[o["src"]]
-            shapes[o["dst"]] = (b, o["cout"], conv_out(h, o["k"], o["s"], o["p"]), conv_out(w, o["k"], o["s"], o["p"]))
+            oh, ow = conv_out(h, o["k"], o["s"], o["p"]), conv_out(w, o["k"], o["s"], o["p"])
+            if o.get("pool"):  # the max pooling runs inside the convolution: the tensor is the pooled one
+                k, s, p = o["pool"]
+                oh, ow = dlp.pool2d_output_size(oh, k, p, s), dlp.pool2d_output_size(ow, k, p, s)
+            shapes[o["dst"]] = (b, o["cout"], oh, ow)
         elif o["op"] == "maxpool":
             b, c, h, w = shapes[o["src"]]
             shapes[o["dst"]] = (b, c, dlp.pool2d_output_size(h, o["k"], o["p"], o["s"]), dlp.pool2d_output_size(w, o["k"], o["p"], o["s"]))
@@ -114,7 +118,7 @@ def infer_shapes(ops, in_shape):
 class GraphRunner:
     """Runs a graph on cuda:0 through the C ABI: operators are created once for a batch size."""
 
-    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False, prepack=False, channels_last=False):
+    def __init__(self, ops, params, in_shape, algo="", dtype="float32", fuse_residual=False, prepack=False, channels_last=False, fuse_stem_pool=False):
         """dtype "float32" or "bfloat16": storage type of activations and weights (bias stays fp32).
         fuse_residual: a residual sum whose later branch is a 1x1 convolution runs in that convolution's epilogue
         (dlp_conv2d_fwd_set_accumulate_first: y = act(conv + bias + y) written over the other branch), which is what
@@ -124,7 +128,9 @@ class GraphRunner:
         its filter again, which is the contract of the reference's enqueue.
         channels_last (bfloat16, algorithm gemm): tensors between convolutions are kept as [image][row][column][channel]
         wherever every operator that touches them can take that layout and one of the readers is faster on it
-        (dlp_conv2d_fwd_set_channels_last; see _plan_layouts).  Input, logits and parameters keep their layout."""
+        (dlp_conv2d_fwd_set_channels_last; see _plan_layouts).  Input, logits and parameters keep their layout.
+        fuse_stem_pool (bfloat16): a max pooling that is the only reader of a convolution runs inside that convolution where
+        dlp_conv2d_fwd_fuse_max_pool takes it (the 7x7 stride-2 stem of a ResNet and its 3x3 stride-2 pooling)."""
         import torch
 
         import dlprimitives_amd as dlp
@@ -134,6 +140,8 @@ class GraphRunner:
         alias = {}
         if fuse_residual:
             ops = self._fuse_residual_sums(ops, alias)
+        if fuse_stem_pool and dtype == "bfloat16":
+            ops = self._fuse_max_pooling(ops, in_shape, algo)
         self.ops = ops
         self.shapes = infer_shapes(ops, in_shape)
         tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
@@ -157,6 +165,8 @@ class GraphRunner:
                 op = dlp.Conv2DForward.create(st, True, o["act"], algo)
                 if o.get("residual"):
                     op.accumulate_before_activation(True)
+                if o.get("pool"):
+                    op.fuse_max_pool(*o["pool"])
                 if o["src"] in self.cl or o["dst"] in self.cl:
                     op.channels_last(o["src"] in self.cl, o["dst"] in self.cl)
                 ws_bytes = max(ws_bytes, op.workspace())
@@ -216,6 +226,30 @@ class GraphRunner:
         return {n for n in shapes if root(n) in chosen}
 
     @staticmethod
+    def _fuse_max_pooling(ops, in_shape, algo):
+        """conv -> maxpool with nothing else reading the convolution's output: the convolution takes the pooling along (key "pool":
+        kernel, stride, pad) and writes the pooling's tensor, where the library can do that; otherwise the pair stays as it is"""
+        import dlprimitives_amd as dlp
+        from dlprimitives_amd.capi import BFLOAT16_DATA, NotImplementedErrorDlprim
+
+        shapes = infer_shapes(ops, in_shape)
+        out = []
+        for o in ops:
+            prev = out[-1] if out else None
+            if (o["op"] == "maxpool" and prev is not None and prev["op"] == "conv" and prev["dst"] == o["src"] and not prev.get("residual")
+                    and sum(1 for q in ops if o["src"] == q["src"] or (isinstance(q["src"], list) and o["src"] in q["src"])) == 1):
+                st = dlp.Conv2DSettings(prev["cin"], prev["cout"], prev["k"], prev["s"], 1, prev["p"], 1, shapes[prev["src"]], dtype=BFLOAT16_DATA)
+                try:
+                    dlp.Conv2DForward.create(st, True, prev["act"], algo).fuse_max_pool(o["k"], o["s"], o["p"])
+                except NotImplementedErrorDlprim:
+                    out.append(o)
+                    continue
+                prev.update(pool=(o["k"], o["s"], o["p"]), pname=prev.get("pname", prev["dst"]), dst=o["dst"])
+                continue
+            out.append(o)
+        return out
+
+    @staticmethod
     def _fuse_residual_sums(ops, alias):
         """add(c, skip) with c = a 1x1 convolution without activation that only the sum reads: the convolution takes the
         sum's activation, reads skip as its old output and writes the sum's tensor, which shares skip's memory; the
@@ -264,8 +298,8 @@ class GraphRunner:
         total = 0.0
         for o in self.ops:
             if o["op"] == "conv":
-                b, c, h, w = self.shapes[o["dst"]]
-                total += 2.0 * b * c * h * w * o["cin"] * o["k"] * o["k"]
+                b, _, h, w = self.shapes[o["src"]]
+                total += 2.0 * b * o["cout"] * conv_out(h, o["k"], o["s"], o["p"]) * conv_out(w, o["k"], o["s"], o["p"]) * o["cin"] * o["k"] * o["k"]
             elif o["op"] == "ip":
                 total += 2.0 * self.shapes[o["dst"]][0] * o["inputs"] * o["outputs"]
         return total

@@ -184,6 +184,16 @@ int dlp_conv2d_fwd_set_accumulate_first(dlp_conv2d_fwd *op, int on);
  * layout of x (no channels-last copy of the input is staged). */
 int dlp_conv2d_fwd_set_channels_last(dlp_conv2d_fwd *op, int x_channels_last, int y_channels_last);
 
+/* Max pooling inside the convolution.  No counterpart in the reference, where the pooling is an operator of its own
+ * (src/ops/pooling.cpp).  After this call enqueue / enqueue_packed write y = max_pool(act(conv + bias)) -- the tensor
+ * [B, channels_out, PH, PW] that Pooling2D with this kernel, stride and pad would make of the convolution's output -- and the
+ * convolution's own output is never written: the stem of a ResNet leaves a quarter of the bytes and the pooling's pass is gone.
+ * Values equal those of the two operators run one after the other.  Served: max pooling 3x3, stride 2, pad 1, ceil_mode 0, behind
+ * the bfloat16 7x7 stride-2 convolution of 3 input channels (algorithm "gemm") whose image rows, output rows (up to 112 pixels) and
+ * pooled rows are multiples of 8 pixels, activations identity / relu / relu6; at enqueue x and y 16-byte aligned and factor 0.
+ * Anything else: DLP_ERR_NOT_IMPLEMENTED and the operator stays as it was.  Not together with channels-last tensors. */
+int dlp_conv2d_fwd_fuse_max_pool(dlp_conv2d_fwd *op, int kernel, int stride, int pad, int ceil_mode);
+
 void dlp_conv2d_fwd_destroy(dlp_conv2d_fwd *op);
 
 /* ---- Depthwise 3x3 convolution followed by a pointwise (1x1) convolution in one launch.  No counterpart in the

@@ -173,6 +173,86 @@ def test_bf16_stem(oracle_mod, c, bhw):
     np.testing.assert_allclose(got, want, rtol=2 ** -8, atol=1e-3)
 
 
+# the stem with its max pooling inside: (case, (batch, H, W)); every one takes workgroup ranges that start in the middle of an image
+STEM_POOL_CASES = [
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (5, 224, 224)),    # the ResNet stem: 56 x 56 pooled
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (130, 64, 64)),    # more images than workgroups: ranges span images; 32 x 32 -> 16 x 16
+    (case(7, 3, 2, 1, 3, 40, False, 1, False), (3, 72, 96)),    # fewer filters than a tile, no bias, no activation (negative maxima); 36 x 48 -> 18 x 24
+    (case(7, 3, 2, 1, 3, 96, True, 1, True), (2, 90, 160)),     # two filter tiles; 45 rows: the last pooled row looks at two rows only; 45 x 80 -> 23 x 40
+    (case(7, 3, 2, 1, 3, 64, True, 1, True), (3, 20, 32)),      # 10 x 16 -> 5 x 8: one run of pooled columns, three units an image
+]
+
+
+@pytest.mark.parametrize("c,bhw", STEM_POOL_CASES, ids=case_id)
+def test_bf16_stem_with_max_pooling_inside(oracle_mod, c, bhw):
+    """dlp_conv2d_fwd_fuse_max_pool against the convolution and Pooling2D run one after the other: the same values bit for bit,
+    and against the oracle's convolution followed by a numpy pooling"""
+    import torch
+
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA
+
+    print("stem+pool", c["pad"], c["cout"], bhw, flush=True)
+    x, w, bias = make_tensors(c, bhw, seed=43)
+    x, w = oracle_mod.bf16_round(x), oracle_mod.bf16_round(w)
+    st = dlp.Conv2DSettings(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"], x.shape, dtype=BFLOAT16_DATA)
+    xd, wd = _bf(x), _bf(w)
+    bd = torch.from_numpy(bias).cuda() if bias is not None else None
+    plain = dlp.Conv2DForward.create(st, bias is not None, c["activation"], "gemm")
+    oshape = dlp.conv2d_output_shape(st, x.shape)
+    mid = torch.full(oshape, float("nan"), dtype=torch.bfloat16, device="cuda:0")
+    ws = torch.empty(max(plain.workspace(), 1), dtype=torch.uint8, device="cuda:0")
+    plain.enqueue(xd, wd, bd, mid, ws)
+    pshape = (oshape[0], oshape[1], dlp.pool2d_output_size(oshape[2], 3, 1, 2), dlp.pool2d_output_size(oshape[3], 3, 1, 2))
+    want = torch.full(pshape, float("nan"), dtype=torch.bfloat16, device="cuda:0")
+    dlp.Pooling2DForward.create_max_pooling(3, 1, 2, dtype=BFLOAT16_DATA).enqueue(mid, want)
+    fused = dlp.Conv2DForward.create(st, bias is not None, c["activation"], "gemm")
+    fused.fuse_max_pool(3, 2, 1)
+    got = torch.full(pshape, float("nan"), dtype=torch.bfloat16, device="cuda:0")
+    fused.enqueue(xd, wd, bd, got, ws)
+    torch.cuda.synchronize()
+    got, want = got.float().cpu().numpy(), want.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    assert np.array_equal(got, want)
+    # and the oracle: its fp32 convolution, pooled here
+    cfg = oracle_mod.make_cfg(c["cin"], c["cout"], c["kernel"], c["stride"], c["dilate"], c["pad"], c["groups"])
+    conv = oracle_mod.conv2d_forward(x[:2], w, bias, cfg, c["activation"], threads=8)
+    padded = np.full(conv.shape[:2] + (conv.shape[2] + 2, conv.shape[3] + 2), -np.inf, np.float32)
+    padded[:, :, 1:-1, 1:-1] = conv
+    ref = np.full((2,) + pshape[1:], -np.inf, np.float32)
+    for dy in range(3):
+        for dx in range(3):
+            ref = np.maximum(ref, padded[:, :, dy:dy + 2 * pshape[2]:2, dx:dx + 2 * pshape[3]:2][:, :, :pshape[2], :pshape[3]])
+    np.testing.assert_allclose(got[:2], ref, rtol=2 ** -8, atol=1e-4 * np.abs(ref).max())
+
+
+def test_bf16_stem_max_pooling_is_refused_where_not_served():
+    import dlprimitives_amd as dlp
+    from dlprimitives_amd.capi import BFLOAT16_DATA, FLOAT_DATA, NotImplementedErrorDlprim
+
+    def stem(dtype, hw=(224, 224), act="relu", k=7, cin=3):
+        st = dlp.Conv2DSettings(cin, 64, k, 2, 1, k // 2, 1, (2, cin) + hw, dtype=dtype)
+        return dlp.Conv2DForward.create(st, True, act, "gemm")
+
+    stem(BFLOAT16_DATA).fuse_max_pool(3, 2, 1)
+    for args in [(2, 2, 0), (3, 1, 1), (3, 2, 0)]:  # other poolings
+        with pytest.raises(NotImplementedErrorDlprim):
+            stem(BFLOAT16_DATA).fuse_max_pool(*args)
+    with pytest.raises(NotImplementedErrorDlprim):
+        stem(BFLOAT16_DATA).fuse_max_pool(3, 2, 1, ceil_mode=True)
+    with pytest.raises(NotImplementedErrorDlprim):
+        stem(FLOAT_DATA).fuse_max_pool(3, 2, 1)               # float tensors
+    with pytest.raises(NotImplementedErrorDlprim):
+        stem(BFLOAT16_DATA, hw=(100, 92)).fuse_max_pool(3, 2, 1)  # rows off the 8-pixel runs
+    with pytest.raises(NotImplementedErrorDlprim):
+        stem(BFLOAT16_DATA, act="tanh").fuse_max_pool(3, 2, 1)
+    with pytest.raises(NotImplementedErrorDlprim):
+        stem(BFLOAT16_DATA, k=3, cin=32).fuse_max_pool(3, 2, 1)   # not the stem kernel
+    op = stem(BFLOAT16_DATA)
+    op.fuse_max_pool(3, 2, 1)
+    with pytest.raises(NotImplementedErrorDlprim):
+        op.channels_last(False, True)
+
 DENSE_1X1_CASES = [
     # 1x1 convolutions of 64 / 128 channels over thousands of pixels (the short-K layers of a ResNet-50 bottleneck): the dense loader
     # with two or four K tiles per workgroup, plain, bit-exact on integers, and with both ways of adding the old y
