@@ -543,20 +543,37 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
                 for (int r = 0; r < 16; r++)
                     acc[cb][r] = b;
             }
-            stem_for<NJ>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
+            // operands of step j + DEPTH are asked for before the matrix instructions of step j: left to itself the compiler reads
+            // each step's operands right in front of their use and every step waits for a whole trip to LDS (deeper than one step
+            // ahead the 128 registers of a 1024-thread workgroup run out, and the block is bound by LDS reads anyway: 3 KB a step)
+            constexpr int DEPTH = 1;
+            stem_u32x4 px[DEPTH + 1];
+            stem_bf16x8 w0[DEPTH + 1], w1[DEPTH + 1];
+            auto fetch = [&](auto jc) {
+                constexpr int j = decltype(jc)::value, slot = j % (DEPTH + 1);
                 constexpr int q0 = 2 * j, q1 = 2 * j + 1;
                 constexpr int o0 = ((q0 / KH) * ROWS + q0 % KH) * PITCH, o1 = ((q1 / KH) * ROWS + q1 % KH) * PITCH;
                 constexpr int d = q1 < Q ? o1 - o0 : 0; // the spare filter row has zero weights: the other half's values do
                 static_assert(d == 0 || d == D1 || d == D2, "filter row distance");
                 static_assert(o0 % 2 == 0, "dword aligned");
                 const uint32_t *pp = (d == D1 ? P1 : d == D2 ? P2 : P0) + o0 / 2;
-                stem_u32x4 px;
-                px[0] = pp[0], px[1] = pp[1], px[2] = pp[2], px[3] = pp[3];
-                const stem_bf16x8 xa = __builtin_bit_cast(stem_bf16x8, px);
-                const stem_bf16x8 w0 = *(const stem_bf16x8 *)(Wb + j * 16), w1 = *(const stem_bf16x8 *)(Wb + 32 * WPITCH + j * 16);
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w0, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w1, acc[1], 0, 0, 0);
+                px[slot][0] = pp[0], px[slot][1] = pp[1], px[slot][2] = pp[2], px[slot][3] = pp[3];
+                w0[slot] = *(const stem_bf16x8 *)(Wb + j * 16);
+                w1[slot] = *(const stem_bf16x8 *)(Wb + 32 * WPITCH + j * 16);
+            };
+            stem_for<DEPTH>([&](auto jc) {
+                if constexpr (decltype(jc)::value < NJ)
+                    fetch(jc);
+            });
+            stem_for<NJ>([&](auto jc) {
+                constexpr int j = decltype(jc)::value, slot = j % (DEPTH + 1);
+                if constexpr (j + DEPTH < NJ)
+                    fetch(std::integral_constant<int, j + DEPTH>{});
+                __builtin_amdgcn_sched_barrier(0); // keep this order: the scheduler would sink the operand reads to their uses
+                const stem_bf16x8 xa = __builtin_bit_cast(stem_bf16x8, px[slot]);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w0[slot], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, w1[slot], acc[1], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             });
 
             // accumulator register r of filter block cb: filter m0 + 32 * cb + l32, pixel blk * 32 + 8 * (r / 4) + 4 * h + r % 4

@@ -94,6 +94,14 @@ public:
         if (x || y)
             throw NotImplementedError("channels_last is not implemented by this Conv2DForward");
     }
+    // Not in the reference (the pooling is an operator of its own there): y becomes the max pooling of the convolution's output,
+    // [B, channels_out, PH, PW], and the convolution's own output is never written (dlp_conv2d_fwd_fuse_max_pool: the bfloat16
+    // 7x7 stride-2 stem and its 3x3 stride-2 pad-1 pooling).  The default refuses.
+    virtual void fuse_max_pool(int kernel, int stride, int pad, bool ceil_mode)
+    {
+        (void)kernel, (void)stride, (void)pad, (void)ceil_mode;
+        throw NotImplementedError("fuse_max_pool is not implemented by this Conv2DForward");
+    }
     static std::unique_ptr<Conv2DForward> create(Context &ctx, Conv2DSettings const &config, bool bias,
                                                  StandardActivations activation = StandardActivations::identity,
                                                  std::string const &algo = std::string());
@@ -130,6 +138,10 @@ public:
 
     void accumulate_before_activation(bool on) override { dlprim::details::check_status(dlp_conv2d_fwd_set_accumulate_first(op_, on ? 1 : 0)); }
     void channels_last(bool x, bool y) override { dlprim::details::check_status(dlp_conv2d_fwd_set_channels_last(op_, x ? 1 : 0, y ? 1 : 0)); }
+    void fuse_max_pool(int kernel, int stride, int pad, bool ceil_mode) override
+    {
+        dlprim::details::check_status(dlp_conv2d_fwd_fuse_max_pool(op_, kernel, stride, pad, ceil_mode ? 1 : 0));
+    }
     size_t packed_size() override { return dlp_conv2d_fwd_packed_bytes(op_); }
     void pack(Tensor &w, Tensor &packed, ExecutionContext const &e) override
     {

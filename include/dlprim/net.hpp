@@ -163,6 +163,9 @@ public:
     // take that layout and a reader is faster on it (plan_layouts; default on; network inputs, outputs and parameters keep the
     // reference's layout, and nothing changes with float_data or keep_intermediate_tensors)
     void channels_last(bool on) { channels_last_ = on; }
+    // A max pooling that is the only reader of a bfloat16 convolution runs inside that convolution where the device code has such a
+    // kernel (the 7x7 stride-2 stem of a ResNet with its 3x3 stride-2 pooling; default on, part of the graph rewrites)
+    void fuse_max_pooling(bool on) { fuse_max_pool_ = on; }
 
     // shapes, rewrites, operators, memory; parameters are allocated (zero on the host) and wait for load_parameters
     void setup()
@@ -224,6 +227,11 @@ public:
                     break;
                 }
                 out = core::Conv2DBase::get_output_shape(n.conv, in);
+                if (n.pool_node >= 0) { // the node writes the pooled tensor
+                    Node const &pl = nodes_[size_t(n.pool_node)];
+                    out = Shape(out[0], out[1], size_t(core::calc_pooling_output_size(int(out[2]), pl.kernel[0], pl.pad[0], pl.stride[0], pl.ceil_mode)),
+                                size_t(core::calc_pooling_output_size(int(out[3]), pl.kernel[1], pl.pad[1], pl.stride[1], pl.ceil_mode)));
+                }
                 Shape const &old = n.planned_in;
                 if (n.conv_op && (old[2] != in[2] || old[3] != in[3])) {
                     create_conv_operator(n, in);
@@ -471,6 +479,7 @@ private:
         std::unique_ptr<core::Conv2DForward> conv_op;
         std::unique_ptr<core::TransposedConv2DForward> tconv_op; // TransposedConvolution2D
         int dw_node = -1; // a 1x1 convolution that also runs the depthwise convolution in front of it: index of that (skipped) node
+        int pool_node = -1; // a convolution that also runs the max pooling behind it: index of that (skipped) node
         std::unique_ptr<core::DepthwisePointwiseForward> dwpw_op;
         int output_pad[2] = {0, 0};
         std::unique_ptr<core::IPForward> ip_op;
@@ -1176,6 +1185,31 @@ private:
         d.skipped = true;
     }
 
+    // A max pooling into the convolution that feeds only it, where the device code runs the pair as one kernel (the bfloat16 7x7
+    // stride-2 stem of a ResNet and its 3x3 stride-2 pooling): the convolution node then writes the pooling's tensor.
+    void try_fuse_max_pool(size_t i)
+    {
+        Node &c = nodes_[i];
+        if (!fuse_max_pool_ || c.kind != k_conv || c.residual || c.dw_node >= 0 || c.pool_node >= 0 || dtype_ != bfloat16_data || keep_intermediate_ || ctx_.is_cpu_context())
+            return;
+        std::string const t = c.outputs[0];
+        const int u = next_user(i, t);
+        if (u < 0 || is_net_output(t) || readers_after(i, t) != 1)
+            return;
+        Node &pl = nodes_[size_t(u)];
+        if (pl.kind != k_pool || !pl.max_mode || pl.inputs[0] != t || pl.kernel[0] != pl.kernel[1] || pl.stride[0] != pl.stride[1] || pl.pad[0] != pl.pad[1])
+            return;
+        try { // the library decides: an operator of this geometry is asked
+            core::Conv2DSettings cfg(c.conv, spec(c.inputs[0]), dtype_);
+            core::Conv2DForward::create(ctx_, cfg, c.bias || c.folded_bn, c.activation, c.algo)->fuse_max_pool(pl.kernel[0], pl.stride[0], pl.pad[0], pl.ceil_mode);
+        } catch (NotImplementedError const &) {
+            return;
+        }
+        c.pool_node = u;
+        c.outputs[0] = pl.outputs[0];
+        pl.skipped = true;
+    }
+
     void rewrite_graph()
     {
         for (size_t i = 0; i < nodes_.size(); i++) {
@@ -1190,6 +1224,9 @@ private:
         for (size_t i = 0; i < nodes_.size(); i++) // after the loop above: both nodes have their final activation and bias
             if (!nodes_[i].skipped)
                 try_fuse_depthwise_pointwise(i);
+        for (size_t i = 0; i < nodes_.size(); i++)
+            if (!nodes_[i].skipped)
+                try_fuse_max_pool(i);
     }
 
     void create_conv_operator(Node &n, Shape const &in)
@@ -1208,6 +1245,10 @@ private:
         n.conv_op = core::Conv2DForward::create(ctx_, cfg, n.bias || n.folded_bn, n.activation, n.algo);
         if (n.residual)
             n.conv_op->accumulate_before_activation(true);
+        if (n.pool_node >= 0) {
+            Node const &pl = nodes_[size_t(n.pool_node)];
+            n.conv_op->fuse_max_pool(pl.kernel[0], pl.stride[0], pl.pad[0], pl.ceil_mode);
+        }
         const bool x_cl = is_channels_last(n.inputs[0]), y_cl = is_channels_last(n.outputs[0]);
         if (x_cl || y_cl)
             n.conv_op->channels_last(x_cl, y_cl);
@@ -1658,6 +1699,7 @@ private:
     size_t workspace_bytes_ = 0, tensor_memory_ = 0;
     bool keep_intermediate_ = false, fuse_ = true, prepack_ = true, ready_ = false;
     bool channels_last_ = true;
+    bool fuse_max_pool_ = true;
     std::set<std::string> cl_groups_; // tensors kept channels-last, by the name their memory goes by (alias_root)
     DataType dtype_ = float_data;
     std::shared_ptr<dlp_graph> graph_;

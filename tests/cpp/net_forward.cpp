@@ -6,12 +6,13 @@
 //   net_forward plan <net.json> [keep] [nofuse]
 //       shape inference, graph rewrites and memory plan on a CPU context (no GPU); prints
 //       "operators <n> tensor_memory <bytes>" and one "tensor <name> <dims...>" line per output
-//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [nchw] [batch=<n>] [resave=<file.dlpw>] [repeat=<n>]
+//   net_forward run <net.json> <params.dlpw> <inputs.bin> <outputs.bin> [keep] [nofuse] [nopack] [graph] [bf16] [nchw] [poolop] [batch=<n>] [resave=<file.dlpw>] [repeat=<n>]
 //       (batch=<n>: the inputs are reshaped to n images and Net::reshape() is called before the pass)
-//       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32; nchw: no channels-last tensors between bf16 convolutions)
+//       (bf16: tensors and weights stored as bfloat16 on the device; files stay float32; nchw: no channels-last tensors between bf16 convolutions;
+//        poolop: the max pooling behind a bf16 stem stays an operator of its own)
 //       loads the network and its parameters on HIP device 0, reads the inputs (float32, in the
 //       network's input order), runs forward and writes the outputs (float32, in output order)
-//   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse] [graph]
+//   net_forward time <net.json> [warmup=<n>] [iters=<n>] [keep] [nofuse] [graph] [bf16] [nchw] [poolop]
 //       (graph: the forward pass is recorded once as a HIP graph and replayed)
 //       random parameters and inputs, ms per forward pass on HIP device 0 (what the reference's
 //       tools/benchmark.cpp reports for its docs/nets_for_benchmark files)
@@ -48,7 +49,7 @@ int main(int argc, char **argv)
             std::cout << v.save() << std::endl;
             return 0;
         }
-        bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false, nchw = false;
+        bool keep = false, fuse = true, graph = false, prepack = true, bf16 = false, nchw = false, poolop = false;
         std::string resave;
         int repeat = 1, warmup = 5, iters = 20, batch = 0;
         const int first_flag = (cmd == "plan" || cmd == "time") ? 3 : 6;
@@ -66,6 +67,8 @@ int main(int argc, char **argv)
                 bf16 = true;
             else if (a == "nchw")
                 nchw = true;
+            else if (a == "poolop")
+                poolop = true;
             else if (a.compare(0, 7, "resave=") == 0)
                 resave = a.substr(7);
             else if (a.compare(0, 7, "repeat=") == 0)
@@ -86,6 +89,7 @@ int main(int argc, char **argv)
             net.fuse(fuse);
             net.prepack(prepack);
             net.channels_last(!nchw);
+            net.fuse_max_pooling(!poolop);
             net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
@@ -106,6 +110,7 @@ int main(int argc, char **argv)
             net.fuse(fuse);
             net.prepack(prepack);
             net.channels_last(!nchw);
+            net.fuse_max_pooling(!poolop);
             net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
             net.load_from_json_file(argv[2]);
             net.setup();
@@ -153,6 +158,7 @@ int main(int argc, char **argv)
         net.fuse(fuse);
         net.prepack(prepack);
             net.channels_last(!nchw);
+            net.fuse_max_pooling(!poolop);
         net.storage_type(bf16 ? dp::bfloat16_data : dp::float_data);
         net.mode(dp::CalculationsMode::predict);
         net.load_from_json_file(argv[2]);

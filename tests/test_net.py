@@ -526,8 +526,9 @@ NETS = {
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("flags", [(), ("nofuse",), ("keep",), ("nofuse", "keep"), ("graph",), ("graph", "nofuse"), ("nopack",), ("bf16",), ("bf16", "nofuse"),
-                                   ("bf16", "nchw"), ("bf16", "graph")],
-                         ids=["default", "nofuse", "keep", "nofuse_keep", "graph", "graph_nofuse", "nopack", "bf16", "bf16_nofuse", "bf16_nchw", "bf16_graph"])
+                                   ("bf16", "nchw"), ("bf16", "graph"), ("bf16", "poolop")],
+                         ids=["default", "nofuse", "keep", "nofuse_keep", "graph", "graph_nofuse", "nopack", "bf16", "bf16_nofuse", "bf16_nchw", "bf16_graph",
+                              "bf16_poolop"])
 @pytest.mark.parametrize("net", list(NETS))
 def test_gpu_net_forward_matches_torch(tmp_path, net, flags):
     if net == "upsampling" and "bf16" in flags:
