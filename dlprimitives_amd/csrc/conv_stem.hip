@@ -353,13 +353,14 @@ typedef uint32_t stem_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t stem_u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kStemPadL16 = 8;     // zero columns left of an input row (keeps the 16-byte LDS stores aligned)
+constexpr int kStemPoolPitch = 120;  // elements per row of convolution results kept for the pooling: 8 to the left, up to 112 columns
 constexpr int kStemStagePitch = 80; // bytes per filter of a wavefront's staged 32 x 32 output block (64 + 16: 16-byte rows)
 
 template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, int NT, bool POOL = false>
 constexpr int stem_bf16_lds_bytes()
 {
     constexpr int ROWS = STRIDE * (R - 1) + KH, QP = (CIN * KH + 1) / 2 * 2;
-    return CIN * ROWS * PITCH * 2 + 64 * (QP * 8 + 8) * 2 + 64 * 4 + (POOL ? 64 * R * (PITCH / 2) * 2 : (NT / 64) * 32 * kStemStagePitch);
+    return CIN * ROWS * PITCH * 2 + 64 * (QP * 8 + 8) * 2 + 64 * 4 + (POOL ? 64 * R * kStemPoolPitch * 2 : (NT / 64) * 32 * kStemStagePitch);
 }
 
 // POOL: the 3x3 stride-2 pad-1 max pooling that follows the stem of every ResNet runs inside the kernel.  The workgroup walks units
@@ -372,7 +373,7 @@ template <int CIN, int KH, int KW, int STRIDE, int R, int PITCH, bool VEC, int N
 __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
 {
     static_assert(!POOL || (VEC && R == 5), "the pooled form: five rows at most and 16-byte input loads");
-    constexpr int OBP = PITCH / 2; // POOL: elements per row of the results in LDS
+    constexpr int OBP = kStemPoolPitch; // POOL: elements per row of the results in LDS
     static_assert(KW <= 7, "a filter row and its leading zero are the eight k of a lane");
     constexpr int K = CIN * KH * KW;
     constexpr int Q = CIN * KH, QP = (Q + 1) / 2 * 2, NJ = QP / 2; // filter rows, two per matrix instruction
@@ -697,6 +698,7 @@ __global__ __launch_bounds__(NT) void conv_stem_bf16_kernel(StemArgs a)
 }
 
 constexpr int kStemR = 8, kStemPitch = 240, kStemPoolR = 5;
+constexpr int kStemPitchBf16 = 240; // 320 (rows of the two lane halves on different LDS banks) measured the same
 
 bool generic_activation(int act) { return act == DLP_ACT_TANH || act == DLP_ACT_SIGMOID; }
 
@@ -716,7 +718,7 @@ bool conv_stem_supported(const ConvGeom &g)
         // a lane's eight k start one element left of the window, on an even LDS column: odd paddings only;
         // rightmost column read: the eighth element of the last output column
         const int e0 = kStemPadL16 - g.pw - 1;
-        return e0 >= 0 && e0 % 2 == 0 && 2 * (g.OW - 1) + e0 + 7 < kStemPitch && g.W + 2 * kStemPadL16 <= kStemPitch;
+        return e0 >= 0 && e0 % 2 == 0 && 2 * (g.OW - 1) + e0 + 7 < kStemPitchBf16 && g.W + 2 * kStemPadL16 <= kStemPitchBf16;
     }
     if (g.pw > kStemPadL || g.Cout % 8 != 0)
         return false;
@@ -729,7 +731,7 @@ bool conv_stem_pool_supported(const ConvGeom &g, int PH, int PW)
     // whole runs of eight pixels in convolution and pooled rows; the last pooling window ends inside the row (the columns
     // right of it are not initialised in LDS) and starts inside the image
     return g.dtype == DLP_BFLOAT16 && conv_stem_supported(g) && g.W % 8 == 0 && g.OW % 8 == 0 && PW % 8 == 0 && PW >= 8 && 2 * PW == g.OW &&
-           PH >= 1 && 2 * (PH - 1) - 1 < g.OH && 8 + g.OW <= kStemPitch / 2 && (long long)g.Cout * PH * PW * 2 < 0x7fffffffLL;
+           PH >= 1 && 2 * (PH - 1) - 1 < g.OH && 8 + g.OW <= kStemPoolPitch && (long long)g.Cout * PH * PW * 2 < 0x7fffffffLL;
 }
 
 int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, const Epilogue &ep, hipStream_t stream, int PH, int PW)
@@ -765,7 +767,7 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     // 16-byte loads: every input row and (fp32) the filter rows of every m tile then start 16-byte aligned
     const bool vec = bf16 ? g.W % 8 == 0 && ((uintptr_t)x & 15) == 0 : g.W % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
     make_magic((uint32_t)g.OW, a.ow_magic, a.ow_shift);
-    a.padw = (uint32_t)(kStemPitch - g.W);
+    a.padw = (uint32_t)((bf16 ? kStemPitchBf16 : kStemPitch) - g.W);
     a.e0 = kStemPadL16 - g.pw - 1;
     make_magic(a.padw, a.padw_magic, a.padw_shift);
     a.factor = ep.factor;
@@ -780,8 +782,8 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
     const dim3 grid((unsigned)((a.total_rows + a.rows_per_wg - 1) / a.rows_per_wg)), block(kStemThreads);
     TimingScope ts("conv_gemm", stream);
     if (pool) {
-        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemPoolR, kStemPitch, kStemThreads, true>();
-        auto kernel = conv_stem_bf16_kernel<3, 7, 7, 2, kStemPoolR, kStemPitch, true, kStemThreads, true>;
+        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemPoolR, kStemPitchBf16, kStemThreads, true>();
+        auto kernel = conv_stem_bf16_kernel<3, 7, 7, 2, kStemPoolR, kStemPitchBf16, true, kStemThreads, true>;
         static bool asked[64] = {}; // per device
         int dev = 0;
         DLP_HIP_TRY(hipGetDevice(&dev));
@@ -795,8 +797,8 @@ int conv_stem_launch(const ConvGeom &g, const void *x, const void *w, void *y, c
         return DLP_OK;
     }
     if (bf16) {
-        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemR, kStemPitch, kStemThreads>();
-        auto kernel = vec ? conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, true, kStemThreads> : conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitch, false, kStemThreads>;
+        constexpr int lds = stem_bf16_lds_bytes<3, 7, 7, 2, kStemR, kStemPitchBf16, kStemThreads>();
+        auto kernel = vec ? conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitchBf16, true, kStemThreads> : conv_stem_bf16_kernel<3, 7, 7, 2, kStemR, kStemPitchBf16, false, kStemThreads>;
         // more than 64 KB of LDS has to be asked for (bands of 16 rows, or two workgroups of 8 wavefronts per CU, were no faster)
         static bool asked[2][64] = {}; // per kernel and device
         int dev = 0;
