@@ -164,7 +164,9 @@ public:
     // reference's layout, and nothing changes with float_data or keep_intermediate_tensors)
     void channels_last(bool on) { channels_last_ = on; }
     // A max pooling that is the only reader of a bfloat16 convolution runs inside that convolution where the device code has such a
-    // kernel (the 7x7 stride-2 stem of a ResNet with its 3x3 stride-2 pooling; default on, part of the graph rewrites)
+    // kernel (the 7x7 stride-2 stem of a ResNet with its 3x3 stride-2 pooling; default on, part of the graph rewrites).  The pair stays
+    // one operator for the life of the network: reshape() to an image size that the kernel does not serve (rows off the multiples of
+    // 8 pixels) throws NotImplementedError, so a network that will see such sizes switches this off before setup()
     void fuse_max_pooling(bool on) { fuse_max_pool_ = on; }
 
     // shapes, rewrites, operators, memory; parameters are allocated (zero on the host) and wait for load_parameters
