@@ -1061,12 +1061,32 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
     // bytes of a pixel. ----
     if (a.y_cl) {
         constexpr int PITCH = BM * 2 + 16;
+        const bool pre = a.pre != 0 && a.factor != 0.0f; // the old y joins before the activation: in the second phase
+        const bool clamp = a.act != DLP_ACT_IDENTITY && !pre;
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+        constexpr int PPR = BM / 8; // pieces of a pixel's row
+        static_assert((BN * PPR) % kThreads == 0 && kThreads % PPR == 0, "pieces are dealt to the threads evenly");
+        const int piece = tid % PPR, pix_t = tid / PPR;
+        const int m = m0 + piece * 8;
+        const uint32_t col_off = (uint32_t)(g * a.M + m) * 2u;
+        constexpr int STEP = kThreads / PPR;           // pixels between a thread's pieces
+        constexpr int PER_THREAD = BN * PPR / kThreads; // pieces per thread
+        auto piece_offset = [&](int u) {
+            const int n = n0 + pix_t + u * STEP;
+            return (n < a.N && m < a.M) ? (uint32_t)n * (uint32_t)a.Cout * 2u + col_off : kOutOfRange;
+        };
+        // the old values of all the thread's pieces are asked for first: they travel while the tile is rounded and staged
+        // (the accumulators are still live here, the operand registers of the main loop are not)
+        u32x4 old[PER_THREAD];
+        if (pre) {
+#pragma unroll
+            for (int u = 0; u < PER_THREAD; u++)
+                old[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(yr, piece_offset(u), 0, 0));
+        }
         float *bias_s = (float *)(smem + BN * PITCH);
         if (tid < BM)
             bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
         __syncthreads();
-        const bool pre = a.pre != 0 && a.factor != 0.0f; // the old y joins before the activation: in the second phase
-        const bool clamp = a.act != DLP_ACT_IDENTITY && !pre;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             unsigned char *rowp = smem + (wn * WTN + j * 32 + l32) * PITCH + (wm * WTM + 4 * h) * 2;
@@ -1094,57 +1114,34 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
             }
         }
         __syncthreads();
-        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
-        constexpr int PPR = BM / 8; // pieces of a pixel's row
-        static_assert((BN * PPR) % kThreads == 0 && kThreads % PPR == 0, "pieces are dealt to the threads evenly");
         // every pixel's run is whole 128-byte lines, and the tensor is too large for the next layer to find it in the last-level cache:
         // streaming stores
         const bool streaming = (a.Cout & 63) == 0 && (BM & 63) == 0 && a.y_bytes >= (96u << 20);
-        const int piece = tid % PPR, pix_t = tid / PPR;
-        const int m = m0 + piece * 8;
-        const uint32_t col_off = (uint32_t)(g * a.M + m) * 2u;
         const unsigned char *src_t = smem + pix_t * PITCH + piece * 16;
-        constexpr int STEP = kThreads / PPR;           // pixels between a thread's pieces
-        constexpr int PER_THREAD = BN * PPR / kThreads; // pieces per thread
-        static_assert(PER_THREAD % 4 == 0, "pieces are handled four at a time");
-#pragma unroll 1
-        for (int q0 = 0; q0 < PER_THREAD; q0 += 4) {
-            uint32_t voff[4];
-            u32x4 old[4], mine[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) { // the old values of four pieces are requested together: two waits for memory per tile, not eight
-                const int n = n0 + pix_t + (q0 + u) * STEP;
-                voff[u] = (n < a.N && m < a.M) ? (uint32_t)n * (uint32_t)a.Cout * 2u + col_off : kOutOfRange;
-                if (pre)
-                    old[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(yr, voff[u], 0, 0));
-            }
+        for (int u = 0; u < PER_THREAD; u++) {
+            u32x4 mine = *(const u32x4 *)(src_t + u * STEP * PITCH);
+            if (pre) {
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-                mine[u] = *(const u32x4 *)(src_t + (q0 + u) * STEP * PITCH);
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                if (pre) {
-#pragma unroll
-                    for (int d = 0; d < 4; d++) {
-                        float lo = fmaf(__builtin_bit_cast(float, old[u][d] << 16), a.factor, __builtin_bit_cast(float, mine[u][d] << 16));
-                        float hi = fmaf(__builtin_bit_cast(float, old[u][d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[u][d] & 0xFFFF0000u));
-                        if (ACT == ACT_CLAMP) {
-                            if (a.act != DLP_ACT_IDENTITY) {
-                                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
-                                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
-                            }
-                        } else {
-                            lo = apply_act(lo, a.act);
-                            hi = apply_act(hi, a.act);
+                for (int d = 0; d < 4; d++) {
+                    float lo = fmaf(__builtin_bit_cast(float, old[u][d] << 16), a.factor, __builtin_bit_cast(float, mine[d] << 16));
+                    float hi = fmaf(__builtin_bit_cast(float, old[u][d] & 0xFFFF0000u), a.factor, __builtin_bit_cast(float, mine[d] & 0xFFFF0000u));
+                    if (ACT == ACT_CLAMP) {
+                        if (a.act != DLP_ACT_IDENTITY) {
+                            lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                            hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
                         }
-                        mine[u][d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+                    } else {
+                        lo = apply_act(lo, a.act);
+                        hi = apply_act(hi, a.act);
                     }
+                    mine[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
                 }
-                if (streaming)
-                    __builtin_amdgcn_raw_buffer_store_b128(mine[u], yr, voff[u], 0, DLP_BF16_STORE_AUX);
-                else
-                    __builtin_amdgcn_raw_buffer_store_b128(mine[u], yr, voff[u], 0, 0);
             }
+            if (streaming)
+                __builtin_amdgcn_raw_buffer_store_b128(mine, yr, piece_offset(u), 0, DLP_BF16_STORE_AUX);
+            else
+                __builtin_amdgcn_raw_buffer_store_b128(mine, yr, piece_offset(u), 0, 0);
         }
         return;
     }
