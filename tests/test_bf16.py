@@ -389,7 +389,7 @@ def test_global_pooling_channels_last(dtype):
     tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     code = BFLOAT16_DATA if dtype == "bfloat16" else FLOAT_DATA
     rng = np.random.default_rng(2)
-    for shape in [(3, 2048, 7, 7), (2, 72, 5, 9), (1, 8, 1, 1)]:
+    for shape in [(3, 2048, 7, 7), (2, 72, 5, 9), (1, 8, 1, 1), (2, 10, 3, 3), (5, 6, 7, 7)]:  # the last two: one channel per thread
         x = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).cuda().to(tdt)
         for make in (dlp.Pooling2DForward.create_global_avg_pooling, dlp.Pooling2DForward.create_global_max_pooling):
             want = torch.empty((shape[0], shape[1], 1, 1), dtype=tdt, device="cuda:0")
