@@ -2124,50 +2124,68 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmArgs a)
     }
 }
 
-// The same for a channels-last bf16 y: a thread sums eight consecutive channels of one pixel (consecutive threads on consecutive
-// pixels: the partial sums are read in whole lines) and writes them as one 16-byte piece.  Cout a multiple of 8.
-template <int ACT>
+// The same for a channels-last bf16 y: a thread sums eight consecutive channels of PX consecutive pixels (consecutive threads on
+// consecutive pixels: the partial sums are read in whole lines, 4 * PX bytes a load) and writes each pixel's eight channels as one
+// 16-byte piece.  Cout a multiple of 8; PX = 4 needs N in fours and 16-byte aligned partial sums.
+template <int ACT, int PX>
 __global__ __launch_bounds__(256) void splitk_reduce_cl_kernel(GemmArgs a)
 {
-    const int c0 = blockIdx.y * 8;
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n >= a.N)
+    typedef float vec_t __attribute__((ext_vector_type(PX)));
+    // PX = 4: eight neighbouring lanes take eight channel groups of the same four pixels, the next eight lanes the next four pixels:
+    // loads of a (slice, channel) and stores of a pixel both come in whole 128-byte lines (with a lane per pixel the stores of a
+    // wavefront were 64 pieces of 16 bytes in 64 different lines)
+    const int c0 = PX == 1 ? (int)blockIdx.y * 8 : ((int)blockIdx.y * 8 + ((int)threadIdx.x & 7)) * 8;
+    const int n = PX == 1 ? (int)(blockIdx.x * blockDim.x + threadIdx.x) : ((int)blockIdx.x * 32 + ((int)threadIdx.x >> 3)) * PX;
+    if (n >= a.N || c0 >= a.Cout)
         return;
     const size_t total = (size_t)a.Cout * a.N;
     const float *pp = a.part + (size_t)c0 * a.N + n;
-    float v[8];
+    // the old y first, then the slices: eight loads on their way per wait (the sums keep the order slice 0, 1, 2 ...)
+    u32x4 *yp = (u32x4 *)((uint16_t *)a.y + (size_t)n * a.Cout + c0);
+    const size_t ystep = (size_t)a.Cout / 8; // 16-byte pieces between pixels
+    const bool pre = a.pre != 0 && a.factor != 0.0f;
+    u32x4 old[PX];
+    if (pre) {
+#pragma unroll
+        for (int q = 0; q < PX; q++)
+            old[q] = yp[q * ystep];
+    }
+    vec_t v[8];
 #pragma unroll
     for (int i = 0; i < 8; i++)
         v[i] = a.bias ? a.bias[c0 + i] : 0.0f;
-    for (int s = 0; s < a.splitk; s++)
+    for (int s = 0; s < a.splitk; s++) {
+        vec_t t[8];
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            v[i] += pp[(size_t)s * total + (size_t)i * a.N];
-    u32x4 *yp = (u32x4 *)((uint16_t *)a.y + (size_t)n * a.Cout + c0);
-    const bool pre = a.pre != 0 && a.factor != 0.0f;
-    u32x4 old = {0u, 0u, 0u, 0u};
-    if (pre)
-        old = *yp;
-    u32x4 out;
+            t[i] = *(const vec_t *)(pp + (size_t)s * total + (size_t)i * a.N);
 #pragma unroll
-    for (int d = 0; d < 4; d++) {
-        float lo = v[2 * d], hi = v[2 * d + 1];
-        if (pre) {
-            lo = fmaf(__builtin_bit_cast(float, old[d] << 16), a.factor, lo);
-            hi = fmaf(__builtin_bit_cast(float, old[d] & 0xFFFF0000u), a.factor, hi);
-        }
-        if (ACT == ACT_CLAMP) {
-            if (a.act != DLP_ACT_IDENTITY) {
-                lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
-                hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
-            }
-        } else {
-            lo = apply_act(lo, a.act);
-            hi = apply_act(hi, a.act);
-        }
-        out[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+        for (int i = 0; i < 8; i++)
+            v[i] += t[i];
     }
-    *yp = out;
+#pragma unroll
+    for (int q = 0; q < PX; q++) {
+        u32x4 out;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            float lo = v[2 * d][q], hi = v[2 * d + 1][q];
+            if (pre) {
+                lo = fmaf(__builtin_bit_cast(float, old[q][d] << 16), a.factor, lo);
+                hi = fmaf(__builtin_bit_cast(float, old[q][d] & 0xFFFF0000u), a.factor, hi);
+            }
+            if (ACT == ACT_CLAMP) {
+                if (a.act != DLP_ACT_IDENTITY) {
+                    lo = clamp_med3(lo, a.clamp_lo, a.clamp_hi);
+                    hi = clamp_med3(hi, a.clamp_lo, a.clamp_hi);
+                }
+            } else {
+                lo = apply_act(lo, a.act);
+                hi = apply_act(hi, a.act);
+            }
+            out[d] = (uint32_t)to_bf16(lo).bits | ((uint32_t)to_bf16(hi).bits << 16);
+        }
+        yp[q * ystep] = out;
+    }
 }
 
 // Weights [Cout][Cin/groups][KH][KW] -> packed[group][m tile][K tile][k][m in tile], zero padded.
@@ -2604,8 +2622,10 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         TimingScope ts("splitk_reduce", stream);
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
-        if (a.y_cl)
-            hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP>), dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.Cout / 8)), dim3(256), 0, stream, a);
+        if (a.y_cl && (a.N & 3) == 0 && ((uintptr_t)a.part & 15) == 0)
+            hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP, 4>), dim3((unsigned)((a.N + 127) / 128), (unsigned)((a.Cout + 63) / 64)), dim3(256), 0, stream, a);
+        else if (a.y_cl)
+            hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP, 1>), dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.Cout / 8)), dim3(256), 0, stream, a);
         else
             hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, ACT_CLAMP>), dim3((unsigned)((a.N + 1023) / 1024), (unsigned)a.Cout), dim3(256), 0, stream, a);
     }

@@ -319,6 +319,7 @@ CHANNELS_LAST_CASES = [
     (case(3, 1, 1, 1, 512, 512, True, 1, True), (3, 7, 7)),       # 7x7 planes, split-K
     (case(3, (2, 0), (1, 2), (2, 1), 64, 96, True, 2, True), (2, 11, 14)),  # groups, dilation, uneven padding and stride together
     (case(5, 2, 1, 1, 32, 48, True, 1, False), (2, 9, 9)),        # 25 taps
+    (case(1, 0, 1, 1, 1024, 96, True, 1, True), (4, 7, 7)),       # split-K, pixels in fours, output channels off the 64 of a reduction workgroup
 ]
 
 
