@@ -2622,7 +2622,9 @@ int launch_bf16_mfma(const ConvGeom &g, const GemmPlan &p, int pxl, GemmArgs &a,
         TimingScope ts("splitk_reduce", stream);
         if (a.Cout > 65535)
             return fail(DLP_ERR_NOT_IMPLEMENTED, "split-K reduction: more than 65535 output channels");
-        if (a.y_cl && (a.N & 3) == 0 && ((uintptr_t)a.part & 15) == 0)
+        // the form with four pixels per thread only where it still gives every CU a workgroup: on the small launches of small batches
+        // (ResNet-50 at batch 16: 56 workgroups instead of 256) it took 75 us more per pass than the plain one
+        if (a.y_cl && (a.N & 3) == 0 && ((uintptr_t)a.part & 15) == 0 && (long long)((a.N + 127) / 128) * ((a.Cout + 63) / 64) >= dlp_cu_count())
             hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP, 4>), dim3((unsigned)((a.N + 127) / 128), (unsigned)((a.Cout + 63) / 64)), dim3(256), 0, stream, a);
         else if (a.y_cl)
             hipLaunchKernelGGL((splitk_reduce_cl_kernel<ACT_CLAMP, 1>), dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.Cout / 8)), dim3(256), 0, stream, a);
