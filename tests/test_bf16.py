@@ -574,3 +574,11 @@ def test_resnet50_bf16_benchmarked_deployment_logits(oracle_mod):
           (len(runner.cl), rel_cl, np.abs(cl_first - first).max() / np.abs(want).max()))
     assert rel_cl <= 1e-2
     assert (cl_first[pick].argmax(1) == want.argmax(1)).all()
+    # ... and with the stem's max pooling inside the stem's kernel, which is the form that bench.py times: the pooled tensor is the
+    # same bit for bit, so the logits are those of the run above
+    del runner
+    runner = graphs.GraphRunner(ops, params, x.shape, algo="gemm", dtype="bfloat16", fuse_residual=True, prepack=True, channels_last=True,
+                                fuse_stem_pool=True)
+    assert sum(1 for o in runner.ops if o.get("pool")) == 1 and not any(o["op"] == "maxpool" for o in runner.ops)
+    pooled = runner.forward(xd).float().cpu().numpy()
+    assert np.array_equal(pooled, cl_first)
