@@ -1008,10 +1008,12 @@ constexpr int LDK = BK2 + 8;
 
 // What a workgroup of the bf16 kernels does with its finished accumulator tile: the split-K partial
 // store, or the epilogue (bias, activation, factor) and the store to y.  `smem` is the kernel's LDS
-// (at least BM * (BN * 2 + 16) + BM * 4 bytes), free after the last barrier of the main loop.
+// (at least BM * (BN * 2 + 16) bytes), free after the last barrier of the main loop.  `bias_s`: the bias of the tile's BM rows in
+// LDS (zero past M), which the kernel stages when it starts -- requested in the epilogue, its trip to memory stood between the
+// last matrix instruction and the first store of every tile (36 us of a ResNet-50 pass at batch 128).
 template <int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], unsigned char *smem, int smem_bytes,
-                                                 int m0, int n0, int g, int slice, int wm, int wn, int h, int l32, int tid)
+                                                 int m0, int n0, int g, int slice, int wm, int wn, int h, int l32, int tid, const float *bias_s)
 {
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -1083,10 +1085,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
             for (int u = 0; u < PER_THREAD; u++)
                 old[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(yr, piece_offset(u), 0, 0));
         }
-        float *bias_s = (float *)(smem + BN * PITCH);
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
+        __syncthreads(); // every wavefront has read its last operands: LDS takes the tile
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             unsigned char *rowp = smem + (wn * WTN + j * 32 + l32) * PITCH + (wm * WTM + 4 * h) * 2;
@@ -1157,10 +1156,7 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
     if (a.pxv != 0) {
         constexpr int PITCH = BN * 2 + 16;
         (void)smem_bytes; // the callers check BM * PITCH + BM * 4 <= their LDS
-        float *bias_s = (float *)(smem + BM * PITCH);
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
+        __syncthreads(); // every wavefront has read its last operands: LDS takes the tile
         const bool pre = a.pre != 0 && a.factor != 0.0f; // the old y joins before the activation: in the second phase
         const bool clamp = a.act != DLP_ACT_IDENTITY && !pre;
 #pragma unroll
@@ -1277,10 +1273,6 @@ __device__ __forceinline__ void bf16_tile_output(const GemmArgs &a, f32x16 (&acc
         return;
     }
     if (a.factor == 0.0f && (a.M & 7) == 0 && a.y_bytes != 0) {
-        float *bias_s = (float *)smem;
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
         const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
         const bool clamp = a.act != DLP_ACT_IDENTITY;
 #pragma unroll
@@ -1405,6 +1397,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM ==
     const int m0 = mt * BM, n0 = nt * BN;
     const int kt_begin = slice * a.kt_per_slice;
     const int kt_end = min(kt_begin + a.kt_per_slice, a.nkt);
+    // the bias of the tile's rows, for the epilogue: in LDS long before it is wanted (the barriers of the main loop lie between)
+    __shared__ float bias_early[BM];
+    if (tid < BM)
+        bias_early[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
 
     const __amdgpu_buffer_rsrc_t xr =
         __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.x - a.x_shift), 0, a.x_bytes + a.x_shift, 0x00020000);
@@ -1752,7 +1748,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((BM ==
 
     static_assert(BM * (BN * 2 + 16) + BM * 4 <= (int)sizeof(smem), "the staged output tile fits the operand buffers");
     static_assert(BN * (BM * 2 + 16) + BM * 4 <= (int)sizeof(smem), "and so does the channels-last one");
-    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, slice, wm, wn, h, l32, tid);
+    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, slice, wm, wn, h, l32, tid, bias_early);
 }
 
 #ifndef DLP_PATCH_BF16_NA
@@ -1812,6 +1808,10 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
     const int nt = tm - g * a.ntiles;
     const int m0 = mt * BM, n0 = nt * BN;
     const int ncb = a.nkt / KHW; // stages
+    // the bias of the tile's rows, for the epilogue: in LDS long before it is wanted (the barriers of the main loop lie between)
+    __shared__ float bias_early[BM];
+    if (tid < BM)
+        bias_early[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.wp_bytes, 0x00020000);
@@ -2003,7 +2003,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_bf16_kernel(GemmArgs a)
         stage(I0{}, cb);
     __syncthreads(); // the operand reads issued after the last barrier are done before LDS is reused
 
-    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid);
+    bf16_tile_output<BM, BN, WM, WN, ACT>(a, acc, smem, (int)sizeof(smem), m0, n0, g, 0, wm, wn, h, l32, tid, bias_early);
 }
 
 // Channels-last copy of a bf16 input for conv_gemm_bf16_kernel<..., XT = 1>: xt[b][py][px][c] = x[b][c][py * sy][px * sx]
