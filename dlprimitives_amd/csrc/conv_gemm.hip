@@ -161,7 +161,8 @@ __device__ __forceinline__ void static_for_all(F &&f)
 
 template <class T, int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
-                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid);
+                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid,
+                                                 const float *bias_s);
 
 // NSET: register sets of tiles in flight = how many K tiles ahead of the matrix instructions the loads are issued.  Two is
 // enough when eight workgroups share a CU and cover each other's waits; launches with few workgroups per CU (small layers,
@@ -231,6 +232,10 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
     const int m0 = mt * BM, n0 = nt * BN;
     const int kt_begin = slice * kt_per_slice;
     const int kt_end = min(kt_begin + kt_per_slice, a.nkt);
+    // the bias of the tile's rows, for the epilogue: in LDS long before it is wanted (the barriers of the main loop lie between)
+    __shared__ float bias_early[BM];
+    if (tid < BM)
+        bias_early[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
 
     // The X resource starts one padding offset before the tensor, so that the
     // per-pixel window origin is a non-negative offset; taps that the masks let
@@ -458,15 +463,17 @@ __global__ __launch_bounds__(kThreads) void conv_gemm_f32_kernel(GemmArgs a)
             k_step(I0{}, I3{}, I2{}, kt + 2);
     }
 
-    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, splitk, image0, wm, wn, h, l32, tid);
+    gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, slice, splitk, image0, wm, wn, h, l32, tid, bias_early);
 }
 
 // What a workgroup does with its finished accumulator tile: the split-K partial store, or the
 // epilogue (bias, activation, factor) and the NCHW store.  `lds` is LDS that is free after the
-// last barrier of the main loop (at least BM floats).
+// last barrier of the main loop (at least BM floats).  `bias_s`: the bias of the tile's BM rows in LDS (zero past M), staged by the
+// kernel when it starts on the tile: requested here, its trip to memory stood between the last matrix instruction and the first store.
 template <class T, int BM, int BN, int WM, int WN, int ACT>
 __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], float *lds, int m0, int n0,
-                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid)
+                                                 int g, int slice, int splitk, uint32_t image0, int wm, int wn, int h, int l32, int tid,
+                                                 const float *bias_s)
 {
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -562,10 +569,6 @@ __device__ __forceinline__ void gemm_tile_output(const GemmArgs &a, f32x16 (&acc
     // is scalar, instead of a bias load and 64-bit address arithmetic per value.
     const bool pre = a.pre != 0 && a.factor != 0.0f;
     if ((a.factor == 0.0f || (pre && sizeof(T) == 4)) && (a.M & 7) == 0 && a.y_bytes != 0) {
-        float *bias_s = lds;
-        if (tid < BM)
-            bias_s[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
-        __syncthreads();
         const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
         const bool clamp = a.act != DLP_ACT_IDENTITY;
 #pragma unroll
@@ -740,6 +743,11 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
     const int nt = (int)fast_div((uint32_t)t, a.mb_magic, a.mb_shift);
     const int mt = mblk * a.sk_mb + (t - nt * a.sk_mb);
     const int m0 = mt * BM, n0 = nt * BN;
+    // the bias of the tile's rows, for the epilogue: in LDS long before it is wanted (the barriers of the stages lie between, and the
+    // barrier that ends a piece lies between the epilogue of the piece before and this store)
+    __shared__ float bias_early[BM];
+    if (tid < BM)
+        bias_early[tid] = (a.bias && m0 + tid < a.M) ? a.bias[g * a.M + m0 + tid] : 0.0f;
 
     // ---- the tile's patch: one segment of consecutive plane pixels per image (wavefront-uniform) ----
     const int HW = a.OHW;                            // pixels of an output plane
@@ -969,7 +977,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_f32_kernel(GemmArgs a)
         }
     }
     if (output)
-        gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, 0, 1, 0u, wm, wn, h, l32, tid);
+        gemm_tile_output<T, BM, BN, WM, WN, ACT>(a, acc, &As[0][0][0], m0, n0, g, 0, 1, 0u, wm, wn, h, l32, tid, bias_early);
     __syncthreads(); // LDS is reused by the next piece
     u += cb_end - cb_begin;
     }
